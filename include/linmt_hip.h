@@ -1,0 +1,241 @@
+/*
+ * linmt_hip.h -- C ABI of liblinmt_hip.so: hand-written gfx950 (MI355X) HIP kernels for the
+ * per-timestep LSTM / attention / softmax / beam path of LiNMT (liqiangnlp/LiNMT).
+ *
+ * Conventions (all taken from the reference so that its layer classes can call these directly):
+ *   - every matrix is COLUMN-MAJOR, element (i,j) at j*ld+i  (reference: IDX2C, src/utility_cu.h:37);
+ *   - activations are H x B (hidden index fastest, one column per sentence / hypothesis);
+ *   - token / mask arrays are int32, -1 is padding before preprocessing, masks are 0/1;
+ *   - every pointer is a DEVICE pointer owned by the caller unless a comment says "host";
+ *   - nothing here allocates, frees or synchronises; work is queued on `stream` (a hipStream_t
+ *     passed as void*, NULL = the default stream);
+ *   - return value: 0 on success, LH_ERR_ARG for an argument the entry point rejects, otherwise
+ *     the positive hipError_t of the failed launch.  lh_last_error() gives a text for the
+ *     calling thread's last failure.  (The reference prints and exit()s instead,
+ *     src/utility_cu.cu:171-214; the C++ layer classes built on this ABI keep that behaviour.)
+ *
+ * Gate stacking: wherever a 4H x B "stacked" matrix appears, rows [0,H) are the input gate i,
+ * [H,2H) the forget gate f, [2H,3H) the candidate g = c' and [3H,4H) the output gate o.
+ */
+#ifndef LINMT_HIP_H_
+#define LINMT_HIP_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LH_OK 0
+#define LH_ERR_ARG (-1)
+
+typedef void *lh_stream_t;
+
+/* Library identification: returns LH_ABI_VERSION of the build. */
+#define LH_ABI_VERSION 1
+int lh_abi_version(void);
+/* Text for the last non-zero status returned to the calling thread ("" if none). */
+const char *lh_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * a1. Index preprocessing.
+ * Replaces VocabTo01Kernel + VocabToNonMinus1Kernel (src/deep_rnn_kernel.cu:49-70) as launched by
+ * InputToHiddenLayer::PreprocessGpuVocabIndices (src/layer_input_to_hidden.h:1478-1513) and
+ * VocabSoftmaxKernel (src/deep_rnn_kernel.h:144-155): idx0 = idx==-1 ? 0 : idx,
+ * mask01 = idx!=-1, mask01_f = (float)mask01.  idx0 may alias idx; mask01_f may be NULL.
+ */
+int lh_preprocess_indices_i32(const int *idx, int n, int *idx0, int *mask01, float *mask01_f,
+                              lh_stream_t stream);
+
+/* Replaces SetupReverseIndices (src/deep_rnn_kernel.cu:348-352): rev[unique[k]] = k, k < n_unique.
+ * rev has (at least) vocab-size entries; entries of ids not in `unique` are left untouched. */
+int lh_setup_reverse_indices_i32(const int *unique, int n_unique, int *rev, int vocab,
+                                 lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a2. Sparse embedding lookup (+ dropout).
+ * Replaces SparseLookupKernel (src/deep_rnn_kernel.h:249-255) followed by DropoutKernel
+ * (src/deep_rnn_kernel.h:1059-1063) in LstmInputHiddenNode::ForwardPropGpu
+ * (src/node_input_to_hidden.h:236-272).  W is E x V, idx0 has B entries in [0,V), out is E x B:
+ *   out[:,b] = W[:,idx0[b]]            and, when drop_mask != NULL,
+ *   out[i,b] = (drop_mask[i,b] < keep) * (1/keep) * out[i,b]      (keep = probability of KEEPING).
+ */
+int lh_embed_lookup_f32(const float *W, int E, int V, const int *idx0, int B,
+                        const float *drop_mask, float keep, float *out, lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a4. Dense contractions on MFMA (v_mfma_f32_32x32x2_f32), fp32 in / fp32 accumulate.
+ * Replaces CublasGemmWrapper (src/utility_cu.h:153-169) at the call sites of the gate products
+ * (src/node_input_to_hidden.h:297-556, src/node_hidden_to_hidden.h:248-386), the attention
+ * projections (src/layer_attention.h:272,327,441,448) and the output projection
+ * (src/layer_loss.h:820), plus the elementwise kernels the reference launches right after them
+ * (MatrixBiasKernel deep_rnn_kernel.h:525, TanhKernel deep_rnn_kernel.cu:277,
+ * TanhAttentionForwardKernel + ZeroHT deep_rnn_kernel.h:1282-1295), which become the epilogue.
+ *
+ *   acc      = sum_{s < nseg} op(A_s) (M x K_s) * op(X_s) (K_s x N)
+ *   v        = alpha * acc + (beta != 0 ? beta * C : 0) + (bias ? bias[m] : 0)
+ *   v        = act == LH_ACT_TANH ? tanhf(v) : v
+ *   C[m,n]   = colmask ? v * colmask[n] : v
+ *
+ * Several segments give the stacked product W*[x;h;h~] without materialising [x;h;h~].
+ * transA: A_s is stored K_s x M (lda >= K_s) and used transposed; transX: X_s is stored N x K_s.
+ * Both flags apply to every segment.  `segs` is a HOST array, nseg <= LH_GEMM_MAX_SEGS.
+ */
+#define LH_GEMM_MAX_SEGS 3
+#define LH_ACT_NONE 0
+#define LH_ACT_TANH 1
+typedef struct lh_gemm_seg {
+  const float *A; /* device */
+  int lda;
+  const float *X; /* device */
+  int ldx;
+  int K;
+} lh_gemm_seg;
+int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
+                float alpha, float beta, const float *bias, int act, const int *colmask, float *C,
+                int ldc, lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a3. Fused LSTM cell forward: bias add, gate nonlinearities, c_t / h_t update, padding mask,
+ * optional cell clip and the dropout mask of the layer above, in one pass over HBM.
+ * Replaces ForwardSigmoidKernel / ForwardSigmoidKernelFeed / ForwardTanhKernel(/Feed)
+ * (src/deep_rnn_kernel.cu:78-117, src/deep_rnn_kernel.h:64-88), ForwardCTKernel (.h:93),
+ * ClipMatKernel (.h:1528), ForwardHTKernel (.cu:121), ZeroCTAndHT (.h:123) as sequenced in
+ * LstmInputHiddenNode::ForwardPropGpu (src/node_input_to_hidden.h:350-621) and
+ * LstmHiddenHiddenNode::ForwardPropGpu (src/node_hidden_to_hidden.h:270-430), and the
+ * DropoutKernel the layer above applies to its copy of h (src/node_hidden_to_hidden.h:208-226).
+ *
+ *   s      = ((pre1 + pre2) + pre3) + bias            (4H x B stacked; pre2 / pre3 may be NULL)
+ *   i,f,o  = 1/(1+exp(-s)), g = tanh(s)               fp32 expf/tanhf; with sigmoid_f64 != 0 the
+ *                                                     three sigmoids are evaluated in double, as
+ *                                                     ForwardSigmoidKernelFeed does
+ *   c      = f*c_prev + i*g ; cell_clip > 0: c = clamp(c, +-cell_clip)
+ *   h      = o*tanhf(c) ; h *= mask01[b] ; c *= mask01[b]        (i,f,g,o are not masked)
+ *   gates  (4H x B, optional) receives i,f,g,o for the backward pass
+ *   h_drop (H x B, optional)  = (next_drop_mask < keep) * (1/keep) * h
+ * ld of every 4H x B operand is 4H, of every H x B operand H.  c may alias c_prev.
+ */
+int lh_lstm_cell_fwd_f32(int H, int B, const float *pre1, const float *pre2, const float *pre3,
+                         const float *bias4h, const float *c_prev, const int *mask01,
+                         int sigmoid_f64, float cell_clip, float *gates, float *c, float *h,
+                         const float *next_drop_mask, float keep, float *h_drop,
+                         lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a6. Attention core: alignment position, window, scores, max-subtracted exp, normalisation,
+ * Gaussian weighting and context vector in one kernel (one workgroup per column).
+ * Replaces SigmoidKernel, AlignmentPosKernel, LowerUpperKernel (src/deep_rnn_kernel.h:1076-1100),
+ * CreateIndicesKernel (src/deep_rnn_kernel.cu:294-316), LoadInHSKernel (.h:1142-1164),
+ * ElemReduceKernelLarge (.h:1309-1342), AlignmentReductionKernel (.h:1198-1241),
+ * GetViterbiAlignmentKernel (.h:1105-1117) and CreateCTKernel (.h:1251-1260) as sequenced in
+ * AttentionNode::ForwardProp (src/layer_attention.h:282-392).
+ *
+ * Inputs:  tanh1 = tanh(W_p*ha) (H x B), v_p (H), wa = W_a^T*ha (H x B), mask01 (B),
+ *          batch_info = [len_0..len_{B-1}, off_0..off_{B-1}]  (src/file_helper.cc:242-243),
+ *          encoder top-layer states: state of encoder timestep tau, column c, is the H floats at
+ *          hs + tau*hs_step_stride + c*hs_col_stride; column c = hs_col ? hs_col[b] : b
+ *          (hs_col lets the beam columns of one sentence share that sentence's states instead
+ *          of the reference's per-beam replicas, src/deep_rnn.h:1633-1643).
+ * Local-p (D >= 0), W = 2D+1:
+ *   sig_b = 1/(1+exp(-(double)(v_p . tanh1[:,b])))  ; p_b = len_b * sig_b
+ *   lo = max(0,(int)p_b - D) ; hi = min(len_b-1,(int)p_b + D)
+ *   idx[b,j] = (mask01[b]==1 && lo+j <= hi) ? lo+j : -1                (B x W, at b + B*j)
+ *   hs_j = idx>=0 ? state(tau = len_b-1-idx + off_b) : 0 ; sc_j = hs_j . wa[:,b]
+ *   mx = max(0, max_valid sc_j) ; e_j = exp(sc_j - mx) ; Z = sum e_j
+ *   g_j = valid ? exp(-(p_b-idx)^2 / (2*sigma^2)) : 1,  sigma^2 = D*D/4.0        (W x B, at j + W*b)
+ *   a_j = valid ? (Z != 0 ? e_j/Z : e_j) * g_j : 0                             (B x W, at b + B*j)
+ *   ctx[:,b] = sum_j a_j * hs_j ; viterbi[b] = idx of the first maximal a_j (-1 if none > -1)
+ * Global "general" (D < 0; not in the reference, the textbook Luong global attention):
+ *   window = all len_b source positions (W = max_len slots, idx = j for j < len_b when
+ *   mask01[b]==1), no p_b / Gaussian (g = 1, p_t/sigma outputs untouched), mx = true maximum.
+ * Outputs p_t (B), sigma (B), indices (B x W), align (B x W), cached_exp (W x B), ctx (H x B),
+ * viterbi (B, optional).  max_len (= the W of the global variant) is ignored for D >= 0.
+ * hs_steps = number of encoder timesteps held in hs; a slot whose tau falls outside [0,hs_steps)
+ * reads as a zero vector instead of touching memory outside the buffer.
+ */
+int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_steps, const float *tanh1,
+                         const float *v_p, const float *wa, const float *hs, long long hs_step_stride,
+                         long long hs_col_stride, const int *hs_col, const int *batch_info,
+                         const int *mask01, float *p_t, float *sigma, int *indices, float *align,
+                         float *cached_exp, float *ctx, int *viterbi, lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a8 / a9. Vocabulary softmax and log-likelihood, one pass over the V x B logits.
+ *
+ * lh_softmax_fwd_f32 replaces MatrixBiasKernel + OutputdistOverflowPreventionKernel
+ * (src/deep_rnn_kernel.h:525-530,353-429) in SoftmaxLayer::GetDistributionGpu
+ * (src/layer_loss.h:822-868): p[:,b] = softmax(logits[:,b] + bias), fp32.  p may alias logits.
+ * bias may be NULL (already added by the GEMM epilogue).
+ *
+ * lh_train_loglik_f32 replaces TrainPerplexityKernel (src/deep_rnn_kernel.h:336-342):
+ *   *accum += sum_{b: mask01[b]==1} log((double)p[tgt0[b], b]).
+ *
+ * lh_logsoftmax_xent_f32 replaces OutputdistPerplexityKernel (src/deep_rnn_kernel.h:433-519) and
+ * the host loop of SoftmaxLayer::ComputeLossGpu (src/layer_loss.h:693-701) without the V x B
+ * double buffer: in double, logp_tgt[b] = log(exp(z_t - mx)) - log(sum_v exp(z_v - mx)) with
+ * z = (double)(logits + bias); *loss_accum += sum_{b: mask01[b]==1} logp_tgt[b] (summed in
+ * column order by one thread, like the reference's host loop).  logp_tgt may be NULL.
+ */
+int lh_softmax_fwd_f32(const float *logits, int ldl, const float *bias, int V, int B, float *p,
+                       int ldp, lh_stream_t stream);
+int lh_train_loglik_f32(const float *p, int ldp, int V, int B, const int *tgt0, const int *mask01,
+                        double *accum, lh_stream_t stream);
+int lh_logsoftmax_xent_f32(const float *logits, int ldl, const float *bias, int V, int B,
+                           const int *tgt0, const int *mask01, double *logp_tgt,
+                           double *loss_accum, lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a10. Beam search step on the device.
+ *
+ * lh_beam_topk_f32: fused log-softmax + per-column top-K.  Replaces the V x beam distribution
+ * copy (src/decoder.h:1413), CopyDistToEigen (:1429-1436), EnsemblesModels' renormalisation
+ * (:1910-1931) and the per-column bounded heap of Decoder::ExpandHypothesis (:398-427).
+ * For each column b < B: mx, lse = log(sum exp(z - mx)), the K largest z (ties: lowest vocab id
+ * wins, as the strict `<` of decoder.h:405 keeps the earlier entry), best first:
+ *   cand_logp[k + K*b] = z_k - mx - lse ; cand_id[k + K*b] = vocab id ; logp_eof[b] = logp of id
+ *   `eof_id` (used by FinishCurrentHypotheses, decoder.h:506).  K <= LH_BEAM_MAX_K, K <= V.
+ *
+ * lh_beam_merge_f32: per-sentence merge of the candidates.  Replaces the global heap walk of
+ * Decoder::ExpandHypothesis (src/decoder.h:429-480) and FinishCurrentHypotheses (:502-525) for
+ * n_sent sentences at once (sentence s owns columns [s*beam, (s+1)*beam)).
+ *   expansion (step < limit[s]): candidates of column i (only i = 0 when step == 0) get
+ *     score = cand_logp + prev_score[i] - rank*diversity (rank 1 = best of its column); walk all
+ *     candidates by (score desc, beam column asc, vocab id asc): id == start_id is dropped;
+ *     id == eof_id is recorded as finished (fin_beam, fin_score = score + penalty) and takes no
+ *     slot; otherwise slot k gets tok, backptr (GLOBAL column index s*beam + i), score + penalty.
+ *     If the candidates run out (the reference pops an empty heap there) the remaining slots get
+ *     tok = eof_id, backptr = s*beam, score = -FLT_MAX.
+ *   finish (step == limit[s]): every column i is recorded as finished with
+ *     fin_score = prev_score[i] + logp_eof[i] + penalty; tok/backptr/score keep column i
+ *     (tok = eof_id, backptr = own column).
+ *   idle (step > limit[s]): tok = eof_id, backptr = own column, score unchanged, no finished.
+ * Outputs per step: tok, backptr, score (n_sent*beam each; score may alias prev_score is NOT
+ * allowed), fin_count (n_sent), fin_beam / fin_score (n_sent*beam, first fin_count[s] valid, in
+ * walk order).  K = beam + 1 in the reference.
+ */
+#define LH_BEAM_MAX_K 64
+int lh_beam_topk_f32(const float *logits, int ldl, const float *bias, int V, int B, int K,
+                     int eof_id, float *cand_logp, int *cand_id, float *logp_eof,
+                     lh_stream_t stream);
+int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const int *limit,
+                      const float *cand_logp, const int *cand_id, const float *logp_eof,
+                      const float *prev_score, float diversity, float penalty, int start_id,
+                      int eof_id, int *tok, int *backptr, float *score, int *fin_count,
+                      int *fin_beam, float *fin_score, lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a11. Hypothesis state gather: dst_t[:,k] = src_t[:,backptr[k]] for n_tensors H x B tensors in
+ * one launch.  Replaces the per-column cudaMemcpy loops of SwapStatesDecoding
+ * (src/layer_input_to_hidden.h:1517-1531, src/layer_hidden_to_hidden.h:569-584), the h~ swap of
+ * NeuralMachineTranslation::SwapDecodingStates (src/deep_rnn.h:1842-1857) and the whole-matrix
+ * copies of TargetCopyPrevStates (src/deep_rnn.h:1861-1872).  src/dst are HOST arrays of device
+ * pointers, n_tensors <= LH_GATHER_MAX_TENSORS; dst_t must not alias any src.
+ * With col_src = NULL and backptr = identity this is also TransferDecodingStatesGpu
+ * (src/layer_input_to_hidden.h:1536-1545) when backptr maps every beam column to its sentence.
+ */
+#define LH_GATHER_MAX_TENSORS 24
+int lh_beam_gather_f32(const float *const *src, float *const *dst, int n_tensors, int H, int B,
+                       const int *backptr, lh_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LINMT_HIP_H_ */

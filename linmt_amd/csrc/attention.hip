@@ -1,0 +1,201 @@
+// Attention core (Luong local-p, and the textbook global "general" variant): alignment position,
+// window indices, scores, max-subtracted exp, normalisation, Gaussian weighting and the context
+// vector in ONE kernel.  One workgroup (4 wavefronts) per column b:
+//   phase 1  v_p . tanh1[:,b]  -> sigmoid -> p_b -> window [lo,hi]           (block reduction)
+//   phase 2  score_j = hs_j . wa[:,b]; wavefront w takes slots j = w, w+4, ...  (DPP/shuffle sums)
+//   phase 3  max / exp / sum / Gaussian over the <= W slots, kept in LDS
+//   phase 4  ctx[:,b] = sum_j a_j hs_j, thread-per-row-quad; the second read of the window comes
+//            from L2 (the W x H window was just streamed by this very workgroup).
+// The reference materialises the window (LoadInHSKernel) and launches eight kernels for this.
+#include "lh_common.h"
+
+namespace {
+
+constexpr int kMaxSlots = 512;
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / lh::kWave;
+
+struct AttnArgs {
+  int H, B, D, W;
+  const float *tanh1, *v_p, *wa, *hs;
+  long long step_stride, col_stride;
+  int hs_steps;
+  const int *hs_col, *batch_info, *mask01;
+  float *p_t, *sigma;
+  int *indices;
+  float *align, *cached_exp, *ctx;
+  int *viterbi;
+};
+
+template <bool VEC>
+__device__ __forceinline__ float dot_wave(const float *__restrict__ x, const float *__restrict__ y,
+                                          int H, int lane) {
+  float acc = 0.f;
+  if constexpr (VEC) {
+    for (int r = lane * 4; r < H; r += lh::kWave * 4) {
+      const float4 a = *reinterpret_cast<const float4 *>(x + r);
+      const float4 b = *reinterpret_cast<const float4 *>(y + r);
+      acc += a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
+    }
+  } else {
+    for (int r = lane; r < H; r += lh::kWave) acc += x[r] * y[r];
+  }
+  return lh::wave_sum(acc);
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void attn_core_kernel(const AttnArgs a) {
+  __shared__ float s_val[kMaxSlots];   // scores, then alignment weights
+  __shared__ int s_tau[kMaxSlots];     // encoder timestep of slot j, -1 = no state to read
+  __shared__ int s_idx[kMaxSlots];     // source position of slot j, -1 = invalid slot
+  __shared__ float s_red[kWaves];
+  __shared__ float s_scalar[2];
+
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x, wave = tid / lh::kWave, lane = tid % lh::kWave;
+  const int H = a.H, B = a.B, W = a.W, D = a.D;
+  const int len = a.batch_info[b];
+  const int off = a.batch_info[B + b];
+  const int m = a.mask01[b];
+  const int col = a.hs_col ? a.hs_col[b] : b;
+  const float *wa = a.wa + (size_t)b * H;
+  const float *hs_c = a.hs + (size_t)col * a.col_stride;
+
+  float p = 0.f;
+  int lo = 0, hi = len - 1;
+  if (D >= 0) {
+    float part = 0.f;
+    const float *t1 = a.tanh1 + (size_t)b * H;
+    for (int r = tid; r < H; r += kThreads) part += a.v_p[r] * t1[r];
+    const float dot = lh::block_sum<kWaves>(part, s_red);
+    const float sig = (float)(1.0 / (1.0 + exp(-1.0 * (double)dot)));
+    p = (float)len * sig;
+    lo = (0 > (int)p - D) ? 0 : ((int)p - D);
+    hi = ((len - 1) < (int)p + D) ? (len - 1) : ((int)p + D);
+    if (tid == 0) {
+      a.p_t[b] = p;
+      a.sigma[b] = sig;
+    }
+  }
+
+  // window indices (reference layout B x W, element (b,j) at b + B*j)
+  for (int j = tid; j < W; j += kThreads) {
+    int idx = -1;
+    if (m == 1 && lo + j <= hi) idx = lo + j;
+    a.indices[b + (size_t)B * j] = idx;
+    s_idx[j] = idx;
+    int tau = -1;
+    if (idx >= 0) {
+      tau = len - 1 - idx + off;
+      if (tau < 0 || tau >= a.hs_steps) tau = -1;  // outside the caller's state buffer: zero vector
+    }
+    s_tau[j] = tau;
+  }
+  __syncthreads();
+
+  // scores
+  for (int j = wave; j < W; j += kWaves) {
+    const int tau = s_tau[j];
+    float sc = 0.f;
+    if (tau >= 0) sc = dot_wave<VEC>(hs_c + (size_t)tau * a.step_stride, wa, H, lane);
+    if (lane == 0) s_val[j] = sc;
+  }
+  __syncthreads();
+
+  // normalisation: every thread reduces the (few) slots redundantly out of LDS
+  float mx = D >= 0 ? 0.f : -FLT_MAX;
+  for (int j = 0; j < W; ++j) {
+    if (s_idx[j] != -1 && s_val[j] > mx) mx = s_val[j];
+  }
+  float Z = 0.f;
+  for (int j = 0; j < W; ++j) {
+    if (s_idx[j] != -1) Z += expf(s_val[j] - mx);
+  }
+  __syncthreads();
+  const float sigma_sq = (float)((D * D) / 4.0);
+  for (int j = tid; j < W; j += kThreads) {
+    const int idx = s_idx[j];
+    float al = 0.f, g = 1.f;
+    if (idx != -1) {
+      const float e = expf(s_val[j] - mx);
+      if (D >= 0) {
+        const float dlt = p - (float)idx;
+        g = expf((-1.f * (dlt * dlt)) / (2.f * sigma_sq));
+      }
+      al = (Z != 0.f) ? (e / Z) * g : e;
+    }
+    a.align[b + (size_t)B * j] = al;
+    a.cached_exp[j + (size_t)W * b] = g;
+    s_val[j] = al;
+  }
+  __syncthreads();
+
+  if (a.viterbi && tid == 0) {
+    float best = -1.f;
+    int best_idx = -1;
+    for (int j = 0; j < W; ++j) {
+      if (best < s_val[j]) {
+        best = s_val[j];
+        best_idx = s_idx[j];
+      }
+    }
+    a.viterbi[b] = best_idx;
+  }
+
+  // context vector
+  float *ctx = a.ctx + (size_t)b * H;
+  if constexpr (VEC) {
+    for (int r = tid * 4; r < H; r += kThreads * 4) {
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int j = 0; j < W; ++j) {
+        const int tau = s_tau[j];
+        if (tau < 0) continue;
+        const float w = s_val[j];
+        const float4 v = *reinterpret_cast<const float4 *>(hs_c + (size_t)tau * a.step_stride + r);
+        acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+      }
+      *reinterpret_cast<float4 *>(ctx + r) = acc;
+    }
+  } else {
+    for (int r = tid; r < H; r += kThreads) {
+      float acc = 0.f;
+      for (int j = 0; j < W; ++j) {
+        const int tau = s_tau[j];
+        if (tau < 0) continue;
+        acc += s_val[j] * hs_c[(size_t)tau * a.step_stride + r];
+      }
+      ctx[r] = acc;
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_steps,
+                                    const float *tanh1, const float *v_p, const float *wa,
+                                    const float *hs, long long hs_step_stride,
+                                    long long hs_col_stride, const int *hs_col,
+                                    const int *batch_info, const int *mask01, float *p_t,
+                                    float *sigma, int *indices, float *align, float *cached_exp,
+                                    float *ctx, int *viterbi, lh_stream_t stream) {
+  if (H <= 0 || B <= 0 || hs_steps <= 0)
+    return lh::fail_arg("lh_attn_core_fwd_f32: H=%d B=%d hs_steps=%d", H, B, hs_steps);
+  const int W = D >= 0 ? 2 * D + 1 : max_len;
+  if (W <= 0 || W > kMaxSlots)
+    return lh::fail_arg("lh_attn_core_fwd_f32: window of %d slots outside [1,%d]", W, kMaxSlots);
+  if (!wa || !hs || !batch_info || !mask01 || !indices || !align || !cached_exp || !ctx)
+    return lh::fail_arg("lh_attn_core_fwd_f32: a required pointer is NULL");
+  if (D >= 0 && (!tanh1 || !v_p || !p_t || !sigma))
+    return lh::fail_arg("lh_attn_core_fwd_f32: local-p needs tanh1, v_p, p_t and sigma");
+  if (hs_step_stride < 0 || hs_col_stride < 0)
+    return lh::fail_arg("lh_attn_core_fwd_f32: negative stride");
+
+  AttnArgs a{H, B, D, W, tanh1, v_p, wa, hs, hs_step_stride, hs_col_stride, hs_steps, hs_col,
+             batch_info, mask01, p_t, sigma, indices, align, cached_exp, ctx, viterbi};
+  const bool vec = H % 4 == 0 && lh::aligned16(wa) && lh::aligned16(hs) && lh::aligned16(ctx) &&
+                   hs_step_stride % 4 == 0 && hs_col_stride % 4 == 0;
+  hipStream_t st = lh::as_stream(stream);
+  if (vec) hipLaunchKernelGGL(attn_core_kernel<true>, dim3(B), dim3(kThreads), 0, st, a);
+  else hipLaunchKernelGGL(attn_core_kernel<false>, dim3(B), dim3(kThreads), 0, st, a);
+  return lh::check_launch("lh_attn_core_fwd_f32");
+}

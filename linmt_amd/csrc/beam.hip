@@ -1,0 +1,179 @@
+// Beam-search bookkeeping on the device: per-sentence merge of the per-column candidates and the
+// back-pointer gather of every recurrent state tensor in one launch.
+#include "lh_common.h"
+
+namespace {
+
+constexpr int kMergeThreads = 256;
+constexpr int kMaxCand = 4096;
+
+struct MergeArgs {
+  int n_sent, beam, K, step;
+  const int *limit;
+  const float *cand_logp;
+  const int *cand_id;
+  const float *logp_eof;
+  const float *prev_score;
+  float diversity, penalty;
+  int start_id, eof_id;
+  int *tok, *backptr;
+  float *score;
+  int *fin_count, *fin_beam;
+  float *fin_score;
+};
+
+// One workgroup per sentence.  Candidates are ranked by counting how many others precede them in
+// the total order (score desc, beam column asc, vocab id asc); thread 0 then walks that order the
+// way Decoder::ExpandHypothesis pops its global heap.
+__global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeArgs a) {
+  __shared__ float s_score[kMaxCand];
+  __shared__ int s_id[kMaxCand];
+  __shared__ short s_col[kMaxCand];
+  __shared__ short s_order[kMaxCand];
+
+  const int s = blockIdx.x, tid = threadIdx.x;
+  const int beam = a.beam, K = a.K;
+  const int c0 = s * beam;  // first global column of this sentence
+  const int limit = a.limit[s];
+
+  if (a.step >= limit) {
+    // finish (== limit) or idle (> limit): no expansion.
+    for (int i = tid; i < beam; i += kMergeThreads) {
+      a.tok[c0 + i] = a.eof_id;
+      a.backptr[c0 + i] = c0 + i;
+      float sc = a.prev_score[c0 + i];
+      if (a.step == limit) {
+        sc = sc + (a.logp_eof[c0 + i] + a.penalty);  // decoder.h:506 adds (log p + penalty)
+        a.fin_beam[c0 + i] = i;
+        a.fin_score[c0 + i] = sc;
+      }
+      a.score[c0 + i] = sc;
+    }
+    if (tid == 0) a.fin_count[s] = a.step == limit ? beam : 0;
+    return;
+  }
+
+  const int cols = a.step == 0 ? 1 : beam;
+  const int C = cols * K;
+  for (int e = tid; e < C; e += kMergeThreads) {
+    const int i = e / K, k = e % K;
+    const float rank_penalty = (float)(k + 1) * a.diversity;
+    s_score[e] = a.cand_logp[(size_t)(c0 + i) * K + k] + a.prev_score[c0 + i] - rank_penalty;
+    s_id[e] = a.cand_id[(size_t)(c0 + i) * K + k];
+    s_col[e] = (short)i;
+  }
+  __syncthreads();
+  for (int e = tid; e < C; e += kMergeThreads) {
+    const float sc = s_score[e];
+    const int id = s_id[e], col = s_col[e];
+    int before = 0;
+    for (int o = 0; o < C; ++o) {
+      const float so = s_score[o];
+      const bool first = so > sc || (so == sc && (s_col[o] < col || (s_col[o] == col && s_id[o] < id)));
+      before += first ? 1 : 0;
+    }
+    s_order[before] = (short)e;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int filled = 0, nfin = 0;
+    for (int r = 0; r < C && filled < beam; ++r) {
+      const int e = s_order[r];
+      const int id = s_id[e];
+      if (id == a.start_id) continue;
+      const float sc = s_score[e] + a.penalty;
+      if (id == a.eof_id) {
+        if (nfin < beam) {  // at most one <EOF> candidate per column exists
+          a.fin_beam[c0 + nfin] = s_col[e];
+          a.fin_score[c0 + nfin] = sc;
+          ++nfin;
+        }
+        continue;
+      }
+      a.tok[c0 + filled] = id;
+      a.backptr[c0 + filled] = c0 + s_col[e];
+      a.score[c0 + filled] = sc;
+      ++filled;
+    }
+    for (; filled < beam; ++filled) {  // candidates exhausted (the reference pops an empty heap)
+      a.tok[c0 + filled] = a.eof_id;
+      a.backptr[c0 + filled] = c0;
+      a.score[c0 + filled] = -FLT_MAX;
+    }
+    a.fin_count[s] = nfin;
+  }
+}
+
+struct GatherArgs {
+  const float *src[LH_GATHER_MAX_TENSORS];
+  float *dst[LH_GATHER_MAX_TENSORS];
+  int H, B;
+  const int *backptr;
+};
+
+template <int VW>
+__global__ __launch_bounds__(256) void beam_gather_kernel(const GatherArgs a) {
+  const int HQ = a.H / VW;
+  const int t = blockIdx.z;
+  const int k = blockIdx.y;
+  int from = a.backptr[k];
+  from = from < 0 ? 0 : (from >= a.B ? a.B - 1 : from);
+  const float *src = a.src[t] + (size_t)from * a.H;
+  float *dst = a.dst[t] + (size_t)k * a.H;
+  for (int q = blockIdx.x * 256 + threadIdx.x; q < HQ; q += gridDim.x * 256) {
+    if constexpr (VW == 4)
+      reinterpret_cast<float4 *>(dst)[q] = reinterpret_cast<const float4 *>(src)[q];
+    else
+      dst[q] = src[q];
+  }
+}
+
+}  // namespace
+
+extern "C" int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const int *limit,
+                                 const float *cand_logp, const int *cand_id, const float *logp_eof,
+                                 const float *prev_score, float diversity, float penalty,
+                                 int start_id, int eof_id, int *tok, int *backptr, float *score,
+                                 int *fin_count, int *fin_beam, float *fin_score,
+                                 lh_stream_t stream) {
+  if (n_sent <= 0 || beam <= 0 || K <= 0 || step < 0)
+    return lh::fail_arg("lh_beam_merge_f32: n_sent=%d beam=%d K=%d step=%d", n_sent, beam, K, step);
+  if ((long long)beam * K > kMaxCand)
+    return lh::fail_arg("lh_beam_merge_f32: beam*K=%lld exceeds %d", (long long)beam * K, kMaxCand);
+  if (!limit || !cand_logp || !cand_id || !logp_eof || !prev_score || !tok || !backptr || !score ||
+      !fin_count || !fin_beam || !fin_score)
+    return lh::fail_arg("lh_beam_merge_f32: a required pointer is NULL");
+  if (score == prev_score) return lh::fail_arg("lh_beam_merge_f32: score aliases prev_score");
+  MergeArgs a{n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof, prev_score, diversity,
+              penalty, start_id, eof_id, tok, backptr, score, fin_count, fin_beam, fin_score};
+  hipLaunchKernelGGL(beam_merge_kernel, dim3(n_sent), dim3(kMergeThreads), 0,
+                     lh::as_stream(stream), a);
+  return lh::check_launch("lh_beam_merge_f32");
+}
+
+extern "C" int lh_beam_gather_f32(const float *const *src, float *const *dst, int n_tensors, int H,
+                                  int B, const int *backptr, lh_stream_t stream) {
+  if (n_tensors < 1 || n_tensors > LH_GATHER_MAX_TENSORS || H <= 0 || B <= 0 || !src || !dst ||
+      !backptr)
+    return lh::fail_arg("lh_beam_gather_f32: n_tensors=%d H=%d B=%d or NULL pointer", n_tensors, H,
+                        B);
+  GatherArgs a{};
+  bool vec = H % 4 == 0;
+  for (int t = 0; t < n_tensors; ++t) {
+    if (!src[t] || !dst[t]) return lh::fail_arg("lh_beam_gather_f32: tensor %d is NULL", t);
+    for (int u = 0; u < n_tensors; ++u)
+      if (dst[t] == src[u]) return lh::fail_arg("lh_beam_gather_f32: dst %d aliases src %d", t, u);
+    a.src[t] = src[t];
+    a.dst[t] = dst[t];
+    vec = vec && lh::aligned16(src[t]) && lh::aligned16(dst[t]);
+  }
+  a.H = H;
+  a.B = B;
+  a.backptr = backptr;
+  const int hq = vec ? H / 4 : H;
+  const dim3 grid((hq + 255) / 256, B, n_tensors), block(256);
+  if (B > 65535) return lh::fail_arg("lh_beam_gather_f32: B=%d exceeds 65535", B);
+  if (vec) hipLaunchKernelGGL(beam_gather_kernel<4>, grid, block, 0, lh::as_stream(stream), a);
+  else hipLaunchKernelGGL(beam_gather_kernel<1>, grid, block, 0, lh::as_stream(stream), a);
+  return lh::check_launch("lh_beam_gather_f32");
+}

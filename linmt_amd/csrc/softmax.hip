@@ -1,0 +1,396 @@
+// Vocabulary softmax / log-likelihood / fused log-softmax + top-K.
+//
+// One workgroup of 1024 threads (16 wavefronts) owns one column of the V x B logits.  The column is
+// read from HBM exactly once with 16-byte loads and stays in registers (NV float4 per thread, chosen
+// so that 4096*NV >= V) through the max, exp-sum and the final normalisation / selection, so the
+// traffic is the algorithmic minimum: V*B*4 bytes in, plus V*B*4 out only for the kernel that has to
+// hand back probabilities.  Columns that are not 16-byte aligned or longer than 65536 rows take a
+// generic strided kernel that re-reads the column (from L2) instead.
+#include "lh_common.h"
+
+namespace {
+
+constexpr int kT = 1024;
+constexpr int kNW = kT / lh::kWave;
+constexpr float kNegInf = -__builtin_huge_valf();
+
+__device__ __forceinline__ float &comp(float4 &v, int c) {
+  return c == 0 ? v.x : (c == 1 ? v.y : (c == 2 ? v.z : v.w));
+}
+
+// Loads column `col` (+bias) into registers; rows >= V read as -inf.
+template <int NV>
+__device__ __forceinline__ void load_column(float4 (&x)[NV], const float *__restrict__ col,
+                                            const float *__restrict__ bias, int V, int tid) {
+  const int V4 = V / 4;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int f = tid + i * kT;
+    float4 v = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
+    if (f < V4) {
+      v = reinterpret_cast<const float4 *>(col)[f];
+      if (bias) {
+        const float4 bb = reinterpret_cast<const float4 *>(bias)[f];
+        v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
+      }
+    }
+    x[i] = v;
+  }
+}
+
+template <int NV>
+__device__ __forceinline__ float local_max(const float4 (&x)[NV]) {
+  float m = kNegInf;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) m = fmaxf(fmaxf(fmaxf(m, x[i].x), fmaxf(x[i].y, x[i].z)), x[i].w);
+  return m;
+}
+
+// ---- probabilities out ----------------------------------------------------------------------
+template <int NV>
+__global__ __launch_bounds__(kT) void softmax_fwd_kernel(const float *__restrict__ logits, int ldl,
+                                                         const float *__restrict__ bias, int V,
+                                                         float *__restrict__ p, int ldp) {
+  __shared__ float red[kNW];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  float4 x[NV];
+  load_column<NV>(x, logits + (size_t)b * ldl, bias, V, tid);
+  const float mx = lh::block_max<kNW>(local_max<NV>(x), red);
+  float part = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    x[i].x = expf(x[i].x - mx); x[i].y = expf(x[i].y - mx);
+    x[i].z = expf(x[i].z - mx); x[i].w = expf(x[i].w - mx);
+    part += (x[i].x + x[i].y) + (x[i].z + x[i].w);
+  }
+  const float sum = lh::block_sum<kNW>(part, red);
+  float4 *out = reinterpret_cast<float4 *>(p + (size_t)b * ldp);
+  const int V4 = V / 4;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int f = tid + i * kT;
+    if (f < V4) out[f] = make_float4(x[i].x / sum, x[i].y / sum, x[i].z / sum, x[i].w / sum);
+  }
+}
+
+// Generic fallback: any V / alignment, column re-read twice.
+__global__ __launch_bounds__(kT) void softmax_fwd_generic_kernel(const float *logits, int ldl,
+                                                                 const float *bias, int V, float *p,
+                                                                 int ldp) {
+  __shared__ float red[kNW];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const float *col = logits + (size_t)b * ldl;
+  float *out = p + (size_t)b * ldp;
+  float m = kNegInf;
+  for (int r = tid; r < V; r += kT) m = fmaxf(m, col[r] + (bias ? bias[r] : 0.f));
+  const float mx = lh::block_max<kNW>(m, red);
+  float part = 0.f;
+  for (int r = tid; r < V; r += kT) {
+    const float e = expf(col[r] + (bias ? bias[r] : 0.f) - mx);
+    out[r] = e;  // p may alias logits: row r is only ever touched by this thread
+    part += e;
+  }
+  const float sum = lh::block_sum<kNW>(part, red);
+  for (int r = tid; r < V; r += kT) out[r] = out[r] / sum;
+}
+
+// ---- training log-likelihood from probabilities (serial, column order, like the reference) ------
+__global__ void train_loglik_kernel(const float *p, int ldp, int B, const int *tgt0,
+                                    const int *mask01, double *accum) {
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  double acc = accum[0];
+  for (int b = 0; b < B; ++b)
+    if (mask01[b] == 1) acc += log((double)p[(size_t)b * ldp + tgt0[b]]);
+  accum[0] = acc;
+}
+
+// ---- double-precision log-softmax of the target row -----------------------------------------
+template <int NV>
+__global__ __launch_bounds__(kT) void logsoftmax_tgt_kernel(const float *__restrict__ logits,
+                                                            int ldl, const float *__restrict__ bias,
+                                                            int V, const int *__restrict__ tgt0,
+                                                            double *__restrict__ logp_tgt) {
+  __shared__ float redf[kNW];
+  __shared__ double redd[kNW];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  float4 x[NV];
+  load_column<NV>(x, logits + (size_t)b * ldl, bias, V, tid);
+  const double mx = (double)lh::block_max<kNW>(local_max<NV>(x), redf);
+  double part = 0.0;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    part += exp((double)x[i].x - mx);  // rows >= V hold -inf and add exp(-inf) = 0
+    part += exp((double)x[i].y - mx);
+    part += exp((double)x[i].z - mx);
+    part += exp((double)x[i].w - mx);
+  }
+  const double sum = lh::block_sum<kNW>(part, redd);
+  const int t = tgt0[b];
+  const int f = t / 4, c = t % 4;
+  if (f % kT == tid && t < V) {
+    const int i = f / kT;
+    float zt = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+      if (k == i) zt = comp(x[k], c);
+    logp_tgt[b] = log(exp((double)zt - mx)) - log(sum);
+  }
+}
+
+__global__ __launch_bounds__(kT) void logsoftmax_tgt_generic_kernel(const float *logits, int ldl,
+                                                                    const float *bias, int V,
+                                                                    const int *tgt0,
+                                                                    double *logp_tgt) {
+  __shared__ float redf[kNW];
+  __shared__ double redd[kNW];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const float *col = logits + (size_t)b * ldl;
+  float m = kNegInf;
+  for (int r = tid; r < V; r += kT) m = fmaxf(m, col[r] + (bias ? bias[r] : 0.f));
+  const double mx = (double)lh::block_max<kNW>(m, redf);
+  double part = 0.0;
+  for (int r = tid; r < V; r += kT) part += exp((double)(col[r] + (bias ? bias[r] : 0.f)) - mx);
+  const double sum = lh::block_sum<kNW>(part, redd);
+  if (tid == 0) {
+    const int t = tgt0[b];
+    if (t >= 0 && t < V) {
+      const float zt = col[t] + (bias ? bias[t] : 0.f);
+      logp_tgt[b] = log(exp((double)zt - mx)) - log(sum);
+    }
+  }
+}
+
+__global__ void masked_sum_kernel(const double *logp_tgt, const int *mask01, int B, double *accum) {
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  double acc = 0.0;
+  for (int b = 0; b < B; ++b)
+    if (mask01[b] == 1) acc += logp_tgt[b];
+  accum[0] += acc;
+}
+
+// ---- fused log-softmax + per-column top-K ---------------------------------------------------
+struct Best {
+  float v;
+  int id;
+};
+__device__ __forceinline__ bool beats(float v1, int i1, float v2, int i2) {
+  return v1 > v2 || (v1 == v2 && i1 < i2);
+}
+__device__ __forceinline__ Best wave_argmax(Best x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(x.v, o, lh::kWave);
+    const int oi = __shfl_xor(x.id, o, lh::kWave);
+    if (beats(ov, oi, x.v, x.id)) {
+      x.v = ov;
+      x.id = oi;
+    }
+  }
+  return x;
+}
+
+constexpr int kIdNone = 0x7fffffff;
+
+template <int NV>
+__global__ __launch_bounds__(kT) void beam_topk_kernel(const float *__restrict__ logits, int ldl,
+                                                       const float *__restrict__ bias, int V, int K,
+                                                       int eof_id, float *__restrict__ cand_logp,
+                                                       int *__restrict__ cand_id,
+                                                       float *__restrict__ logp_eof) {
+  __shared__ float red[kNW];
+  __shared__ float s_v[kNW * LH_BEAM_MAX_K];
+  __shared__ int s_id[kNW * LH_BEAM_MAX_K];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const int wave = tid / lh::kWave, lane = tid % lh::kWave;
+  float4 x[NV];
+  load_column<NV>(x, logits + (size_t)b * ldl, bias, V, tid);
+  const float mx = lh::block_max<kNW>(local_max<NV>(x), red);
+  float part = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+    part += (expf(x[i].x - mx) + expf(x[i].y - mx)) + (expf(x[i].z - mx) + expf(x[i].w - mx));
+  const float lse = logf(lh::block_sum<kNW>(part, red));
+
+  if (eof_id >= 0 && eof_id < V && (eof_id / 4) % kT == tid) {
+    const int i = (eof_id / 4) / kT, c = eof_id % 4;
+    float z = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+      if (k == i) z = comp(x[k], c);
+    logp_eof[b] = (z - mx) - lse;
+  }
+
+  // Stage 1: every wavefront extracts the K best of its 256*NV values, best first.
+  for (int r = 0; r < K; ++r) {
+    Best me{kNegInf, kIdNone};
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int base = (tid + i * kT) * 4;  // ids grow with i and c: strict > keeps the lowest id
+      if (x[i].x > me.v) { me.v = x[i].x; me.id = base; }
+      if (x[i].y > me.v) { me.v = x[i].y; me.id = base + 1; }
+      if (x[i].z > me.v) { me.v = x[i].z; me.id = base + 2; }
+      if (x[i].w > me.v) { me.v = x[i].w; me.id = base + 3; }
+    }
+    const Best w = wave_argmax(me);
+    if (lane == 0) {
+      s_v[wave * K + r] = w.v;
+      s_id[wave * K + r] = w.id;
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int base = (tid + i * kT) * 4;
+      if (base + 0 == w.id) x[i].x = kNegInf;
+      if (base + 1 == w.id) x[i].y = kNegInf;
+      if (base + 2 == w.id) x[i].z = kNegInf;
+      if (base + 3 == w.id) x[i].w = kNegInf;
+    }
+  }
+  __syncthreads();
+
+  // Stage 2: wavefront 0 merges the kNW*K survivors (<= 16 per lane).
+  if (wave == 0) {
+    const int total = kNW * K;
+    float cv[kNW];
+    int ci[kNW];
+#pragma unroll
+    for (int q = 0; q < kNW; ++q) {
+      const int e = lane + q * lh::kWave;
+      cv[q] = e < total ? s_v[e] : kNegInf;
+      ci[q] = e < total ? s_id[e] : kIdNone;
+    }
+    for (int r = 0; r < K; ++r) {
+      Best me{kNegInf, kIdNone};
+#pragma unroll
+      for (int q = 0; q < kNW; ++q)
+        if (beats(cv[q], ci[q], me.v, me.id)) { me.v = cv[q]; me.id = ci[q]; }
+      const Best w = wave_argmax(me);
+      if (lane == 0) {
+        cand_logp[(size_t)b * K + r] = (w.v - mx) - lse;
+        cand_id[(size_t)b * K + r] = w.id;
+      }
+#pragma unroll
+      for (int q = 0; q < kNW; ++q)
+        if (ci[q] == w.id) cv[q] = kNegInf, ci[q] = kIdNone;
+    }
+  }
+}
+
+// Generic fallback for the fused top-K: K sweeps over the column with an exclusion threshold.
+__global__ __launch_bounds__(kT) void beam_topk_generic_kernel(const float *logits, int ldl,
+                                                               const float *bias, int V, int K,
+                                                               int eof_id, float *cand_logp,
+                                                               int *cand_id, float *logp_eof) {
+  __shared__ float red[kNW];
+  __shared__ float s_v[kNW];
+  __shared__ int s_id[kNW];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const int wave = tid / lh::kWave, lane = tid % lh::kWave;
+  const float *col = logits + (size_t)b * ldl;
+  float m = kNegInf;
+  for (int r = tid; r < V; r += kT) m = fmaxf(m, col[r] + (bias ? bias[r] : 0.f));
+  const float mx = lh::block_max<kNW>(m, red);
+  float part = 0.f;
+  for (int r = tid; r < V; r += kT) part += expf(col[r] + (bias ? bias[r] : 0.f) - mx);
+  const float lse = logf(lh::block_sum<kNW>(part, red));
+  if (tid == 0 && eof_id >= 0 && eof_id < V)
+    logp_eof[b] = ((col[eof_id] + (bias ? bias[eof_id] : 0.f)) - mx) - lse;
+  // (pv, pi) = previously selected entry; round r picks the best entry that it beats.
+  float pv = __builtin_huge_valf();
+  int pi = -1;
+  for (int r = 0; r < K; ++r) {
+    Best me{kNegInf, kIdNone};
+    for (int q = tid; q < V; q += kT) {
+      const float z = col[q] + (bias ? bias[q] : 0.f);
+      if (beats(pv, pi, z, q) && beats(z, q, me.v, me.id)) { me.v = z; me.id = q; }
+    }
+    Best w = wave_argmax(me);
+    __syncthreads();
+    if (lane == 0) { s_v[wave] = w.v; s_id[wave] = w.id; }
+    __syncthreads();
+    w.v = s_v[0]; w.id = s_id[0];
+    for (int q = 1; q < kNW; ++q)
+      if (beats(s_v[q], s_id[q], w.v, w.id)) { w.v = s_v[q]; w.id = s_id[q]; }
+    if (tid == 0) {
+      cand_logp[(size_t)b * K + r] = (w.v - mx) - lse;
+      cand_id[(size_t)b * K + r] = w.id;
+    }
+    pv = w.v;
+    pi = w.id;
+  }
+}
+
+int pick_nv(const float *base, int ld, const float *bias, int V) {
+  if (V % 4 != 0 || ld % 4 != 0 || !lh::aligned16(base) || !lh::aligned16(bias)) return 0;
+  for (int nv = 2; nv <= 16; nv *= 2)
+    if (V <= kT * 4 * nv) return nv;
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int lh_softmax_fwd_f32(const float *logits, int ldl, const float *bias, int V, int B,
+                                  float *p, int ldp, lh_stream_t stream) {
+  if (V <= 0 || B <= 0 || !logits || !p || ldl < V || ldp < V)
+    return lh::fail_arg("lh_softmax_fwd_f32: V=%d B=%d ldl=%d ldp=%d or NULL pointer", V, B, ldl,
+                        ldp);
+  hipStream_t st = lh::as_stream(stream);
+  int nv = pick_nv(logits, ldl, bias, V);
+  if (ldp % 4 != 0 || !lh::aligned16(p)) nv = 0;
+  const dim3 grid(B), block(kT);
+  switch (nv) {
+    case 2: hipLaunchKernelGGL(softmax_fwd_kernel<2>, grid, block, 0, st, logits, ldl, bias, V, p, ldp); break;
+    case 4: hipLaunchKernelGGL(softmax_fwd_kernel<4>, grid, block, 0, st, logits, ldl, bias, V, p, ldp); break;
+    case 8: hipLaunchKernelGGL(softmax_fwd_kernel<8>, grid, block, 0, st, logits, ldl, bias, V, p, ldp); break;
+    case 16: hipLaunchKernelGGL(softmax_fwd_kernel<16>, grid, block, 0, st, logits, ldl, bias, V, p, ldp); break;
+    default: hipLaunchKernelGGL(softmax_fwd_generic_kernel, grid, block, 0, st, logits, ldl, bias, V, p, ldp);
+  }
+  return lh::check_launch("lh_softmax_fwd_f32");
+}
+
+extern "C" int lh_train_loglik_f32(const float *p, int ldp, int V, int B, const int *tgt0,
+                                   const int *mask01, double *accum, lh_stream_t stream) {
+  if (V <= 0 || B <= 0 || !p || !tgt0 || !mask01 || !accum || ldp < V)
+    return lh::fail_arg("lh_train_loglik_f32: V=%d B=%d ldp=%d or NULL pointer", V, B, ldp);
+  hipLaunchKernelGGL(train_loglik_kernel, dim3(1), dim3(64), 0, lh::as_stream(stream), p, ldp, B,
+                     tgt0, mask01, accum);
+  return lh::check_launch("lh_train_loglik_f32");
+}
+
+extern "C" int lh_logsoftmax_xent_f32(const float *logits, int ldl, const float *bias, int V, int B,
+                                      const int *tgt0, const int *mask01, double *logp_tgt,
+                                      double *loss_accum, lh_stream_t stream) {
+  if (V <= 0 || B <= 0 || !logits || !tgt0 || !mask01 || !logp_tgt || !loss_accum || ldl < V)
+    return lh::fail_arg("lh_logsoftmax_xent_f32: V=%d B=%d ldl=%d or NULL pointer", V, B, ldl);
+  hipStream_t st = lh::as_stream(stream);
+  const dim3 grid(B), block(kT);
+  switch (pick_nv(logits, ldl, bias, V)) {
+    case 2: hipLaunchKernelGGL(logsoftmax_tgt_kernel<2>, grid, block, 0, st, logits, ldl, bias, V, tgt0, logp_tgt); break;
+    case 4: hipLaunchKernelGGL(logsoftmax_tgt_kernel<4>, grid, block, 0, st, logits, ldl, bias, V, tgt0, logp_tgt); break;
+    case 8: hipLaunchKernelGGL(logsoftmax_tgt_kernel<8>, grid, block, 0, st, logits, ldl, bias, V, tgt0, logp_tgt); break;
+    case 16: hipLaunchKernelGGL(logsoftmax_tgt_kernel<16>, grid, block, 0, st, logits, ldl, bias, V, tgt0, logp_tgt); break;
+    default: hipLaunchKernelGGL(logsoftmax_tgt_generic_kernel, grid, block, 0, st, logits, ldl, bias, V, tgt0, logp_tgt);
+  }
+  int rc = lh::check_launch("lh_logsoftmax_xent_f32");
+  if (rc != LH_OK) return rc;
+  hipLaunchKernelGGL(masked_sum_kernel, dim3(1), dim3(64), 0, st, logp_tgt, mask01, B, loss_accum);
+  return lh::check_launch("lh_logsoftmax_xent_f32 (sum)");
+}
+
+extern "C" int lh_beam_topk_f32(const float *logits, int ldl, const float *bias, int V, int B, int K,
+                                int eof_id, float *cand_logp, int *cand_id, float *logp_eof,
+                                lh_stream_t stream) {
+  if (V <= 0 || B <= 0 || !logits || !cand_logp || !cand_id || !logp_eof || ldl < V)
+    return lh::fail_arg("lh_beam_topk_f32: V=%d B=%d ldl=%d or NULL pointer", V, B, ldl);
+  if (K < 1 || K > LH_BEAM_MAX_K || K > V)
+    return lh::fail_arg("lh_beam_topk_f32: K=%d outside [1,min(%d,V=%d)]", K, LH_BEAM_MAX_K, V);
+  hipStream_t st = lh::as_stream(stream);
+  const dim3 grid(B), block(kT);
+  switch (pick_nv(logits, ldl, bias, V)) {
+    case 2: hipLaunchKernelGGL(beam_topk_kernel<2>, grid, block, 0, st, logits, ldl, bias, V, K, eof_id, cand_logp, cand_id, logp_eof); break;
+    case 4: hipLaunchKernelGGL(beam_topk_kernel<4>, grid, block, 0, st, logits, ldl, bias, V, K, eof_id, cand_logp, cand_id, logp_eof); break;
+    case 8: hipLaunchKernelGGL(beam_topk_kernel<8>, grid, block, 0, st, logits, ldl, bias, V, K, eof_id, cand_logp, cand_id, logp_eof); break;
+    case 16: hipLaunchKernelGGL(beam_topk_kernel<16>, grid, block, 0, st, logits, ldl, bias, V, K, eof_id, cand_logp, cand_id, logp_eof); break;
+    default: hipLaunchKernelGGL(beam_topk_generic_kernel, grid, block, 0, st, logits, ldl, bias, V, K, eof_id, cand_logp, cand_id, logp_eof);
+  }
+  return lh::check_launch("lh_beam_topk_f32");
+}

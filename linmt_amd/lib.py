@@ -1,0 +1,195 @@
+"""ctypes binding of liblinmt_hip.so (the C ABI declared in include/linmt_hip.h).
+
+The library is the product; this module only gives Python (tests, smoke, benchmark) a way to call
+it with device pointers taken from torch tensors.  There is no fallback of any kind: if the built
+library is missing, loading raises, and every wrapper raises on a non-zero status.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblinmt_hip.so")
+
+LH_ACT_NONE = 0
+LH_ACT_TANH = 1
+LH_GEMM_MAX_SEGS = 3
+LH_BEAM_MAX_K = 64
+LH_GATHER_MAX_TENSORS = 24
+
+c_f32p = C.c_void_p  # device pointers travel as plain addresses
+c_i32p = C.c_void_p
+c_f64p = C.c_void_p
+
+
+class GemmSeg(C.Structure):
+    _fields_ = [("A", C.c_void_p), ("lda", C.c_int), ("X", C.c_void_p), ("ldx", C.c_int),
+                ("K", C.c_int)]
+
+
+# name -> (restype, argtypes); mirrors include/linmt_hip.h one to one.
+SIGNATURES = {
+    "lh_abi_version": (C.c_int, []),
+    "lh_last_error": (C.c_char_p, []),
+    "lh_preprocess_indices_i32": (C.c_int, [c_i32p, C.c_int, c_i32p, c_i32p, c_f32p, C.c_void_p]),
+    "lh_setup_reverse_indices_i32": (C.c_int, [c_i32p, C.c_int, c_i32p, C.c_int, C.c_void_p]),
+    "lh_embed_lookup_f32": (C.c_int, [c_f32p, C.c_int, C.c_int, c_i32p, C.c_int, c_f32p,
+                                      C.c_float, c_f32p, C.c_void_p]),
+    "lh_gemm_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int, C.c_int,
+                              C.c_float, C.c_float, c_f32p, C.c_int, c_i32p, c_f32p, C.c_int,
+                              C.c_void_p]),
+    "lh_lstm_cell_fwd_f32": (C.c_int, [C.c_int, C.c_int, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p,
+                                       c_i32p, C.c_int, C.c_float, c_f32p, c_f32p, c_f32p, c_f32p,
+                                       C.c_float, c_f32p, C.c_void_p]),
+    "lh_attn_core_fwd_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, c_f32p, c_f32p,
+                                       c_f32p, c_f32p, C.c_longlong, C.c_longlong, c_i32p, c_i32p,
+                                       c_i32p, c_f32p, c_f32p, c_i32p, c_f32p, c_f32p, c_f32p,
+                                       c_i32p, C.c_void_p]),
+    "lh_softmax_fwd_f32": (C.c_int, [c_f32p, C.c_int, c_f32p, C.c_int, C.c_int, c_f32p, C.c_int,
+                                     C.c_void_p]),
+    "lh_train_loglik_f32": (C.c_int, [c_f32p, C.c_int, C.c_int, C.c_int, c_i32p, c_i32p, c_f64p,
+                                      C.c_void_p]),
+    "lh_logsoftmax_xent_f32": (C.c_int, [c_f32p, C.c_int, c_f32p, C.c_int, C.c_int, c_i32p, c_i32p,
+                                         c_f64p, c_f64p, C.c_void_p]),
+    "lh_beam_topk_f32": (C.c_int, [c_f32p, C.c_int, c_f32p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                   c_f32p, c_i32p, c_f32p, C.c_void_p]),
+    "lh_beam_merge_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, c_i32p, c_f32p, c_i32p,
+                                    c_f32p, c_f32p, C.c_float, C.c_float, C.c_int, C.c_int, c_i32p,
+                                    c_i32p, c_f32p, c_i32p, c_i32p, c_f32p, C.c_void_p]),
+    "lh_beam_gather_f32": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int,
+                                     C.c_int, C.c_int, c_i32p, C.c_void_p]),
+}
+
+_lib = None
+
+
+class LinmtHipError(RuntimeError):
+    pass
+
+
+def load():
+    """Loads liblinmt_hip.so and checks that it exports every declared entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise LinmtHipError(
+            f"{LIB_PATH} is missing: build it with `make -C linmt_amd/csrc` "
+            "(or __graft_entry__.build()); there is no CPU fallback")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def _ptr(t):
+    """Device (or host) address of a torch tensor / None."""
+    if t is None:
+        return None
+    return C.c_void_p(t.data_ptr())
+
+
+def check(status, what):
+    if status != 0:
+        msg = load().lh_last_error().decode("utf-8", "replace")
+        raise LinmtHipError(f"{what} failed with status {status}: {msg}")
+
+
+def _stream(stream):
+    if stream is None:
+        import torch
+        return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return C.c_void_p(stream)
+
+
+# ---- thin wrappers over torch tensors (column-major data lives in whatever tensor holds it) ------
+def preprocess_indices(idx, idx0, mask01, mask01_f=None, stream=None):
+    check(load().lh_preprocess_indices_i32(_ptr(idx), idx.numel(), _ptr(idx0), _ptr(mask01),
+                                           _ptr(mask01_f), _stream(stream)),
+          "lh_preprocess_indices_i32")
+
+
+def setup_reverse_indices(unique, rev, vocab, stream=None):
+    check(load().lh_setup_reverse_indices_i32(_ptr(unique), unique.numel(), _ptr(rev), vocab,
+                                              _stream(stream)), "lh_setup_reverse_indices_i32")
+
+
+def embed_lookup(W, E, V, idx0, B, out, drop_mask=None, keep=1.0, stream=None):
+    check(load().lh_embed_lookup_f32(_ptr(W), E, V, _ptr(idx0), B, _ptr(drop_mask), keep,
+                                     _ptr(out), _stream(stream)), "lh_embed_lookup_f32")
+
+
+def gemm(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0, bias=None,
+         act=LH_ACT_NONE, colmask=None, stream=None):
+    """segs: list of (A, lda, X, ldx, K) with torch tensors A, X."""
+    arr = (GemmSeg * len(segs))()
+    for i, (A, lda, X, ldx, K) in enumerate(segs):
+        arr[i].A = A.data_ptr()
+        arr[i].lda = lda
+        arr[i].X = X.data_ptr()
+        arr[i].ldx = ldx
+        arr[i].K = K
+    check(load().lh_gemm_f32(M, N, arr, len(segs), int(transA), int(transX), alpha, beta,
+                             _ptr(bias), act, _ptr(colmask), _ptr(C_out), ldc, _stream(stream)),
+          "lh_gemm_f32")
+
+
+def lstm_cell_fwd(H, B, pre1, bias4h, c_prev, mask01, c, h, pre2=None, pre3=None,
+                  sigmoid_f64=False, cell_clip=0.0, gates=None, next_drop_mask=None, keep=1.0,
+                  h_drop=None, stream=None):
+    check(load().lh_lstm_cell_fwd_f32(H, B, _ptr(pre1), _ptr(pre2), _ptr(pre3), _ptr(bias4h),
+                                      _ptr(c_prev), _ptr(mask01), int(sigmoid_f64), cell_clip,
+                                      _ptr(gates), _ptr(c), _ptr(h), _ptr(next_drop_mask), keep,
+                                      _ptr(h_drop), _stream(stream)), "lh_lstm_cell_fwd_f32")
+
+
+def attn_core_fwd(H, B, D, max_len, hs_steps, tanh1, v_p, wa, hs, hs_step_stride, hs_col_stride,
+                  hs_col, batch_info, mask01, p_t, sigma, indices, align, cached_exp, ctx,
+                  viterbi=None, stream=None):
+    check(load().lh_attn_core_fwd_f32(H, B, D, max_len, hs_steps, _ptr(tanh1), _ptr(v_p), _ptr(wa),
+                                      _ptr(hs), hs_step_stride, hs_col_stride, _ptr(hs_col),
+                                      _ptr(batch_info), _ptr(mask01), _ptr(p_t), _ptr(sigma),
+                                      _ptr(indices), _ptr(align), _ptr(cached_exp), _ptr(ctx),
+                                      _ptr(viterbi), _stream(stream)), "lh_attn_core_fwd_f32")
+
+
+def softmax_fwd(logits, ldl, bias, V, B, p, ldp, stream=None):
+    check(load().lh_softmax_fwd_f32(_ptr(logits), ldl, _ptr(bias), V, B, _ptr(p), ldp,
+                                    _stream(stream)), "lh_softmax_fwd_f32")
+
+
+def train_loglik(p, ldp, V, B, tgt0, mask01, accum, stream=None):
+    check(load().lh_train_loglik_f32(_ptr(p), ldp, V, B, _ptr(tgt0), _ptr(mask01), _ptr(accum),
+                                     _stream(stream)), "lh_train_loglik_f32")
+
+
+def logsoftmax_xent(logits, ldl, bias, V, B, tgt0, mask01, logp_tgt, loss_accum, stream=None):
+    check(load().lh_logsoftmax_xent_f32(_ptr(logits), ldl, _ptr(bias), V, B, _ptr(tgt0),
+                                        _ptr(mask01), _ptr(logp_tgt), _ptr(loss_accum),
+                                        _stream(stream)), "lh_logsoftmax_xent_f32")
+
+
+def beam_topk(logits, ldl, bias, V, B, K, eof_id, cand_logp, cand_id, logp_eof, stream=None):
+    check(load().lh_beam_topk_f32(_ptr(logits), ldl, _ptr(bias), V, B, K, eof_id, _ptr(cand_logp),
+                                  _ptr(cand_id), _ptr(logp_eof), _stream(stream)),
+          "lh_beam_topk_f32")
+
+
+def beam_merge(n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof, prev_score, diversity,
+               penalty, start_id, eof_id, tok, backptr, score, fin_count, fin_beam, fin_score,
+               stream=None):
+    check(load().lh_beam_merge_f32(n_sent, beam, K, step, _ptr(limit), _ptr(cand_logp),
+                                   _ptr(cand_id), _ptr(logp_eof), _ptr(prev_score), diversity,
+                                   penalty, start_id, eof_id, _ptr(tok), _ptr(backptr),
+                                   _ptr(score), _ptr(fin_count), _ptr(fin_beam), _ptr(fin_score),
+                                   _stream(stream)), "lh_beam_merge_f32")
+
+
+def beam_gather(src, dst, H, B, backptr, stream=None):
+    n = len(src)
+    s = (C.c_void_p * n)(*[t.data_ptr() for t in src])
+    d = (C.c_void_p * n)(*[t.data_ptr() for t in dst])
+    check(load().lh_beam_gather_f32(s, d, n, H, B, _ptr(backptr), _stream(stream)),
+          "lh_beam_gather_f32")

@@ -1,0 +1,117 @@
+/*
+ * CPU oracle for the LiNMT per-timestep LSTM / attention / softmax / beam path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This is a host restatement of the reference's CUDA kernels and host
+ * beam search, written from its sources (each function cites the file:line it follows).  Only the
+ * tests, the smoke check and the cpu_baseline leg of the benchmark may load it; the product path
+ * (liblinmt_hip.so and the C++ layer classes) never calls into it.
+ *
+ * Layout conventions are the reference's: column-major, activations H x B, int32 ids, -1 padding.
+ *
+ * Parity pins (what fixes each function besides this restatement) are listed next to the
+ * functions in linmt_oracle.cpp; functions that only our reading of the source pins say so.
+ */
+#ifndef LINMT_ORACLE_H_
+#define LINMT_ORACLE_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- elementwise / lookup ------------------------------------------------------------------ */
+void orc_preprocess_indices(const int *idx, int n, int *idx0, int *mask01, float *mask01_f);
+void orc_setup_reverse_indices(const int *unique, int n_unique, int *rev);
+void orc_embed_lookup(const float *W, int E, int V, const int *idx0, int B, const float *drop_mask,
+                      float keep, float *out);
+void orc_dropout(float *x, const float *mask, float keep, long long n);
+
+/* C = alpha * op(A) op(X) + beta * C, fp32 accumulation (column-major, flags as in cuBLAS). */
+void orc_gemm(int M, int N, int K, const float *A, int lda, int transA, const float *X, int ldx,
+              int transX, float alpha, float beta, float *C, int ldc);
+
+/* LSTM cell, stacked 4H x B pre-activations (rows i,f,g,o); feed != 0 selects the kernels of the
+ * feed-input branch (double-precision sigmoid). */
+void orc_lstm_cell_fwd(int H, int B, const float *pre1, const float *pre2, const float *pre3,
+                       const float *bias4h, const float *c_prev, const int *mask01, int feed,
+                       float cell_clip, float *gates, float *c, float *h);
+
+/* Attention core with the argument meaning of lh_attn_core_fwd_f32. */
+void orc_attn_core_fwd(int H, int B, int D, int max_len, int hs_steps, const float *tanh1,
+                       const float *v_p, const float *wa, const float *hs,
+                       long long hs_step_stride, long long hs_col_stride, const int *hs_col,
+                       const int *batch_info, const int *mask01, float *p_t, float *sigma,
+                       int *indices, float *align, float *cached_exp, float *ctx, int *viterbi);
+
+/* Whole attention node forward (dropout excluded: ha = h_t). Writes h_tild (H x B); the other
+ * outputs may be NULL. Scratch is allocated inside. */
+void orc_attn_node_fwd(int H, int B, int D, int max_len, int hs_steps, const float *h_t,
+                       const float *W_a, const float *W_p, const float *v_p, const float *b_out,
+                       const float *W_c1, const float *W_c2, const float *hs,
+                       long long hs_step_stride, long long hs_col_stride, const int *hs_col,
+                       const int *batch_info, const int *mask01, float *h_tild, float *p_t,
+                       int *indices, float *align, float *ctx);
+
+/* ---- softmax / loss -------------------------------------------------------------------------- */
+void orc_softmax_fwd(const float *logits, int ldl, const float *bias, int V, int B, float *p,
+                     int ldp);
+void orc_train_loglik(const float *p, int ldp, int V, int B, const int *tgt0, const int *mask01,
+                      double *accum);
+void orc_logsoftmax_xent(const float *logits, int ldl, const float *bias, int V, int B,
+                         const int *tgt0, const int *mask01, double *logp_tgt, double *loss_accum);
+
+/* ---- beam ------------------------------------------------------------------------------------ */
+/* One ExpandHypothesis call for one sentence, from the V x beam probability matrix p (column-major),
+ * including the host renormalisation of EnsemblesModels (one model).  Outputs as lh_beam_merge_f32
+ * (backptr is the LOCAL beam column here). */
+void orc_beam_expand(const float *p, int V, int beam, int step, const float *prev_score,
+                     float diversity, float penalty, int start_id, int eof_id, int *tok,
+                     int *backptr, float *score, int *fin_count, int *fin_beam, float *fin_score);
+void orc_beam_gather(const float *src, float *dst, int H, int B, const int *backptr);
+
+/* ---- whole model ----------------------------------------------------------------------------- */
+typedef struct orc_model_config {
+  int layers;        /* LSTM layers per side */
+  int H;             /* lstm_size == embedding size */
+  int V_src, V_tgt;
+  int attention;     /* 0 none, 1 local-p, 2 global-general (build-defined) */
+  int D;             /* attention window half-width */
+  int feed_input;
+  int longest_sent;  /* longest_sentence_ of the reference (already including its +4) */
+} orc_model_config;
+
+typedef struct orc_model orc_model;
+orc_model *orc_model_create(const orc_model_config *cfg);
+void orc_model_destroy(orc_model *m);
+/* Host pointer to a parameter, reference names: "src.0.W", "src.0.M_i", "src.1.W_hi", "tgt.0.Q_c",
+ * "tgt.0.b_f", "attn.W_a", "attn.v_p", "attn.b_out", "attn.W_c1", "softmax.D", "softmax.b_d" ...;
+ * *n_elems receives the element count.  NULL if the name is unknown. */
+float *orc_model_param(orc_model *m, const char *name, long long *n_elems);
+/* Must be called after parameters were written (refreshes cached transposes). */
+void orc_model_commit(orc_model *m);
+
+typedef struct orc_decode_opts {
+  int beam;
+  float max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta;
+  int num_threads; /* 0 = leave OpenMP default */
+} orc_decode_opts;
+
+/* Beam-decodes ONE sentence the way EnsembleFactory::DecodeFile does (src_ids in ORIGINAL order,
+ * the function reverses them like the preprocessing does).  best_tokens receives the 1-best without
+ * <START>/<EOF> (capacity cap), *best_len its length, *best_score its rescored value.  If
+ * hyp_tokens != NULL it receives every finished hypothesis (row-major, hyp_cap rows x cap tokens,
+ * including <START>/<EOF>), hyp_len / hyp_score their lengths and RAW scores, *n_hyp the count.
+ * Returns the number of target steps that were run (forward passes of the decoder). */
+int orc_decode_sentence(orc_model *m, const int *src_ids, int S, const orc_decode_opts *o,
+                        int *best_tokens, int cap, int *best_len, float *best_score,
+                        int *hyp_tokens, int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp);
+
+/* Teacher-forced forward + cross-entropy (GetError): src B x S and tgt_in/tgt_out B x T, all
+ * column-major with -1 padding (source reversed + left-padded, target right-padded).
+ * Returns sum over non-pad target positions of log p(target) (natural log, double). */
+double orc_forward_xent(orc_model *m, const int *src, int S, const int *tgt_in, const int *tgt_out,
+                        int T, int B, const int *batch_info, int num_threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

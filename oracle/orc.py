@@ -1,0 +1,265 @@
+"""numpy binding of the CPU oracle (oracle/liblinmt_oracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the cpu_baseline
+leg of bench.py as the checker / reported baseline.  Nothing under linmt_amd/ imports this.
+All arrays are numpy, column-major data is passed as Fortran-ordered 2-D arrays (or flat arrays
+holding the column-major data).
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblinmt_oracle.so")
+_lib = None
+
+
+def build():
+    subprocess.check_call(["make", "-C", _HERE, "-s"])
+
+
+class ModelConfig(C.Structure):
+    _fields_ = [("layers", C.c_int), ("H", C.c_int), ("V_src", C.c_int), ("V_tgt", C.c_int),
+                ("attention", C.c_int), ("D", C.c_int), ("feed_input", C.c_int),
+                ("longest_sent", C.c_int)]
+
+
+class DecodeOpts(C.Structure):
+    _fields_ = [("beam", C.c_int), ("max_ratio", C.c_float), ("min_ratio", C.c_float),
+                ("penalty", C.c_float), ("diversity", C.c_float), ("lp_alpha", C.c_float),
+                ("cp_beta", C.c_float), ("num_threads", C.c_int)]
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        _lib = C.CDLL(LIB_PATH)
+        _lib.orc_model_create.restype = C.c_void_p
+        _lib.orc_model_param.restype = C.c_void_p
+        _lib.orc_forward_xent.restype = C.c_double
+        _lib.orc_decode_sentence.restype = C.c_int
+    return _lib
+
+
+def _p(a):
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"] or a.flags["F_CONTIGUOUS"], "oracle arrays must be contiguous"
+    # data_as() keeps a reference to the array, so temporaries made in the argument list stay alive
+    # until the foreign call has returned.
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _f(v):
+    return C.c_float(v)
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def preprocess_indices(idx):
+    idx = i32(idx).ravel()
+    idx0 = np.empty_like(idx)
+    m = np.empty_like(idx)
+    mf = np.empty(idx.shape, np.float32)
+    lib().orc_preprocess_indices(_p(idx), idx.size, _p(idx0), _p(m), _p(mf))
+    return idx0, m, mf
+
+
+def setup_reverse_indices(unique, vocab):
+    unique = i32(unique)
+    rev = np.full(vocab, -7, np.int32)
+    lib().orc_setup_reverse_indices(_p(unique), unique.size, _p(rev))
+    return rev
+
+
+def embed_lookup(W, idx0, drop_mask=None, keep=1.0):
+    """W: (E,V) Fortran; returns (E,B) Fortran."""
+    E, V = W.shape
+    W = np.asfortranarray(W, np.float32)
+    idx0 = i32(idx0)
+    out = np.empty((E, idx0.size), np.float32, order="F")
+    dm = None if drop_mask is None else np.asfortranarray(drop_mask, np.float32)
+    lib().orc_embed_lookup(_p(W), E, V, _p(idx0), idx0.size, _p(dm), _f(keep), _p(out))
+    return out
+
+
+def gemm(A, X, transA=False, transX=False, alpha=1.0, beta=0.0, C0=None):
+    A = np.asfortranarray(A, np.float32)
+    X = np.asfortranarray(X, np.float32)
+    M, K = (A.shape[1], A.shape[0]) if transA else A.shape
+    N = X.shape[0] if transX else X.shape[1]
+    out = np.zeros((M, N), np.float32, order="F") if C0 is None else np.asfortranarray(
+        C0, np.float32).copy(order="F")
+    lib().orc_gemm(M, N, K, _p(A), A.shape[0], int(transA), _p(X), X.shape[0], int(transX),
+                   _f(alpha), _f(beta), _p(out), M)
+    return out
+
+
+def lstm_cell_fwd(pre1, bias4h, c_prev, mask01, pre2=None, pre3=None, feed=False, cell_clip=0.0):
+    """pre*: (4H,B) Fortran; returns gates (4H,B), c (H,B), h (H,B)."""
+    H4, B = pre1.shape
+    H = H4 // 4
+    fa = lambda a: None if a is None else np.asfortranarray(a, np.float32)
+    pre1, pre2, pre3, c_prev = fa(pre1), fa(pre2), fa(pre3), fa(c_prev)
+    gates = np.empty((H4, B), np.float32, order="F")
+    c = np.empty((H, B), np.float32, order="F")
+    h = np.empty((H, B), np.float32, order="F")
+    lib().orc_lstm_cell_fwd(H, B, _p(pre1), _p(pre2), _p(pre3), _p(f32(bias4h)), _p(c_prev),
+                            _p(i32(mask01)), int(feed), _f(cell_clip), _p(gates), _p(c), _p(h))
+    return gates, c, h
+
+
+def attn_core_fwd(H, B, D, max_len, hs_steps, tanh1, v_p, wa, hs, step_stride, col_stride, hs_col,
+                  batch_info, mask01):
+    W = 2 * D + 1 if D >= 0 else max_len
+    out = dict(p_t=np.zeros(B, np.float32), sigma=np.zeros(B, np.float32),
+               indices=np.empty((B, W), np.int32, order="F"),
+               align=np.empty((B, W), np.float32, order="F"),
+               cached_exp=np.empty((W, B), np.float32, order="F"),
+               ctx=np.empty((H, B), np.float32, order="F"), viterbi=np.empty(B, np.int32))
+    fa = lambda a: None if a is None else np.asfortranarray(a, np.float32)
+    lib().orc_attn_core_fwd(H, B, D, max_len, hs_steps, _p(fa(tanh1)), _p(None if v_p is None else f32(v_p)),
+                            _p(fa(wa)), _p(f32(hs)), C.c_longlong(step_stride),
+                            C.c_longlong(col_stride), _p(None if hs_col is None else i32(hs_col)),
+                            _p(i32(batch_info)), _p(i32(mask01)), _p(out["p_t"]), _p(out["sigma"]),
+                            _p(out["indices"]), _p(out["align"]), _p(out["cached_exp"]),
+                            _p(out["ctx"]), _p(out["viterbi"]))
+    return out
+
+
+def attn_node_fwd(H, B, D, max_len, hs_steps, h_t, W_a, W_p, v_p, b_out, W_c1, W_c2, hs,
+                  step_stride, col_stride, hs_col, batch_info, mask01):
+    W = 2 * D + 1 if D >= 0 else max_len
+    fa = lambda a: None if a is None else np.asfortranarray(a, np.float32)
+    out = dict(h_tild=np.empty((H, B), np.float32, order="F"), p_t=np.zeros(B, np.float32),
+               indices=np.empty((B, W), np.int32, order="F"),
+               align=np.empty((B, W), np.float32, order="F"),
+               ctx=np.empty((H, B), np.float32, order="F"))
+    lib().orc_attn_node_fwd(H, B, D, max_len, hs_steps, _p(fa(h_t)), _p(fa(W_a)), _p(fa(W_p)),
+                            _p(None if v_p is None else f32(v_p)), _p(f32(b_out)), _p(fa(W_c1)),
+                            _p(fa(W_c2)), _p(f32(hs)), C.c_longlong(step_stride),
+                            C.c_longlong(col_stride), _p(None if hs_col is None else i32(hs_col)),
+                            _p(i32(batch_info)), _p(i32(mask01)), _p(out["h_tild"]), _p(out["p_t"]),
+                            _p(out["indices"]), _p(out["align"]), _p(out["ctx"]))
+    return out
+
+
+def softmax_fwd(logits, bias=None):
+    logits = np.asfortranarray(logits, np.float32)
+    V, B = logits.shape
+    p = np.empty((V, B), np.float32, order="F")
+    lib().orc_softmax_fwd(_p(logits), V, _p(None if bias is None else f32(bias)), V, B, _p(p), V)
+    return p
+
+
+def train_loglik(p, tgt0, mask01, accum=0.0):
+    p = np.asfortranarray(p, np.float32)
+    V, B = p.shape
+    acc = np.array([accum], np.float64)
+    lib().orc_train_loglik(_p(p), V, V, B, _p(i32(tgt0)), _p(i32(mask01)), _p(acc))
+    return float(acc[0])
+
+
+def logsoftmax_xent(logits, bias, tgt0, mask01):
+    logits = np.asfortranarray(logits, np.float32)
+    V, B = logits.shape
+    lp = np.empty(B, np.float64)
+    acc = np.zeros(1, np.float64)
+    lib().orc_logsoftmax_xent(_p(logits), V, _p(None if bias is None else f32(bias)), V, B,
+                              _p(i32(tgt0)), _p(i32(mask01)), _p(lp), _p(acc))
+    return lp, float(acc[0])
+
+
+def beam_expand(p, step, prev_score, diversity=0.0, penalty=0.0, start_id=0, eof_id=1):
+    """p: (V, beam) Fortran probabilities.  Returns dict(tok, backptr, score, fin_beam, fin_score)."""
+    p = np.asfortranarray(p, np.float32)
+    V, beam = p.shape
+    tok = np.empty(beam, np.int32)
+    bp = np.empty(beam, np.int32)
+    sc = np.empty(beam, np.float32)
+    fc = np.zeros(1, np.int32)
+    fb = np.zeros(max(beam, 1) * 2 + 4, np.int32)
+    fs = np.zeros(max(beam, 1) * 2 + 4, np.float32)
+    lib().orc_beam_expand(_p(p), V, beam, step, _p(f32(prev_score)), _f(diversity), _f(penalty),
+                          start_id, eof_id, _p(tok), _p(bp), _p(sc), _p(fc), _p(fb), _p(fs))
+    n = int(fc[0])
+    return dict(tok=tok, backptr=bp, score=sc, fin_beam=fb[:n].copy(), fin_score=fs[:n].copy())
+
+
+def beam_gather(src, backptr):
+    src = np.asfortranarray(src, np.float32)
+    H, B = src.shape
+    dst = np.empty((H, B), np.float32, order="F")
+    lib().orc_beam_gather(_p(src), _p(dst), H, B, _p(i32(backptr)))
+    return dst
+
+
+class Model:
+    """Host model of the oracle; parameters are numpy views into the oracle's own buffers."""
+
+    def __init__(self, layers, H, V_src, V_tgt, attention=1, D=10, feed_input=1, longest_sent=104):
+        self.cfg = ModelConfig(layers, H, V_src, V_tgt, attention, D, feed_input, longest_sent)
+        self.handle = C.c_void_p(lib().orc_model_create(C.byref(self.cfg)))
+
+    def param(self, name):
+        n = C.c_longlong(0)
+        ptr = lib().orc_model_param(self.handle, name.encode(), C.byref(n))
+        if not ptr:
+            raise KeyError(name)
+        buf = (C.c_float * n.value).from_address(ptr)
+        return np.frombuffer(buf, dtype=np.float32)
+
+    def set_params(self, params):
+        for name, arr in params.items():
+            dst = self.param(name)
+            src = np.asarray(arr, np.float32)
+            assert src.size == dst.size, (name, src.shape, dst.size)
+            dst[:] = src.ravel(order="F")
+        lib().orc_model_commit(self.handle)
+
+    def decode_sentence(self, src_ids, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0,
+                        diversity=0.0, lp_alpha=0.65, cp_beta=0.20, num_threads=0, hyp_cap=4096):
+        src_ids = i32(src_ids)
+        cap = self.cfg.longest_sent + 2
+        o = DecodeOpts(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta,
+                       num_threads)
+        best = np.zeros(cap, np.int32)
+        blen = C.c_int(0)
+        bscore = C.c_float(0)
+        ht = np.zeros((hyp_cap, cap), np.int32)
+        hl = np.zeros(hyp_cap, np.int32)
+        hs = np.zeros(hyp_cap, np.float32)
+        nh = C.c_int(0)
+        steps = lib().orc_decode_sentence(self.handle, _p(src_ids), src_ids.size, C.byref(o),
+                                          _p(best), cap, C.byref(blen), C.byref(bscore), _p(ht),
+                                          _p(hl), _p(hs), hyp_cap, C.byref(nh))
+        n = min(nh.value, hyp_cap)
+        hyps = [(ht[i, :hl[i]].copy(), float(hs[i])) for i in range(n)]
+        return dict(best=best[:blen.value].copy(), best_score=float(bscore.value), hyps=hyps,
+                    steps=steps)
+
+    def forward_xent(self, src, tgt_in, tgt_out, batch_info, num_threads=0):
+        """src (B,S), tgt_in/tgt_out (B,T) int arrays with -1 padding (column t = timestep t)."""
+        src = np.asfortranarray(src, np.int32)
+        tgt_in = np.asfortranarray(tgt_in, np.int32)
+        tgt_out = np.asfortranarray(tgt_out, np.int32)
+        B, S = src.shape
+        T = tgt_in.shape[1]
+        return lib().orc_forward_xent(self.handle, _p(src), S, _p(tgt_in), _p(tgt_out), T, B,
+                                      _p(i32(batch_info)), num_threads)
+
+    def __del__(self):
+        try:
+            lib().orc_model_destroy(self.handle)
+        except Exception:
+            pass

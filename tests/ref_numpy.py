@@ -1,0 +1,202 @@
+"""Independent float64 numpy statement of the model mathematics (textbook LSTM, Luong attention,
+softmax, sort-based beam search).  It shares no code with the oracle: it exists to pin the oracle
+(tests/test_oracle_pins.py) -- a dropped term, a wrong gate order or a transposed weight in the
+oracle shows up as a mismatch here."""
+import numpy as np
+
+GATES = ["i", "f", "c", "o"]
+
+
+def sigmoid(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+def make_params(rng, layers, H, V_src, V_tgt, attention=True, feed_input=True, scale=0.08):
+    """Reference initialisation: uniform[-scale, scale], forget-gate bias 1
+    (src/utility_cu.cu:77-78, src/layer_input_to_hidden.h:651-655)."""
+    P = {}
+
+    def u(*shape):
+        return rng.uniform(-scale, scale, size=shape).astype(np.float32)
+
+    for side, V in (("src", V_src), ("tgt", V_tgt)):
+        for l in range(layers):
+            pfx = f"{side}.{l}."
+            for g in GATES:
+                P[pfx + "W_h" + g] = u(H, H)
+                P[pfx + "M_" + g] = u(H, H)
+                P[pfx + "b_" + g] = u(H)
+                if side == "tgt" and l == 0 and attention and feed_input:
+                    P[pfx + "Q_" + g] = u(H, H)
+            P[pfx + "b_f"] = np.ones(H, np.float32)
+            if l == 0:
+                P[pfx + "W"] = u(H, V)
+    if attention:
+        for n in ("W_a", "W_p", "W_c1", "W_c2"):
+            P["attn." + n] = u(H, H)
+        P["attn.v_p"] = u(H)
+        P["attn.b_out"] = u(H)
+    P["softmax.D"] = u(V_tgt, H)
+    P["softmax.b_d"] = u(V_tgt)
+    return P
+
+
+def lstm_step(P, pfx, x, h, c, h_tild=None, mask=None):
+    P = {k: v.astype(np.float64) for k, v in P.items() if k.startswith(pfx)}
+    s = {}
+    for g in GATES:
+        v = P[pfx + "M_" + g] @ x + P[pfx + "W_h" + g] @ h + P[pfx + "b_" + g][:, None]
+        if h_tild is not None:
+            v = v + P[pfx + "Q_" + g] @ h_tild
+        s[g] = v
+    i, f, o, g = sigmoid(s["i"]), sigmoid(s["f"]), sigmoid(s["o"]), np.tanh(s["c"])
+    c_new = f * c + i * g
+    h_new = o * np.tanh(c_new)
+    if mask is not None:
+        c_new = c_new * mask[None, :]
+        h_new = h_new * mask[None, :]
+    return h_new, c_new, (i, f, g, o)
+
+
+def attention_local_p(P, h_t, hs_of, lens, mask, D):
+    """hs_of(b, pos) -> encoder top state (H,) of ORIGINAL source position pos of column b."""
+    H, B = h_t.shape
+    Wp, Wa = P["attn.W_p"].astype(np.float64), P["attn.W_a"].astype(np.float64)
+    Wc1, Wc2 = P["attn.W_c1"].astype(np.float64), P["attn.W_c2"].astype(np.float64)
+    vp, bo = P["attn.v_p"].astype(np.float64), P["attn.b_out"].astype(np.float64)
+    out = np.zeros((H, B))
+    aligns = []
+    for b in range(B):
+        ha = h_t[:, b]
+        p = lens[b] * sigmoid(vp @ np.tanh(Wp @ ha))
+        # window on the fp32 position the kernels truncate
+        pf = np.float32(lens[b]) * np.float32(sigmoid(vp @ np.tanh(Wp @ ha)))
+        lo = max(0, int(pf) - D) if D >= 0 else 0
+        hi = min(lens[b] - 1, int(pf) + D) if D >= 0 else lens[b] - 1
+        pos = list(range(lo, hi + 1))[: (2 * D + 1) if D >= 0 else None]
+        ctx = np.zeros(H)
+        a_full = {}
+        if mask[b] == 1 and pos:
+            hs = np.stack([hs_of(b, s) for s in pos], axis=1)  # H x n
+            sc = ha @ Wa @ hs
+            e = np.exp(sc - sc.max())
+            a = e / e.sum()
+            if D >= 0:
+                a = a * np.exp(-((p - np.array(pos)) ** 2) / (2 * (D * D / 4.0)))
+            ctx = hs @ a
+            a_full = dict(zip(pos, a))
+        out[:, b] = np.tanh(Wc1 @ ctx + Wc2 @ ha + bo) * mask[b]
+        aligns.append(a_full)
+    return out, aligns
+
+
+def log_softmax(z):
+    z = z - z.max(axis=0, keepdims=True)
+    return z - np.log(np.exp(z).sum(axis=0, keepdims=True))
+
+
+def encode(P, layers, H, src_ids):
+    """Single sentence: returns per-layer final (h,c) and the top states by ORIGINAL position."""
+    S = len(src_ids)
+    h = [np.zeros((H, 1)) for _ in range(layers)]
+    c = [np.zeros((H, 1)) for _ in range(layers)]
+    top = {}
+    for t in range(S):
+        pos = S - 1 - t  # the source is fed reversed
+        x = P["src.0.W"].astype(np.float64)[:, [src_ids[pos]]]
+        for l in range(layers):
+            h[l], c[l], _ = lstm_step(P, f"src.{l}.", x, h[l], c[l])
+            x = h[l]
+        top[pos] = h[layers - 1][:, 0].copy()
+    return h, c, top
+
+
+def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=True, max_ratio=1.5,
+                min_ratio=0.5, penalty=0.0, diversity=0.0, lp_alpha=0.65, cp_beta=0.2,
+                longest=104, margins=None):
+    """Sort-based beam search with the reference's rules (src/decoder.h:355-699).  Returns
+    (best_tokens, best_score, hyps); margins (list) collects the smallest score gaps seen, so a test
+    can skip seeds whose decisions are closer than fp32 can resolve."""
+    S = len(src_ids)
+    beam = min(beam, int(np.sqrt(V)))
+    he, ce, top = encode(P, layers, H, src_ids)
+    h = [np.repeat(he[l], beam, axis=1) for l in range(layers)]
+    c = [np.repeat(ce[l], beam, axis=1) for l in range(layers)]
+    h_tild = np.zeros((H, beam))
+    tokens = np.zeros(beam, int)
+    scores = np.zeros(beam)
+    hist = [[0] for _ in range(beam)]
+    hyps = []
+    D64 = P["softmax.D"].astype(np.float64)
+    bd = P["softmax.b_d"].astype(np.float64)
+    Wt = P["tgt.0.W"].astype(np.float64)
+    ones = np.ones(beam, int)
+    limit = min(int(np.float32(max_ratio) * S), longest - 2)
+
+    def forward(step):
+        nonlocal h, c
+        x = Wt[:, tokens]
+        nh, nc = [], []
+        for l in range(layers):
+            ht = h_tild if (l == 0 and feed_input and attention and step != 0) else None
+            a, b_, _ = lstm_step(P, f"tgt.{l}.", x, h[l], c[l], ht)
+            nh.append(a)
+            nc.append(b_)
+            x = a
+        topv = x
+        ht_new = None
+        if attention:
+            ht_new, _ = attention_local_p(P, topv, lambda b, s: top[s], [S] * beam, ones, D)
+            topv = ht_new
+        return nh, nc, ht_new, log_softmax(D64 @ topv + bd[:, None])
+
+    for step in range(limit):
+        nh, nc, ht_new, lp = forward(step)
+        cands = []
+        for i in range(1 if step == 0 else beam):
+            order = np.lexsort((np.arange(V), -lp[:, i]))[: beam + 1]
+            if margins is not None:
+                full = np.sort(lp[:, i])[::-1]
+                margins.append(full[beam] - full[beam + 1])
+            for rank, v in enumerate(order):
+                cands.append((lp[v, i] + scores[i] - (rank + 1) * diversity, i, int(v)))
+        cands.sort(key=lambda t: (-t[0], t[1], t[2]))
+        if margins is not None:
+            sc = np.array([t[0] for t in cands])
+            margins.append(np.min(sc[:-1] - sc[1:]))
+        new_tok, new_bp, new_sc = [], [], []
+        for s_, i, v in cands:
+            if len(new_tok) == beam:
+                break
+            if v == 0:
+                continue
+            if v == 1:
+                hyps.append((hist[i] + [1], s_ + penalty))
+                continue
+            new_tok.append(v)
+            new_bp.append(i)
+            new_sc.append(s_ + penalty)
+        assert len(new_tok) == beam
+        hist = [hist[i] + [v] for i, v in zip(new_bp, new_tok)]
+        tokens = np.array(new_tok)
+        scores = np.array(new_sc)
+        h = [x[:, new_bp] for x in nh]
+        c = [x[:, new_bp] for x in nc]
+        if attention:
+            h_tild = ht_new[:, new_bp]
+    _, _, _, lp = forward(limit if limit > 0 else 1)
+    for i in range(beam):
+        hyps.append((hist[i] + [1], scores[i] + lp[1, i] + penalty))
+
+    best, best_s = None, None
+    for toks, s_ in hyps:
+        n = len(toks)
+        r = s_
+        if lp_alpha != 0:
+            r = r / (((5.0 + n) ** lp_alpha) / (6.0 ** lp_alpha))
+        if cp_beta != 0:
+            cp = cp_beta * S * np.log(min((n - 2) / S, 1.0)) if n > 2 else -np.inf
+            r = r + max(cp, -20.0)
+        if n / S > min_ratio and (best is None or r > best_s):
+            best, best_s = toks, r
+    return (best[1:-1] if best is not None else []), best_s, hyps
