@@ -222,18 +222,19 @@ int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const int *limit,
                       int *fin_beam, float *fin_score, lh_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
- * a11. Hypothesis state gather: dst_t[:,k] = src_t[:,backptr[k]] for n_tensors H x B tensors in
- * one launch.  Replaces the per-column cudaMemcpy loops of SwapStatesDecoding
+ * a11. Hypothesis state gather: dst_t[:,k] = src_t[:,backptr[k]], k < B, for n_tensors tensors in
+ * one launch (dst_t is H x B, src_t is H x B_src; a backptr outside [0,B_src) is clamped into it).  Replaces the per-column cudaMemcpy loops of SwapStatesDecoding
  * (src/layer_input_to_hidden.h:1517-1531, src/layer_hidden_to_hidden.h:569-584), the h~ swap of
  * NeuralMachineTranslation::SwapDecodingStates (src/deep_rnn.h:1842-1857) and the whole-matrix
  * copies of TargetCopyPrevStates (src/deep_rnn.h:1861-1872).  src/dst are HOST arrays of device
  * pointers, n_tensors <= LH_GATHER_MAX_TENSORS; dst_t must not alias any src.
- * With col_src = NULL and backptr = identity this is also TransferDecodingStatesGpu
- * (src/layer_input_to_hidden.h:1536-1545) when backptr maps every beam column to its sentence.
+ * With backptr[k] = sentence of beam column k and B_src = number of sentences this is also
+ * TransferDecodingStatesGpu (src/layer_input_to_hidden.h:1536-1545), the broadcast of the encoder's
+ * final state to the beam columns.
  */
 #define LH_GATHER_MAX_TENSORS 24
 int lh_beam_gather_f32(const float *const *src, float *const *dst, int n_tensors, int H, int B,
-                       const int *backptr, lh_stream_t stream);
+                       int B_src, const int *backptr, lh_stream_t stream);
 
 #ifdef __cplusplus
 }

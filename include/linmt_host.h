@@ -1,0 +1,82 @@
+/*
+ * linmt_host.h -- C facade of liblinmt_host.so, the C++ layer classes (InputToHiddenLayer,
+ * HiddenToHiddenLayer, AttentionLayer, SoftmaxLayer, Decoder, NeuralMachineTranslation) that sit on
+ * top of the kernel ABI of linmt_hip.h.  C++ callers use the classes of linmt_amd/host/nmt.h
+ * directly; this facade exists for callers without a C++ toolchain (the Python tests and the
+ * benchmark drive the classes through it), in the style of the reference's own C entry points
+ * python_decoder_init / python_decoder_do_job (src/decoder_sentence.h:94-97,
+ * src/decoder_sentence.cu:844-874).
+ *
+ * All pointers are HOST pointers.  Matrices are column-major; token arrays are int32 with -1 padding.
+ * Every function returns 0 on success and -1 on failure; lnmt_last_error() describes the failure.
+ */
+#ifndef LINMT_HOST_H_
+#define LINMT_HOST_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct lnmt_config {
+  int num_layers;
+  int lstm_size;
+  int embedding_size;       /* 0 = lstm_size */
+  int source_vocab_size;
+  int target_vocab_size;
+  int minibatch_size;       /* scoring: columns; decoding: ignored */
+  int longest_sentence;     /* reference's longest_sentence_ (with its +4) */
+  int attention_mode;       /* 0 none, 1 local-p, 2 global general */
+  int attention_width;      /* D */
+  int feed_input;
+  int sequence_to_sequence; /* 0 = target-side language model */
+  int clip_cell;
+  float cell_clip_threshold;
+} lnmt_config;
+
+typedef struct lnmt_decode_options {
+  int beam_size;
+  float max_decoding_ratio, min_decoding_ratio, penalty, diversity, lp_alpha, cp_beta;
+} lnmt_decode_options;
+
+typedef struct lnmt_model lnmt_model;
+
+const char *lnmt_last_error(void);
+
+/* NeuralMachineTranslation + InitModel (scoring, one node per timestep). */
+lnmt_model *lnmt_model_create_scoring(const lnmt_config *cfg);
+/* NeuralMachineTranslation + InitModelDecoding for up to n_sent sentences x beam hypotheses. */
+lnmt_model *lnmt_model_create_decoding(const lnmt_config *cfg, int n_sent, int beam_size);
+void lnmt_model_destroy(lnmt_model *m);
+
+/* Parameters by reference name ("src.0.W", "src.1.M_i", "tgt.0.Q_c", "tgt.2.b_f", "attn.W_a",
+ * "softmax.D", ...), each a column-major matrix as the reference stores it. */
+int lnmt_model_set_param(lnmt_model *m, const char *name, const float *data, long long n);
+int lnmt_model_get_param(lnmt_model *m, const char *name, float *data, long long n);
+
+/* NeuralMachineTranslation::GetError: sum of log p(target) over the non-pad target positions. */
+int lnmt_get_error(lnmt_model *m, const int *source, int source_length, const int *target_in,
+                   const int *target_out, int target_length, const int *batch_information,
+                   int minibatch_size, double *loss);
+
+/* Copies a state of the last lnmt_get_error call: kind 0 = h, 1 = c of (side 0 src / 1 tgt, layer,
+ * timestep); kind 2 = attention output h~ of target timestep; kind 3 = alignments (B x W) of target
+ * timestep.  n = number of floats the caller's buffer holds. */
+int lnmt_get_state(lnmt_model *m, int kind, int side, int layer, int timestep, float *data,
+                   long long n);
+
+/* Batched EnsembleFactory::DecodeFile.  sentences: concatenated source ids in ORIGINAL order,
+ * lengths[n].  Outputs: best (n x cap, row-major), best_len[n], best_score[n], steps[n]; if
+ * hyp_tokens != NULL also every finished hypothesis: hyp_tokens (n x hyp_cap x cap), hyp_len and
+ * hyp_score (n x hyp_cap), n_hyp[n]. */
+int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int *lengths, int n,
+                      const lnmt_decode_options *o, int *best, int cap, int *best_len,
+                      float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
+                      float *hyp_score, int hyp_cap, int *n_hyp);
+
+/* The model's HIP stream (hipStream_t as void*), for callers that time with HIP events. */
+void *lnmt_model_stream(lnmt_model *m);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
 struct GatherArgs {
   const float *src[LH_GATHER_MAX_TENSORS];
   float *dst[LH_GATHER_MAX_TENSORS];
-  int H, B;
+  int H, B_src;
   const int *backptr;
 };
 
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void beam_gather_kernel(const GatherArgs a) {
   const int t = blockIdx.z;
   const int k = blockIdx.y;
   int from = a.backptr[k];
-  from = from < 0 ? 0 : (from >= a.B ? a.B - 1 : from);
+  from = from < 0 ? 0 : (from >= a.B_src ? a.B_src - 1 : from);
   const float *src = a.src[t] + (size_t)from * a.H;
   float *dst = a.dst[t] + (size_t)k * a.H;
   for (int q = blockIdx.x * 256 + threadIdx.x; q < HQ; q += gridDim.x * 256) {
@@ -152,11 +152,11 @@ extern "C" int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const in
 }
 
 extern "C" int lh_beam_gather_f32(const float *const *src, float *const *dst, int n_tensors, int H,
-                                  int B, const int *backptr, lh_stream_t stream) {
-  if (n_tensors < 1 || n_tensors > LH_GATHER_MAX_TENSORS || H <= 0 || B <= 0 || !src || !dst ||
-      !backptr)
-    return lh::fail_arg("lh_beam_gather_f32: n_tensors=%d H=%d B=%d or NULL pointer", n_tensors, H,
-                        B);
+                                  int B, int B_src, const int *backptr, lh_stream_t stream) {
+  if (n_tensors < 1 || n_tensors > LH_GATHER_MAX_TENSORS || H <= 0 || B <= 0 || B_src <= 0 ||
+      !src || !dst || !backptr)
+    return lh::fail_arg("lh_beam_gather_f32: n_tensors=%d H=%d B=%d B_src=%d or NULL pointer",
+                        n_tensors, H, B, B_src);
   GatherArgs a{};
   bool vec = H % 4 == 0;
   for (int t = 0; t < n_tensors; ++t) {
@@ -168,7 +168,7 @@ extern "C" int lh_beam_gather_f32(const float *const *src, float *const *dst, in
     vec = vec && lh::aligned16(src[t]) && lh::aligned16(dst[t]);
   }
   a.H = H;
-  a.B = B;
+  a.B_src = B_src;
   a.backptr = backptr;
   const int hq = vec ? H / 4 : H;
   const dim3 grid((hq + 255) / 256, B, n_tensors), block(256);

@@ -1,0 +1,171 @@
+"""ctypes binding of liblinmt_host.so (C facade of the C++ layer classes, include/linmt_host.h).
+
+Python plumbing for the tests and the benchmark only; the computation happens in the C++ classes
+and the HIP kernels.  No fallback: a missing library raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblinmt_host.so")
+_lib = None
+
+
+class HostError(RuntimeError):
+    pass
+
+
+class Config(C.Structure):
+    _fields_ = [("num_layers", C.c_int), ("lstm_size", C.c_int), ("embedding_size", C.c_int),
+                ("source_vocab_size", C.c_int), ("target_vocab_size", C.c_int),
+                ("minibatch_size", C.c_int), ("longest_sentence", C.c_int),
+                ("attention_mode", C.c_int), ("attention_width", C.c_int), ("feed_input", C.c_int),
+                ("sequence_to_sequence", C.c_int), ("clip_cell", C.c_int),
+                ("cell_clip_threshold", C.c_float)]
+
+
+class DecodeOptions(C.Structure):
+    _fields_ = [("beam_size", C.c_int), ("max_decoding_ratio", C.c_float),
+                ("min_decoding_ratio", C.c_float), ("penalty", C.c_float),
+                ("diversity", C.c_float), ("lp_alpha", C.c_float), ("cp_beta", C.c_float)]
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise HostError(f"{LIB_PATH} is missing: build it with __graft_entry__.build(); "
+                        "there is no CPU fallback")
+    lib = C.CDLL(LIB_PATH)
+    lib.lnmt_last_error.restype = C.c_char_p
+    lib.lnmt_model_create_scoring.restype = C.c_void_p
+    lib.lnmt_model_create_scoring.argtypes = [C.POINTER(Config)]
+    lib.lnmt_model_create_decoding.restype = C.c_void_p
+    lib.lnmt_model_create_decoding.argtypes = [C.POINTER(Config), C.c_int, C.c_int]
+    lib.lnmt_model_destroy.argtypes = [C.c_void_p]
+    lib.lnmt_model_destroy.restype = None
+    lib.lnmt_model_set_param.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
+    lib.lnmt_model_get_param.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
+    lib.lnmt_get_error.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+                                   C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_double)]
+    lib.lnmt_get_state.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                   C.c_longlong]
+    lib.lnmt_decode_batch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                      C.POINTER(DecodeOptions), C.c_void_p, C.c_int, C.c_void_p,
+                                      C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                      C.c_int, C.c_void_p]
+    lib.lnmt_model_stream.restype = C.c_void_p
+    lib.lnmt_model_stream.argtypes = [C.c_void_p]
+    _lib = lib
+    return lib
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise HostError(f"{what}: {load().lnmt_last_error().decode('utf-8', 'replace')}")
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+class Model:
+    def __init__(self, num_layers, lstm_size, source_vocab_size, target_vocab_size,
+                 longest_sentence=104, attention_mode=1, attention_width=10, feed_input=True,
+                 minibatch_size=1, embedding_size=0, sequence_to_sequence=True, decoding=None,
+                 clip_cell=False, cell_clip_threshold=50.0):
+        """decoding=(n_sent, beam) builds the batched decoder, otherwise the scoring model."""
+        self.cfg = Config(num_layers, lstm_size, embedding_size, source_vocab_size,
+                          target_vocab_size, minibatch_size, longest_sentence, attention_mode,
+                          attention_width, int(feed_input), int(sequence_to_sequence),
+                          int(clip_cell), cell_clip_threshold)
+        lib = load()
+        if decoding is not None:
+            self.n_sent, self.beam = decoding
+            h = lib.lnmt_model_create_decoding(C.byref(self.cfg), self.n_sent, self.beam)
+        else:
+            h = lib.lnmt_model_create_scoring(C.byref(self.cfg))
+        if not h:
+            raise HostError("model creation failed: "
+                            + lib.lnmt_last_error().decode("utf-8", "replace"))
+        self.handle = C.c_void_p(h)
+
+    def close(self):
+        if getattr(self, "handle", None):
+            load().lnmt_model_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def stream(self):
+        return load().lnmt_model_stream(self.handle)
+
+    def set_params(self, params):
+        """params: name -> 2-D/1-D array in mathematical layout (rows x cols)."""
+        for name, arr in params.items():
+            flat = np.ascontiguousarray(np.asarray(arr, np.float32).ravel(order="F"))
+            _check(load().lnmt_model_set_param(self.handle, name.encode(), _p(flat), flat.size),
+                   f"set_param({name})")
+
+    def get_param(self, name, shape):
+        out = np.empty(int(np.prod(shape)), np.float32)
+        _check(load().lnmt_model_get_param(self.handle, name.encode(), _p(out), out.size),
+               f"get_param({name})")
+        return out.reshape(shape, order="F")
+
+    def get_error(self, src, tgt_in, tgt_out, batch_info):
+        """src (B,S), tgt_in/tgt_out (B,T) int arrays, -1 padding; returns sum log p(target)."""
+        src = np.asfortranarray(src, np.int32) if src is not None else None
+        tgt_in = np.asfortranarray(tgt_in, np.int32)
+        tgt_out = np.asfortranarray(tgt_out, np.int32)
+        B, T = tgt_in.shape
+        S = src.shape[1] if src is not None else 0
+        bi = None if batch_info is None else np.ascontiguousarray(batch_info, np.int32)
+        loss = C.c_double(0)
+        _check(load().lnmt_get_error(self.handle, _p(src), S, _p(tgt_in), _p(tgt_out), T, _p(bi), B,
+                                     C.byref(loss)), "get_error")
+        return loss.value
+
+    def get_state(self, kind, side, layer, timestep, rows, cols):
+        out = np.empty(rows * cols, np.float32)
+        _check(load().lnmt_get_state(self.handle, kind, side, layer, timestep, _p(out), out.size),
+               "get_state")
+        return out.reshape((rows, cols), order="F")
+
+    def decode_batch(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0,
+                     diversity=0.0, lp_alpha=0.65, cp_beta=0.20, with_hyps=False, hyp_cap=256):
+        n = len(sentences)
+        lengths = np.array([len(s) for s in sentences], np.int32)
+        flat = np.ascontiguousarray(np.concatenate([np.asarray(s, np.int32) for s in sentences]))
+        cap = self.cfg.longest_sentence + 2
+        o = DecodeOptions(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta)
+        best = np.zeros((n, cap), np.int32)
+        blen = np.zeros(n, np.int32)
+        bscore = np.zeros(n, np.float32)
+        steps = np.zeros(n, np.int32)
+        nh = np.zeros(n, np.int32)
+        ht = hl = hs = None
+        if with_hyps:
+            ht = np.zeros((n, hyp_cap, cap), np.int32)
+            hl = np.zeros((n, hyp_cap), np.int32)
+            hs = np.zeros((n, hyp_cap), np.float32)
+        _check(load().lnmt_decode_batch(self.handle, _p(flat), _p(lengths), n, C.byref(o), _p(best),
+                                        cap, _p(blen), _p(bscore), _p(steps), _p(ht), _p(hl),
+                                        _p(hs), hyp_cap, _p(nh)), "decode_batch")
+        res = []
+        for i in range(n):
+            r = dict(best=best[i, :blen[i]].copy(), best_score=float(bscore[i]),
+                     steps=int(steps[i]), n_hyp=int(nh[i]))
+            if with_hyps:
+                k = min(int(nh[i]), hyp_cap)
+                r["hyps"] = [(ht[i, j, :hl[i, j]].copy(), float(hs[i, j])) for j in range(k)]
+            res.append(r)
+        return res

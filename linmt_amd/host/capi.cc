@@ -1,0 +1,181 @@
+// C facade over the C++ layer classes (declared in include/linmt_host.h).
+#include <cstring>
+#include <memory>
+
+#include "../../include/linmt_host.h"
+#include "nmt.h"
+
+using namespace linmt;
+
+struct lnmt_model {
+  std::unique_ptr<NeuralMachineTranslation> nmt;
+};
+
+namespace {
+
+thread_local std::string g_error;
+
+GlobalConfiguration ToConfig(const lnmt_config *c) {
+  GlobalConfiguration g;
+  g.num_layers_ = c->num_layers;
+  g.lstm_size_ = c->lstm_size;
+  g.embedding_size_ = c->embedding_size;
+  g.source_vocab_size_ = c->source_vocab_size;
+  g.target_vocab_size_ = c->target_vocab_size;
+  g.minibatch_size_ = c->minibatch_size;
+  g.longest_sentence_ = c->longest_sentence;
+  g.attention_mode_ = c->attention_mode;
+  g.attention_width_ = c->attention_width;
+  g.feed_input_mode_ = c->feed_input != 0;
+  g.sequence_to_sequence_mode_ = c->sequence_to_sequence != 0;
+  g.clip_cell_mode_ = c->clip_cell != 0;
+  g.cell_clip_threshold_ = c->cell_clip_threshold;
+  return g;
+}
+
+template <typename F>
+int Guard(F &&f) {
+  try {
+    f();
+    return 0;
+  } catch (const std::exception &e) {
+    g_error = e.what();
+    return -1;
+  }
+}
+
+}  // namespace
+
+extern "C" const char *lnmt_last_error(void) { return g_error.c_str(); }
+
+extern "C" lnmt_model *lnmt_model_create_scoring(const lnmt_config *cfg) {
+  lnmt_model *m = nullptr;
+  if (Guard([&] {
+        std::unique_ptr<lnmt_model> p(new lnmt_model());
+        p->nmt.reset(new NeuralMachineTranslation(ToConfig(cfg)));
+        p->nmt->InitModel();
+        m = p.release();
+      }) != 0)
+    return nullptr;
+  return m;
+}
+
+extern "C" lnmt_model *lnmt_model_create_decoding(const lnmt_config *cfg, int n_sent,
+                                                  int beam_size) {
+  lnmt_model *m = nullptr;
+  if (Guard([&] {
+        if (n_sent < 1 || beam_size < 1) throw LinmtError("n_sent and beam_size must be positive");
+        std::unique_ptr<lnmt_model> p(new lnmt_model());
+        p->nmt.reset(new NeuralMachineTranslation(ToConfig(cfg)));
+        p->nmt->InitModelDecoding(n_sent, beam_size);
+        m = p.release();
+      }) != 0)
+    return nullptr;
+  return m;
+}
+
+extern "C" void lnmt_model_destroy(lnmt_model *m) { delete m; }
+
+extern "C" int lnmt_model_set_param(lnmt_model *m, const char *name, const float *data,
+                                    long long n) {
+  return Guard([&] {
+    if (!m->nmt->SetParam(name, data, (size_t)n))
+      throw LinmtError(std::string("unknown parameter or wrong size: ") + name);
+    m->nmt->Synchronize();
+  });
+}
+
+extern "C" int lnmt_model_get_param(lnmt_model *m, const char *name, float *data, long long n) {
+  return Guard([&] {
+    std::vector<float> v;
+    if (!m->nmt->GetParam(name, &v) || (long long)v.size() != n)
+      throw LinmtError(std::string("unknown parameter or wrong size: ") + name);
+    memcpy(data, v.data(), sizeof(float) * v.size());
+  });
+}
+
+extern "C" int lnmt_get_error(lnmt_model *m, const int *source, int source_length,
+                              const int *target_in, const int *target_out, int target_length,
+                              const int *batch_information, int minibatch_size, double *loss) {
+  return Guard([&] {
+    *loss = m->nmt->GetError(source, source_length, target_in, target_out, target_length,
+                             batch_information, minibatch_size);
+  });
+}
+
+extern "C" int lnmt_get_state(lnmt_model *m, int kind, int side, int layer, int timestep,
+                              float *data, long long n) {
+  return Guard([&] {
+    NeuralMachineTranslation &M = *m->nmt;
+    const float *src = nullptr;
+    size_t count = 0;
+    if (kind == 0 || kind == 1) {
+      if (layer < 0 || layer >= M.cfg_.num_layers_) throw LinmtError("layer out of range");
+      LstmLayer &L = side == 0 ? M.SourceLayer(layer) : M.TargetLayer(layer);
+      if (timestep < 0 || timestep >= L.num_nodes_) throw LinmtError("timestep out of range");
+      src = kind == 0 ? L.v_nodes_[timestep].p_device_h_t_ : L.v_nodes_[timestep].p_device_c_t_;
+      count = (size_t)L.lstm_size_ * L.minibatch_size_;
+    } else if (kind == 2 || kind == 3) {
+      AttentionLayer &A = M.attention_layer_;
+      if (timestep < 0 || timestep >= A.num_nodes_) throw LinmtError("timestep out of range");
+      src = kind == 2 ? A.v_nodes_[timestep].p_device_final_tmp_2_
+                      : A.v_nodes_[timestep].p_device_alignments_;
+      count = kind == 2 ? (size_t)A.lstm_size_ * A.minibatch_size_
+                        : (size_t)A.window_ * A.minibatch_size_;
+    } else {
+      throw LinmtError("unknown state kind");
+    }
+    if ((size_t)n < count) count = (size_t)n;
+    HipErrorWrapper(hipMemcpyAsync(data, src, sizeof(float) * count, hipMemcpyDeviceToHost,
+                                   M.stream_),
+                    "state download failed");
+    M.Synchronize();
+  });
+}
+
+extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int *lengths, int n,
+                                 const lnmt_decode_options *o, int *best, int cap, int *best_len,
+                                 float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
+                                 float *hyp_score, int hyp_cap, int *n_hyp) {
+  return Guard([&] {
+    std::vector<std::vector<int>> sents(n);
+    size_t off = 0;
+    for (int i = 0; i < n; ++i) {
+      if (lengths[i] < 0) throw LinmtError("negative sentence length");
+      sents[i].assign(sentences + off, sentences + off + lengths[i]);
+      off += lengths[i];
+    }
+    DecodeOptions d;
+    d.beam_size_ = o->beam_size;
+    d.max_decoding_ratio_ = o->max_decoding_ratio;
+    d.min_decoding_ratio_ = o->min_decoding_ratio;
+    d.penalty_ = o->penalty;
+    d.diversity_ = o->diversity;
+    d.lp_alpha_ = o->lp_alpha;
+    d.cp_beta_ = o->cp_beta;
+    std::vector<SentenceResult> res;
+    m->nmt->DecodeBatch(sents, d, &res);
+    for (int i = 0; i < n; ++i) {
+      const SentenceResult &r = res[i];
+      const int bl = std::min((int)r.best.size(), cap);
+      for (int j = 0; j < bl; ++j) best[(size_t)i * cap + j] = r.best[j];
+      best_len[i] = bl;
+      best_score[i] = r.best_score;
+      if (steps) steps[i] = r.steps;
+      if (n_hyp) n_hyp[i] = (int)r.hypotheses.size();
+      if (hyp_tokens) {
+        const int nh = std::min((int)r.hypotheses.size(), hyp_cap);
+        for (int h = 0; h < nh; ++h) {
+          const Hypothesis &hy = r.hypotheses[h];
+          const int len = std::min((int)hy.tokens.size(), cap);
+          for (int j = 0; j < len; ++j)
+            hyp_tokens[((size_t)i * hyp_cap + h) * cap + j] = hy.tokens[j];
+          hyp_len[(size_t)i * hyp_cap + h] = (int)hy.tokens.size();
+          hyp_score[(size_t)i * hyp_cap + h] = hy.score;
+        }
+      }
+    }
+  });
+}
+
+extern "C" void *lnmt_model_stream(lnmt_model *m) { return m->nmt->stream_; }

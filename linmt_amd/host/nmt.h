@@ -1,0 +1,304 @@
+// C++ layer classes of the LSTM / attention / softmax / beam path, keeping the reference's class and
+// method names (src/layer_input_to_hidden.h, src/layer_hidden_to_hidden.h, src/layer_attention.h,
+// src/layer_loss.h, src/deep_rnn.h, src/decoder.h) on top of the C ABI of liblinmt_hip.so.
+//
+// What changed against the reference, by design:
+//   * one HIP stream per model instead of 28 streams + ~45 events per layer: every node's
+//     ForwardProp() is a short, ordered list of launches (stacked gate GEMM -> fused cell);
+//   * the four gate matrices of an operand are stored stacked (4H x K, rows i,f,c',o) so that the
+//     8-12 SGEMMs of a cell are one multi-segment MFMA GEMM; M_i, W_hi, ... remain addressable as
+//     strided views (ld = 4H) and by their reference names through SetParam/GetParam;
+//   * "send h_t above" is pointer passing (the reference memcpy's because of `&& false`,
+//     src/deep_rnn.h:544,586);
+//   * decoding runs many sentences at once: the target-side minibatch is n_sent*beam columns,
+//     sentence s owns columns [s*beam,(s+1)*beam); beam selection, back-pointers and the state swap
+//     stay on the device, the host only reads the per-step (token, back-pointer, score) history.
+#pragma once
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "hip_util.h"
+
+namespace linmt {
+
+// Subset of GlobalConfiguration (src/global_configuration.h:93-310) that the path reads.
+struct GlobalConfiguration {
+  int num_layers_ = 1;
+  int lstm_size_ = 100;
+  int embedding_size_ = 0;  // 0: same as lstm_size_ (the reference's only case, global_configuration.h:220)
+  int source_vocab_size_ = 0;
+  int target_vocab_size_ = 0;
+  int minibatch_size_ = 1;        // training / scoring columns
+  int longest_sentence_ = 100;    // already including the reference's +4 (global_configuration.cc:290)
+  int attention_mode_ = 0;        // 0 none, 1 local-p (reference), 2 global general (build-defined)
+  int attention_width_ = 10;      // D
+  bool feed_input_mode_ = false;
+  bool sequence_to_sequence_mode_ = true;  // false: target-side language model (--nlm)
+  bool clip_cell_mode_ = false;
+  float cell_clip_threshold_ = 50.f;
+};
+
+class NeuralMachineTranslation;
+class LstmLayer;
+class AttentionLayer;
+
+// A strided view of one gate block of a stacked parameter (reference: p_device_m_i_, p_device_w_hi_ ...).
+struct MatrixView {
+  float *ptr;
+  int ld;
+};
+
+// ---------------------------------------------------------------------------------------------
+// LstmInputHiddenNode (src/node_input_to_hidden.h:33-150) and LstmHiddenHiddenNode
+// (src/node_hidden_to_hidden.h:34-131): one object per timestep (one in all when decoding).
+class LstmNode {
+ public:
+  int index_ = 0;
+  LstmLayer *p_layer_ = nullptr;
+  int minibatch_size_ = 0;  // columns processed by ForwardProp (<= the layer's allocation)
+
+  // inputs: aliases of buffers owned elsewhere, as in the reference
+  int *p_device_input_vocab_indices_ = nullptr;     // layer 1 only: ids of this step, -1 -> 0
+  int *p_device_input_vocab_indices_01_ = nullptr;  // 0/1 padding mask of this step
+  float *p_device_h_t_prev_ = nullptr;
+  float *p_device_c_t_prev_ = nullptr;
+  float *p_device_h_tild_ = nullptr;     // attention output of step t-1 (feed input, layer 1 target)
+  float *p_device_h_t_below_ = nullptr;  // layers >= 2
+
+  // buffers owned by the layer, one slice per node
+  float *p_device_sparse_lookup_ = nullptr;  // layer 1: E x B embedding columns
+  float *p_device_gates_ = nullptr;          // 4H x B: i_t, f_t, c_prime_t_tanh, o_t (NULL when not kept)
+  float *p_device_c_t_ = nullptr;
+  float *p_device_h_t_ = nullptr;
+
+  // InputToHidden: UpdateVectorsForwardGpu(idx0, mask01, h_prev, c_prev) (node_input_to_hidden.h:100);
+  // HiddenToHidden: UpdateVectorsForwardGpu(mask01, h_prev, c_prev) (node_hidden_to_hidden.h:94).
+  void UpdateVectorsForwardGpu(int *p_device_input_vocab_indices, int *p_device_input_vocab_indices_01,
+                               float *p_device_h_t_prev, float *p_device_c_t_prev);
+  void UpdateVectorsForwardGpu(int *p_device_input_vocab_indices_01, float *p_device_h_t_prev,
+                               float *p_device_c_t_prev);
+  // ForwardPropGpu of both node kinds (node_input_to_hidden.h:218-636, node_hidden_to_hidden.h:194-444).
+  void ForwardProp();
+};
+
+// InputToHiddenLayer (src/layer_input_to_hidden.h:37-378) / HiddenToHiddenLayer
+// (src/layer_hidden_to_hidden.h:33-317) share everything but the source of x.
+class LstmLayer {
+ public:
+  NeuralMachineTranslation *p_neural_mt_ = nullptr;
+  bool input_layer_mode_ = true;  // true: InputToHiddenLayer (owns the embedding W)
+  bool source_side_mode_ = true;
+  int layer_number_ = 0;
+  int lstm_size_ = 0;
+  int input_size_ = 0;  // E for layer 1, H above
+  int vocab_size_ = 0;
+  int minibatch_size_ = 0;
+  int num_nodes_ = 0;
+  bool feed_input_mode_ = false;
+  bool keep_gates_ = false;
+
+  // parameters (stacked: rows [g*H,(g+1)*H) belong to gate g in the order i, f, c', o)
+  DeviceArray<float> p_device_w_;        // E x V embedding (layer 1)
+  DeviceArray<float> p_device_m_stack_;  // 4H x input_size : M_i, M_f, M_c, M_o
+  DeviceArray<float> p_device_w_h_stack_;  // 4H x H : W_hi, W_hf, W_hc, W_ho
+  DeviceArray<float> p_device_q_stack_;    // 4H x H : Q_i, Q_f, Q_c, Q_o (feed input)
+  DeviceArray<float> p_device_b_stack_;    // 4H     : b_i, b_f, b_c, b_o
+  MatrixView p_device_m(int gate) { return {p_device_m_stack_.get() + (size_t)gate * lstm_size_, 4 * lstm_size_}; }
+  MatrixView p_device_w_h(int gate) { return {p_device_w_h_stack_.get() + (size_t)gate * lstm_size_, 4 * lstm_size_}; }
+  MatrixView p_device_q(int gate) { return {p_device_q_stack_.get() + (size_t)gate * lstm_size_, 4 * lstm_size_}; }
+
+  // activations
+  DeviceArray<float> p_device_init_hidden_vec_, p_device_init_cell_vec_;  // zeros
+  DeviceArray<float> h_all_, c_all_, gates_all_, lookup_all_, preact_;
+  DeviceArray<float> p_device_h_t_previous_, p_device_c_t_previous_;  // decode: PreviousTargetState
+  DeviceArray<int> p_device_input_vocab_indices_full_, p_device_input_vocab_indices_01_full_;
+  std::vector<LstmNode> v_nodes_;
+
+  void Init(NeuralMachineTranslation *model, bool input_layer, bool source_side, int layer_number,
+            int minibatch_size, int num_nodes, bool keep_gates, bool with_previous_state);
+  // InitFeedInput (layer_input_to_hidden.h:299): allocates Q and switches the nodes to feed input.
+  void InitFeedInput();
+  // PreprocessGpuVocabIndices (layer_input_to_hidden.h:1478-1513, layer_hidden_to_hidden.h:541-560):
+  // host ids (B x T column-major, -1 padding) -> device idx0 / mask01 for all T steps.
+  void PreprocessGpuVocabIndices(const int *p_host_input_vocab_indices, int current_length,
+                                 int minibatch_size);
+  // Reference parameter names: "W", "M_i".."M_c", "W_hi".."W_ho", "b_i".."b_o", "Q_i".."Q_c".
+  bool SetParam(const std::string &name, const float *host, size_t n);
+  bool GetParam(const std::string &name, std::vector<float> *out);
+};
+
+// ---------------------------------------------------------------------------------------------
+// AttentionNode / AttentionLayer (src/layer_attention.h:28-131, 704-845).
+class AttentionNode {
+ public:
+  int index_ = 0;
+  AttentionLayer *p_attention_layer_ = nullptr;
+  int minibatch_size_ = 0;
+  float *p_device_h_t_ = nullptr;           // input: top decoder layer state
+  int *p_device_indices_mask_ = nullptr;    // 0/1 mask of the target step
+  float *p_device_tanh_1_ = nullptr, *p_device_sigma_1_ = nullptr, *p_device_p_t_ = nullptr;
+  float *p_device_h_t_wa_cache_ = nullptr, *p_device_alignments_ = nullptr;
+  float *p_device_cached_exp_ = nullptr, *p_device_c_t_ = nullptr, *p_device_final_tmp_2_ = nullptr;
+  int *p_device_indices_ = nullptr;
+  void ForwardProp();  // layer_attention.h:243-483
+};
+
+class AttentionLayer {
+ public:
+  NeuralMachineTranslation *p_neural_mt_ = nullptr;
+  int lstm_size_ = 0, minibatch_size_ = 0, d_ = 0, num_nodes_ = 0, window_ = 0;
+  bool global_mode_ = false;  // build-defined global "general" attention
+  DeviceArray<float> p_device_w_a_, p_device_w_p_, p_device_v_p_, p_device_output_bias_,
+      p_device_w_c_p1_, p_device_w_c_p2_;
+  DeviceArray<float> tanh_1_all_, sigma_1_all_, p_t_all_, wa_all_, alignments_all_, cached_exp_all_,
+      c_t_all_, final_all_;
+  DeviceArray<int> indices_all_, p_device_batch_information_, p_device_hs_col_;
+  // encoder top-layer states (owned by the top source layer): state(tau, col) = base + tau*step + col*colstride
+  const float *p_device_total_hs_ = nullptr;
+  long long hs_step_stride_ = 0, hs_col_stride_ = 0;
+  int hs_steps_ = 0;       // timesteps currently held
+  bool use_hs_col_ = false;  // decode: beam columns share their sentence's states
+  std::vector<AttentionNode> v_nodes_;
+
+  void Init(NeuralMachineTranslation *model, int minibatch_size, int num_nodes, int longest_sent);
+  // PreprocessMinibatchInformation (layer_attention.h:977): [len_0.., offset_0..] for B columns.
+  void PreprocessMinibatchInformation(const int *p_host_batch_information, int minibatch_size);
+  bool SetParam(const std::string &name, const float *host, size_t n);
+  bool GetParam(const std::string &name, std::vector<float> *out);
+};
+
+// ---------------------------------------------------------------------------------------------
+// BaseLossLayer (src/layer_loss.h:42-103) and SoftmaxLayer (:150-360).
+class BaseLossLayer {
+ public:
+  virtual ~BaseLossLayer() {}
+  virtual void ForwardProp(int index) = 0;
+  virtual double ComputeLossGpu(int index) = 0;
+  virtual void BackPropPreprocessGpu(float *p_device_h_t, int step) = 0;
+  virtual void GetDistributionGpuDecoderWrapper() = 0;
+  virtual float *GetDistPtr() = 0;
+  virtual void SetHTPtr(int index, float *p_device_h_t) = 0;
+  virtual float *GetHTPtr(int index) = 0;
+  virtual double GetTrainPerplexity() = 0;
+  virtual void PreprocessGpuVocabIndices(const int *p_host_output_vocab_indices_target,
+                                         int current_target_length, int minibatch_size) = 0;
+};
+
+class SoftmaxLayer : public BaseLossLayer {
+ public:
+  NeuralMachineTranslation *p_neural_mt_ = nullptr;
+  int lstm_size_ = 0, output_vocab_size_ = 0, minibatch_size_ = 0, num_nodes_ = 0;
+  int current_minibatch_ = 0;
+  bool training_perplexity_mode_ = false;
+  DeviceArray<float> p_device_d_, p_device_b_d_;
+  DeviceArray<float> p_device_outputdist_;           // V x B logits / probabilities (one step)
+  DeviceArray<double> p_device_logp_tgt_, p_device_loss_, p_device_train_perplexity_;
+  DeviceArray<int> p_device_output_vocab_indices_, p_device_output_vocab_indices_01_;
+  DeviceArray<float> p_device_output_vocab_indices_01_float_;
+  std::vector<float *> v_h_t_;  // per node: input of the softmax (SetHTPtr)
+  int *p_device_output_vocab_indices_single_ = nullptr, *p_device_output_vocab_indices_01_single_ = nullptr;
+
+  void Init(NeuralMachineTranslation *model, int minibatch_size, int num_nodes);
+  void ForwardProp(int index) override;                     // layer_loss.h:480-516
+  void GetDistributionGpu(float *p_device_h_t);             // layer_loss.h:797-883
+  double ComputeLossGpu(int index) override;                // layer_loss.h:673-704 (+ GetPerplexityGpu :708)
+  void BackPropPreprocessGpu(float *p_device_h_t, int step) override;  // layer_loss.h:630-650
+  void GetDistributionGpuDecoderWrapper() override;
+  float *GetDistPtr() override { return p_device_outputdist_.get(); }
+  void SetHTPtr(int index, float *p) override { v_h_t_[index] = p; }
+  float *GetHTPtr(int index) override { return v_h_t_[index]; }
+  double GetTrainPerplexity() override;
+  void PreprocessGpuVocabIndices(const int *p_host_output_vocab_indices_target,
+                                 int current_target_length, int minibatch_size) override;
+  // logits only (D*h + b_d), used by the on-device beam step
+  void ComputeLogits(float *p_device_h_t, int minibatch);
+  bool SetParam(const std::string &name, const float *host, size_t n);
+  bool GetParam(const std::string &name, std::vector<float> *out);
+};
+
+// ---------------------------------------------------------------------------------------------
+// Decoder (src/decoder.h:148-245): hypothesis bookkeeping.  The selection itself
+// (ExpandHypothesis / FinishCurrentHypotheses) runs on the device; this class owns the device-side
+// beam buffers and rebuilds the hypotheses from the recorded history.
+struct Hypothesis {
+  std::vector<int> tokens;  // <START> ... <EOF>
+  float score = 0.f;        // log-probability (+ penalties), before length / coverage rescoring
+};
+
+struct DecodeOptions {
+  int beam_size_ = 12;
+  float max_decoding_ratio_ = 1.5f, min_decoding_ratio_ = 0.5f;
+  float penalty_ = 0.f, diversity_ = 0.f, lp_alpha_ = 0.65f, cp_beta_ = 0.20f;
+};
+
+struct SentenceResult {
+  std::vector<int> best;  // 1-best without <START>/<EOF>
+  float best_score = 0.f;
+  std::vector<Hypothesis> hypotheses;  // in the order the reference's v_hypotheses_ would hold them
+  int steps = 0;                       // decoder forward passes this sentence took part in
+};
+
+class Decoder {
+ public:
+  static constexpr int start_symbol_ = 0, end_symbol_ = 1;
+  int beam_size_ = 0, n_sent_ = 0, max_steps_ = 0;
+  DeviceArray<float> cand_logp_, logp_eof_, score_[2], fin_score_hist_, score_hist_;
+  DeviceArray<int> cand_id_, limit_, tok_hist_, backptr_hist_, fin_count_hist_, fin_beam_hist_,
+      current_indices_;
+  void Init(int beam_size, int n_sent, int max_steps);
+  // OutputKBestHypotheses (decoder.h:529-699) for one sentence, num_hypotheses = 1.
+  static void OutputKBestHypotheses(const std::vector<Hypothesis> &hyps, int source_length,
+                                    const DecodeOptions &o, SentenceResult *out);
+};
+
+// ---------------------------------------------------------------------------------------------
+// NeuralMachineTranslation (src/deep_rnn.h): wiring and the forward drivers.
+class NeuralMachineTranslation {
+ public:
+  GlobalConfiguration cfg_;
+  hipStream_t stream_ = nullptr;
+  bool decode_mode_ = false;
+  int beam_size_ = 0, n_sent_ = 0;
+
+  LstmLayer input_layer_source_, input_layer_target_;
+  std::vector<std::unique_ptr<LstmLayer>> v_hidden_layers_source_, v_hidden_layers_target_;
+  AttentionLayer attention_layer_;
+  SoftmaxLayer softmax_layer_;
+  BaseLossLayer *p_softmax_layer_ = &softmax_layer_;
+  Decoder decoder_;
+  DeviceArray<float> p_device_h_tild_previous_;  // decode: gathered h~ of the previous step
+  DeviceArray<int> p_device_ones_, p_device_sentence_of_column_;
+
+  explicit NeuralMachineTranslation(const GlobalConfiguration &cfg);
+  ~NeuralMachineTranslation();
+  // InitModel (deep_rnn.h:249-692): one node per timestep, B = cfg.minibatch_size_.
+  void InitModel();
+  // InitModelDecoding (deep_rnn.h:697-922), batched: n_sent sentences x beam hypotheses.
+  void InitModelDecoding(int n_sent, int beam_size);
+
+  LstmLayer &SourceLayer(int l) { return l == 0 ? input_layer_source_ : *v_hidden_layers_source_[l - 1]; }
+  LstmLayer &TargetLayer(int l) { return l == 0 ? input_layer_target_ : *v_hidden_layers_target_[l - 1]; }
+
+  // GetError (deep_rnn.h:2173-2317): teacher-forced forward + sum of log p(target).
+  double GetError(const int *p_host_source, int source_length, const int *p_host_target_in,
+                  const int *p_host_target_out, int target_length, const int *p_host_batch_information,
+                  int minibatch_size);
+  // ForwardPropSource (deep_rnn.h:1572-1721) for n_sent sentences (B x S ids, reversed, left-padded).
+  void ForwardPropSource(const int *p_host_source, int source_length, int n_sent);
+  // ForwardPropTarget (deep_rnn.h:1754-1836) on the first `minibatch` beam columns.
+  void ForwardPropTarget(int curr_index, int *p_device_current_indices, int minibatch);
+  // SwapDecodingStates + TargetCopyPrevStates (deep_rnn.h:1842-1872) in one gather launch.
+  void SwapDecodingStates(const int *p_device_backptr, int minibatch);
+  // EnsembleFactory::DecodeFile (decoder.h:1702-1776) for a batch of sentences (ids in ORIGINAL
+  // order, ragged).  Results come back in input order.
+  void DecodeBatch(const std::vector<std::vector<int>> &sentences, const DecodeOptions &o,
+                   std::vector<SentenceResult> *results);
+
+  bool SetParam(const std::string &name, const float *host, size_t n);
+  bool GetParam(const std::string &name, std::vector<float> *out);
+  void Synchronize();
+};
+
+}  // namespace linmt

@@ -1,0 +1,472 @@
+// LSTM, attention and softmax layer classes: parameter storage and the per-node forward bodies,
+// each a short ordered list of launches into liblinmt_hip.so on the model's single stream.
+#include <cstring>
+
+#include "nmt.h"
+
+namespace linmt {
+
+namespace {
+
+int GateIndex(char g) {  // stacked order i, f, c', o
+  switch (g) {
+    case 'i': return 0;
+    case 'f': return 1;
+    case 'c': return 2;
+    case 'o': return 3;
+    default: return -1;
+  }
+}
+
+// Host H x K column-major block <-> rows [gate*H, (gate+1)*H) of a stacked 4H x K device matrix.
+void UploadGateBlock(DeviceArray<float> &stack, int gate, int H, int K, const float *host,
+                     hipStream_t s) {
+  HipErrorWrapper(hipMemcpy2DAsync(stack.get() + (size_t)gate * H, sizeof(float) * 4 * H, host,
+                                   sizeof(float) * H, sizeof(float) * H, K, hipMemcpyHostToDevice, s),
+                  "parameter upload failed");
+}
+void DownloadGateBlock(const DeviceArray<float> &stack, int gate, int H, int K, float *host,
+                       hipStream_t s) {
+  HipErrorWrapper(hipMemcpy2DAsync(host, sizeof(float) * H, stack.get() + (size_t)gate * H,
+                                   sizeof(float) * 4 * H, sizeof(float) * H, K,
+                                   hipMemcpyDeviceToHost, s),
+                  "parameter download failed");
+}
+
+bool SetFlat(DeviceArray<float> &a, const float *host, size_t n, hipStream_t s) {
+  if (n != a.size()) return false;
+  a.Upload(host, n, s);
+  return true;
+}
+bool GetFlat(const DeviceArray<float> &a, std::vector<float> *out, hipStream_t s) {
+  out->resize(a.size());
+  a.Download(out->data(), a.size(), s);
+  HipErrorWrapper(hipStreamSynchronize(s), "parameter download failed");
+  return true;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+void LstmLayer::Init(NeuralMachineTranslation *model, bool input_layer, bool source_side,
+                     int layer_number, int minibatch_size, int num_nodes, bool keep_gates,
+                     bool with_previous_state) {
+  p_neural_mt_ = model;
+  const GlobalConfiguration &cfg = model->cfg_;
+  hipStream_t s = model->stream_;
+  input_layer_mode_ = input_layer;
+  source_side_mode_ = source_side;
+  layer_number_ = layer_number;
+  lstm_size_ = cfg.lstm_size_;
+  const int E = cfg.embedding_size_ > 0 ? cfg.embedding_size_ : cfg.lstm_size_;
+  input_size_ = input_layer ? E : lstm_size_;
+  vocab_size_ = source_side ? cfg.source_vocab_size_ : cfg.target_vocab_size_;
+  minibatch_size_ = minibatch_size;
+  num_nodes_ = num_nodes;
+  keep_gates_ = keep_gates;
+  const size_t H = lstm_size_, B = minibatch_size;
+
+  if (input_layer) p_device_w_.Alloc((size_t)input_size_ * vocab_size_);
+  p_device_m_stack_.Alloc(4 * H * input_size_);
+  p_device_w_h_stack_.Alloc(4 * H * H);
+  p_device_b_stack_.Alloc(4 * H);
+  p_device_m_stack_.Zero(s);
+  p_device_w_h_stack_.Zero(s);
+  p_device_b_stack_.Zero(s);
+
+  p_device_init_hidden_vec_.Alloc(H * B);
+  p_device_init_cell_vec_.Alloc(H * B);
+  p_device_init_hidden_vec_.Zero(s);
+  p_device_init_cell_vec_.Zero(s);
+  h_all_.Alloc(H * B * num_nodes);
+  c_all_.Alloc(H * B * num_nodes);
+  if (keep_gates) gates_all_.Alloc(4 * H * B * num_nodes);
+  if (input_layer) lookup_all_.Alloc((size_t)input_size_ * B * (keep_gates ? num_nodes : 1));
+  preact_.Alloc(4 * H * B);
+  if (with_previous_state) {
+    p_device_h_t_previous_.Alloc(H * B);
+    p_device_c_t_previous_.Alloc(H * B);
+  }
+  p_device_input_vocab_indices_full_.Alloc(B * (size_t)cfg.longest_sentence_);
+  p_device_input_vocab_indices_01_full_.Alloc(B * (size_t)cfg.longest_sentence_);
+
+  v_nodes_.assign(num_nodes, LstmNode());
+  for (int i = 0; i < num_nodes; ++i) {
+    LstmNode &n = v_nodes_[i];
+    n.index_ = i;
+    n.p_layer_ = this;
+    n.minibatch_size_ = minibatch_size;
+    n.p_device_h_t_ = h_all_.get() + H * B * i;
+    n.p_device_c_t_ = c_all_.get() + H * B * i;
+    n.p_device_gates_ = keep_gates ? gates_all_.get() + 4 * H * B * i : nullptr;
+    if (input_layer)
+      n.p_device_sparse_lookup_ = lookup_all_.get() + (keep_gates ? (size_t)input_size_ * B * i : 0);
+  }
+}
+
+void LstmLayer::InitFeedInput() {
+  feed_input_mode_ = true;
+  p_device_q_stack_.Alloc(4 * (size_t)lstm_size_ * lstm_size_);
+  p_device_q_stack_.Zero(p_neural_mt_->stream_);
+}
+
+void LstmLayer::PreprocessGpuVocabIndices(const int *p_host_input_vocab_indices, int current_length,
+                                          int minibatch_size) {
+  const size_t n = (size_t)minibatch_size * current_length;
+  if (n > p_device_input_vocab_indices_full_.size())
+    throw LinmtError("PreprocessGpuVocabIndices: sentence longer than longest_sentence_");
+  hipStream_t s = p_neural_mt_->stream_;
+  p_device_input_vocab_indices_full_.Upload(p_host_input_vocab_indices, n, s);
+  LhErrorWrapper(lh_preprocess_indices_i32(p_device_input_vocab_indices_full_.get(), (int)n,
+                                           p_device_input_vocab_indices_full_.get(),
+                                           p_device_input_vocab_indices_01_full_.get(), nullptr, s),
+                 "PreprocessGpuVocabIndices");
+}
+
+bool LstmLayer::SetParam(const std::string &name, const float *host, size_t n) {
+  hipStream_t s = p_neural_mt_->stream_;
+  const int H = lstm_size_;
+  if (name == "W") return input_layer_mode_ && SetFlat(p_device_w_, host, n, s);
+  if (name.size() == 3 && name[0] == 'M' && name[1] == '_') {
+    const int g = GateIndex(name[2]);
+    if (g < 0 || n != (size_t)H * input_size_) return false;
+    UploadGateBlock(p_device_m_stack_, g, H, input_size_, host, s);
+    return true;
+  }
+  if (name.size() == 4 && name.compare(0, 3, "W_h") == 0) {
+    const int g = GateIndex(name[3]);
+    if (g < 0 || n != (size_t)H * H) return false;
+    UploadGateBlock(p_device_w_h_stack_, g, H, H, host, s);
+    return true;
+  }
+  if (name.size() == 3 && name[0] == 'Q' && name[1] == '_') {
+    const int g = GateIndex(name[2]);
+    if (g < 0 || !feed_input_mode_ || n != (size_t)H * H) return false;
+    UploadGateBlock(p_device_q_stack_, g, H, H, host, s);
+    return true;
+  }
+  if (name.size() == 3 && name[0] == 'b' && name[1] == '_') {
+    const int g = GateIndex(name[2]);
+    if (g < 0 || n != (size_t)H) return false;
+    p_device_b_stack_.Upload(host, H, s, (size_t)g * H);
+    return true;
+  }
+  return false;
+}
+
+bool LstmLayer::GetParam(const std::string &name, std::vector<float> *out) {
+  hipStream_t s = p_neural_mt_->stream_;
+  const int H = lstm_size_;
+  if (name == "W") return input_layer_mode_ && GetFlat(p_device_w_, out, s);
+  const DeviceArray<float> *stack = nullptr;
+  int g = -1, K = 0;
+  if (name.size() == 3 && name[0] == 'M' && name[1] == '_') { stack = &p_device_m_stack_; g = GateIndex(name[2]); K = input_size_; }
+  else if (name.size() == 4 && name.compare(0, 3, "W_h") == 0) { stack = &p_device_w_h_stack_; g = GateIndex(name[3]); K = H; }
+  else if (name.size() == 3 && name[0] == 'Q' && name[1] == '_' && feed_input_mode_) { stack = &p_device_q_stack_; g = GateIndex(name[2]); K = H; }
+  else if (name.size() == 3 && name[0] == 'b' && name[1] == '_') {
+    g = GateIndex(name[2]);
+    if (g < 0) return false;
+    out->resize(H);
+    p_device_b_stack_.Download(out->data(), H, s, (size_t)g * H);
+    HipErrorWrapper(hipStreamSynchronize(s), "parameter download failed");
+    return true;
+  }
+  if (!stack || g < 0) return false;
+  out->resize((size_t)H * K);
+  DownloadGateBlock(*stack, g, H, K, out->data(), s);
+  HipErrorWrapper(hipStreamSynchronize(s), "parameter download failed");
+  return true;
+}
+
+void LstmNode::UpdateVectorsForwardGpu(int *p_device_input_vocab_indices,
+                                       int *p_device_input_vocab_indices_01,
+                                       float *p_device_h_t_prev, float *p_device_c_t_prev) {
+  p_device_input_vocab_indices_ = p_device_input_vocab_indices;
+  p_device_input_vocab_indices_01_ = p_device_input_vocab_indices_01;
+  p_device_h_t_prev_ = p_device_h_t_prev;
+  p_device_c_t_prev_ = p_device_c_t_prev;
+}
+
+void LstmNode::UpdateVectorsForwardGpu(int *p_device_input_vocab_indices_01,
+                                       float *p_device_h_t_prev, float *p_device_c_t_prev) {
+  p_device_input_vocab_indices_01_ = p_device_input_vocab_indices_01;
+  p_device_h_t_prev_ = p_device_h_t_prev;
+  p_device_c_t_prev_ = p_device_c_t_prev;
+}
+
+// One cell-step: [embedding lookup] -> ONE stacked multi-segment GEMM (x, h_{t-1}[, h~_{t-1}]) ->
+// ONE fused cell kernel.  The reference runs 1 + 8..12 SGEMMs + 7 elementwise kernels on 9 streams
+// here (src/node_input_to_hidden.h:218-636).
+void LstmNode::ForwardProp() {
+  LstmLayer &L = *p_layer_;
+  NeuralMachineTranslation &M = *L.p_neural_mt_;
+  hipStream_t s = M.stream_;
+  const int H = L.lstm_size_, B = minibatch_size_;
+  const float *x = nullptr;
+  if (L.input_layer_mode_) {
+    LhErrorWrapper(lh_embed_lookup_f32(L.p_device_w_.get(), L.input_size_, L.vocab_size_,
+                                       p_device_input_vocab_indices_, B, nullptr, 1.f,
+                                       p_device_sparse_lookup_, s),
+                   "LstmInputHiddenNode::ForwardPropGpu sparse lookup");
+    x = p_device_sparse_lookup_;
+  } else {
+    x = p_device_h_t_below_;
+  }
+  // feed input only from the second target step on (node_input_to_hidden.h:325)
+  const bool feed = L.feed_input_mode_ && 0 != index_;
+  lh_gemm_seg segs[3];
+  int nseg = 0;
+  segs[nseg++] = {L.p_device_m_stack_.get(), 4 * H, x, L.input_size_, L.input_size_};
+  segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
+  if (feed) segs[nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
+  LhErrorWrapper(lh_gemm_f32(4 * H, B, segs, nseg, 0, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
+                             L.preact_.get(), 4 * H, s),
+                 "LstmNode::ForwardPropGpu stacked gate product");
+  LhErrorWrapper(lh_lstm_cell_fwd_f32(H, B, L.preact_.get(), nullptr, nullptr,
+                                      L.p_device_b_stack_.get(), p_device_c_t_prev_,
+                                      p_device_input_vocab_indices_01_, feed ? 1 : 0,
+                                      M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f,
+                                      p_device_gates_, p_device_c_t_, p_device_h_t_, nullptr, 1.f,
+                                      nullptr, s),
+                 "LstmNode::ForwardPropGpu fused cell");
+}
+
+// ---------------------------------------------------------------------------------------------
+void AttentionLayer::Init(NeuralMachineTranslation *model, int minibatch_size, int num_nodes,
+                          int longest_sent) {
+  p_neural_mt_ = model;
+  const GlobalConfiguration &cfg = model->cfg_;
+  hipStream_t s = model->stream_;
+  lstm_size_ = cfg.lstm_size_;
+  minibatch_size_ = minibatch_size;
+  num_nodes_ = num_nodes;
+  global_mode_ = cfg.attention_mode_ == 2;
+  d_ = cfg.attention_width_;
+  window_ = global_mode_ ? longest_sent : 2 * d_ + 1;
+  const size_t H = lstm_size_, B = minibatch_size, W = window_;
+  p_device_w_a_.Alloc(H * H);
+  p_device_w_p_.Alloc(H * H);
+  p_device_v_p_.Alloc(H);
+  p_device_output_bias_.Alloc(H);
+  p_device_w_c_p1_.Alloc(H * H);
+  p_device_w_c_p2_.Alloc(H * H);
+  for (DeviceArray<float> *a : {&p_device_w_a_, &p_device_w_p_, &p_device_v_p_,
+                                &p_device_output_bias_, &p_device_w_c_p1_, &p_device_w_c_p2_})
+    a->Zero(s);
+  tanh_1_all_.Alloc(H * B * num_nodes);
+  sigma_1_all_.Alloc(B * num_nodes);
+  p_t_all_.Alloc(B * num_nodes);
+  wa_all_.Alloc(H * B * num_nodes);
+  alignments_all_.Alloc(B * W * num_nodes);
+  cached_exp_all_.Alloc(B * W * num_nodes);
+  c_t_all_.Alloc(H * B * num_nodes);
+  final_all_.Alloc(H * B * num_nodes);
+  indices_all_.Alloc(B * W * num_nodes);
+  p_device_batch_information_.Alloc(2 * B);
+  p_device_hs_col_.Alloc(B);
+  v_nodes_.assign(num_nodes, AttentionNode());
+  for (int i = 0; i < num_nodes; ++i) {
+    AttentionNode &n = v_nodes_[i];
+    n.index_ = i;
+    n.p_attention_layer_ = this;
+    n.minibatch_size_ = minibatch_size;
+    n.p_device_tanh_1_ = tanh_1_all_.get() + H * B * i;
+    n.p_device_sigma_1_ = sigma_1_all_.get() + B * i;
+    n.p_device_p_t_ = p_t_all_.get() + B * i;
+    n.p_device_h_t_wa_cache_ = wa_all_.get() + H * B * i;
+    n.p_device_alignments_ = alignments_all_.get() + B * W * i;
+    n.p_device_cached_exp_ = cached_exp_all_.get() + B * W * i;
+    n.p_device_c_t_ = c_t_all_.get() + H * B * i;
+    n.p_device_final_tmp_2_ = final_all_.get() + H * B * i;
+    n.p_device_indices_ = indices_all_.get() + B * W * i;
+  }
+}
+
+void AttentionLayer::PreprocessMinibatchInformation(const int *p_host_batch_information,
+                                                    int minibatch_size) {
+  // host layout [len_0..len_{B-1}, off_0..off_{B-1}] for the columns in use
+  hipStream_t s = p_neural_mt_->stream_;
+  if ((size_t)2 * minibatch_size > p_device_batch_information_.size())
+    throw LinmtError("PreprocessMinibatchInformation: too many columns");
+  p_device_batch_information_.Upload(p_host_batch_information, 2 * (size_t)minibatch_size, s);
+}
+
+bool AttentionLayer::SetParam(const std::string &name, const float *host, size_t n) {
+  hipStream_t s = p_neural_mt_->stream_;
+  if (name == "W_a") return SetFlat(p_device_w_a_, host, n, s);
+  if (name == "W_p") return SetFlat(p_device_w_p_, host, n, s);
+  if (name == "v_p") return SetFlat(p_device_v_p_, host, n, s);
+  if (name == "b_out") return SetFlat(p_device_output_bias_, host, n, s);
+  if (name == "W_c1") return SetFlat(p_device_w_c_p1_, host, n, s);
+  if (name == "W_c2") return SetFlat(p_device_w_c_p2_, host, n, s);
+  return false;
+}
+
+bool AttentionLayer::GetParam(const std::string &name, std::vector<float> *out) {
+  hipStream_t s = p_neural_mt_->stream_;
+  if (name == "W_a") return GetFlat(p_device_w_a_, out, s);
+  if (name == "W_p") return GetFlat(p_device_w_p_, out, s);
+  if (name == "v_p") return GetFlat(p_device_v_p_, out, s);
+  if (name == "b_out") return GetFlat(p_device_output_bias_, out, s);
+  if (name == "W_c1") return GetFlat(p_device_w_c_p1_, out, s);
+  if (name == "W_c2") return GetFlat(p_device_w_c_p2_, out, s);
+  return false;
+}
+
+// Four launches instead of the reference's 5 SGEMMs + 12 kernels (src/layer_attention.h:243-483):
+// tanh(W_p ha) [GEMM + tanh epilogue], W_a^T ha [GEMM], the fused core, and
+// tanh(W_c1 ctx + W_c2 ha + b_out) * mask [two-segment GEMM + bias/tanh/mask epilogue].
+void AttentionNode::ForwardProp() {
+  AttentionLayer &A = *p_attention_layer_;
+  hipStream_t s = A.p_neural_mt_->stream_;
+  const int H = A.lstm_size_, B = minibatch_size_;
+  const float *ha = p_device_h_t_;  // no dropout outside training
+  if (!A.global_mode_) {
+    lh_gemm_seg seg{A.p_device_w_p_.get(), H, ha, H, H};
+    LhErrorWrapper(lh_gemm_f32(H, B, &seg, 1, 0, 0, 1.f, 0.f, nullptr, LH_ACT_TANH, nullptr,
+                               p_device_tanh_1_, H, s),
+                   "AttentionNode::ForwardProp p_device_tanh_1_");
+  }
+  {
+    lh_gemm_seg seg{A.p_device_w_a_.get(), H, ha, H, H};
+    LhErrorWrapper(lh_gemm_f32(H, B, &seg, 1, 1, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
+                               p_device_h_t_wa_cache_, H, s),
+                   "AttentionNode::ForwardProp p_device_h_t_wa_cache_");
+  }
+  LhErrorWrapper(
+      lh_attn_core_fwd_f32(H, B, A.global_mode_ ? -1 : A.d_, A.window_, A.hs_steps_,
+                           p_device_tanh_1_, A.p_device_v_p_.get(), p_device_h_t_wa_cache_,
+                           A.p_device_total_hs_, A.hs_step_stride_, A.hs_col_stride_,
+                           A.use_hs_col_ ? A.p_device_hs_col_.get() : nullptr,
+                           A.p_device_batch_information_.get(), p_device_indices_mask_,
+                           p_device_p_t_, p_device_sigma_1_, p_device_indices_,
+                           p_device_alignments_, p_device_cached_exp_, p_device_c_t_, nullptr, s),
+      "AttentionNode::ForwardProp attention core");
+  lh_gemm_seg segs[2] = {{A.p_device_w_c_p1_.get(), H, p_device_c_t_, H, H},
+                         {A.p_device_w_c_p2_.get(), H, ha, H, H}};
+  LhErrorWrapper(lh_gemm_f32(H, B, segs, 2, 0, 0, 1.f, 0.f, A.p_device_output_bias_.get(),
+                             LH_ACT_TANH, p_device_indices_mask_, p_device_final_tmp_2_, H, s),
+                 "AttentionNode::ForwardProp p_device_final_tmp_2_");
+}
+
+// ---------------------------------------------------------------------------------------------
+void SoftmaxLayer::Init(NeuralMachineTranslation *model, int minibatch_size, int num_nodes) {
+  p_neural_mt_ = model;
+  const GlobalConfiguration &cfg = model->cfg_;
+  hipStream_t s = model->stream_;
+  lstm_size_ = cfg.lstm_size_;
+  output_vocab_size_ = cfg.target_vocab_size_;
+  minibatch_size_ = minibatch_size;
+  current_minibatch_ = minibatch_size;
+  num_nodes_ = num_nodes;
+  const size_t H = lstm_size_, V = output_vocab_size_, B = minibatch_size;
+  p_device_d_.Alloc(V * H);
+  p_device_b_d_.Alloc(V);
+  p_device_d_.Zero(s);
+  p_device_b_d_.Zero(s);
+  p_device_outputdist_.Alloc(V * B);
+  p_device_logp_tgt_.Alloc(B);
+  p_device_loss_.Alloc(1);
+  p_device_train_perplexity_.Alloc(1);
+  p_device_loss_.Zero(s);
+  p_device_train_perplexity_.Zero(s);
+  const size_t T = cfg.longest_sentence_;
+  p_device_output_vocab_indices_.Alloc(B * T);
+  p_device_output_vocab_indices_01_.Alloc(B * T);
+  p_device_output_vocab_indices_01_float_.Alloc(B * T);
+  v_h_t_.assign(num_nodes, nullptr);
+}
+
+void SoftmaxLayer::PreprocessGpuVocabIndices(const int *p_host_output_vocab_indices_target,
+                                             int current_target_length, int minibatch_size) {
+  const size_t n = (size_t)minibatch_size * current_target_length;
+  if (n > p_device_output_vocab_indices_.size())
+    throw LinmtError("SoftmaxLayer::PreprocessGpuVocabIndices: target longer than longest_sentence_");
+  hipStream_t s = p_neural_mt_->stream_;
+  p_device_output_vocab_indices_.Upload(p_host_output_vocab_indices_target, n, s);
+  // VocabSoftmaxKernel rewrites -1 -> 0 in place and builds both masks (deep_rnn_kernel.h:144-155)
+  LhErrorWrapper(lh_preprocess_indices_i32(p_device_output_vocab_indices_.get(), (int)n,
+                                           p_device_output_vocab_indices_.get(),
+                                           p_device_output_vocab_indices_01_.get(),
+                                           p_device_output_vocab_indices_01_float_.get(), s),
+                 "SoftmaxLayer::PreprocessGpuVocabIndices");
+  current_minibatch_ = minibatch_size;
+}
+
+void SoftmaxLayer::BackPropPreprocessGpu(float *p_device_h_t, int step) {
+  // layer_loss.h:630-650: select the target ids / masks of this step (step = t * minibatch)
+  (void)p_device_h_t;
+  p_device_output_vocab_indices_single_ = p_device_output_vocab_indices_.get() + step;
+  p_device_output_vocab_indices_01_single_ = p_device_output_vocab_indices_01_.get() + step;
+}
+
+void SoftmaxLayer::ComputeLogits(float *p_device_h_t, int minibatch) {
+  // D*h with the bias of MatrixBiasKernel (deep_rnn_kernel.h:525) folded into the epilogue
+  lh_gemm_seg seg{p_device_d_.get(), output_vocab_size_, p_device_h_t, lstm_size_, lstm_size_};
+  LhErrorWrapper(lh_gemm_f32(output_vocab_size_, minibatch, &seg, 1, 0, 0, 1.f, 0.f,
+                             p_device_b_d_.get(), LH_ACT_NONE, nullptr, p_device_outputdist_.get(),
+                             output_vocab_size_, p_neural_mt_->stream_),
+                 "SoftmaxLayer::GetDistributionGpu p_device_outputdist");
+}
+
+void SoftmaxLayer::GetDistributionGpu(float *p_device_h_t) {
+  hipStream_t s = p_neural_mt_->stream_;
+  const int V = output_vocab_size_, B = current_minibatch_;
+  ComputeLogits(p_device_h_t, B);
+  LhErrorWrapper(lh_softmax_fwd_f32(p_device_outputdist_.get(), V, nullptr, V, B,
+                                    p_device_outputdist_.get(), V, s),
+                 "SoftmaxLayer::GetDistributionGpu softmax");
+  if (training_perplexity_mode_)
+    LhErrorWrapper(lh_train_loglik_f32(p_device_outputdist_.get(), V, V, B,
+                                       p_device_output_vocab_indices_single_,
+                                       p_device_output_vocab_indices_01_single_,
+                                       p_device_train_perplexity_.get(), s),
+                   "SoftmaxLayer::GetDistributionGpu train perplexity");
+}
+
+void SoftmaxLayer::ForwardProp(int index) { GetDistributionGpu(v_h_t_[index]); }
+
+void SoftmaxLayer::GetDistributionGpuDecoderWrapper() { GetDistributionGpu(v_h_t_[0]); }
+
+// GetPerplexityGpu + the host loop of ComputeLossGpu (layer_loss.h:673-750) as one fused pass; the
+// masked sum is accumulated on the device into p_device_loss_ and also returned for this step.
+double SoftmaxLayer::ComputeLossGpu(int index) {
+  hipStream_t s = p_neural_mt_->stream_;
+  const int V = output_vocab_size_, B = current_minibatch_;
+  double before = 0, after = 0;
+  p_device_loss_.Download(&before, 1, s);
+  ComputeLogits(v_h_t_[index], B);
+  LhErrorWrapper(lh_logsoftmax_xent_f32(p_device_outputdist_.get(), V, nullptr, V, B,
+                                        p_device_output_vocab_indices_single_,
+                                        p_device_output_vocab_indices_01_single_,
+                                        p_device_logp_tgt_.get(), p_device_loss_.get(), s),
+                 "SoftmaxLayer::ComputeLossGpu");
+  p_device_loss_.Download(&after, 1, s);
+  HipErrorWrapper(hipStreamSynchronize(s), "SoftmaxLayer::ComputeLossGpu");
+  return after - before;
+}
+
+double SoftmaxLayer::GetTrainPerplexity() {
+  hipStream_t s = p_neural_mt_->stream_;
+  double v = 0;
+  p_device_train_perplexity_.Download(&v, 1, s);
+  HipErrorWrapper(hipStreamSynchronize(s), "SoftmaxLayer::GetTrainPerplexity");
+  p_device_train_perplexity_.Zero(s);
+  return v;
+}
+
+bool SoftmaxLayer::SetParam(const std::string &name, const float *host, size_t n) {
+  hipStream_t s = p_neural_mt_->stream_;
+  if (name == "D") return SetFlat(p_device_d_, host, n, s);
+  if (name == "b_d") return SetFlat(p_device_b_d_, host, n, s);
+  return false;
+}
+
+bool SoftmaxLayer::GetParam(const std::string &name, std::vector<float> *out) {
+  hipStream_t s = p_neural_mt_->stream_;
+  if (name == "D") return GetFlat(p_device_d_, out, s);
+  if (name == "b_d") return GetFlat(p_device_b_d_, out, s);
+  return false;
+}
+
+}  // namespace linmt

@@ -1,0 +1,548 @@
+// NeuralMachineTranslation: model wiring and the forward drivers (scoring and batched beam decode).
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <numeric>
+
+#include "nmt.h"
+
+namespace linmt {
+
+NeuralMachineTranslation::NeuralMachineTranslation(const GlobalConfiguration &cfg) : cfg_(cfg) {
+  if (cfg_.embedding_size_ <= 0) cfg_.embedding_size_ = cfg_.lstm_size_;
+  HipErrorWrapper(hipStreamCreate(&stream_), "stream creation failed");
+}
+
+NeuralMachineTranslation::~NeuralMachineTranslation() {
+  if (stream_) {
+    (void)hipStreamSynchronize(stream_);
+    (void)hipStreamDestroy(stream_);
+  }
+}
+
+void NeuralMachineTranslation::Synchronize() {
+  HipErrorWrapper(hipStreamSynchronize(stream_), "stream synchronize failed");
+}
+
+// One node per timestep on both sides, minibatch = cfg.minibatch_size_ (deep_rnn.h:249-692).
+void NeuralMachineTranslation::InitModel() {
+  decode_mode_ = false;
+  const int B = cfg_.minibatch_size_, T = cfg_.longest_sentence_, L = cfg_.num_layers_;
+  const bool seq2seq = cfg_.sequence_to_sequence_mode_;
+  if (seq2seq) {
+    input_layer_source_.Init(this, true, true, 0, B, T, false, false);
+    for (int l = 1; l < L; ++l) {
+      v_hidden_layers_source_.emplace_back(new LstmLayer());
+      v_hidden_layers_source_.back()->Init(this, false, true, l, B, T, false, false);
+    }
+  }
+  input_layer_target_.Init(this, true, false, 0, B, T, false, false);
+  for (int l = 1; l < L; ++l) {
+    v_hidden_layers_target_.emplace_back(new LstmLayer());
+    v_hidden_layers_target_.back()->Init(this, false, false, l, B, T, false, false);
+  }
+  if (cfg_.attention_mode_ && seq2seq) {
+    attention_layer_.Init(this, B, T, T);
+    LstmLayer &top_src = SourceLayer(L - 1);
+    attention_layer_.p_device_total_hs_ = top_src.h_all_.get();
+    attention_layer_.hs_step_stride_ = (long long)cfg_.lstm_size_ * B;
+    attention_layer_.hs_col_stride_ = cfg_.lstm_size_;
+    attention_layer_.use_hs_col_ = false;
+    if (cfg_.feed_input_mode_) input_layer_target_.InitFeedInput();
+  }
+  softmax_layer_.Init(this, B, T);
+  // wiring that does not change between minibatches: h_below and h~ pointers
+  for (int side = 0; side < (seq2seq ? 2 : 1); ++side) {
+    for (int l = 1; l < L; ++l) {
+      LstmLayer &below = side == 0 && seq2seq ? SourceLayer(l - 1) : TargetLayer(l - 1);
+      LstmLayer &cur = side == 0 && seq2seq ? SourceLayer(l) : TargetLayer(l);
+      for (int t = 0; t < T; ++t) cur.v_nodes_[t].p_device_h_t_below_ = below.v_nodes_[t].p_device_h_t_;
+    }
+  }
+  Synchronize();
+}
+
+// Source side: n_sent columns, one node per source position (the states are needed by attention);
+// target side: ONE node, n_sent*beam columns, previous-state buffers (deep_rnn.h:697-922).
+void NeuralMachineTranslation::InitModelDecoding(int n_sent, int beam_size) {
+  decode_mode_ = true;
+  n_sent_ = n_sent;
+  beam_size_ = beam_size;
+  const int L = cfg_.num_layers_, T = cfg_.longest_sentence_, H = cfg_.lstm_size_;
+  const int B = n_sent * beam_size;
+  input_layer_source_.Init(this, true, true, 0, n_sent, T, false, false);
+  for (int l = 1; l < L; ++l) {
+    v_hidden_layers_source_.emplace_back(new LstmLayer());
+    v_hidden_layers_source_.back()->Init(this, false, true, l, n_sent, T, false, false);
+    for (int t = 0; t < T; ++t)
+      v_hidden_layers_source_.back()->v_nodes_[t].p_device_h_t_below_ =
+          SourceLayer(l - 1).v_nodes_[t].p_device_h_t_;
+  }
+  input_layer_target_.Init(this, true, false, 0, B, 1, false, true);
+  for (int l = 1; l < L; ++l) {
+    v_hidden_layers_target_.emplace_back(new LstmLayer());
+    v_hidden_layers_target_.back()->Init(this, false, false, l, B, 1, false, true);
+    v_hidden_layers_target_.back()->v_nodes_[0].p_device_h_t_below_ =
+        TargetLayer(l - 1).v_nodes_[0].p_device_h_t_;
+  }
+  if (cfg_.attention_mode_) {
+    attention_layer_.Init(this, B, 1, T);
+    LstmLayer &top_src = SourceLayer(L - 1);
+    attention_layer_.p_device_total_hs_ = top_src.h_all_.get();
+    attention_layer_.hs_step_stride_ = (long long)H * n_sent;
+    attention_layer_.hs_col_stride_ = H;
+    attention_layer_.use_hs_col_ = true;
+    if (cfg_.feed_input_mode_) {
+      input_layer_target_.InitFeedInput();
+      p_device_h_tild_previous_.Alloc((size_t)H * B);
+      p_device_h_tild_previous_.Zero(stream_);
+      input_layer_target_.v_nodes_[0].p_device_h_tild_ = p_device_h_tild_previous_.get();
+    }
+  }
+  softmax_layer_.Init(this, B, 1);
+  std::vector<int> ones(B, 1), sent(B);
+  for (int b = 0; b < B; ++b) sent[b] = b / beam_size;
+  p_device_ones_.Alloc(B);
+  p_device_ones_.Upload(ones.data(), B, stream_);
+  p_device_sentence_of_column_.Alloc(B);
+  p_device_sentence_of_column_.Upload(sent.data(), B, stream_);
+  if (cfg_.attention_mode_) attention_layer_.p_device_hs_col_.Upload(sent.data(), B, stream_);
+  decoder_.Init(beam_size, n_sent, T);
+  Synchronize();
+}
+
+bool NeuralMachineTranslation::SetParam(const std::string &name, const float *host, size_t n) {
+  // "src.<l>.<leaf>", "tgt.<l>.<leaf>", "attn.<leaf>", "softmax.<leaf>"
+  const size_t d1 = name.find('.');
+  if (d1 == std::string::npos) return false;
+  const std::string head = name.substr(0, d1);
+  if (head == "attn") return cfg_.attention_mode_ && attention_layer_.SetParam(name.substr(d1 + 1), host, n);
+  if (head == "softmax") return softmax_layer_.SetParam(name.substr(d1 + 1), host, n);
+  const size_t d2 = name.find('.', d1 + 1);
+  if (d2 == std::string::npos) return false;
+  const int l = std::atoi(name.substr(d1 + 1, d2 - d1 - 1).c_str());
+  if (l < 0 || l >= cfg_.num_layers_) return false;
+  const std::string leaf = name.substr(d2 + 1);
+  if (head == "src") return cfg_.sequence_to_sequence_mode_ && SourceLayer(l).SetParam(leaf, host, n);
+  if (head == "tgt") return TargetLayer(l).SetParam(leaf, host, n);
+  return false;
+}
+
+bool NeuralMachineTranslation::GetParam(const std::string &name, std::vector<float> *out) {
+  const size_t d1 = name.find('.');
+  if (d1 == std::string::npos) return false;
+  const std::string head = name.substr(0, d1);
+  if (head == "attn") return cfg_.attention_mode_ && attention_layer_.GetParam(name.substr(d1 + 1), out);
+  if (head == "softmax") return softmax_layer_.GetParam(name.substr(d1 + 1), out);
+  const size_t d2 = name.find('.', d1 + 1);
+  if (d2 == std::string::npos) return false;
+  const int l = std::atoi(name.substr(d1 + 1, d2 - d1 - 1).c_str());
+  if (l < 0 || l >= cfg_.num_layers_) return false;
+  const std::string leaf = name.substr(d2 + 1);
+  if (head == "src") return cfg_.sequence_to_sequence_mode_ && SourceLayer(l).GetParam(leaf, out);
+  if (head == "tgt") return TargetLayer(l).GetParam(leaf, out);
+  return false;
+}
+
+// Teacher-forced forward + log-likelihood of the targets (deep_rnn.h:2173-2317).  Index arrays are
+// B x length column-major with -1 padding; source reversed and left-padded, target right-padded
+// (input_file_preprocess.cc:633,684-690).
+double NeuralMachineTranslation::GetError(const int *p_host_source, int source_length,
+                                          const int *p_host_target_in,
+                                          const int *p_host_target_out, int target_length,
+                                          const int *p_host_batch_information, int minibatch_size) {
+  if (decode_mode_) throw LinmtError("GetError: model was initialised for decoding");
+  const int L = cfg_.num_layers_, B = minibatch_size;
+  if (B > cfg_.minibatch_size_ || source_length > cfg_.longest_sentence_ ||
+      target_length > cfg_.longest_sentence_)
+    throw LinmtError("GetError: minibatch exceeds the allocated size");
+  const bool seq2seq = cfg_.sequence_to_sequence_mode_;
+  if (seq2seq) {
+    for (int l = 0; l < L; ++l)
+      SourceLayer(l).PreprocessGpuVocabIndices(p_host_source, source_length, B);
+  }
+  for (int l = 0; l < L; ++l) TargetLayer(l).PreprocessGpuVocabIndices(p_host_target_in, target_length, B);
+  softmax_layer_.PreprocessGpuVocabIndices(p_host_target_out, target_length, B);
+  const bool attention = cfg_.attention_mode_ && seq2seq;
+  if (attention) {
+    attention_layer_.PreprocessMinibatchInformation(p_host_batch_information, B);
+    // the batch information is uploaded for B columns: lengths at [0,B), offsets at [B,2B)
+    attention_layer_.hs_step_stride_ = (long long)cfg_.lstm_size_ * SourceLayer(L - 1).minibatch_size_;
+    attention_layer_.hs_steps_ = source_length;
+  }
+  softmax_layer_.p_device_loss_.Zero(stream_);
+
+  if (seq2seq) {
+    for (int t = 0; t < source_length; ++t) {
+      const size_t step = (size_t)t * B;
+      for (int l = 0; l < L; ++l) {
+        LstmLayer &Ls = SourceLayer(l);
+        LstmNode &n = Ls.v_nodes_[t];
+        n.minibatch_size_ = B;
+        float *hp = t == 0 ? Ls.p_device_init_hidden_vec_.get() : Ls.v_nodes_[t - 1].p_device_h_t_;
+        float *cp = t == 0 ? Ls.p_device_init_cell_vec_.get() : Ls.v_nodes_[t - 1].p_device_c_t_;
+        if (l == 0)
+          n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_full_.get() + step,
+                                    Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+        else
+          n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+        n.ForwardProp();
+      }
+    }
+  }
+  for (int t = 0; t < target_length; ++t) {
+    const size_t step = (size_t)t * B;
+    for (int l = 0; l < L; ++l) {
+      LstmLayer &Lt = TargetLayer(l);
+      LstmNode &n = Lt.v_nodes_[t];
+      n.minibatch_size_ = B;
+      float *hp, *cp;
+      if (t == 0) {
+        if (seq2seq) {  // encoder layer l at the last source step (deep_rnn.h:2259-2265)
+          hp = SourceLayer(l).v_nodes_[source_length - 1].p_device_h_t_;
+          cp = SourceLayer(l).v_nodes_[source_length - 1].p_device_c_t_;
+        } else {
+          hp = Lt.p_device_init_hidden_vec_.get();
+          cp = Lt.p_device_init_cell_vec_.get();
+        }
+      } else {
+        hp = Lt.v_nodes_[t - 1].p_device_h_t_;
+        cp = Lt.v_nodes_[t - 1].p_device_c_t_;
+      }
+      if (l == 0) {
+        n.UpdateVectorsForwardGpu(Lt.p_device_input_vocab_indices_full_.get() + step,
+                                  Lt.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+        if (attention && cfg_.feed_input_mode_ && t > 0)
+          n.p_device_h_tild_ = attention_layer_.v_nodes_[t - 1].p_device_final_tmp_2_;
+      } else {
+        n.UpdateVectorsForwardGpu(Lt.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+      }
+      n.ForwardProp();
+    }
+    float *top = TargetLayer(L - 1).v_nodes_[t].p_device_h_t_;
+    if (attention) {
+      AttentionNode &an = attention_layer_.v_nodes_[t];
+      an.minibatch_size_ = B;
+      an.p_device_h_t_ = top;
+      an.p_device_indices_mask_ = TargetLayer(L - 1).p_device_input_vocab_indices_01_full_.get() + step;
+      an.ForwardProp();
+      top = an.p_device_final_tmp_2_;
+    }
+    softmax_layer_.SetHTPtr(t, top);
+    softmax_layer_.BackPropPreprocessGpu(top, (int)step);
+    // ComputeLossGpu without the per-step host read-back: accumulate on the device
+    softmax_layer_.ComputeLogits(top, B);
+    LhErrorWrapper(
+        lh_logsoftmax_xent_f32(softmax_layer_.p_device_outputdist_.get(), cfg_.target_vocab_size_,
+                               nullptr, cfg_.target_vocab_size_, B,
+                               softmax_layer_.p_device_output_vocab_indices_single_,
+                               softmax_layer_.p_device_output_vocab_indices_01_single_,
+                               softmax_layer_.p_device_logp_tgt_.get(),
+                               softmax_layer_.p_device_loss_.get(), stream_),
+        "GetError loss");
+  }
+  double loss = 0;
+  softmax_layer_.p_device_loss_.Download(&loss, 1, stream_);
+  Synchronize();
+  return loss;
+}
+
+// Encoder for n_sent sentences at once; ids are n_sent x source_length column-major, reversed and
+// left-padded with -1, so that every sentence ends at the last step and padded prefixes keep the
+// state at exactly zero (deep_rnn.h:1572-1646 runs one sentence with B = 1).
+void NeuralMachineTranslation::ForwardPropSource(const int *p_host_source, int source_length,
+                                                 int n_sent) {
+  const int L = cfg_.num_layers_;
+  for (int l = 0; l < L; ++l) SourceLayer(l).PreprocessGpuVocabIndices(p_host_source, source_length, n_sent);
+  for (int t = 0; t < source_length; ++t) {
+    const size_t step = (size_t)t * n_sent;
+    for (int l = 0; l < L; ++l) {
+      LstmLayer &Ls = SourceLayer(l);
+      LstmNode &n = Ls.v_nodes_[t];
+      n.minibatch_size_ = n_sent;
+      float *hp = t == 0 ? Ls.p_device_init_hidden_vec_.get() : Ls.v_nodes_[t - 1].p_device_h_t_;
+      float *cp = t == 0 ? Ls.p_device_init_cell_vec_.get() : Ls.v_nodes_[t - 1].p_device_c_t_;
+      if (l == 0)
+        n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_full_.get() + step,
+                                  Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+      else
+        n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+      n.ForwardProp();
+    }
+  }
+}
+
+void NeuralMachineTranslation::ForwardPropTarget(int curr_index, int *p_device_current_indices,
+                                                 int minibatch) {
+  const int L = cfg_.num_layers_;
+  input_layer_target_.v_nodes_[0].index_ = curr_index;  // deep_rnn.h:1760
+  for (int l = 0; l < L; ++l) {
+    LstmLayer &Lt = TargetLayer(l);
+    LstmNode &n = Lt.v_nodes_[0];
+    n.minibatch_size_ = minibatch;
+    if (l == 0)
+      n.UpdateVectorsForwardGpu(p_device_current_indices, p_device_ones_.get(),
+                                Lt.p_device_h_t_previous_.get(), Lt.p_device_c_t_previous_.get());
+    else
+      n.UpdateVectorsForwardGpu(p_device_ones_.get(), Lt.p_device_h_t_previous_.get(),
+                                Lt.p_device_c_t_previous_.get());
+    n.ForwardProp();
+  }
+  float *top = TargetLayer(L - 1).v_nodes_[0].p_device_h_t_;
+  if (cfg_.attention_mode_) {
+    AttentionNode &an = attention_layer_.v_nodes_[0];
+    an.minibatch_size_ = minibatch;
+    an.p_device_h_t_ = top;
+    an.p_device_indices_mask_ = p_device_ones_.get();
+    an.ForwardProp();
+    top = an.p_device_final_tmp_2_;
+  }
+  softmax_layer_.SetHTPtr(0, top);
+  softmax_layer_.ComputeLogits(top, minibatch);
+}
+
+void NeuralMachineTranslation::SwapDecodingStates(const int *p_device_backptr, int minibatch) {
+  const int L = cfg_.num_layers_;
+  const float *src[LH_GATHER_MAX_TENSORS];
+  float *dst[LH_GATHER_MAX_TENSORS];
+  int n = 0;
+  for (int l = 0; l < L; ++l) {
+    LstmLayer &Lt = TargetLayer(l);
+    src[n] = Lt.v_nodes_[0].p_device_h_t_;
+    dst[n++] = Lt.p_device_h_t_previous_.get();
+    src[n] = Lt.v_nodes_[0].p_device_c_t_;
+    dst[n++] = Lt.p_device_c_t_previous_.get();
+  }
+  if (cfg_.attention_mode_ && cfg_.feed_input_mode_) {
+    src[n] = attention_layer_.v_nodes_[0].p_device_final_tmp_2_;
+    dst[n++] = p_device_h_tild_previous_.get();
+  }
+  LhErrorWrapper(lh_beam_gather_f32(src, dst, n, cfg_.lstm_size_, minibatch, minibatch,
+                                    p_device_backptr, stream_),
+                 "SwapDecodingStates");
+}
+
+// ---------------------------------------------------------------------------------------------
+void Decoder::Init(int beam_size, int n_sent, int max_steps) {
+  beam_size_ = beam_size;
+  n_sent_ = n_sent;
+  max_steps_ = max_steps;
+  const size_t B = (size_t)beam_size * n_sent, K = beam_size + 1, T = max_steps;
+  cand_logp_.Alloc(K * B);
+  cand_id_.Alloc(K * B);
+  logp_eof_.Alloc(B);
+  score_[0].Alloc(B);
+  score_[1].Alloc(B);
+  limit_.Alloc(n_sent);
+  current_indices_.Alloc(B);
+  tok_hist_.Alloc(T * B);
+  backptr_hist_.Alloc(T * B);
+  score_hist_.Alloc(T * B);
+  fin_count_hist_.Alloc(T * n_sent);
+  fin_beam_hist_.Alloc(T * B);
+  fin_score_hist_.Alloc(T * B);
+}
+
+// Length normalisation, coverage penalty, minimum-ratio filter, best-first (decoder.h:529-600);
+// with alignment export off every alignment-score row is the all-zero vector the reference starts
+// from (decoder.h:364-370), which is what the coverage term is computed from here too.
+void Decoder::OutputKBestHypotheses(const std::vector<Hypothesis> &hyps, int source_length,
+                                    const DecodeOptions &o, SentenceResult *out) {
+  int best = -1;
+  float best_score = 0.f;
+  for (size_t i = 0; i < hyps.size(); ++i) {
+    float s = hyps[i].score;
+    const int size = (int)hyps[i].tokens.size();
+    if (0 != o.lp_alpha_) {
+      const float lp = powf((float)(5 + size), o.lp_alpha_) / powf((float)(5 + 1), o.lp_alpha_);
+      s /= lp;
+    }
+    if (0 != o.cp_beta_) {
+      float sum = 0;
+      for (int k = 0; k < source_length; ++k) sum += 0.01f;
+      const float unit = 0.01f / sum;
+      float cp_x_y = 0;
+      for (int k = 0; k < source_length; ++k) {
+        float col = 0;
+        for (int j = 1; j < size - 1; ++j) col += unit;
+        cp_x_y += std::log(std::min(col, 1.0f));
+      }
+      cp_x_y *= o.cp_beta_;
+      if (cp_x_y < -20) cp_x_y = -20;
+      s += cp_x_y;
+    }
+    const float len_ratio = ((float)size) / source_length;
+    if (len_ratio > o.min_decoding_ratio_ && (best < 0 || best_score < s)) {
+      best = (int)i;
+      best_score = s;
+    }
+  }
+  out->best.clear();
+  out->best_score = 0.f;
+  if (best >= 0) {
+    const std::vector<int> &t = hyps[best].tokens;
+    out->best.assign(t.begin() + 1, t.end() - 1);
+    out->best_score = best_score;
+  }
+}
+
+// Batched EnsembleFactory::DecodeFile (decoder.h:1702-1776), one model.  Sentences are processed
+// longest first so that at every step the still-active sentences are a prefix of the columns and
+// the kernels simply run on fewer columns as sentences reach their length limit.
+void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &sentences,
+                                           const DecodeOptions &o,
+                                           std::vector<SentenceResult> *results) {
+  if (!decode_mode_) throw LinmtError("DecodeBatch: call InitModelDecoding first");
+  const int n = (int)sentences.size();
+  int beam = o.beam_size_;
+  if (beam > (int)std::sqrt((double)cfg_.target_vocab_size_))  // decoder.h:1662-1664
+    beam = (int)std::sqrt((double)cfg_.target_vocab_size_);
+  if (n < 1 || n > n_sent_ || beam != beam_size_)
+    throw LinmtError("DecodeBatch: batch does not match InitModelDecoding(n_sent, beam)");
+  const int longest = cfg_.longest_sentence_;
+  std::vector<int> order(n);
+  std::iota(order.begin(), order.end(), 0);
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
+    return sentences[a].size() > sentences[b].size();
+  });
+  const int S = (int)sentences[order[0]].size();
+  if (S < 1 || S > longest) throw LinmtError("DecodeBatch: source sentence length out of range");
+  if (sentences[order[n - 1]].empty()) throw LinmtError("DecodeBatch: empty source sentence");
+
+  // reversed, left-padded source block; per-sentence step limits; attention batch information
+  std::vector<int> src((size_t)n * S, -1), limit(n), binfo(2 * (size_t)n * beam);
+  int max_limit = 0;
+  for (int k = 0; k < n; ++k) {
+    const std::vector<int> &w = sentences[order[k]];
+    const int len = (int)w.size();
+    for (int t = 0; t < len; ++t) src[(size_t)(S - len + t) * n + k] = w[len - 1 - t];
+    limit[k] = std::min((int)(o.max_decoding_ratio_ * len), longest - 2);  // decoder.h:1734
+    max_limit = std::max(max_limit, limit[k]);
+    for (int j = 0; j < beam; ++j) {
+      binfo[(size_t)k * beam + j] = len;
+      binfo[(size_t)n * beam + (size_t)k * beam + j] = S - len;
+    }
+  }
+  const int B = n * beam, K = beam + 1, H = cfg_.lstm_size_, L = cfg_.num_layers_;
+  Decoder &d = decoder_;
+  if (max_limit + 1 > d.max_steps_) throw LinmtError("DecodeBatch: too many decoding steps");
+
+  // InitDecoder (decoder.h:334-350): <START> everywhere, scores 0
+  std::vector<int> start(B, Decoder::start_symbol_);
+  d.current_indices_.Upload(start.data(), B, stream_);
+  d.score_[0].Zero(stream_);
+  d.limit_.Upload(limit.data(), n, stream_);
+  if (cfg_.attention_mode_) {
+    attention_layer_.PreprocessMinibatchInformation(binfo.data(), B);
+    attention_layer_.hs_step_stride_ = (long long)H * SourceLayer(L - 1).minibatch_size_;
+    attention_layer_.hs_steps_ = S;
+    if (attention_layer_.global_mode_ && S > attention_layer_.window_)
+      throw LinmtError("DecodeBatch: source longer than the attention window");
+  }
+
+  // the encoder layers were allocated for n_sent_ columns; run them on n (ld is lstm_size_, so a
+  // smaller batch simply uses the first n columns of every step's buffer)
+  if (n != n_sent_ && cfg_.attention_mode_)
+    attention_layer_.hs_step_stride_ = (long long)H * n_sent_;
+  ForwardPropSource(src.data(), S, n);
+
+  // TransferDecodingStatesGpu (layer_input_to_hidden.h:1536-1545): encoder's final (h, c) of layer
+  // l, sentence s -> every beam column of s.
+  {
+    const float *gs[LH_GATHER_MAX_TENSORS];
+    float *gd[LH_GATHER_MAX_TENSORS];
+    int g = 0;
+    for (int l = 0; l < L; ++l) {
+      gs[g] = SourceLayer(l).v_nodes_[S - 1].p_device_h_t_;
+      gd[g++] = TargetLayer(l).p_device_h_t_previous_.get();
+      gs[g] = SourceLayer(l).v_nodes_[S - 1].p_device_c_t_;
+      gd[g++] = TargetLayer(l).p_device_c_t_previous_.get();
+    }
+    LhErrorWrapper(lh_beam_gather_f32(gs, gd, g, H, B, n, p_device_sentence_of_column_.get(), stream_),
+                   "TransferDecodingStatesGpu");
+  }
+
+  int cur = 0;
+  std::vector<int> active_at(max_limit + 1);
+  std::vector<std::vector<int>> bi_keep;
+  for (int step = 0; step <= max_limit; ++step) {
+    int n_active = 0;
+    while (n_active < n && limit[n_active] >= step) ++n_active;  // limits are non-increasing
+    active_at[step] = n_active;
+    const int Ba = n_active * beam;
+    if (cfg_.attention_mode_ && (step == 0 || n_active != active_at[step - 1])) {
+      // the batch information is [len_0..len_{Ba-1}, off_0..off_{Ba-1}] for the columns in use, so
+      // it is laid out again whenever the number of active columns changes
+      bi_keep.emplace_back(2 * (size_t)Ba);  // kept alive until the stream has been synchronised
+      std::vector<int> &bi = bi_keep.back();
+      for (int b = 0; b < Ba; ++b) {
+        bi[b] = binfo[b];
+        bi[(size_t)Ba + b] = binfo[(size_t)B + b];
+      }
+      attention_layer_.PreprocessMinibatchInformation(bi.data(), Ba);
+    }
+    ForwardPropTarget(step, d.current_indices_.get(), Ba);
+    LhErrorWrapper(lh_beam_topk_f32(softmax_layer_.GetDistPtr(), cfg_.target_vocab_size_, nullptr,
+                                    cfg_.target_vocab_size_, Ba, K, Decoder::end_symbol_,
+                                    d.cand_logp_.get(), d.cand_id_.get(), d.logp_eof_.get(), stream_),
+                   "beam top-k");
+    const size_t off = (size_t)step * B;
+    LhErrorWrapper(
+        lh_beam_merge_f32(n_active, beam, K, step, d.limit_.get(), d.cand_logp_.get(),
+                          d.cand_id_.get(), d.logp_eof_.get(), d.score_[cur].get(), o.diversity_,
+                          o.penalty_, Decoder::start_symbol_, Decoder::end_symbol_,
+                          d.tok_hist_.get() + off, d.backptr_hist_.get() + off,
+                          d.score_[cur ^ 1].get(), d.fin_count_hist_.get() + (size_t)step * n,
+                          d.fin_beam_hist_.get() + off, d.fin_score_hist_.get() + off, stream_),
+        "beam merge");
+    cur ^= 1;
+    if (step < max_limit) {
+      SwapDecodingStates(d.backptr_hist_.get() + off, Ba);
+      HipErrorWrapper(hipMemcpyAsync(d.current_indices_.get(), d.tok_hist_.get() + off,
+                                     sizeof(int) * Ba, hipMemcpyDeviceToDevice, stream_),
+                      "current indices copy");
+    }
+  }
+
+  // one read-back for the whole batch
+  const size_t steps = (size_t)max_limit + 1;
+  std::vector<int> tok(steps * B), bp(steps * B), fcount(steps * n), fbeam(steps * B);
+  std::vector<float> fscore(steps * B);
+  d.tok_hist_.Download(tok.data(), tok.size(), stream_);
+  d.backptr_hist_.Download(bp.data(), bp.size(), stream_);
+  d.fin_count_hist_.Download(fcount.data(), fcount.size(), stream_);
+  d.fin_beam_hist_.Download(fbeam.data(), fbeam.size(), stream_);
+  d.fin_score_hist_.Download(fscore.data(), fscore.size(), stream_);
+  Synchronize();
+
+  // Rebuild v_hypotheses_ by walking the back-pointers (equivalent to the row copies of
+  // eigen_top_sentences_ in decoder.h:440-471).
+  results->assign(n, SentenceResult());
+  for (int k = 0; k < n; ++k) {
+    SentenceResult &r = (*results)[order[k]];
+    r.steps = limit[k] + 1;
+    const int c0 = k * beam;
+    auto prefix = [&](int step, int column, std::vector<int> *out) {
+      // tokens chosen at steps 0..step-1 along the path that ends in `column` before step `step`
+      out->assign(step + 1, Decoder::start_symbol_);
+      int col = column;
+      for (int t = step - 1; t >= 0; --t) {
+        (*out)[t + 1] = tok[(size_t)t * B + col];
+        col = bp[(size_t)t * B + col];
+      }
+    };
+    for (int step = 0; step <= limit[k]; ++step) {
+      const int nf = fcount[(size_t)step * n + k];
+      for (int f = 0; f < nf; ++f) {
+        Hypothesis h;
+        prefix(step, c0 + fbeam[(size_t)step * B + c0 + f], &h.tokens);
+        h.tokens.push_back(Decoder::end_symbol_);
+        h.score = fscore[(size_t)step * B + c0 + f];
+        r.hypotheses.push_back(std::move(h));
+      }
+    }
+    Decoder::OutputKBestHypotheses(r.hypotheses, (int)sentences[order[k]].size(), o, &r);
+  }
+}
+
+}  // namespace linmt

@@ -56,7 +56,7 @@ SIGNATURES = {
                                     c_f32p, c_f32p, C.c_float, C.c_float, C.c_int, C.c_int, c_i32p,
                                     c_i32p, c_f32p, c_i32p, c_i32p, c_f32p, C.c_void_p]),
     "lh_beam_gather_f32": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int,
-                                     C.c_int, C.c_int, c_i32p, C.c_void_p]),
+                                     C.c_int, C.c_int, C.c_int, c_i32p, C.c_void_p]),
 }
 
 _lib = None
@@ -187,9 +187,10 @@ def beam_merge(n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof, prev_
                                    _stream(stream)), "lh_beam_merge_f32")
 
 
-def beam_gather(src, dst, H, B, backptr, stream=None):
+def beam_gather(src, dst, H, B, backptr, B_src=None, stream=None):
     n = len(src)
+    B_src = B if B_src is None else B_src
     s = (C.c_void_p * n)(*[t.data_ptr() for t in src])
     d = (C.c_void_p * n)(*[t.data_ptr() for t in dst])
-    check(load().lh_beam_gather_f32(s, d, n, H, B, _ptr(backptr), _stream(stream)),
+    check(load().lh_beam_gather_f32(s, d, n, H, B, B_src, _ptr(backptr), _stream(stream)),
           "lh_beam_gather_f32")

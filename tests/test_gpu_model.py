@@ -1,0 +1,195 @@
+"""GPU parity of the C++ layer classes (through the C facade of liblinmt_host.so) against the CPU
+oracle on the same seeded weights and inputs: beam decoding (tokens, back-pointer paths and finished
+hypotheses bit-exact; scores within tolerance) and teacher-forced scoring."""
+import numpy as np
+import pytest
+
+from conftest import assert_close
+import ref_numpy as R
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def host():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from linmt_amd import host as h
+    h.load()
+    return h
+
+
+def _pair(orc, host, rng, layers, H, Vs, Vt, D, longest, scale, decoding=None, minibatch=1,
+          attention=1, feed=True):
+    P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(attention), feed_input=feed,
+                      scale=scale)
+    om = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=int(feed),
+                   longest_sent=longest)
+    om.set_params(P)
+    gm = host.Model(layers, H, Vs, Vt, longest_sentence=longest, attention_mode=attention,
+                    attention_width=D, feed_input=feed, minibatch_size=minibatch,
+                    decoding=decoding)
+    gm.set_params(P)
+    return P, om, gm
+
+
+def _compare_decode(orc_res, gpu_res, what):
+    assert gpu_res["best"].tolist() == orc_res["best"].tolist(), f"{what}: 1-best tokens"
+    assert_close(gpu_res["best_score"], orc_res["best_score"], f"{what}: 1-best score", rtol=1e-4,
+                 atol=1e-4)
+    assert gpu_res["steps"] == orc_res["steps"], f"{what}: decoder steps"
+    assert len(gpu_res["hyps"]) == len(orc_res["hyps"]), f"{what}: number of finished hypotheses"
+    for (gt, gs), (wt, ws) in zip(gpu_res["hyps"], orc_res["hyps"]):
+        assert gt.tolist() == wt.tolist(), f"{what}: hypothesis tokens"
+        assert_close(gs, ws, f"{what}: hypothesis score", rtol=1e-4, atol=1e-4)
+
+
+def test_param_roundtrip(orc, host):
+    rng = np.random.default_rng(0)
+    P, om, gm = _pair(orc, host, rng, 2, 16, 20, 23, 2, 20, 0.5, decoding=(2, 3))
+    for name in ("src.0.W", "src.1.M_c", "tgt.0.Q_o", "tgt.1.W_hf", "tgt.0.b_f", "attn.W_a",
+                 "attn.v_p", "softmax.D", "softmax.b_d"):
+        assert np.array_equal(gm.get_param(name, P[name].shape), P[name]), name
+    with pytest.raises(host.HostError):
+        gm.set_params({"tgt.0.nope": np.zeros(3, np.float32)})
+    gm.close()
+
+
+@pytest.mark.parametrize("layers,H,Vs,Vt,D,beam,n_sent,seed",
+                         [(2, 64, 120, 150, 3, 4, 7, 1), (1, 32, 50, 60, 10, 5, 3, 2),
+                          (4, 48, 80, 400, 2, 12, 5, 3)])
+def test_decode_batch_vs_oracle_small(orc, host, layers, H, Vs, Vt, D, beam, n_sent, seed):
+    """Ragged batch of sentences decoded at once equals independent single-sentence searches of the
+    oracle (the reference decodes one sentence at a time, src/decoder.h:1702-1776)."""
+    rng = np.random.default_rng(seed)
+    longest = 40
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, longest, 0.4, decoding=(n_sent, beam))
+    sents = [rng.integers(0, Vs, size=int(rng.integers(1, 16))) for _ in range(n_sent)]
+    sents[0] = rng.integers(0, Vs, size=15)
+    got = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    for i, s in enumerate(sents):
+        want = om.decode_sentence(s, beam=beam)
+        _compare_decode(want, got[i], f"sentence {i} (len {len(s)})")
+    # a second batch with fewer sentences on the same model (state from the first must not leak)
+    got2 = gm.decode_batch(sents[:2], beam=beam, with_hyps=True)
+    for i in range(2):
+        _compare_decode(om.decode_sentence(sents[i], beam=beam), got2[i], f"rerun sentence {i}")
+    gm.close()
+
+
+def test_decode_options_vs_oracle(orc, host):
+    """Penalty, diversity, length normalisation and coverage penalty switched on and off."""
+    rng = np.random.default_rng(4)
+    P, om, gm = _pair(orc, host, rng, 2, 32, 60, 70, 2, 30, 0.5, decoding=(3, 4))
+    sents = [rng.integers(0, 60, size=n) for n in (9, 4, 6)]
+    for kw in (dict(penalty=0.3, diversity=0.1), dict(lp_alpha=0.0, cp_beta=0.0),
+               dict(max_ratio=0.7, min_ratio=0.2), dict(lp_alpha=1.0, cp_beta=0.5, penalty=-0.2)):
+        got = gm.decode_batch(sents, beam=4, with_hyps=True, **kw)
+        for i, s in enumerate(sents):
+            _compare_decode(om.decode_sentence(s, beam=4, **kw), got[i], f"{kw} sentence {i}")
+    gm.close()
+
+
+def test_decode_no_attention_and_no_feed(orc, host):
+    rng = np.random.default_rng(5)
+    for attention, feed in ((0, False), (1, False)):
+        P, om, gm = _pair(orc, host, rng, 2, 32, 60, 70, 2, 30, 0.5, decoding=(3, 3),
+                          attention=attention, feed=feed)
+        sents = [rng.integers(0, 60, size=n) for n in (7, 3, 5)]
+        got = gm.decode_batch(sents, beam=3, with_hyps=True)
+        for i, s in enumerate(sents):
+            _compare_decode(om.decode_sentence(s, beam=3), got[i],
+                            f"attention={attention} feed={feed} sentence {i}")
+        gm.close()
+
+
+def test_decode_config3_architecture(orc, host):
+    """The headline architecture at full width (4+4 layers, H=1000, V=30000, beam 12, local-p D=10,
+    feed input) on a few short sentences the CPU oracle finishes in seconds."""
+    rng = np.random.default_rng(6)
+    layers, H, V, D, beam = 4, 1000, 30000, 10, 12
+    P, om, gm = _pair(orc, host, rng, layers, H, V, V, D, 104, 0.08, decoding=(4, beam))
+    sents = [rng.integers(0, V, size=n) for n in (6, 4, 5, 3)]
+    got = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    for i, s in enumerate(sents):
+        _compare_decode(om.decode_sentence(s, beam=beam), got[i], f"config-3 sentence {i}")
+    gm.close()
+
+
+def _ragged_minibatch(rng, B, S, T, Vs, Vt, min_len=1):
+    lens_s = rng.integers(min_len, S + 1, size=B)
+    lens_t = rng.integers(max(min_len, 2), T + 1, size=B)
+    lens_s[0], lens_t[0] = S, T
+    src = np.full((B, S), -1, np.int32)
+    tin = np.full((B, T), -1, np.int32)
+    tout = np.full((B, T), -1, np.int32)
+    for b in range(B):
+        s = rng.integers(0, Vs, size=lens_s[b])
+        t = rng.integers(3, Vt, size=lens_t[b] - 1)
+        src[b, S - lens_s[b]:] = s[::-1]
+        tin[b, :lens_t[b]] = np.concatenate([[0], t])
+        tout[b, :lens_t[b]] = np.concatenate([t, [1]])
+    bi = np.concatenate([lens_s, S - lens_s]).astype(np.int32)
+    return src, tin, tout, bi, int(lens_t.sum())
+
+
+@pytest.mark.parametrize("layers,H,Vs,Vt,D,B,S,T,attention,feed",
+                         [(2, 64, 90, 110, 3, 9, 12, 10, 1, True),
+                          (4, 128, 300, 500, 10, 16, 20, 18, 1, True),
+                          (2, 64, 90, 110, 3, 9, 12, 10, 2, True),   # global general (build-defined)
+                          (2, 64, 90, 110, 3, 9, 12, 10, 0, False)])
+def test_get_error_vs_oracle(orc, host, layers, H, Vs, Vt, D, B, S, T, attention, feed):
+    rng = np.random.default_rng(7)
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 30, 0.3, minibatch=B,
+                      attention=attention, feed=feed)
+    src, tin, tout, bi, n_words = _ragged_minibatch(rng, B, S, T, Vs, Vt)
+    want = om.forward_xent(src, tin, tout, bi)
+    got = gm.get_error(src, tin, tout, bi)
+    assert_close(got, want, "sum log p(target)", rtol=1e-5, atol=1e-3)
+    assert_close(got / n_words, want / n_words, "per-word log-likelihood", rtol=1e-4, atol=1e-5)
+    # smaller minibatch on the same allocation
+    got2 = gm.get_error(src[:4], tin[:4], tout[:4], np.concatenate([bi[:4], bi[B:B + 4]]))
+    want2 = om.forward_xent(src[:4], tin[:4], tout[:4], np.concatenate([bi[:4], bi[B:B + 4]]))
+    assert_close(got2, want2, "sub-batch", rtol=1e-5, atol=1e-3)
+    # padded source prefix keeps the state at exactly zero; padded target columns are zeroed
+    for b in range(B):
+        pad = S - bi[b]
+        if pad > 0:
+            h = gm.get_state(0, 0, layers - 1, pad - 1, H, B)
+            assert np.all(h[:, b] == 0)
+    gm.close()
+
+
+def test_config1_single_layer_lstm(orc, host):
+    """Config 1: single-layer LSTM, E=H=256, B=32, T=30, V=5000, uniform ids; language-model path
+    (no encoder, no attention).  Final-step log-probs enter through the summed log-likelihood."""
+    rng = np.random.default_rng(8)
+    H, V, B, T = 256, 5000, 32, 30
+    P = R.make_params(rng, 1, H, V, V, attention=False, feed_input=False, scale=0.08)
+    gm = host.Model(1, H, V, V, longest_sentence=34, attention_mode=0, feed_input=False,
+                    minibatch_size=B, sequence_to_sequence=False)
+    gm.set_params({k: v for k, v in P.items() if not k.startswith("src.")})
+    tin = rng.integers(0, V, size=(B, T)).astype(np.int32)
+    tout = rng.integers(0, V, size=(B, T)).astype(np.int32)
+    got = gm.get_error(None, tin, tout, None)
+    # oracle: step the cell by hand with the oracle's kernels-level functions
+    Wih = np.concatenate([P[f"tgt.0.M_{g}"] for g in R.GATES], axis=0)
+    Whh = np.concatenate([P[f"tgt.0.W_h{g}"] for g in R.GATES], axis=0)
+    bias = np.concatenate([P[f"tgt.0.b_{g}"] for g in R.GATES])
+    h = np.zeros((H, B), np.float32)
+    c = np.zeros((H, B), np.float32)
+    want = 0.0
+    ones = np.ones(B, np.int32)
+    for t in range(T):
+        x = orc.embed_lookup(P["tgt.0.W"], tin[:, t])
+        gates, c, h = orc.lstm_cell_fwd(orc.gemm(Wih, x), bias, c, ones, orc.gemm(Whh, h))
+        gh = gm.get_state(0, 1, 0, t, H, B)
+        gc = gm.get_state(1, 1, 0, t, H, B)
+        assert_close(gh, h, f"h_t at t={t}")
+        assert_close(gc, c, f"c_t at t={t}")
+        lp, loss = orc.logsoftmax_xent(orc.gemm(P["softmax.D"], h), P["softmax.b_d"], tout[:, t],
+                                       ones)
+        want += loss
+    assert_close(got, want, "config-1 log-likelihood", rtol=1e-5, atol=1e-3)
+    gm.close()
