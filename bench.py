@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X: beam-12 decoding of the 4+4-layer, 1000-hidden,
+30k-vocabulary encoder-decoder with local-p attention and input feeding (BASELINE.json configs[2]).
+
+One "step" = one pass of the hot path over one batch: a full batched beam search (encoder, every
+decoder step with on-device top-k / merge / state gather, hypothesis read-back) over 64 synthetic
+source sentences.  Prints ONE JSON line (see README / DESIGN.md for the fields).
+
+  python bench.py --gpus 1 --steps K --warmup W
+
+Only one GPU is used; --gpus N with N > 1 exits with a message.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+SEED = 20161030
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_FP32_PEAK_TFLOPS = 157.3
+
+
+def make_params(rng, layers, H, Vs, Vt, scale=0.08):
+    """uniform[-0.08, 0.08], forget-gate bias 1 (reference initialisation)."""
+    P = {}
+    u = lambda *s: rng.uniform(-scale, scale, size=s).astype(np.float32)
+    for side, V in (("src", Vs), ("tgt", Vt)):
+        for l in range(layers):
+            pfx = f"{side}.{l}."
+            for g in "ifco":
+                P[pfx + "W_h" + g] = u(H, H)
+                P[pfx + "M_" + g] = u(H, H)
+                P[pfx + "b_" + g] = u(H)
+                if side == "tgt" and l == 0:
+                    P[pfx + "Q_" + g] = u(H, H)
+            P[pfx + "b_f"] = np.ones(H, np.float32)
+            if l == 0:
+                P[pfx + "W"] = u(H, V)
+    for n in ("W_a", "W_p", "W_c1", "W_c2"):
+        P["attn." + n] = u(H, H)
+    P["attn.v_p"] = u(H)
+    P["attn.b_out"] = u(H)
+    P["softmax.D"] = u(Vt, H)
+    P["softmax.b_d"] = u(Vt)
+    return P
+
+
+def zipf_ids(rng, n, V, s=1.1, lo=0):
+    """Zipf(s) over the ids lo..V-1 (rank 1 = id lo)."""
+    ranks = np.arange(1, V - lo + 1, dtype=np.float64)
+    p = ranks ** (-s)
+    p /= p.sum()
+    return (rng.choice(V - lo, size=n, p=p) + lo).astype(np.int32)
+
+
+def make_sentences(rng, n_sent, V, lo_len=10, hi_len=60):
+    lens = rng.integers(lo_len, hi_len + 1, size=n_sent)
+    return [zipf_ids(rng, int(L), V) for L in lens]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--cpu-sentences", type=int, default=6,
+                    help="sentences of the same workload decoded by the CPU oracle for cpu_baseline")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--profile-level", type=int, default=1,
+                    help="1: HIP events around the output projection during the timed steps; "
+                         "2: one extra untimed pass with every launch bracketed (kernel table)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (the path shards over sentences with no "
+              f"communication; no multi-GPU run is part of it); --gpus {args.gpus} is not supported",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from linmt_amd import host
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    host.load()
+
+    layers, H, V, D, beam, n_sent, longest = 4, 1000, 30000, 10, 12, 64, 104
+    rng = np.random.default_rng(SEED)
+    P = make_params(rng, layers, H, V, V)
+    sents = make_sentences(rng, n_sent, V)
+    model = host.Model(layers, H, V, V, longest_sentence=longest, attention_mode=1,
+                       attention_width=D, feed_input=True, decoding=(n_sent, beam))
+    model.set_params(P)
+
+    for _ in range(args.warmup):
+        model.decode_batch(sents, beam=beam)
+    model.profile(1 if args.profile_level >= 1 else 0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    tokens = 0
+    for _ in range(args.steps):
+        res = model.decode_batch(sents, beam=beam)  # ends with a stream synchronisation
+        tokens += sum(len(r["best"]) for r in res)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    prof1 = model.profile_totals()
+    ms_per_step = dt * 1e3 / args.steps
+    value = tokens / dt
+
+    roofline = None
+    if "logits_gemm" in prof1:
+        g = prof1["logits_gemm"]
+        achieved = g["work"] / (g["ms"] * 1e-3) / 1e12
+        roofline = {"kernel": "gemm_kernel<128,128,2,2,false,false,true> (output projection D*h+b_d)",
+                    "bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP32_PEAK_TFLOPS,
+                    "unit": "TFLOP/s", "frac": round(achieved / MFMA_FP32_PEAK_TFLOPS, 4),
+                    "traffic": None, "launches": g["launches"],
+                    "avg_launch_us": round(g["ms"] * 1e3 / g["launches"], 2)}
+
+    kernels = {}
+    if args.profile_level >= 2:
+        model.profile(2)
+        model.decode_batch(sents, beam=beam)
+        for name, t in model.profile_totals().items():
+            rate = t["work"] / (t["ms"] * 1e-3)
+            is_gemm = name.endswith("gemm")
+            kernels[name] = {"ms": round(t["ms"], 3), "launches": t["launches"],
+                             "rate": round(rate / (1e12 if is_gemm else 1e9), 2),
+                             "unit": "TFLOP/s" if is_gemm else "GB/s",
+                             "frac": round(rate / ((MFMA_FP32_PEAK_TFLOPS * 1e12) if is_gemm
+                                                   else (HBM_PEAK_GBS * 1e9)), 4)}
+        model.profile(0)
+
+    cpu_baseline = None
+    parity = None
+    if not args.no_cpu_baseline and args.cpu_sentences > 0:
+        from oracle import orc  # the checker / reported baseline, never the measured path
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+        om = orc.Model(layers, H, V, V, attention=1, D=D, feed_input=1, longest_sent=longest)
+        om.set_params(P)
+        # bounded sample: the shortest sentences of the same batch (about 10-30 s of CPU work)
+        order = np.argsort([len(s) for s in sents], kind="stable")[: args.cpu_sentences]
+        om.decode_sentence(sents[order[0]][:3], beam=beam, num_threads=cores)  # warm-up
+        c0 = time.perf_counter()
+        cpu_tokens, same = 0, 0
+        for i in order:
+            r = om.decode_sentence(sents[i], beam=beam, num_threads=cores)
+            cpu_tokens += len(r["best"])
+            same += int(r["best"].tolist() == res[i]["best"].tolist())
+        cdt = time.perf_counter() - c0
+        cpu_baseline = {"value": round(cpu_tokens / cdt, 2), "unit": "target tokens/s",
+                        "cores": cores, "kind": "port",
+                        "sample": f"the {len(order)} shortest of the 64 benchmark sentences "
+                                  f"({cpu_tokens} target tokens, {cdt:.1f} s), decoded one at a "
+                                  f"time by the CPU restatement (oracle/) with OpenMP"}
+        parity = {"sentences_checked": int(len(order)), "one_best_identical": int(same)}
+
+    out = {
+        "metric": "target tokens/sec (beam-12 decode, 1 GPU)",
+        "value": round(value, 1),
+        "unit": "target tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 2),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[2]: beam-12 decode, 64 sentences/batch (768 live "
+                               "hypotheses), 4+4 LSTM layers, hidden=emb=1000, vocab 30k/30k, "
+                               "local-p attention D=10 + input feeding, source len U[10,60] Zipf "
+                               "ids, max target 1.5x source, random-init uniform[-0.08,0.08]",
+                   "tokens_per_step": tokens // max(args.steps, 1),
+                   "seed": SEED},
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+    }
+    if kernels:
+        out["kernels"] = kernels
+    if parity:
+        out["parity"] = parity
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -59,6 +59,11 @@ def load():
                                       C.c_int, C.c_void_p]
     lib.lnmt_model_stream.restype = C.c_void_p
     lib.lnmt_model_stream.argtypes = [C.c_void_p]
+    lib.lnmt_profile_set_level.argtypes = [C.c_void_p, C.c_int]
+    lib.lnmt_profile_tag_name.restype = C.c_char_p
+    lib.lnmt_profile_tag_name.argtypes = [C.c_int]
+    lib.lnmt_profile_read.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_double),
+                                      C.POINTER(C.c_double), C.POINTER(C.c_longlong)]
     _lib = lib
     return lib
 
@@ -107,6 +112,22 @@ class Model:
     @property
     def stream(self):
         return load().lnmt_model_stream(self.handle)
+
+    def profile(self, level):
+        """0 off, 1 output projection only, 2 every launch (HIP events on the model's stream)."""
+        _check(load().lnmt_profile_set_level(self.handle, level), "profile_set_level")
+
+    def profile_totals(self):
+        lib = load()
+        out = {}
+        for t in range(lib.lnmt_profile_tag_count()):
+            ms, work, n = C.c_double(0), C.c_double(0), C.c_longlong(0)
+            _check(lib.lnmt_profile_read(self.handle, t, C.byref(ms), C.byref(work), C.byref(n)),
+                   "profile_read")
+            if n.value:
+                out[lib.lnmt_profile_tag_name(t).decode()] = dict(ms=ms.value, work=work.value,
+                                                                  launches=n.value)
+        return out
 
     def set_params(self, params):
         """params: name -> 2-D/1-D array in mathematical layout (rows x cols)."""

@@ -179,3 +179,27 @@ extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int 
 }
 
 extern "C" void *lnmt_model_stream(lnmt_model *m) { return m->nmt->stream_; }
+
+extern "C" int lnmt_profile_set_level(lnmt_model *m, int level) {
+  return Guard([&] {
+    m->nmt->Synchronize();
+    m->nmt->profiler_.Collect();
+    m->nmt->profiler_.Reset();
+    m->nmt->profiler_.level_ = level;
+  });
+}
+
+extern "C" int lnmt_profile_tag_count(void) { return kTagCount; }
+
+extern "C" const char *lnmt_profile_tag_name(int tag) { return ProfileTagName(tag); }
+
+extern "C" int lnmt_profile_read(lnmt_model *m, int tag, double *ms, double *work,
+                                 long long *launches) {
+  return Guard([&] {
+    if (tag < 0 || tag >= kTagCount) throw LinmtError("profile tag out of range");
+    const ProfileTotals &t = m->nmt->profiler_.totals_[tag];
+    *ms = t.ms;
+    *work = t.work;
+    *launches = t.launches;
+  });
+}

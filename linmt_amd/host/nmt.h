@@ -20,6 +20,7 @@
 #include <vector>
 
 #include "hip_util.h"
+#include "profiler.h"
 
 namespace linmt {
 
@@ -261,6 +262,7 @@ class NeuralMachineTranslation {
   hipStream_t stream_ = nullptr;
   bool decode_mode_ = false;
   int beam_size_ = 0, n_sent_ = 0;
+  Profiler profiler_;  // live HIP-event timing on stream_, off by default
 
   LstmLayer input_layer_source_, input_layer_target_;
   std::vector<std::unique_ptr<LstmLayer>> v_hidden_layers_source_, v_hidden_layers_target_;

@@ -204,6 +204,7 @@ void LstmNode::ForwardProp() {
   const int H = L.lstm_size_, B = minibatch_size_;
   const float *x = nullptr;
   if (L.input_layer_mode_) {
+    ProfileScope ps(M.profiler_, kTagEmbedLookup, 8.0 * L.input_size_ * B);
     LhErrorWrapper(lh_embed_lookup_f32(L.p_device_w_.get(), L.input_size_, L.vocab_size_,
                                        p_device_input_vocab_indices_, B, nullptr, 1.f,
                                        p_device_sparse_lookup_, s),
@@ -219,9 +220,14 @@ void LstmNode::ForwardProp() {
   segs[nseg++] = {L.p_device_m_stack_.get(), 4 * H, x, L.input_size_, L.input_size_};
   segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
   if (feed) segs[nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
-  LhErrorWrapper(lh_gemm_f32(4 * H, B, segs, nseg, 0, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
+  {
+    const double k_total = (double)L.input_size_ + H + (feed ? H : 0);
+    ProfileScope ps(M.profiler_, kTagGateGemm, 2.0 * 4 * H * k_total * B);
+    LhErrorWrapper(lh_gemm_f32(4 * H, B, segs, nseg, 0, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
                              L.preact_.get(), 4 * H, s),
                  "LstmNode::ForwardPropGpu stacked gate product");
+  }
+  ProfileScope pc(M.profiler_, kTagLstmCell, (p_device_gates_ ? 44.0 : 28.0) * H * B);
   LhErrorWrapper(lh_lstm_cell_fwd_f32(H, B, L.preact_.get(), nullptr, nullptr,
                                       L.p_device_b_stack_.get(), p_device_c_t_prev_,
                                       p_device_input_vocab_indices_01_, feed ? 1 : 0,
@@ -321,18 +327,24 @@ void AttentionNode::ForwardProp() {
   hipStream_t s = A.p_neural_mt_->stream_;
   const int H = A.lstm_size_, B = minibatch_size_;
   const float *ha = p_device_h_t_;  // no dropout outside training
+  Profiler &prof = A.p_neural_mt_->profiler_;
+  const double hhb = 2.0 * H * H * B;
   if (!A.global_mode_) {
     lh_gemm_seg seg{A.p_device_w_p_.get(), H, ha, H, H};
+    ProfileScope ps(prof, kTagAttnProjGemm, hhb);
     LhErrorWrapper(lh_gemm_f32(H, B, &seg, 1, 0, 0, 1.f, 0.f, nullptr, LH_ACT_TANH, nullptr,
                                p_device_tanh_1_, H, s),
                    "AttentionNode::ForwardProp p_device_tanh_1_");
   }
   {
     lh_gemm_seg seg{A.p_device_w_a_.get(), H, ha, H, H};
+    ProfileScope ps(prof, kTagAttnProjGemm, hhb);
     LhErrorWrapper(lh_gemm_f32(H, B, &seg, 1, 1, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
                                p_device_h_t_wa_cache_, H, s),
                    "AttentionNode::ForwardProp p_device_h_t_wa_cache_");
   }
+  {
+  ProfileScope ps(prof, kTagAttnCore, 4.0 * B * ((double)A.window_ * H + 2.0 * H + 2.0 * A.window_));
   LhErrorWrapper(
       lh_attn_core_fwd_f32(H, B, A.global_mode_ ? -1 : A.d_, A.window_, A.hs_steps_,
                            p_device_tanh_1_, A.p_device_v_p_.get(), p_device_h_t_wa_cache_,
@@ -342,6 +354,8 @@ void AttentionNode::ForwardProp() {
                            p_device_p_t_, p_device_sigma_1_, p_device_indices_,
                            p_device_alignments_, p_device_cached_exp_, p_device_c_t_, nullptr, s),
       "AttentionNode::ForwardProp attention core");
+  }
+  ProfileScope po(prof, kTagAttnOutGemm, 2.0 * hhb);
   lh_gemm_seg segs[2] = {{A.p_device_w_c_p1_.get(), H, p_device_c_t_, H, H},
                          {A.p_device_w_c_p2_.get(), H, ha, H, H}};
   LhErrorWrapper(lh_gemm_f32(H, B, segs, 2, 0, 0, 1.f, 0.f, A.p_device_output_bias_.get(),
@@ -403,6 +417,8 @@ void SoftmaxLayer::BackPropPreprocessGpu(float *p_device_h_t, int step) {
 void SoftmaxLayer::ComputeLogits(float *p_device_h_t, int minibatch) {
   // D*h with the bias of MatrixBiasKernel (deep_rnn_kernel.h:525) folded into the epilogue
   lh_gemm_seg seg{p_device_d_.get(), output_vocab_size_, p_device_h_t, lstm_size_, lstm_size_};
+  ProfileScope ps(p_neural_mt_->profiler_, kTagLogitsGemm,
+                  2.0 * output_vocab_size_ * (double)lstm_size_ * minibatch);
   LhErrorWrapper(lh_gemm_f32(output_vocab_size_, minibatch, &seg, 1, 0, 0, 1.f, 0.f,
                              p_device_b_d_.get(), LH_ACT_NONE, nullptr, p_device_outputdist_.get(),
                              output_vocab_size_, p_neural_mt_->stream_),
@@ -413,6 +429,7 @@ void SoftmaxLayer::GetDistributionGpu(float *p_device_h_t) {
   hipStream_t s = p_neural_mt_->stream_;
   const int V = output_vocab_size_, B = current_minibatch_;
   ComputeLogits(p_device_h_t, B);
+  ProfileScope ps(p_neural_mt_->profiler_, kTagSoftmax, 8.0 * V * B);
   LhErrorWrapper(lh_softmax_fwd_f32(p_device_outputdist_.get(), V, nullptr, V, B,
                                     p_device_outputdist_.get(), V, s),
                  "SoftmaxLayer::GetDistributionGpu softmax");

@@ -11,6 +11,7 @@ namespace linmt {
 NeuralMachineTranslation::NeuralMachineTranslation(const GlobalConfiguration &cfg) : cfg_(cfg) {
   if (cfg_.embedding_size_ <= 0) cfg_.embedding_size_ = cfg_.lstm_size_;
   HipErrorWrapper(hipStreamCreate(&stream_), "stream creation failed");
+  profiler_.stream_ = stream_;
 }
 
 NeuralMachineTranslation::~NeuralMachineTranslation() {
@@ -232,6 +233,7 @@ double NeuralMachineTranslation::GetError(const int *p_host_source, int source_l
     softmax_layer_.BackPropPreprocessGpu(top, (int)step);
     // ComputeLossGpu without the per-step host read-back: accumulate on the device
     softmax_layer_.ComputeLogits(top, B);
+    ProfileScope px(profiler_, kTagXent, 4.0 * cfg_.target_vocab_size_ * B);
     LhErrorWrapper(
         lh_logsoftmax_xent_f32(softmax_layer_.p_device_outputdist_.get(), cfg_.target_vocab_size_,
                                nullptr, cfg_.target_vocab_size_, B,
@@ -244,6 +246,7 @@ double NeuralMachineTranslation::GetError(const int *p_host_source, int source_l
   double loss = 0;
   softmax_layer_.p_device_loss_.Download(&loss, 1, stream_);
   Synchronize();
+  profiler_.Collect();
   return loss;
 }
 
@@ -317,6 +320,7 @@ void NeuralMachineTranslation::SwapDecodingStates(const int *p_device_backptr, i
     src[n] = attention_layer_.v_nodes_[0].p_device_final_tmp_2_;
     dst[n++] = p_device_h_tild_previous_.get();
   }
+  ProfileScope ps(profiler_, kTagBeamGather, 8.0 * n * cfg_.lstm_size_ * minibatch);
   LhErrorWrapper(lh_beam_gather_f32(src, dst, n, cfg_.lstm_size_, minibatch, minibatch,
                                     p_device_backptr, stream_),
                  "SwapDecodingStates");
@@ -482,11 +486,15 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
       attention_layer_.PreprocessMinibatchInformation(bi.data(), Ba);
     }
     ForwardPropTarget(step, d.current_indices_.get(), Ba);
-    LhErrorWrapper(lh_beam_topk_f32(softmax_layer_.GetDistPtr(), cfg_.target_vocab_size_, nullptr,
+    {
+      ProfileScope ps(profiler_, kTagBeamTopK, 4.0 * cfg_.target_vocab_size_ * Ba);
+      LhErrorWrapper(lh_beam_topk_f32(softmax_layer_.GetDistPtr(), cfg_.target_vocab_size_, nullptr,
                                     cfg_.target_vocab_size_, Ba, K, Decoder::end_symbol_,
                                     d.cand_logp_.get(), d.cand_id_.get(), d.logp_eof_.get(), stream_),
                    "beam top-k");
+    }
     const size_t off = (size_t)step * B;
+    ProfileScope pm(profiler_, kTagBeamMerge, 8.0 * K * Ba);
     LhErrorWrapper(
         lh_beam_merge_f32(n_active, beam, K, step, d.limit_.get(), d.cand_logp_.get(),
                           d.cand_id_.get(), d.logp_eof_.get(), d.score_[cur].get(), o.diversity_,
@@ -514,6 +522,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   d.fin_beam_hist_.Download(fbeam.data(), fbeam.size(), stream_);
   d.fin_score_hist_.Download(fscore.data(), fscore.size(), stream_);
   Synchronize();
+  profiler_.Collect();
 
   // Rebuild v_hypotheses_ by walking the back-pointers (equivalent to the row copies of
   // eigen_top_sentences_ in decoder.h:440-471).

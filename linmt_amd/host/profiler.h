@@ -1,0 +1,113 @@
+// Live per-kernel timing with HIP events recorded on the model's own stream (the stream the
+// kernels are launched on).  Level 0 records nothing; level 1 brackets only the output projection
+// (the dominant kernel of a decode step); level 2 brackets every launch of the path.
+#pragma once
+#include <vector>
+
+#include "hip_util.h"
+
+namespace linmt {
+
+enum ProfileTag {
+  kTagEmbedLookup = 0,
+  kTagGateGemm,
+  kTagLstmCell,
+  kTagAttnProjGemm,   // tanh(W_p ha) and W_a^T ha
+  kTagAttnCore,
+  kTagAttnOutGemm,    // tanh(W_c1 ctx + W_c2 ha + b)
+  kTagLogitsGemm,     // D h~ + b_d
+  kTagSoftmax,
+  kTagXent,
+  kTagBeamTopK,
+  kTagBeamMerge,
+  kTagBeamGather,
+  kTagCount
+};
+
+inline const char *ProfileTagName(int t) {
+  static const char *names[kTagCount] = {"embed_lookup", "gate_gemm", "lstm_cell", "attn_proj_gemm",
+                                         "attn_core", "attn_out_gemm", "logits_gemm", "softmax",
+                                         "xent", "beam_topk", "beam_merge", "beam_gather"};
+  return t >= 0 && t < kTagCount ? names[t] : "";
+}
+
+struct ProfileTotals {
+  double ms = 0;     // summed launch durations
+  double work = 0;   // summed algorithmic work (flop for GEMMs, bytes otherwise)
+  long long launches = 0;
+};
+
+class Profiler {
+ public:
+  int level_ = 0;
+  hipStream_t stream_ = nullptr;
+  ProfileTotals totals_[kTagCount];
+
+  ~Profiler() {
+    for (hipEvent_t e : pool_) (void)hipEventDestroy(e);
+  }
+  bool Wants(int tag) const { return level_ >= 2 || (level_ == 1 && tag == kTagLogitsGemm); }
+  // Returns the slot to hand back to End(); scopes may nest or overlap.
+  size_t Begin(int tag, double work) {
+    Pending p{tag, Take(), Take(), work};
+    HipErrorWrapper(hipEventRecord(pool_[p.start], stream_), "profile event record failed");
+    pending_.push_back(p);
+    return pending_.size() - 1;
+  }
+  void End(size_t slot) {
+    HipErrorWrapper(hipEventRecord(pool_[pending_[slot].stop], stream_),
+                    "profile event record failed");
+  }
+  // Call after the stream has been synchronised: folds the recorded pairs into the totals.
+  void Collect() {
+    for (const Pending &p : pending_) {
+      float ms = 0.f;
+      HipErrorWrapper(hipEventElapsedTime(&ms, pool_[p.start], pool_[p.stop]),
+                      "profile event elapsed failed");
+      totals_[p.tag].ms += ms;
+      totals_[p.tag].work += p.work;
+      totals_[p.tag].launches += 1;
+    }
+    pending_.clear();
+    next_ = 0;
+  }
+  void Reset() {
+    for (ProfileTotals &t : totals_) t = ProfileTotals();
+  }
+
+ private:
+  struct Pending {
+    int tag;
+    size_t start, stop;
+    double work;
+  };
+  size_t Take() {
+    if (next_ == pool_.size()) {
+      hipEvent_t e;
+      HipErrorWrapper(hipEventCreate(&e), "profile event creation failed");
+      pool_.push_back(e);
+    }
+    return next_++;
+  }
+  std::vector<hipEvent_t> pool_;
+  std::vector<Pending> pending_;
+  size_t next_ = 0;
+};
+
+// Brackets the launches issued while it is alive.
+class ProfileScope {
+ public:
+  ProfileScope(Profiler &p, int tag, double work) : p_(p), on_(p.Wants(tag)) {
+    if (on_) slot_ = p_.Begin(tag, work);
+  }
+  ~ProfileScope() noexcept(false) {
+    if (on_) p_.End(slot_);
+  }
+
+ private:
+  Profiler &p_;
+  bool on_;
+  size_t slot_ = 0;
+};
+
+}  // namespace linmt
