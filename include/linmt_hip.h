@@ -92,6 +92,21 @@ typedef struct lh_gemm_seg {
 int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
                 float alpha, float beta, const float *bias, int act, const int *colmask, float *C,
                 int ldc, lh_stream_t stream);
+/* Same, with the activation applied only to rows m < act_rows.  Lets two products that share X
+ * run as one launch on row-stacked weights, e.g. [W_p ; W_a^T] * ha with tanh on the W_p half
+ * (src/layer_attention.h:272-275 and :327). */
+int lh_gemm_act_rows_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
+                         float alpha, float beta, const float *bias, int act, int act_rows,
+                         const int *colmask, float *C, int ldc, lh_stream_t stream);
+/* Name of the kernel instance lh_gemm_f32 would launch for this problem (tile shape and operand
+ * flags), as profilers print it; no counterpart in the reference.  Pointers in `segs` are only
+ * inspected for alignment. */
+int lh_gemm_kernel_name(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
+                        char *name, int name_cap);
+/* Tuning and test aid (no counterpart in the reference): forces tile configuration `config` for
+ * every later lh_gemm_* call of the process, config < 0 restores the built-in choice.  Returns the
+ * number of configurations (so 0 <= config < return value), LH_ERR_ARG if config is too large. */
+int lh_gemm_set_config_override(int config);
 
 /* ------------------------------------------------------------------------------------------
  * a3. Fused LSTM cell forward: bias add, gate nonlinearities, c_t / h_t update, padding mask,

@@ -1,13 +1,20 @@
 // fp32 GEMM on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32) with a fused epilogue.
 //
-// Layout: everything column-major.  A workgroup of 4 wavefronts owns a BM x BN tile of C and walks
-// K in slabs of 16.  Both operand slabs are staged in LDS k-major ([k][m] and [k][n]) so that the
-// 64 lanes of an MFMA operand read are one contiguous 128-byte run per k (no bank conflicts).
-// The MFMA is issued "swapped" (its 32x2 operand comes from X, its 2x32 operand from A), which makes
-// the 32 lanes of an accumulator register hold 32 consecutive m of one column n: stores to the
+// Layout: everything column-major.  A workgroup of WM x WN x WK wavefronts owns a BM x BN tile of C
+// and walks K in slabs of BK.  Both operand slabs are staged in LDS k-major ([k][m] and [k][n]) so
+// that the 64 lanes of an MFMA operand read are contiguous runs (no bank conflicts).  The MFMA is
+// issued "swapped" (its 32x2 operand comes from X, its 2x32 operand from A), which makes the 32
+// lanes of an accumulator register hold 32 consecutive m of one column n: stores to the
 // column-major C are full 128-byte segments.
-// Global loads of slab s+1 are issued before the MFMAs of slab s and land in the second LDS buffer
-// afterwards (one barrier per slab).
+// Pipelining: the global loads of slab s+1 are issued before the MFMAs of slab s and land in the
+// second LDS buffer afterwards (one barrier per slab); inside a slab the LDS operand reads of
+// k-step i+1 are issued before the MFMAs of k-step i.  A slab's load latency (about a microsecond
+// from HBM) is therefore hidden only by that slab's own MFMAs plus whatever other workgroups the CU
+// holds: products with few workgroups per CU use deep slabs (BK up to 128, LDS up to 139 KB) so
+// that the latency is paid per 128 k instead of per 16.
+// WK > 1 splits every slab's k range over WK wavefront groups (intra-workgroup split-K) and reduces
+// the partial accumulators through LDS in a fixed order: this is what keeps skinny products
+// (few columns, or M around 1000) from leaving most of the 256 CUs' matrix pipes idle.
 // Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to XCDs) owns a
 // contiguous range of tiles with n fastest: the tiles that share a slice of A (the large operand:
 // stacked gate weights, the V x H output embedding) hit the same XCD's L2.
@@ -17,9 +24,7 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int BK = 16;
 constexpr int PAD = 4;
-constexpr int NT = 256;
 
 struct GemmArgs {
   const float *A[LH_GEMM_MAX_SEGS];
@@ -32,6 +37,7 @@ struct GemmArgs {
   float alpha, beta;
   const float *bias;
   int act;
+  int act_rows;  // tanh applies to rows < act_rows
   const int *colmask;
   float *C;
   int ldc;
@@ -41,35 +47,38 @@ struct GemmArgs {
 // Stages one BK x BD operand slab: global -> registers (load), registers -> LDS [BK][BD+PAD] (store).
 // KC = false: the operand is contiguous along the tile's outer dimension d (m or n);
 // KC = true : the operand is contiguous along k (one run of BK floats per d).
-template <int BD, bool KC, bool VEC>
+// The loads are branch-free: an element outside the operand is fetched from a clamped (valid)
+// address and replaced by zero when it is written to LDS.
+template <int BD, int BK, int NT, bool KC, bool VEC>
 struct SlabStage {
   static constexpr int kVecTotal = BD * BK / 4;
+  static constexpr int kTotal = BD * BK;
   static constexpr int NV = (kVecTotal + NT - 1) / NT;
-  static constexpr int NS = BD * BK / NT;
+  static constexpr int NS = (kTotal + NT - 1) / NT;
+  static_assert((VEC ? NV : NS) <= 32, "validity mask is 32 bits");
   float4 v[VEC ? NV : 1];
   float s[VEC ? 1 : NS];
+  unsigned ok;  // bit i: element i of this thread lies inside the operand
 
   __device__ __forceinline__ void load(const float *__restrict__ base, int ld, int d0, int k0,
                                        int dlim, int klim, int tid) {
+    ok = 0u;
     if constexpr (VEC) {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int f = tid + i * NT;
-        float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (f < kVecTotal) {
-          if constexpr (!KC) {
-            const int k = k0 + f / (BD / 4);
-            const int d = d0 + (f % (BD / 4)) * 4;
-            if (k < klim && d < dlim)
-              val = *reinterpret_cast<const float4 *>(base + (size_t)k * ld + d);
-          } else {
-            const int d = d0 + f / (BK / 4);
-            const int k = k0 + (f % (BK / 4)) * 4;
-            if (d < dlim && k < klim)
-              val = *reinterpret_cast<const float4 *>(base + (size_t)d * ld + k);
-          }
+        int k, d;
+        if constexpr (!KC) {
+          k = k0 + f / (BD / 4);
+          d = d0 + (f % (BD / 4)) * 4;
+        } else {
+          d = d0 + f / (BK / 4);
+          k = k0 + (f % (BK / 4)) * 4;
         }
-        v[i] = val;
+        const bool in = f < kVecTotal && k < klim && d < dlim;
+        const size_t off = KC ? (size_t)d * ld + k : (size_t)k * ld + d;
+        v[i] = *reinterpret_cast<const float4 *>(base + (in ? off : (size_t)0));
+        ok |= in ? (1u << i) : 0u;
       }
     } else {
 #pragma unroll
@@ -83,10 +92,10 @@ struct SlabStage {
           d = d0 + e / BK;
           k = k0 + e % BK;
         }
-        float val = 0.f;
-        if (k < klim && d < dlim)
-          val = KC ? base[(size_t)d * ld + k] : base[(size_t)k * ld + d];
-        s[i] = val;
+        const bool in = e < kTotal && k < klim && d < dlim;
+        const size_t off = KC ? (size_t)d * ld + k : (size_t)k * ld + d;
+        s[i] = base[in ? off : (size_t)0];
+        ok |= in ? (1u << i) : 0u;
       }
     }
   }
@@ -98,17 +107,19 @@ struct SlabStage {
       for (int i = 0; i < NV; ++i) {
         const int f = tid + i * NT;
         if (f < kVecTotal) {
+          const bool in = (ok >> i) & 1u;
+          const float4 val = in ? v[i] : make_float4(0.f, 0.f, 0.f, 0.f);
           if constexpr (!KC) {
             const int k = f / (BD / 4);
             const int d = (f % (BD / 4)) * 4;
-            *reinterpret_cast<float4 *>(lds + k * LD + d) = v[i];
+            *reinterpret_cast<float4 *>(lds + k * LD + d) = val;
           } else {
             const int d = f / (BK / 4);
             const int k = (f % (BK / 4)) * 4;
-            lds[(k + 0) * LD + d] = v[i].x;
-            lds[(k + 1) * LD + d] = v[i].y;
-            lds[(k + 2) * LD + d] = v[i].z;
-            lds[(k + 3) * LD + d] = v[i].w;
+            lds[(k + 0) * LD + d] = val.x;
+            lds[(k + 1) * LD + d] = val.y;
+            lds[(k + 2) * LD + d] = val.z;
+            lds[(k + 3) * LD + d] = val.w;
           }
         }
       }
@@ -116,30 +127,46 @@ struct SlabStage {
 #pragma unroll
       for (int i = 0; i < NS; ++i) {
         const int e = tid + i * NT;
-        int k, d;
-        if constexpr (!KC) {
-          k = e / BD;
-          d = e % BD;
-        } else {
-          d = e / BK;
-          k = e % BK;
+        if (e < kTotal) {
+          int k, d;
+          if constexpr (!KC) {
+            k = e / BD;
+            d = e % BD;
+          } else {
+            d = e / BK;
+            k = e % BK;
+          }
+          lds[k * LD + d] = ((ok >> i) & 1u) ? s[i] : 0.f;
         }
-        lds[k * LD + d] = s[i];
       }
     }
   }
 };
 
-template <int BM, int BN, int WM, int WN, bool TA, bool TX, bool VEC>
-__global__ __launch_bounds__(NT) void gemm_kernel(const GemmArgs g) {
-  static_assert(WM * WN == NT / lh::kWave, "4 wavefronts per workgroup");
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+
+template <int BM, int BN, int WK, int BK>
+constexpr int smem_floats() {
+  return cmax(2 * BK * (BM + PAD + BN + PAD), (WK - 1) * BM * BN);
+}
+
+extern __shared__ __attribute__((aligned(16))) float smem[];
+
+template <int BM, int BN, int WM, int WN, int WK, int BK, bool TA, bool TX, bool VEC>
+__global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs g) {
+  constexpr int NT = 64 * WM * WN * WK;
   constexpr int TM = BM / WM, TN = BN / WN;
   constexpr int FM = TM / 32, FN = TN / 32;
-  static_assert(FM >= 1 && FN >= 1, "wave tile must hold at least one 32x32 MFMA tile");
+  static_assert(FM >= 1 && FN >= 1 && TM % 32 == 0 && TN % 32 == 0, "wave tile = 32x32 MFMA tiles");
+  constexpr int KPW = BK / WK;  // k values one wavefront group consumes per slab
+  static_assert(KPW >= 2 && KPW % 2 == 0 && BK % 4 == 0, "slab depth");
+  constexpr int NSTEP = KPW / 2;
   constexpr int LDA = BM + PAD, LDX = BN + PAD;
+  constexpr int kSlabFloats = BK * (LDA + LDX);
+  static_assert(smem_floats<BM, BN, WK, BK>() * 4 <= 160 * 1024, "LDS capacity of a CU");
 
-  __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
-  __shared__ __attribute__((aligned(16))) float Xs[2][BK * LDX];
+  float *const As0 = smem, *const Xs0 = smem + BK * LDA;
+  float *const As1 = smem + kSlabFloats, *const Xs1 = As1 + BK * LDA;
 
   // XCD-aware tile assignment.
   const int nwg = gridDim.x, id = blockIdx.x;
@@ -151,7 +178,8 @@ __global__ __launch_bounds__(NT) void gemm_kernel(const GemmArgs g) {
 
   const int tid = threadIdx.x;
   const int wave = tid / lh::kWave, lane = tid % lh::kWave;
-  const int wm = wave % WM, wn = wave / WM;
+  const int wk = wave / (WM * WN), wmn = wave % (WM * WN);
+  const int wm = wmn % WM, wn = wmn / WM;
   const int l32 = lane % 32, lhi = lane / 32;
 
   floatx16 acc[FN][FM];
@@ -162,52 +190,100 @@ __global__ __launch_bounds__(NT) void gemm_kernel(const GemmArgs g) {
 #pragma unroll
       for (int j = 0; j < 16; ++j) acc[a][b][j] = 0.f;
 
-  SlabStage<BM, TA, VEC> sa;
-  SlabStage<BN, !TX, VEC> sx;
+  SlabStage<BM, BK, NT, TA, VEC> sa;
+  SlabStage<BN, BK, NT, !TX, VEC> sx;
 
-  int total = 0;
-  for (int s = 0; s < g.nseg; ++s) total += (g.K[s] + BK - 1) / BK;
+  // segment descriptors live in scalar registers; the cursor selects among them without touching
+  // the kernel-argument memory again inside the loop
+  const float *const A0 = g.A[0], *const A1 = g.A[1], *const A2 = g.A[2];
+  const float *const X0 = g.X[0], *const X1 = g.X[1], *const X2 = g.X[2];
+  const int lda0 = g.lda[0], lda1 = g.lda[1], lda2 = g.lda[2];
+  const int ldx0 = g.ldx[0], ldx1 = g.ldx[1], ldx2 = g.ldx[2];
+  const int K0 = g.K[0], K1 = g.K[1], K2 = g.K[2];
+  const int M = g.M, N = g.N;
+  int total = (K0 + BK - 1) / BK;
+  if (g.nseg > 1) total += (K1 + BK - 1) / BK;
+  if (g.nseg > 2) total += (K2 + BK - 1) / BK;
 
-  int seg = 0, k0 = 0;
-  sa.load(g.A[0], g.lda[0], m0, 0, g.M, g.K[0], tid);
-  sx.load(g.X[0], g.ldx[0], n0, 0, g.N, g.K[0], tid);
-  sa.store(As[0], tid);
-  sx.store(Xs[0], tid);
+  int lseg = 0, lk0 = 0;  // cursor of the next slab to load
+#define LH_ISSUE()                                                  \
+  do {                                                              \
+    const float *Ab = lseg == 0 ? A0 : (lseg == 1 ? A1 : A2);       \
+    const float *Xb = lseg == 0 ? X0 : (lseg == 1 ? X1 : X2);       \
+    const int la = lseg == 0 ? lda0 : (lseg == 1 ? lda1 : lda2);    \
+    const int lx = lseg == 0 ? ldx0 : (lseg == 1 ? ldx1 : ldx2);    \
+    const int Ks = lseg == 0 ? K0 : (lseg == 1 ? K1 : K2);          \
+    sa.load(Ab, la, m0, lk0, M, Ks, tid);                           \
+    sx.load(Xb, lx, n0, lk0, N, Ks, tid);                           \
+    lk0 += BK;                                                      \
+    if (lk0 >= Ks) {                                                \
+      ++lseg;                                                       \
+      lk0 = 0;                                                      \
+    }                                                               \
+  } while (0)
+
+  LH_ISSUE();
+  sa.store(As0, tid);
+  sx.store(Xs0, tid);
   __syncthreads();
 
   for (int s = 0; s < total; ++s) {
-    int nseg = seg, nk0 = k0 + BK;
-    if (nk0 >= g.K[seg]) {
-      nseg = seg + 1;
-      nk0 = 0;
-    }
     const bool has_next = s + 1 < total;
-    if (has_next) {
-      sa.load(g.A[nseg], g.lda[nseg], m0, nk0, g.M, g.K[nseg], tid);
-      sx.load(g.X[nseg], g.ldx[nseg], n0, nk0, g.N, g.K[nseg], tid);
-    }
-    const float *as = As[s & 1] + wm * TM + l32;
-    const float *xs = Xs[s & 1] + wn * TN + l32;
+    if (has_next) LH_ISSUE();
+    const float *as = ((s & 1) ? As1 : As0) + (wk * KPW + lhi) * LDA + wm * TM + l32;
+    const float *xs = ((s & 1) ? Xs1 : Xs0) + (wk * KPW + lhi) * LDX + wn * TN + l32;
+    float fa[2][FM], fx[2][FN];
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 2) {
-      float fa[FM], fx[FN];
+    for (int b = 0; b < FM; ++b) fa[0][b] = as[b * 32];
 #pragma unroll
-      for (int b = 0; b < FM; ++b) fa[b] = as[(kk + lhi) * LDA + b * 32];
+    for (int a = 0; a < FN; ++a) fx[0][a] = xs[a * 32];
 #pragma unroll
-      for (int a = 0; a < FN; ++a) fx[a] = xs[(kk + lhi) * LDX + a * 32];
+    for (int i = 0; i < NSTEP; ++i) {
+      const int cur = i & 1, nxt = cur ^ 1;
+      if (i + 1 < NSTEP) {
+#pragma unroll
+        for (int b = 0; b < FM; ++b) fa[nxt][b] = as[(2 * (i + 1)) * LDA + b * 32];
+#pragma unroll
+        for (int a = 0; a < FN; ++a) fx[nxt][a] = xs[(2 * (i + 1)) * LDX + a * 32];
+      }
 #pragma unroll
       for (int a = 0; a < FN; ++a)
 #pragma unroll
         for (int b = 0; b < FM; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fx[a], fa[b], acc[a][b], 0, 0, 0);
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fx[cur][a], fa[cur][b], acc[a][b], 0, 0, 0);
     }
     if (has_next) {
-      sa.store(As[(s + 1) & 1], tid);
-      sx.store(Xs[(s + 1) & 1], tid);
+      sa.store((s & 1) ? As0 : As1, tid);
+      sx.store((s & 1) ? Xs0 : Xs1, tid);
     }
     __syncthreads();
-    seg = nseg;
-    k0 = nk0;
+  }
+#undef LH_ISSUE
+
+  if constexpr (WK > 1) {
+    // Fixed-order reduction of the WK partial tiles through LDS (the slab buffers are dead now).
+    constexpr int kPerWave = FN * FM * 16 * 64;
+    if (wk > 0) {
+      float *dst = smem + ((wk - 1) * (WM * WN) + wmn) * kPerWave + lane;
+#pragma unroll
+      for (int a = 0; a < FN; ++a)
+#pragma unroll
+        for (int b = 0; b < FM; ++b)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) dst[((a * FM + b) * 16 + j) * 64] = acc[a][b][j];
+    }
+    __syncthreads();
+    if (wk > 0) return;
+#pragma unroll
+    for (int p = 0; p < WK - 1; ++p) {
+      const float *src = smem + (p * (WM * WN) + wmn) * kPerWave + lane;
+#pragma unroll
+      for (int a = 0; a < FN; ++a)
+#pragma unroll
+        for (int b = 0; b < FM; ++b)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) acc[a][b][j] += src[((a * FM + b) * 16 + j) * 64];
+    }
   }
 
   // Epilogue: accumulator register j of lane l is C[m = .. + l%32][n = .. + 8*(j/4) + 4*(l/32) + j%4].
@@ -219,6 +295,7 @@ __global__ __launch_bounds__(NT) void gemm_kernel(const GemmArgs g) {
       const int m = m0 + wm * TM + b * 32 + l32;
       if (m >= g.M) continue;
       const float bv = g.bias ? g.bias[m] : 0.f;
+      const bool do_tanh = g.act == LH_ACT_TANH && m < g.act_rows;
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const int n = n0 + wn * TN + a * 32 + (j / 4) * 8 + lhi * 4 + (j % 4);
@@ -227,7 +304,7 @@ __global__ __launch_bounds__(NT) void gemm_kernel(const GemmArgs g) {
         float v = alpha * acc[a][b][j];
         if (beta != 0.f) v += beta * *cp;
         v += bv;
-        if (g.act == LH_ACT_TANH) v = tanhf(v);
+        if (do_tanh) v = tanhf(v);
         if (g.colmask) v *= (float)g.colmask[n];
         *cp = v;
       }
@@ -235,49 +312,122 @@ __global__ __launch_bounds__(NT) void gemm_kernel(const GemmArgs g) {
   }
 }
 
-template <int BM, int BN, int WM, int WN>
+// ---- configurations -----------------------------------------------------------------------
+struct Config {
+  int bm, bn, wm, wn, wk, bk;
+};
+// X(index, BM, BN, WM, WN, WK, BK)
+#define LH_GEMM_CONFIGS(X)                                                     \
+  X(0, 128, 128, 2, 2, 1, 16)  /* large products: output projection         */ \
+  X(1, 128, 128, 2, 2, 1, 32)                                                  \
+  X(2, 128, 96, 4, 1, 1, 16)                                                   \
+  X(3, 128, 64, 2, 2, 1, 16)                                                   \
+  X(4, 128, 64, 2, 2, 1, 32)                                                   \
+  X(5, 64, 96, 2, 1, 2, 32)    /* stacked gate products at a few hundred columns */ \
+  X(6, 64, 96, 2, 1, 2, 64)                                                    \
+  X(7, 64, 64, 2, 2, 1, 16)    /* also the only shape built for unaligned operands */ \
+  X(8, 64, 64, 2, 2, 1, 64)                                                    \
+  X(9, 64, 64, 2, 2, 1, 128)                                                   \
+  X(10, 32, 96, 1, 3, 2, 32)   /* M around 1000 */                             \
+  X(11, 32, 96, 1, 3, 2, 128)                                                  \
+  X(12, 32, 64, 1, 2, 4, 32)   /* skinny */                                    \
+  X(13, 32, 64, 1, 2, 4, 128)                                                  \
+  X(14, 32, 32, 1, 1, 8, 64)   /* very skinny */                               \
+  X(15, 32, 32, 1, 1, 8, 128)                                                  \
+  X(16, 128, 32, 4, 1, 1, 16)                                                  \
+  X(17, 128, 32, 4, 1, 1, 64)                                                  \
+  X(18, 64, 32, 2, 1, 4, 32)                                                   \
+  X(19, 64, 32, 2, 1, 4, 128)
+
+#define LH_CFG_ENTRY(I, BM, BN, WM, WN, WK, BK) {BM, BN, WM, WN, WK, BK},
+const Config kConfigs[] = {LH_GEMM_CONFIGS(LH_CFG_ENTRY)};
+#undef LH_CFG_ENTRY
+constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
+constexpr int kUnalignedConfig = 7;
+
+template <typename KernelT>
+int launch_kernel(KernelT kernel, int smem_bytes, dim3 grid, dim3 block, hipStream_t st,
+                  const GemmArgs &g) {
+  if (smem_bytes > 64 * 1024) {
+    // more dynamic LDS than the default limit: raised once per kernel instance
+    static thread_local const void *raised[64];
+    static thread_local int n_raised = 0;
+    bool done = false;
+    for (int i = 0; i < n_raised; ++i) done = done || raised[i] == (const void *)kernel;
+    if (!done) {
+      hipError_t e = hipFuncSetAttribute((const void *)kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes);
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return lh::fail_arg("lh_gemm_f32: cannot reserve %d bytes of LDS: %s", smem_bytes,
+                            hipGetErrorString(e));
+      }
+      if (n_raised < 64) raised[n_raised++] = (const void *)kernel;
+    }
+  }
+  hipLaunchKernelGGL(kernel, grid, block, smem_bytes, st, g);
+  return lh::check_launch("lh_gemm_f32");
+}
+
+template <int BM, int BN, int WM, int WN, int WK, int BK, bool ALLOW_UNALIGNED>
 int launch_cfg(const GemmArgs &g0, bool ta, bool tx, bool vec, hipStream_t st) {
   GemmArgs g = g0;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
-  const dim3 grid(g.tiles_m * g.tiles_n), block(NT);
+  const dim3 grid(g.tiles_m * g.tiles_n), block(64 * WM * WN * WK);
+  constexpr int bytes = smem_floats<BM, BN, WK, BK>() * 4;
 #define LH_GEMM_LAUNCH(TA, TX, VEC) \
-  hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, TA, TX, VEC>), grid, block, 0, st, g)
-  if (!ta && !tx) {
-    if (vec) LH_GEMM_LAUNCH(false, false, true); else LH_GEMM_LAUNCH(false, false, false);
-  } else if (ta && !tx) {
-    if (vec) LH_GEMM_LAUNCH(true, false, true); else LH_GEMM_LAUNCH(true, false, false);
-  } else {
-    if (vec) LH_GEMM_LAUNCH(false, true, true); else LH_GEMM_LAUNCH(false, true, false);
+  return launch_kernel(gemm_kernel<BM, BN, WM, WN, WK, BK, TA, TX, VEC>, bytes, grid, block, st, g)
+  if (vec) {
+    if (!ta && !tx) LH_GEMM_LAUNCH(false, false, true);
+    else if (ta) LH_GEMM_LAUNCH(true, false, true);
+    else LH_GEMM_LAUNCH(false, true, true);
+  }
+  if constexpr (ALLOW_UNALIGNED) {
+    if (!ta && !tx) LH_GEMM_LAUNCH(false, false, false);
+    else if (ta) LH_GEMM_LAUNCH(true, false, false);
+    else LH_GEMM_LAUNCH(false, true, false);
   }
 #undef LH_GEMM_LAUNCH
-  return lh::check_launch("lh_gemm_f32");
+  return lh::fail_arg("lh_gemm_f32: internal error, unaligned operands reached an aligned-only tile");
 }
 
-// Tile choice.  256 CUs: prefer the largest tile that still gives every CU about two workgroups;
-// if none does, take the shape with the most workgroups that does not over-pad N.
-int pick_tile(int M, int N) {
-  struct Cand { int bm, bn; };
-  static const Cand cands[4] = {{128, 128}, {128, 64}, {64, 64}, {128, 32}};
-  int best = 3, best_wg = -1;
-  for (int c = 0; c < 4; ++c) {
-    const int bm = cands[c].bm, bn = cands[c].bn;
-    if (bn > 32 && N <= bn / 2) continue;  // more than half of every n-tile would be padding
-    const int wg = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-    if (wg >= 448) return c;
-    if (wg > best_wg) {
-      best_wg = wg;
-      best = c;
-    }
+int launch_index(int c, const GemmArgs &g, bool ta, bool tx, bool vec, hipStream_t st) {
+  switch (c) {
+#define LH_CFG_CASE(I, BM, BN, WM, WN, WK, BK) \
+  case I:                                      \
+    return launch_cfg<BM, BN, WM, WN, WK, BK, I == kUnalignedConfig>(g, ta, tx, vec, st);
+    LH_GEMM_CONFIGS(LH_CFG_CASE)
+#undef LH_CFG_CASE
+    default: return lh::fail_arg("lh_gemm_f32: configuration %d does not exist", c);
   }
-  return best;
 }
 
-}  // namespace
+int g_config_override = -1;  // tuning / test aid, see lh_gemm_set_config_override
 
-extern "C" int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
-                           float alpha, float beta, const float *bias, int act, const int *colmask,
-                           float *C, int ldc, lh_stream_t stream) {
+// Tile choice, from sweeps of every configuration over the products of the path on MI355X.
+int pick_config(int M, int N, long long ktot, bool vec) {
+  if (!vec) return kUnalignedConfig;
+  const int forced = g_config_override;
+  if (forced >= 0 && forced < kNumConfigs) return forced;
+  (void)ktot;
+  const long long tiles32 = (long long)((M + 31) / 32) * ((N + 31) / 32);  // 32x32 MFMA tiles
+  if (N <= 64) return M >= 16384 ? 18 : 14;        // encoder steps, single-sentence decoding
+  if (tiles32 >= 256 * 40) return 3;               // >= 40 MFMA tiles per CU (output projection)
+  if (tiles32 >= 256 * 10) return N >= 512 || N % 96 == 0 ? 5 : 7;  // e.g. 4000 x 768 gate products
+  if (tiles32 >= 256 * 7) return 7;
+  return 18;                                       // M around 1000: many small tiles, split K
+}
+
+struct Prepared {
+  GemmArgs g;
+  bool ta, tx, vec;
+  int config;
+};
+
+int prepare(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX, float alpha,
+            float beta, const float *bias, int act, int act_rows, const int *colmask, float *C,
+            int ldc, Prepared *out) {
   if (M <= 0 || N <= 0) return lh::fail_arg("lh_gemm_f32: M=%d N=%d must be positive", M, N);
   if (!segs || nseg < 1 || nseg > LH_GEMM_MAX_SEGS)
     return lh::fail_arg("lh_gemm_f32: nseg=%d outside [1,%d]", nseg, LH_GEMM_MAX_SEGS);
@@ -285,8 +435,10 @@ extern "C" int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int 
   if (act != LH_ACT_NONE && act != LH_ACT_TANH) return lh::fail_arg("lh_gemm_f32: act=%d", act);
   if (!C || ldc < M) return lh::fail_arg("lh_gemm_f32: C=%p ldc=%d (M=%d)", (void *)C, ldc, M);
 
-  GemmArgs g{};
+  GemmArgs &g = out->g;
+  g = GemmArgs{};
   bool vec = true;
+  long long ktot = 0;
   for (int s = 0; s < nseg; ++s) {
     const lh_gemm_seg &e = segs[s];
     if (!e.A || !e.X || e.K <= 0)
@@ -301,11 +453,19 @@ extern "C" int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int 
     g.lda[s] = e.lda;
     g.ldx[s] = e.ldx;
     g.K[s] = e.K;
+    ktot += e.K;
     // 16-byte loads need aligned bases / leading dimensions and a contiguous extent that is a
     // multiple of 4 (the guards test only the first element of a float4).
     const int a_extent = transA ? e.K : M, x_extent = transX ? N : e.K;
     vec = vec && lh::aligned16(e.A) && lh::aligned16(e.X) && e.lda % 4 == 0 && e.ldx % 4 == 0 &&
           a_extent % 4 == 0 && x_extent % 4 == 0;
+  }
+  for (int s = nseg; s < LH_GEMM_MAX_SEGS; ++s) {  // unused slots mirror segment 0 (never read)
+    g.A[s] = g.A[0];
+    g.X[s] = g.X[0];
+    g.lda[s] = g.lda[0];
+    g.ldx[s] = g.ldx[0];
+    g.K[s] = g.K[0];
   }
   g.nseg = nseg;
   g.M = M;
@@ -314,16 +474,60 @@ extern "C" int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int 
   g.beta = beta;
   g.bias = bias;
   g.act = act;
+  g.act_rows = act_rows;
   g.colmask = colmask;
   g.C = C;
   g.ldc = ldc;
+  out->ta = transA != 0;
+  out->tx = transX != 0;
+  out->vec = vec;
+  out->config = pick_config(M, N, ktot, vec);
+  return LH_OK;
+}
 
-  const bool ta = transA != 0, tx = transX != 0;
-  hipStream_t st = lh::as_stream(stream);
-  switch (pick_tile(M, N)) {
-    case 0: return launch_cfg<128, 128, 2, 2>(g, ta, tx, vec, st);
-    case 1: return launch_cfg<128, 64, 2, 2>(g, ta, tx, vec, st);
-    case 2: return launch_cfg<64, 64, 2, 2>(g, ta, tx, vec, st);
-    default: return launch_cfg<128, 32, 4, 1>(g, ta, tx, vec, st);
-  }
+}  // namespace
+
+extern "C" int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
+                           float alpha, float beta, const float *bias, int act, const int *colmask,
+                           float *C, int ldc, lh_stream_t stream) {
+  Prepared p;
+  const int rc = prepare(M, N, segs, nseg, transA, transX, alpha, beta, bias, act, M, colmask, C,
+                         ldc, &p);
+  if (rc != LH_OK) return rc;
+  return launch_index(p.config, p.g, p.ta, p.tx, p.vec, lh::as_stream(stream));
+}
+
+extern "C" int lh_gemm_act_rows_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA,
+                                    int transX, float alpha, float beta, const float *bias, int act,
+                                    int act_rows, const int *colmask, float *C, int ldc,
+                                    lh_stream_t stream) {
+  if (act_rows < 0 || act_rows > M)
+    return lh::fail_arg("lh_gemm_act_rows_f32: act_rows=%d outside [0,M=%d]", act_rows, M);
+  Prepared p;
+  const int rc = prepare(M, N, segs, nseg, transA, transX, alpha, beta, bias, act, act_rows,
+                         colmask, C, ldc, &p);
+  if (rc != LH_OK) return rc;
+  return launch_index(p.config, p.g, p.ta, p.tx, p.vec, lh::as_stream(stream));
+}
+
+extern "C" int lh_gemm_set_config_override(int config) {
+  if (config >= kNumConfigs)
+    return lh::fail_arg("lh_gemm_set_config_override: %d >= %d", config, kNumConfigs);
+  g_config_override = config < 0 ? -1 : config;
+  return kNumConfigs;
+}
+
+extern "C" int lh_gemm_kernel_name(int M, int N, const lh_gemm_seg *segs, int nseg, int transA,
+                                   int transX, char *name, int name_cap) {
+  if (!name || name_cap < 1) return lh::fail_arg("lh_gemm_kernel_name: no output buffer");
+  Prepared p;
+  float dummy;
+  const int rc = prepare(M, N, segs, nseg, transA, transX, 1.f, 0.f, nullptr, LH_ACT_NONE, M,
+                         nullptr, &dummy, M, &p);
+  if (rc != LH_OK) return rc;
+  const Config &k = kConfigs[p.config];
+  snprintf(name, name_cap, "gemm_kernel<%d, %d, %d, %d, %d, %d, %s, %s, %s>", k.bm, k.bn, k.wm,
+           k.wn, k.wk, k.bk, p.ta ? "true" : "false", p.tx ? "true" : "false",
+           p.vec ? "true" : "false");
+  return LH_OK;
 }

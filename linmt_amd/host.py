@@ -60,10 +60,10 @@ def load():
     lib.lnmt_model_stream.restype = C.c_void_p
     lib.lnmt_model_stream.argtypes = [C.c_void_p]
     lib.lnmt_profile_set_level.argtypes = [C.c_void_p, C.c_int]
-    lib.lnmt_profile_tag_name.restype = C.c_char_p
-    lib.lnmt_profile_tag_name.argtypes = [C.c_int]
-    lib.lnmt_profile_read.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_double),
-                                      C.POINTER(C.c_double), C.POINTER(C.c_longlong)]
+    lib.lnmt_profile_count.argtypes = [C.c_void_p]
+    lib.lnmt_profile_entry.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.c_int,
+                                       C.POINTER(C.c_double), C.POINTER(C.c_double),
+                                       C.POINTER(C.c_longlong)]
     _lib = lib
     return lib
 
@@ -118,15 +118,15 @@ class Model:
         _check(load().lnmt_profile_set_level(self.handle, level), "profile_set_level")
 
     def profile_totals(self):
+        """name -> dict(ms, work, launches); matrix products are keyed 'site|kernel instance'."""
         lib = load()
         out = {}
-        for t in range(lib.lnmt_profile_tag_count()):
+        for i in range(lib.lnmt_profile_count(self.handle)):
+            name = C.create_string_buffer(256)
             ms, work, n = C.c_double(0), C.c_double(0), C.c_longlong(0)
-            _check(lib.lnmt_profile_read(self.handle, t, C.byref(ms), C.byref(work), C.byref(n)),
-                   "profile_read")
-            if n.value:
-                out[lib.lnmt_profile_tag_name(t).decode()] = dict(ms=ms.value, work=work.value,
-                                                                  launches=n.value)
+            _check(lib.lnmt_profile_entry(self.handle, i, name, 256, C.byref(ms), C.byref(work),
+                                          C.byref(n)), "profile_entry")
+            out[name.value.decode()] = dict(ms=ms.value, work=work.value, launches=n.value)
         return out
 
     def set_params(self, params):

@@ -189,17 +189,18 @@ extern "C" int lnmt_profile_set_level(lnmt_model *m, int level) {
   });
 }
 
-extern "C" int lnmt_profile_tag_count(void) { return kTagCount; }
+extern "C" int lnmt_profile_count(lnmt_model *m) { return (int)m->nmt->profiler_.totals_.size(); }
 
-extern "C" const char *lnmt_profile_tag_name(int tag) { return ProfileTagName(tag); }
-
-extern "C" int lnmt_profile_read(lnmt_model *m, int tag, double *ms, double *work,
-                                 long long *launches) {
+extern "C" int lnmt_profile_entry(lnmt_model *m, int index, char *name, int name_cap, double *ms,
+                                  double *work, long long *launches) {
   return Guard([&] {
-    if (tag < 0 || tag >= kTagCount) throw LinmtError("profile tag out of range");
-    const ProfileTotals &t = m->nmt->profiler_.totals_[tag];
-    *ms = t.ms;
-    *work = t.work;
-    *launches = t.launches;
+    const auto &tot = m->nmt->profiler_.totals_;
+    if (index < 0 || index >= (int)tot.size()) throw LinmtError("profile entry out of range");
+    auto it = tot.begin();
+    std::advance(it, index);
+    snprintf(name, name_cap, "%s", it->first.c_str());
+    *ms = it->second.ms;
+    *work = it->second.work;
+    *launches = it->second.launches;
   });
 }

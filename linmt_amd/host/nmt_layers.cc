@@ -221,8 +221,7 @@ void LstmNode::ForwardProp() {
   segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
   if (feed) segs[nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
   {
-    const double k_total = (double)L.input_size_ + H + (feed ? H : 0);
-    ProfileScope ps(M.profiler_, kTagGateGemm, 2.0 * 4 * H * k_total * B);
+    ProfileScope ps(M.profiler_, kTagGateGemm, 4 * H, B, segs, nseg, 0, 0);
     LhErrorWrapper(lh_gemm_f32(4 * H, B, segs, nseg, 0, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
                              L.preact_.get(), 4 * H, s),
                  "LstmNode::ForwardPropGpu stacked gate product");
@@ -328,17 +327,16 @@ void AttentionNode::ForwardProp() {
   const int H = A.lstm_size_, B = minibatch_size_;
   const float *ha = p_device_h_t_;  // no dropout outside training
   Profiler &prof = A.p_neural_mt_->profiler_;
-  const double hhb = 2.0 * H * H * B;
   if (!A.global_mode_) {
     lh_gemm_seg seg{A.p_device_w_p_.get(), H, ha, H, H};
-    ProfileScope ps(prof, kTagAttnProjGemm, hhb);
+    ProfileScope ps(prof, kTagAttnProjGemm, H, B, &seg, 1, 0, 0);
     LhErrorWrapper(lh_gemm_f32(H, B, &seg, 1, 0, 0, 1.f, 0.f, nullptr, LH_ACT_TANH, nullptr,
                                p_device_tanh_1_, H, s),
                    "AttentionNode::ForwardProp p_device_tanh_1_");
   }
   {
     lh_gemm_seg seg{A.p_device_w_a_.get(), H, ha, H, H};
-    ProfileScope ps(prof, kTagAttnProjGemm, hhb);
+    ProfileScope ps(prof, kTagAttnProjGemm, H, B, &seg, 1, 1, 0);
     LhErrorWrapper(lh_gemm_f32(H, B, &seg, 1, 1, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
                                p_device_h_t_wa_cache_, H, s),
                    "AttentionNode::ForwardProp p_device_h_t_wa_cache_");
@@ -355,9 +353,9 @@ void AttentionNode::ForwardProp() {
                            p_device_alignments_, p_device_cached_exp_, p_device_c_t_, nullptr, s),
       "AttentionNode::ForwardProp attention core");
   }
-  ProfileScope po(prof, kTagAttnOutGemm, 2.0 * hhb);
   lh_gemm_seg segs[2] = {{A.p_device_w_c_p1_.get(), H, p_device_c_t_, H, H},
                          {A.p_device_w_c_p2_.get(), H, ha, H, H}};
+  ProfileScope po(prof, kTagAttnOutGemm, H, B, segs, 2, 0, 0);
   LhErrorWrapper(lh_gemm_f32(H, B, segs, 2, 0, 0, 1.f, 0.f, A.p_device_output_bias_.get(),
                              LH_ACT_TANH, p_device_indices_mask_, p_device_final_tmp_2_, H, s),
                  "AttentionNode::ForwardProp p_device_final_tmp_2_");
@@ -417,8 +415,8 @@ void SoftmaxLayer::BackPropPreprocessGpu(float *p_device_h_t, int step) {
 void SoftmaxLayer::ComputeLogits(float *p_device_h_t, int minibatch) {
   // D*h with the bias of MatrixBiasKernel (deep_rnn_kernel.h:525) folded into the epilogue
   lh_gemm_seg seg{p_device_d_.get(), output_vocab_size_, p_device_h_t, lstm_size_, lstm_size_};
-  ProfileScope ps(p_neural_mt_->profiler_, kTagLogitsGemm,
-                  2.0 * output_vocab_size_ * (double)lstm_size_ * minibatch);
+  ProfileScope ps(p_neural_mt_->profiler_, kTagLogitsGemm, output_vocab_size_, minibatch, &seg, 1, 0,
+                  0);
   LhErrorWrapper(lh_gemm_f32(output_vocab_size_, minibatch, &seg, 1, 0, 0, 1.f, 0.f,
                              p_device_b_d_.get(), LH_ACT_NONE, nullptr, p_device_outputdist_.get(),
                              output_vocab_size_, p_neural_mt_->stream_),

@@ -1,7 +1,10 @@
 // Live per-kernel timing with HIP events recorded on the model's own stream (the stream the
-// kernels are launched on).  Level 0 records nothing; level 1 brackets only the output projection
-// (the dominant kernel of a decode step); level 2 brackets every launch of the path.
+// kernels are launched on).  Level 0 records nothing; level 1 brackets the matrix products (the
+// dominant kernels of a decode step), keyed by the kernel instance the GEMM entry point picks;
+// level 2 brackets every launch of the path.
 #pragma once
+#include <map>
+#include <string>
 #include <vector>
 
 #include "hip_util.h"
@@ -31,6 +34,10 @@ inline const char *ProfileTagName(int t) {
   return t >= 0 && t < kTagCount ? names[t] : "";
 }
 
+inline bool ProfileTagIsGemm(int t) {
+  return t == kTagGateGemm || t == kTagAttnProjGemm || t == kTagAttnOutGemm || t == kTagLogitsGemm;
+}
+
 struct ProfileTotals {
   double ms = 0;     // summed launch durations
   double work = 0;   // summed algorithmic work (flop for GEMMs, bytes otherwise)
@@ -41,15 +48,16 @@ class Profiler {
  public:
   int level_ = 0;
   hipStream_t stream_ = nullptr;
-  ProfileTotals totals_[kTagCount];
+  // key: "<call site>" or "<call site>|<kernel instance>" for matrix products
+  std::map<std::string, ProfileTotals> totals_;
 
   ~Profiler() {
     for (hipEvent_t e : pool_) (void)hipEventDestroy(e);
   }
-  bool Wants(int tag) const { return level_ >= 2 || (level_ == 1 && tag == kTagLogitsGemm); }
+  bool Wants(int tag) const { return level_ >= 2 || (level_ == 1 && ProfileTagIsGemm(tag)); }
   // Returns the slot to hand back to End(); scopes may nest or overlap.
-  size_t Begin(int tag, double work) {
-    Pending p{tag, Take(), Take(), work};
+  size_t Begin(const std::string &key, double work) {
+    Pending p{key, Take(), Take(), work};
     HipErrorWrapper(hipEventRecord(pool_[p.start], stream_), "profile event record failed");
     pending_.push_back(p);
     return pending_.size() - 1;
@@ -64,20 +72,19 @@ class Profiler {
       float ms = 0.f;
       HipErrorWrapper(hipEventElapsedTime(&ms, pool_[p.start], pool_[p.stop]),
                       "profile event elapsed failed");
-      totals_[p.tag].ms += ms;
-      totals_[p.tag].work += p.work;
-      totals_[p.tag].launches += 1;
+      ProfileTotals &t = totals_[p.key];
+      t.ms += ms;
+      t.work += p.work;
+      t.launches += 1;
     }
     pending_.clear();
     next_ = 0;
   }
-  void Reset() {
-    for (ProfileTotals &t : totals_) t = ProfileTotals();
-  }
+  void Reset() { totals_.clear(); }
 
  private:
   struct Pending {
-    int tag;
+    std::string key;
     size_t start, stop;
     double work;
   };
@@ -98,7 +105,19 @@ class Profiler {
 class ProfileScope {
  public:
   ProfileScope(Profiler &p, int tag, double work) : p_(p), on_(p.Wants(tag)) {
-    if (on_) slot_ = p_.Begin(tag, work);
+    if (on_) slot_ = p_.Begin(ProfileTagName(tag), work);
+  }
+  // Matrix product: the key carries the kernel instance lh_gemm_f32 will launch for this problem.
+  ProfileScope(Profiler &p, int tag, int M, int N, const lh_gemm_seg *segs, int nseg, int transA,
+               int transX)
+      : p_(p), on_(p.Wants(tag)) {
+    if (!on_) return;
+    char name[160] = {0};
+    LhErrorWrapper(lh_gemm_kernel_name(M, N, segs, nseg, transA, transX, name, sizeof(name)),
+                   "lh_gemm_kernel_name");
+    double k = 0;
+    for (int s = 0; s < nseg; ++s) k += segs[s].K;
+    slot_ = p_.Begin(std::string(ProfileTagName(tag)) + "|" + name, 2.0 * M * (double)N * k);
   }
   ~ProfileScope() noexcept(false) {
     if (on_) p_.End(slot_);

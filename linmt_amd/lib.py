@@ -37,6 +37,12 @@ SIGNATURES = {
     "lh_gemm_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int, C.c_int,
                               C.c_float, C.c_float, c_f32p, C.c_int, c_i32p, c_f32p, C.c_int,
                               C.c_void_p]),
+    "lh_gemm_act_rows_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
+                                       C.c_int, C.c_float, C.c_float, c_f32p, C.c_int, C.c_int,
+                                       c_i32p, c_f32p, C.c_int, C.c_void_p]),
+    "lh_gemm_kernel_name": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
+                                      C.c_int, C.c_char_p, C.c_int]),
+    "lh_gemm_set_config_override": (C.c_int, [C.c_int]),
     "lh_lstm_cell_fwd_f32": (C.c_int, [C.c_int, C.c_int, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p,
                                        c_i32p, C.c_int, C.c_float, c_f32p, c_f32p, c_f32p, c_f32p,
                                        C.c_float, c_f32p, C.c_void_p]),
@@ -121,9 +127,7 @@ def embed_lookup(W, E, V, idx0, B, out, drop_mask=None, keep=1.0, stream=None):
                                      _ptr(out), _stream(stream)), "lh_embed_lookup_f32")
 
 
-def gemm(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0, bias=None,
-         act=LH_ACT_NONE, colmask=None, stream=None):
-    """segs: list of (A, lda, X, ldx, K) with torch tensors A, X."""
+def _segs(segs):
     arr = (GemmSeg * len(segs))()
     for i, (A, lda, X, ldx, K) in enumerate(segs):
         arr[i].A = A.data_ptr()
@@ -131,9 +135,29 @@ def gemm(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0
         arr[i].X = X.data_ptr()
         arr[i].ldx = ldx
         arr[i].K = K
-    check(load().lh_gemm_f32(M, N, arr, len(segs), int(transA), int(transX), alpha, beta,
-                             _ptr(bias), act, _ptr(colmask), _ptr(C_out), ldc, _stream(stream)),
-          "lh_gemm_f32")
+    return arr
+
+
+def gemm(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0, bias=None,
+         act=LH_ACT_NONE, colmask=None, act_rows=None, stream=None):
+    """segs: list of (A, lda, X, ldx, K) with torch tensors A, X."""
+    arr = _segs(segs)
+    if act_rows is None:
+        check(load().lh_gemm_f32(M, N, arr, len(segs), int(transA), int(transX), alpha, beta,
+                                 _ptr(bias), act, _ptr(colmask), _ptr(C_out), ldc,
+                                 _stream(stream)), "lh_gemm_f32")
+    else:
+        check(load().lh_gemm_act_rows_f32(M, N, arr, len(segs), int(transA), int(transX), alpha,
+                                          beta, _ptr(bias), act, act_rows, _ptr(colmask),
+                                          _ptr(C_out), ldc, _stream(stream)),
+              "lh_gemm_act_rows_f32")
+
+
+def gemm_kernel_name(M, N, segs, transA=False, transX=False):
+    buf = C.create_string_buffer(128)
+    check(load().lh_gemm_kernel_name(M, N, _segs(segs), len(segs), int(transA), int(transX), buf,
+                                     128), "lh_gemm_kernel_name")
+    return buf.value.decode()
 
 
 def lstm_cell_fwd(H, B, pre1, bias4h, c_prev, mask01, c, h, pre2=None, pre3=None,

@@ -106,6 +106,40 @@ def test_gemm_vs_float64(lh, M, N, Ks, tA, tX):
     assert_close(host(out, (M, N)), want2, "epilogue")
 
 
+def test_gemm_every_tile_configuration(lh):
+    """Each tile configuration (incl. the intra-workgroup split-K ones) on shapes with ragged edges,
+    several K segments and both transposes; also the row-limited activation and the kernel name."""
+    rng = np.random.default_rng(21)
+    n_cfg = lh.load().lh_gemm_set_config_override(-1)
+    assert n_cfg >= 1
+    shapes = [(200, 76, (100, 36), False, False), (129, 97, (68,), True, False),
+              (96, 33, (40,), False, True), (70, 130, (17, 9), False, False)]
+    try:
+        for cfg in range(n_cfg):
+            assert lh.load().lh_gemm_set_config_override(cfg) == n_cfg
+            for M, N, Ks, tA, tX in shapes:
+                As = [uni(rng, *((K, M) if tA else (M, K)), s=0.5) for K in Ks]
+                Xs = [uni(rng, *((N, K) if tX else (K, N))) for K in Ks]
+                want = sum((A.T if tA else A).astype(np.float64) @ (X.T if tX else X)
+                           for A, X in zip(As, Xs))
+                segs = [(dev(A), A.shape[0], dev(X), X.shape[0], K) for A, X, K in zip(As, Xs, Ks)]
+                out = torch.full((M * N,), 3.0, device="cuda")
+                lh.gemm(M, N, segs, out, M, transA=tA, transX=tX)
+                assert_close(host(out, (M, N)), want, f"config {cfg} shape {(M, N, Ks, tA, tX)}")
+                bias = uni(rng, M)
+                lh.gemm(M, N, segs, out, M, transA=tA, transX=tX, bias=dev(bias),
+                        act=lh.LH_ACT_TANH, act_rows=M // 2)
+                w2 = want + bias[:, None]
+                w2[: M // 2] = np.tanh(w2[: M // 2])
+                assert_close(host(out, (M, N)), w2, f"config {cfg} tanh on the first rows only")
+                name = lh.gemm_kernel_name(M, N, segs, tA, tX)
+                assert name.startswith("gemm_kernel<") and name.endswith(">")
+    finally:
+        lh.load().lh_gemm_set_config_override(-1)
+    with pytest.raises(lh.LinmtHipError):
+        lh.check(lh.load().lh_gemm_set_config_override(10 ** 6), "override")
+
+
 def test_gemm_ldc_and_padding_untouched(lh):
     """ldc > M: the rows between M and ldc must not be written."""
     rng = np.random.default_rng(3)
