@@ -111,6 +111,27 @@ int orc_decode_sentence(orc_model *m, const int *src_ids, int S, const orc_decod
 double orc_forward_xent(orc_model *m, const int *src, int S, const int *tgt_in, const int *tgt_out,
                         int T, int B, const int *batch_info, int num_threads);
 
+/* ---- training: gradients and update (linmt_oracle_train.cpp) ------------------------------------ */
+typedef struct orc_trainer orc_trainer;
+orc_trainer *orc_trainer_create(orc_model *m, const orc_model_config *cfg);
+void orc_trainer_destroy(orc_trainer *t);
+/* NeuralMachineTranslation::ComputeGradients without its final UpdateWeights: forward with stored
+ * activations, then the backward pass.  Arguments as orc_forward_xent; src_unique / tgt_unique are
+ * the unique non-pad input ids of the minibatch (the reference's *_wgrad lists).  Returns the summed
+ * log-likelihood.  Gradients are of the log-likelihood (ascent convention), unscaled. */
+double orc_compute_gradients(orc_trainer *t, const int *src, int S, const int *tgt_in,
+                             const int *tgt_out, int T, int B, const int *batch_info,
+                             const int *src_unique, int n_src_unique, const int *tgt_unique,
+                             int n_tgt_unique);
+/* Gradient by parameter name; "src.0.W" / "tgt.0.W" are the H x n_unique small gradients whose
+ * column k belongs to vocabulary id unique[k]. */
+float *orc_trainer_grad(orc_trainer *t, const char *name, long long *n_elems);
+/* NeuralMachineTranslation::UpdateWeights: scale by 1/minibatch_size, clip (0 none, 1 per matrix,
+ * 2 global norm, 3 element clamp), theta += learning_rate * g, clear.  Returns the global norm
+ * (mode 2) or 0. */
+float orc_update_weights(orc_trainer *t, float learning_rate, int clip_mode, float norm_clip,
+                         float individual_clip, int minibatch_size);
+
 #ifdef __cplusplus
 }
 #endif

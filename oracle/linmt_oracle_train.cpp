@@ -1,0 +1,503 @@
+// CPU oracle, training half: teacher-forced forward with stored activations, the reference's
+// backward pass and its weight update.  TEST INFRASTRUCTURE ONLY (see linmt_oracle.h).
+//
+// Follows NeuralMachineTranslation::ComputeGradients (src/deep_rnn.h:984-1299) node by node, in the
+// reference's order (target steps last to first, layers top to bottom, then the source side), with
+// every gradient accumulated per step in fp32 as the reference's beta = 1 SGEMMs do:
+//   softmax        src/layer_loss.h:547-626 (GetHTGradientGpu), :887-972 (D and b_d gradients)
+//   attention      src/layer_attention.h:487-698 and the kernels of src/deep_rnn_kernel.h:1348-1520
+//   LSTM cell      src/node_input_to_hidden.h:647-983, :997-1300; src/node_hidden_to_hidden.h:537-1108
+//   embedding      WSmallGradientKernel, src/deep_rnn_kernel.h:270-285
+//   update         src/deep_rnn.h:1326-1412; src/layer_input_to_hidden.h:1062-1276,1283-1360,1428-1470
+//
+// pin: tests compare every gradient with central differences of an independent float64 numpy
+// restatement of the forward pass (the reference's own check, src/layer_input_to_hidden.h:1016-1051,
+// is the same method), and the update with its closed form.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "linmt_oracle.h"
+
+namespace {
+
+inline size_t idx2c(size_t i, size_t j, size_t ld) { return j * ld + i; }
+const char *kGate[4] = {"i", "f", "c", "o"};  // stacked order i, f, c' (tanh), o
+
+typedef std::vector<float> Vec;
+
+struct CellTape {
+  Vec x, h_prev, c_prev, h_tild_prev, gates, c, h;
+  std::vector<int> idx0, mask;
+  bool feed = false;
+};
+
+struct AttnTape {
+  Vec tanh1, sigma, p_t, wa, align, cached_exp, ctx, h_tild;
+  std::vector<int> indices;
+};
+
+}  // namespace
+
+struct orc_trainer {
+  orc_model *m = nullptr;
+  orc_model_config cfg;
+  std::map<std::string, Vec> grads;
+  std::vector<int> uniq[2];  // unique vocabulary ids of the minibatch, source / target input side
+};
+
+namespace {
+
+float *P(orc_trainer *t, const std::string &name) {
+  long long n = 0;
+  float *p = orc_model_param(t->m, name.c_str(), &n);
+  if (!p) {
+    fprintf(stderr, "orc_trainer: unknown parameter %s\n", name.c_str());
+    exit(EXIT_FAILURE);
+  }
+  return p;
+}
+
+Vec &G(orc_trainer *t, const std::string &name, size_t n) {
+  Vec &g = t->grads[name];
+  if (g.size() != n) g.assign(n, 0.f);
+  return g;
+}
+
+// y = P x for the H x H parameter `name` (col-major), optionally transposed.
+void apply(orc_trainer *t, const std::string &name, int transA, const float *x, int B, float beta,
+           float *y) {
+  const int H = t->cfg.H;
+  orc_gemm(H, B, H, P(t, name), H, transA, x, H, 0, 1.f, beta, y, H);
+}
+
+// grad(name) += a b^T  (a, b: H x B)
+void outer_acc(orc_trainer *t, const std::string &name, const float *a, const float *b, int B) {
+  const int H = t->cfg.H;
+  Vec &g = G(t, name, (size_t)H * H);
+  orc_gemm(H, H, B, a, H, 0, b, H, 1, 1.f, 1.f, g.data(), H);
+}
+
+// grad(name) += a 1
+void rowsum_acc(orc_trainer *t, const std::string &name, const float *a, int rows, int B) {
+  Vec &g = G(t, name, rows);
+  for (int r = 0; r < rows; ++r) {
+    float s = 0.f;
+    for (int b = 0; b < B; ++b) s += a[idx2c(r, b, rows)];
+    g[r] += s;
+  }
+}
+
+// Forward of one LSTM node with its tape.
+void cell_forward(orc_trainer *t, const std::string &pfx, int B, CellTape &tp) {
+  const int H = t->cfg.H;
+  Vec p1((size_t)4 * H * B), p2((size_t)4 * H * B), p3, tmp((size_t)H * B), bias((size_t)4 * H);
+  if (tp.feed) p3.resize((size_t)4 * H * B);
+  for (int g = 0; g < 4; ++g) {
+    const std::string gn = kGate[g];
+    auto put = [&](Vec &dst) {
+      for (int b = 0; b < B; ++b)
+        memcpy(&dst[idx2c((size_t)g * H, b, (size_t)4 * H)], &tmp[(size_t)b * H], sizeof(float) * H);
+    };
+    apply(t, pfx + "M_" + gn, 0, tp.x.data(), B, 0.f, tmp.data());
+    put(p1);
+    apply(t, pfx + "W_h" + gn, 0, tp.h_prev.data(), B, 0.f, tmp.data());
+    put(p2);
+    if (tp.feed) {
+      apply(t, pfx + "Q_" + gn, 0, tp.h_tild_prev.data(), B, 0.f, tmp.data());
+      put(p3);
+    }
+    memcpy(&bias[(size_t)g * H], P(t, pfx + "b_" + gn), sizeof(float) * H);
+  }
+  tp.gates.assign((size_t)4 * H * B, 0.f);
+  tp.c.assign((size_t)H * B, 0.f);
+  tp.h.assign((size_t)H * B, 0.f);
+  orc_lstm_cell_fwd(H, B, p1.data(), p2.data(), tp.feed ? p3.data() : nullptr, bias.data(),
+                    tp.c_prev.data(), tp.mask.data(), tp.feed ? 1 : 0, 0.f, tp.gates.data(),
+                    tp.c.data(), tp.h.data());
+}
+
+// Backward of one LSTM node.  dh_above may be NULL (zero).  dh_next / dc_next are the errors handed
+// back by node t+1 and are replaced by the ones for node t-1.  dx receives M^T d (H x B);
+// dh_tild_below (feed input, t > 0) receives Q^T d.
+void cell_backward(orc_trainer *t, const std::string &pfx, int B, const CellTape &tp,
+                   const float *dh_above, Vec &dh_next, Vec &dc_next, Vec &dx, Vec *dh_tild_below) {
+  const int H = t->cfg.H;
+  const size_t n = (size_t)H * B;
+  Vec d[4];
+  for (auto &v : d) v.assign(n, 0.f);
+  Vec dc_prev(n, 0.f);
+  for (int b = 0; b < B; ++b)
+    for (int r = 0; r < H; ++r) {
+      const size_t o = idx2c(r, b, H);
+      const float it = tp.gates[idx2c(0 * (size_t)H + r, b, (size_t)4 * H)];
+      const float ft = tp.gates[idx2c(1 * (size_t)H + r, b, (size_t)4 * H)];
+      const float gt = tp.gates[idx2c(2 * (size_t)H + r, b, (size_t)4 * H)];
+      const float ot = tp.gates[idx2c(3 * (size_t)H + r, b, (size_t)4 * H)];
+      // d_errn_to_t_ht = d_errn_to_tp1_ht + d_errt_ht (geam), node_input_to_hidden.h:700
+      float dh = dh_next[o] + (dh_above ? dh_above[o] : 0.f);
+      // DErrtCTKernel, deep_rnn_kernel.h:152: dh * o * (1 - tanh(c)^2)
+      const float tc = tanhf(tp.c[o]);
+      float dc = dc_next[o] + dh * ot * (1.0f - tc * tc);
+      // ZeroColumnsKernel on both
+      dh = dh * tp.mask[b];
+      dc = dc * tp.mask[b];
+      d[3][o] = dh * tc * ot * (1 - ot);                 // DErrnToTOTKernel
+      d[1][o] = dc * tp.c_prev[o] * ft * (1 - ft);       // DErrnToTFTITKernel
+      d[2][o] = dc * it * (1 - gt * gt);                 // DErrnToTTanhcptKernel
+      d[0][o] = dc * gt * it * (1 - it);                 // DErrnToTFTITKernel
+      dc_prev[o] = dc * ft;                              // ElementwiseMultKernel
+    }
+  Vec dh_prev(n, 0.f);
+  dx.assign(n, 0.f);
+  for (int g = 0; g < 4; ++g) {
+    const std::string gn = kGate[g];
+    apply(t, pfx + "W_h" + gn, 1, d[g].data(), B, 1.f, dh_prev.data());
+    apply(t, pfx + "M_" + gn, 1, d[g].data(), B, 1.f, dx.data());
+  }
+  if (tp.feed && dh_tild_below) {
+    dh_tild_below->assign(n, 0.f);
+    for (int g = 0; g < 4; ++g)
+      apply(t, pfx + std::string("Q_") + kGate[g], 1, d[g].data(), B, 1.f, dh_tild_below->data());
+  }
+  // ComputeGradientsGpu
+  for (int g = 0; g < 4; ++g) {
+    const std::string gn = kGate[g];
+    outer_acc(t, pfx + "W_h" + gn, d[g].data(), tp.h_prev.data(), B);
+    outer_acc(t, pfx + "M_" + gn, d[g].data(), tp.x.data(), B);
+    if (tp.feed) outer_acc(t, pfx + "Q_" + gn, d[g].data(), tp.h_tild_prev.data(), B);
+    rowsum_acc(t, pfx + "b_" + gn, d[g].data(), H, B);
+  }
+  dh_next = dh_prev;
+  dc_next = dc_prev;
+}
+
+// WSmallGradientKernel: small_grad[:, rev[idx0_b]] += dx[:, b].  Pad columns carry dx = 0.
+void scatter_embedding(orc_trainer *t, const std::string &name, int side, const Vec &dx,
+                       const CellTape &tp, int B) {
+  const int H = t->cfg.H;
+  const std::vector<int> &u = t->uniq[side];
+  Vec &g = G(t, name, (size_t)H * u.size());
+  for (int b = 0; b < B; ++b) {
+    if (!tp.mask[b]) continue;
+    int k = -1;
+    for (size_t j = 0; j < u.size(); ++j)
+      if (u[j] == tp.idx0[b]) {
+        k = (int)j;
+        break;
+      }
+    if (k < 0) {
+      fprintf(stderr, "orc_trainer: id %d missing from the unique list\n", tp.idx0[b]);
+      exit(EXIT_FAILURE);
+    }
+    for (int r = 0; r < H; ++r) g[idx2c(r, k, H)] += dx[idx2c(r, b, H)];
+  }
+}
+
+}  // namespace
+
+extern "C" orc_trainer *orc_trainer_create(orc_model *m, const orc_model_config *cfg) {
+  orc_trainer *t = new orc_trainer();
+  t->m = m;
+  t->cfg = *cfg;
+  return t;
+}
+
+extern "C" void orc_trainer_destroy(orc_trainer *t) { delete t; }
+
+extern "C" float *orc_trainer_grad(orc_trainer *t, const char *name, long long *n_elems) {
+  const auto it = t->grads.find(name);
+  if (it == t->grads.end()) return nullptr;
+  if (n_elems) *n_elems = (long long)it->second.size();
+  return it->second.data();
+}
+
+extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, const int *tgt_in,
+                                        const int *tgt_out, int T, int B, const int *batch_info,
+                                        const int *src_unique, int n_src_unique,
+                                        const int *tgt_unique, int n_tgt_unique) {
+  const orc_model_config &cfg = t->cfg;
+  const int H = cfg.H, L = cfg.layers, V = cfg.V_tgt;
+  const size_t n = (size_t)H * B;
+  const bool attn = cfg.attention != 0;
+  const bool feed_cfg = attn && cfg.feed_input;
+  const int D = cfg.attention == 1 ? cfg.D : -1;
+  const int W = D >= 0 ? 2 * D + 1 : S;
+  t->uniq[0].assign(src_unique, src_unique + n_src_unique);
+  t->uniq[1].assign(tgt_unique, tgt_unique + n_tgt_unique);
+  for (auto &kv : t->grads) std::fill(kv.second.begin(), kv.second.end(), 0.f);
+  G(t, "src.0.W", (size_t)H * n_src_unique);
+  G(t, "tgt.0.W", (size_t)H * n_tgt_unique);
+
+  // ------------------------------------------------------------------------------ forward
+  std::vector<std::vector<CellTape>> enc(S, std::vector<CellTape>(L)), dec(T, std::vector<CellTape>(L));
+  std::vector<AttnTape> att(T);
+  Vec zeros(n, 0.f);
+  Vec hs((size_t)S * n);
+  for (int s = 0; s < S; ++s)
+    for (int l = 0; l < L; ++l) {
+      CellTape &tp = enc[s][l];
+      tp.idx0.resize(B);
+      tp.mask.resize(B);
+      orc_preprocess_indices(src + (size_t)s * B, B, tp.idx0.data(), tp.mask.data(), nullptr);
+      tp.x.assign(n, 0.f);
+      if (l == 0)
+        orc_embed_lookup(P(t, "src.0.W"), H, cfg.V_src, tp.idx0.data(), B, nullptr, 1.f, tp.x.data());
+      else
+        tp.x = enc[s][l - 1].h;
+      tp.h_prev = s ? enc[s - 1][l].h : zeros;
+      tp.c_prev = s ? enc[s - 1][l].c : zeros;
+      cell_forward(t, "src." + std::to_string(l) + ".", B, tp);
+      if (l == L - 1) memcpy(&hs[(size_t)s * n], tp.h.data(), sizeof(float) * n);
+    }
+  double loglik = 0;
+  std::vector<Vec> dz(T);           // (onehot - p) * mask, V x B per step
+  std::vector<std::vector<int>> tgt_mask(T);
+  for (int s = 0; s < T; ++s) {
+    for (int l = 0; l < L; ++l) {
+      CellTape &tp = dec[s][l];
+      tp.idx0.resize(B);
+      tp.mask.resize(B);
+      orc_preprocess_indices(tgt_in + (size_t)s * B, B, tp.idx0.data(), tp.mask.data(), nullptr);
+      tp.x.assign(n, 0.f);
+      if (l == 0)
+        orc_embed_lookup(P(t, "tgt.0.W"), H, V, tp.idx0.data(), B, nullptr, 1.f, tp.x.data());
+      else
+        tp.x = dec[s][l - 1].h;
+      tp.h_prev = s ? dec[s - 1][l].h : (S ? enc[S - 1][l].h : zeros);
+      tp.c_prev = s ? dec[s - 1][l].c : (S ? enc[S - 1][l].c : zeros);
+      tp.feed = l == 0 && feed_cfg && s != 0;
+      if (tp.feed) tp.h_tild_prev = att[s - 1].h_tild;
+      cell_forward(t, "tgt." + std::to_string(l) + ".", B, tp);
+    }
+    const float *top = dec[s][L - 1].h.data();
+    if (attn) {
+      AttnTape &a = att[s];
+      a.tanh1.assign(n, 0.f);
+      a.wa.assign(n, 0.f);
+      a.sigma.assign(B, 0.f);
+      a.p_t.assign(B, 0.f);
+      a.align.assign((size_t)B * W, 0.f);
+      a.cached_exp.assign((size_t)B * W, 1.f);
+      a.indices.assign((size_t)B * W, -1);
+      a.ctx.assign(n, 0.f);
+      a.h_tild.assign(n, 0.f);
+      if (D >= 0) {
+        apply(t, "attn.W_p", 0, top, B, 0.f, a.tanh1.data());
+        for (auto &v : a.tanh1) v = tanhf(v);
+      }
+      apply(t, "attn.W_a", 1, top, B, 0.f, a.wa.data());
+      orc_attn_core_fwd(H, B, D, S, S, a.tanh1.data(), P(t, "attn.v_p"), a.wa.data(), hs.data(),
+                        (long long)n, H, nullptr, batch_info, dec[s][L - 1].mask.data(),
+                        a.p_t.data(), a.sigma.data(), a.indices.data(), a.align.data(),
+                        a.cached_exp.data(), a.ctx.data(), nullptr);
+      Vec t1(n), t2(n);
+      apply(t, "attn.W_c1", 0, a.ctx.data(), B, 0.f, t1.data());
+      apply(t, "attn.W_c2", 0, top, B, 0.f, t2.data());
+      const float *b_out = P(t, "attn.b_out");
+      for (int b = 0; b < B; ++b)
+        for (int r = 0; r < H; ++r) {
+          const size_t o = idx2c(r, b, H);
+          a.h_tild[o] = tanhf(t1[o] + t2[o] + b_out[r]) * dec[s][L - 1].mask[b];
+        }
+      top = a.h_tild.data();
+    }
+    // softmax: p, log-likelihood, and the output error (onehot - p) * mask of GetHTGradientGpu
+    Vec logits((size_t)V * B), p((size_t)V * B);
+    orc_gemm(V, B, H, P(t, "softmax.D"), V, 0, top, H, 0, 1.f, 0.f, logits.data(), V);
+    orc_softmax_fwd(logits.data(), V, P(t, "softmax.b_d"), V, B, p.data(), V);
+    std::vector<int> t0(B);
+    tgt_mask[s].resize(B);
+    orc_preprocess_indices(tgt_out + (size_t)s * B, B, t0.data(), tgt_mask[s].data(), nullptr);
+    orc_train_loglik(p.data(), V, V, B, t0.data(), tgt_mask[s].data(), &loglik);
+    dz[s].assign((size_t)V * B, 0.f);
+    for (int b = 0; b < B; ++b) {
+      if (!tgt_mask[s][b]) continue;
+      for (int v = 0; v < V; ++v) dz[s][idx2c(v, b, V)] = -p[idx2c(v, b, V)];
+      dz[s][idx2c(t0[b], b, V)] += 1.f;
+    }
+  }
+
+  // ------------------------------------------------------------------------------ backward, target
+  std::vector<Vec> dh_next(L, Vec(n, 0.f)), dc_next(L, Vec(n, 0.f));
+  std::vector<Vec> dHS(S, Vec(n, 0.f));  // error into the top source layer, per source step
+  Vec dh_tild_feed;                      // Q^T d from the input layer of step t+1
+  bool have_feed = false;
+  Vec &gD = G(t, "softmax.D", (size_t)V * H);
+  for (int s = T - 1; s >= 0; --s) {
+    const float *h_in = attn ? att[s].h_tild.data() : dec[s][L - 1].h.data();
+    Vec dht(n, 0.f);
+    orc_gemm(H, B, V, P(t, "softmax.D"), V, 1, dz[s].data(), V, 0, 1.f, 0.f, dht.data(), H);
+    orc_gemm(V, H, B, dz[s].data(), V, 0, h_in, H, 1, 1.f, 1.f, gD.data(), V);
+    rowsum_acc(t, "softmax.b_d", dz[s].data(), V, B);
+
+    Vec dh_top;  // error into the top decoder layer
+    if (attn) {
+      const AttnTape &a = att[s];
+      const CellTape &topc = dec[s][L - 1];
+      const float *ha = topc.h.data();
+      Vec delta = dht;
+      if (feed_cfg && have_feed)
+        for (size_t i = 0; i < n; ++i) delta[i] += dh_tild_feed[i];
+      for (int b = 0; b < B; ++b)
+        for (int r = 0; r < H; ++r) {
+          const size_t o = idx2c(r, b, H);
+          delta[o] = delta[o] * topc.mask[b];                          // ZeroHT
+          delta[o] = delta[o] * (1 - a.h_tild[o] * a.h_tild[o]);       // TanhGradKernel
+        }
+      outer_acc(t, "attn.W_c1", delta.data(), a.ctx.data(), B);
+      outer_acc(t, "attn.W_c2", delta.data(), ha, B);
+      rowsum_acc(t, "attn.b_out", delta.data(), H, B);
+      Vec dctx(n, 0.f), dha(n, 0.f);
+      apply(t, "attn.W_c1", 1, delta.data(), B, 0.f, dctx.data());
+      apply(t, "attn.W_c2", 1, delta.data(), B, 0.f, dha.data());
+      const float sigma_sq = (float)((D * D) / 4.0);
+      Vec hsum(n, 0.f), u(n, 0.f), w(n, 0.f);
+      for (int b = 0; b < B; ++b) {
+        const int len = batch_info[b], off = batch_info[B + b];
+        std::vector<float> das(W, 0.f), r(W, 0.f);
+        std::vector<const float *> hsp(W, nullptr);
+        std::vector<int> tau(W, -1);
+        for (int j = 0; j < W; ++j) {
+          const int idx = a.indices[idx2c(b, j, B)];
+          if (idx == -1) continue;
+          tau[j] = len - 1 - idx + off;
+          hsp[j] = &hs[(size_t)tau[j] * n + (size_t)b * H];
+          float acc = 0.f;  // ErrorAlignmentsKernelLarge
+          for (int k = 0; k < H; ++k) acc += dctx[idx2c(k, b, H)] * hsp[j][k];
+          das[j] = acc;
+        }
+        // ErrorHSAndCTKernelLarge
+        for (int j = 0; j < W; ++j)
+          if (tau[j] >= 0)
+            for (int k = 0; k < H; ++k)
+              dHS[tau[j]][idx2c(k, b, H)] += dctx[idx2c(k, b, H)] * a.align[idx2c(b, j, B)];
+        if (D >= 0) {
+          float dp = 0.f;  // ErrorPTKernel (all slots; invalid ones carry alignment 0)
+          for (int j = 0; j < W; ++j)
+            dp += das[j] * a.align[idx2c(b, j, B)] *
+                  ((a.indices[idx2c(b, j, B)] - a.p_t[b]) / sigma_sq);
+          const float sg = a.sigma[b];
+          for (int k = 0; k < H; ++k) {
+            const size_t o = idx2c(k, b, H);
+            u[o] = dp * sg * (1 - sg) * len * a.tanh1[o];                               // AttentionVPErrorKernel
+            w[o] = dp * len * P(t, "attn.v_p")[k] * sg * (1 - sg) * (1 - a.tanh1[o] * a.tanh1[o]);  // GradWPKernel
+          }
+        }
+        for (int j = 0; j < W; ++j) {  // GetHTScalingsWaGradKernel
+          const float aj = a.align[idx2c(b, j, B)], gj = a.cached_exp[idx2c(j, b, W)];
+          float v = das[j] * aj * (1 - aj / gj);
+          for (int k = 0; k < W; ++k)
+            if (k != j) v += -1 * das[k] * a.align[idx2c(b, k, B)] * aj / gj;
+          r[j] = v;
+        }
+        for (int j = 0; j < W; ++j) {
+          if (tau[j] < 0) continue;  // hs_mat holds zeros there; CopyErrorsSource skips index -1
+          for (int k = 0; k < H; ++k) {
+            hsum[idx2c(k, b, H)] += hsp[j][k] * r[j];                       // ScaleHTKernel + AddTwoMats
+            dHS[tau[j]][idx2c(k, b, H)] += a.wa[idx2c(k, b, H)] * r[j];     // ScaleHTKernel + CopyErrorsSource
+          }
+        }
+      }
+      if (D >= 0) {
+        rowsum_acc(t, "attn.v_p", u.data(), H, B);
+        outer_acc(t, "attn.W_p", w.data(), ha, B);
+        apply(t, "attn.W_p", 1, w.data(), B, 1.f, dha.data());
+      }
+      outer_acc(t, "attn.W_a", ha, hsum.data(), B);
+      apply(t, "attn.W_a", 0, hsum.data(), B, 1.f, dha.data());
+      dh_top = dha;
+    } else {
+      dh_top = dht;
+    }
+
+    Vec dx, dh_above = dh_top;
+    for (int l = L - 1; l >= 0; --l) {
+      Vec feed_out;
+      cell_backward(t, "tgt." + std::to_string(l) + ".", B, dec[s][l], dh_above.data(), dh_next[l],
+                    dc_next[l], dx, dec[s][l].feed ? &feed_out : nullptr);
+      if (l == 0) {
+        scatter_embedding(t, "tgt.0.W", 1, dx, dec[s][0], B);
+        have_feed = dec[s][0].feed;
+        if (have_feed) dh_tild_feed = feed_out;
+      } else {
+        dh_above = dx;
+      }
+    }
+  }
+  // ------------------------------------------------------------------------------ backward, source
+  for (int s = S - 1; s >= 0; --s) {
+    Vec dx, dh_above = attn ? dHS[s] : zeros;
+    for (int l = L - 1; l >= 0; --l) {
+      cell_backward(t, "src." + std::to_string(l) + ".", B, enc[s][l], dh_above.data(), dh_next[l],
+                    dc_next[l], dx, nullptr);
+      if (l == 0)
+        scatter_embedding(t, "src.0.W", 0, dx, enc[s][0], B);
+      else
+        dh_above = dx;
+    }
+  }
+  return loglik;
+}
+
+// NeuralMachineTranslation::UpdateWeights.  Every gradient is first divided by the minibatch size
+// (ScaleGradients); then
+//   clip_mode 2 (global, --whole-clip-gradients): norm over every gradient EXCEPT the two embedding
+//     small gradients (they are absent from CalculateGlobalNorm, layer_input_to_hidden.h:1062-1098),
+//     and if it exceeds the threshold every gradient INCLUDING those two is rescaled
+//     (UpdateGlobalParams, :1102-1141);
+//   clip_mode 1 (per matrix, NormClipGpuV2): each named matrix is rescaled to the threshold alone;
+//   clip_mode 3 (individual): every element clamped to +-individual_clip;
+//   clip_mode 0: nothing.
+// Then theta += learning_rate * g (embeddings: only the columns of the unique ids) and the gradients
+// are cleared.  Returns the global norm (clip_mode 2) or 0.
+extern "C" float orc_update_weights(orc_trainer *t, float learning_rate, int clip_mode,
+                                    float norm_clip, float individual_clip, int minibatch_size) {
+  const int H = t->cfg.H;
+  for (auto &kv : t->grads)
+    for (auto &v : kv.second) v = (1.0f / minibatch_size) * v;
+  float global = 0.f;
+  auto sumsq = [](const Vec &g) {
+    float s = 0.f;
+    for (float v : g) s += v * v;
+    return s;
+  };
+  if (clip_mode == 2) {
+    for (auto &kv : t->grads)
+      if (kv.first != "src.0.W" && kv.first != "tgt.0.W") global += sumsq(kv.second);
+    global = std::sqrt(global);
+    if (global > norm_clip)
+      for (auto &kv : t->grads)
+        for (auto &v : kv.second) v = (norm_clip / global) * v;
+  } else if (clip_mode == 1) {
+    for (auto &kv : t->grads) {
+      const float nrm = std::sqrt(sumsq(kv.second));
+      if (nrm > norm_clip)
+        for (auto &v : kv.second) v = (norm_clip / nrm) * v;
+    }
+  } else if (clip_mode == 3) {
+    for (auto &kv : t->grads)
+      for (auto &v : kv.second)
+        v = v > individual_clip ? individual_clip : (v < -individual_clip ? -individual_clip : v);
+  }
+  for (auto &kv : t->grads) {
+    long long n = 0;
+    float *p = orc_model_param(t->m, kv.first.c_str(), &n);
+    if (!p) continue;
+    if (kv.first == "src.0.W" || kv.first == "tgt.0.W") {
+      const std::vector<int> &u = t->uniq[kv.first == "src.0.W" ? 0 : 1];
+      for (size_t k = 0; k < u.size(); ++k)  // UpdateSparseGradient
+        for (int r = 0; r < H; ++r)
+          p[idx2c(r, u[k], H)] += learning_rate * kv.second[idx2c(r, k, H)];
+    } else {
+      for (long long i = 0; i < n; ++i) p[i] += learning_rate * kv.second[i];
+    }
+    std::fill(kv.second.begin(), kv.second.end(), 0.f);
+  }
+  orc_model_commit(t->m);
+  return global;
+}

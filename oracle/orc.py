@@ -42,6 +42,10 @@ def lib():
         _lib.orc_model_param.restype = C.c_void_p
         _lib.orc_forward_xent.restype = C.c_double
         _lib.orc_decode_sentence.restype = C.c_int
+        _lib.orc_trainer_create.restype = C.c_void_p
+        _lib.orc_trainer_grad.restype = C.c_void_p
+        _lib.orc_compute_gradients.restype = C.c_double
+        _lib.orc_update_weights.restype = C.c_float
     return _lib
 
 
@@ -258,8 +262,69 @@ class Model:
         return lib().orc_forward_xent(self.handle, _p(src), S, _p(tgt_in), _p(tgt_out), T, B,
                                       _p(i32(batch_info)), num_threads)
 
+    # ---- training -------------------------------------------------------------------------------
+    def compute_gradients(self, src, tgt_in, tgt_out, batch_info, src_unique, tgt_unique):
+        """Forward + backward (no update).  Returns (sum log p, {name: gradient}); matrices come back
+        as Fortran-ordered 2-D arrays, the embedding gradients as (H, n_unique)."""
+        if getattr(self, "trainer", None) is None:
+            self.trainer = C.c_void_p(lib().orc_trainer_create(self.handle, C.byref(self.cfg)))
+        src = np.asfortranarray(src, np.int32)
+        tgt_in = np.asfortranarray(tgt_in, np.int32)
+        tgt_out = np.asfortranarray(tgt_out, np.int32)
+        B, S = src.shape
+        T = tgt_in.shape[1]
+        su, tu = i32(src_unique), i32(tgt_unique)
+        ll = lib().orc_compute_gradients(self.trainer, _p(src), S, _p(tgt_in), _p(tgt_out), T, B,
+                                         _p(i32(batch_info)), _p(su), su.size, _p(tu), tu.size)
+        return ll, {name: self.grad(name) for name in self.param_names()}
+
+    def param_names(self):
+        c = self.cfg
+        names = []
+        for side in ("src", "tgt"):
+            for l in range(c.layers):
+                for g in "ifco":
+                    names += [f"{side}.{l}.W_h{g}", f"{side}.{l}.M_{g}", f"{side}.{l}.b_{g}"]
+                    if side == "tgt" and l == 0 and c.feed_input and c.attention:
+                        names.append(f"{side}.{l}.Q_{g}")
+                if l == 0:
+                    names.append(f"{side}.{l}.W")
+        if c.attention:
+            names += ["attn.W_a", "attn.W_c1", "attn.W_c2", "attn.b_out"]
+            if c.attention == 1:
+                names += ["attn.W_p", "attn.v_p"]
+        return names + ["softmax.D", "softmax.b_d"]
+
+    def grad(self, name):
+        n = C.c_longlong(0)
+        ptr = lib().orc_trainer_grad(self.trainer, name.encode(), C.byref(n))
+        if not ptr:
+            raise KeyError(name)
+        flat = np.frombuffer((C.c_float * n.value).from_address(ptr), dtype=np.float32).copy()
+        H = self.cfg.H
+        if name == "softmax.D":
+            return flat.reshape((self.cfg.V_tgt, H), order="F")
+        if flat.size % H == 0 and flat.size > H and not name.endswith("b_d"):
+            return flat.reshape((H, flat.size // H), order="F")
+        return flat
+
+    def update_weights(self, learning_rate, clip_mode, norm_clip, individual_clip, minibatch_size):
+        return float(lib().orc_update_weights(self.trainer, _f(learning_rate), clip_mode,
+                                              _f(norm_clip), _f(individual_clip), minibatch_size))
+
+    def get_param(self, name):
+        flat = self.param(name).copy()
+        H = self.cfg.H
+        if name == "softmax.D":
+            return flat.reshape((self.cfg.V_tgt, H), order="F")
+        if flat.size % H == 0 and flat.size > H and not name.endswith("b_d"):
+            return flat.reshape((H, flat.size // H), order="F")
+        return flat
+
     def __del__(self):
         try:
+            if getattr(self, "trainer", None) is not None:
+                lib().orc_trainer_destroy(self.trainer)
             lib().orc_model_destroy(self.handle)
         except Exception:
             pass

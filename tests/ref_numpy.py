@@ -200,3 +200,53 @@ def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=Tr
         if n / S > min_ratio and (best is None or r > best_s):
             best, best_s = toks, r
     return (best[1:-1] if best is not None else []), best_s, hyps
+
+
+def minibatch_loglik(P, layers, H, D, sents, attention=True, feed_input=True):
+    """Teacher-forced sum of log p(target) over a list of (source ids, target ids without
+    <START>/<EOF>) sentence pairs, float64, one sentence at a time (no padding involved)."""
+    P = {k: np.asarray(v, np.float64) for k, v in P.items()}
+    total = 0.0
+    for s, t in sents:
+        he, ce, top = encode(P, layers, H, s)
+        h, c = [x.copy() for x in he], [x.copy() for x in ce]
+        h_tild = None
+        for step, (wi, wo) in enumerate(zip(np.concatenate([[0], t]), np.concatenate([t, [1]]))):
+            x = P["tgt.0.W"][:, [int(wi)]]
+            for l in range(layers):
+                ht = h_tild if (l == 0 and step != 0 and attention and feed_input) else None
+                h[l], c[l], _ = lstm_step(P, f"tgt.{l}.", x, h[l], c[l], ht)
+                x = h[l]
+            if attention:
+                h_tild, _ = attention_local_p(P, x, lambda _b, pos: top[pos], [len(s)], [1], D)
+                x = h_tild
+            lp = log_softmax(P["softmax.D"] @ x + P["softmax.b_d"][:, None])
+            total += lp[int(wo), 0]
+    return total
+
+
+def pack_minibatch(sents):
+    """Reference minibatch layout (src/file_helper.cc:113-381): source reversed and left-padded,
+    target right-padded, -1 padding, batch_info = [len..., S - len...], unique non-pad input ids in
+    first-occurrence order."""
+    B = len(sents)
+    S = max(len(s) for s, _ in sents)
+    T = max(len(t) + 1 for _, t in sents)
+    src = np.full((B, S), -1, np.int32)
+    tin = np.full((B, T), -1, np.int32)
+    tout = np.full((B, T), -1, np.int32)
+    for b, (s, t) in enumerate(sents):
+        src[b, S - len(s):] = np.asarray(s)[::-1]
+        tin[b, :len(t) + 1] = np.concatenate([[0], t])
+        tout[b, :len(t) + 1] = np.concatenate([t, [1]])
+    lens = np.array([len(s) for s, _ in sents])
+    bi = np.concatenate([lens, S - lens]).astype(np.int32)
+
+    def uniq(a):
+        seen = []
+        for v in a.ravel(order="F"):
+            if v != -1 and v not in seen:
+                seen.append(int(v))
+        return np.array(seen, np.int32)
+
+    return src, tin, tout, bi, uniq(src), uniq(tin)

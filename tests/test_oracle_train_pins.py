@@ -1,0 +1,141 @@
+"""Pins for the training half of the CPU oracle (oracle/linmt_oracle_train.cpp).
+
+The oracle restates the reference's backward pass from its sources; nothing in the reference holds
+expected gradients.  What fixes it here is the method the reference itself uses for its gradient
+check (src/layer_input_to_hidden.h:1016-1051): central differences of the forward pass -- taken on
+an INDEPENDENT float64 numpy forward (tests/ref_numpy.py), so a dropped term, a transposed operand
+or a wrong gate in the backward restatement fails.  The update is pinned by its closed form."""
+import numpy as np
+import pytest
+
+import ref_numpy as R
+
+
+def _sentences(rng, Vs, Vt, lens_s, lens_t):
+    return [(rng.integers(0, Vs, size=a), rng.integers(3, Vt, size=b)) for a, b in zip(lens_s, lens_t)]
+
+
+def _model(orc, rng, layers, H, Vs, Vt, attention, feed, D, scale=0.5):
+    P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(attention), feed_input=bool(feed),
+                      scale=scale)
+    m = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=feed, longest_sent=40)
+    m.set_params(P)
+    return P, m
+
+
+CASES = [
+    dict(layers=2, attention=1, feed=1, D=2, seed=21),
+    dict(layers=1, attention=1, feed=0, D=1, seed=22),
+    dict(layers=2, attention=0, feed=0, D=2, seed=23),
+    dict(layers=3, attention=1, feed=1, D=3, seed=24),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: f"L{c['layers']}a{c['attention']}f{c['feed']}")
+def test_gradients_vs_central_differences(orc, case):
+    rng = np.random.default_rng(case["seed"])
+    layers, H, Vs, Vt, D = case["layers"], 7, 13, 11, case["D"]
+    P, m = _model(orc, rng, layers, H, Vs, Vt, case["attention"], case["feed"], D)
+    sents = _sentences(rng, Vs, Vt, [5, 3, 7, 4], [4, 6, 2, 5])
+    src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
+    ll, grads = m.compute_gradients(src, tin, tout, bi, su, tu)
+    kw = dict(attention=bool(case["attention"]), feed_input=bool(case["feed"]))
+    P64 = {k: v.astype(np.float64) for k, v in P.items()}
+    want_ll = R.minibatch_loglik(P64, layers, H, D, sents, **kw)
+    assert abs(ll - want_ll) < 1e-4 * max(1.0, abs(want_ll))
+
+    def dense(name, g):
+        # embedding gradients come back per unique id
+        if name in ("src.0.W", "tgt.0.W"):
+            full = np.zeros_like(P64[name])
+            full[:, su if name == "src.0.W" else tu] = g
+            return full
+        return g.reshape(P64[name].shape, order="F") if g.ndim == 1 and P64[name].ndim == 1 else g
+
+    eps = 1e-5
+    checked = 0
+    for name in m.param_names():
+        g = dense(name, grads[name]).astype(np.float64)
+        assert g.shape == P64[name].shape, name
+        for _ in range(2):
+            direction = rng.standard_normal(P64[name].shape)
+            Pp, Pm = dict(P64), dict(P64)
+            Pp[name] = P64[name] + eps * direction
+            Pm[name] = P64[name] - eps * direction
+            fd = (R.minibatch_loglik(Pp, layers, H, D, sents, **kw)
+                  - R.minibatch_loglik(Pm, layers, H, D, sents, **kw)) / (2 * eps)
+            got = float(np.sum(g * direction))
+            scale = float(np.sqrt(np.sum(g * g) * np.sum(direction * direction)))
+            assert abs(got - fd) <= 2e-3 * scale + 1e-5, (name, got, fd, scale)
+            checked += 1
+    assert checked == 2 * len(m.param_names())
+
+
+def test_embedding_rows_outside_the_minibatch_get_no_gradient(orc):
+    """Dense view of the scatter: ids that do not occur have zero finite-difference gradient, and an
+    id occurring several times gets the sum (compare with a per-occurrence float64 accumulation)."""
+    rng = np.random.default_rng(31)
+    layers, H, Vs, Vt, D = 1, 6, 9, 10, 1
+    P, m = _model(orc, rng, layers, H, Vs, Vt, 1, 1, D)
+    sents = [(np.array([4, 4, 2, 4]), np.array([5, 5, 5])), (np.array([2, 4]), np.array([5, 7]))]
+    src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
+    assert su.tolist() == [4, 2] and tu.tolist() == [0, 5, 7]
+    _, grads = m.compute_gradients(src, tin, tout, bi, su, tu)
+    P64 = {k: v.astype(np.float64) for k, v in P.items()}
+    eps = 1e-5
+    for name, uniq, V in (("src.0.W", su, Vs), ("tgt.0.W", tu, Vt)):
+        for k, vid in enumerate(uniq):
+            for r in (0, H - 1):
+                Pp, Pm = dict(P64), dict(P64)
+                Pp[name] = P64[name].copy()
+                Pm[name] = P64[name].copy()
+                Pp[name][r, vid] += eps
+                Pm[name][r, vid] -= eps
+                fd = (R.minibatch_loglik(Pp, layers, H, D, sents)
+                      - R.minibatch_loglik(Pm, layers, H, D, sents)) / (2 * eps)
+                assert abs(grads[name][r, k] - fd) <= 2e-3 * max(1.0, abs(fd)), (name, vid, r)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_update_closed_form(orc, mode):
+    rng = np.random.default_rng(41 + mode)
+    layers, H, Vs, Vt, D = 2, 6, 9, 10, 1
+    P, m = _model(orc, rng, layers, H, Vs, Vt, 1, 1, D, scale=0.8)
+    sents = _sentences(rng, Vs, Vt, [5, 3, 4], [4, 3, 5])
+    src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
+    _, grads = m.compute_gradients(src, tin, tout, bi, su, tu)
+    B, lr = len(sents), 0.7
+    g = {k: v.astype(np.float64) / B for k, v in grads.items()}
+    dense_names = [k for k in g if k not in ("src.0.W", "tgt.0.W")]
+    total = np.sqrt(sum(np.sum(g[k] ** 2) for k in dense_names))
+    # thresholds chosen so that the clip is active
+    norm_clip = 0.5 * total if mode == 2 else 0.5 * min(np.sqrt(np.sum(g[k] ** 2)) for k in dense_names
+                                                         if np.sum(g[k] ** 2) > 0) * 3
+    ind = 0.25 * max(np.abs(v).max() for v in g.values())
+    if mode == 2:
+        g = {k: v * (norm_clip / total) for k, v in g.items()}  # embeddings rescaled too
+    elif mode == 1:
+        for k in g:
+            n = np.sqrt(np.sum(g[k] ** 2))
+            if n > norm_clip:
+                g[k] = g[k] * (norm_clip / n)
+    elif mode == 3:
+        g = {k: np.clip(v, -ind, ind) for k, v in g.items()}
+    want = {}
+    for k in g:
+        want[k] = P[k].astype(np.float64).copy()
+        if k == "src.0.W":
+            want[k][:, su] += lr * g[k]
+        elif k == "tgt.0.W":
+            want[k][:, tu] += lr * g[k]
+        else:
+            want[k] += lr * g[k].reshape(want[k].shape, order="F")
+    got_norm = m.update_weights(lr, mode, norm_clip, ind, B)
+    if mode == 2:
+        assert abs(got_norm - total) <= 1e-5 * total
+    for k in g:
+        np.testing.assert_allclose(m.get_param(k).reshape(want[k].shape, order="F"), want[k],
+                                   rtol=2e-5, atol=2e-6, err_msg=k)
+    # gradients are cleared by the update
+    for k in g:
+        assert not np.any(m.grad(k)), k
