@@ -251,6 +251,116 @@ int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const int *limit,
 int lh_beam_gather_f32(const float *const *src, float *const *dst, int n_tensors, int H, int B,
                        int B_src, const int *backptr, lh_stream_t stream);
 
+/* ==========================================================================================
+ * Training half of the path (backward pass and update).
+ * ========================================================================================== */
+
+/* ------------------------------------------------------------------------------------------
+ * a16. Softmax output error and log-likelihood in one pass over the V x B logits.
+ * Replaces, for one step, the forward OutputdistOverflowPreventionKernel
+ * (src/deep_rnn_kernel.h:353-429), TrainPerplexityKernel (:336-342) and the elementwise part of
+ * SoftmaxLayer::GetHTGradientGpu / ComputeDGradientGpu / ComputeBDGradientGpu
+ * (src/layer_loss.h:547-626, 887-972), which all consume p and the one-hot target:
+ *   p        = softmax(logits[:,b] + bias)
+ *   dz[:,b]  = mask01[b] * (onehot(tgt0[b]) - p)               (may alias logits)
+ *   logp_tgt[b] = log((double)p[tgt0[b]]) ; *loss_accum += sum_{b: mask01[b]==1} logp_tgt[b]
+ * With dz the three gradient products of the reference are plain GEMMs / row sums:
+ *   dh~ = D^T dz ; dD += dz h~^T ; db_d += dz 1.
+ */
+int lh_softmax_xent_grad_f32(const float *logits, int ldl, const float *bias, int V, int B,
+                             const int *tgt0, const int *mask01, float *dz, int ldz,
+                             double *logp_tgt, double *loss_accum, lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a13. Fused LSTM cell backward: everything between the incoming errors and the four gate errors.
+ * Replaces the two geam sums, DErrtCTKernel (src/deep_rnn_kernel.h:152), ZeroColumnsKernel,
+ * DErrnToTOTKernel, DErrnToTFTITKernel (twice), DErrnToTTanhcptKernel, ElementwiseMultKernel and
+ * the ClipMatKernel calls on incoming errors, as sequenced in LstmInputHiddenNode::BackPropGpu
+ * (src/node_input_to_hidden.h:647-983) and LstmHiddenHiddenNode::BackPropGpu
+ * (src/node_hidden_to_hidden.h:537-900):
+ *   dh  = clamp(dh_next, clip_next) + clamp(dh_above, clip_above)     (NULL = 0; clip <= 0 = off)
+ *   dc  = dc_next + dh * o * (1 - tanh(c)^2) ; dh *= mask01[b] ; dc *= mask01[b]
+ *   do  = dh * tanh(c) * o(1-o) ; df = dc * c_prev * f(1-f) ; di = dc * g * i(1-i)
+ *   dg  = dc * i * (1 - g^2) ; dc_prev = dc * f
+ * gates (4H x B: i,f,g,o as written by lh_lstm_cell_fwd_f32), c, c_prev are the stored forward
+ * values; dgates (4H x B) receives di,df,dg,do in the same stacking, so that
+ *   [dx ; dh_prev ; dh~_prev] = [M | W_h | Q]^T dgates   and   d[M | W_h | Q] += dgates [x;h;h~]^T
+ * are single GEMMs on the stacked weights.  dc_prev may alias dc_next.
+ * The reference clamps the errors it hands back (dh_{t-1}, dh~_{t-1}, dx) to +-error_clip when
+ * --clip-cell is on; here the consumer clamps on read, which is the same values.
+ */
+int lh_lstm_cell_bwd_f32(int H, int B, const float *dh_above, const float *dh_next,
+                         const float *dc_next, const float *gates, const float *c,
+                         const float *c_prev, const int *mask01, float clip_above, float clip_next,
+                         float *dgates, float *dc_prev, lh_stream_t stream);
+
+/* out[r] = beta*out[r] + sum_c A[r,c] for a column-major rows x cols matrix.  Replaces the
+ * cublasSgemv-with-ones bias gradients (src/node_input_to_hidden.h:1215-1240,
+ * src/layer_attention.h:541, :600, src/layer_loss.h:938-972).  Fixed summation order. */
+int lh_rowsum_acc_f32(const float *A, long long lda, int rows, long long cols, float beta,
+                      float *out, lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a14. Embedding gradient.  Replaces WSmallGradientKernel (src/deep_rnn_kernel.h:270-285), whose
+ * atomicAdd scatter makes the sum order vary from run to run: here the caller lists, per unique
+ * id k, the dx columns that carry that id (seg_cols[seg_start[k] .. seg_start[k+1])), and
+ *   small_grad[:,k] = beta*small_grad[:,k] + sum_{s} dx[:, seg_cols[s]]       (E rows)
+ * in list order.  Padding columns are simply not listed.
+ */
+int lh_embed_gather_grad_f32(const float *dx, long long ldx, int E, int n_unique,
+                             const int *seg_start, const int *seg_cols, float beta,
+                             float *small_grad, long long ldg, lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a15. Attention backward.
+ * lh_attn_delta_f32 replaces AddTwoMatsKernel (feed-input error), ZeroHT and TanhGradKernel at the
+ * top of AttentionNode::BackProp (src/layer_attention.h:490-512):
+ *   delta = (dht + clamp(dht_feed, clip_feed)) * mask01[b] * (1 - h_tild^2)    (dht_feed may be NULL)
+ * lh_attn_core_bwd_f32 replaces ErrorAlignmentsKernelLarge, ErrorHSAndCTKernelLarge, ErrorPTKernel,
+ * AttentionVPErrorKernel, GradWPKernel, GetHTScalingsWaGradKernel and the 2D+1 rounds of
+ * ScaleHTKernel / AddTwoMatsKernel / CopyErrorsSource (src/layer_attention.h:572-660,
+ * src/deep_rnn_kernel.h:1348-1520), one workgroup per column; the stored forward values come from
+ * lh_attn_core_fwd_f32 (same layouts), dctx = W_c1^T delta:
+ *   das_j  = dctx[:,b] . hs_j
+ *   dp     = sum_j das_j a_j (idx_j - p_b)/sigma^2                               (local-p only)
+ *   r_j    = das_j a_j - (a_j/g_j) * sum_k das_k a_k
+ *   hsum[:,b] = sum_j r_j hs_j
+ *   dhs(tau_j)[:,b] += dctx[:,b] a_j + wa[:,b] r_j        (valid slots; dhs has the layout of hs)
+ *   u[:,b] = dp sig(1-sig) len tanh1[:,b] ; w[:,b] = dp len sig(1-sig) v_p (1 - tanh1[:,b]^2)
+ * after which dv_p += u 1, dW_p += w ha^T, dW_a += ha hsum^T and dha = W_c2^T delta + W_p^T w +
+ * W_a hsum are row sums / GEMMs.  Every column must own its states (no hs_col sharing).
+ */
+int lh_attn_delta_f32(int H, int B, const float *dht, const float *dht_feed, const float *h_tild,
+                      const int *mask01, float clip_feed, float *delta, lh_stream_t stream);
+int lh_attn_core_bwd_f32(int H, int B, int D, int max_len, int hs_steps, const float *dctx,
+                         const float *tanh1, const float *v_p, const float *wa, const float *hs,
+                         long long hs_step_stride, long long hs_col_stride, const int *batch_info,
+                         const float *p_t, const float *sigma, const int *indices,
+                         const float *align, const float *cached_exp, float *dhs, float *hsum,
+                         float *u, float *w, lh_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * a17. Gradient norm and the fused scale / clip / SGD / clear step.
+ * lh_grad_sumsq_f32 replaces BasicComputeNormP1/P2 + the blocking copy of NormClipGpuV2P1
+ * (src/deep_rnn_kernel.h:618-708): *accum += sum (scale*g)^2 over a rows x cols view (leading
+ * dimension ld), accumulated in double on the device; workspace holds LH_SUMSQ_WORKSPACE doubles.
+ * lh_sgd_step_f32 replaces ScaleFunctor (ScaleGradients), ReScaleNormFunctor (NormClipGpuV2 /
+ * NormClipGpuV2P2), ClipMatKernel (individual clip), the geam / AddGradVecs / UpdateSparseGradient
+ * updates (src/layer_input_to_hidden.h:1145-1276, src/deep_rnn_kernel.h:883-894) and the
+ * cudaMemset of ClearGradients, in one pass:
+ *   v = grad_scale * g ; f = sumsq ? (sqrt(*sumsq) > norm_clip ? norm_clip/sqrt(*sumsq) : 1) : 1
+ *   v = f*v ; individual_clip > 0: v = clamp(v, +-individual_clip)
+ *   theta[:, col_index ? col_index[c] : c] += learning_rate * v ; g = 0
+ * sumsq is read on the device, so no host synchronisation sits between norm and update.
+ */
+#define LH_SUMSQ_WORKSPACE 1024
+int lh_grad_sumsq_f32(const float *g, long long rows, long long cols, long long ld, float scale,
+                      double *workspace, double *accum, lh_stream_t stream);
+int lh_sgd_step_f32(float *theta, long long ld_theta, float *g, long long ld_g, long long rows,
+                    long long cols, const int *col_index, float learning_rate, float grad_scale,
+                    const double *sumsq, float norm_clip, float individual_clip,
+                    lh_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -160,6 +160,77 @@ __global__ __launch_bounds__(kT) void logsoftmax_tgt_generic_kernel(const float 
   }
 }
 
+// ---- training: output error (onehot - p) * mask and log p(target) in one pass ---------------
+// dz may alias logits: a column is fully in registers (or each row is owned by one thread) before
+// anything is written.
+template <int NV>
+__global__ __launch_bounds__(kT) void softmax_xent_grad_kernel(
+    const float *__restrict__ logits, int ldl, const float *__restrict__ bias, int V,
+    const int *__restrict__ tgt0, const int *__restrict__ mask01, float *dz, int ldz,
+    double *__restrict__ logp_tgt) {
+  __shared__ float red[kNW];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  float4 x[NV];
+  load_column<NV>(x, logits + (size_t)b * ldl, bias, V, tid);
+  const float mx = lh::block_max<kNW>(local_max<NV>(x), red);
+  float part = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    x[i].x = expf(x[i].x - mx); x[i].y = expf(x[i].y - mx);
+    x[i].z = expf(x[i].z - mx); x[i].w = expf(x[i].w - mx);
+    part += (x[i].x + x[i].y) + (x[i].z + x[i].w);
+  }
+  const float sum = lh::block_sum<kNW>(part, red);
+  const float m = (float)mask01[b];
+  const int t = tgt0[b];
+  float4 *out = reinterpret_cast<float4 *>(dz + (size_t)b * ldz);
+  const int V4 = V / 4;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int f = tid + i * kT;
+    if (f < V4) {
+      float4 p = make_float4(x[i].x / sum, x[i].y / sum, x[i].z / sum, x[i].w / sum);
+      float4 d = make_float4(-p.x * m, -p.y * m, -p.z * m, -p.w * m);
+      if (t / 4 == f) {
+        const int c = t % 4;
+        logp_tgt[b] = log((double)comp(p, c));
+        comp(d, c) += m;
+      }
+      out[f] = d;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kT) void softmax_xent_grad_generic_kernel(
+    const float *logits, int ldl, const float *bias, int V, const int *tgt0, const int *mask01,
+    float *dz, int ldz, double *logp_tgt) {
+  __shared__ float red[kNW];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const float *col = logits + (size_t)b * ldl;
+  float *out = dz + (size_t)b * ldz;
+  float mxl = kNegInf;
+  for (int r = tid; r < V; r += kT) mxl = fmaxf(mxl, col[r] + (bias ? bias[r] : 0.f));
+  const float mx = lh::block_max<kNW>(mxl, red);
+  float part = 0.f;
+  for (int r = tid; r < V; r += kT) {
+    const float e = expf(col[r] + (bias ? bias[r] : 0.f) - mx);
+    out[r] = e;
+    part += e;
+  }
+  const float sum = lh::block_sum<kNW>(part, red);
+  const float m = (float)mask01[b];
+  const int t = tgt0[b];
+  for (int r = tid; r < V; r += kT) {
+    const float p = out[r] / sum;
+    float d = -p * m;
+    if (r == t) {
+      logp_tgt[b] = log((double)p);
+      d += m;
+    }
+    out[r] = d;
+  }
+}
+
 __global__ void masked_sum_kernel(const double *logp_tgt, const int *mask01, int B, double *accum) {
   if (blockIdx.x != 0 || threadIdx.x != 0) return;
   double acc = 0.0;
@@ -374,6 +445,31 @@ extern "C" int lh_logsoftmax_xent_f32(const float *logits, int ldl, const float 
   if (rc != LH_OK) return rc;
   hipLaunchKernelGGL(masked_sum_kernel, dim3(1), dim3(64), 0, st, logp_tgt, mask01, B, loss_accum);
   return lh::check_launch("lh_logsoftmax_xent_f32 (sum)");
+}
+
+extern "C" int lh_softmax_xent_grad_f32(const float *logits, int ldl, const float *bias, int V,
+                                        int B, const int *tgt0, const int *mask01, float *dz,
+                                        int ldz, double *logp_tgt, double *loss_accum,
+                                        lh_stream_t stream) {
+  if (V <= 0 || B <= 0 || !logits || !tgt0 || !mask01 || !dz || !logp_tgt || !loss_accum ||
+      ldl < V || ldz < V)
+    return lh::fail_arg("lh_softmax_xent_grad_f32: V=%d B=%d ldl=%d ldz=%d or NULL pointer", V, B,
+                        ldl, ldz);
+  hipStream_t st = lh::as_stream(stream);
+  int nv = pick_nv(logits, ldl, bias, V);
+  if (ldz % 4 != 0 || !lh::aligned16(dz)) nv = 0;
+  const dim3 grid(B), block(kT);
+  switch (nv) {
+    case 2: hipLaunchKernelGGL(softmax_xent_grad_kernel<2>, grid, block, 0, st, logits, ldl, bias, V, tgt0, mask01, dz, ldz, logp_tgt); break;
+    case 4: hipLaunchKernelGGL(softmax_xent_grad_kernel<4>, grid, block, 0, st, logits, ldl, bias, V, tgt0, mask01, dz, ldz, logp_tgt); break;
+    case 8: hipLaunchKernelGGL(softmax_xent_grad_kernel<8>, grid, block, 0, st, logits, ldl, bias, V, tgt0, mask01, dz, ldz, logp_tgt); break;
+    case 16: hipLaunchKernelGGL(softmax_xent_grad_kernel<16>, grid, block, 0, st, logits, ldl, bias, V, tgt0, mask01, dz, ldz, logp_tgt); break;
+    default: hipLaunchKernelGGL(softmax_xent_grad_generic_kernel, grid, block, 0, st, logits, ldl, bias, V, tgt0, mask01, dz, ldz, logp_tgt);
+  }
+  int rc = lh::check_launch("lh_softmax_xent_grad_f32");
+  if (rc != LH_OK) return rc;
+  hipLaunchKernelGGL(masked_sum_kernel, dim3(1), dim3(64), 0, st, logp_tgt, mask01, B, loss_accum);
+  return lh::check_launch("lh_softmax_xent_grad_f32 (sum)");
 }
 
 extern "C" int lh_beam_topk_f32(const float *logits, int ldl, const float *bias, int V, int B, int K,

@@ -63,8 +63,29 @@ SIGNATURES = {
                                     c_i32p, c_f32p, c_i32p, c_i32p, c_f32p, C.c_void_p]),
     "lh_beam_gather_f32": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int,
                                      C.c_int, C.c_int, C.c_int, c_i32p, C.c_void_p]),
+    "lh_softmax_xent_grad_f32": (C.c_int, [c_f32p, C.c_int, c_f32p, C.c_int, C.c_int, c_i32p,
+                                           c_i32p, c_f32p, C.c_int, c_f64p, c_f64p, C.c_void_p]),
+    "lh_lstm_cell_bwd_f32": (C.c_int, [C.c_int, C.c_int, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p,
+                                       c_f32p, c_i32p, C.c_float, C.c_float, c_f32p, c_f32p,
+                                       C.c_void_p]),
+    "lh_rowsum_acc_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_int, C.c_longlong, C.c_float, c_f32p,
+                                    C.c_void_p]),
+    "lh_embed_gather_grad_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_int, C.c_int, c_i32p, c_i32p,
+                                           C.c_float, c_f32p, C.c_longlong, C.c_void_p]),
+    "lh_attn_delta_f32": (C.c_int, [C.c_int, C.c_int, c_f32p, c_f32p, c_f32p, c_i32p, C.c_float,
+                                    c_f32p, C.c_void_p]),
+    "lh_attn_core_bwd_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, c_f32p, c_f32p,
+                                       c_f32p, c_f32p, c_f32p, C.c_longlong, C.c_longlong, c_i32p,
+                                       c_f32p, c_f32p, c_i32p, c_f32p, c_f32p, c_f32p, c_f32p,
+                                       c_f32p, c_f32p, C.c_void_p]),
+    "lh_grad_sumsq_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_longlong, C.c_longlong, C.c_float,
+                                    c_f64p, c_f64p, C.c_void_p]),
+    "lh_sgd_step_f32": (C.c_int, [c_f32p, C.c_longlong, c_f32p, C.c_longlong, C.c_longlong,
+                                  C.c_longlong, c_i32p, C.c_float, C.c_float, c_f64p, C.c_float,
+                                  C.c_float, C.c_void_p]),
 }
 
+LH_SUMSQ_WORKSPACE = 1024
 _lib = None
 
 
@@ -218,3 +239,59 @@ def beam_gather(src, dst, H, B, backptr, B_src=None, stream=None):
     d = (C.c_void_p * n)(*[t.data_ptr() for t in dst])
     check(load().lh_beam_gather_f32(s, d, n, H, B, B_src, _ptr(backptr), _stream(stream)),
           "lh_beam_gather_f32")
+
+
+# ---- training half ------------------------------------------------------------------------------
+def softmax_xent_grad(logits, ldl, bias, V, B, tgt0, mask01, dz, ldz, logp_tgt, loss_accum,
+                      stream=None):
+    check(load().lh_softmax_xent_grad_f32(_ptr(logits), ldl, _ptr(bias), V, B, _ptr(tgt0),
+                                          _ptr(mask01), _ptr(dz), ldz, _ptr(logp_tgt),
+                                          _ptr(loss_accum), _stream(stream)),
+          "lh_softmax_xent_grad_f32")
+
+
+def lstm_cell_bwd(H, B, gates, c, c_prev, mask01, dgates, dc_prev, dh_above=None, dh_next=None,
+                  dc_next=None, clip_above=0.0, clip_next=0.0, stream=None):
+    check(load().lh_lstm_cell_bwd_f32(H, B, _ptr(dh_above), _ptr(dh_next), _ptr(dc_next),
+                                      _ptr(gates), _ptr(c), _ptr(c_prev), _ptr(mask01), clip_above,
+                                      clip_next, _ptr(dgates), _ptr(dc_prev), _stream(stream)),
+          "lh_lstm_cell_bwd_f32")
+
+
+def rowsum_acc(A, lda, rows, cols, out, beta=0.0, stream=None):
+    check(load().lh_rowsum_acc_f32(_ptr(A), lda, rows, cols, beta, _ptr(out), _stream(stream)),
+          "lh_rowsum_acc_f32")
+
+
+def embed_gather_grad(dx, ldx, E, n_unique, seg_start, seg_cols, small_grad, ldg, beta=0.0,
+                      stream=None):
+    check(load().lh_embed_gather_grad_f32(_ptr(dx), ldx, E, n_unique, _ptr(seg_start),
+                                          _ptr(seg_cols), beta, _ptr(small_grad), ldg,
+                                          _stream(stream)), "lh_embed_gather_grad_f32")
+
+
+def attn_delta(H, B, dht, h_tild, mask01, delta, dht_feed=None, clip_feed=0.0, stream=None):
+    check(load().lh_attn_delta_f32(H, B, _ptr(dht), _ptr(dht_feed), _ptr(h_tild), _ptr(mask01),
+                                   clip_feed, _ptr(delta), _stream(stream)), "lh_attn_delta_f32")
+
+
+def attn_core_bwd(H, B, D, max_len, hs_steps, dctx, tanh1, v_p, wa, hs, hs_step_stride,
+                  hs_col_stride, batch_info, p_t, sigma, indices, align, cached_exp, dhs, hsum, u,
+                  w, stream=None):
+    check(load().lh_attn_core_bwd_f32(H, B, D, max_len, hs_steps, _ptr(dctx), _ptr(tanh1),
+                                      _ptr(v_p), _ptr(wa), _ptr(hs), hs_step_stride, hs_col_stride,
+                                      _ptr(batch_info), _ptr(p_t), _ptr(sigma), _ptr(indices),
+                                      _ptr(align), _ptr(cached_exp), _ptr(dhs), _ptr(hsum), _ptr(u),
+                                      _ptr(w), _stream(stream)), "lh_attn_core_bwd_f32")
+
+
+def grad_sumsq(g, rows, cols, ld, scale, workspace, accum, stream=None):
+    check(load().lh_grad_sumsq_f32(_ptr(g), rows, cols, ld, scale, _ptr(workspace), _ptr(accum),
+                                   _stream(stream)), "lh_grad_sumsq_f32")
+
+
+def sgd_step(theta, ld_theta, g, ld_g, rows, cols, learning_rate, grad_scale, col_index=None,
+             sumsq=None, norm_clip=0.0, individual_clip=0.0, stream=None):
+    check(load().lh_sgd_step_f32(_ptr(theta), ld_theta, _ptr(g), ld_g, rows, cols,
+                                 _ptr(col_index), learning_rate, grad_scale, _ptr(sumsq),
+                                 norm_clip, individual_clip, _stream(stream)), "lh_sgd_step_f32")

@@ -112,6 +112,24 @@ double orc_forward_xent(orc_model *m, const int *src, int S, const int *tgt_in, 
                         int T, int B, const int *batch_info, int num_threads);
 
 /* ---- training: gradients and update (linmt_oracle_train.cpp) ------------------------------------ */
+/* Kernel-granularity functions with the argument meaning of lh_lstm_cell_bwd_f32,
+ * lh_softmax_xent_grad_f32, lh_attn_delta_f32 and lh_attn_core_bwd_f32. */
+void orc_lstm_cell_bwd(int H, int B, const float *dh_above, const float *dh_next,
+                       const float *dc_next, const float *gates, const float *c,
+                       const float *c_prev, const int *mask01, float clip_above, float clip_next,
+                       float *dgates, float *dc_prev);
+void orc_softmax_xent_grad(const float *logits, int ldl, const float *bias, int V, int B,
+                           const int *tgt0, const int *mask01, float *dz, int ldz,
+                           double *logp_tgt, double *loss_accum);
+void orc_attn_delta(int H, int B, const float *dht, const float *dht_feed, const float *h_tild,
+                    const int *mask01, float clip_feed, float *delta);
+void orc_attn_core_bwd(int H, int B, int D, int max_len, int hs_steps, const float *dctx,
+                       const float *tanh1, const float *v_p, const float *wa, const float *hs,
+                       long long hs_step_stride, long long hs_col_stride, const int *batch_info,
+                       const float *p_t, const float *sigma, const int *indices,
+                       const float *align, const float *cached_exp, float *dhs, float *hsum,
+                       float *u, float *w);
+
 typedef struct orc_trainer orc_trainer;
 orc_trainer *orc_trainer_create(orc_model *m, const orc_model_config *cfg);
 void orc_trainer_destroy(orc_trainer *t);

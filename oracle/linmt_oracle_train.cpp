@@ -128,30 +128,15 @@ void cell_backward(orc_trainer *t, const std::string &pfx, int B, const CellTape
                    const float *dh_above, Vec &dh_next, Vec &dc_next, Vec &dx, Vec *dh_tild_below) {
   const int H = t->cfg.H;
   const size_t n = (size_t)H * B;
-  Vec d[4];
-  for (auto &v : d) v.assign(n, 0.f);
-  Vec dc_prev(n, 0.f);
-  for (int b = 0; b < B; ++b)
-    for (int r = 0; r < H; ++r) {
-      const size_t o = idx2c(r, b, H);
-      const float it = tp.gates[idx2c(0 * (size_t)H + r, b, (size_t)4 * H)];
-      const float ft = tp.gates[idx2c(1 * (size_t)H + r, b, (size_t)4 * H)];
-      const float gt = tp.gates[idx2c(2 * (size_t)H + r, b, (size_t)4 * H)];
-      const float ot = tp.gates[idx2c(3 * (size_t)H + r, b, (size_t)4 * H)];
-      // d_errn_to_t_ht = d_errn_to_tp1_ht + d_errt_ht (geam), node_input_to_hidden.h:700
-      float dh = dh_next[o] + (dh_above ? dh_above[o] : 0.f);
-      // DErrtCTKernel, deep_rnn_kernel.h:152: dh * o * (1 - tanh(c)^2)
-      const float tc = tanhf(tp.c[o]);
-      float dc = dc_next[o] + dh * ot * (1.0f - tc * tc);
-      // ZeroColumnsKernel on both
-      dh = dh * tp.mask[b];
-      dc = dc * tp.mask[b];
-      d[3][o] = dh * tc * ot * (1 - ot);                 // DErrnToTOTKernel
-      d[1][o] = dc * tp.c_prev[o] * ft * (1 - ft);       // DErrnToTFTITKernel
-      d[2][o] = dc * it * (1 - gt * gt);                 // DErrnToTTanhcptKernel
-      d[0][o] = dc * gt * it * (1 - it);                 // DErrnToTFTITKernel
-      dc_prev[o] = dc * ft;                              // ElementwiseMultKernel
-    }
+  Vec dg((size_t)4 * n, 0.f), dc_prev(n, 0.f);
+  orc_lstm_cell_bwd(H, B, dh_above, dh_next.data(), dc_next.data(), tp.gates.data(), tp.c.data(),
+                    tp.c_prev.data(), tp.mask.data(), 0.f, 0.f, dg.data(), dc_prev.data());
+  Vec d[4];  // unstack: the reference keeps one H x B error per gate
+  for (int g = 0; g < 4; ++g) {
+    d[g].resize(n);
+    for (int b = 0; b < B; ++b)
+      memcpy(&d[g][(size_t)b * H], &dg[idx2c((size_t)g * H, b, (size_t)4 * H)], sizeof(float) * H);
+  }
   Vec dh_prev(n, 0.f);
   dx.assign(n, 0.f);
   for (int g = 0; g < 4; ++g) {
@@ -199,6 +184,131 @@ void scatter_embedding(orc_trainer *t, const std::string &name, int side, const 
 }
 
 }  // namespace
+
+// ---- kernel-granularity restatements (argument meaning of the lh_* entry points) ------------------
+
+// LstmInputHiddenNode::BackPropGpu up to the four gate errors (src/node_input_to_hidden.h:694-860):
+// geam sums, DErrtCTKernel (deep_rnn_kernel.h:152), ZeroColumnsKernel, DErrnToTOTKernel,
+// DErrnToTFTITKernel, DErrnToTTanhcptKernel, ElementwiseMultKernel; ClipMatKernel (:876,:951) on
+// the errors handed back is applied where they are consumed.
+extern "C" void orc_lstm_cell_bwd(int H, int B, const float *dh_above, const float *dh_next,
+                                  const float *dc_next, const float *gates, const float *c,
+                                  const float *c_prev, const int *mask01, float clip_above,
+                                  float clip_next, float *dgates, float *dc_prev) {
+  auto clamp = [](float x, float lim) {
+    return lim > 0.f ? (x > lim ? lim : (x < -lim ? -lim : x)) : x;
+  };
+  for (int b = 0; b < B; ++b)
+    for (int r = 0; r < H; ++r) {
+      const size_t o = idx2c(r, b, H);
+      const float it = gates[idx2c(0 * (size_t)H + r, b, (size_t)4 * H)];
+      const float ft = gates[idx2c(1 * (size_t)H + r, b, (size_t)4 * H)];
+      const float gt = gates[idx2c(2 * (size_t)H + r, b, (size_t)4 * H)];
+      const float ot = gates[idx2c(3 * (size_t)H + r, b, (size_t)4 * H)];
+      float dh = (dh_next ? clamp(dh_next[o], clip_next) : 0.f) +
+                 (dh_above ? clamp(dh_above[o], clip_above) : 0.f);
+      const float tc = tanhf(c[o]);
+      float dc = (dc_next ? dc_next[o] : 0.f) + dh * ot * (1.0f - tc * tc);
+      dh = dh * mask01[b];
+      dc = dc * mask01[b];
+      dgates[idx2c(3 * (size_t)H + r, b, (size_t)4 * H)] = dh * tc * ot * (1 - ot);
+      dgates[idx2c(1 * (size_t)H + r, b, (size_t)4 * H)] = dc * c_prev[o] * ft * (1 - ft);
+      dgates[idx2c(2 * (size_t)H + r, b, (size_t)4 * H)] = dc * it * (1 - gt * gt);
+      dgates[idx2c(0 * (size_t)H + r, b, (size_t)4 * H)] = dc * gt * it * (1 - it);
+      dc_prev[o] = dc * ft;
+    }
+}
+
+// Output error of SoftmaxLayer::GetHTGradientGpu / ComputeDGradientGpu (src/layer_loss.h:547-626,
+// 887-972) on top of the forward softmax: dz = mask * (onehot - p).
+extern "C" void orc_softmax_xent_grad(const float *logits, int ldl, const float *bias, int V, int B,
+                                      const int *tgt0, const int *mask01, float *dz, int ldz,
+                                      double *logp_tgt, double *loss_accum) {
+  Vec p((size_t)V * B);
+  orc_softmax_fwd(logits, ldl, bias, V, B, p.data(), V);
+  orc_train_loglik(p.data(), V, V, B, tgt0, mask01, loss_accum);
+  for (int b = 0; b < B; ++b) {
+    if (logp_tgt) logp_tgt[b] = log((double)p[idx2c(tgt0[b], b, V)]);
+    for (int v = 0; v < V; ++v) dz[idx2c(v, b, ldz)] = -p[idx2c(v, b, V)] * mask01[b];
+    dz[idx2c(tgt0[b], b, ldz)] += (float)mask01[b];
+  }
+}
+
+// AddTwoMatsKernel + ZeroHT + TanhGradKernel, src/layer_attention.h:490-512.
+extern "C" void orc_attn_delta(int H, int B, const float *dht, const float *dht_feed,
+                               const float *h_tild, const int *mask01, float clip_feed,
+                               float *delta) {
+  for (int b = 0; b < B; ++b)
+    for (int r = 0; r < H; ++r) {
+      const size_t o = idx2c(r, b, H);
+      float v = dht[o];
+      if (dht_feed) {
+        float f = dht_feed[o];
+        if (clip_feed > 0.f) f = f > clip_feed ? clip_feed : (f < -clip_feed ? -clip_feed : f);
+        v += f;
+      }
+      v = v * mask01[b];
+      delta[o] = v * (1 - h_tild[o] * h_tild[o]);
+    }
+}
+
+// src/layer_attention.h:572-660 with ErrorAlignmentsKernelLarge, ErrorHSAndCTKernelLarge,
+// ErrorPTKernel, AttentionVPErrorKernel, GradWPKernel, GetHTScalingsWaGradKernel, ScaleHTKernel,
+// AddTwoMatsKernel and CopyErrorsSource (src/deep_rnn_kernel.h:1348-1520).
+extern "C" void orc_attn_core_bwd(int H, int B, int D, int max_len, int hs_steps, const float *dctx,
+                                  const float *tanh1, const float *v_p, const float *wa,
+                                  const float *hs, long long hs_step_stride,
+                                  long long hs_col_stride, const int *batch_info, const float *p_t,
+                                  const float *sigma, const int *indices, const float *align,
+                                  const float *cached_exp, float *dhs, float *hsum, float *u,
+                                  float *w) {
+  const int W = D >= 0 ? 2 * D + 1 : max_len;
+  const float sigma_sq = (float)((D * D) / 4.0);
+  for (int b = 0; b < B; ++b) {
+    const int len = batch_info[b], off = batch_info[B + b];
+    std::vector<float> das(W, 0.f), r(W, 0.f);
+    std::vector<long long> at(W, -1);
+    for (int j = 0; j < W; ++j) {
+      const int idx = indices[idx2c(b, j, B)];
+      if (idx == -1) continue;
+      const int tau = len - 1 - idx + off;
+      if (tau < 0 || tau >= hs_steps) continue;
+      at[j] = (long long)tau * hs_step_stride + (long long)b * hs_col_stride;
+      float acc = 0.f;  // ErrorAlignmentsKernelLarge
+      for (int k = 0; k < H; ++k) acc += dctx[idx2c(k, b, H)] * hs[at[j] + k];
+      das[j] = acc;
+    }
+    for (int j = 0; j < W; ++j)  // ErrorHSAndCTKernelLarge
+      if (at[j] >= 0)
+        for (int k = 0; k < H; ++k) dhs[at[j] + k] += dctx[idx2c(k, b, H)] * align[idx2c(b, j, B)];
+    if (D >= 0) {
+      float dp = 0.f;  // ErrorPTKernel (all slots; invalid ones carry alignment 0)
+      for (int j = 0; j < W; ++j)
+        dp += das[j] * align[idx2c(b, j, B)] * ((indices[idx2c(b, j, B)] - p_t[b]) / sigma_sq);
+      const float sg = sigma[b];
+      for (int k = 0; k < H; ++k) {
+        const size_t o = idx2c(k, b, H);
+        u[o] = dp * sg * (1 - sg) * len * tanh1[o];                               // AttentionVPErrorKernel
+        w[o] = dp * len * v_p[k] * sg * (1 - sg) * (1 - tanh1[o] * tanh1[o]);     // GradWPKernel
+      }
+    }
+    for (int j = 0; j < W; ++j) {  // GetHTScalingsWaGradKernel
+      const float aj = align[idx2c(b, j, B)], gj = cached_exp[idx2c(j, b, W)];
+      float v = das[j] * aj * (1 - aj / gj);
+      for (int k = 0; k < W; ++k)
+        if (k != j) v += -1 * das[k] * align[idx2c(b, k, B)] * aj / gj;
+      r[j] = v;
+    }
+    for (int k = 0; k < H; ++k) hsum[idx2c(k, b, H)] = 0.f;
+    for (int j = 0; j < W; ++j) {
+      if (at[j] < 0) continue;  // hs_mat holds zeros there; CopyErrorsSource skips index -1
+      for (int k = 0; k < H; ++k) {
+        hsum[idx2c(k, b, H)] += hs[at[j] + k] * r[j];   // ScaleHTKernel + AddTwoMatsKernel
+        dhs[at[j] + k] += wa[idx2c(k, b, H)] * r[j];    // ScaleHTKernel + CopyErrorsSource
+      }
+    }
+  }
+}
 
 extern "C" orc_trainer *orc_trainer_create(orc_model *m, const orc_model_config *cfg) {
   orc_trainer *t = new orc_trainer();
@@ -307,24 +417,19 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
       top = a.h_tild.data();
     }
     // softmax: p, log-likelihood, and the output error (onehot - p) * mask of GetHTGradientGpu
-    Vec logits((size_t)V * B), p((size_t)V * B);
+    Vec logits((size_t)V * B);
     orc_gemm(V, B, H, P(t, "softmax.D"), V, 0, top, H, 0, 1.f, 0.f, logits.data(), V);
-    orc_softmax_fwd(logits.data(), V, P(t, "softmax.b_d"), V, B, p.data(), V);
     std::vector<int> t0(B);
     tgt_mask[s].resize(B);
     orc_preprocess_indices(tgt_out + (size_t)s * B, B, t0.data(), tgt_mask[s].data(), nullptr);
-    orc_train_loglik(p.data(), V, V, B, t0.data(), tgt_mask[s].data(), &loglik);
     dz[s].assign((size_t)V * B, 0.f);
-    for (int b = 0; b < B; ++b) {
-      if (!tgt_mask[s][b]) continue;
-      for (int v = 0; v < V; ++v) dz[s][idx2c(v, b, V)] = -p[idx2c(v, b, V)];
-      dz[s][idx2c(t0[b], b, V)] += 1.f;
-    }
+    orc_softmax_xent_grad(logits.data(), V, P(t, "softmax.b_d"), V, B, t0.data(),
+                          tgt_mask[s].data(), dz[s].data(), V, nullptr, &loglik);
   }
 
   // ------------------------------------------------------------------------------ backward, target
   std::vector<Vec> dh_next(L, Vec(n, 0.f)), dc_next(L, Vec(n, 0.f));
-  std::vector<Vec> dHS(S, Vec(n, 0.f));  // error into the top source layer, per source step
+  Vec dHS((size_t)S * n, 0.f);  // error into the top source layer, laid out like hs
   Vec dh_tild_feed;                      // Q^T d from the input layer of step t+1
   bool have_feed = false;
   Vec &gD = G(t, "softmax.D", (size_t)V * H);
@@ -340,69 +445,20 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
       const AttnTape &a = att[s];
       const CellTape &topc = dec[s][L - 1];
       const float *ha = topc.h.data();
-      Vec delta = dht;
-      if (feed_cfg && have_feed)
-        for (size_t i = 0; i < n; ++i) delta[i] += dh_tild_feed[i];
-      for (int b = 0; b < B; ++b)
-        for (int r = 0; r < H; ++r) {
-          const size_t o = idx2c(r, b, H);
-          delta[o] = delta[o] * topc.mask[b];                          // ZeroHT
-          delta[o] = delta[o] * (1 - a.h_tild[o] * a.h_tild[o]);       // TanhGradKernel
-        }
+      Vec delta(n, 0.f);
+      orc_attn_delta(H, B, dht.data(), (feed_cfg && have_feed) ? dh_tild_feed.data() : nullptr,
+                     a.h_tild.data(), topc.mask.data(), 0.f, delta.data());
       outer_acc(t, "attn.W_c1", delta.data(), a.ctx.data(), B);
       outer_acc(t, "attn.W_c2", delta.data(), ha, B);
       rowsum_acc(t, "attn.b_out", delta.data(), H, B);
       Vec dctx(n, 0.f), dha(n, 0.f);
       apply(t, "attn.W_c1", 1, delta.data(), B, 0.f, dctx.data());
       apply(t, "attn.W_c2", 1, delta.data(), B, 0.f, dha.data());
-      const float sigma_sq = (float)((D * D) / 4.0);
       Vec hsum(n, 0.f), u(n, 0.f), w(n, 0.f);
-      for (int b = 0; b < B; ++b) {
-        const int len = batch_info[b], off = batch_info[B + b];
-        std::vector<float> das(W, 0.f), r(W, 0.f);
-        std::vector<const float *> hsp(W, nullptr);
-        std::vector<int> tau(W, -1);
-        for (int j = 0; j < W; ++j) {
-          const int idx = a.indices[idx2c(b, j, B)];
-          if (idx == -1) continue;
-          tau[j] = len - 1 - idx + off;
-          hsp[j] = &hs[(size_t)tau[j] * n + (size_t)b * H];
-          float acc = 0.f;  // ErrorAlignmentsKernelLarge
-          for (int k = 0; k < H; ++k) acc += dctx[idx2c(k, b, H)] * hsp[j][k];
-          das[j] = acc;
-        }
-        // ErrorHSAndCTKernelLarge
-        for (int j = 0; j < W; ++j)
-          if (tau[j] >= 0)
-            for (int k = 0; k < H; ++k)
-              dHS[tau[j]][idx2c(k, b, H)] += dctx[idx2c(k, b, H)] * a.align[idx2c(b, j, B)];
-        if (D >= 0) {
-          float dp = 0.f;  // ErrorPTKernel (all slots; invalid ones carry alignment 0)
-          for (int j = 0; j < W; ++j)
-            dp += das[j] * a.align[idx2c(b, j, B)] *
-                  ((a.indices[idx2c(b, j, B)] - a.p_t[b]) / sigma_sq);
-          const float sg = a.sigma[b];
-          for (int k = 0; k < H; ++k) {
-            const size_t o = idx2c(k, b, H);
-            u[o] = dp * sg * (1 - sg) * len * a.tanh1[o];                               // AttentionVPErrorKernel
-            w[o] = dp * len * P(t, "attn.v_p")[k] * sg * (1 - sg) * (1 - a.tanh1[o] * a.tanh1[o]);  // GradWPKernel
-          }
-        }
-        for (int j = 0; j < W; ++j) {  // GetHTScalingsWaGradKernel
-          const float aj = a.align[idx2c(b, j, B)], gj = a.cached_exp[idx2c(j, b, W)];
-          float v = das[j] * aj * (1 - aj / gj);
-          for (int k = 0; k < W; ++k)
-            if (k != j) v += -1 * das[k] * a.align[idx2c(b, k, B)] * aj / gj;
-          r[j] = v;
-        }
-        for (int j = 0; j < W; ++j) {
-          if (tau[j] < 0) continue;  // hs_mat holds zeros there; CopyErrorsSource skips index -1
-          for (int k = 0; k < H; ++k) {
-            hsum[idx2c(k, b, H)] += hsp[j][k] * r[j];                       // ScaleHTKernel + AddTwoMats
-            dHS[tau[j]][idx2c(k, b, H)] += a.wa[idx2c(k, b, H)] * r[j];     // ScaleHTKernel + CopyErrorsSource
-          }
-        }
-      }
+      orc_attn_core_bwd(H, B, D, S, S, dctx.data(), a.tanh1.data(), D >= 0 ? P(t, "attn.v_p") : nullptr,
+                        a.wa.data(), hs.data(), (long long)n, H, batch_info, a.p_t.data(),
+                        a.sigma.data(), a.indices.data(), a.align.data(), a.cached_exp.data(),
+                        dHS.data(), hsum.data(), u.data(), w.data());
       if (D >= 0) {
         rowsum_acc(t, "attn.v_p", u.data(), H, B);
         outer_acc(t, "attn.W_p", w.data(), ha, B);
@@ -431,7 +487,7 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
   }
   // ------------------------------------------------------------------------------ backward, source
   for (int s = S - 1; s >= 0; --s) {
-    Vec dx, dh_above = attn ? dHS[s] : zeros;
+    Vec dx, dh_above = attn ? Vec(dHS.begin() + (size_t)s * n, dHS.begin() + (size_t)(s + 1) * n) : zeros;
     for (int l = L - 1; l >= 0; --l) {
       cell_backward(t, "src." + std::to_string(l) + ".", B, enc[s][l], dh_above.data(), dh_next[l],
                     dc_next[l], dx, nullptr);

@@ -208,6 +208,59 @@ def beam_gather(src, backptr):
     return dst
 
 
+# ---- training kernels (argument meaning of the lh_* entry points of the same name) -----------------
+def _fa(a):
+    return None if a is None else np.asfortranarray(a, np.float32)
+
+
+def lstm_cell_bwd(gates, c, c_prev, mask01, dh_above=None, dh_next=None, dc_next=None,
+                  clip_above=0.0, clip_next=0.0):
+    """gates (4H,B), c / c_prev (H,B).  Returns dgates (4H,B), dc_prev (H,B)."""
+    H4, B = gates.shape
+    H = H4 // 4
+    dg = np.empty((H4, B), np.float32, order="F")
+    dcp = np.empty((H, B), np.float32, order="F")
+    lib().orc_lstm_cell_bwd(H, B, _p(_fa(dh_above)), _p(_fa(dh_next)), _p(_fa(dc_next)),
+                            _p(_fa(gates)), _p(_fa(c)), _p(_fa(c_prev)), _p(i32(mask01)),
+                            _f(clip_above), _f(clip_next), _p(dg), _p(dcp))
+    return dg, dcp
+
+
+def softmax_xent_grad(logits, bias, tgt0, mask01):
+    """Returns dz (V,B), logp_tgt (B,) float64, masked sum of logp_tgt."""
+    logits = _fa(logits)
+    V, B = logits.shape
+    dz = np.empty((V, B), np.float32, order="F")
+    lp = np.zeros(B, np.float64)
+    acc = np.zeros(1, np.float64)
+    lib().orc_softmax_xent_grad(_p(logits), V, _p(None if bias is None else f32(bias)), V, B,
+                                _p(i32(tgt0)), _p(i32(mask01)), _p(dz), V, _p(lp), _p(acc))
+    return dz, lp, float(acc[0])
+
+
+def attn_delta(dht, h_tild, mask01, dht_feed=None, clip_feed=0.0):
+    H, B = dht.shape
+    out = np.empty((H, B), np.float32, order="F")
+    lib().orc_attn_delta(H, B, _p(_fa(dht)), _p(_fa(dht_feed)), _p(_fa(h_tild)), _p(i32(mask01)),
+                         _f(clip_feed), _p(out))
+    return out
+
+
+def attn_core_bwd(H, B, D, max_len, hs_steps, dctx, tanh1, v_p, wa, hs, step_stride, col_stride,
+                  batch_info, fwd, dhs0):
+    """fwd: the dict attn_core_fwd returned.  dhs0: flat float32 array laid out like hs; a copy
+    with the step's contribution added comes back as out['dhs']."""
+    out = dict(dhs=f32(dhs0).copy(), hsum=np.empty((H, B), np.float32, order="F"),
+               u=np.zeros((H, B), np.float32, order="F"), w=np.zeros((H, B), np.float32, order="F"))
+    lib().orc_attn_core_bwd(H, B, D, max_len, hs_steps, _p(_fa(dctx)), _p(_fa(tanh1)),
+                            _p(None if v_p is None else f32(v_p)), _p(_fa(wa)), _p(f32(hs)),
+                            C.c_longlong(step_stride), C.c_longlong(col_stride),
+                            _p(i32(batch_info)), _p(fwd["p_t"]), _p(fwd["sigma"]),
+                            _p(fwd["indices"]), _p(fwd["align"]), _p(fwd["cached_exp"]),
+                            _p(out["dhs"]), _p(out["hsum"]), _p(out["u"]), _p(out["w"]))
+    return out
+
+
 class Model:
     """Host model of the oracle; parameters are numpy views into the oracle's own buffers."""
 
