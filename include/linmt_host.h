@@ -38,6 +38,16 @@ typedef struct lnmt_decode_options {
   float max_decoding_ratio, min_decoding_ratio, penalty, diversity, lp_alpha, cp_beta;
 } lnmt_decode_options;
 
+/* Training options (src/global_configuration.h:107-123, src/utility_cu.cu:82-96). */
+typedef struct lnmt_train_options {
+  float learning_rate;
+  int grad_clip_mode;          /* 0 none, 1 per-matrix norm (reference default), 2 global norm
+                                  (--whole-clip-gradients), 3 element clamp (--ind-clip-gradients) */
+  float norm_clip;             /* threshold of modes 1 and 2 */
+  float individual_clip;       /* threshold of mode 3 */
+  float error_clip_threshold;  /* clamp of the errors handed back in time when clip_cell is set */
+} lnmt_train_options;
+
 typedef struct lnmt_model lnmt_model;
 
 const char *lnmt_last_error(void);
@@ -46,6 +56,8 @@ const char *lnmt_last_error(void);
 lnmt_model *lnmt_model_create_scoring(const lnmt_config *cfg);
 /* NeuralMachineTranslation + InitModelDecoding for up to n_sent sentences x beam hypotheses. */
 lnmt_model *lnmt_model_create_decoding(const lnmt_config *cfg, int n_sent, int beam_size);
+/* NeuralMachineTranslation + InitModel with stored activations and gradient buffers. */
+lnmt_model *lnmt_model_create_training(const lnmt_config *cfg, const lnmt_train_options *t);
 void lnmt_model_destroy(lnmt_model *m);
 
 /* Parameters by reference name ("src.0.W", "src.1.M_i", "tgt.0.Q_c", "tgt.2.b_f", "attn.W_a",
@@ -57,6 +69,23 @@ int lnmt_model_get_param(lnmt_model *m, const char *name, float *data, long long
 int lnmt_get_error(lnmt_model *m, const int *source, int source_length, const int *target_in,
                    const int *target_out, int target_length, const int *batch_information,
                    int minibatch_size, double *loss);
+
+/* NeuralMachineTranslation::ComputeGradients up to (not including) its UpdateWeights call: forward
+ * with stored activations and the backward pass of one minibatch of exactly cfg.minibatch_size
+ * columns.  source_wgrad / target_wgrad: the unique non-pad input ids of the minibatch
+ * (FileHelper's *_wgrad lists).  *loss receives the summed log p(target).  Gradients are of the
+ * log-likelihood and unscaled; they accumulate until lnmt_update_weights or lnmt_clear_gradients. */
+int lnmt_compute_gradients(lnmt_model *m, const int *source, int source_length,
+                           const int *target_in, const int *target_out, int target_length,
+                           const int *source_wgrad, int len_source_wgrad, const int *target_wgrad,
+                           int len_target_wgrad, const int *batch_information, int minibatch_size,
+                           double *loss);
+/* Gradient by parameter name; "src.0.W" / "tgt.0.W" are E x len_wgrad (column k = id wgrad[k]). */
+int lnmt_model_get_grad(lnmt_model *m, const char *name, float *data, long long n);
+/* NeuralMachineTranslation::UpdateWeights + ClearGradients.  *global_norm (may be NULL) receives
+ * the norm the global clip used (0 in the other modes). */
+int lnmt_update_weights(lnmt_model *m, double *global_norm);
+int lnmt_clear_gradients(lnmt_model *m);
 
 /* Copies a state of the last lnmt_get_error call: kind 0 = h, 1 = c of (side 0 src / 1 tgt, layer,
  * timestep); kind 2 = attention output h~ of target timestep; kind 3 = alignments (B x W) of target

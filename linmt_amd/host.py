@@ -26,6 +26,11 @@ class Config(C.Structure):
                 ("cell_clip_threshold", C.c_float)]
 
 
+class TrainOptions(C.Structure):
+    _fields_ = [("learning_rate", C.c_float), ("grad_clip_mode", C.c_int), ("norm_clip", C.c_float),
+                ("individual_clip", C.c_float), ("error_clip_threshold", C.c_float)]
+
+
 class DecodeOptions(C.Structure):
     _fields_ = [("beam_size", C.c_int), ("max_decoding_ratio", C.c_float),
                 ("min_decoding_ratio", C.c_float), ("penalty", C.c_float),
@@ -45,6 +50,14 @@ def load():
     lib.lnmt_model_create_scoring.argtypes = [C.POINTER(Config)]
     lib.lnmt_model_create_decoding.restype = C.c_void_p
     lib.lnmt_model_create_decoding.argtypes = [C.POINTER(Config), C.c_int, C.c_int]
+    lib.lnmt_model_create_training.restype = C.c_void_p
+    lib.lnmt_model_create_training.argtypes = [C.POINTER(Config), C.POINTER(TrainOptions)]
+    lib.lnmt_compute_gradients.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+                                           C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                                           C.c_void_p, C.c_int, C.POINTER(C.c_double)]
+    lib.lnmt_model_get_grad.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
+    lib.lnmt_update_weights.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
+    lib.lnmt_clear_gradients.argtypes = [C.c_void_p]
     lib.lnmt_model_destroy.argtypes = [C.c_void_p]
     lib.lnmt_model_destroy.restype = None
     lib.lnmt_model_set_param.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
@@ -81,8 +94,10 @@ class Model:
     def __init__(self, num_layers, lstm_size, source_vocab_size, target_vocab_size,
                  longest_sentence=104, attention_mode=1, attention_width=10, feed_input=True,
                  minibatch_size=1, embedding_size=0, sequence_to_sequence=True, decoding=None,
-                 clip_cell=False, cell_clip_threshold=50.0):
-        """decoding=(n_sent, beam) builds the batched decoder, otherwise the scoring model."""
+                 clip_cell=False, cell_clip_threshold=50.0, training=None):
+        """decoding=(n_sent, beam) builds the batched decoder; training=dict(learning_rate,
+        grad_clip_mode, norm_clip, individual_clip, error_clip_threshold) the training model;
+        otherwise the scoring model."""
         self.cfg = Config(num_layers, lstm_size, embedding_size, source_vocab_size,
                           target_vocab_size, minibatch_size, longest_sentence, attention_mode,
                           attention_width, int(feed_input), int(sequence_to_sequence),
@@ -91,6 +106,11 @@ class Model:
         if decoding is not None:
             self.n_sent, self.beam = decoding
             h = lib.lnmt_model_create_decoding(C.byref(self.cfg), self.n_sent, self.beam)
+        elif training is not None:
+            t = TrainOptions(training.get("learning_rate", 0.7), training.get("grad_clip_mode", 1),
+                             training.get("norm_clip", 5.0), training.get("individual_clip", 0.1),
+                             training.get("error_clip_threshold", 1000.0))
+            h = lib.lnmt_model_create_training(C.byref(self.cfg), C.byref(t))
         else:
             h = lib.lnmt_model_create_scoring(C.byref(self.cfg))
         if not h:
@@ -154,6 +174,37 @@ class Model:
         _check(load().lnmt_get_error(self.handle, _p(src), S, _p(tgt_in), _p(tgt_out), T, _p(bi), B,
                                      C.byref(loss)), "get_error")
         return loss.value
+
+    def compute_gradients(self, src, tgt_in, tgt_out, batch_info, src_unique, tgt_unique):
+        """Forward + backward of one minibatch (no update); returns sum log p(target)."""
+        src = np.asfortranarray(src, np.int32) if src is not None else None
+        tgt_in = np.asfortranarray(tgt_in, np.int32)
+        tgt_out = np.asfortranarray(tgt_out, np.int32)
+        B, T = tgt_in.shape
+        S = src.shape[1] if src is not None else 0
+        bi = None if batch_info is None else np.ascontiguousarray(batch_info, np.int32)
+        su = None if src_unique is None else np.ascontiguousarray(src_unique, np.int32)
+        tu = np.ascontiguousarray(tgt_unique, np.int32)
+        loss = C.c_double(0)
+        _check(load().lnmt_compute_gradients(self.handle, _p(src), S, _p(tgt_in), _p(tgt_out), T,
+                                             _p(su), 0 if su is None else su.size, _p(tu), tu.size,
+                                             _p(bi), B, C.byref(loss)), "compute_gradients")
+        return loss.value
+
+    def get_grad(self, name, shape):
+        out = np.empty(int(np.prod(shape)), np.float32)
+        _check(load().lnmt_model_get_grad(self.handle, name.encode(), _p(out), out.size),
+               f"get_grad({name})")
+        return out.reshape(shape, order="F")
+
+    def update_weights(self):
+        """UpdateWeights + ClearGradients; returns the global norm (0 unless grad_clip_mode 2)."""
+        nrm = C.c_double(0)
+        _check(load().lnmt_update_weights(self.handle, C.byref(nrm)), "update_weights")
+        return nrm.value
+
+    def clear_gradients(self):
+        _check(load().lnmt_clear_gradients(self.handle), "clear_gradients")
 
     def get_state(self, kind, side, layer, timestep, rows, cols):
         out = np.empty(rows * cols, np.float32)

@@ -74,7 +74,66 @@ extern "C" lnmt_model *lnmt_model_create_decoding(const lnmt_config *cfg, int n_
   return m;
 }
 
+extern "C" lnmt_model *lnmt_model_create_training(const lnmt_config *cfg,
+                                                  const lnmt_train_options *t) {
+  lnmt_model *m = nullptr;
+  if (Guard([&] {
+        GlobalConfiguration g = ToConfig(cfg);
+        g.train_mode_ = true;
+        g.learning_rate_ = t->learning_rate;
+        g.grad_clip_mode_ = t->grad_clip_mode;
+        g.norm_clip_ = t->norm_clip;
+        g.individual_norm_clip_threshold_ = t->individual_clip;
+        g.error_clip_threshold_ = t->error_clip_threshold;
+        if (g.grad_clip_mode_ < 0 || g.grad_clip_mode_ > 3) throw LinmtError("grad_clip_mode outside [0,3]");
+        if ((g.grad_clip_mode_ == 1 || g.grad_clip_mode_ == 2) && !(g.norm_clip_ > 0.f))
+          throw LinmtError("norm_clip must be positive");
+        std::unique_ptr<lnmt_model> p(new lnmt_model());
+        p->nmt.reset(new NeuralMachineTranslation(g));
+        p->nmt->InitModel();
+        m = p.release();
+      }) != 0)
+    return nullptr;
+  return m;
+}
+
 extern "C" void lnmt_model_destroy(lnmt_model *m) { delete m; }
+
+extern "C" int lnmt_compute_gradients(lnmt_model *m, const int *source, int source_length,
+                                      const int *target_in, const int *target_out,
+                                      int target_length, const int *source_wgrad,
+                                      int len_source_wgrad, const int *target_wgrad,
+                                      int len_target_wgrad, const int *batch_information,
+                                      int minibatch_size, double *loss) {
+  return Guard([&] {
+    *loss = m->nmt->ComputeGradients(source, source_length, target_in, target_out, target_length,
+                                     source_wgrad, len_source_wgrad, target_wgrad,
+                                     len_target_wgrad, batch_information, minibatch_size);
+  });
+}
+
+extern "C" int lnmt_model_get_grad(lnmt_model *m, const char *name, float *data, long long n) {
+  return Guard([&] {
+    std::vector<float> v;
+    if (!m->nmt->GetGrad(name, &v) || (long long)v.size() != n)
+      throw LinmtError(std::string("unknown gradient or wrong size: ") + name);
+    memcpy(data, v.data(), sizeof(float) * v.size());
+  });
+}
+
+extern "C" int lnmt_update_weights(lnmt_model *m, double *global_norm) {
+  return Guard([&] {
+    m->nmt->UpdateWeights();
+    if (global_norm) *global_norm = m->nmt->last_global_norm_;
+  });
+}
+
+extern "C" int lnmt_clear_gradients(lnmt_model *m) {
+  return Guard([&] {
+    m->nmt->ClearGradients();
+    m->nmt->Synchronize();
+  });
+}
 
 extern "C" int lnmt_model_set_param(lnmt_model *m, const char *name, const float *data,
                                     long long n) {

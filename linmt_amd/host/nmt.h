@@ -39,6 +39,16 @@ struct GlobalConfiguration {
   bool sequence_to_sequence_mode_ = true;  // false: target-side language model (--nlm)
   bool clip_cell_mode_ = false;
   float cell_clip_threshold_ = 50.f;
+  float error_clip_threshold_ = 1000.f;  // utility_cu.cu:91, active with clip_cell_mode_
+  // training (global_configuration.h:107-123)
+  bool train_mode_ = false;               // keep the activations and allocate gradients
+  float learning_rate_ = 0.7f;
+  // The reference's three mutually exclusive flags (global_configuration.cc:780-797):
+  // 1 = clip_gradient_mode_ (per-matrix norm clip, the default), 2 = global_grad_clip_mode__
+  // (--whole-clip-gradients), 3 = individual_grad_clip_mode__ (--ind-clip-gradients), 0 = none.
+  int grad_clip_mode_ = 1;
+  float norm_clip_ = 5.f;
+  float individual_norm_clip_threshold_ = 0.1f;
 };
 
 class NeuralMachineTranslation;
@@ -73,6 +83,17 @@ class LstmNode {
   float *p_device_gates_ = nullptr;          // 4H x B: i_t, f_t, c_prime_t_tanh, o_t (NULL when not kept)
   float *p_device_c_t_ = nullptr;
   float *p_device_h_t_ = nullptr;
+  float *p_device_d_gates_ = nullptr;  // training: 4H x B gate errors of this step
+  float *p_device_d_x_ = nullptr;      // training: error w.r.t. this step's input (M^T d)
+
+  // BackPropGpu (node_input_to_hidden.h:647-983, node_hidden_to_hidden.h:537-900): fused cell
+  // backward and W_h^T d; upper layers and the feed-input branch also produce M^T d / Q^T d here.
+  // dh_above: error from the layer above (above_is_lstm) or from the attention node / softmax
+  // (NULL = none); dh_next / dc_next: errors from step t+1 (NULL = none).  The errors for step t-1
+  // land in the layer's p_device_d_errn_to_t_ht_m1_ / _ct_m1_.  batched_dx: M^T d is left to one
+  // GEMM over all steps (BackPropInputAllSteps).
+  void BackPropGpu(const float *dh_above, bool above_is_lstm, const float *dh_next,
+                   const float *dc_next, bool batched_dx);
 
   // InputToHidden: UpdateVectorsForwardGpu(idx0, mask01, h_prev, c_prev) (node_input_to_hidden.h:100);
   // HiddenToHidden: UpdateVectorsForwardGpu(mask01, h_prev, c_prev) (node_hidden_to_hidden.h:94).
@@ -121,6 +142,31 @@ class LstmLayer {
             int minibatch_size, int num_nodes, bool keep_gates, bool with_previous_state);
   // InitFeedInput (layer_input_to_hidden.h:299): allocates Q and switches the nodes to feed input.
   void InitFeedInput();
+
+  // ---- training --------------------------------------------------------------------------------
+  DeviceArray<float> p_device_m_grad_, p_device_w_h_grad_, p_device_q_grad_, p_device_b_grad_;
+  DeviceArray<float> p_device_small_w_grad_;  // E x (number of unique ids), layer 1
+  DeviceArray<float> d_gates_all_, d_x_all_;  // per-step gate errors / input errors
+  DeviceArray<float> p_device_d_errn_to_t_ht_m1_, p_device_d_errn_to_t_ct_m1_;  // recurrent errors
+  DeviceArray<float> p_device_errn_to_t_h_tild_;  // Q^T d: error into the attention node of t-1
+  DeviceArray<int> p_device_input_vocab_indices_wgrad_, p_device_wgrad_seg_start_,
+      p_device_wgrad_seg_cols_;
+  int w_grad_length_ = 0;  // unique ids of the current minibatch
+  void InitTraining();
+  // Unique-id list of the minibatch (the reference's *_wgrad arrays, file_helper.cc:281-380) plus,
+  // per unique id, the (timestep, column) positions that carry it.
+  void PreprocessWGrad(const int *p_host_indices, int current_length, int minibatch_size,
+                       const int *p_host_wgrad, int len_wgrad);
+  // ComputeGradientsGpu over all steps at once (node_input_to_hidden.h:997-1300): weight / bias
+  // gradients as GEMMs with K = minibatch x steps, and the embedding gradient.
+  // h_prev0 / c-less: state fed to step 0 (NULL = zeros).
+  void ComputeGradientsAllSteps(int steps, const float *p_device_h_prev0,
+                                const float *p_device_h_tild_all);
+  // d_x_all_ = M^T d for every step in one GEMM.
+  void BackPropInputAllSteps(int steps);
+  void ClearGradients();
+  bool GetGrad(const std::string &name, std::vector<float> *out);
+
   // PreprocessGpuVocabIndices (layer_input_to_hidden.h:1478-1513, layer_hidden_to_hidden.h:541-560):
   // host ids (B x T column-major, -1 padding) -> device idx0 / mask01 for all T steps.
   void PreprocessGpuVocabIndices(const int *p_host_input_vocab_indices, int current_length,
@@ -143,7 +189,12 @@ class AttentionNode {
   float *p_device_h_t_wa_cache_ = nullptr, *p_device_alignments_ = nullptr;
   float *p_device_cached_exp_ = nullptr, *p_device_c_t_ = nullptr, *p_device_final_tmp_2_ = nullptr;
   int *p_device_indices_ = nullptr;
+  float *p_device_d_errt_ht_tild_ = nullptr;  // training: delta of this step (H x B)
+  float *p_device_h_s_sum_ = nullptr, *p_device_u_ = nullptr, *p_device_w_ = nullptr;
   void ForwardProp();  // layer_attention.h:243-483
+  // layer_attention.h:487-698.  dht: error from the softmax; dht_feed: Q^T d of step t+1 (or NULL).
+  // Leaves the error for the top decoder layer in the layer's p_device_errn_to_t_ht_p1_.
+  void BackProp(const float *dht, const float *dht_feed);
 };
 
 class AttentionLayer {
@@ -162,6 +213,17 @@ class AttentionLayer {
   int hs_steps_ = 0;       // timesteps currently held
   bool use_hs_col_ = false;  // decode: beam columns share their sentence's states
   std::vector<AttentionNode> v_nodes_;
+
+  // ---- training --------------------------------------------------------------------------------
+  DeviceArray<float> p_device_w_a_grad_, p_device_w_p_grad_, p_device_v_p_grad_,
+      p_device_output_bias_grad_, p_device_w_c_p1_grad_, p_device_w_c_p2_grad_;
+  DeviceArray<float> delta_all_, h_s_sum_all_, u_all_, w_all_;
+  DeviceArray<float> p_device_errn_to_t_ct_, p_device_errn_to_t_ht_p1_;
+  DeviceArray<float> p_device_total_hs_error_;  // layout of the encoder's top-layer states
+  void InitTraining();
+  void ComputeGradientsAllSteps(int steps, const float *p_device_h_t_all);
+  void ClearGradients();
+  bool GetGrad(const std::string &name, std::vector<float> *out);
 
   void Init(NeuralMachineTranslation *model, int minibatch_size, int num_nodes, int longest_sent);
   // PreprocessMinibatchInformation (layer_attention.h:977): [len_0.., offset_0..] for B columns.
@@ -215,6 +277,18 @@ class SoftmaxLayer : public BaseLossLayer {
                                  int current_target_length, int minibatch_size) override;
   // logits only (D*h + b_d), used by the on-device beam step
   void ComputeLogits(float *p_device_h_t, int minibatch);
+
+  // ---- training --------------------------------------------------------------------------------
+  DeviceArray<float> p_device_d_grad_, p_device_b_d_grad_;
+  DeviceArray<float> p_device_d_errt_ht_all_;  // D^T dz for every step (H x B x steps)
+  DeviceArray<float> dz_chunk_;                // V x (B x chunk steps) logits, then output errors
+  int chunk_steps_ = 0;
+  void InitTraining();
+  // ForwardProp + BackProp1 + BackProp2 of every step (layer_loss.h:480-516, 547-626, 887-972) as
+  // chunked GEMMs over B x steps columns; accumulates the log-likelihood into p_device_loss_.
+  void ForwardBackwardAllSteps(const float *p_device_h_t_all, int steps);
+  void ClearGradients();
+  bool GetGrad(const std::string &name, std::vector<float> *out);
   bool SetParam(const std::string &name, const float *host, size_t n);
   bool GetParam(const std::string &name, std::vector<float> *out);
 };
@@ -298,9 +372,33 @@ class NeuralMachineTranslation {
   void DecodeBatch(const std::vector<std::vector<int>> &sentences, const DecodeOptions &o,
                    std::vector<SentenceResult> *results);
 
+  // ---- training --------------------------------------------------------------------------------
+  DeviceArray<double> p_device_norm_workspace_, p_device_norms_;
+  double last_global_norm_ = 0;
+  // ComputeGradients (deep_rnn.h:984-1299) without its final UpdateWeights(): forward with stored
+  // activations, backward, gradients left in the layers.  *_wgrad are the unique non-pad input ids
+  // of the minibatch.  Returns the summed log-likelihood of the targets.
+  double ComputeGradients(const int *p_host_source, int source_length, const int *p_host_target_in,
+                          const int *p_host_target_out, int target_length,
+                          const int *p_host_source_wgrad, int len_source_wgrad,
+                          const int *p_host_target_wgrad, int len_target_wgrad,
+                          const int *p_host_batch_information, int minibatch_size);
+  // UpdateWeights (deep_rnn.h:1326-1412) + ClearGradients: scale, clip, theta += lr * g, zero.
+  void UpdateWeights();
+  void ClearGradients();
+  bool GetGrad(const std::string &name, std::vector<float> *out);
+
   bool SetParam(const std::string &name, const float *host, size_t n);
   bool GetParam(const std::string &name, std::vector<float> *out);
   void Synchronize();
+
+ private:
+  // encoder + decoder + attention of a teacher-forced minibatch (shared by GetError and
+  // ComputeGradients); per_step_loss: also run the loss of every step as GetError does.
+  void ForwardTeacherForced(const int *p_host_source, int source_length,
+                            const int *p_host_target_in, const int *p_host_target_out,
+                            int target_length, const int *p_host_batch_information,
+                            int minibatch_size, bool per_step_loss);
 };
 
 }  // namespace linmt

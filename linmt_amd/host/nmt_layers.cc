@@ -102,12 +102,18 @@ void LstmLayer::Init(NeuralMachineTranslation *model, bool input_layer, bool sou
     if (input_layer)
       n.p_device_sparse_lookup_ = lookup_all_.get() + (keep_gates ? (size_t)input_size_ * B * i : 0);
   }
+  if (cfg.train_mode_ && keep_gates) InitTraining();
 }
 
 void LstmLayer::InitFeedInput() {
   feed_input_mode_ = true;
   p_device_q_stack_.Alloc(4 * (size_t)lstm_size_ * lstm_size_);
   p_device_q_stack_.Zero(p_neural_mt_->stream_);
+  if (p_neural_mt_->cfg_.train_mode_ && keep_gates_) {
+    p_device_q_grad_.Alloc(4 * (size_t)lstm_size_ * lstm_size_);
+    p_device_q_grad_.Zero(p_neural_mt_->stream_);
+    p_device_errn_to_t_h_tild_.Alloc((size_t)lstm_size_ * minibatch_size_);
+  }
 }
 
 void LstmLayer::PreprocessGpuVocabIndices(const int *p_host_input_vocab_indices, int current_length,

@@ -30,17 +30,18 @@ void NeuralMachineTranslation::InitModel() {
   decode_mode_ = false;
   const int B = cfg_.minibatch_size_, T = cfg_.longest_sentence_, L = cfg_.num_layers_;
   const bool seq2seq = cfg_.sequence_to_sequence_mode_;
+  const bool keep = cfg_.train_mode_;  // training keeps i,f,g,o and the looked-up embeddings per step
   if (seq2seq) {
-    input_layer_source_.Init(this, true, true, 0, B, T, false, false);
+    input_layer_source_.Init(this, true, true, 0, B, T, keep, false);
     for (int l = 1; l < L; ++l) {
       v_hidden_layers_source_.emplace_back(new LstmLayer());
-      v_hidden_layers_source_.back()->Init(this, false, true, l, B, T, false, false);
+      v_hidden_layers_source_.back()->Init(this, false, true, l, B, T, keep, false);
     }
   }
-  input_layer_target_.Init(this, true, false, 0, B, T, false, false);
+  input_layer_target_.Init(this, true, false, 0, B, T, keep, false);
   for (int l = 1; l < L; ++l) {
     v_hidden_layers_target_.emplace_back(new LstmLayer());
-    v_hidden_layers_target_.back()->Init(this, false, false, l, B, T, false, false);
+    v_hidden_layers_target_.back()->Init(this, false, false, l, B, T, keep, false);
   }
   if (cfg_.attention_mode_ && seq2seq) {
     attention_layer_.Init(this, B, T, T);
@@ -50,8 +51,14 @@ void NeuralMachineTranslation::InitModel() {
     attention_layer_.hs_col_stride_ = cfg_.lstm_size_;
     attention_layer_.use_hs_col_ = false;
     if (cfg_.feed_input_mode_) input_layer_target_.InitFeedInput();
+    if (cfg_.train_mode_) attention_layer_.InitTraining();
   }
   softmax_layer_.Init(this, B, T);
+  if (cfg_.train_mode_) {
+    softmax_layer_.InitTraining();
+    p_device_norm_workspace_.Alloc(LH_SUMSQ_WORKSPACE);
+    p_device_norms_.Alloc(512);
+  }
   // wiring that does not change between minibatches: h_below and h~ pointers
   for (int side = 0; side < (seq2seq ? 2 : 1); ++side) {
     for (int l = 1; l < L; ++l) {
@@ -152,6 +159,20 @@ double NeuralMachineTranslation::GetError(const int *p_host_source, int source_l
                                           const int *p_host_target_in,
                                           const int *p_host_target_out, int target_length,
                                           const int *p_host_batch_information, int minibatch_size) {
+  ForwardTeacherForced(p_host_source, source_length, p_host_target_in, p_host_target_out,
+                       target_length, p_host_batch_information, minibatch_size, true);
+  double loss = 0;
+  softmax_layer_.p_device_loss_.Download(&loss, 1, stream_);
+  Synchronize();
+  profiler_.Collect();
+  return loss;
+}
+
+void NeuralMachineTranslation::ForwardTeacherForced(const int *p_host_source, int source_length,
+                                                    const int *p_host_target_in,
+                                                    const int *p_host_target_out, int target_length,
+                                                    const int *p_host_batch_information,
+                                                    int minibatch_size, bool per_step_loss) {
   if (decode_mode_) throw LinmtError("GetError: model was initialised for decoding");
   const int L = cfg_.num_layers_, B = minibatch_size;
   if (B > cfg_.minibatch_size_ || source_length > cfg_.longest_sentence_ ||
@@ -231,6 +252,7 @@ double NeuralMachineTranslation::GetError(const int *p_host_source, int source_l
     }
     softmax_layer_.SetHTPtr(t, top);
     softmax_layer_.BackPropPreprocessGpu(top, (int)step);
+    if (!per_step_loss) continue;
     // ComputeLossGpu without the per-step host read-back: accumulate on the device
     softmax_layer_.ComputeLogits(top, B);
     ProfileScope px(profiler_, kTagXent, 4.0 * cfg_.target_vocab_size_ * B);
@@ -243,11 +265,6 @@ double NeuralMachineTranslation::GetError(const int *p_host_source, int source_l
                                softmax_layer_.p_device_loss_.get(), stream_),
         "GetError loss");
   }
-  double loss = 0;
-  softmax_layer_.p_device_loss_.Download(&loss, 1, stream_);
-  Synchronize();
-  profiler_.Collect();
-  return loss;
 }
 
 // Encoder for n_sent sentences at once; ids are n_sent x source_length column-major, reversed and

@@ -24,18 +24,30 @@ enum ProfileTag {
   kTagBeamTopK,
   kTagBeamMerge,
   kTagBeamGather,
+  kTagErrorGemm,       // W^T d: errors handed to t-1 / the layer below / the attention node
+  kTagWeightGradGemm,  // d x^T accumulated over all steps
+  kTagLstmCellBwd,
+  kTagAttnBwd,
+  kTagSoftmaxGrad,
+  kTagRowSum,
+  kTagEmbedGrad,
+  kTagUpdate,
   kTagCount
 };
 
 inline const char *ProfileTagName(int t) {
   static const char *names[kTagCount] = {"embed_lookup", "gate_gemm", "lstm_cell", "attn_proj_gemm",
                                          "attn_core", "attn_out_gemm", "logits_gemm", "softmax",
-                                         "xent", "beam_topk", "beam_merge", "beam_gather"};
+                                         "xent", "beam_topk", "beam_merge", "beam_gather",
+                                         "error_gemm", "weight_grad_gemm", "lstm_cell_bwd",
+                                         "attn_bwd", "softmax_grad", "row_sum", "embed_grad",
+                                         "update"};
   return t >= 0 && t < kTagCount ? names[t] : "";
 }
 
 inline bool ProfileTagIsGemm(int t) {
-  return t == kTagGateGemm || t == kTagAttnProjGemm || t == kTagAttnOutGemm || t == kTagLogitsGemm;
+  return t == kTagGateGemm || t == kTagAttnProjGemm || t == kTagAttnOutGemm ||
+         t == kTagLogitsGemm || t == kTagErrorGemm || t == kTagWeightGradGemm;
 }
 
 struct ProfileTotals {

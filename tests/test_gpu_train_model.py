@@ -1,0 +1,143 @@
+"""GPU parity of the training path of the C++ layer classes (ComputeGradients / UpdateWeights through
+the C facade) against the CPU oracle on the same seeded weights and minibatches.  The oracle's
+backward is itself pinned by central differences (tests/test_oracle_train_pins.py).  fp32 results
+within rtol=1e-4 / atol=2e-5 (the GPU sums over minibatch x steps in one GEMM, the oracle step by
+step, so the last bits differ)."""
+import numpy as np
+import pytest
+
+from conftest import assert_close
+import ref_numpy as R
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def host():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from linmt_amd import host as h
+    h.load()
+    return h
+
+
+def _minibatch(rng, Vs, Vt, lens_s, lens_t):
+    sents = [(rng.integers(0, Vs, size=a), rng.integers(3, Vt, size=b)) for a, b in zip(lens_s, lens_t)]
+    return sents, R.pack_minibatch(sents)
+
+
+def _pair(orc, host, rng, layers, H, Vs, Vt, D, attention, feed, B, training, scale=0.5, clip_cell=False):
+    P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(attention), feed_input=bool(feed),
+                      scale=scale)
+    om = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=int(feed), longest_sent=40)
+    om.set_params(P)
+    gm = host.Model(layers, H, Vs, Vt, longest_sentence=40, attention_mode=attention,
+                    attention_width=D, feed_input=bool(feed), minibatch_size=B, training=training,
+                    clip_cell=clip_cell)
+    gm.set_params(P)
+    return P, om, gm
+
+
+def _grad_shape(P, name, su, tu):
+    if name == "src.0.W":
+        return (P[name].shape[0], len(su))
+    if name == "tgt.0.W":
+        return (P[name].shape[0], len(tu))
+    return P[name].shape
+
+
+CASES = [
+    dict(layers=2, H=16, attention=1, feed=1, D=2, seed=61),
+    dict(layers=1, H=13, attention=1, feed=0, D=1, seed=62),   # H % 4 != 0: scalar kernel paths
+    dict(layers=2, H=16, attention=0, feed=0, D=2, seed=63),
+    dict(layers=3, H=32, attention=1, feed=1, D=10, seed=64),  # window wider than the sentences
+    dict(layers=2, H=16, attention=2, feed=1, D=2, seed=65),   # global attention
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: f"L{c['layers']}H{c['H']}a{c['attention']}f{c['feed']}")
+def test_compute_gradients_vs_oracle(orc, host, case):
+    rng = np.random.default_rng(case["seed"])
+    Vs, Vt = 29, 41
+    lens_s, lens_t = [5, 3, 9, 4, 7, 1], [4, 6, 2, 8, 5, 3]
+    B = len(lens_s)
+    P, om, gm = _pair(orc, host, rng, case["layers"], case["H"], Vs, Vt, case["D"],
+                      case["attention"], case["feed"], B, dict(grad_clip_mode=0))
+    sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
+    want_ll, want = om.compute_gradients(src, tin, tout, bi, su, tu)
+    got_ll = gm.compute_gradients(src, tin, tout, bi, su, tu)
+    assert_close(got_ll, want_ll, "sum log p(target)", rtol=1e-5, atol=1e-4)
+    for name in om.param_names():
+        shape = _grad_shape(P, name, su, tu)
+        g = gm.get_grad(name, shape)
+        assert_close(g, np.asarray(want[name]).reshape(shape, order="F"), f"gradient of {name}",
+                     atol=2e-5)
+    # the same minibatch again without an update accumulates (the reference clears only in
+    # ClearGradients): every gradient doubles
+    gm.compute_gradients(src, tin, tout, bi, su, tu)
+    for name in ("softmax.D", "tgt.0.M_i", "tgt.0.W", "src.0.b_f" if True else ""):
+        shape = _grad_shape(P, name, su, tu)
+        assert_close(gm.get_grad(name, shape), 2 * np.asarray(want[name]).reshape(shape, order="F"),
+                     f"accumulated gradient of {name}", atol=4e-5)
+    gm.clear_gradients()
+    assert not np.any(gm.get_grad("softmax.D", P["softmax.D"].shape))
+    gm.close()
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_update_weights_vs_oracle(orc, host, mode):
+    rng = np.random.default_rng(70 + mode)
+    layers, H, Vs, Vt, D = 2, 16, 29, 41, 2
+    lens_s, lens_t = [5, 3, 9, 4], [4, 6, 2, 8]
+    B = len(lens_s)
+    lr = 0.7
+    # thresholds low enough that every clip is active on these gradients
+    opts = dict(learning_rate=lr, grad_clip_mode=mode, norm_clip=0.05, individual_clip=0.002)
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 1, 1, B, opts, scale=0.8)
+    for it in range(2):  # the second minibatch starts from cleared gradients and updated weights
+        sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
+        want_ll, _ = om.compute_gradients(src, tin, tout, bi, su, tu)
+        got_ll = gm.compute_gradients(src, tin, tout, bi, su, tu)
+        assert_close(got_ll, want_ll, f"minibatch {it}: sum log p", rtol=1e-5, atol=1e-4)
+        want_norm = om.update_weights(lr, mode, opts["norm_clip"], opts["individual_clip"], B)
+        got_norm = gm.update_weights()
+        if mode == 2:
+            assert want_norm > opts["norm_clip"]
+            assert_close(got_norm, want_norm, "global gradient norm", rtol=1e-4, atol=1e-6)
+        for name in om.param_names():
+            assert_close(gm.get_param(name, P[name].shape),
+                         om.get_param(name).reshape(P[name].shape, order="F"),
+                         f"minibatch {it}: updated {name}", atol=2e-6)
+        assert not np.any(gm.get_grad("tgt.1.W_ho", (H, H)))
+    gm.close()
+
+
+def test_gradients_with_error_clip(orc, host):
+    """--clip-cell: cell values clamped forward, the errors handed back in time clamped backward.
+    The thresholds are set low enough to be active; the oracle has no such mode, so the check is
+    the property that a clamp which never binds changes nothing, and that a binding one does."""
+    rng = np.random.default_rng(81)
+    layers, H, Vs, Vt, D = 2, 16, 29, 41, 2
+    lens_s, lens_t = [5, 3, 9, 4], [4, 6, 2, 8]
+    B = len(lens_s)
+    sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
+    outs = []
+    for clip_cell, err in ((False, 1000.0), (True, 1000.0), (True, 1e-3)):
+        r2 = np.random.default_rng(82)
+        P, om, gm = _pair(orc, host, r2, layers, H, Vs, Vt, D, 1, 1, B,
+                          dict(grad_clip_mode=0, error_clip_threshold=err), clip_cell=clip_cell)
+        gm.compute_gradients(src, tin, tout, bi, su, tu)
+        outs.append(gm.get_grad("src.0.M_i", (H, H)))
+        gm.close()
+    assert np.array_equal(outs[0], outs[1])
+    assert not np.allclose(outs[0], outs[2], rtol=1e-3, atol=1e-7)
+
+
+def test_training_rejects_partial_minibatch(orc, host):
+    rng = np.random.default_rng(90)
+    P, om, gm = _pair(orc, host, rng, 1, 16, 29, 41, 2, 1, 1, 4, dict(grad_clip_mode=0))
+    sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, 29, 41, [3, 4], [2, 3])
+    with pytest.raises(host.HostError):
+        gm.compute_gradients(src, tin, tout, bi, su, tu)
+    gm.close()

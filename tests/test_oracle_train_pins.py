@@ -28,6 +28,7 @@ CASES = [
     dict(layers=1, attention=1, feed=0, D=1, seed=22),
     dict(layers=2, attention=0, feed=0, D=2, seed=23),
     dict(layers=3, attention=1, feed=1, D=3, seed=24),
+    dict(layers=2, attention=2, feed=1, D=-1, seed=25),  # global attention: no window, no Gaussian
 ]
 
 
