@@ -26,22 +26,26 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_FP32_PEAK_TFLOPS = 157.3
 
 
-def make_params(rng, layers, H, Vs, Vt, scale=0.08):
+def make_params(rng, layers, H, Vs, Vt, scale=0.08, E=None, fast=False):
     """uniform[-0.08, 0.08], forget-gate bias 1 (reference initialisation)."""
     P = {}
-    u = lambda *s: rng.uniform(-scale, scale, size=s).astype(np.float32)
+    E = H if E is None else E
+    if fast:  # float32 generator: the 0.8 G parameters of the training workload in seconds
+        u = lambda *s: ((rng.random(size=s, dtype=np.float32) * 2 - 1) * np.float32(scale))
+    else:
+        u = lambda *s: rng.uniform(-scale, scale, size=s).astype(np.float32)
     for side, V in (("src", Vs), ("tgt", Vt)):
         for l in range(layers):
             pfx = f"{side}.{l}."
             for g in "ifco":
                 P[pfx + "W_h" + g] = u(H, H)
-                P[pfx + "M_" + g] = u(H, H)
+                P[pfx + "M_" + g] = u(H, E if l == 0 else H)
                 P[pfx + "b_" + g] = u(H)
                 if side == "tgt" and l == 0:
                     P[pfx + "Q_" + g] = u(H, H)
             P[pfx + "b_f"] = np.ones(H, np.float32)
             if l == 0:
-                P[pfx + "W"] = u(H, V)
+                P[pfx + "W"] = u(E, V)
     for n in ("W_a", "W_p", "W_c1", "W_c2"):
         P["attn." + n] = u(H, H)
     P["attn.v_p"] = u(H)
@@ -163,6 +167,75 @@ def bench_fused_kernels(torch, steps, warmup):
             "launches_timed": steps, "kernels": out}
 
 
+def bench_training(torch, host, steps, warmup, small):
+    """One training minibatch (forward with stored activations, backward, global-norm clip at 5,
+    SGD update) of the 8+8-layer, 2048-hidden, 1024-embedding, 50k-vocabulary model with local-p
+    attention and input feeding, batch 256, lengths uniform in [20,80] (BASELINE.json configs[4],
+    without its dropout).  Prints target tokens/s and the per-kernel-site table."""
+    rng = np.random.default_rng(SEED)
+    if small:
+        L, H, E, V, B, lo, hi = 2, 512, 256, 8000, 64, 10, 30
+    else:
+        L, H, E, V, B, lo, hi = 8, 2048, 1024, 50000, 256, 20, 80
+    longest = hi + 4
+    t0 = time.time()
+    m = host.Model(L, H, V, V, longest_sentence=longest, attention_mode=1, attention_width=10,
+                   feed_input=True, minibatch_size=B, embedding_size=E,
+                   training=dict(learning_rate=0.1, grad_clip_mode=2, norm_clip=5.0))
+    m.set_params(make_params(rng, L, H, V, V, E=E, fast=True))
+    t_init = time.time() - t0
+    ls = rng.integers(lo, hi + 1, size=B)
+    lt = rng.integers(lo, hi + 1, size=B)
+    S, T = int(ls.max()), int(lt.max())
+    src = np.full((B, S), -1, np.int32)
+    tin = np.full((B, T), -1, np.int32)
+    tout = np.full((B, T), -1, np.int32)
+    for b in range(B):
+        src[b, S - ls[b]:] = zipf_ids(rng, ls[b], V)
+        t = zipf_ids(rng, lt[b] - 1, V, lo=3)
+        tin[b, :lt[b]] = np.concatenate([[0], t])
+        tout[b, :lt[b]] = np.concatenate([t, [1]])
+    bi = np.concatenate([ls, S - ls]).astype(np.int32)
+    su = np.unique(src[src >= 0]).astype(np.int32)
+    tu = np.unique(tin[tin >= 0]).astype(np.int32)
+    n_tgt, n_src = int(lt.sum()), int(ls.sum())
+
+    def step():
+        ll = m.compute_gradients(src, tin, tout, bi, su, tu)
+        return ll, m.update_weights()
+
+    for _ in range(warmup):
+        step()
+    m.profile(2)
+    torch.cuda.synchronize()
+    t0 = time.time()
+    for _ in range(steps):
+        ll, nrm = step()
+    torch.cuda.synchronize()
+    dt = (time.time() - t0) / steps
+    tot = m.profile_totals()
+    rows = []
+    for k, v in sorted(tot.items(), key=lambda kv: -kv[1]["ms"]):
+        is_gemm = "|" in k
+        us = v["ms"] * 1e3 / max(v["launches"], 1)
+        rate = v["work"] / max(v["ms"], 1e-9) / 1e9 if is_gemm else v["work"] / max(v["ms"], 1e-9) / 1e6
+        rows.append({"site": k, "ms_per_step": round(v["ms"] / steps, 3),
+                     "launches_per_step": v["launches"] // steps, "us_per_launch": round(us, 1),
+                     ("TFLOP/s" if is_gemm else "GB/s"): round(rate, 1)})
+    out = {"metric": "target tokens/sec (training step: forward + backward + clip + SGD)",
+           "value": round(n_tgt / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+           "warmup": warmup, "ms_per_step": round(dt * 1e3, 2), "higher_is_better": True,
+           "dtype": "f32", "data": "synthetic",
+           "config": {"workload": ("configs[4] without dropout" if not small else "reduced smoke size")
+                      + f": {L}+{L} layers, H={H}, E={E}, V={V}, batch {B}, S={S}, T={T}, "
+                      f"{n_src} source + {n_tgt} target tokens"},
+           "loglik_per_target_token": round(ll / n_tgt, 4), "global_grad_norm": round(nrm, 4),
+           "kernel_ms_per_step": round(sum(v["ms"] for v in tot.values()) / steps, 2),
+           "model_build_s": round(t_init, 1), "kernels": rows}
+    m.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -178,6 +251,10 @@ def main():
                     help="instead of the decode benchmark, time the fused HBM-bound kernels alone "
                          "(at the benchmark's size and at a size that saturates HBM) and print "
                          "one JSON line with their achieved GB/s")
+    ap.add_argument("--train", action="store_true",
+                    help="instead of the decode benchmark, time one training minibatch of "
+                         "BASELINE.json configs[4] (without dropout) and print one JSON line")
+    ap.add_argument("--train-small", action="store_true", help="--train at a reduced size")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU (the path shards over sentences with no "
@@ -193,6 +270,9 @@ def main():
     host.load()
     if args.kernels:
         print(json.dumps(bench_fused_kernels(torch, args.steps, args.warmup)))
+        return
+    if args.train or args.train_small:
+        print(json.dumps(bench_training(torch, host, args.steps, args.warmup, args.train_small)))
         return
 
     layers, H, V, D, beam, n_sent, longest = 4, 1000, 30000, 10, 12, 64, 104
