@@ -255,6 +255,13 @@ int lh_beam_gather_f32(const float *const *src, float *const *dst, int n_tensors
  * Training half of the path (backward pass and update).
  * ========================================================================================== */
 
+/* Uniform numbers in (0, 1] for the dropout masks: out[i] is a fixed function of (seed, i).
+ * Replaces curandGenerateUniform (src/utility_cu.cu:218-226) at the mask sites
+ * (src/node_input_to_hidden.h:268, src/node_hidden_to_hidden.h:220, src/layer_attention.h:259,
+ * src/layer_loss.h:504); the values differ from cuRAND's XORWOW stream, the distribution and the
+ * (0, 1] range do not.  A mask keeps an element when mask < keep. */
+int lh_uniform_f32(float *out, long long n, unsigned long long seed, lh_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * a16. Softmax output error and log-likelihood in one pass over the V x B logits.
  * Replaces, for one step, the forward OutputdistOverflowPreventionKernel
@@ -288,11 +295,17 @@ int lh_softmax_xent_grad_f32(const float *logits, int ldl, const float *bias, in
  * are single GEMMs on the stacked weights.  dc_prev may alias dc_next.
  * The reference clamps the errors it hands back (dh_{t-1}, dh~_{t-1}, dx) to +-error_clip when
  * --clip-cell is on; here the consumer clamps on read, which is the same values.
+ * above_drop_mask (H x B, optional): the consumer above (next layer, attention node or softmax) read
+ * a dropped copy of this node's h, so its error comes back through the same mask, as the
+ * DropoutKernel calls on d_errn_to_t_h_below (src/node_hidden_to_hidden.h:782), errn_to_t_ht_p1
+ * (src/layer_attention.h:683) and d_errt_ht (src/layer_loss.h:598) do:
+ *   dh_above <- clamp(dh_above) * (above_drop_mask < keep) * (1/keep).
  */
 int lh_lstm_cell_bwd_f32(int H, int B, const float *dh_above, const float *dh_next,
                          const float *dc_next, const float *gates, const float *c,
                          const float *c_prev, const int *mask01, float clip_above, float clip_next,
-                         float *dgates, float *dc_prev, lh_stream_t stream);
+                         const float *above_drop_mask, float keep, float *dgates, float *dc_prev,
+                         lh_stream_t stream);
 
 /* out[r] = beta*out[r] + sum_c A[r,c] for a column-major rows x cols matrix.  Replaces the
  * cublasSgemv-with-ones bias gradients (src/node_input_to_hidden.h:1215-1240,
@@ -305,11 +318,14 @@ int lh_rowsum_acc_f32(const float *A, long long lda, int rows, long long cols, f
  * atomicAdd scatter makes the sum order vary from run to run: here the caller lists, per unique
  * id k, the dx columns that carry that id (seg_cols[seg_start[k] .. seg_start[k+1])), and
  *   small_grad[:,k] = beta*small_grad[:,k] + sum_{s} dx[:, seg_cols[s]]       (E rows)
- * in list order.  Padding columns are simply not listed.
+ * in list order.  Padding columns are simply not listed.  drop_mask (laid out like dx, optional):
+ * every dx element is first multiplied by (drop_mask < keep) * (1/keep), the embedding dropout of
+ * WSmallGradientKernelDropout (src/deep_rnn_kernel.h:288-303).
  */
 int lh_embed_gather_grad_f32(const float *dx, long long ldx, int E, int n_unique,
-                             const int *seg_start, const int *seg_cols, float beta,
-                             float *small_grad, long long ldg, lh_stream_t stream);
+                             const int *seg_start, const int *seg_cols, const float *drop_mask,
+                             float keep, float beta, float *small_grad, long long ldg,
+                             lh_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * a15. Attention backward.

@@ -46,6 +46,9 @@ typedef struct lnmt_train_options {
   float norm_clip;             /* threshold of modes 1 and 2 */
   float individual_clip;       /* threshold of mode 3 */
   float error_clip_threshold;  /* clamp of the errors handed back in time when clip_cell is set */
+  float dropout_keep;          /* probability of KEEPING a unit (the reference's dropout_rate_);
+                                  <= 0 or >= 1 switches dropout off */
+  unsigned long long dropout_seed;
 } lnmt_train_options;
 
 typedef struct lnmt_model lnmt_model;
@@ -85,6 +88,11 @@ int lnmt_model_get_grad(lnmt_model *m, const char *name, float *data, long long 
 /* NeuralMachineTranslation::UpdateWeights + ClearGradients.  *global_norm (may be NULL) receives
  * the norm the global clip used (0 in the other modes). */
 int lnmt_update_weights(lnmt_model *m, double *global_norm);
+/* The dropout masks the last lnmt_compute_gradients call drew (uniform numbers, kept when
+ * < dropout_keep): kind 0 = embeddings of side (0 src / 1 tgt), kind 1 = the mask under which the
+ * consumer above `layer` read that layer's h.  Layout rows x minibatch x steps column-major;
+ * n = floats the buffer holds (copies min(n, available)).  For parity checks. */
+int lnmt_get_dropout_mask(lnmt_model *m, int kind, int side, int layer, float *data, long long n);
 int lnmt_clear_gradients(lnmt_model *m);
 
 /* Copies a state of the last lnmt_get_error call: kind 0 = h, 1 = c of (side 0 src / 1 tgt, layer,

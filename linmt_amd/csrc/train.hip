@@ -36,6 +36,8 @@ struct CellBwdArgs {
   const float *dh_above, *dh_next, *dc_next, *gates, *c, *c_prev;
   const int *mask01;
   float clip_above, clip_next;
+  const float *above_drop_mask;
+  float keep;
   float *dgates, *dc_prev;
 };
 
@@ -63,8 +65,17 @@ __global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(const CellBwdArgs a)
   }
   if (a.dh_above) {
     t.load(a.dh_above + o1);
+    if (a.above_drop_mask) {  // the layer above saw a dropped copy of h: same mask on the way back
+      Vec<VW> u;
+      u.load(a.above_drop_mask + o1);
+      const float inv = 1.0f / a.keep;
 #pragma unroll
-    for (int i = 0; i < VW; ++i) dh.v[i] += clampf(t.v[i], a.clip_above);
+      for (int i = 0; i < VW; ++i)
+        dh.v[i] += clampf(t.v[i], a.clip_above) * (float)(a.keep > u.v[i]) * inv;
+    } else {
+#pragma unroll
+      for (int i = 0; i < VW; ++i) dh.v[i] += clampf(t.v[i], a.clip_above);
+    }
   }
   if (a.dc_next) dc.load(a.dc_next + o1);
   const float m = (float)a.mask01[b];
@@ -127,7 +138,8 @@ __global__ __launch_bounds__(256) void rowsum_kernel(const float *__restrict__ A
 template <int VW>
 __global__ __launch_bounds__(256) void embed_gather_grad_kernel(
     const float *__restrict__ dx, long long ldx, int E, const int *__restrict__ seg_start,
-    const int *__restrict__ seg_cols, float beta, float *__restrict__ small_grad, long long ldg) {
+    const int *__restrict__ seg_cols, const float *__restrict__ drop_mask, float keep, float beta,
+    float *__restrict__ small_grad, long long ldg) {
   const int k = blockIdx.x;
   const int r = (blockIdx.y * 256 + threadIdx.x) * VW;
   if (r >= E) return;
@@ -135,10 +147,19 @@ __global__ __launch_bounds__(256) void embed_gather_grad_kernel(
   Vec<VW> acc, t;
 #pragma unroll
   for (int i = 0; i < VW; ++i) acc.v[i] = 0.f;
+  const float inv = drop_mask ? 1.0f / keep : 1.0f;
   for (int s = s0; s < s1; ++s) {
-    t.load(dx + (long long)seg_cols[s] * ldx + r);
+    const long long o = (long long)seg_cols[s] * ldx + r;
+    t.load(dx + o);
+    if (drop_mask) {
+      Vec<VW> u;
+      u.load(drop_mask + o);
 #pragma unroll
-    for (int i = 0; i < VW; ++i) acc.v[i] += t.v[i];
+      for (int i = 0; i < VW; ++i) acc.v[i] += t.v[i] * (float)(keep > u.v[i]) * inv;
+    } else {
+#pragma unroll
+      for (int i = 0; i < VW; ++i) acc.v[i] += t.v[i];
+    }
   }
   float *o = small_grad + (long long)k * ldg + r;
   if (beta != 0.f) {
@@ -376,21 +397,51 @@ __global__ __launch_bounds__(256) void sgd_step_kernel(float *__restrict__ theta
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Counter-based uniform numbers in (0, 1]: element i is a fixed function of (seed, i), so a mask can
+// be regenerated and does not depend on the launch shape.
+__device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+  return z ^ (z >> 31);
+}
+__global__ __launch_bounds__(256) void uniform_kernel(float *out, long long n,
+                                                      unsigned long long seed) {
+  const unsigned long long base = mix64(seed + 0x9e3779b97f4a7c15ULL);
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const unsigned long long r = mix64(base + (unsigned long long)i * 0x9e3779b97f4a7c15ULL);
+    out[i] = ((float)(unsigned)(r >> 40) + 1.0f) * (1.0f / 16777216.0f);  // 24 bits -> (0, 1]
+  }
+}
+
 }  // namespace
+
+extern "C" int lh_uniform_f32(float *out, long long n, unsigned long long seed, lh_stream_t stream) {
+  if (n < 0 || (n > 0 && !out)) return lh::fail_arg("lh_uniform_f32: n=%lld or NULL pointer", n);
+  if (n == 0) return LH_OK;
+  long long blocks = (n + 256 * 8 - 1) / (256 * 8);
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(uniform_kernel, dim3((unsigned)blocks), dim3(256), 0, lh::as_stream(stream), out,
+                     n, seed);
+  return lh::check_launch("lh_uniform_f32");
+}
 
 extern "C" int lh_lstm_cell_bwd_f32(int H, int B, const float *dh_above, const float *dh_next,
                                     const float *dc_next, const float *gates, const float *c,
                                     const float *c_prev, const int *mask01, float clip_above,
-                                    float clip_next, float *dgates, float *dc_prev,
-                                    lh_stream_t stream) {
+                                    float clip_next, const float *above_drop_mask, float keep,
+                                    float *dgates, float *dc_prev, lh_stream_t stream) {
   if (H <= 0 || B <= 0) return lh::fail_arg("lh_lstm_cell_bwd_f32: H=%d B=%d", H, B);
   if (!gates || !c || !c_prev || !mask01 || !dgates || !dc_prev)
     return lh::fail_arg("lh_lstm_cell_bwd_f32: a required pointer is NULL");
+  if (above_drop_mask && (!dh_above || !(keep > 0.f)))
+    return lh::fail_arg("lh_lstm_cell_bwd_f32: above_drop_mask needs dh_above and keep > 0");
   CellBwdArgs a{H, B, dh_above, dh_next, dc_next, gates, c, c_prev, mask01, clip_above, clip_next,
-                dgates, dc_prev};
+                above_drop_mask, keep, dgates, dc_prev};
   const bool vec = H % 4 == 0 && lh::aligned16(dh_above) && lh::aligned16(dh_next) &&
                    lh::aligned16(dc_next) && lh::aligned16(gates) && lh::aligned16(c) &&
-                   lh::aligned16(c_prev) && lh::aligned16(dgates) && lh::aligned16(dc_prev);
+                   lh::aligned16(c_prev) && lh::aligned16(dgates) && lh::aligned16(dc_prev) &&
+                   lh::aligned16(above_drop_mask);
   const long long work = (long long)(vec ? H / 4 : H) * B;
   const dim3 grid((unsigned)((work + 255) / 256)), block(256);
   hipStream_t st = lh::as_stream(stream);
@@ -410,21 +461,23 @@ extern "C" int lh_rowsum_acc_f32(const float *A, long long lda, int rows, long l
 }
 
 extern "C" int lh_embed_gather_grad_f32(const float *dx, long long ldx, int E, int n_unique,
-                                        const int *seg_start, const int *seg_cols, float beta,
+                                        const int *seg_start, const int *seg_cols,
+                                        const float *drop_mask, float keep, float beta,
                                         float *small_grad, long long ldg, lh_stream_t stream) {
   if (E <= 0 || n_unique < 0 || !dx || !seg_start || !seg_cols || !small_grad || ldx < E || ldg < E)
     return lh::fail_arg("lh_embed_gather_grad_f32: E=%d n_unique=%d ldx=%lld ldg=%lld or NULL pointer",
                         E, n_unique, ldx, ldg);
   if (n_unique == 0) return LH_OK;
+  if (drop_mask && !(keep > 0.f)) return lh::fail_arg("lh_embed_gather_grad_f32: keep must be > 0");
   const bool vec = E % 4 == 0 && ldx % 4 == 0 && ldg % 4 == 0 && lh::aligned16(dx) &&
-                   lh::aligned16(small_grad);
+                   lh::aligned16(small_grad) && lh::aligned16(drop_mask);
   hipStream_t st = lh::as_stream(stream);
   if (vec)
     hipLaunchKernelGGL(embed_gather_grad_kernel<4>, dim3(n_unique, (E / 4 + 255) / 256), dim3(256),
-                       0, st, dx, ldx, E, seg_start, seg_cols, beta, small_grad, ldg);
+                       0, st, dx, ldx, E, seg_start, seg_cols, drop_mask, keep, beta, small_grad, ldg);
   else
     hipLaunchKernelGGL(embed_gather_grad_kernel<1>, dim3(n_unique, (E + 255) / 256), dim3(256), 0,
-                       st, dx, ldx, E, seg_start, seg_cols, beta, small_grad, ldg);
+                       st, dx, ldx, E, seg_start, seg_cols, drop_mask, keep, beta, small_grad, ldg);
   return lh::check_launch("lh_embed_gather_grad_f32");
 }
 

@@ -28,7 +28,8 @@ class Config(C.Structure):
 
 class TrainOptions(C.Structure):
     _fields_ = [("learning_rate", C.c_float), ("grad_clip_mode", C.c_int), ("norm_clip", C.c_float),
-                ("individual_clip", C.c_float), ("error_clip_threshold", C.c_float)]
+                ("individual_clip", C.c_float), ("error_clip_threshold", C.c_float),
+                ("dropout_keep", C.c_float), ("dropout_seed", C.c_ulonglong)]
 
 
 class DecodeOptions(C.Structure):
@@ -58,6 +59,8 @@ def load():
     lib.lnmt_model_get_grad.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
     lib.lnmt_update_weights.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
     lib.lnmt_clear_gradients.argtypes = [C.c_void_p]
+    lib.lnmt_get_dropout_mask.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                          C.c_longlong]
     lib.lnmt_model_destroy.argtypes = [C.c_void_p]
     lib.lnmt_model_destroy.restype = None
     lib.lnmt_model_set_param.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
@@ -109,7 +112,8 @@ class Model:
         elif training is not None:
             t = TrainOptions(training.get("learning_rate", 0.7), training.get("grad_clip_mode", 1),
                              training.get("norm_clip", 5.0), training.get("individual_clip", 0.1),
-                             training.get("error_clip_threshold", 1000.0))
+                             training.get("error_clip_threshold", 1000.0),
+                             training.get("dropout_keep", 0.0), training.get("dropout_seed", 1))
             h = lib.lnmt_model_create_training(C.byref(self.cfg), C.byref(t))
         else:
             h = lib.lnmt_model_create_scoring(C.byref(self.cfg))
@@ -202,6 +206,13 @@ class Model:
         nrm = C.c_double(0)
         _check(load().lnmt_update_weights(self.handle, C.byref(nrm)), "update_weights")
         return nrm.value
+
+    def get_dropout_mask(self, kind, side, layer, rows, B, steps):
+        """(steps, B, rows) view of the masks of the last compute_gradients call."""
+        out = np.empty(rows * B * steps, np.float32)
+        _check(load().lnmt_get_dropout_mask(self.handle, kind, side, layer, _p(out), out.size),
+               "get_dropout_mask")
+        return out.reshape((steps, B, rows))
 
     def clear_gradients(self):
         _check(load().lnmt_clear_gradients(self.handle), "clear_gradients")

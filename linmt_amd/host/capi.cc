@@ -1,4 +1,5 @@
 // C facade over the C++ layer classes (declared in include/linmt_host.h).
+#include <algorithm>
 #include <cstring>
 #include <memory>
 
@@ -85,6 +86,9 @@ extern "C" lnmt_model *lnmt_model_create_training(const lnmt_config *cfg,
         g.norm_clip_ = t->norm_clip;
         g.individual_norm_clip_threshold_ = t->individual_clip;
         g.error_clip_threshold_ = t->error_clip_threshold;
+        g.dropout_mode_ = t->dropout_keep > 0.f && t->dropout_keep < 1.f;
+        g.dropout_rate_ = g.dropout_mode_ ? t->dropout_keep : 1.f;
+        g.dropout_seed_ = t->dropout_seed;
         if (g.grad_clip_mode_ < 0 || g.grad_clip_mode_ > 3) throw LinmtError("grad_clip_mode outside [0,3]");
         if ((g.grad_clip_mode_ == 1 || g.grad_clip_mode_ == 2) && !(g.norm_clip_ > 0.f))
           throw LinmtError("norm_clip must be positive");
@@ -125,6 +129,20 @@ extern "C" int lnmt_update_weights(lnmt_model *m, double *global_norm) {
   return Guard([&] {
     m->nmt->UpdateWeights();
     if (global_norm) *global_norm = m->nmt->last_global_norm_;
+  });
+}
+
+extern "C" int lnmt_get_dropout_mask(lnmt_model *m, int kind, int side, int layer, float *data,
+                                     long long n) {
+  return Guard([&] {
+    NeuralMachineTranslation &M = *m->nmt;
+    if (layer < 0 || layer >= M.cfg_.num_layers_) throw LinmtError("layer out of range");
+    LstmLayer &L = side == 0 ? M.SourceLayer(layer) : M.TargetLayer(layer);
+    const DeviceArray<float> &a = kind == 0 ? L.dropout_mask_all_ : L.out_dropout_mask_all_;
+    if (a.size() == 0) throw LinmtError("this layer has no such dropout mask");
+    const size_t count = std::min<size_t>((size_t)n, a.size());
+    a.Download(data, count, M.stream_);
+    M.Synchronize();
   });
 }
 

@@ -49,6 +49,10 @@ struct GlobalConfiguration {
   int grad_clip_mode_ = 1;
   float norm_clip_ = 5.f;
   float individual_norm_clip_threshold_ = 0.1f;
+  // dropout (global_configuration.h:129-130): dropout_rate_ is the probability of KEEPING a unit
+  bool dropout_mode_ = false;
+  float dropout_rate_ = 1.0f;
+  unsigned long long dropout_seed_ = 1;
 };
 
 class NeuralMachineTranslation;
@@ -83,6 +87,9 @@ class LstmNode {
   float *p_device_gates_ = nullptr;          // 4H x B: i_t, f_t, c_prime_t_tanh, o_t (NULL when not kept)
   float *p_device_c_t_ = nullptr;
   float *p_device_h_t_ = nullptr;
+  float *p_device_dropout_mask_ = nullptr;      // layer 1: mask of the looked-up embeddings
+  float *p_device_out_dropout_mask_ = nullptr;  // mask under which the consumer above reads h_t
+  float *p_device_h_t_dropped_ = nullptr;       // that dropped copy (the recurrence keeps h_t)
   float *p_device_d_gates_ = nullptr;  // training: 4H x B gate errors of this step
   float *p_device_d_x_ = nullptr;      // training: error w.r.t. this step's input (M^T d)
 
@@ -152,6 +159,11 @@ class LstmLayer {
   DeviceArray<int> p_device_input_vocab_indices_wgrad_, p_device_wgrad_seg_start_,
       p_device_wgrad_seg_cols_;
   int w_grad_length_ = 0;  // unique ids of the current minibatch
+  // dropout: uniform masks for every step, regenerated per minibatch (the reference draws them
+  // with cuRAND inside each node's forward, node_input_to_hidden.h:264-272, node_hidden_to_hidden.h:208-226)
+  DeviceArray<float> dropout_mask_all_, out_dropout_mask_all_, h_dropped_all_;
+  bool out_dropout_ = false;  // the consumer above reads a dropped copy of this layer's h
+  void GenerateDropoutMasks(int steps, unsigned long long seed);
   void InitTraining();
   // Unique-id list of the minibatch (the reference's *_wgrad arrays, file_helper.cc:281-380) plus,
   // per unique id, the (timestep, column) positions that carry it.
@@ -375,6 +387,14 @@ class NeuralMachineTranslation {
   // ---- training --------------------------------------------------------------------------------
   DeviceArray<double> p_device_norm_workspace_, p_device_norms_;
   double last_global_norm_ = 0;
+  bool apply_dropout_ = false;          // true only inside ComputeGradients
+  unsigned long long minibatch_counter_ = 0;
+  // What the consumer above layer `L` reads at step t: the dropped copy while training with
+  // dropout, h_t otherwise.
+  float *UpwardState(LstmLayer &L, int t) {
+    return apply_dropout_ && L.out_dropout_ ? L.v_nodes_[t].p_device_h_t_dropped_
+                                            : L.v_nodes_[t].p_device_h_t_;
+  }
   // ComputeGradients (deep_rnn.h:984-1299) without its final UpdateWeights(): forward with stored
   // activations, backward, gradients left in the layers.  *_wgrad are the unique non-pad input ids
   // of the minibatch.  Returns the summed log-likelihood of the targets.

@@ -210,10 +210,12 @@ void LstmNode::ForwardProp() {
   const int H = L.lstm_size_, B = minibatch_size_;
   const float *x = nullptr;
   if (L.input_layer_mode_) {
-    ProfileScope ps(M.profiler_, kTagEmbedLookup, 8.0 * L.input_size_ * B);
+    const bool drop = M.apply_dropout_ && p_device_dropout_mask_;
+    ProfileScope ps(M.profiler_, kTagEmbedLookup, (drop ? 12.0 : 8.0) * L.input_size_ * B);
     LhErrorWrapper(lh_embed_lookup_f32(L.p_device_w_.get(), L.input_size_, L.vocab_size_,
-                                       p_device_input_vocab_indices_, B, nullptr, 1.f,
-                                       p_device_sparse_lookup_, s),
+                                       p_device_input_vocab_indices_, B,
+                                       drop ? p_device_dropout_mask_ : nullptr,
+                                       drop ? M.cfg_.dropout_rate_ : 1.f, p_device_sparse_lookup_, s),
                    "LstmInputHiddenNode::ForwardPropGpu sparse lookup");
     x = p_device_sparse_lookup_;
   } else {
@@ -232,13 +234,16 @@ void LstmNode::ForwardProp() {
                              L.preact_.get(), 4 * H, s),
                  "LstmNode::ForwardPropGpu stacked gate product");
   }
-  ProfileScope pc(M.profiler_, kTagLstmCell, (p_device_gates_ ? 44.0 : 28.0) * H * B);
+  const bool drop_out = M.apply_dropout_ && L.out_dropout_;
+  ProfileScope pc(M.profiler_, kTagLstmCell, ((p_device_gates_ ? 44.0 : 28.0) + (drop_out ? 8.0 : 0.0)) * H * B);
   LhErrorWrapper(lh_lstm_cell_fwd_f32(H, B, L.preact_.get(), nullptr, nullptr,
                                       L.p_device_b_stack_.get(), p_device_c_t_prev_,
                                       p_device_input_vocab_indices_01_, feed ? 1 : 0,
                                       M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f,
-                                      p_device_gates_, p_device_c_t_, p_device_h_t_, nullptr, 1.f,
-                                      nullptr, s),
+                                      p_device_gates_, p_device_c_t_, p_device_h_t_,
+                                      drop_out ? p_device_out_dropout_mask_ : nullptr,
+                                      drop_out ? M.cfg_.dropout_rate_ : 1.f,
+                                      drop_out ? p_device_h_t_dropped_ : nullptr, s),
                  "LstmNode::ForwardPropGpu fused cell");
 }
 

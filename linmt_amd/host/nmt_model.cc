@@ -206,8 +206,10 @@ void NeuralMachineTranslation::ForwardTeacherForced(const int *p_host_source, in
         if (l == 0)
           n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_full_.get() + step,
                                     Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
-        else
+        else {
           n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+          n.p_device_h_t_below_ = UpwardState(SourceLayer(l - 1), t);
+        }
         n.ForwardProp();
       }
     }
@@ -238,10 +240,11 @@ void NeuralMachineTranslation::ForwardTeacherForced(const int *p_host_source, in
           n.p_device_h_tild_ = attention_layer_.v_nodes_[t - 1].p_device_final_tmp_2_;
       } else {
         n.UpdateVectorsForwardGpu(Lt.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+        n.p_device_h_t_below_ = UpwardState(TargetLayer(l - 1), t);
       }
       n.ForwardProp();
     }
-    float *top = TargetLayer(L - 1).v_nodes_[t].p_device_h_t_;
+    float *top = UpwardState(TargetLayer(L - 1), t);
     if (attention) {
       AttentionNode &an = attention_layer_.v_nodes_[t];
       an.minibatch_size_ = B;

@@ -86,10 +86,39 @@ void LstmLayer::InitTraining() {
   p_device_m_grad_.Zero(s);
   p_device_w_h_grad_.Zero(s);
   p_device_b_grad_.Zero(s);
+  const GlobalConfiguration &cfg = p_neural_mt_->cfg_;
+  if (cfg.dropout_mode_) {
+    // every layer's h is read through a mask by the consumer above, except the top source layer,
+    // whose states the attention nodes read undropped
+    out_dropout_ = !(source_side_mode_ && layer_number_ == cfg.num_layers_ - 1);
+    if (input_layer_mode_) dropout_mask_all_.Alloc(in * B * T);
+    if (out_dropout_) {
+      out_dropout_mask_all_.Alloc(H * B * T);
+      h_dropped_all_.Alloc(H * B * T);
+    }
+  }
   for (int i = 0; i < num_nodes_; ++i) {
     v_nodes_[i].p_device_d_gates_ = d_gates_all_.get() + 4 * H * B * i;
     v_nodes_[i].p_device_d_x_ = d_x_all_.get() + in * B * i;
+    if (dropout_mask_all_.size()) v_nodes_[i].p_device_dropout_mask_ = dropout_mask_all_.get() + in * B * i;
+    if (out_dropout_) {
+      v_nodes_[i].p_device_out_dropout_mask_ = out_dropout_mask_all_.get() + H * B * i;
+      v_nodes_[i].p_device_h_t_dropped_ = h_dropped_all_.get() + H * B * i;
+    }
   }
+}
+
+void LstmLayer::GenerateDropoutMasks(int steps, unsigned long long seed) {
+  hipStream_t s = p_neural_mt_->stream_;
+  const long long B = minibatch_size_;
+  if (dropout_mask_all_.size())
+    LhErrorWrapper(lh_uniform_f32(dropout_mask_all_.get(), (long long)input_size_ * B * steps,
+                                  seed * 2 + 0, s),
+                   "dropout mask (embeddings)");
+  if (out_dropout_)
+    LhErrorWrapper(lh_uniform_f32(out_dropout_mask_all_.get(), (long long)lstm_size_ * B * steps,
+                                  seed * 2 + 1, s),
+                   "dropout mask (upward output)");
 }
 
 void LstmLayer::PreprocessWGrad(const int *p_host_indices, int current_length, int minibatch_size,
@@ -129,13 +158,15 @@ void LstmNode::BackPropGpu(const float *dh_above, bool above_is_lstm, const floa
   hipStream_t s = M.stream_;
   const int H = L.lstm_size_, B = minibatch_size_;
   const float clip = M.cfg_.clip_cell_mode_ ? M.cfg_.error_clip_threshold_ : 0.f;
+  const bool drop = M.apply_dropout_ && L.out_dropout_ && dh_above != nullptr;
   {
-    ProfileScope ps(M.profiler_, kTagLstmCellBwd, 56.0 * H * B);
+    ProfileScope ps(M.profiler_, kTagLstmCellBwd, (drop ? 60.0 : 56.0) * H * B);
     LhErrorWrapper(lh_lstm_cell_bwd_f32(H, B, dh_above, dh_next, dc_next, p_device_gates_,
                                         p_device_c_t_, p_device_c_t_prev_,
                                         p_device_input_vocab_indices_01_, above_is_lstm ? clip : 0.f,
-                                        clip, p_device_d_gates_, L.p_device_d_errn_to_t_ct_m1_.get(),
-                                        s),
+                                        clip, drop ? p_device_out_dropout_mask_ : nullptr,
+                                        M.cfg_.dropout_rate_, p_device_d_gates_,
+                                        L.p_device_d_errn_to_t_ct_m1_.get(), s),
                    "LstmNode::BackPropGpu fused cell backward");
   }
   lh_gemm_seg seg{L.p_device_w_h_stack_.get(), 4 * H, p_device_d_gates_, 4 * H, 4 * H};
@@ -193,9 +224,12 @@ void LstmLayer::ComputeGradientsAllSteps(int steps, const float *p_device_h_prev
   if (input_layer_mode_) {
     BackPropInputAllSteps(steps);
     ProfileScope ps(M.profiler_, kTagEmbedGrad, 4.0 * in * N + 4.0 * in * w_grad_length_);
+    const bool drop = M.apply_dropout_ && dropout_mask_all_.size();
     LhErrorWrapper(lh_embed_gather_grad_f32(d_x_all_.get(), in, in, w_grad_length_,
                                             p_device_wgrad_seg_start_.get(),
-                                            p_device_wgrad_seg_cols_.get(), 1.f,
+                                            p_device_wgrad_seg_cols_.get(),
+                                            drop ? dropout_mask_all_.get() : nullptr,
+                                            M.cfg_.dropout_rate_, 1.f,
                                             p_device_small_w_grad_.get(), in, s),
                    "LstmLayer::ComputeGradients small_w_grad");
   }
@@ -419,6 +453,19 @@ double NeuralMachineTranslation::ComputeGradients(
   const bool feed = attention && cfg_.feed_input_mode_;
   if (T < 1 || (seq2seq && S < 1)) throw LinmtError("ComputeGradients: empty minibatch");
 
+  apply_dropout_ = cfg_.dropout_mode_;
+  if (apply_dropout_) {
+    ++minibatch_counter_;
+    for (int l = 0; l < L; ++l) {
+      const unsigned long long base = cfg_.dropout_seed_ * 0x100000001b3ULL + minibatch_counter_ * 4096;
+      if (seq2seq) SourceLayer(l).GenerateDropoutMasks(S, base + 2 * l);
+      TargetLayer(l).GenerateDropoutMasks(T, base + 2 * l + 1);
+    }
+  }
+  struct DropoutOff {
+    bool &flag;
+    ~DropoutOff() { flag = false; }
+  } dropout_off{apply_dropout_};
   ForwardTeacherForced(p_host_source, S, p_host_target_in, p_host_target_out, T,
                        p_host_batch_information, B, false);
   if (seq2seq) input_layer_source_.PreprocessWGrad(p_host_source, S, B, p_host_source_wgrad, len_source_wgrad);
@@ -426,7 +473,9 @@ double NeuralMachineTranslation::ComputeGradients(
 
   // softmax over all steps: log-likelihood, D^T dz for every step, D and b_d gradients
   LstmLayer &top_tgt = TargetLayer(L - 1);
-  const float *h_for_softmax = attention ? attention_layer_.final_all_.get() : top_tgt.h_all_.get();
+  // what the attention nodes / the softmax read of the top decoder layer, all steps
+  const float *top_up_all = UpwardState(top_tgt, 0);
+  const float *h_for_softmax = attention ? attention_layer_.final_all_.get() : top_up_all;
   softmax_layer_.ForwardBackwardAllSteps(h_for_softmax, T);
   const float *dht_all = softmax_layer_.p_device_d_errt_ht_all_.get();
 
@@ -457,7 +506,7 @@ double NeuralMachineTranslation::ComputeGradients(
     const float *h0 = seq2seq ? SourceLayer(l).v_nodes_[S - 1].p_device_h_t_ : nullptr;
     TargetLayer(l).ComputeGradientsAllSteps(T, h0, attention ? attention_layer_.final_all_.get() : nullptr);
   }
-  if (attention) attention_layer_.ComputeGradientsAllSteps(T, top_tgt.h_all_.get());
+  if (attention) attention_layer_.ComputeGradientsAllSteps(T, top_up_all);
 
   // source side, one layer at a time (nothing couples a layer's step t to the layer above's t-1)
   if (seq2seq) {

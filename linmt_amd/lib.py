@@ -65,13 +65,15 @@ SIGNATURES = {
                                      C.c_int, C.c_int, C.c_int, c_i32p, C.c_void_p]),
     "lh_softmax_xent_grad_f32": (C.c_int, [c_f32p, C.c_int, c_f32p, C.c_int, C.c_int, c_i32p,
                                            c_i32p, c_f32p, C.c_int, c_f64p, c_f64p, C.c_void_p]),
+    "lh_uniform_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_ulonglong, C.c_void_p]),
     "lh_lstm_cell_bwd_f32": (C.c_int, [C.c_int, C.c_int, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p,
-                                       c_f32p, c_i32p, C.c_float, C.c_float, c_f32p, c_f32p,
-                                       C.c_void_p]),
+                                       c_f32p, c_i32p, C.c_float, C.c_float, c_f32p, C.c_float,
+                                       c_f32p, c_f32p, C.c_void_p]),
     "lh_rowsum_acc_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_int, C.c_longlong, C.c_float, c_f32p,
                                     C.c_void_p]),
     "lh_embed_gather_grad_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_int, C.c_int, c_i32p, c_i32p,
-                                           C.c_float, c_f32p, C.c_longlong, C.c_void_p]),
+                                           c_f32p, C.c_float, C.c_float, c_f32p, C.c_longlong,
+                                           C.c_void_p]),
     "lh_attn_delta_f32": (C.c_int, [C.c_int, C.c_int, c_f32p, c_f32p, c_f32p, c_i32p, C.c_float,
                                     c_f32p, C.c_void_p]),
     "lh_attn_core_bwd_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, c_f32p, c_f32p,
@@ -250,11 +252,17 @@ def softmax_xent_grad(logits, ldl, bias, V, B, tgt0, mask01, dz, ldz, logp_tgt, 
           "lh_softmax_xent_grad_f32")
 
 
+def uniform(out, n, seed, stream=None):
+    check(load().lh_uniform_f32(_ptr(out), n, seed, _stream(stream)), "lh_uniform_f32")
+
+
 def lstm_cell_bwd(H, B, gates, c, c_prev, mask01, dgates, dc_prev, dh_above=None, dh_next=None,
-                  dc_next=None, clip_above=0.0, clip_next=0.0, stream=None):
+                  dc_next=None, clip_above=0.0, clip_next=0.0, above_drop_mask=None, keep=1.0,
+                  stream=None):
     check(load().lh_lstm_cell_bwd_f32(H, B, _ptr(dh_above), _ptr(dh_next), _ptr(dc_next),
                                       _ptr(gates), _ptr(c), _ptr(c_prev), _ptr(mask01), clip_above,
-                                      clip_next, _ptr(dgates), _ptr(dc_prev), _stream(stream)),
+                                      clip_next, _ptr(above_drop_mask), keep, _ptr(dgates),
+                                      _ptr(dc_prev), _stream(stream)),
           "lh_lstm_cell_bwd_f32")
 
 
@@ -264,10 +272,11 @@ def rowsum_acc(A, lda, rows, cols, out, beta=0.0, stream=None):
 
 
 def embed_gather_grad(dx, ldx, E, n_unique, seg_start, seg_cols, small_grad, ldg, beta=0.0,
-                      stream=None):
+                      drop_mask=None, keep=1.0, stream=None):
     check(load().lh_embed_gather_grad_f32(_ptr(dx), ldx, E, n_unique, _ptr(seg_start),
-                                          _ptr(seg_cols), beta, _ptr(small_grad), ldg,
-                                          _stream(stream)), "lh_embed_gather_grad_f32")
+                                          _ptr(seg_cols), _ptr(drop_mask), keep, beta,
+                                          _ptr(small_grad), ldg, _stream(stream)),
+          "lh_embed_gather_grad_f32")
 
 
 def attn_delta(H, B, dht, h_tild, mask01, delta, dht_feed=None, clip_feed=0.0, stream=None):

@@ -117,7 +117,7 @@ double orc_forward_xent(orc_model *m, const int *src, int S, const int *tgt_in, 
 void orc_lstm_cell_bwd(int H, int B, const float *dh_above, const float *dh_next,
                        const float *dc_next, const float *gates, const float *c,
                        const float *c_prev, const int *mask01, float clip_above, float clip_next,
-                       float *dgates, float *dc_prev);
+                       const float *above_drop_mask, float keep, float *dgates, float *dc_prev);
 void orc_softmax_xent_grad(const float *logits, int ldl, const float *bias, int V, int B,
                            const int *tgt0, const int *mask01, float *dz, int ldz,
                            double *logp_tgt, double *loss_accum);
@@ -133,6 +133,17 @@ void orc_attn_core_bwd(int H, int B, int D, int max_len, int hs_steps, const flo
 typedef struct orc_trainer orc_trainer;
 orc_trainer *orc_trainer_create(orc_model *m, const orc_model_config *cfg);
 void orc_trainer_destroy(orc_trainer *t);
+/* Dropout for the following orc_compute_gradients calls (keep <= 0 switches it off).  Masks are
+ * uniform numbers, an element survives when mask < keep and is scaled by 1/keep (DropoutKernel,
+ * src/deep_rnn_kernel.h:1059-1063).  src_embed / tgt_embed: H x B x steps masks of the looked-up
+ * embeddings (src/node_input_to_hidden.h:264-272); src_out / tgt_out: layers x (H x B x steps),
+ * mask (l, step) is the one under which the consumer above layer l reads that layer's h: the next
+ * layer (src/node_hidden_to_hidden.h:208-226), the attention node (src/layer_attention.h:253-261)
+ * or, without attention, the softmax (src/layer_loss.h:501-507).  The top source layer's mask is
+ * unused (the attention nodes read its states undropped). */
+void orc_trainer_set_dropout(orc_trainer *t, float keep, const float *src_embed,
+                             const float *tgt_embed, const float *src_out, const float *tgt_out,
+                             int S, int T, int B);
 /* NeuralMachineTranslation::ComputeGradients without its final UpdateWeights: forward with stored
  * activations, then the backward pass.  Arguments as orc_forward_xent; src_unique / tgt_unique are
  * the unique non-pad input ids of the minibatch (the reference's *_wgrad lists).  Returns the summed

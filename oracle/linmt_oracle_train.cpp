@@ -48,6 +48,11 @@ struct orc_trainer {
   orc_model_config cfg;
   std::map<std::string, Vec> grads;
   std::vector<int> uniq[2];  // unique vocabulary ids of the minibatch, source / target input side
+  // dropout (keep <= 0: off): uniform masks, an element is kept when mask < keep.
+  // embed[side]: H x B x steps; out[side]: layers x (H x B x steps), the mask under which the
+  // consumer above layer l (next layer, attention node, or softmax) reads that layer's h.
+  float keep = 0.f;
+  Vec drop_embed[2], drop_out[2];
 };
 
 namespace {
@@ -125,12 +130,14 @@ void cell_forward(orc_trainer *t, const std::string &pfx, int B, CellTape &tp) {
 // back by node t+1 and are replaced by the ones for node t-1.  dx receives M^T d (H x B);
 // dh_tild_below (feed input, t > 0) receives Q^T d.
 void cell_backward(orc_trainer *t, const std::string &pfx, int B, const CellTape &tp,
-                   const float *dh_above, Vec &dh_next, Vec &dc_next, Vec &dx, Vec *dh_tild_below) {
+                   const float *dh_above, const float *above_drop_mask, Vec &dh_next, Vec &dc_next,
+                   Vec &dx, Vec *dh_tild_below) {
   const int H = t->cfg.H;
   const size_t n = (size_t)H * B;
   Vec dg((size_t)4 * n, 0.f), dc_prev(n, 0.f);
   orc_lstm_cell_bwd(H, B, dh_above, dh_next.data(), dc_next.data(), tp.gates.data(), tp.c.data(),
-                    tp.c_prev.data(), tp.mask.data(), 0.f, 0.f, dg.data(), dc_prev.data());
+                    tp.c_prev.data(), tp.mask.data(), 0.f, 0.f, above_drop_mask, t->keep, dg.data(),
+                    dc_prev.data());
   Vec d[4];  // unstack: the reference keeps one H x B error per gate
   for (int g = 0; g < 4; ++g) {
     d[g].resize(n);
@@ -163,7 +170,7 @@ void cell_backward(orc_trainer *t, const std::string &pfx, int B, const CellTape
 
 // WSmallGradientKernel: small_grad[:, rev[idx0_b]] += dx[:, b].  Pad columns carry dx = 0.
 void scatter_embedding(orc_trainer *t, const std::string &name, int side, const Vec &dx,
-                       const CellTape &tp, int B) {
+                       const CellTape &tp, int B, const float *drop_mask) {
   const int H = t->cfg.H;
   const std::vector<int> &u = t->uniq[side];
   Vec &g = G(t, name, (size_t)H * u.size());
@@ -179,7 +186,12 @@ void scatter_embedding(orc_trainer *t, const std::string &name, int side, const 
       fprintf(stderr, "orc_trainer: id %d missing from the unique list\n", tp.idx0[b]);
       exit(EXIT_FAILURE);
     }
-    for (int r = 0; r < H; ++r) g[idx2c(r, k, H)] += dx[idx2c(r, b, H)];
+    for (int r = 0; r < H; ++r) {
+      float sum = dx[idx2c(r, b, H)];
+      // WSmallGradientKernelDropout, deep_rnn_kernel.h:300
+      if (drop_mask) sum = sum * (t->keep > drop_mask[idx2c(r, b, H)]) * (1 / t->keep);
+      g[idx2c(r, k, H)] += sum;
+    }
   }
 }
 
@@ -194,7 +206,8 @@ void scatter_embedding(orc_trainer *t, const std::string &name, int side, const 
 extern "C" void orc_lstm_cell_bwd(int H, int B, const float *dh_above, const float *dh_next,
                                   const float *dc_next, const float *gates, const float *c,
                                   const float *c_prev, const int *mask01, float clip_above,
-                                  float clip_next, float *dgates, float *dc_prev) {
+                                  float clip_next, const float *above_drop_mask, float keep,
+                                  float *dgates, float *dc_prev) {
   auto clamp = [](float x, float lim) {
     return lim > 0.f ? (x > lim ? lim : (x < -lim ? -lim : x)) : x;
   };
@@ -205,8 +218,10 @@ extern "C" void orc_lstm_cell_bwd(int H, int B, const float *dh_above, const flo
       const float ft = gates[idx2c(1 * (size_t)H + r, b, (size_t)4 * H)];
       const float gt = gates[idx2c(2 * (size_t)H + r, b, (size_t)4 * H)];
       const float ot = gates[idx2c(3 * (size_t)H + r, b, (size_t)4 * H)];
-      float dh = (dh_next ? clamp(dh_next[o], clip_next) : 0.f) +
-                 (dh_above ? clamp(dh_above[o], clip_above) : 0.f);
+      float above = dh_above ? clamp(dh_above[o], clip_above) : 0.f;
+      // DropoutKernel (deep_rnn_kernel.h:1059) on the error handed down by the consumer above
+      if (dh_above && above_drop_mask) above = (keep > above_drop_mask[o]) * (1 / keep) * above;
+      float dh = (dh_next ? clamp(dh_next[o], clip_next) : 0.f) + above;
       const float tc = tanhf(c[o]);
       float dc = (dc_next ? dc_next[o] : 0.f) + dh * ot * (1.0f - tc * tc);
       dh = dh * mask01[b];
@@ -319,6 +334,18 @@ extern "C" orc_trainer *orc_trainer_create(orc_model *m, const orc_model_config 
 
 extern "C" void orc_trainer_destroy(orc_trainer *t) { delete t; }
 
+extern "C" void orc_trainer_set_dropout(orc_trainer *t, float keep, const float *src_embed,
+                                        const float *tgt_embed, const float *src_out,
+                                        const float *tgt_out, int S, int T, int B) {
+  t->keep = keep;
+  const size_t n = (size_t)t->cfg.H * B, L = t->cfg.layers;
+  if (!(keep > 0.f)) return;
+  t->drop_embed[0].assign(src_embed, src_embed + n * S);
+  t->drop_embed[1].assign(tgt_embed, tgt_embed + n * T);
+  t->drop_out[0].assign(src_out, src_out + n * S * L);
+  t->drop_out[1].assign(tgt_out, tgt_out + n * T * L);
+}
+
 extern "C" float *orc_trainer_grad(orc_trainer *t, const char *name, long long *n_elems) {
   const auto it = t->grads.find(name);
   if (it == t->grads.end()) return nullptr;
@@ -343,8 +370,29 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
   G(t, "src.0.W", (size_t)H * n_src_unique);
   G(t, "tgt.0.W", (size_t)H * n_tgt_unique);
 
+  const bool drop = t->keep > 0.f;
+  if (drop && (t->drop_embed[0].size() != n * S || t->drop_embed[1].size() != n * T ||
+               t->drop_out[0].size() != n * S * L || t->drop_out[1].size() != n * T * L)) {
+    fprintf(stderr, "orc_trainer: dropout masks do not match this minibatch\n");
+    exit(EXIT_FAILURE);
+  }
+  auto out_mask = [&](int side, int l, int s) -> const float * {
+    if (!drop) return nullptr;
+    const int steps = side == 0 ? S : T;
+    return t->drop_out[side].data() + ((size_t)l * steps + s) * n;
+  };
+  auto embed_mask = [&](int side, int s) -> const float * {
+    return drop ? t->drop_embed[side].data() + (size_t)s * n : nullptr;
+  };
+  auto dropped = [&](const Vec &h, const float *mask) {
+    Vec r = h;
+    if (mask) orc_dropout(r.data(), mask, t->keep, (long long)n);
+    return r;
+  };
+
   // ------------------------------------------------------------------------------ forward
   std::vector<std::vector<CellTape>> enc(S, std::vector<CellTape>(L)), dec(T, std::vector<CellTape>(L));
+  std::vector<Vec> ha_all(T);  // what the attention node / softmax reads of the top decoder layer
   std::vector<AttnTape> att(T);
   Vec zeros(n, 0.f);
   Vec hs((size_t)S * n);
@@ -356,9 +404,10 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
       orc_preprocess_indices(src + (size_t)s * B, B, tp.idx0.data(), tp.mask.data(), nullptr);
       tp.x.assign(n, 0.f);
       if (l == 0)
-        orc_embed_lookup(P(t, "src.0.W"), H, cfg.V_src, tp.idx0.data(), B, nullptr, 1.f, tp.x.data());
+        orc_embed_lookup(P(t, "src.0.W"), H, cfg.V_src, tp.idx0.data(), B, embed_mask(0, s),
+                         drop ? t->keep : 1.f, tp.x.data());
       else
-        tp.x = enc[s][l - 1].h;
+        tp.x = dropped(enc[s][l - 1].h, out_mask(0, l - 1, s));
       tp.h_prev = s ? enc[s - 1][l].h : zeros;
       tp.c_prev = s ? enc[s - 1][l].c : zeros;
       cell_forward(t, "src." + std::to_string(l) + ".", B, tp);
@@ -375,16 +424,20 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
       orc_preprocess_indices(tgt_in + (size_t)s * B, B, tp.idx0.data(), tp.mask.data(), nullptr);
       tp.x.assign(n, 0.f);
       if (l == 0)
-        orc_embed_lookup(P(t, "tgt.0.W"), H, V, tp.idx0.data(), B, nullptr, 1.f, tp.x.data());
+        orc_embed_lookup(P(t, "tgt.0.W"), H, V, tp.idx0.data(), B, embed_mask(1, s),
+                         drop ? t->keep : 1.f, tp.x.data());
       else
-        tp.x = dec[s][l - 1].h;
+        tp.x = dropped(dec[s][l - 1].h, out_mask(1, l - 1, s));
       tp.h_prev = s ? dec[s - 1][l].h : (S ? enc[S - 1][l].h : zeros);
       tp.c_prev = s ? dec[s - 1][l].c : (S ? enc[S - 1][l].c : zeros);
       tp.feed = l == 0 && feed_cfg && s != 0;
       if (tp.feed) tp.h_tild_prev = att[s - 1].h_tild;
       cell_forward(t, "tgt." + std::to_string(l) + ".", B, tp);
     }
-    const float *top = dec[s][L - 1].h.data();
+    // the attention node (layer_attention.h:253-261) or, without attention, the softmax
+    // (layer_loss.h:501-507) works on a dropped copy of the top layer's h
+    ha_all[s] = dropped(dec[s][L - 1].h, out_mask(1, L - 1, s));
+    const float *top = ha_all[s].data();
     if (attn) {
       AttnTape &a = att[s];
       a.tanh1.assign(n, 0.f);
@@ -434,7 +487,7 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
   bool have_feed = false;
   Vec &gD = G(t, "softmax.D", (size_t)V * H);
   for (int s = T - 1; s >= 0; --s) {
-    const float *h_in = attn ? att[s].h_tild.data() : dec[s][L - 1].h.data();
+    const float *h_in = attn ? att[s].h_tild.data() : ha_all[s].data();
     Vec dht(n, 0.f);
     orc_gemm(H, B, V, P(t, "softmax.D"), V, 1, dz[s].data(), V, 0, 1.f, 0.f, dht.data(), H);
     orc_gemm(V, H, B, dz[s].data(), V, 0, h_in, H, 1, 1.f, 1.f, gD.data(), V);
@@ -444,7 +497,7 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
     if (attn) {
       const AttnTape &a = att[s];
       const CellTape &topc = dec[s][L - 1];
-      const float *ha = topc.h.data();
+      const float *ha = ha_all[s].data();
       Vec delta(n, 0.f);
       orc_attn_delta(H, B, dht.data(), (feed_cfg && have_feed) ? dh_tild_feed.data() : nullptr,
                      a.h_tild.data(), topc.mask.data(), 0.f, delta.data());
@@ -474,10 +527,11 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
     Vec dx, dh_above = dh_top;
     for (int l = L - 1; l >= 0; --l) {
       Vec feed_out;
-      cell_backward(t, "tgt." + std::to_string(l) + ".", B, dec[s][l], dh_above.data(), dh_next[l],
-                    dc_next[l], dx, dec[s][l].feed ? &feed_out : nullptr);
+      cell_backward(t, "tgt." + std::to_string(l) + ".", B, dec[s][l], dh_above.data(),
+                    out_mask(1, l, s), dh_next[l], dc_next[l], dx,
+                    dec[s][l].feed ? &feed_out : nullptr);
       if (l == 0) {
-        scatter_embedding(t, "tgt.0.W", 1, dx, dec[s][0], B);
+        scatter_embedding(t, "tgt.0.W", 1, dx, dec[s][0], B, embed_mask(1, s));
         have_feed = dec[s][0].feed;
         if (have_feed) dh_tild_feed = feed_out;
       } else {
@@ -489,10 +543,11 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
   for (int s = S - 1; s >= 0; --s) {
     Vec dx, dh_above = attn ? Vec(dHS.begin() + (size_t)s * n, dHS.begin() + (size_t)(s + 1) * n) : zeros;
     for (int l = L - 1; l >= 0; --l) {
-      cell_backward(t, "src." + std::to_string(l) + ".", B, enc[s][l], dh_above.data(), dh_next[l],
-                    dc_next[l], dx, nullptr);
+      // the top source layer is read undropped by the attention nodes
+      cell_backward(t, "src." + std::to_string(l) + ".", B, enc[s][l], dh_above.data(),
+                    l == L - 1 ? nullptr : out_mask(0, l, s), dh_next[l], dc_next[l], dx, nullptr);
       if (l == 0)
-        scatter_embedding(t, "src.0.W", 0, dx, enc[s][0], B);
+        scatter_embedding(t, "src.0.W", 0, dx, enc[s][0], B, embed_mask(0, s));
       else
         dh_above = dx;
     }

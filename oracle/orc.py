@@ -214,7 +214,7 @@ def _fa(a):
 
 
 def lstm_cell_bwd(gates, c, c_prev, mask01, dh_above=None, dh_next=None, dc_next=None,
-                  clip_above=0.0, clip_next=0.0):
+                  clip_above=0.0, clip_next=0.0, above_drop_mask=None, keep=1.0):
     """gates (4H,B), c / c_prev (H,B).  Returns dgates (4H,B), dc_prev (H,B)."""
     H4, B = gates.shape
     H = H4 // 4
@@ -222,7 +222,8 @@ def lstm_cell_bwd(gates, c, c_prev, mask01, dh_above=None, dh_next=None, dc_next
     dcp = np.empty((H, B), np.float32, order="F")
     lib().orc_lstm_cell_bwd(H, B, _p(_fa(dh_above)), _p(_fa(dh_next)), _p(_fa(dc_next)),
                             _p(_fa(gates)), _p(_fa(c)), _p(_fa(c_prev)), _p(i32(mask01)),
-                            _f(clip_above), _f(clip_next), _p(dg), _p(dcp))
+                            _f(clip_above), _f(clip_next), _p(_fa(above_drop_mask)), _f(keep),
+                            _p(dg), _p(dcp))
     return dg, dcp
 
 
@@ -316,11 +317,28 @@ class Model:
                                       _p(i32(batch_info)), num_threads)
 
     # ---- training -------------------------------------------------------------------------------
+    def _trainer(self):
+        if getattr(self, "trainer", None) is None:
+            self.trainer = C.c_void_p(lib().orc_trainer_create(self.handle, C.byref(self.cfg)))
+        return self.trainer
+
+    def set_dropout(self, keep, B=1, src_embed=None, tgt_embed=None, src_out=None, tgt_out=None):
+        """Masks as flat float32 arrays in device layout: embed (steps, B, H) C-order = H x B x steps
+        column-major; out (layers, steps, B, H).  keep <= 0 switches dropout off."""
+        t = self._trainer()
+        if not keep > 0:
+            lib().orc_trainer_set_dropout(t, _f(0.0), None, None, None, None, 0, 0, 0)
+            return
+        H, L = self.cfg.H, self.cfg.layers
+        se, te, so, to = (f32(a).ravel() for a in (src_embed, tgt_embed, src_out, tgt_out))
+        S, T = se.size // (H * B), te.size // (H * B)
+        assert so.size == L * S * H * B and to.size == L * T * H * B
+        lib().orc_trainer_set_dropout(t, _f(keep), _p(se), _p(te), _p(so), _p(to), S, T, B)
+
     def compute_gradients(self, src, tgt_in, tgt_out, batch_info, src_unique, tgt_unique):
         """Forward + backward (no update).  Returns (sum log p, {name: gradient}); matrices come back
         as Fortran-ordered 2-D arrays, the embedding gradients as (H, n_unique)."""
-        if getattr(self, "trainer", None) is None:
-            self.trainer = C.c_void_p(lib().orc_trainer_create(self.handle, C.byref(self.cfg)))
+        self._trainer()
         src = np.asfortranarray(src, np.int32)
         tgt_in = np.asfortranarray(tgt_in, np.int32)
         tgt_out = np.asfortranarray(tgt_out, np.int32)

@@ -202,21 +202,49 @@ def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=Tr
     return (best[1:-1] if best is not None else []), best_s, hyps
 
 
-def minibatch_loglik(P, layers, H, D, sents, attention=True, feed_input=True):
+def minibatch_loglik(P, layers, H, D, sents, attention=True, feed_input=True, drop=None):
     """Teacher-forced sum of log p(target) over a list of (source ids, target ids without
-    <START>/<EOF>) sentence pairs, float64, one sentence at a time (no padding involved)."""
+    <START>/<EOF>) sentence pairs, float64, one sentence at a time (no padding involved).
+    drop = dict(keep, src_embed (S,B,H), tgt_embed (T,B,H), src_out (L,S,B,H), tgt_out (L,T,B,H)):
+    uniform masks indexed by the minibatch's own timestep (source sentences sit right-aligned in
+    their S steps); an element is kept when mask < keep and scaled by 1/keep.  Inverted dropout on
+    the embeddings and on what each layer hands UP (to the next layer, the attention node, or the
+    softmax when there is no attention); the recurrent path and the encoder states read by the
+    attention are not dropped."""
     P = {k: np.asarray(v, np.float64) for k, v in P.items()}
     total = 0.0
-    for s, t in sents:
-        he, ce, top = encode(P, layers, H, s)
+    S_max = max(len(s) for s, _ in sents)
+
+    def dr(x, mask):
+        if drop is None:
+            return x
+        return x * ((mask < drop["keep"]) / drop["keep"])[:, None]
+
+    for b, (s, t) in enumerate(sents):
+        if drop is None:
+            he, ce, top = encode(P, layers, H, s)
+        else:
+            S = len(s)
+            he = [np.zeros((H, 1)) for _ in range(layers)]
+            ce = [np.zeros((H, 1)) for _ in range(layers)]
+            top = {}
+            for k in range(S):
+                pos, step = S - 1 - k, S_max - S + k
+                x = dr(P["src.0.W"][:, [int(s[pos])]], drop["src_embed"][step, b])
+                for l in range(layers):
+                    he[l], ce[l], _ = lstm_step(P, f"src.{l}.", x, he[l], ce[l])
+                    x = dr(he[l], drop["src_out"][l, step, b])
+                top[pos] = he[layers - 1][:, 0].copy()
         h, c = [x.copy() for x in he], [x.copy() for x in ce]
         h_tild = None
         for step, (wi, wo) in enumerate(zip(np.concatenate([[0], t]), np.concatenate([t, [1]]))):
             x = P["tgt.0.W"][:, [int(wi)]]
+            if drop is not None:
+                x = dr(x, drop["tgt_embed"][step, b])
             for l in range(layers):
                 ht = h_tild if (l == 0 and step != 0 and attention and feed_input) else None
                 h[l], c[l], _ = lstm_step(P, f"tgt.{l}.", x, h[l], c[l], ht)
-                x = h[l]
+                x = h[l] if drop is None else dr(h[l], drop["tgt_out"][l, step, b])
             if attention:
                 h_tild, _ = attention_local_p(P, x, lambda _b, pos: top[pos], [len(s)], [1], D)
                 x = h_tild

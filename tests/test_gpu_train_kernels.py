@@ -31,6 +31,15 @@ def test_lstm_cell_bwd(lh, orc, H, B, clip):
         assert_close(host(dg, (4 * H, B)), want_dg, "dgates")
         assert_close(host(dc, (H, B)), want_dc, "dc_prev")
         assert not np.any(host(dg, (4 * H, B))[:, mask == 0])
+    # the consumer above read a dropped copy of h: its error returns through the same mask
+    u = rng.random((H, B)).astype(np.float32)
+    want_dg, want_dc = orc.lstm_cell_bwd(gates, c, c_prev, mask, dha, dhn, dcn, clip, clip, u, 0.7)
+    dg = torch.empty(4 * H * B, device="cuda")
+    dc = torch.empty(H * B, device="cuda")
+    lh.lstm_cell_bwd(H, B, dev(gates), dev(c), dev(c_prev), dev(mask), dg, dc, dev(dha), dev(dhn),
+                     dev(dcn), clip, clip, dev(u), 0.7)
+    assert_close(host(dg, (4 * H, B)), want_dg, "dgates (dropout)")
+    assert_close(host(dc, (H, B)), want_dc, "dc_prev (dropout)")
 
 
 @pytest.mark.parametrize("V,B", [(5000, 32), (30000, 24), (37, 5), (50000, 8)])
@@ -87,6 +96,34 @@ def test_embed_gather_grad(lh, E, U, N):
         lh.embed_gather_grad(dev(dx), E, E, U, dev(seg_start), dev(seg_cols), g, E, beta)
         want = np.stack([dx[:, c].astype(np.float64).sum(axis=1) for c in cols], axis=1) + beta * g0
         assert_close(host(g, (E, U)), want, "small gradient", rtol=1e-4, atol=1e-5)
+    # embedding dropout: each dx element passes through (mask < keep) / keep first
+    u, keep = rng.random((E, N)).astype(np.float32), 0.8
+    g = dev(g0)
+    lh.embed_gather_grad(dev(dx), E, E, U, dev(seg_start), dev(seg_cols), g, E, 0.0, dev(u), keep)
+    dxm = dx.astype(np.float64) * (u < keep) / keep
+    want = np.stack([dxm[:, c].sum(axis=1) for c in cols], axis=1)
+    assert_close(host(g, (E, U)), want, "small gradient (dropout)", rtol=1e-4, atol=1e-5)
+
+
+def test_uniform_generator(lh):
+    """Own design (the reference draws from cuRAND): values in (0, 1], reproducible per seed,
+    independent of n, different across seeds, uniform to within sampling error."""
+    n = 1 << 22
+    a, b, c = (torch.empty(n, device="cuda") for _ in range(3))
+    lh.uniform(a, n, 1234)
+    lh.uniform(b, n, 1234)
+    lh.uniform(c, n // 3, 1235)
+    A, B_, C_ = host(a, (n,)), host(b, (n,)), host(c, (n,))[: n // 3]
+    assert np.array_equal(A, B_)
+    assert A.min() > 0.0 and A.max() <= 1.0
+    assert not np.array_equal(A[: n // 3], C_)
+    assert abs(A.mean() - 0.5) < 1e-3 and abs((A < 0.8).mean() - 0.8) < 1e-3
+    hist = np.histogram(A, bins=64, range=(0, 1))[0] / n
+    assert np.all(np.abs(hist - 1 / 64) < 5e-4)
+    assert abs(np.corrcoef(A[:-1], A[1:])[0, 1]) < 3e-3
+    d = torch.empty(1000, device="cuda")
+    lh.uniform(d, 1000, 1234)
+    assert np.array_equal(host(d, (1000,)), A[:1000])
 
 
 @pytest.mark.parametrize("H,B", [(1000, 64), (9, 4)])

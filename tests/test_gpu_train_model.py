@@ -134,6 +134,44 @@ def test_gradients_with_error_clip(orc, host):
     assert not np.allclose(outs[0], outs[2], rtol=1e-3, atol=1e-7)
 
 
+@pytest.mark.parametrize("attention", [1, 0])
+def test_compute_gradients_with_dropout_vs_oracle(orc, host, attention):
+    """The model draws its own masks (one uniform tensor per layer and minibatch); the test reads
+    them back and hands the very same masks to the oracle."""
+    rng = np.random.default_rng(95 + attention)
+    layers, H, Vs, Vt, D, keep = 3, 16, 29, 41, 2, 0.7
+    lens_s, lens_t = [5, 3, 9, 4, 7, 1], [4, 6, 2, 8, 5, 3]
+    B = len(lens_s)
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, attention, attention, B,
+                      dict(grad_clip_mode=0, dropout_keep=keep, dropout_seed=7))
+    sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
+    S, T = src.shape[1], tin.shape[1]
+    lls = []
+    for it in range(2):  # a second minibatch draws new masks
+        got_ll = gm.compute_gradients(src, tin, tout, bi, su, tu)
+        se = gm.get_dropout_mask(0, 0, 0, H, B, S)
+        te = gm.get_dropout_mask(0, 1, 0, H, B, T)
+        so = np.stack([gm.get_dropout_mask(1, 0, l, H, B, S) if l < layers - 1
+                       else np.ones((S, B, H), np.float32) for l in range(layers)])
+        to = np.stack([gm.get_dropout_mask(1, 1, l, H, B, T) for l in range(layers)])
+        assert 0.6 < (te < keep).mean() < 0.8
+        om.set_dropout(keep, B, se, te, so, to)
+        want_ll, want = om.compute_gradients(src, tin, tout, bi, su, tu)
+        assert_close(got_ll, want_ll, "sum log p(target)", rtol=1e-5, atol=1e-4)
+        for name in om.param_names():
+            shape = _grad_shape(P, name, su, tu)
+            assert_close(gm.get_grad(name, shape), np.asarray(want[name]).reshape(shape, order="F"),
+                         f"gradient of {name}", atol=2e-5)
+        gm.clear_gradients()
+        lls.append(got_ll)
+    assert abs(lls[0] - lls[1]) > 1e-3  # different masks, different result
+    # scoring on the same model applies no dropout
+    om.set_dropout(0.0)
+    assert_close(gm.get_error(src, tin, tout, bi), om.forward_xent(src, tin, tout, bi),
+                 "GetError on a training model", rtol=1e-5, atol=1e-4)
+    gm.close()
+
+
 def test_training_rejects_partial_minibatch(orc, host):
     rng = np.random.default_rng(90)
     P, om, gm = _pair(orc, host, rng, 1, 16, 29, 41, 2, 1, 1, 4, dict(grad_clip_mode=0))

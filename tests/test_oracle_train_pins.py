@@ -72,6 +72,48 @@ def test_gradients_vs_central_differences(orc, case):
     assert checked == 2 * len(m.param_names())
 
 
+@pytest.mark.parametrize("attention", [1, 0])
+def test_gradients_with_dropout_vs_central_differences(orc, attention):
+    """Same check with dropout masks: embeddings, every layer's upward output, the attention /
+    softmax input.  keep = 0.6 so that many elements are dropped."""
+    rng = np.random.default_rng(27 + attention)
+    layers, H, Vs, Vt, D, keep = 2, 7, 13, 11, 2, 0.6
+    P, m = _model(orc, rng, layers, H, Vs, Vt, attention, attention, D)
+    sents = _sentences(rng, Vs, Vt, [5, 3, 7, 4], [4, 6, 2, 5])
+    src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
+    B, S, T = len(sents), src.shape[1], tin.shape[1]
+    drop = dict(keep=keep, src_embed=rng.random((S, B, H)).astype(np.float32),
+                tgt_embed=rng.random((T, B, H)).astype(np.float32),
+                src_out=rng.random((layers, S, B, H)).astype(np.float32),
+                tgt_out=rng.random((layers, T, B, H)).astype(np.float32))
+    m.set_dropout(keep, B, drop["src_embed"], drop["tgt_embed"], drop["src_out"], drop["tgt_out"])
+    ll, grads = m.compute_gradients(src, tin, tout, bi, su, tu)
+    kw = dict(attention=bool(attention), feed_input=bool(attention), drop=drop)
+    P64 = {k: v.astype(np.float64) for k, v in P.items()}
+    want_ll = R.minibatch_loglik(P64, layers, H, D, sents, **kw)
+    assert abs(ll - want_ll) < 1e-4 * max(1.0, abs(want_ll))
+    # dropout changes the result (the masks are really applied)
+    assert abs(want_ll - R.minibatch_loglik(P64, layers, H, D, sents, attention=bool(attention),
+                                            feed_input=bool(attention))) > 1e-3
+    eps = 1e-5
+    for name in m.param_names():
+        g = grads[name].astype(np.float64)
+        if name in ("src.0.W", "tgt.0.W"):
+            full = np.zeros_like(P64[name])
+            full[:, su if name == "src.0.W" else tu] = g
+            g = full
+        direction = rng.standard_normal(P64[name].shape)
+        Pp, Pm = dict(P64), dict(P64)
+        Pp[name] = P64[name] + eps * direction
+        Pm[name] = P64[name] - eps * direction
+        fd = (R.minibatch_loglik(Pp, layers, H, D, sents, **kw)
+              - R.minibatch_loglik(Pm, layers, H, D, sents, **kw)) / (2 * eps)
+        got = float(np.sum(g * direction))
+        scale = float(np.sqrt(np.sum(g * g) * np.sum(direction * direction)))
+        assert abs(got - fd) <= 2e-3 * scale + 1e-5, (name, got, fd, scale)
+    m.set_dropout(0.0)
+
+
 def test_embedding_rows_outside_the_minibatch_get_no_gradient(orc):
     """Dense view of the scatter: ids that do not occur have zero finite-difference gradient, and an
     id occurring several times gets the sum (compare with a per-occurrence float64 accumulation)."""
