@@ -46,9 +46,16 @@ __device__ __forceinline__ float local_max(const float4 (&x)[NV]) {
   return m;
 }
 
+// exp for the bandwidth-bound passes: one multiply + v_exp_f32 instead of expf's range handling.
+// The argument is <= 0 here (max already subtracted), so there is no overflow; the result is within
+// ~|x| * 2^-24 relative of expf, far inside the tolerance of the probabilities and log-sums.
+__device__ __forceinline__ float exp_neg(float x) {
+  return __builtin_amdgcn_exp2f(x * 1.44269504088896341f);
+}
+
 // ---- probabilities out ----------------------------------------------------------------------
 template <int NV>
-__global__ __launch_bounds__(kT) void softmax_fwd_kernel(const float *__restrict__ logits, int ldl,
+__global__ __launch_bounds__(kT, (NV <= 8 ? 8 : 4)) void softmax_fwd_kernel(const float *__restrict__ logits, int ldl,
                                                          const float *__restrict__ bias, int V,
                                                          float *__restrict__ p, int ldp) {
   __shared__ float red[kNW];
@@ -59,8 +66,8 @@ __global__ __launch_bounds__(kT) void softmax_fwd_kernel(const float *__restrict
   float part = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    x[i].x = expf(x[i].x - mx); x[i].y = expf(x[i].y - mx);
-    x[i].z = expf(x[i].z - mx); x[i].w = expf(x[i].w - mx);
+    x[i].x = exp_neg(x[i].x - mx); x[i].y = exp_neg(x[i].y - mx);
+    x[i].z = exp_neg(x[i].z - mx); x[i].w = exp_neg(x[i].w - mx);
     part += (x[i].x + x[i].y) + (x[i].z + x[i].w);
   }
   const float sum = lh::block_sum<kNW>(part, red);
@@ -106,7 +113,7 @@ __global__ void train_loglik_kernel(const float *p, int ldp, int B, const int *t
 
 // ---- double-precision log-softmax of the target row -----------------------------------------
 template <int NV>
-__global__ __launch_bounds__(kT) void logsoftmax_tgt_kernel(const float *__restrict__ logits,
+__global__ __launch_bounds__(kT, (NV <= 8 ? 8 : 4)) void logsoftmax_tgt_kernel(const float *__restrict__ logits,
                                                             int ldl, const float *__restrict__ bias,
                                                             int V, const int *__restrict__ tgt0,
                                                             double *__restrict__ logp_tgt) {
@@ -164,7 +171,7 @@ __global__ __launch_bounds__(kT) void logsoftmax_tgt_generic_kernel(const float 
 // dz may alias logits: a column is fully in registers (or each row is owned by one thread) before
 // anything is written.
 template <int NV>
-__global__ __launch_bounds__(kT) void softmax_xent_grad_kernel(
+__global__ __launch_bounds__(kT, (NV <= 8 ? 8 : 4)) void softmax_xent_grad_kernel(
     const float *__restrict__ logits, int ldl, const float *__restrict__ bias, int V,
     const int *__restrict__ tgt0, const int *__restrict__ mask01, float *dz, int ldz,
     double *__restrict__ logp_tgt) {
@@ -176,8 +183,8 @@ __global__ __launch_bounds__(kT) void softmax_xent_grad_kernel(
   float part = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    x[i].x = expf(x[i].x - mx); x[i].y = expf(x[i].y - mx);
-    x[i].z = expf(x[i].z - mx); x[i].w = expf(x[i].w - mx);
+    x[i].x = exp_neg(x[i].x - mx); x[i].y = exp_neg(x[i].y - mx);
+    x[i].z = exp_neg(x[i].z - mx); x[i].w = exp_neg(x[i].w - mx);
     part += (x[i].x + x[i].y) + (x[i].z + x[i].w);
   }
   const float sum = lh::block_sum<kNW>(part, red);
@@ -193,8 +200,12 @@ __global__ __launch_bounds__(kT) void softmax_xent_grad_kernel(
       float4 d = make_float4(-p.x * m, -p.y * m, -p.z * m, -p.w * m);
       if (t / 4 == f) {
         const int c = t % 4;
-        logp_tgt[b] = log((double)comp(p, c));
-        comp(d, c) += m;
+        const float pt = c == 0 ? p.x : (c == 1 ? p.y : (c == 2 ? p.z : p.w));
+        logp_tgt[b] = log((double)pt);
+        d.x += c == 0 ? m : 0.f;
+        d.y += c == 1 ? m : 0.f;
+        d.z += c == 2 ? m : 0.f;
+        d.w += c == 3 ? m : 0.f;
       }
       out[f] = d;
     }
@@ -231,12 +242,16 @@ __global__ __launch_bounds__(kT) void softmax_xent_grad_generic_kernel(
   }
 }
 
-__global__ void masked_sum_kernel(const double *logp_tgt, const int *mask01, int B, double *accum) {
-  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+// accum[0] += sum of logp_tgt over unmasked columns: one 1024-thread workgroup, strided partial
+// sums folded in a fixed order (double, so the order is immaterial at the tolerance of the loss).
+__global__ __launch_bounds__(kT) void masked_sum_kernel(const double *logp_tgt, const int *mask01,
+                                                        int B, double *accum) {
+  __shared__ double redd[kNW];
   double acc = 0.0;
-  for (int b = 0; b < B; ++b)
+  for (int b = threadIdx.x; b < B; b += kT)
     if (mask01[b] == 1) acc += logp_tgt[b];
-  accum[0] += acc;
+  const double s = lh::block_sum<kNW>(acc, redd);
+  if (threadIdx.x == 0) accum[0] += s;
 }
 
 // ---- fused log-softmax + per-column top-K ---------------------------------------------------
@@ -262,24 +277,68 @@ __device__ __forceinline__ Best wave_argmax(Best x) {
 
 constexpr int kIdNone = 0x7fffffff;
 
+// Selection without arg-max rounds over the whole column.  Any threshold tau with at least K
+// elements >= tau contains the true top K among the elements >= tau; those are collected into a
+// short LDS list and ranked by counting (rank r < K is output slot r) under the strict total order
+// (value desc, vocab id asc), which is what K rounds of arg-max with lowest-id tie breaking give.
+//   fast path: tau = K-th largest of G group maxima (G = 16 wavefronts for K <= 16, else 64
+//     quarter-wavefronts): K groups hold an element >= tau.  Values only, a few instructions per
+//     element; the list has a few dozen entries on ordinary logits.
+//   exact path (list overflow: massive ties, winners packed into one group): per-thread bests with
+//     ids, the K best of each wavefront's 64 thread-bests, tau = K-th best of those 16*K survivors
+//     as a (value, id) pair.  Never more than K*NV*4 <= kListCap elements pass it.
+constexpr int kListCap = 4096;
+
 template <int NV>
-__global__ __launch_bounds__(kT) void beam_topk_kernel(const float *__restrict__ logits, int ldl,
-                                                       const float *__restrict__ bias, int V, int K,
-                                                       int eof_id, float *__restrict__ cand_logp,
-                                                       int *__restrict__ cand_id,
-                                                       float *__restrict__ logp_eof) {
+__device__ __forceinline__ void collect(const float4 (&x)[NV], int tid, int V, float tv, int ti,
+                                        float *l_v, int *l_id, int *count) {
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int base = (tid + i * kT) * 4;
+    const float m4 = fmaxf(fmaxf(x[i].x, x[i].y), fmaxf(x[i].z, x[i].w));
+    if (m4 >= tv) {  // rare: most float4 hold nothing near the threshold
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float v = c == 0 ? x[i].x : (c == 1 ? x[i].y : (c == 2 ? x[i].z : x[i].w));
+        const int id = base + c;
+        if (id < V && !beats(tv, ti, v, id)) {
+          const int pos = atomicAdd(count, 1);
+          if (pos < kListCap) {
+            l_v[pos] = v;
+            l_id[pos] = id;
+          }
+        }
+      }
+    }
+  }
+}
+
+// Up to NV = 8 the register budget is held to 64 per thread so that two workgroups share a CU and
+// one column's selection overlaps the other's loads.
+template <int NV>
+__global__ __launch_bounds__(kT, (NV <= 8 ? 8 : 4)) void beam_topk_kernel(
+    const float *__restrict__ logits, int ldl, const float *__restrict__ bias, int V, int K,
+    int eof_id, float *__restrict__ cand_logp, int *__restrict__ cand_id,
+    float *__restrict__ logp_eof) {
   __shared__ float red[kNW];
-  __shared__ float s_v[kNW * LH_BEAM_MAX_K];
-  __shared__ int s_id[kNW * LH_BEAM_MAX_K];
+  __shared__ float s_v[kT];
+  __shared__ int s_id[kT];
+  __shared__ float q_v[kT];  // exact path: survivors, kNW * K <= kT entries
+  __shared__ int q_id[kT];
+  __shared__ float l_v[kListCap];
+  __shared__ int l_id[kListCap];
+  __shared__ int s_count, s_tau_id;
+  __shared__ float s_tau_v;
   const int b = blockIdx.x, tid = threadIdx.x;
-  const int wave = tid / lh::kWave, lane = tid % lh::kWave;
+  const int wave = tid / lh::kWave;
   float4 x[NV];
   load_column<NV>(x, logits + (size_t)b * ldl, bias, V, tid);
-  const float mx = lh::block_max<kNW>(local_max<NV>(x), red);
+  const float tmax = local_max<NV>(x);
+  const float mx = lh::block_max<kNW>(tmax, red);
   float part = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i)
-    part += (expf(x[i].x - mx) + expf(x[i].y - mx)) + (expf(x[i].z - mx) + expf(x[i].w - mx));
+    part += (exp_neg(x[i].x - mx) + exp_neg(x[i].y - mx)) + (exp_neg(x[i].z - mx) + exp_neg(x[i].w - mx));
   const float lse = logf(lh::block_sum<kNW>(part, red));
 
   if (eof_id >= 0 && eof_id < V && (eof_id / 4) % kT == tid) {
@@ -291,9 +350,30 @@ __global__ __launch_bounds__(kT) void beam_topk_kernel(const float *__restrict__
     logp_eof[b] = (z - mx) - lse;
   }
 
-  // Stage 1: every wavefront extracts the K best of its 256*NV values, best first.
-  for (int r = 0; r < K; ++r) {
-    Best me{kNegInf, kIdNone};
+  // ---- fast path: threshold from group maxima ----------------------------------------------
+  {
+    const int G = K <= 16 ? kNW : 64;
+    const int gs = kT / G;  // 64 or 16 lanes
+    float gm = tmax;
+    for (int o = gs / 2; o > 0; o >>= 1) gm = fmaxf(gm, __shfl_xor(gm, o, lh::kWave));
+    if (tid % gs == 0) s_v[tid / gs] = gm;
+    if (tid == 0) s_count = 0;
+    __syncthreads();
+    if (tid < G) {
+      const float mine = s_v[tid];
+      int rank = 0;
+      for (int q = 0; q < G; ++q) rank += (s_v[q] > mine || (s_v[q] == mine && q < tid)) ? 1 : 0;
+      if (rank == K - 1) s_tau_v = mine;
+    }
+    __syncthreads();
+    collect<NV>(x, tid, V, s_tau_v, kIdNone, l_v, l_id, &s_count);  // every element >= tau
+    __syncthreads();
+  }
+  if (s_count > kListCap) {
+    // ---- exact path ---------------------------------------------------------------------------
+    // thread best; a thread without a finite value gets a unique id above every vocabulary id so
+    // that the order stays strict
+    Best me{kNegInf, 0x40000000 + tid};
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int base = (tid + i * kT) * 4;  // ids grow with i and c: strict > keeps the lowest id
@@ -302,46 +382,56 @@ __global__ __launch_bounds__(kT) void beam_topk_kernel(const float *__restrict__
       if (x[i].z > me.v) { me.v = x[i].z; me.id = base + 2; }
       if (x[i].w > me.v) { me.v = x[i].w; me.id = base + 3; }
     }
-    const Best w = wave_argmax(me);
-    if (lane == 0) {
-      s_v[wave * K + r] = w.v;
-      s_id[wave * K + r] = w.id;
-    }
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int base = (tid + i * kT) * 4;
-      if (base + 0 == w.id) x[i].x = kNegInf;
-      if (base + 1 == w.id) x[i].y = kNegInf;
-      if (base + 2 == w.id) x[i].z = kNegInf;
-      if (base + 3 == w.id) x[i].w = kNegInf;
-    }
-  }
-  __syncthreads();
-
-  // Stage 2: wavefront 0 merges the kNW*K survivors (<= 16 per lane).
-  if (wave == 0) {
-    const int total = kNW * K;
-    float cv[kNW];
-    int ci[kNW];
-#pragma unroll
-    for (int q = 0; q < kNW; ++q) {
-      const int e = lane + q * lh::kWave;
-      cv[q] = e < total ? s_v[e] : kNegInf;
-      ci[q] = e < total ? s_id[e] : kIdNone;
-    }
-    for (int r = 0; r < K; ++r) {
-      Best me{kNegInf, kIdNone};
-#pragma unroll
-      for (int q = 0; q < kNW; ++q)
-        if (beats(cv[q], ci[q], me.v, me.id)) { me.v = cv[q]; me.id = ci[q]; }
-      const Best w = wave_argmax(me);
-      if (lane == 0) {
-        cand_logp[(size_t)b * K + r] = (w.v - mx) - lse;
-        cand_id[(size_t)b * K + r] = w.id;
+    __syncthreads();
+    s_v[tid] = me.v;
+    s_id[tid] = me.id;
+    if (tid == 0) s_count = 0;
+    __syncthreads();
+    {  // rank inside the wavefront, keep ranks < K
+      int rank = 0;
+      const int w0 = wave * lh::kWave;
+#pragma unroll 8
+      for (int q = 0; q < lh::kWave; ++q) rank += beats(s_v[w0 + q], s_id[w0 + q], me.v, me.id) ? 1 : 0;
+      if (rank < K) {
+        q_v[wave * K + rank] = me.v;
+        q_id[wave * K + rank] = me.id;
       }
-#pragma unroll
-      for (int q = 0; q < kNW; ++q)
-        if (ci[q] == w.id) cv[q] = kNegInf, ci[q] = kIdNone;
+    }
+    __syncthreads();
+    {  // the K-th best of the kNW*K survivors, comparisons of one survivor split over `parts` threads
+      const int total = kNW * K;
+      const int parts = kT / total;  // >= 1 because K <= 64
+      if (tid < total) s_id[tid] = 0;  // thread bests no longer needed: reuse as rank counters
+      __syncthreads();
+      const int e = tid / parts, p = tid - e * parts;
+      if (e < total) {
+        const float v = q_v[e];
+        const int id = q_id[e];
+        int cnt = 0;
+#pragma unroll 4
+        for (int q = p; q < total; q += parts) cnt += beats(q_v[q], q_id[q], v, id) ? 1 : 0;
+        if (cnt) atomicAdd(&s_id[e], cnt);
+      }
+      __syncthreads();
+      if (tid < total && s_id[tid] == K - 1) {
+        s_tau_v = q_v[tid];
+        s_tau_id = q_id[tid];
+      }
+    }
+    __syncthreads();
+    collect<NV>(x, tid, V, s_tau_v, s_tau_id, l_v, l_id, &s_count);
+    __syncthreads();
+  }
+  const int n = s_count < kListCap ? s_count : kListCap;
+  for (int e = tid; e < n; e += kT) {
+    const float v = l_v[e];
+    const int id = l_id[e];
+    int rank = 0;
+#pragma unroll 4
+    for (int q = 0; q < n; ++q) rank += beats(l_v[q], l_id[q], v, id) ? 1 : 0;
+    if (rank < K) {
+      cand_logp[(size_t)b * K + rank] = (v - mx) - lse;
+      cand_id[(size_t)b * K + rank] = id;
     }
   }
 }
@@ -443,7 +533,7 @@ extern "C" int lh_logsoftmax_xent_f32(const float *logits, int ldl, const float 
   }
   int rc = lh::check_launch("lh_logsoftmax_xent_f32");
   if (rc != LH_OK) return rc;
-  hipLaunchKernelGGL(masked_sum_kernel, dim3(1), dim3(64), 0, st, logp_tgt, mask01, B, loss_accum);
+  hipLaunchKernelGGL(masked_sum_kernel, dim3(1), dim3(kT), 0, st, logp_tgt, mask01, B, loss_accum);
   return lh::check_launch("lh_logsoftmax_xent_f32 (sum)");
 }
 
@@ -468,7 +558,7 @@ extern "C" int lh_softmax_xent_grad_f32(const float *logits, int ldl, const floa
   }
   int rc = lh::check_launch("lh_softmax_xent_grad_f32");
   if (rc != LH_OK) return rc;
-  hipLaunchKernelGGL(masked_sum_kernel, dim3(1), dim3(64), 0, st, logp_tgt, mask01, B, loss_accum);
+  hipLaunchKernelGGL(masked_sum_kernel, dim3(1), dim3(kT), 0, st, logp_tgt, mask01, B, loss_accum);
   return lh::check_launch("lh_softmax_xent_grad_f32 (sum)");
 }
 

@@ -410,6 +410,32 @@ def test_beam_topk_ties_take_lowest_id(lh):
     assert_close(host(cl, (K, B))[:, 0], np.full(K, -np.log(V)), "uniform log-prob")
 
 
+@pytest.mark.parametrize("V,K", [(30000, 13), (50000, 64), (5000, 13), (300, 64), (37, 5)])
+def test_beam_topk_adversarial_layouts(lh, V, K):
+    """Layouts that stress the selection: the winners packed into the rows one thread owns (ids
+    congruent modulo 4096), winners spread one per thread, long runs of exact ties, tiny
+    vocabularies.  Expected = full sort by (value desc, id asc)."""
+    rng = np.random.default_rng(77)
+    B = 6
+    z = uni(rng, V, B, s=1.0)
+    own = np.array([i for i in range(V) if (i // 4) % 1024 == 3])      # rows of one thread
+    z[own[: min(len(own), 40)], 0] += 10.0
+    z[rng.permutation(V)[: min(V, 200)], 1] += 10.0
+    z[:, 2] = np.round(z[:, 2] * 4) / 4                                    # heavy ties
+    z[:, 3] = 0.25                                                         # everything ties
+    z[own[: min(len(own), 20)], 4] = 5.0                                   # tied winners in one thread
+    cl = torch.empty(K * B, device="cuda")
+    ci = torch.empty(K * B, dtype=torch.int32, device="cuda")
+    le = torch.empty(B, device="cuda")
+    lh.beam_topk(dev(z), V, None, V, B, K, 1, cl, ci, le)
+    gi, gl = host(ci, (K, B)), host(cl, (K, B))
+    lse = scipy.special.logsumexp(z.astype(np.float64), axis=0)
+    for b in range(B):
+        order = np.lexsort((np.arange(V), -z[:, b]))[:K]
+        assert gi[:, b].tolist() == order.tolist(), f"column {b}"
+        assert_close(gl[:, b], z[order, b] - lse[b], f"log-probs of column {b}", atol=2e-5)
+
+
 def test_beam_gather(lh, orc):
     rng = np.random.default_rng(10)
     H, B, n = 1000, 768, 9
