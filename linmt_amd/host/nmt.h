@@ -84,6 +84,7 @@ class LstmNode {
 
   // buffers owned by the layer, one slice per node
   float *p_device_sparse_lookup_ = nullptr;  // layer 1: E x B embedding columns
+  float *p_device_pre_x_ = nullptr;  // 4H x B: M*x of this step when the layer computed it for all steps
   float *p_device_gates_ = nullptr;          // 4H x B: i_t, f_t, c_prime_t_tanh, o_t (NULL when not kept)
   float *p_device_c_t_ = nullptr;
   float *p_device_h_t_ = nullptr;
@@ -141,6 +142,17 @@ class LstmLayer {
   // activations
   DeviceArray<float> p_device_init_hidden_vec_, p_device_init_cell_vec_;  // zeros
   DeviceArray<float> h_all_, c_all_, gates_all_, lookup_all_, preact_;
+  // Input products hoisted off the recurrence.  Whenever every step's input is known before the
+  // recurrence starts (the whole source side, run layer by layer; the teacher-forced target input
+  // layer), M*[x_0 .. x_{T-1}] is ONE GEMM over B*T columns into pre_x_all_ and a step only adds
+  // W_h*h_{t-1} (+ Q*h~_{t-1}).  When decoding, the target input layer reads M*W[:,token] from the
+  // precomputed 4H x V product mw_fold_ instead (a 4H-row "embedding" lookup).
+  DeviceArray<float> pre_x_all_, mw_fold_;
+  bool input_hoistable_ = false;  // buffers exist
+  bool input_hoisted_ = false;    // this pass uses them
+  bool mw_fold_dirty_ = true;
+  void ForwardPropInputAllSteps(int steps);
+  void BuildEmbeddingFold();
   DeviceArray<float> p_device_h_t_previous_, p_device_c_t_previous_;  // decode: PreviousTargetState
   DeviceArray<int> p_device_input_vocab_indices_full_, p_device_input_vocab_indices_01_full_;
   std::vector<LstmNode> v_nodes_;
@@ -415,6 +427,7 @@ class NeuralMachineTranslation {
  private:
   // encoder + decoder + attention of a teacher-forced minibatch (shared by GetError and
   // ComputeGradients); per_step_loss: also run the loss of every step as GetError does.
+  void RunSourceSide(int source_length, int minibatch_size);
   void ForwardTeacherForced(const int *p_host_source, int source_length,
                             const int *p_host_target_in, const int *p_host_target_out,
                             int target_length, const int *p_host_batch_information,

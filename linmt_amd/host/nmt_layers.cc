@@ -81,7 +81,12 @@ void LstmLayer::Init(NeuralMachineTranslation *model, bool input_layer, bool sou
   h_all_.Alloc(H * B * num_nodes);
   c_all_.Alloc(H * B * num_nodes);
   if (keep_gates) gates_all_.Alloc(4 * H * B * num_nodes);
-  if (input_layer) lookup_all_.Alloc((size_t)input_size_ * B * (keep_gates ? num_nodes : 1));
+  // every step's input is known up front on the source side and for the teacher-forced target
+  // input layer (num_nodes > 1); a decoding target layer has a single node
+  input_hoistable_ = num_nodes > 1 && (source_side || input_layer);
+  if (input_layer)
+    lookup_all_.Alloc((size_t)input_size_ * B * (keep_gates || input_hoistable_ ? num_nodes : 1));
+  if (input_hoistable_) pre_x_all_.Alloc(4 * H * B * num_nodes);
   preact_.Alloc(4 * H * B);
   if (with_previous_state) {
     p_device_h_t_previous_.Alloc(H * B);
@@ -100,7 +105,9 @@ void LstmLayer::Init(NeuralMachineTranslation *model, bool input_layer, bool sou
     n.p_device_c_t_ = c_all_.get() + H * B * i;
     n.p_device_gates_ = keep_gates ? gates_all_.get() + 4 * H * B * i : nullptr;
     if (input_layer)
-      n.p_device_sparse_lookup_ = lookup_all_.get() + (keep_gates ? (size_t)input_size_ * B * i : 0);
+      n.p_device_sparse_lookup_ =
+          lookup_all_.get() + (keep_gates || input_hoistable_ ? (size_t)input_size_ * B * i : 0);
+    if (input_hoistable_) n.p_device_pre_x_ = pre_x_all_.get() + 4 * H * B * i;
   }
   if (cfg.train_mode_ && keep_gates) InitTraining();
 }
@@ -132,6 +139,7 @@ void LstmLayer::PreprocessGpuVocabIndices(const int *p_host_input_vocab_indices,
 bool LstmLayer::SetParam(const std::string &name, const float *host, size_t n) {
   hipStream_t s = p_neural_mt_->stream_;
   const int H = lstm_size_;
+  if (name == "W" || name[0] == 'M') mw_fold_dirty_ = true;
   if (name == "W") return input_layer_mode_ && SetFlat(p_device_w_, host, n, s);
   if (name.size() == 3 && name[0] == 'M' && name[1] == '_') {
     const int g = GateIndex(name[2]);
@@ -208,35 +216,52 @@ void LstmNode::ForwardProp() {
   NeuralMachineTranslation &M = *L.p_neural_mt_;
   hipStream_t s = M.stream_;
   const int H = L.lstm_size_, B = minibatch_size_;
-  const float *x = nullptr;
-  if (L.input_layer_mode_) {
-    const bool drop = M.apply_dropout_ && p_device_dropout_mask_;
-    ProfileScope ps(M.profiler_, kTagEmbedLookup, (drop ? 12.0 : 8.0) * L.input_size_ * B);
-    LhErrorWrapper(lh_embed_lookup_f32(L.p_device_w_.get(), L.input_size_, L.vocab_size_,
-                                       p_device_input_vocab_indices_, B,
-                                       drop ? p_device_dropout_mask_ : nullptr,
-                                       drop ? M.cfg_.dropout_rate_ : 1.f, p_device_sparse_lookup_, s),
-                   "LstmInputHiddenNode::ForwardPropGpu sparse lookup");
-    x = p_device_sparse_lookup_;
-  } else {
-    x = p_device_h_t_below_;
-  }
   // feed input only from the second target step on (node_input_to_hidden.h:325)
   const bool feed = L.feed_input_mode_ && 0 != index_;
+  const bool folded = M.decode_mode_ && L.input_layer_mode_ && !L.source_side_mode_;
+  float *pre = L.preact_.get();
   lh_gemm_seg segs[3];
   int nseg = 0;
-  segs[nseg++] = {L.p_device_m_stack_.get(), 4 * H, x, L.input_size_, L.input_size_};
+  float beta = 0.f;
+  if (L.input_hoisted_) {
+    // M*x of every step is already in pre_x_all_: this step only adds the recurrent products
+    pre = p_device_pre_x_;
+    beta = 1.f;
+  } else if (folded) {
+    // M*W[:,token] is a column of the precomputed 4H x V product
+    if (L.mw_fold_dirty_) L.BuildEmbeddingFold();
+    ProfileScope ps(M.profiler_, kTagEmbedLookup, 8.0 * 4 * H * B);
+    LhErrorWrapper(lh_embed_lookup_f32(L.mw_fold_.get(), 4 * H, L.vocab_size_,
+                                       p_device_input_vocab_indices_, B, nullptr, 1.f, pre, s),
+                   "LstmInputHiddenNode::ForwardPropGpu folded lookup");
+    beta = 1.f;
+  } else {
+    const float *x = nullptr;
+    if (L.input_layer_mode_) {
+      const bool drop = M.apply_dropout_ && p_device_dropout_mask_;
+      ProfileScope ps(M.profiler_, kTagEmbedLookup, (drop ? 12.0 : 8.0) * L.input_size_ * B);
+      LhErrorWrapper(lh_embed_lookup_f32(L.p_device_w_.get(), L.input_size_, L.vocab_size_,
+                                         p_device_input_vocab_indices_, B,
+                                         drop ? p_device_dropout_mask_ : nullptr,
+                                         drop ? M.cfg_.dropout_rate_ : 1.f, p_device_sparse_lookup_, s),
+                     "LstmInputHiddenNode::ForwardPropGpu sparse lookup");
+      x = p_device_sparse_lookup_;
+    } else {
+      x = p_device_h_t_below_;
+    }
+    segs[nseg++] = {L.p_device_m_stack_.get(), 4 * H, x, L.input_size_, L.input_size_};
+  }
   segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
   if (feed) segs[nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
   {
     ProfileScope ps(M.profiler_, kTagGateGemm, 4 * H, B, segs, nseg, 0, 0);
-    LhErrorWrapper(lh_gemm_f32(4 * H, B, segs, nseg, 0, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
-                             L.preact_.get(), 4 * H, s),
-                 "LstmNode::ForwardPropGpu stacked gate product");
+    LhErrorWrapper(lh_gemm_f32(4 * H, B, segs, nseg, 0, 0, 1.f, beta, nullptr, LH_ACT_NONE, nullptr,
+                               pre, 4 * H, s),
+                   "LstmNode::ForwardPropGpu stacked gate product");
   }
   const bool drop_out = M.apply_dropout_ && L.out_dropout_;
   ProfileScope pc(M.profiler_, kTagLstmCell, ((p_device_gates_ ? 44.0 : 28.0) + (drop_out ? 8.0 : 0.0)) * H * B);
-  LhErrorWrapper(lh_lstm_cell_fwd_f32(H, B, L.preact_.get(), nullptr, nullptr,
+  LhErrorWrapper(lh_lstm_cell_fwd_f32(H, B, pre, nullptr, nullptr,
                                       L.p_device_b_stack_.get(), p_device_c_t_prev_,
                                       p_device_input_vocab_indices_01_, feed ? 1 : 0,
                                       M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f,
@@ -245,6 +270,44 @@ void LstmNode::ForwardProp() {
                                       drop_out ? M.cfg_.dropout_rate_ : 1.f,
                                       drop_out ? p_device_h_t_dropped_ : nullptr, s),
                  "LstmNode::ForwardPropGpu fused cell");
+}
+
+// M*[x_0 .. x_{steps-1}] in one GEMM (input layer: after ONE lookup of all steps' embeddings).
+// Needs the node slices to be contiguous, i.e. the pass must use every allocated column.
+void LstmLayer::ForwardPropInputAllSteps(int steps) {
+  NeuralMachineTranslation &M = *p_neural_mt_;
+  hipStream_t s = M.stream_;
+  const int H = lstm_size_, N = minibatch_size_ * steps;
+  const float *x_all = nullptr;
+  if (input_layer_mode_) {
+    const bool drop = M.apply_dropout_ && dropout_mask_all_.size();
+    ProfileScope ps(M.profiler_, kTagEmbedLookup, (drop ? 12.0 : 8.0) * input_size_ * N);
+    LhErrorWrapper(lh_embed_lookup_f32(p_device_w_.get(), input_size_, vocab_size_,
+                                       p_device_input_vocab_indices_full_.get(), N,
+                                       drop ? dropout_mask_all_.get() : nullptr,
+                                       drop ? M.cfg_.dropout_rate_ : 1.f, lookup_all_.get(), s),
+                   "InputToHiddenLayer sparse lookup, all steps");
+    x_all = lookup_all_.get();
+  } else {
+    x_all = v_nodes_[0].p_device_h_t_below_;
+  }
+  lh_gemm_seg seg{p_device_m_stack_.get(), 4 * H, x_all, input_size_, input_size_};
+  ProfileScope ps(M.profiler_, kTagGateGemm, 4 * H, N, &seg, 1, 0, 0);
+  LhErrorWrapper(lh_gemm_f32(4 * H, N, &seg, 1, 0, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
+                             pre_x_all_.get(), 4 * H, s),
+                 "LstmLayer input products, all steps");
+}
+
+// mw_fold_ = M_stack * W (4H x V): the input product of every vocabulary entry, for decoding.
+void LstmLayer::BuildEmbeddingFold() {
+  NeuralMachineTranslation &M = *p_neural_mt_;
+  const int H = lstm_size_;
+  if (mw_fold_.size() == 0) mw_fold_.Alloc((size_t)4 * H * vocab_size_);
+  lh_gemm_seg seg{p_device_m_stack_.get(), 4 * H, p_device_w_.get(), input_size_, input_size_};
+  LhErrorWrapper(lh_gemm_f32(4 * H, vocab_size_, &seg, 1, 0, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
+                             mw_fold_.get(), 4 * H, M.stream_),
+                 "LstmLayer embedding fold");
+  mw_fold_dirty_ = false;
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -194,25 +194,11 @@ void NeuralMachineTranslation::ForwardTeacherForced(const int *p_host_source, in
   }
   softmax_layer_.p_device_loss_.Zero(stream_);
 
-  if (seq2seq) {
-    for (int t = 0; t < source_length; ++t) {
-      const size_t step = (size_t)t * B;
-      for (int l = 0; l < L; ++l) {
-        LstmLayer &Ls = SourceLayer(l);
-        LstmNode &n = Ls.v_nodes_[t];
-        n.minibatch_size_ = B;
-        float *hp = t == 0 ? Ls.p_device_init_hidden_vec_.get() : Ls.v_nodes_[t - 1].p_device_h_t_;
-        float *cp = t == 0 ? Ls.p_device_init_cell_vec_.get() : Ls.v_nodes_[t - 1].p_device_c_t_;
-        if (l == 0)
-          n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_full_.get() + step,
-                                    Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
-        else {
-          n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
-          n.p_device_h_t_below_ = UpwardState(SourceLayer(l - 1), t);
-        }
-        n.ForwardProp();
-      }
-    }
+  if (seq2seq) RunSourceSide(source_length, B);
+  {
+    LstmLayer &L0 = input_layer_target_;
+    L0.input_hoisted_ = L0.input_hoistable_ && B == L0.minibatch_size_;
+    if (L0.input_hoisted_) L0.ForwardPropInputAllSteps(target_length);
   }
   for (int t = 0; t < target_length; ++t) {
     const size_t step = (size_t)t * B;
@@ -277,21 +263,33 @@ void NeuralMachineTranslation::ForwardPropSource(const int *p_host_source, int s
                                                  int n_sent) {
   const int L = cfg_.num_layers_;
   for (int l = 0; l < L; ++l) SourceLayer(l).PreprocessGpuVocabIndices(p_host_source, source_length, n_sent);
-  for (int t = 0; t < source_length; ++t) {
-    const size_t step = (size_t)t * n_sent;
-    for (int l = 0; l < L; ++l) {
-      LstmLayer &Ls = SourceLayer(l);
+  RunSourceSide(source_length, n_sent);
+}
+
+// The source side has no coupling from a layer's step t to the layer above's step t-1, so it runs
+// one layer at a time: the layer's input products for all steps in one GEMM, then the recurrence.
+void NeuralMachineTranslation::RunSourceSide(int source_length, int B) {
+  const int L = cfg_.num_layers_;
+  for (int l = 0; l < L; ++l) {
+    LstmLayer &Ls = SourceLayer(l);
+    for (int t = 0; t < source_length; ++t) {
+      const size_t step = (size_t)t * B;
       LstmNode &n = Ls.v_nodes_[t];
-      n.minibatch_size_ = n_sent;
+      n.minibatch_size_ = B;
       float *hp = t == 0 ? Ls.p_device_init_hidden_vec_.get() : Ls.v_nodes_[t - 1].p_device_h_t_;
       float *cp = t == 0 ? Ls.p_device_init_cell_vec_.get() : Ls.v_nodes_[t - 1].p_device_c_t_;
-      if (l == 0)
+      if (l == 0) {
         n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_full_.get() + step,
                                   Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
-      else
+      } else {
         n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
-      n.ForwardProp();
+        n.p_device_h_t_below_ = UpwardState(SourceLayer(l - 1), t);
+      }
     }
+    // the hoisted GEMM reads / writes the node slices as one matrix: every allocated column in use
+    Ls.input_hoisted_ = Ls.input_hoistable_ && B == Ls.minibatch_size_;
+    if (Ls.input_hoisted_) Ls.ForwardPropInputAllSteps(source_length);
+    for (int t = 0; t < source_length; ++t) Ls.v_nodes_[t].ForwardProp();
   }
 }
 
