@@ -30,6 +30,7 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
   __shared__ int s_id[kMaxCand];
   __shared__ short s_col[kMaxCand];
   __shared__ short s_order[kMaxCand];
+  __shared__ unsigned char s_flag[kMaxCand];
 
   const int s = blockIdx.x, tid = threadIdx.x;
   const int beam = a.beam, K = a.K;
@@ -63,37 +64,57 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
     s_col[e] = (short)i;
   }
   __syncthreads();
+  // rank of every candidate in the total order; s_order[rank] = candidate, s_flag[rank] = what the
+  // walk does with it (1 takes a slot, 2 finished hypothesis, 0 dropped <START>)
   for (int e = tid; e < C; e += kMergeThreads) {
     const float sc = s_score[e];
     const int id = s_id[e], col = s_col[e];
     int before = 0;
+#pragma unroll 4
     for (int o = 0; o < C; ++o) {
       const float so = s_score[o];
       const bool first = so > sc || (so == sc && (s_col[o] < col || (s_col[o] == col && s_id[o] < id)));
       before += first ? 1 : 0;
     }
     s_order[before] = (short)e;
+    s_flag[before] = id == a.start_id ? 0 : (id == a.eof_id ? 2 : 1);
   }
   __syncthreads();
+  // The reference pops the global heap until `beam` slots are filled.  Entry r is reached iff fewer
+  // than `beam` slot-taking entries precede it; its slot / finished index is the count of such
+  // entries before it -- a prefix count every thread takes for its own entries, so nothing walks
+  // the list serially.
+  for (int r = tid; r < C; r += kMergeThreads) {
+    int slots = 0, fins = 0;
+#pragma unroll 4
+    for (int q = 0; q < r; ++q) {
+      const int f = s_flag[q];
+      slots += f == 1 ? 1 : 0;
+      fins += f == 2 ? 1 : 0;
+    }
+    const int f = s_flag[r];
+    if (slots < beam && f != 0) {
+      const int e = s_order[r];
+      const float sc = s_score[e] + a.penalty;
+      if (f == 2) {
+        if (fins < beam) {  // at most one <EOF> candidate per column exists
+          a.fin_beam[c0 + fins] = s_col[e];
+          a.fin_score[c0 + fins] = sc;
+        }
+      } else {
+        a.tok[c0 + slots] = s_id[e];
+        a.backptr[c0 + slots] = c0 + s_col[e];
+        a.score[c0 + slots] = sc;
+      }
+    }
+  }
   if (tid == 0) {
+    // totals: slots filled (the rest is padding) and finished hypotheses recorded
     int filled = 0, nfin = 0;
     for (int r = 0; r < C && filled < beam; ++r) {
-      const int e = s_order[r];
-      const int id = s_id[e];
-      if (id == a.start_id) continue;
-      const float sc = s_score[e] + a.penalty;
-      if (id == a.eof_id) {
-        if (nfin < beam) {  // at most one <EOF> candidate per column exists
-          a.fin_beam[c0 + nfin] = s_col[e];
-          a.fin_score[c0 + nfin] = sc;
-          ++nfin;
-        }
-        continue;
-      }
-      a.tok[c0 + filled] = id;
-      a.backptr[c0 + filled] = c0 + s_col[e];
-      a.score[c0 + filled] = sc;
-      ++filled;
+      const int f = s_flag[r];
+      filled += f == 1 ? 1 : 0;
+      nfin += (f == 2 && nfin < beam) ? 1 : 0;
     }
     for (; filled < beam; ++filled) {  // candidates exhausted (the reference pops an empty heap)
       a.tok[c0 + filled] = a.eof_id;

@@ -487,6 +487,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   int cur = 0;
   std::vector<int> active_at(max_limit + 1);
   std::vector<std::vector<int>> bi_keep;
+  int *p_device_step_indices = d.current_indices_.get();  // <START> for every column
   for (int step = 0; step <= max_limit; ++step) {
     int n_active = 0;
     while (n_active < n && limit[n_active] >= step) ++n_active;  // limits are non-increasing
@@ -503,7 +504,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
       }
       attention_layer_.PreprocessMinibatchInformation(bi.data(), Ba);
     }
-    ForwardPropTarget(step, d.current_indices_.get(), Ba);
+    ForwardPropTarget(step, p_device_step_indices, Ba);
     {
       ProfileScope ps(profiler_, kTagBeamTopK, 4.0 * cfg_.target_vocab_size_ * Ba);
       LhErrorWrapper(lh_beam_topk_f32(softmax_layer_.GetDistPtr(), cfg_.target_vocab_size_, nullptr,
@@ -512,21 +513,22 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
                    "beam top-k");
     }
     const size_t off = (size_t)step * B;
-    ProfileScope pm(profiler_, kTagBeamMerge, 8.0 * K * Ba);
-    LhErrorWrapper(
-        lh_beam_merge_f32(n_active, beam, K, step, d.limit_.get(), d.cand_logp_.get(),
-                          d.cand_id_.get(), d.logp_eof_.get(), d.score_[cur].get(), o.diversity_,
-                          o.penalty_, Decoder::start_symbol_, Decoder::end_symbol_,
-                          d.tok_hist_.get() + off, d.backptr_hist_.get() + off,
-                          d.score_[cur ^ 1].get(), d.fin_count_hist_.get() + (size_t)step * n,
-                          d.fin_beam_hist_.get() + off, d.fin_score_hist_.get() + off, stream_),
-        "beam merge");
+    {
+      ProfileScope pm(profiler_, kTagBeamMerge, 8.0 * K * Ba);
+      LhErrorWrapper(
+          lh_beam_merge_f32(n_active, beam, K, step, d.limit_.get(), d.cand_logp_.get(),
+                            d.cand_id_.get(), d.logp_eof_.get(), d.score_[cur].get(), o.diversity_,
+                            o.penalty_, Decoder::start_symbol_, Decoder::end_symbol_,
+                            d.tok_hist_.get() + off, d.backptr_hist_.get() + off,
+                            d.score_[cur ^ 1].get(), d.fin_count_hist_.get() + (size_t)step * n,
+                            d.fin_beam_hist_.get() + off, d.fin_score_hist_.get() + off, stream_),
+          "beam merge");
+    }
     cur ^= 1;
     if (step < max_limit) {
       SwapDecodingStates(d.backptr_hist_.get() + off, Ba);
-      HipErrorWrapper(hipMemcpyAsync(d.current_indices_.get(), d.tok_hist_.get() + off,
-                                     sizeof(int) * Ba, hipMemcpyDeviceToDevice, stream_),
-                      "current indices copy");
+      // the tokens just chosen are the next step's input ids, read in place from the history
+      p_device_step_indices = d.tok_hist_.get() + off;
     }
   }
 
