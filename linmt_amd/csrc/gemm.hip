@@ -153,7 +153,7 @@ constexpr int smem_floats() {
 extern __shared__ __attribute__((aligned(16))) float smem[];
 
 template <int BM, int BN, int WM, int WN, int WK, int BK, bool TA, bool TX, bool VEC>
-__global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(64 * WM * WN * WK) void gemm_generic_kernel(const GemmArgs g) {
   constexpr int NT = 64 * WM * WN * WK;
   constexpr int TM = BM / WM, TN = BN / WN;
   constexpr int FM = TM / 32, FN = TN / 32;
@@ -287,7 +287,345 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
   }
 
   // Epilogue: accumulator register j of lane l is C[m = .. + l%32][n = .. + 8*(j/4) + 4*(l/32) + j%4].
+  // Everything the epilogue reads (old C for beta, the column mask, the bias) is fetched for a whole
+  // 32x32 accumulator tile with independent loads before any of it is used, so the loads of one tile
+  // overlap instead of costing one memory round trip each.
   const float alpha = g.alpha, beta = g.beta;
+  const bool use_beta = beta != 0.f;
+  const int *const colmask = g.colmask;
+#pragma unroll
+  for (int a = 0; a < FN; ++a) {
+#pragma unroll
+    for (int b = 0; b < FM; ++b) {
+      const int m = m0 + wm * TM + b * 32 + l32;
+      const bool m_ok = m < g.M;
+      const int mc = m_ok ? m : 0;
+      const float bv = g.bias ? g.bias[mc] : 0.f;
+      const bool do_tanh = g.act == LH_ACT_TANH && m < g.act_rows;
+      const int nb = n0 + wn * TN + a * 32 + lhi * 4;
+      if constexpr (BM * BN <= 32 * 64) {
+        // Small tiles run with few workgroups per CU, where a serial chain of loads in the epilogue
+        // is a visible part of the launch: fetch four columns' worth before using any.
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float old[4], cm[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int n = nb + q * 8 + r;
+            const int nc = n < g.N ? n : 0;
+            old[r] = use_beta ? g.C[(size_t)nc * g.ldc + mc] : 0.f;
+            cm[r] = colmask ? (float)colmask[nc] : 1.f;
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int n = nb + q * 8 + r;
+            float v = alpha * acc[a][b][q * 4 + r];
+            if (use_beta) v += beta * old[r];
+            v += bv;
+            if (do_tanh) v = tanhf(v);
+            if (colmask) v *= cm[r];
+            if (m_ok && n < g.N) g.C[(size_t)n * g.ldc + m] = v;
+          }
+        }
+      } else {
+        // Large tiles: many workgroups share a CU and hide each other's epilogue; keep the register
+        // footprint (and with it the number of resident workgroups) minimal.
+        if (!m_ok) continue;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int n = nb + (j / 4) * 8 + (j % 4);
+          if (n >= g.N) continue;
+          float *cp = g.C + (size_t)n * g.ldc + m;
+          float v = alpha * acc[a][b][j];
+          if (use_beta) v += beta * *cp;
+          v += bv;
+          if (do_tanh) v = tanhf(v);
+          if (colmask) v *= (float)colmask[n];
+          *cp = v;
+        }
+      }
+    }
+  }
+}
+
+
+// =============================================================================================
+// Main kernel (16-byte aligned operands).  What shapes it:
+//   * On CDNA a VALU instruction and an MFMA do not overlap inside a SIMD: every non-MFMA vector
+//     instruction in the loop costs about four cycles of matrix-pipe time.  The loop therefore
+//     carries almost none.  Global addresses are a uniform base (scalar registers) plus
+//     per-thread 32-bit byte offsets computed once per K segment; bounds along M / N are folded
+//     into those offsets (out-of-range rows re-read the tile origin: they only feed rows and
+//     columns of C that are never written); the K tail of a segment, one slab at most, is the only
+//     place that masks data.  Staging is 16-byte copies global -> registers -> LDS with no
+//     shuffling, for either memory order:
+//   * an operand that is contiguous along k in memory lives in LDS as [k/4][d][4], and an MFMA
+//     operand fragment for four k-steps is one ds_read_b128 per lane;
+//   * an operand that is contiguous along d lives in LDS as [k][d], and a fragment is one
+//     ds_read_b32 per k-step.
+//     In both, lanes 0-31 take k = 8g+q and lanes 32-63 k = 8g+4+q for step q of group g: the K
+//     order inside a slab is a fixed permutation applied to both operands, which leaves the dot
+//     products unchanged.
+__device__ __forceinline__ float4 keep_if(float4 w, bool c) {
+  // per component: a select between two float4 objects makes the compiler pick an address
+  w.x = c ? w.x : 0.f;
+  w.y = c ? w.y : 0.f;
+  w.z = c ? w.z : 0.f;
+  w.w = c ? w.w : 0.f;
+  return w;
+}
+
+template <int BD, int BK, int NT, bool KC>
+struct Stage {
+  static constexpr int KQ = BK / 4;
+  // KC: 16-byte units per k-quad row.  Consecutive lanes of a staging store walk k-quads first, so
+  // the row stride is chosen to spread 16 lanes over the 16 bank groups.
+  static constexpr int LDQ = BD + (KQ >= 16 ? 1 : 16 / KQ);
+  // !KC: floats per k row; = 8 mod 16 puts the two lane halves of a fragment read (4 rows apart)
+  // on opposite halves of the banks.
+  static constexpr int LDD = BD + 8;
+  static constexpr int kFloats = KC ? KQ * LDQ * 4 : BK * LDD;
+  static constexpr int kUnits = KQ * BD;  // 16-byte units in a slab
+  static constexpr int NU = (kUnits + NT - 1) / NT;
+  static_assert(NU <= 32, "validity mask is 32 bits");
+  static_assert(BD % 16 == 0 && BK % 16 == 0, "tile extents");
+
+  float4 v[NU];
+  unsigned goff[NU];  // byte offset of each unit from the slab origin
+  unsigned ok;        // K-tail validity, one bit per unit
+
+  // unit u of the slab: (d, k) of its first element and its float offset in LDS
+  static __device__ __forceinline__ int unit_d(int u) { return KC ? u / KQ : (u % (BD / 4)) * 4; }
+  static __device__ __forceinline__ int unit_k(int u) { return KC ? (u % KQ) * 4 : u / (BD / 4); }
+  static __device__ __forceinline__ int unit_lds(int u) {
+    return KC ? ((u % KQ) * LDQ + u / KQ) * 4 : (u / (BD / 4)) * LDD + (u % (BD / 4)) * 4;
+  }
+  // dn = rows/columns of the operand that exist from the tile origin on
+  __device__ __forceinline__ void set_ld(int ld, int tid, int dn) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int u = tid + i * NT;
+      const int d = unit_d(u), k = unit_k(u);
+      const unsigned off = KC ? (unsigned)(d * ld + k) * 4u : (unsigned)(k * ld + d) * 4u;
+      goff[i] = d < dn ? off : 0u;
+    }
+  }
+  // kn (< BK) = k values left in the segment: units past it re-read the slab origin and are
+  // zeroed before they reach LDS.
+  __device__ __forceinline__ void clamp_tail(int tid, int kn) {
+    ok = 0u;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const bool in = unit_k(tid + i * NT) < kn;
+      goff[i] = in ? goff[i] : 0u;
+      ok |= in ? (1u << i) : 0u;
+    }
+  }
+  __device__ __forceinline__ void load(const float *__restrict__ base, int tid) {
+    const char *b = reinterpret_cast<const char *>(base);
+#pragma unroll
+    for (int i = 0; i < NU; ++i)
+      if (tid + i * NT < kUnits) v[i] = *reinterpret_cast<const float4 *>(b + goff[i]);
+  }
+  __device__ __forceinline__ void zero_tail() {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) v[i] = keep_if(v[i], (ok >> i) & 1u);
+  }
+  __device__ __forceinline__ void store(float *__restrict__ buf, int tid) const {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int u = tid + i * NT;
+      if (u < kUnits) *reinterpret_cast<float4 *>(buf + unit_lds(u)) = v[i];
+    }
+  }
+  // Fragment reads.  origin = float offset for (first k of the wavefront's share, lane half, row d).
+  static __device__ __forceinline__ int frag_origin(int k0, int lhi, int d) {
+    return KC ? ((k0 / 4 + lhi) * LDQ + d) * 4 : (k0 + 4 * lhi) * LDD + d;
+  }
+  static __device__ __forceinline__ void read_frag(const float *__restrict__ origin, int grp,
+                                                   int frag, float (&out)[4]) {
+    if constexpr (KC) {
+      const float4 t =
+          *reinterpret_cast<const float4 *>(origin + (2 * grp * LDQ + frag * 32) * 4);
+      out[0] = t.x, out[1] = t.y, out[2] = t.z, out[3] = t.w;
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) out[q] = origin[(8 * grp + q) * LDD + frag * 32];
+    }
+  }
+};
+
+template <int BM, int BN, int WM, int WN, int WK, int BK, bool TA, bool TX>
+constexpr int smem2_floats() {
+  constexpr int NT = 64 * WM * WN * WK;
+  return cmax(2 * (Stage<BM, BK, NT, TA>::kFloats + Stage<BN, BK, NT, !TX>::kFloats),
+              (WK - 1) * BM * BN);
+}
+
+template <int BM, int BN, int WM, int WN, int WK, int BK, bool TA, bool TX>
+__global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs g) {
+  constexpr int NT = 64 * WM * WN * WK;
+  constexpr int TM = BM / WM, TN = BN / WN;
+  constexpr int FM = TM / 32, FN = TN / 32;
+  static_assert(FM >= 1 && FN >= 1 && TM % 32 == 0 && TN % 32 == 0, "wave tile = 32x32 MFMA tiles");
+  constexpr int KPW = BK / WK;  // k values one wavefront group consumes per slab
+  static_assert(KPW % 8 == 0, "a fragment group covers 8 k (4 per lane half)");
+  constexpr int NG = KPW / 8;
+  using SA = Stage<BM, BK, NT, TA>;
+  using SX = Stage<BN, BK, NT, !TX>;
+  constexpr int kAF = SA::kFloats, kSlab = SA::kFloats + SX::kFloats;
+  static_assert(smem2_floats<BM, BN, WM, WN, WK, BK, TA, TX>() * 4 <= 160 * 1024,
+                "LDS capacity of a CU");
+
+  // XCD-aware tile assignment.
+  const int nwg = gridDim.x, id = blockIdx.x;
+  const int xcd = id % 8, within = id / 8;
+  const int per = nwg / 8, rem = nwg % 8;
+  const int logical = xcd * per + (xcd < rem ? xcd : rem) + within;
+  const int m0 = (logical / g.tiles_n) * BM;
+  const int n0 = (logical % g.tiles_n) * BN;
+
+  const int tid = threadIdx.x;
+  const int wave = tid / lh::kWave, lane = tid % lh::kWave;
+  const int wk = wave / (WM * WN), wmn = wave % (WM * WN);
+  const int wm = wmn % WM, wn = wmn / WM;
+  const int l32 = lane % 32, lhi = lane / 32;
+
+  floatx16 acc[FN][FM];
+#pragma unroll
+  for (int a = 0; a < FN; ++a)
+#pragma unroll
+    for (int b = 0; b < FM; ++b)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[a][b][j] = 0.f;
+
+  SA sa;
+  SX sx;
+  const int fa_off = SA::frag_origin(wk * KPW, lhi, wm * TM + l32);
+  const int fx_off = kAF + SX::frag_origin(wk * KPW, lhi, wn * TN + l32);
+
+  const float *const A0 = g.A[0], *const A1 = g.A[1], *const A2 = g.A[2];
+  const float *const X0 = g.X[0], *const X1 = g.X[1], *const X2 = g.X[2];
+  const int lda0 = g.lda[0], lda1 = g.lda[1], lda2 = g.lda[2];
+  const int ldx0 = g.ldx[0], ldx1 = g.ldx[1], ldx2 = g.ldx[2];
+  const int K0 = g.K[0], K1 = g.K[1], K2 = g.K[2];
+  const int M = g.M, N = g.N;
+  int total = (K0 + BK - 1) / BK;
+  if (g.nseg > 1) total += (K1 + BK - 1) / BK;
+  if (g.nseg > 2) total += (K2 + BK - 1) / BK;
+
+  int lseg = 0, lk0 = 0;  // cursor of the next slab to load
+  bool tail = false;      // the slab in the staging registers ends its segment short of BK
+#define LH_ISSUE()                                                                   \
+  do {                                                                               \
+    const float *Ab = lseg == 0 ? A0 : (lseg == 1 ? A1 : A2);                        \
+    const float *Xb = lseg == 0 ? X0 : (lseg == 1 ? X1 : X2);                        \
+    const int la = lseg == 0 ? lda0 : (lseg == 1 ? lda1 : lda2);                     \
+    const int lx = lseg == 0 ? ldx0 : (lseg == 1 ? ldx1 : ldx2);                     \
+    const int Ks = lseg == 0 ? K0 : (lseg == 1 ? K1 : K2);                           \
+    if (lk0 == 0) {                                                                  \
+      sa.set_ld(la, tid, M - m0);                                                    \
+      sx.set_ld(lx, tid, N - n0);                                                    \
+    }                                                                                \
+    const float *pa = TA ? Ab + (size_t)m0 * la + lk0 : Ab + (size_t)lk0 * la + m0;  \
+    const float *px = !TX ? Xb + (size_t)n0 * lx + lk0 : Xb + (size_t)lk0 * lx + n0; \
+    tail = Ks - lk0 < BK;                                                            \
+    if (tail) {                                                                      \
+      sa.clamp_tail(tid, Ks - lk0);                                                  \
+      sx.clamp_tail(tid, Ks - lk0);                                                  \
+    }                                                                                \
+    sa.load(pa, tid);                                                                \
+    sx.load(px, tid);                                                                \
+    lk0 += BK;                                                                       \
+    if (lk0 >= Ks) {                                                                 \
+      ++lseg;                                                                        \
+      lk0 = 0;                                                                       \
+    }                                                                                \
+  } while (0)
+#define LH_STASH(BUF)         \
+  do {                        \
+    float *sb = (BUF);        \
+    if (tail) {               \
+      sa.zero_tail();         \
+      sx.zero_tail();         \
+    }                         \
+    sa.store(sb, tid);        \
+    sx.store(sb + kAF, tid);  \
+  } while (0)
+
+  LH_ISSUE();
+  LH_STASH(smem);
+  __syncthreads();
+  int cur = 0;  // float offset of the slab buffer being consumed
+  for (int s = 0; s < total; ++s) {
+    const bool has_next = s + 1 < total;
+    if (has_next) LH_ISSUE();
+    {
+      const float *as = smem + cur + fa_off;
+      const float *xs = smem + cur + fx_off;
+      float fa[2][FM][4], fx[2][FN][4];
+#pragma unroll
+      for (int b = 0; b < FM; ++b) SA::read_frag(as, 0, b, fa[0][b]);
+#pragma unroll
+      for (int a = 0; a < FN; ++a) SX::read_frag(xs, 0, a, fx[0][a]);
+#pragma unroll
+      for (int grp = 0; grp < NG; ++grp) {
+        const int c = grp & 1, n = c ^ 1;
+        if (grp + 1 < NG) {
+#pragma unroll
+          for (int b = 0; b < FM; ++b) SA::read_frag(as, grp + 1, b, fa[n][b]);
+#pragma unroll
+          for (int a = 0; a < FN; ++a) SX::read_frag(xs, grp + 1, a, fx[n][a]);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int a = 0; a < FN; ++a)
+#pragma unroll
+            for (int b = 0; b < FM; ++b)
+              // operands swapped on purpose: the transposed product puts consecutive m in
+              // consecutive lanes of every accumulator register
+              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fx[c][a][q], fa[c][b][q],
+                                                               acc[a][b], 0, 0, 0);
+      }
+    }
+    if (has_next) LH_STASH(smem + (kSlab - cur));
+    __syncthreads();
+    cur = kSlab - cur;
+  }
+#undef LH_ISSUE
+#undef LH_STASH
+
+  if constexpr (WK > 1) {
+    // Fixed-order reduction of the WK partial tiles through LDS (the slab buffers are dead now).
+    constexpr int kPerWave = FN * FM * 16 * 64;
+    if (wk > 0) {
+      float *dst = smem + ((wk - 1) * (WM * WN) + wmn) * kPerWave + lane;
+#pragma unroll
+      for (int a = 0; a < FN; ++a)
+#pragma unroll
+        for (int b = 0; b < FM; ++b)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) dst[((a * FM + b) * 16 + j) * 64] = acc[a][b][j];
+    }
+    __syncthreads();
+    if (wk > 0) return;
+#pragma unroll
+    for (int p = 0; p < WK - 1; ++p) {
+      const float *src = smem + (p * (WM * WN) + wmn) * kPerWave + lane;
+#pragma unroll
+      for (int a = 0; a < FN; ++a)
+#pragma unroll
+        for (int b = 0; b < FM; ++b)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) acc[a][b][j] += src[((a * FM + b) * 16 + j) * 64];
+    }
+  }
+
+  // Epilogue: accumulator register j of lane l is C[m = .. + l%32][n = .. + 8*(j/4) + 4*(l/32) + j%4].
+  const float alpha = g.alpha, beta = g.beta;
+  const bool use_beta = beta != 0.f;
+  const int *const colmask = g.colmask;
 #pragma unroll
   for (int a = 0; a < FN; ++a) {
 #pragma unroll
@@ -296,21 +634,23 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
       if (m >= g.M) continue;
       const float bv = g.bias ? g.bias[m] : 0.f;
       const bool do_tanh = g.act == LH_ACT_TANH && m < g.act_rows;
+      const int nb = n0 + wn * TN + a * 32 + lhi * 4;
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        const int n = n0 + wn * TN + a * 32 + (j / 4) * 8 + lhi * 4 + (j % 4);
+        const int n = nb + (j / 4) * 8 + (j % 4);
         if (n >= g.N) continue;
         float *cp = g.C + (size_t)n * g.ldc + m;
         float v = alpha * acc[a][b][j];
-        if (beta != 0.f) v += beta * *cp;
+        if (use_beta) v += beta * *cp;
         v += bv;
         if (do_tanh) v = tanhf(v);
-        if (g.colmask) v *= (float)g.colmask[n];
+        if (colmask) v *= (float)colmask[n];
         *cp = v;
       }
     }
   }
 }
+
 
 // ---- configurations -----------------------------------------------------------------------
 struct Config {
@@ -375,20 +715,24 @@ int launch_cfg(const GemmArgs &g0, bool ta, bool tx, bool vec, hipStream_t st) {
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   const dim3 grid(g.tiles_m * g.tiles_n), block(64 * WM * WN * WK);
-  constexpr int bytes = smem_floats<BM, BN, WK, BK>() * 4;
-#define LH_GEMM_LAUNCH(TA, TX, VEC) \
-  return launch_kernel(gemm_kernel<BM, BN, WM, WN, WK, BK, TA, TX, VEC>, bytes, grid, block, st, g)
   if (vec) {
-    if (!ta && !tx) LH_GEMM_LAUNCH(false, false, true);
-    else if (ta) LH_GEMM_LAUNCH(true, false, true);
-    else LH_GEMM_LAUNCH(false, true, true);
+    #define LH_GEMM_LAUNCH(TA, TX)                                                           \
+  return launch_kernel(gemm_kernel<BM, BN, WM, WN, WK, BK, TA, TX>,                      \
+                       smem2_floats<BM, BN, WM, WN, WK, BK, TA, TX>() * 4, grid, block, st, g)
+    if (!ta && !tx) LH_GEMM_LAUNCH(false, false);
+    else if (ta) LH_GEMM_LAUNCH(true, false);
+    else LH_GEMM_LAUNCH(false, true);
+#undef LH_GEMM_LAUNCH
   }
   if constexpr (ALLOW_UNALIGNED) {
-    if (!ta && !tx) LH_GEMM_LAUNCH(false, false, false);
-    else if (ta) LH_GEMM_LAUNCH(true, false, false);
-    else LH_GEMM_LAUNCH(false, true, false);
-  }
+    constexpr int bytes = smem_floats<BM, BN, WK, BK>() * 4;
+#define LH_GEMM_LAUNCH(TA, TX) \
+  return launch_kernel(gemm_generic_kernel<BM, BN, WM, WN, WK, BK, TA, TX, false>, bytes, grid, block, st, g)
+    if (!ta && !tx) LH_GEMM_LAUNCH(false, false);
+    else if (ta) LH_GEMM_LAUNCH(true, false);
+    else LH_GEMM_LAUNCH(false, true);
 #undef LH_GEMM_LAUNCH
+  }
   return lh::fail_arg("lh_gemm_f32: internal error, unaligned operands reached an aligned-only tile");
 }
 
@@ -457,8 +801,10 @@ int prepare(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int tra
     // 16-byte loads need aligned bases / leading dimensions and a contiguous extent that is a
     // multiple of 4 (the guards test only the first element of a float4).
     const int a_extent = transA ? e.K : M, x_extent = transX ? N : e.K;
+    // ... and the main kernel keeps per-thread byte offsets inside a slab in 32 bits.
+    constexpr int kMaxLd = 1 << 22;
     vec = vec && lh::aligned16(e.A) && lh::aligned16(e.X) && e.lda % 4 == 0 && e.ldx % 4 == 0 &&
-          a_extent % 4 == 0 && x_extent % 4 == 0;
+          a_extent % 4 == 0 && x_extent % 4 == 0 && e.lda < kMaxLd && e.ldx < kMaxLd;
   }
   for (int s = nseg; s < LH_GEMM_MAX_SEGS; ++s) {  // unused slots mirror segment 0 (never read)
     g.A[s] = g.A[0];
@@ -526,8 +872,11 @@ extern "C" int lh_gemm_kernel_name(int M, int N, const lh_gemm_seg *segs, int ns
                          nullptr, &dummy, M, &p);
   if (rc != LH_OK) return rc;
   const Config &k = kConfigs[p.config];
-  snprintf(name, name_cap, "gemm_kernel<%d, %d, %d, %d, %d, %d, %s, %s, %s>", k.bm, k.bn, k.wm,
-           k.wn, k.wk, k.bk, p.ta ? "true" : "false", p.tx ? "true" : "false",
-           p.vec ? "true" : "false");
+  if (p.vec)
+    snprintf(name, name_cap, "gemm_kernel<%d, %d, %d, %d, %d, %d, %s, %s>", k.bm, k.bn, k.wm, k.wn,
+             k.wk, k.bk, p.ta ? "true" : "false", p.tx ? "true" : "false");
+  else
+    snprintf(name, name_cap, "gemm_generic_kernel<%d, %d, %d, %d, %d, %d, %s, %s, false>", k.bm,
+             k.bn, k.wm, k.wn, k.wk, k.bk, p.ta ? "true" : "false", p.tx ? "true" : "false");
   return LH_OK;
 }

@@ -113,7 +113,9 @@ def test_gemm_every_tile_configuration(lh):
     n_cfg = lh.load().lh_gemm_set_config_override(-1)
     assert n_cfg >= 1
     shapes = [(200, 76, (100, 36), False, False), (129, 97, (68,), True, False),
-              (96, 33, (40,), False, True), (70, 130, (17, 9), False, False)]
+              (96, 33, (40,), False, True), (70, 130, (17, 9), False, False),
+              (96, 36, (40, 24), False, True), (72, 132, (20, 12, 136), False, False),
+              (260, 68, (132, 8), True, False)]
     try:
         for cfg in range(n_cfg):
             assert lh.load().lh_gemm_set_config_override(cfg) == n_cfg
@@ -133,7 +135,7 @@ def test_gemm_every_tile_configuration(lh):
                 w2[: M // 2] = np.tanh(w2[: M // 2])
                 assert_close(host(out, (M, N)), w2, f"config {cfg} tanh on the first rows only")
                 name = lh.gemm_kernel_name(M, N, segs, tA, tX)
-                assert name.startswith("gemm_kernel<") and name.endswith(">")
+                assert name.startswith(("gemm_kernel<", "gemm_generic_kernel<")) and name.endswith(">")
     finally:
         lh.load().lh_gemm_set_config_override(-1)
     with pytest.raises(lh.LinmtHipError):
