@@ -20,6 +20,8 @@
 #ifndef LINMT_HIP_H_
 #define LINMT_HIP_H_
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -98,15 +100,34 @@ int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int
 int lh_gemm_act_rows_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
                          float alpha, float beta, const float *bias, int act, int act_rows,
                          const int *colmask, float *C, int ldc, lh_stream_t stream);
-/* Name of the kernel instance lh_gemm_f32 would launch for this problem (tile shape and operand
+/* Same product, allowed to split the K dimension across workgroups when the output alone has
+ * too few tiles to fill the GPU (the recurrent gate and attention products of a decoding step;
+ * no counterpart in the reference, where cuBLAS makes that choice internally).  Each share
+ * writes its partial sums into a plane of `workspace`; a second launch adds the planes in a fixed
+ * order and applies the epilogue, so results do not depend on scheduling.  `workspace` is device
+ * memory, 16-byte aligned, `workspace_bytes` long; its contents before and after a call mean
+ * nothing.  Calls that share a workspace must be ordered on one stream.  A null or small
+ * workspace only limits the split (a plane is M x N floats); 64 MiB covers every product here. */
+int lh_gemm_ws_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
+                   float alpha, float beta, const float *bias, int act, int act_rows,
+                   const int *colmask, float *C, int ldc, void *workspace, size_t workspace_bytes,
+                   lh_stream_t stream);
+/* Name of the kernel instance lh_gemm_ws_f32 would launch for this problem (tile shape and operand
  * flags), as profilers print it; no counterpart in the reference.  Pointers in `segs` are only
- * inspected for alignment. */
+ * inspected for alignment; workspace_bytes = 0 describes lh_gemm_f32 / lh_gemm_act_rows_f32. */
 int lh_gemm_kernel_name(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
-                        char *name, int name_cap);
-/* Tuning and test aid (no counterpart in the reference): forces tile configuration `config` for
- * every later lh_gemm_* call of the process, config < 0 restores the built-in choice.  Returns the
- * number of configurations (so 0 <= config < return value), LH_ERR_ARG if config is too large. */
+                        size_t workspace_bytes, char *name, int name_cap);
+/* Tuning and test aids (no counterpart in the reference).
+ * lh_gemm_set_config_override: forces tile configuration `config` for every later lh_gemm_* call
+ * of the process, config < 0 restores the built-in choice.  Returns the number of configurations
+ * (so 0 <= config < return value), LH_ERR_ARG if config is too large.
+ * lh_gemm_set_splits_override: likewise forces the K split of lh_gemm_ws_f32 (as far as the
+ * workspace allows), splits <= 0 restores the built-in choice; returns the largest split.
+ * lh_gemm_config_info: info = {BM, BN, WM, WN, WK, BK, workgroups resident per CU, LDS bytes} of a
+ * configuration for the given operand flags. */
 int lh_gemm_set_config_override(int config);
+int lh_gemm_set_splits_override(int splits);
+int lh_gemm_config_info(int config, int transA, int transX, int info[8]);
 
 /* ------------------------------------------------------------------------------------------
  * a3. Fused LSTM cell forward: bias add, gate nonlinearities, c_t / h_t update, padding mask,

@@ -42,6 +42,13 @@ struct GemmArgs {
   float *C;
   int ldc;
   int tiles_m, tiles_n;
+  // K split across workgroups (main kernel only): workgroup (tile, split) takes slabs
+  // [split * slabs_per_split, ...) of the concatenated segments and writes its raw partial tile
+  // into plane `split` of the workspace (ws_ld x N floats each, column-major like C); a second
+  // kernel adds the planes up in split order and applies the epilogue.
+  int splits, slabs_per_split;
+  float *ws_part;
+  int ws_ld;
 };
 
 // Stages one BK x BD operand slab: global -> registers (load), registers -> LDS [BK][BD+PAD] (store).
@@ -482,8 +489,12 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
   const int xcd = id % 8, within = id / 8;
   const int per = nwg / 8, rem = nwg % 8;
   const int logical = xcd * per + (xcd < rem ? xcd : rem) + within;
-  const int m0 = (logical / g.tiles_n) * BM;
-  const int n0 = (logical % g.tiles_n) * BN;
+  // the splits of a tile are neighbours: same XCD, so the partial tiles meet in its L2
+  const int splits = g.splits;
+  const int tile = splits == 1 ? logical : logical / splits;
+  const int split = splits == 1 ? 0 : logical % splits;
+  const int m0 = (tile / g.tiles_n) * BM;
+  const int n0 = (tile % g.tiles_n) * BN;
 
   const int tid = threadIdx.x;
   const int wave = tid / lh::kWave, lane = tid % lh::kWave;
@@ -510,12 +521,24 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
   const int ldx0 = g.ldx[0], ldx1 = g.ldx[1], ldx2 = g.ldx[2];
   const int K0 = g.K[0], K1 = g.K[1], K2 = g.K[2];
   const int M = g.M, N = g.N;
-  int total = (K0 + BK - 1) / BK;
-  if (g.nseg > 1) total += (K1 + BK - 1) / BK;
-  if (g.nseg > 2) total += (K2 + BK - 1) / BK;
-
-  int lseg = 0, lk0 = 0;  // cursor of the next slab to load
-  bool tail = false;      // the slab in the staging registers ends its segment short of BK
+  const int slabs0 = (K0 + BK - 1) / BK;
+  const int slabs1 = g.nseg > 1 ? (K1 + BK - 1) / BK : 0;
+  const int slabs2 = g.nseg > 2 ? (K2 + BK - 1) / BK : 0;
+  // this workgroup's share of the slab sequence (the host never makes an empty share)
+  const int first = split * g.slabs_per_split;
+  const int total = min(g.slabs_per_split, slabs0 + slabs1 + slabs2 - first);
+  int lseg = 0, lk0 = first;  // cursor of the next slab to load: segment, k offset inside it
+  if (lk0 >= slabs0) {
+    lk0 -= slabs0;
+    lseg = 1;
+    if (lk0 >= slabs1) {
+      lk0 -= slabs1;
+      lseg = 2;
+    }
+  }
+  lk0 *= BK;
+  bool new_seg = true;  // the per-thread offsets must be rebuilt for the segment's leading dimension
+  bool tail = false;    // the slab in the staging registers ends its segment short of BK
 #define LH_ISSUE()                                                                   \
   do {                                                                               \
     const float *Ab = lseg == 0 ? A0 : (lseg == 1 ? A1 : A2);                        \
@@ -523,7 +546,7 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
     const int la = lseg == 0 ? lda0 : (lseg == 1 ? lda1 : lda2);                     \
     const int lx = lseg == 0 ? ldx0 : (lseg == 1 ? ldx1 : ldx2);                     \
     const int Ks = lseg == 0 ? K0 : (lseg == 1 ? K1 : K2);                           \
-    if (lk0 == 0) {                                                                  \
+    if (new_seg) {                                                                   \
       sa.set_ld(la, tid, M - m0);                                                    \
       sx.set_ld(lx, tid, N - n0);                                                    \
     }                                                                                \
@@ -537,6 +560,7 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
     sa.load(pa, tid);                                                                \
     sx.load(px, tid);                                                                \
     lk0 += BK;                                                                       \
+    new_seg = tail || lk0 >= Ks; /* a clamped tail also dirtied the offsets */       \
     if (lk0 >= Ks) {                                                                 \
       ++lseg;                                                                        \
       lk0 = 0;                                                                       \
@@ -609,37 +633,46 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
           for (int j = 0; j < 16; ++j) dst[((a * FM + b) * 16 + j) * 64] = acc[a][b][j];
     }
     __syncthreads();
-    if (wk > 0) return;
+    if (wk == 0) {
 #pragma unroll
-    for (int p = 0; p < WK - 1; ++p) {
-      const float *src = smem + (p * (WM * WN) + wmn) * kPerWave + lane;
+      for (int p = 0; p < WK - 1; ++p) {
+        const float *src = smem + (p * (WM * WN) + wmn) * kPerWave + lane;
 #pragma unroll
-      for (int a = 0; a < FN; ++a)
+        for (int a = 0; a < FN; ++a)
 #pragma unroll
-        for (int b = 0; b < FM; ++b)
+          for (int b = 0; b < FM; ++b)
 #pragma unroll
-          for (int j = 0; j < 16; ++j) acc[a][b][j] += src[((a * FM + b) * 16 + j) * 64];
+            for (int j = 0; j < 16; ++j) acc[a][b][j] += src[((a * FM + b) * 16 + j) * 64];
+      }
     }
   }
 
+  if (wk > 0) return;
+
   // Epilogue: accumulator register j of lane l is C[m = .. + l%32][n = .. + 8*(j/4) + 4*(l/32) + j%4].
-  const float alpha = g.alpha, beta = g.beta;
-  const bool use_beta = beta != 0.f;
-  const int *const colmask = g.colmask;
+  // A split product stores the bare partial sums in its plane of the workspace instead.
+  const bool partial = splits > 1;
+  const float alpha = partial ? 1.f : g.alpha, beta = g.beta;
+  const bool use_beta = !partial && beta != 0.f;
+  const int *const colmask = partial ? nullptr : g.colmask;
+  const float *const bias = partial ? nullptr : g.bias;
+  const int act_rows = partial || g.act != LH_ACT_TANH ? 0 : g.act_rows;
+  float *const Cb = partial ? g.ws_part + (size_t)split * g.ws_ld * g.N : g.C;
+  const int ldc = partial ? g.ws_ld : g.ldc;
 #pragma unroll
   for (int a = 0; a < FN; ++a) {
 #pragma unroll
     for (int b = 0; b < FM; ++b) {
       const int m = m0 + wm * TM + b * 32 + l32;
       if (m >= g.M) continue;
-      const float bv = g.bias ? g.bias[m] : 0.f;
-      const bool do_tanh = g.act == LH_ACT_TANH && m < g.act_rows;
+      const float bv = bias ? bias[m] : 0.f;
+      const bool do_tanh = m < act_rows;
       const int nb = n0 + wn * TN + a * 32 + lhi * 4;
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const int n = nb + (j / 4) * 8 + (j % 4);
         if (n >= g.N) continue;
-        float *cp = g.C + (size_t)n * g.ldc + m;
+        float *cp = Cb + (size_t)n * ldc + m;
         float v = alpha * acc[a][b][j];
         if (use_beta) v += beta * *cp;
         v += bv;
@@ -651,6 +684,24 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
   }
 }
 
+// Second half of a split product: C = epilogue(sum of the partial planes, in split order).
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs g) {
+  const size_t plane = (size_t)g.ws_ld * g.N;
+  const size_t total = (size_t)g.M * g.N;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+    const int n = (int)(i / g.M), m = (int)(i % g.M);
+    const float *p = g.ws_part + (size_t)n * g.ws_ld + m;
+    float acc = 0.f;
+    for (int s = 0; s < g.splits; ++s) acc += p[s * plane];
+    float *cp = g.C + (size_t)n * g.ldc + m;
+    float v = g.alpha * acc;
+    if (g.beta != 0.f) v += g.beta * *cp;
+    if (g.bias) v += g.bias[m];
+    if (g.act == LH_ACT_TANH && m < g.act_rows) v = tanhf(v);
+    if (g.colmask) v *= (float)g.colmask[n];
+    *cp = v;
+  }
+}
 
 // ---- configurations -----------------------------------------------------------------------
 struct Config {
@@ -677,7 +728,11 @@ struct Config {
   X(16, 128, 32, 4, 1, 1, 16)                                                  \
   X(17, 128, 32, 4, 1, 1, 64)                                                  \
   X(18, 64, 32, 2, 1, 4, 32)                                                   \
-  X(19, 64, 32, 2, 1, 4, 128)
+  X(19, 64, 32, 2, 1, 4, 128)                                                  \
+  X(20, 128, 128, 2, 2, 1, 64) /* deep slabs: one workgroup per CU hides its own latency */ \
+  X(21, 128, 64, 2, 2, 1, 64)                                                  \
+  X(22, 128, 128, 2, 2, 2, 64) /* ... or two wavefronts per SIMD inside the workgroup */ \
+  X(23, 128, 64, 2, 2, 2, 64)
 
 #define LH_CFG_ENTRY(I, BM, BN, WM, WN, WK, BK) {BM, BN, WM, WN, WK, BK},
 const Config kConfigs[] = {LH_GEMM_CONFIGS(LH_CFG_ENTRY)};
@@ -714,15 +769,27 @@ int launch_cfg(const GemmArgs &g0, bool ta, bool tx, bool vec, hipStream_t st) {
   GemmArgs g = g0;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
-  const dim3 grid(g.tiles_m * g.tiles_n), block(64 * WM * WN * WK);
+  if (!vec) g.splits = 1;
+  int slabs = 0;
+  for (int s = 0; s < g.nseg; ++s) slabs += (g.K[s] + BK - 1) / BK;
+  g.slabs_per_split = (slabs + g.splits - 1) / g.splits;
+  g.splits = (slabs + g.slabs_per_split - 1) / g.slabs_per_split;  // no empty share
+  const dim3 grid(g.tiles_m * g.tiles_n * g.splits), block(64 * WM * WN * WK);
   if (vec) {
-    #define LH_GEMM_LAUNCH(TA, TX)                                                           \
-  return launch_kernel(gemm_kernel<BM, BN, WM, WN, WK, BK, TA, TX>,                      \
-                       smem2_floats<BM, BN, WM, WN, WK, BK, TA, TX>() * 4, grid, block, st, g)
+    int rc;
+#define LH_GEMM_LAUNCH(TA, TX)                                                              \
+  rc = launch_kernel(gemm_kernel<BM, BN, WM, WN, WK, BK, TA, TX>,                           \
+                     smem2_floats<BM, BN, WM, WN, WK, BK, TA, TX>() * 4, grid, block, st, g)
     if (!ta && !tx) LH_GEMM_LAUNCH(false, false);
     else if (ta) LH_GEMM_LAUNCH(true, false);
     else LH_GEMM_LAUNCH(false, true);
 #undef LH_GEMM_LAUNCH
+    if (rc != LH_OK || g.splits == 1) return rc;
+    const size_t total = (size_t)g.M * g.N;
+    const size_t blocks = (total + 1023) / 1024;  // four elements per thread
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)(blocks < 8192 ? blocks : 8192)),
+                       dim3(256), 0, st, g);
+    return lh::check_launch("lh_gemm_ws_f32 split reduction");
   }
   if constexpr (ALLOW_UNALIGNED) {
     constexpr int bytes = smem_floats<BM, BN, WK, BK>() * 4;
@@ -747,20 +814,140 @@ int launch_index(int c, const GemmArgs &g, bool ta, bool tx, bool vec, hipStream
   }
 }
 
-int g_config_override = -1;  // tuning / test aid, see lh_gemm_set_config_override
+template <int BM, int BN, int WM, int WN, int WK, int BK>
+int occupancy_cfg(bool ta, bool tx, int *blocks_per_cu, int *lds_bytes) {
+  constexpr int block = 64 * WM * WN * WK;
+  hipError_t e;
+#define LH_GEMM_OCC(TA, TX)                                                                       \
+  do {                                                                                            \
+    constexpr int bytes = smem2_floats<BM, BN, WM, WN, WK, BK, TA, TX>() * 4;                     \
+    *lds_bytes = bytes;                                                                           \
+    auto kernel = gemm_kernel<BM, BN, WM, WN, WK, BK, TA, TX>;                                    \
+    if (bytes > 64 * 1024)                                                                        \
+      (void)hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                bytes);                                                           \
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, kernel, block, bytes);        \
+  } while (0)
+  if (!ta && !tx) LH_GEMM_OCC(false, false);
+  else if (ta) LH_GEMM_OCC(true, false);
+  else LH_GEMM_OCC(false, true);
+#undef LH_GEMM_OCC
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return lh::fail_arg("lh_gemm_config_info: occupancy query failed: %s", hipGetErrorString(e));
+  }
+  return LH_OK;
+}
 
-// Tile choice, from sweeps of every configuration over the products of the path on MI355X.
-int pick_config(int M, int N, long long ktot, bool vec) {
-  if (!vec) return kUnalignedConfig;
-  const int forced = g_config_override;
-  if (forced >= 0 && forced < kNumConfigs) return forced;
-  (void)ktot;
-  const long long tiles32 = (long long)((M + 31) / 32) * ((N + 31) / 32);  // 32x32 MFMA tiles
-  if (N <= 64) return M >= 16384 ? 18 : 14;        // encoder steps, single-sentence decoding
-  if (tiles32 >= 256 * 40) return 3;               // >= 40 MFMA tiles per CU (output projection)
-  if (tiles32 >= 256 * 10) return N >= 512 || N % 96 == 0 ? 5 : 7;  // e.g. 4000 x 768 gate products
-  if (tiles32 >= 256 * 7) return 7;
-  return 18;                                       // M around 1000: many small tiles, split K
+int occupancy_index(int c, bool ta, bool tx, int *blocks_per_cu, int *lds_bytes) {
+  switch (c) {
+#define LH_CFG_CASE(I, BM, BN, WM, WN, WK, BK) \
+  case I: return occupancy_cfg<BM, BN, WM, WN, WK, BK>(ta, tx, blocks_per_cu, lds_bytes);
+    LH_GEMM_CONFIGS(LH_CFG_CASE)
+#undef LH_CFG_CASE
+    default: return lh::fail_arg("lh_gemm_config_info: configuration %d does not exist", c);
+  }
+}
+
+int g_config_override = -1;  // tuning / test aids, see lh_gemm_set_config_override
+int g_splits_override = 0;
+
+constexpr int kMaxSplits = 16;
+
+// Leading dimension of a partial plane, and the largest split count <= want whose planes fit.
+int plane_ld(int M) { return (M + 3) & ~3; }
+int fit_splits(int M, int N, int want, size_t workspace_bytes) {
+  if (want <= 1) return 1;
+  const size_t plane = (size_t)plane_ld(M) * N * sizeof(float);
+  const size_t fit = workspace_bytes / plane;
+  const size_t s = fit < (size_t)want ? fit : (size_t)want;
+  return s < 1 ? 1 : (int)(s > kMaxSplits ? kMaxSplits : s);
+}
+
+// ---- choice of tile configuration and K split ------------------------------------------------
+// Cost model over a measured table.  For one configuration, T1(K) is the time of a launch that
+// gives every CU a single workgroup and Tocc(K) of one that gives every CU as many as fit at once
+// (both linear in the K depth of a workgroup's share).  A product whose fullest CU receives n
+// workgroups then takes about (n / occ) * Tocc + T(n % occ), T interpolated between T1 and Tocc;
+// a split adds the pass that sums the partial planes.  The cheapest (configuration, split) wins.
+struct Tuning {
+  int occ;           // workgroups resident per CU
+  float f1, s1;      // one workgroup per CU: fixed us, us per k
+  float focc, socc;  // CU full
+};
+#include "gemm_tuning.inc"
+constexpr int kCUs = 256;
+constexpr float kReduceFixedUs = 2.5f, kReduceBytesPerUs = 3.0e6f;
+
+float predict_us(const Tuning &t, const Config &k, int M, int N, const int *K, int nseg, int want,
+                 int *splits) {
+  const long long tiles = (long long)((M + k.bm - 1) / k.bm) * ((N + k.bn - 1) / k.bn);
+  int slabs = 0;
+  for (int s = 0; s < nseg; ++s) slabs += (K[s] + k.bk - 1) / k.bk;
+  const int share = (slabs + want - 1) / want;
+  const int S = (slabs + share - 1) / share;
+  *splits = S;
+  const float depth = (float)share * k.bk;
+  // Workgroups per CU: dispatch is dynamic, so a fractional load costs less than a whole extra
+  // round but leaves a tail of about half a workgroup.
+  const float per_cu = (float)(tiles * S) / kCUs;
+  const float load = fminf(per_cu + 0.5f, ceilf(per_cu));
+  const float t1 = t.f1 + t.s1 * depth, tocc = t.focc + t.socc * depth;
+  const float rounds = floorf(load / (float)t.occ);
+  const float rest = load - rounds * (float)t.occ;
+  float us = rounds * tocc;
+  if (rest > 1e-6f)
+    us += rest <= 1.f || t.occ == 1 ? t1 : t1 + (tocc - t1) * (rest - 1.f) / (float)(t.occ - 1);
+  if (S > 1) us += kReduceFixedUs + (float)(S + 1) * (float)M * (float)N * 4.f / kReduceBytesPerUs;
+  return us;
+}
+
+void pick_config(int M, int N, const int *K, int nseg, bool ta, bool tx, bool vec,
+                 size_t workspace_bytes, int *config, int *splits) {
+  *splits = 1;
+  if (!vec) {
+    *config = kUnalignedConfig;
+    return;
+  }
+  // The decoder repeats a handful of problems thousands of times: remember the answers.
+  struct Memo {
+    int M, N, K[LH_GEMM_MAX_SEGS], flags, config, splits;
+    size_t workspace_bytes;
+  };
+  static thread_local Memo memo[64];
+  const int flags = 1 + (ta ? 2 : 0) + (tx ? 4 : 0) + 8 * nseg + 64 * (g_config_override + 1) +
+                    4096 * g_splits_override;
+  int Kk[LH_GEMM_MAX_SEGS] = {0, 0, 0};
+  for (int s = 0; s < nseg; ++s) Kk[s] = K[s];
+  const unsigned h = ((unsigned)M * 2654435761u) ^ ((unsigned)N * 40503u) ^ ((unsigned)Kk[0] * 97u) ^
+                     ((unsigned)Kk[1] * 31u) ^ (unsigned)Kk[2] ^ ((unsigned)flags << 20);
+  Memo &e = memo[(h ^ (h >> 13)) % 64];
+  if (e.flags == flags && e.M == M && e.N == N && e.K[0] == Kk[0] && e.K[1] == Kk[1] &&
+      e.K[2] == Kk[2] && e.workspace_bytes == workspace_bytes) {
+    *config = e.config;
+    *splits = e.splits;
+    return;
+  }
+  static const int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
+  const Tuning *table = kTuning[ta ? 1 : (tx ? 2 : 0)];
+  float best = 3.0e38f;
+  *config = kUnalignedConfig;
+  for (int c = 0; c < kNumConfigs; ++c) {
+    if (g_config_override >= 0 && c != g_config_override) continue;
+    for (int want : kSplitChoices) {
+      if (g_splits_override > 0) want = fit_splits(M, N, g_splits_override, workspace_bytes);
+      if (want > 1 && fit_splits(M, N, want, workspace_bytes) < want) break;
+      int S;
+      const float us = predict_us(table[c], kConfigs[c], M, N, K, nseg, want, &S);
+      if (us < best) {
+        best = us;
+        *config = c;
+        *splits = S;
+      }
+      if (g_splits_override > 0) break;
+    }
+  }
+  e = Memo{M, N, {Kk[0], Kk[1], Kk[2]}, flags, *config, *splits, workspace_bytes};
 }
 
 struct Prepared {
@@ -771,7 +958,7 @@ struct Prepared {
 
 int prepare(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX, float alpha,
             float beta, const float *bias, int act, int act_rows, const int *colmask, float *C,
-            int ldc, Prepared *out) {
+            int ldc, void *workspace, size_t workspace_bytes, Prepared *out) {
   if (M <= 0 || N <= 0) return lh::fail_arg("lh_gemm_f32: M=%d N=%d must be positive", M, N);
   if (!segs || nseg < 1 || nseg > LH_GEMM_MAX_SEGS)
     return lh::fail_arg("lh_gemm_f32: nseg=%d outside [1,%d]", nseg, LH_GEMM_MAX_SEGS);
@@ -782,7 +969,6 @@ int prepare(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int tra
   GemmArgs &g = out->g;
   g = GemmArgs{};
   bool vec = true;
-  long long ktot = 0;
   for (int s = 0; s < nseg; ++s) {
     const lh_gemm_seg &e = segs[s];
     if (!e.A || !e.X || e.K <= 0)
@@ -797,7 +983,6 @@ int prepare(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int tra
     g.lda[s] = e.lda;
     g.ldx[s] = e.ldx;
     g.K[s] = e.K;
-    ktot += e.K;
     // 16-byte loads need aligned bases / leading dimensions and a contiguous extent that is a
     // multiple of 4 (the guards test only the first element of a float4).
     const int a_extent = transA ? e.K : M, x_extent = transX ? N : e.K;
@@ -827,33 +1012,42 @@ int prepare(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int tra
   out->ta = transA != 0;
   out->tx = transX != 0;
   out->vec = vec;
-  out->config = pick_config(M, N, ktot, vec);
+  if (!workspace || !lh::aligned16(workspace)) workspace_bytes = 0;
+  pick_config(M, N, g.K, nseg, transA != 0, transX != 0, vec, workspace_bytes, &out->config,
+              &g.splits);
+  g.ws_part = static_cast<float *>(workspace);
+  g.ws_ld = plane_ld(M);
   return LH_OK;
 }
 
 }  // namespace
 
+extern "C" int lh_gemm_ws_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA,
+                              int transX, float alpha, float beta, const float *bias, int act,
+                              int act_rows, const int *colmask, float *C, int ldc, void *workspace,
+                              size_t workspace_bytes, lh_stream_t stream) {
+  if (act_rows < 0 || act_rows > M)
+    return lh::fail_arg("lh_gemm_f32: act_rows=%d outside [0,M=%d]", act_rows, M);
+  Prepared p;
+  const int rc = prepare(M, N, segs, nseg, transA, transX, alpha, beta, bias, act, act_rows,
+                         colmask, C, ldc, workspace, workspace_bytes, &p);
+  if (rc != LH_OK) return rc;
+  return launch_index(p.config, p.g, p.ta, p.tx, p.vec, lh::as_stream(stream));
+}
+
 extern "C" int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
                            float alpha, float beta, const float *bias, int act, const int *colmask,
                            float *C, int ldc, lh_stream_t stream) {
-  Prepared p;
-  const int rc = prepare(M, N, segs, nseg, transA, transX, alpha, beta, bias, act, M, colmask, C,
-                         ldc, &p);
-  if (rc != LH_OK) return rc;
-  return launch_index(p.config, p.g, p.ta, p.tx, p.vec, lh::as_stream(stream));
+  return lh_gemm_ws_f32(M, N, segs, nseg, transA, transX, alpha, beta, bias, act, M, colmask, C,
+                        ldc, nullptr, 0, stream);
 }
 
 extern "C" int lh_gemm_act_rows_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA,
                                     int transX, float alpha, float beta, const float *bias, int act,
                                     int act_rows, const int *colmask, float *C, int ldc,
                                     lh_stream_t stream) {
-  if (act_rows < 0 || act_rows > M)
-    return lh::fail_arg("lh_gemm_act_rows_f32: act_rows=%d outside [0,M=%d]", act_rows, M);
-  Prepared p;
-  const int rc = prepare(M, N, segs, nseg, transA, transX, alpha, beta, bias, act, act_rows,
-                         colmask, C, ldc, &p);
-  if (rc != LH_OK) return rc;
-  return launch_index(p.config, p.g, p.ta, p.tx, p.vec, lh::as_stream(stream));
+  return lh_gemm_ws_f32(M, N, segs, nseg, transA, transX, alpha, beta, bias, act, act_rows, colmask,
+                        C, ldc, nullptr, 0, stream);
 }
 
 extern "C" int lh_gemm_set_config_override(int config) {
@@ -863,13 +1057,31 @@ extern "C" int lh_gemm_set_config_override(int config) {
   return kNumConfigs;
 }
 
+extern "C" int lh_gemm_set_splits_override(int splits) {
+  if (splits > kMaxSplits)
+    return lh::fail_arg("lh_gemm_set_splits_override: %d > %d", splits, kMaxSplits);
+  g_splits_override = splits < 0 ? 0 : splits;
+  return kMaxSplits;
+}
+
+extern "C" int lh_gemm_config_info(int config, int transA, int transX, int info[8]) {
+  if (config < 0 || config >= kNumConfigs || !info || (transA && transX))
+    return lh::fail_arg("lh_gemm_config_info: config=%d of %d, info=%p", config, kNumConfigs,
+                        (void *)info);
+  const Config &k = kConfigs[config];
+  info[0] = k.bm, info[1] = k.bn, info[2] = k.wm, info[3] = k.wn, info[4] = k.wk, info[5] = k.bk;
+  return occupancy_index(config, transA != 0, transX != 0, &info[6], &info[7]);
+}
+
 extern "C" int lh_gemm_kernel_name(int M, int N, const lh_gemm_seg *segs, int nseg, int transA,
-                                   int transX, char *name, int name_cap) {
+                                   int transX, size_t workspace_bytes, char *name, int name_cap) {
   if (!name || name_cap < 1) return lh::fail_arg("lh_gemm_kernel_name: no output buffer");
   Prepared p;
   float dummy;
+  // any aligned non-null address stands in for the workspace: nothing is launched
   const int rc = prepare(M, N, segs, nseg, transA, transX, 1.f, 0.f, nullptr, LH_ACT_NONE, M,
-                         nullptr, &dummy, M, &p);
+                         nullptr, &dummy, M, workspace_bytes ? (void *)(uintptr_t)256 : nullptr,
+                         workspace_bytes, &p);
   if (rc != LH_OK) return rc;
   const Config &k = kConfigs[p.config];
   if (p.vec)

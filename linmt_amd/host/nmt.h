@@ -361,6 +361,14 @@ class NeuralMachineTranslation {
   bool decode_mode_ = false;
   int beam_size_ = 0, n_sent_ = 0;
   Profiler profiler_;  // live HIP-event timing on stream_, off by default
+  // Scratch of lh_gemm_ws_f32 (split-K partial sums); every product of the model runs on
+  // stream_, which is the ordering that sharing it requires.
+  static constexpr size_t kGemmWorkspaceBytes = size_t(64) << 20;
+  DeviceArray<char> gemm_workspace_;
+  // Every dense product of the model: profiling key, workspace, error text.
+  void Gemm(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg, int trans_a, int trans_x,
+            float beta, const float *bias, int act, const int *colmask, float *C, int ldc,
+            const char *what);
 
   LstmLayer input_layer_source_, input_layer_target_;
   std::vector<std::unique_ptr<LstmLayer>> v_hidden_layers_source_, v_hidden_layers_target_;

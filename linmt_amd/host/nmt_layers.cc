@@ -253,12 +253,8 @@ void LstmNode::ForwardProp() {
   }
   segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
   if (feed) segs[nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
-  {
-    ProfileScope ps(M.profiler_, kTagGateGemm, 4 * H, B, segs, nseg, 0, 0);
-    LhErrorWrapper(lh_gemm_f32(4 * H, B, segs, nseg, 0, 0, 1.f, beta, nullptr, LH_ACT_NONE, nullptr,
-                               pre, 4 * H, s),
-                   "LstmNode::ForwardPropGpu stacked gate product");
-  }
+  M.Gemm(kTagGateGemm, 4 * H, B, segs, nseg, 0, 0, beta, nullptr, LH_ACT_NONE, nullptr, pre, 4 * H,
+         "LstmNode::ForwardPropGpu stacked gate product");
   const bool drop_out = M.apply_dropout_ && L.out_dropout_;
   ProfileScope pc(M.profiler_, kTagLstmCell, ((p_device_gates_ ? 44.0 : 28.0) + (drop_out ? 8.0 : 0.0)) * H * B);
   LhErrorWrapper(lh_lstm_cell_fwd_f32(H, B, pre, nullptr, nullptr,
@@ -292,10 +288,8 @@ void LstmLayer::ForwardPropInputAllSteps(int steps) {
     x_all = v_nodes_[0].p_device_h_t_below_;
   }
   lh_gemm_seg seg{p_device_m_stack_.get(), 4 * H, x_all, input_size_, input_size_};
-  ProfileScope ps(M.profiler_, kTagGateGemm, 4 * H, N, &seg, 1, 0, 0);
-  LhErrorWrapper(lh_gemm_f32(4 * H, N, &seg, 1, 0, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
-                             pre_x_all_.get(), 4 * H, s),
-                 "LstmLayer input products, all steps");
+  M.Gemm(kTagGateGemm, 4 * H, N, &seg, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr, pre_x_all_.get(),
+         4 * H, "LstmLayer input products, all steps");
 }
 
 // mw_fold_ = M_stack * W (4H x V): the input product of every vocabulary entry, for decoding.
@@ -304,9 +298,8 @@ void LstmLayer::BuildEmbeddingFold() {
   const int H = lstm_size_;
   if (mw_fold_.size() == 0) mw_fold_.Alloc((size_t)4 * H * vocab_size_);
   lh_gemm_seg seg{p_device_m_stack_.get(), 4 * H, p_device_w_.get(), input_size_, input_size_};
-  LhErrorWrapper(lh_gemm_f32(4 * H, vocab_size_, &seg, 1, 0, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
-                             mw_fold_.get(), 4 * H, M.stream_),
-                 "LstmLayer embedding fold");
+  M.Gemm(kTagGateGemm, 4 * H, vocab_size_, &seg, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
+         mw_fold_.get(), 4 * H, "LstmLayer embedding fold");
   mw_fold_dirty_ = false;
 }
 
@@ -403,17 +396,14 @@ void AttentionNode::ForwardProp() {
   Profiler &prof = A.p_neural_mt_->profiler_;
   if (!A.global_mode_) {
     lh_gemm_seg seg{A.p_device_w_p_.get(), H, ha, H, H};
-    ProfileScope ps(prof, kTagAttnProjGemm, H, B, &seg, 1, 0, 0);
-    LhErrorWrapper(lh_gemm_f32(H, B, &seg, 1, 0, 0, 1.f, 0.f, nullptr, LH_ACT_TANH, nullptr,
-                               p_device_tanh_1_, H, s),
-                   "AttentionNode::ForwardProp p_device_tanh_1_");
+    A.p_neural_mt_->Gemm(kTagAttnProjGemm, H, B, &seg, 1, 0, 0, 0.f, nullptr, LH_ACT_TANH, nullptr,
+                         p_device_tanh_1_, H, "AttentionNode::ForwardProp p_device_tanh_1_");
   }
   {
     lh_gemm_seg seg{A.p_device_w_a_.get(), H, ha, H, H};
-    ProfileScope ps(prof, kTagAttnProjGemm, H, B, &seg, 1, 1, 0);
-    LhErrorWrapper(lh_gemm_f32(H, B, &seg, 1, 1, 0, 1.f, 0.f, nullptr, LH_ACT_NONE, nullptr,
-                               p_device_h_t_wa_cache_, H, s),
-                   "AttentionNode::ForwardProp p_device_h_t_wa_cache_");
+    A.p_neural_mt_->Gemm(kTagAttnProjGemm, H, B, &seg, 1, 1, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
+                         p_device_h_t_wa_cache_, H,
+                         "AttentionNode::ForwardProp p_device_h_t_wa_cache_");
   }
   {
   ProfileScope ps(prof, kTagAttnCore, 4.0 * B * ((double)A.window_ * H + 2.0 * H + 2.0 * A.window_));
@@ -429,10 +419,9 @@ void AttentionNode::ForwardProp() {
   }
   lh_gemm_seg segs[2] = {{A.p_device_w_c_p1_.get(), H, p_device_c_t_, H, H},
                          {A.p_device_w_c_p2_.get(), H, ha, H, H}};
-  ProfileScope po(prof, kTagAttnOutGemm, H, B, segs, 2, 0, 0);
-  LhErrorWrapper(lh_gemm_f32(H, B, segs, 2, 0, 0, 1.f, 0.f, A.p_device_output_bias_.get(),
-                             LH_ACT_TANH, p_device_indices_mask_, p_device_final_tmp_2_, H, s),
-                 "AttentionNode::ForwardProp p_device_final_tmp_2_");
+  A.p_neural_mt_->Gemm(kTagAttnOutGemm, H, B, segs, 2, 0, 0, 0.f, A.p_device_output_bias_.get(),
+                       LH_ACT_TANH, p_device_indices_mask_, p_device_final_tmp_2_, H,
+                       "AttentionNode::ForwardProp p_device_final_tmp_2_");
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -489,12 +478,9 @@ void SoftmaxLayer::BackPropPreprocessGpu(float *p_device_h_t, int step) {
 void SoftmaxLayer::ComputeLogits(float *p_device_h_t, int minibatch) {
   // D*h with the bias of MatrixBiasKernel (deep_rnn_kernel.h:525) folded into the epilogue
   lh_gemm_seg seg{p_device_d_.get(), output_vocab_size_, p_device_h_t, lstm_size_, lstm_size_};
-  ProfileScope ps(p_neural_mt_->profiler_, kTagLogitsGemm, output_vocab_size_, minibatch, &seg, 1, 0,
-                  0);
-  LhErrorWrapper(lh_gemm_f32(output_vocab_size_, minibatch, &seg, 1, 0, 0, 1.f, 0.f,
-                             p_device_b_d_.get(), LH_ACT_NONE, nullptr, p_device_outputdist_.get(),
-                             output_vocab_size_, p_neural_mt_->stream_),
-                 "SoftmaxLayer::GetDistributionGpu p_device_outputdist");
+  p_neural_mt_->Gemm(kTagLogitsGemm, output_vocab_size_, minibatch, &seg, 1, 0, 0, 0.f,
+                     p_device_b_d_.get(), LH_ACT_NONE, nullptr, p_device_outputdist_.get(),
+                     output_vocab_size_, "SoftmaxLayer::GetDistributionGpu p_device_outputdist");
 }
 
 void SoftmaxLayer::GetDistributionGpu(float *p_device_h_t) {

@@ -12,6 +12,17 @@ NeuralMachineTranslation::NeuralMachineTranslation(const GlobalConfiguration &cf
   if (cfg_.embedding_size_ <= 0) cfg_.embedding_size_ = cfg_.lstm_size_;
   HipErrorWrapper(hipStreamCreate(&stream_), "stream creation failed");
   profiler_.stream_ = stream_;
+  gemm_workspace_.Alloc(kGemmWorkspaceBytes);
+}
+
+void NeuralMachineTranslation::Gemm(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg,
+                                    int trans_a, int trans_x, float beta, const float *bias, int act,
+                                    const int *colmask, float *C, int ldc, const char *what) {
+  ProfileScope ps(profiler_, tag, gemm_workspace_.size(), rows, cols, segs, nseg, trans_a, trans_x);
+  LhErrorWrapper(lh_gemm_ws_f32(rows, cols, segs, nseg, trans_a, trans_x, 1.f, beta, bias, act, rows,
+                                colmask, C, ldc, gemm_workspace_.get(), gemm_workspace_.size(),
+                                stream_),
+                 what);
 }
 
 NeuralMachineTranslation::~NeuralMachineTranslation() {

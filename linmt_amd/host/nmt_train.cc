@@ -33,10 +33,7 @@ int GateIndex(char g) {
 
 void Gemm(NeuralMachineTranslation &M, int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg,
           int tA, int tX, float beta, float *C, int ldc, const char *what) {
-  ProfileScope ps(M.profiler_, tag, rows, cols, segs, nseg, tA, tX);
-  LhErrorWrapper(lh_gemm_f32(rows, cols, segs, nseg, tA, tX, 1.f, beta, nullptr, LH_ACT_NONE, nullptr,
-                             C, ldc, M.stream_),
-                 what);
+  M.Gemm(tag, rows, cols, segs, nseg, tA, tX, beta, nullptr, LH_ACT_NONE, nullptr, C, ldc, what);
 }
 
 void RowSum(NeuralMachineTranslation &M, const float *A, long long lda, int rows, long long cols,
@@ -405,10 +402,8 @@ void SoftmaxLayer::ForwardBackwardAllSteps(const float *p_device_h_t_all, int st
     float *dz = dz_chunk_.get();
     {
       lh_gemm_seg seg{p_device_d_.get(), V, h, H, H};
-      ProfileScope ps(M.profiler_, kTagLogitsGemm, V, N, &seg, 1, 0, 0);
-      LhErrorWrapper(lh_gemm_f32(V, N, &seg, 1, 0, 0, 1.f, 0.f, p_device_b_d_.get(), LH_ACT_NONE,
-                                 nullptr, dz, V, s),
-                     "SoftmaxLayer::ForwardProp logits");
+      M.Gemm(kTagLogitsGemm, V, N, &seg, 1, 0, 0, 0.f, p_device_b_d_.get(), LH_ACT_NONE, nullptr, dz, V,
+             "SoftmaxLayer::ForwardProp logits");
     }
     {
       ProfileScope ps(M.profiler_, kTagSoftmaxGrad, 8.0 * V * N);

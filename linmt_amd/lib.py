@@ -40,9 +40,14 @@ SIGNATURES = {
     "lh_gemm_act_rows_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
                                        C.c_int, C.c_float, C.c_float, c_f32p, C.c_int, C.c_int,
                                        c_i32p, c_f32p, C.c_int, C.c_void_p]),
+    "lh_gemm_ws_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int, C.c_int,
+                                 C.c_float, C.c_float, c_f32p, C.c_int, C.c_int, c_i32p, c_f32p,
+                                 C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
     "lh_gemm_kernel_name": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
-                                      C.c_int, C.c_char_p, C.c_int]),
+                                      C.c_int, C.c_size_t, C.c_char_p, C.c_int]),
     "lh_gemm_set_config_override": (C.c_int, [C.c_int]),
+    "lh_gemm_set_splits_override": (C.c_int, [C.c_int]),
+    "lh_gemm_config_info": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int * 8)]),
     "lh_lstm_cell_fwd_f32": (C.c_int, [C.c_int, C.c_int, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p,
                                        c_i32p, C.c_int, C.c_float, c_f32p, c_f32p, c_f32p, c_f32p,
                                        C.c_float, c_f32p, C.c_void_p]),
@@ -162,10 +167,17 @@ def _segs(segs):
 
 
 def gemm(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0, bias=None,
-         act=LH_ACT_NONE, colmask=None, act_rows=None, stream=None):
-    """segs: list of (A, lda, X, ldx, K) with torch tensors A, X."""
+         act=LH_ACT_NONE, colmask=None, act_rows=None, workspace=None, stream=None):
+    """segs: list of (A, lda, X, ldx, K) with torch tensors A, X.  workspace: torch tensor
+    whose memory the K split may use (lh_gemm_ws_f32)."""
     arr = _segs(segs)
-    if act_rows is None:
+    if workspace is not None:
+        check(load().lh_gemm_ws_f32(M, N, arr, len(segs), int(transA), int(transX), alpha, beta,
+                                    _ptr(bias), act, M if act_rows is None else act_rows,
+                                    _ptr(colmask), _ptr(C_out), ldc, workspace.data_ptr(),
+                                    workspace.numel() * workspace.element_size(),
+                                    _stream(stream)), "lh_gemm_ws_f32")
+    elif act_rows is None:
         check(load().lh_gemm_f32(M, N, arr, len(segs), int(transA), int(transX), alpha, beta,
                                  _ptr(bias), act, _ptr(colmask), _ptr(C_out), ldc,
                                  _stream(stream)), "lh_gemm_f32")
@@ -176,11 +188,19 @@ def gemm(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0
               "lh_gemm_act_rows_f32")
 
 
-def gemm_kernel_name(M, N, segs, transA=False, transX=False):
+def gemm_kernel_name(M, N, segs, transA=False, transX=False, workspace_bytes=0):
     buf = C.create_string_buffer(128)
-    check(load().lh_gemm_kernel_name(M, N, _segs(segs), len(segs), int(transA), int(transX), buf,
-                                     128), "lh_gemm_kernel_name")
+    check(load().lh_gemm_kernel_name(M, N, _segs(segs), len(segs), int(transA), int(transX),
+                                     workspace_bytes, buf, 128), "lh_gemm_kernel_name")
     return buf.value.decode()
+
+
+def gemm_config_info(config, transA=False, transX=False):
+    """dict(BM, BN, WM, WN, WK, BK, occupancy, lds_bytes) of one tile configuration."""
+    info = (C.c_int * 8)()
+    check(load().lh_gemm_config_info(config, int(transA), int(transX), C.byref(info)),
+          "lh_gemm_config_info")
+    return dict(zip(("BM", "BN", "WM", "WN", "WK", "BK", "occupancy", "lds_bytes"), list(info)))
 
 
 def lstm_cell_fwd(H, B, pre1, bias4h, c_prev, mask01, c, h, pre2=None, pre3=None,

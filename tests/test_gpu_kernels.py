@@ -106,6 +106,53 @@ def test_gemm_vs_float64(lh, M, N, Ks, tA, tX):
     assert_close(host(out, (M, N)), want2, "epilogue")
 
 
+def test_gemm_split_k(lh):
+    """K split across workgroups (lh_gemm_ws_f32): forced split counts on several tile
+    configurations, ragged edges, several segments with K tails, the full epilogue; repeated calls
+    give identical bits whatever the workspace held before."""
+    rng = np.random.default_rng(22)
+    L = lh.load()
+    n_cfg = L.lh_gemm_set_config_override(-1)
+    max_split = L.lh_gemm_set_splits_override(0)
+    assert max_split >= 8
+    ws = torch.full((2 << 20,), float("nan"), device="cuda")
+    shapes = [(200, 76, (100, 36), False, False), (132, 100, (260,), True, False),
+              (96, 36, (40, 24, 72), False, True), (1000, 96, (1000, 1000), False, False)]
+    try:
+        for cfg in (0, 3, 5, 7, 11, 14, 19):
+            assert L.lh_gemm_set_config_override(cfg) == n_cfg
+            for splits in (2, 3, 7, max_split):
+                assert L.lh_gemm_set_splits_override(splits) == max_split
+                for M, N, Ks, tA, tX in shapes:
+                    As = [uni(rng, *((K, M) if tA else (M, K)), s=0.5) for K in Ks]
+                    Xs = [uni(rng, *((N, K) if tX else (K, N))) for K in Ks]
+                    acc = sum((A.T if tA else A).astype(np.float64) @ (X.T if tX else X)
+                              for A, X in zip(As, Xs))
+                    segs = [(dev(A), A.shape[0], dev(X), X.shape[0], K)
+                            for A, X, K in zip(As, Xs, Ks)]
+                    bias = uni(rng, M)
+                    cmask = rng.integers(0, 2, size=N).astype(np.int32)
+                    C0 = uni(rng, M, N)
+                    want = np.tanh(-0.5 * acc + 0.25 * C0 + bias[:, None]) * cmask[None, :]
+                    outs = []
+                    for _ in range(2):
+                        out = dev(C0)
+                        lh.gemm(M, N, segs, out, M, transA=tA, transX=tX, alpha=-0.5, beta=0.25,
+                                bias=dev(bias), act=lh.LH_ACT_TANH, colmask=dev(cmask),
+                                workspace=ws)
+                        outs.append(host(out, (M, N)))
+                    what = f"config {cfg} splits {splits} shape {(M, N, Ks, tA, tX)}"
+                    assert_close(outs[0], want, what)
+                    assert np.array_equal(outs[0], outs[1]), what + ": not reproducible"
+    finally:
+        L.lh_gemm_set_config_override(-1)
+        L.lh_gemm_set_splits_override(0)
+    info = lh.gemm_config_info(3)
+    assert (info["BM"], info["BN"], info["BK"]) == (128, 64, 16) and info["occupancy"] >= 1
+    with pytest.raises(lh.LinmtHipError):
+        lh.check(L.lh_gemm_set_splits_override(10 ** 6), "override")
+
+
 def test_gemm_every_tile_configuration(lh):
     """Each tile configuration (incl. the intra-workgroup split-K ones) on shapes with ragged edges,
     several K segments and both transposes; also the row-limited activation and the kernel name."""
