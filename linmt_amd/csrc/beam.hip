@@ -31,6 +31,7 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
   __shared__ short s_col[kMaxCand];
   __shared__ short s_order[kMaxCand];
   __shared__ unsigned char s_flag[kMaxCand];
+  __shared__ int s_total[2];  // slot-taking candidates; finished hypotheses the walk reaches
 
   const int s = blockIdx.x, tid = threadIdx.x;
   const int beam = a.beam, K = a.K;
@@ -56,6 +57,7 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
 
   const int cols = a.step == 0 ? 1 : beam;
   const int C = cols * K;
+  if (tid < 2) s_total[tid] = 0;
   for (int e = tid; e < C; e += kMergeThreads) {
     const int i = e / K, k = e % K;
     const float rank_penalty = (float)(k + 1) * a.diversity;
@@ -93,10 +95,12 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
       fins += f == 2 ? 1 : 0;
     }
     const int f = s_flag[r];
+    if (f == 1) atomicAdd(&s_total[0], 1);
     if (slots < beam && f != 0) {
       const int e = s_order[r];
       const float sc = s_score[e] + a.penalty;
       if (f == 2) {
+        atomicAdd(&s_total[1], 1);
         if (fins < beam) {  // at most one <EOF> candidate per column exists
           a.fin_beam[c0 + fins] = s_col[e];
           a.fin_score[c0 + fins] = sc;
@@ -108,21 +112,14 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
       }
     }
   }
-  if (tid == 0) {
-    // totals: slots filled (the rest is padding) and finished hypotheses recorded
-    int filled = 0, nfin = 0;
-    for (int r = 0; r < C && filled < beam; ++r) {
-      const int f = s_flag[r];
-      filled += f == 1 ? 1 : 0;
-      nfin += (f == 2 && nfin < beam) ? 1 : 0;
-    }
-    for (; filled < beam; ++filled) {  // candidates exhausted (the reference pops an empty heap)
-      a.tok[c0 + filled] = a.eof_id;
-      a.backptr[c0 + filled] = c0;
-      a.score[c0 + filled] = -FLT_MAX;
-    }
-    a.fin_count[s] = nfin;
+  __syncthreads();
+  // slots left empty when the candidates run out (the reference pops an empty heap)
+  for (int i = min(s_total[0], beam) + tid; i < beam; i += kMergeThreads) {
+    a.tok[c0 + i] = a.eof_id;
+    a.backptr[c0 + i] = c0;
+    a.score[c0 + i] = -FLT_MAX;
   }
+  if (tid == 0) a.fin_count[s] = min(s_total[1], beam);
 }
 
 struct GatherArgs {
