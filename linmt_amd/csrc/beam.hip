@@ -4,7 +4,8 @@
 
 namespace {
 
-constexpr int kMergeThreads = 256;
+constexpr int kMergeThreads = 1024;
+constexpr int kParts = 4;  // lanes that share one candidate in the merge
 constexpr int kMaxCand = 4096;
 
 struct MergeArgs {
@@ -67,33 +68,45 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
   }
   __syncthreads();
   // rank of every candidate in the total order; s_order[rank] = candidate, s_flag[rank] = what the
-  // walk does with it (1 takes a slot, 2 finished hypothesis, 0 dropped <START>)
-  for (int e = tid; e < C; e += kMergeThreads) {
+  // walk does with it (1 takes a slot, 2 finished hypothesis, 0 dropped <START>).  Four
+  // neighbouring lanes share a candidate and each compares it with a quarter of the others.
+  const int part = tid % kParts;
+  for (int e = tid / kParts; e < C; e += kMergeThreads / kParts) {
     const float sc = s_score[e];
     const int id = s_id[e], col = s_col[e];
     int before = 0;
 #pragma unroll 4
-    for (int o = 0; o < C; ++o) {
+    for (int o = part; o < C; o += kParts) {
       const float so = s_score[o];
       const bool first = so > sc || (so == sc && (s_col[o] < col || (s_col[o] == col && s_id[o] < id)));
       before += first ? 1 : 0;
     }
-    s_order[before] = (short)e;
-    s_flag[before] = id == a.start_id ? 0 : (id == a.eof_id ? 2 : 1);
+#pragma unroll
+    for (int d = 1; d < kParts; d *= 2) before += __shfl_xor(before, d);
+    if (part == 0) {
+      s_order[before] = (short)e;
+      s_flag[before] = id == a.start_id ? 0 : (id == a.eof_id ? 2 : 1);
+    }
   }
   __syncthreads();
   // The reference pops the global heap until `beam` slots are filled.  Entry r is reached iff fewer
   // than `beam` slot-taking entries precede it; its slot / finished index is the count of such
-  // entries before it -- a prefix count every thread takes for its own entries, so nothing walks
+  // entries before it -- a prefix count taken per entry (again by four lanes), so nothing walks
   // the list serially.
-  for (int r = tid; r < C; r += kMergeThreads) {
+  for (int r = tid / kParts; r < C; r += kMergeThreads / kParts) {
     int slots = 0, fins = 0;
 #pragma unroll 4
-    for (int q = 0; q < r; ++q) {
+    for (int q = part; q < r; q += kParts) {
       const int f = s_flag[q];
       slots += f == 1 ? 1 : 0;
       fins += f == 2 ? 1 : 0;
     }
+#pragma unroll
+    for (int d = 1; d < kParts; d *= 2) {
+      slots += __shfl_xor(slots, d);
+      fins += __shfl_xor(fins, d);
+    }
+    if (part != 0) continue;
     const int f = s_flag[r];
     if (f == 1) atomicAdd(&s_total[0], 1);
     if (slots < beam && f != 0) {
