@@ -122,6 +122,43 @@ int lnmt_profile_count(lnmt_model *m);
 int lnmt_profile_entry(lnmt_model *m, int index, char *name, int name_cap, double *ms, double *work,
                        long long *launches);
 
+/* ------------------------------------------------------------------------------------------
+ * Files either side of the path.
+ *
+ * Model file: the reference's text checkpoint (first line "layers lstm_size target_vocab
+ * source_vocab attention feed_input multi_source combine_lstm char_cnn", the two vocabulary
+ * mappings between lines of '=', then every matrix as rows of numbers and an empty line).
+ * lnmt_read_model_information = the first-line parse the reference does before it builds a
+ * decoder (info[9] in the order above); lnmt_model_load_weights =
+ * NeuralMachineTranslation::LoadWeights (src/deep_rnn.h:1878-1968) and fails when the header does
+ * not describe the model; lnmt_model_dump_model writes a complete file (header, placeholder
+ * vocabulary mappings, DumpWeights src/deep_rnn.h:2124-2146) that the reference can load. */
+int lnmt_read_model_information(const char *model_file, int info[9]);
+int lnmt_model_load_weights(lnmt_model *m, const char *model_file);
+int lnmt_model_dump_model(lnmt_model *m, const char *model_file);
+/* Parameter names in model-file order: returns the count; name i is copied into `name`. */
+int lnmt_model_file_param(lnmt_model *m, int index, char *name, int name_cap, int *rows, int *cols);
+
+/* FileHelper (src/file_helper.h:28-112): reader of the reference's integerised training file
+ * (four lines per sentence pair, all pairs of a minibatch padded to common lengths).
+ * source_vocab_size = -1 for a target-side language model.  lnmt_file_helper_read_minibatch =
+ * ReadMinibatch (src/file_helper.cc:113-272): returns 1 while the epoch continues, 0 when this
+ * read reached the end of the file, -1 on error.  After it, lnmt_file_helper_get copies one of the
+ * arrays (what: 0 source input, 1 source output, 2 target input, 3 target output -- all
+ * minibatch x length column-major --, 4 / 5 source / target *_wgrad lists, 6 batch information)
+ * into `data` (n = capacity in ints) and returns the number of valid entries;
+ * lnmt_file_helper_info fills {current_source_length, current_target_length,
+ * words_in_minibatch, length_source_wgrad, length_target_wgrad, nums_lines_in_file, total_words,
+ * total_target_words}. */
+typedef struct lnmt_file_helper lnmt_file_helper;
+lnmt_file_helper *lnmt_file_helper_create(const char *file_name, int minibatch_size,
+                                          int longest_sentence, int source_vocab_size,
+                                          int target_vocab_size);
+void lnmt_file_helper_destroy(lnmt_file_helper *f);
+int lnmt_file_helper_read_minibatch(lnmt_file_helper *f);
+int lnmt_file_helper_get(lnmt_file_helper *f, int what, int *data, long long n);
+int lnmt_file_helper_info(lnmt_file_helper *f, int info[8]);
+
 #ifdef __cplusplus
 }
 #endif

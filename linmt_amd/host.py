@@ -80,6 +80,18 @@ def load():
     lib.lnmt_profile_entry.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.c_int,
                                        C.POINTER(C.c_double), C.POINTER(C.c_double),
                                        C.POINTER(C.c_longlong)]
+    lib.lnmt_read_model_information.argtypes = [C.c_char_p, C.POINTER(C.c_int * 9)]
+    lib.lnmt_model_load_weights.argtypes = [C.c_void_p, C.c_char_p]
+    lib.lnmt_model_dump_model.argtypes = [C.c_void_p, C.c_char_p]
+    lib.lnmt_model_file_param.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.c_int,
+                                          C.POINTER(C.c_int), C.POINTER(C.c_int)]
+    lib.lnmt_file_helper_create.restype = C.c_void_p
+    lib.lnmt_file_helper_create.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]
+    lib.lnmt_file_helper_destroy.argtypes = [C.c_void_p]
+    lib.lnmt_file_helper_destroy.restype = None
+    lib.lnmt_file_helper_read_minibatch.argtypes = [C.c_void_p]
+    lib.lnmt_file_helper_get.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_longlong]
+    lib.lnmt_file_helper_info.argtypes = [C.c_void_p, C.POINTER(C.c_int * 8)]
     _lib = lib
     return lib
 
@@ -165,6 +177,26 @@ class Model:
         _check(load().lnmt_model_get_param(self.handle, name.encode(), _p(out), out.size),
                f"get_param({name})")
         return out.reshape(shape, order="F")
+
+    def load_weights(self, path):
+        """NeuralMachineTranslation::LoadWeights: fill the parameters from a reference model file."""
+        _check(load().lnmt_model_load_weights(self.handle, os.fsencode(path)), "load_weights")
+
+    def dump_model(self, path):
+        """Write a complete reference-format model file (placeholder vocabulary mappings)."""
+        _check(load().lnmt_model_dump_model(self.handle, os.fsencode(path)), "dump_model")
+
+    def model_file_order(self):
+        """[(name, rows, cols)] in the order the model file stores the matrices."""
+        lib, out = load(), []
+        name, r, c = C.create_string_buffer(64), C.c_int(), C.c_int()
+        n = lib.lnmt_model_file_param(self.handle, 0, name, 64, C.byref(r), C.byref(c))
+        if n < 0:
+            _check(-1, "model_file_order")
+        for i in range(n):
+            lib.lnmt_model_file_param(self.handle, i, name, 64, C.byref(r), C.byref(c))
+            out.append((name.value.decode(), r.value, c.value))
+        return out
 
     def get_error(self, src, tgt_in, tgt_out, batch_info):
         """src (B,S), tgt_in/tgt_out (B,T) int arrays, -1 padding; returns sum log p(target)."""
@@ -252,3 +284,64 @@ class Model:
                 r["hyps"] = [(ht[i, j, :hl[i, j]].copy(), float(hs[i, j])) for j in range(k)]
             res.append(r)
         return res
+
+
+def read_model_information(path):
+    """dict of the first line of a reference model file."""
+    info = (C.c_int * 9)()
+    _check(load().lnmt_read_model_information(os.fsencode(path), C.byref(info)),
+           "read_model_information")
+    keys = ("num_layers", "lstm_size", "target_vocab_size", "source_vocab_size", "attention_model",
+            "feed_input", "multi_source", "combine_lstm", "char_cnn")
+    return dict(zip(keys, list(info)))
+
+
+class FileHelper:
+    """The reference's training-file reader (FileHelper, src/file_helper.h): four lines per
+    sentence pair; read_minibatch() returns the arrays of one minibatch."""
+
+    ARRAYS = ("source_in", "source_out", "target_in", "target_out", "source_wgrad", "target_wgrad",
+              "batch_information")
+
+    def __init__(self, path, minibatch_size, longest_sentence, source_vocab_size,
+                 target_vocab_size):
+        self.B, self.cap = minibatch_size, minibatch_size * longest_sentence
+        self.handle = load().lnmt_file_helper_create(os.fsencode(path), minibatch_size,
+                                                     longest_sentence, source_vocab_size,
+                                                     target_vocab_size)
+        if not self.handle:
+            _check(-1, "FileHelper")
+
+    def close(self):
+        if self.handle:
+            load().lnmt_file_helper_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def read_minibatch(self):
+        """(same_epoch, dict): id blocks as (B, length) arrays, the two unique-id lists, the batch
+        information and the counters of FileHelper."""
+        lib = load()
+        rc = lib.lnmt_file_helper_read_minibatch(self.handle)
+        if rc < 0:
+            _check(-1, "read_minibatch")
+        info = (C.c_int * 8)()
+        _check(lib.lnmt_file_helper_info(self.handle, C.byref(info)), "file_helper_info")
+        S, T = info[0], info[1]
+        out = dict(current_source_length=S, current_target_length=T, words_in_minibatch=info[2],
+                   nums_lines_in_file=info[5], total_words=info[6], total_target_words=info[7])
+        buf = np.empty(max(self.cap, 2 * self.B), np.int32)
+        for what, key in enumerate(self.ARRAYS):
+            n = lib.lnmt_file_helper_get(self.handle, what, _p(buf), buf.size)
+            if n < 0:
+                _check(-1, f"file_helper_get({key})")
+            a = buf[:n].copy()
+            if what < 4:
+                a = a.reshape((self.B, S if what < 2 else T), order="F")
+            out[key] = a
+        return bool(rc), out

@@ -4,6 +4,7 @@
 #include <memory>
 
 #include "../../include/linmt_host.h"
+#include "file_helper.h"
 #include "nmt.h"
 
 using namespace linmt;
@@ -279,5 +280,97 @@ extern "C" int lnmt_profile_entry(lnmt_model *m, int index, char *name, int name
     *ms = it->second.ms;
     *work = it->second.work;
     *launches = it->second.launches;
+  });
+}
+
+// ---- files either side of the path -------------------------------------------------------------
+extern "C" int lnmt_read_model_information(const char *model_file, int info[9]) {
+  return Guard([&] {
+    const ModelInformation m = ReadModelInformation(model_file);
+    const int v[9] = {m.num_layers,  m.lstm_size,    m.target_vocab_size, m.source_vocab_size, m.attention_model,
+                      m.feed_input,  m.multi_source, m.combine_lstm,      m.char_cnn};
+    std::copy(v, v + 9, info);
+  });
+}
+
+extern "C" int lnmt_model_load_weights(lnmt_model *m, const char *model_file) {
+  return Guard([&] { m->nmt->LoadWeights(model_file); });
+}
+
+extern "C" int lnmt_model_dump_model(lnmt_model *m, const char *model_file) {
+  return Guard([&] { m->nmt->DumpModel(model_file, nullptr, nullptr); });
+}
+
+extern "C" int lnmt_model_file_param(lnmt_model *m, int index, char *name, int name_cap, int *rows,
+                                     int *cols) {
+  int count = -1;
+  Guard([&] {
+    const auto order = m->nmt->ModelFileOrder();
+    if (index >= 0 && index < (int)order.size() && name && name_cap > 0) {
+      snprintf(name, name_cap, "%s", order[index].name.c_str());
+      if (rows) *rows = order[index].rows;
+      if (cols) *cols = order[index].cols;
+    }
+    count = (int)order.size();
+  });
+  return count;
+}
+
+struct lnmt_file_helper {
+  std::unique_ptr<FileHelper> fh;
+};
+
+extern "C" lnmt_file_helper *lnmt_file_helper_create(const char *file_name, int minibatch_size,
+                                                     int longest_sentence, int source_vocab_size,
+                                                     int target_vocab_size) {
+  lnmt_file_helper *f = nullptr;
+  Guard([&] {
+    std::unique_ptr<lnmt_file_helper> p(new lnmt_file_helper());
+    p->fh.reset(new FileHelper(file_name, minibatch_size, longest_sentence, source_vocab_size,
+                               target_vocab_size));
+    f = p.release();
+  });
+  return f;
+}
+
+extern "C" void lnmt_file_helper_destroy(lnmt_file_helper *f) { delete f; }
+
+extern "C" int lnmt_file_helper_read_minibatch(lnmt_file_helper *f) {
+  int same_epoch = 0;
+  if (Guard([&] { same_epoch = f->fh->ReadMinibatch() ? 1 : 0; }) != 0) return -1;
+  return same_epoch;
+}
+
+extern "C" int lnmt_file_helper_get(lnmt_file_helper *f, int what, int *data, long long n) {
+  int valid = -1;
+  Guard([&] {
+    const FileHelper &h = *f->fh;
+    const std::vector<int> *v = nullptr;
+    long long count = 0;
+    const long long B = h.minibatch_size_;
+    switch (what) {
+      case 0: v = &h.p_host_input_vocab_indices_source_; count = B * h.current_source_length_; break;
+      case 1: v = &h.p_host_output_vocab_indices_source_; count = B * h.current_source_length_; break;
+      case 2: v = &h.p_host_input_vocab_indices_target_; count = B * h.current_target_length_; break;
+      case 3: v = &h.p_host_output_vocab_indices_target_; count = B * h.current_target_length_; break;
+      case 4: v = &h.p_host_input_vocab_indices_source_wgrad_; count = h.length_source_wgrad_; break;
+      case 5: v = &h.p_host_input_vocab_indices_target_wgrad_; count = h.length_target_wgrad_; break;
+      case 6: v = &h.p_host_batch_information_; count = 2 * B; break;
+      default: throw LinmtError("lnmt_file_helper_get: unknown array " + std::to_string(what));
+    }
+    if (count > n) throw LinmtError("lnmt_file_helper_get: the buffer is too small");
+    std::copy(v->begin(), v->begin() + count, data);
+    valid = (int)count;
+  });
+  return valid;
+}
+
+extern "C" int lnmt_file_helper_info(lnmt_file_helper *f, int info[8]) {
+  return Guard([&] {
+    const FileHelper &h = *f->fh;
+    const int v[8] = {h.current_source_length_, h.current_target_length_, h.words_in_minibatch_,
+                      h.length_source_wgrad_,   h.length_target_wgrad_,   h.nums_lines_in_file_,
+                      h.total_words_,           h.total_target_words_};
+    std::copy(v, v + 8, info);
   });
 }

@@ -339,6 +339,13 @@ struct SentenceResult {
   int steps = 0;                       // decoder forward passes this sentence took part in
 };
 
+// First line of a model file (src/utility_cc.cc:76-98, written by AddModelInformation).
+struct ModelInformation {
+  int num_layers = 0, lstm_size = 0, target_vocab_size = 0, source_vocab_size = 0;
+  int attention_model = 0, feed_input = 0, multi_source = 0, combine_lstm = 0, char_cnn = 0;
+};
+ModelInformation ReadModelInformation(const std::string &model_file);
+
 class Decoder {
  public:
   static constexpr int start_symbol_ = 0, end_symbol_ = 1;
@@ -431,6 +438,23 @@ class NeuralMachineTranslation {
   bool SetParam(const std::string &name, const float *host, size_t n);
   bool GetParam(const std::string &name, std::vector<float> *out);
   void Synchronize();
+
+  // ---- model file (host/model_io.cc) -------------------------------------------------------------
+  // The reference's text model file: header line, the two vocabulary mappings between lines of
+  // '=', then every matrix as rows of numbers followed by an empty line, in the order of
+  // DumpWeights (deep_rnn.h:2124-2146).  LoadWeights (deep_rnn.h:1878-1968) checks the header
+  // against cfg_ and fills the parameters; DumpWeights appends the matrices to a file that already
+  // holds the header part; DumpModel writes header, mappings (null: placeholder words) and matrices.
+  void LoadWeights(const std::string &input_weight_file);
+  void DumpWeights(const std::string &output_weight_file);
+  void DumpModel(const std::string &output_weight_file, const std::vector<std::string> *source_words,
+                 const std::vector<std::string> *target_words);
+  // every parameter name in the order the model file stores them, with its (rows, cols)
+  struct ParamShape {
+    std::string name;
+    int rows, cols;
+  };
+  std::vector<ParamShape> ModelFileOrder() const;
 
  private:
   // encoder + decoder + attention of a teacher-forced minibatch (shared by GetError and

@@ -1,0 +1,80 @@
+"""The reference's text model file through the C++ layer classes: LoadWeights on a hand-made file
+whose numbers say which matrix / row / column they are (tests/golden/tiny_model.nmt), and
+DumpModel -> LoadWeights round trips.  The matrix order checked here is the one the reference's
+DumpWeightsGpu functions write (layer_input_to_hidden.h:1556-1590: W_h*/b_* interleaved, W, then
+M_i M_f M_o M_c, then Q_i Q_f Q_o Q_c; attention after the last target layer; softmax last).
+Parity unpinned against a reference-written model file: the checkout holds none."""
+import os
+
+import numpy as np
+import pytest
+
+import ref_numpy as R
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module")
+def host():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from linmt_amd import host as h
+    h.load()
+    return h
+
+
+def test_load_weights_puts_every_matrix_where_the_reference_order_says(host):
+    L, H, Vt, Vs = 2, 3, 6, 5
+    m = host.Model(L, H, Vs, Vt, longest_sentence=10, attention_mode=1, attention_width=2,
+                   feed_input=True, minibatch_size=2)
+    m.load_weights(os.path.join(GOLDEN, "tiny_model.nmt"))
+    # the file's k-th matrix holds k + i/10 + j/100 at (i, j); walk the order independently
+    names = []
+    for side, vocab, feed in (("src", Vs, False), ("tgt", Vt, True)):
+        for l in range(L):
+            p = f"{side}.{l}."
+            for g in "ifco":
+                names += [(p + "W_h" + g, (H, H)), (p + "b_" + g, (H, 1))]
+            if l == 0:
+                names.append((p + "W", (H, vocab)))
+            names += [(p + "M_" + g, (H, H)) for g in "ifoc"]
+            if feed and l == 0:
+                names += [(p + "Q_" + g, (H, H)) for g in "ifoc"]
+    names += [("attn.W_a", (H, H)), ("attn.W_p", (H, H)), ("attn.v_p", (H, 1)), ("attn.b_out", (H, 1)),
+              ("attn.W_c1", (H, H)), ("attn.W_c2", (H, H)), ("softmax.D", (Vt, H)), ("softmax.b_d", (Vt, 1))]
+    assert [(n, r, c) for n, (r, c) in names] == m.model_file_order()
+    for k, (name, (r, c)) in enumerate(names):
+        want = k + np.arange(r)[:, None] / 10 + np.arange(c)[None, :] / 100
+        got = m.get_param(name, (r, c))
+        assert np.allclose(got, want, rtol=0, atol=1e-5), name
+
+
+@pytest.mark.parametrize("layers,attention,feed,s2s", [(1, 1, True, True), (3, 1, False, True),
+                                                       (2, 0, False, True), (2, 0, False, False)])
+def test_dump_then_load_round_trip(host, tmp_path, layers, attention, feed, s2s):
+    rng = np.random.default_rng(5)
+    H, Vs, Vt = 8, 11, 13
+    P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(attention), feed_input=feed, scale=0.5)
+    if not s2s:
+        P = {k: v for k, v in P.items() if not k.startswith("src.")}
+    kw = dict(longest_sentence=12, attention_mode=attention, attention_width=3, feed_input=feed,
+              minibatch_size=2, sequence_to_sequence=s2s)
+    a = host.Model(layers, H, Vs, Vt, **kw)
+    a.set_params(P)
+    path = str(tmp_path / "model.nmt")
+    a.dump_model(path)
+    info = host.read_model_information(path)
+    assert (info["num_layers"], info["lstm_size"], info["target_vocab_size"]) == (layers, H, Vt)
+    assert info["attention_model"] == int(bool(attention)) and info["feed_input"] == int(feed)
+    b = host.Model(layers, H, Vs, Vt, **kw)
+    b.load_weights(path)
+    for name, arr in P.items():
+        got = b.get_param(name, np.atleast_2d(arr.reshape(arr.shape[0], -1)).shape)
+        # the reference writes digits10 + 2 = 8 significant digits
+        assert np.allclose(got, arr.reshape(got.shape), rtol=1e-7, atol=0), name
+    # a file for another architecture is refused
+    c = host.Model(layers + 1, H, Vs, Vt, **kw)
+    with pytest.raises(host.HostError):
+        c.load_weights(path)
