@@ -129,7 +129,8 @@ int lnmt_profile_entry(lnmt_model *m, int index, char *name, int name_cap, doubl
  * source_vocab attention feed_input multi_source combine_lstm char_cnn", the two vocabulary
  * mappings between lines of '=', then every matrix as rows of numbers and an empty line).
  * lnmt_read_model_information = the first-line parse the reference does before it builds a
- * decoder (info[9] in the order above); lnmt_model_load_weights =
+ * decoder (DecoderModelWrapper::ExtractModelInformation, src/decoder.h:1182-1210; info[9] in the
+ * order above); lnmt_model_load_weights =
  * NeuralMachineTranslation::LoadWeights (src/deep_rnn.h:1878-1968) and fails when the header does
  * not describe the model; lnmt_model_dump_model writes a complete file (header, placeholder
  * vocabulary mappings, DumpWeights src/deep_rnn.h:2124-2146) that the reference can load. */

@@ -339,7 +339,8 @@ struct SentenceResult {
   int steps = 0;                       // decoder forward passes this sentence took part in
 };
 
-// First line of a model file (src/utility_cc.cc:76-98, written by AddModelInformation).
+// First line of a model file: written by AddModelInformation (src/utility_cc.cc:76-98), parsed by
+// DecoderModelWrapper::ExtractModelInformation (src/decoder.h:1182-1210).
 struct ModelInformation {
   int num_layers = 0, lstm_size = 0, target_vocab_size = 0, source_vocab_size = 0;
   int attention_model = 0, feed_input = 0, multi_source = 0, combine_lstm = 0, char_cnn = 0;
