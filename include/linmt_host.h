@@ -160,6 +160,38 @@ int lnmt_file_helper_read_minibatch(lnmt_file_helper *f);
 int lnmt_file_helper_get(lnmt_file_helper *f, int what, int *data, long long n);
 int lnmt_file_helper_info(lnmt_file_helper *f, int info[8]);
 
+/* Dispatcher::Tuning (src/dispatcher.cu:96-384): the training loop -- minibatches from the
+ * training file, ComputeGradients + UpdateWeights, the reference's learning-rate schedules
+ * (google: halve at the half epoch and after every epoch from epoch_to_start_halving on; stanford:
+ * halve after every epoch from epoch_to_start_halving_full on; schedule: multiply by
+ * decrease_factor when dev perplexity + margin >= the previous one), best-model dumping, final
+ * model file.  The model must have been created with lnmt_model_create_training.  Events
+ * (kind: 0 words/s over the last screen_print_rate minibatches, 1 dev perplexity at the half
+ * epoch, 2 dev perplexity at the epoch's end, 3 new learning rate, 4 best model dumped (its
+ * perplexity), 5 epoch end (summed training log-likelihood), 6 final model written) are copied
+ * into `events` up to event_cap; *n_events receives how many happened. */
+typedef struct lnmt_tuning_options {
+  const char *train_file, *dev_file;               /* integerised files (dev_file may be NULL) */
+  const char *output_weight_file, *best_model_file; /* NULL = not written */
+  int epochs;
+  int google_learning_rate, epoch_to_start_halving;
+  int stanford_learning_rate, epoch_to_start_halving_full;
+  int learning_rate_schedule;
+  float decrease_factor;
+  double margin;
+  int best_model_mode;
+  int screen_print_rate;
+} lnmt_tuning_options;
+typedef struct lnmt_tuning_event {
+  int kind, epoch, minibatch;
+  double value;
+} lnmt_tuning_event;
+int lnmt_tuning(lnmt_model *m, const lnmt_tuning_options *o, lnmt_tuning_event *events,
+                int event_cap, int *n_events, long long *words, double *seconds,
+                float *final_learning_rate);
+/* NeuralMachineTranslation::GetPerplexity (src/deep_rnn.h:1490-1568) over an integerised file. */
+int lnmt_get_perplexity(lnmt_model *m, const char *file_name, double *perplexity);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,21 @@ class TrainOptions(C.Structure):
                 ("dropout_keep", C.c_float), ("dropout_seed", C.c_ulonglong)]
 
 
+class TuningOptions(C.Structure):
+    _fields_ = [("train_file", C.c_char_p), ("dev_file", C.c_char_p),
+                ("output_weight_file", C.c_char_p), ("best_model_file", C.c_char_p),
+                ("epochs", C.c_int), ("google_learning_rate", C.c_int),
+                ("epoch_to_start_halving", C.c_int), ("stanford_learning_rate", C.c_int),
+                ("epoch_to_start_halving_full", C.c_int), ("learning_rate_schedule", C.c_int),
+                ("decrease_factor", C.c_float), ("margin", C.c_double),
+                ("best_model_mode", C.c_int), ("screen_print_rate", C.c_int)]
+
+
+class TuningEvent(C.Structure):
+    _fields_ = [("kind", C.c_int), ("epoch", C.c_int), ("minibatch", C.c_int),
+                ("value", C.c_double)]
+
+
 class DecodeOptions(C.Structure):
     _fields_ = [("beam_size", C.c_int), ("max_decoding_ratio", C.c_float),
                 ("min_decoding_ratio", C.c_float), ("penalty", C.c_float),
@@ -92,6 +107,10 @@ def load():
     lib.lnmt_file_helper_read_minibatch.argtypes = [C.c_void_p]
     lib.lnmt_file_helper_get.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_longlong]
     lib.lnmt_file_helper_info.argtypes = [C.c_void_p, C.POINTER(C.c_int * 8)]
+    lib.lnmt_tuning.argtypes = [C.c_void_p, C.POINTER(TuningOptions), C.POINTER(TuningEvent),
+                                C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_longlong),
+                                C.POINTER(C.c_double), C.POINTER(C.c_float)]
+    lib.lnmt_get_perplexity.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_double)]
     _lib = lib
     return lib
 
@@ -177,6 +196,38 @@ class Model:
         _check(load().lnmt_model_get_param(self.handle, name.encode(), _p(out), out.size),
                f"get_param({name})")
         return out.reshape(shape, order="F")
+
+    EVENT_KINDS = ("speed", "half_epoch_perplexity", "epoch_perplexity", "learning_rate",
+                   "dump_best_model", "epoch_end", "dump_final")
+
+    def tuning(self, train_file, dev_file=None, output_weight_file=None, best_model_file=None,
+               epochs=10, google_learning_rate=False, epoch_to_start_halving=6,
+               stanford_learning_rate=False, epoch_to_start_halving_full=6,
+               learning_rate_schedule=False, decrease_factor=0.5, margin=0.0,
+               best_model_mode=False, screen_print_rate=20):
+        """Dispatcher::Tuning.  Returns dict(events=[(kind, epoch, minibatch, value)], words,
+        seconds, final_learning_rate)."""
+        enc = lambda p: None if p is None else os.fsencode(p)  # noqa: E731
+        o = TuningOptions(enc(train_file), enc(dev_file), enc(output_weight_file),
+                          enc(best_model_file), epochs, int(google_learning_rate),
+                          epoch_to_start_halving, int(stanford_learning_rate),
+                          epoch_to_start_halving_full, int(learning_rate_schedule),
+                          decrease_factor, margin, int(best_model_mode), screen_print_rate)
+        cap = 65536
+        ev = (TuningEvent * cap)()
+        n, words, secs, lr = C.c_int(), C.c_longlong(), C.c_double(), C.c_float()
+        _check(load().lnmt_tuning(self.handle, C.byref(o), ev, cap, C.byref(n), C.byref(words),
+                                  C.byref(secs), C.byref(lr)), "tuning")
+        events = [(self.EVENT_KINDS[ev[i].kind], ev[i].epoch, ev[i].minibatch, ev[i].value)
+                  for i in range(min(n.value, cap))]
+        return dict(events=events, words=words.value, seconds=secs.value,
+                    final_learning_rate=lr.value)
+
+    def get_perplexity(self, path):
+        out = C.c_double()
+        _check(load().lnmt_get_perplexity(self.handle, os.fsencode(path), C.byref(out)),
+               "get_perplexity")
+        return out.value
 
     def load_weights(self, path):
         """NeuralMachineTranslation::LoadWeights: fill the parameters from a reference model file."""

@@ -4,6 +4,7 @@
 #include <memory>
 
 #include "../../include/linmt_host.h"
+#include "dispatcher.h"
 #include "file_helper.h"
 #include "nmt.h"
 
@@ -373,4 +374,41 @@ extern "C" int lnmt_file_helper_info(lnmt_file_helper *f, int info[8]) {
                       h.total_words_,           h.total_target_words_};
     std::copy(v, v + 8, info);
   });
+}
+
+extern "C" int lnmt_tuning(lnmt_model *m, const lnmt_tuning_options *o, lnmt_tuning_event *events,
+                           int event_cap, int *n_events, long long *words, double *seconds,
+                           float *final_learning_rate) {
+  return Guard([&] {
+    if (!o || !o->train_file) throw LinmtError("lnmt_tuning: no training file");
+    TuningConfiguration c;
+    c.train_file_name_ = o->train_file;
+    c.test_file_name_ = o->dev_file ? o->dev_file : "";
+    c.output_weight_file_ = o->output_weight_file ? o->output_weight_file : "";
+    c.best_model_file_name_ = o->best_model_file ? o->best_model_file : "";
+    c.epochs_number_ = o->epochs;
+    c.google_learning_rate_ = o->google_learning_rate != 0;
+    c.epoch_to_start_halving_ = o->epoch_to_start_halving;
+    c.stanford_learning_rate_ = o->stanford_learning_rate != 0;
+    c.epoch_to_start_halving_full_ = o->epoch_to_start_halving_full;
+    c.learning_rate_schedule_ = o->learning_rate_schedule != 0;
+    c.decrease_factor_ = o->decrease_factor;
+    c.margin_ = o->margin;
+    c.best_model_mode_ = o->best_model_mode != 0;
+    c.screen_print_rate_ = o->screen_print_rate > 0 ? o->screen_print_rate : 20;
+    if (c.learning_rate_schedule_ && c.test_file_name_.empty())
+      throw LinmtError("lnmt_tuning: the perplexity schedule needs a dev file");
+    const TuningReport r = Dispatcher::Tuning(*m->nmt, c);
+    const int n = (int)r.events.size();
+    for (int i = 0; i < n && i < event_cap; ++i)
+      events[i] = {(int)r.events[i].kind, r.events[i].epoch, r.events[i].minibatch, r.events[i].value};
+    if (n_events) *n_events = n;
+    if (words) *words = r.words;
+    if (seconds) *seconds = r.seconds;
+    if (final_learning_rate) *final_learning_rate = r.final_learning_rate;
+  });
+}
+
+extern "C" int lnmt_get_perplexity(lnmt_model *m, const char *file_name, double *perplexity) {
+  return Guard([&] { *perplexity = m->nmt->GetPerplexity(file_name); });
 }

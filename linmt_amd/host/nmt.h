@@ -448,6 +448,11 @@ class NeuralMachineTranslation {
   // holds the header part; DumpModel writes header, mappings (null: placeholder words) and matrices.
   void LoadWeights(const std::string &input_weight_file);
   void DumpWeights(const std::string &output_weight_file);
+  // DumpBestModel (deep_rnn.h:1971-2040): header + mappings of const_model_name, current matrices.
+  void DumpBestModel(const std::string &best_model_name, const std::string &const_model_name);
+  // GetPerplexity (deep_rnn.h:1490-1568) over an integerised file (host/dispatcher.cc).
+  double GetPerplexity(const std::string &test_file_name);
+  void UpdateLearningRate(float new_learning_rate);
   void DumpModel(const std::string &output_weight_file, const std::vector<std::string> *source_words,
                  const std::vector<std::string> *target_words);
   // every parameter name in the order the model file stores them, with its (rows, cols)
