@@ -82,7 +82,7 @@ TuningReport Dispatcher::Tuning(NeuralMachineTranslation &neural, TuningConfigur
   double old_perplexity = 0.0, train_loglik = 0.0;
 
   // dev perplexity, the stall rule and the best-model dump: the same block at the half epoch and
-  // at the epoch's end (src/dispatcher.cu:246-272 and :312-337)
+  // at the epoch's end (src/dispatcher.cu:240-272 and :306-337)
   auto evaluate = [&](TuningEvent::Kind kind) {
     const double new_perplexity = neural.GetPerplexity(configuration.test_file_name_);
     emit(kind, current_epoch, current_batch_num, new_perplexity);
