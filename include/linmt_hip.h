@@ -112,11 +112,23 @@ int lh_gemm_ws_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, 
                    float alpha, float beta, const float *bias, int act, int act_rows,
                    const int *colmask, float *C, int ldc, void *workspace, size_t workspace_bytes,
                    lh_stream_t stream);
-/* Name of the kernel instance lh_gemm_ws_f32 would launch for this problem (tile shape and operand
- * flags), as profilers print it; no counterpart in the reference.  Pointers in `segs` are only
- * inspected for alignment; workspace_bytes = 0 describes lh_gemm_f32 / lh_gemm_act_rows_f32. */
+/* The plain product for a consumer that can add up partial sums itself (the LSTM cell kernel takes
+ * three addends): like lh_gemm_ws_f32 with alpha = 1 and no bias / activation / mask, but a split
+ * product is left unreduced.  *planes receives S, 1 <= S <= max_planes:
+ *   S == 1: C = beta * C + product, as usual;
+ *   S  > 1: C is NOT touched; plane s (0 <= s < S) is the ((M + 3) & ~3) x N column-major block at
+ *           (float *)workspace + s * ((M + 3) & ~3) * N, and product = sum of the planes (the
+ *           caller adds beta * C).
+ * No counterpart in the reference. */
+int lh_gemm_planes_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
+                       float beta, float *C, int ldc, void *workspace, size_t workspace_bytes,
+                       int max_planes, int *planes, lh_stream_t stream);
+/* Name of the kernel instance lh_gemm_ws_f32 (max_planes = 0) or lh_gemm_planes_f32 would launch
+ * for this problem (tile shape and operand flags), as profilers print it; no counterpart in the
+ * reference.  Pointers in `segs` are only inspected for alignment; workspace_bytes = 0 describes
+ * lh_gemm_f32 / lh_gemm_act_rows_f32. */
 int lh_gemm_kernel_name(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
-                        size_t workspace_bytes, char *name, int name_cap);
+                        size_t workspace_bytes, int max_planes, char *name, int name_cap);
 /* Tuning and test aids (no counterpart in the reference).
  * lh_gemm_set_config_override: forces tile configuration `config` for every later lh_gemm_* call
  * of the process, config < 0 restores the built-in choice.  Returns the number of configurations

@@ -49,6 +49,7 @@ struct GemmArgs {
   int splits, slabs_per_split;
   float *ws_part;
   int ws_ld;
+  int leave_partial;  // host only: the caller sums the planes itself, no reduction launch
 };
 
 // Stages one BK x BD operand slab: global -> registers (load), registers -> LDS [BK][BD+PAD] (store).
@@ -789,7 +790,7 @@ int launch_cfg(const GemmArgs &g0, bool ta, bool tx, bool vec, hipStream_t st) {
     else if (ta) LH_GEMM_LAUNCH(true, false);
     else LH_GEMM_LAUNCH(false, true);
 #undef LH_GEMM_LAUNCH
-    if (rc != LH_OK || g.splits == 1) return rc;
+    if (rc != LH_OK || g.splits == 1 || g.leave_partial) return rc;
     const size_t total = (size_t)g.M * g.N;
     const size_t blocks = (total + 1023) / 1024;  // four elements per thread
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)(blocks < 8192 ? blocks : 8192)),
@@ -885,7 +886,7 @@ constexpr int kCUs = 256;
 constexpr float kReduceFixedUs = 2.5f, kReduceBytesPerUs = 3.0e6f;
 
 float predict_us(const Tuning &t, const Config &k, int M, int N, const int *K, int nseg, int want,
-                 int *splits) {
+                 bool reduce_free, int *splits) {
   const long long tiles = (long long)((M + k.bm - 1) / k.bm) * ((N + k.bn - 1) / k.bn);
   int slabs = 0;
   for (int s = 0; s < nseg; ++s) slabs += (K[s] + k.bk - 1) / k.bk;
@@ -903,12 +904,16 @@ float predict_us(const Tuning &t, const Config &k, int M, int N, const int *K, i
   float us = rounds * tocc;
   if (rest > 1e-6f)
     us += rest <= 1.f || t.occ == 1 ? t1 : t1 + (tocc - t1) * (rest - 1.f) / (float)(t.occ - 1);
-  if (S > 1) us += kReduceFixedUs + (float)(S + 1) * (float)M * (float)N * 4.f / kReduceBytesPerUs;
+  if (S > 1 && !reduce_free)
+    us += kReduceFixedUs + (float)(S + 1) * (float)M * (float)N * 4.f / kReduceBytesPerUs;
+  if (S > 1 && reduce_free)  // the consumer reads S planes instead of one matrix
+    us += (float)(S - 1) * (float)M * (float)N * 4.f / kReduceBytesPerUs;
   return us;
 }
 
+// max_planes > 0: the caller consumes up to that many partial planes itself (no reduction pass).
 void pick_config(int M, int N, const int *K, int nseg, bool ta, bool tx, bool vec,
-                 size_t workspace_bytes, int *config, int *splits) {
+                 size_t workspace_bytes, int max_planes, int *config, int *splits) {
   *splits = 1;
   if (!vec) {
     *config = kUnalignedConfig;
@@ -921,7 +926,7 @@ void pick_config(int M, int N, const int *K, int nseg, bool ta, bool tx, bool ve
   };
   static thread_local Memo memo[64];
   const int flags = 1 + (ta ? 2 : 0) + (tx ? 4 : 0) + 8 * nseg + 64 * (g_config_override + 1) +
-                    4096 * g_splits_override;
+                    4096 * g_splits_override + 131072 * max_planes;
   int Kk[LH_GEMM_MAX_SEGS] = {0, 0, 0};
   for (int s = 0; s < nseg; ++s) Kk[s] = K[s];
   const unsigned h = ((unsigned)M * 2654435761u) ^ ((unsigned)N * 40503u) ^ ((unsigned)Kk[0] * 97u) ^
@@ -941,15 +946,16 @@ void pick_config(int M, int N, const int *K, int nseg, bool ta, bool tx, bool ve
     if (g_config_override >= 0 && c != g_config_override) continue;
     for (int want : kSplitChoices) {
       if (g_splits_override > 0) want = fit_splits(M, N, g_splits_override, workspace_bytes);
+      if (max_planes > 0 && want > max_planes) want = max_planes;
       if (want > 1 && fit_splits(M, N, want, workspace_bytes) < want) break;
       int S;
-      const float us = predict_us(table[c], kConfigs[c], M, N, K, nseg, want, &S);
+      const float us = predict_us(table[c], kConfigs[c], M, N, K, nseg, want, max_planes > 0, &S);
       if (us < best) {
         best = us;
         *config = c;
         *splits = S;
       }
-      if (g_splits_override > 0) break;
+      if (g_splits_override > 0 || (max_planes > 0 && want >= max_planes)) break;
     }
   }
   e = Memo{M, N, {Kk[0], Kk[1], Kk[2]}, flags, *config, *splits, workspace_bytes};
@@ -963,7 +969,7 @@ struct Prepared {
 
 int prepare(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX, float alpha,
             float beta, const float *bias, int act, int act_rows, const int *colmask, float *C,
-            int ldc, void *workspace, size_t workspace_bytes, Prepared *out) {
+            int ldc, void *workspace, size_t workspace_bytes, int max_planes, Prepared *out) {
   if (M <= 0 || N <= 0) return lh::fail_arg("lh_gemm_f32: M=%d N=%d must be positive", M, N);
   if (!segs || nseg < 1 || nseg > LH_GEMM_MAX_SEGS)
     return lh::fail_arg("lh_gemm_f32: nseg=%d outside [1,%d]", nseg, LH_GEMM_MAX_SEGS);
@@ -1018,8 +1024,9 @@ int prepare(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int tra
   out->tx = transX != 0;
   out->vec = vec;
   if (!workspace || !lh::aligned16(workspace)) workspace_bytes = 0;
-  pick_config(M, N, g.K, nseg, transA != 0, transX != 0, vec, workspace_bytes, &out->config,
-              &g.splits);
+  pick_config(M, N, g.K, nseg, transA != 0, transX != 0, vec, workspace_bytes, max_planes,
+              &out->config, &g.splits);
+  g.leave_partial = max_planes > 0 ? 1 : 0;
   g.ws_part = static_cast<float *>(workspace);
   g.ws_ld = plane_ld(M);
   return LH_OK;
@@ -1035,8 +1042,28 @@ extern "C" int lh_gemm_ws_f32(int M, int N, const lh_gemm_seg *segs, int nseg, i
     return lh::fail_arg("lh_gemm_f32: act_rows=%d outside [0,M=%d]", act_rows, M);
   Prepared p;
   const int rc = prepare(M, N, segs, nseg, transA, transX, alpha, beta, bias, act, act_rows,
-                         colmask, C, ldc, workspace, workspace_bytes, &p);
+                         colmask, C, ldc, workspace, workspace_bytes, 0, &p);
   if (rc != LH_OK) return rc;
+  return launch_index(p.config, p.g, p.ta, p.tx, p.vec, lh::as_stream(stream));
+}
+
+extern "C" int lh_gemm_planes_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA,
+                                  int transX, float beta, float *C, int ldc, void *workspace,
+                                  size_t workspace_bytes, int max_planes, int *planes,
+                                  lh_stream_t stream) {
+  if (!planes || max_planes < 1)
+    return lh::fail_arg("lh_gemm_planes_f32: planes=%p max_planes=%d", (void *)planes, max_planes);
+  Prepared p;
+  const int rc = prepare(M, N, segs, nseg, transA, transX, 1.f, beta, nullptr, LH_ACT_NONE, M,
+                         nullptr, C, ldc, workspace, workspace_bytes, max_planes, &p);
+  if (rc != LH_OK) return rc;
+  // the split the launch will really use (no empty share), as launch_cfg computes it
+  const Config &k = kConfigs[p.config];
+  int slabs = 0;
+  for (int s = 0; s < p.g.nseg; ++s) slabs += (p.g.K[s] + k.bk - 1) / k.bk;
+  const int want = p.vec ? p.g.splits : 1;
+  const int share = (slabs + want - 1) / want;
+  *planes = (slabs + share - 1) / share;
   return launch_index(p.config, p.g, p.ta, p.tx, p.vec, lh::as_stream(stream));
 }
 
@@ -1079,14 +1106,15 @@ extern "C" int lh_gemm_config_info(int config, int transA, int transX, int info[
 }
 
 extern "C" int lh_gemm_kernel_name(int M, int N, const lh_gemm_seg *segs, int nseg, int transA,
-                                   int transX, size_t workspace_bytes, char *name, int name_cap) {
+                                   int transX, size_t workspace_bytes, int max_planes, char *name,
+                                   int name_cap) {
   if (!name || name_cap < 1) return lh::fail_arg("lh_gemm_kernel_name: no output buffer");
   Prepared p;
   float dummy;
   // any aligned non-null address stands in for the workspace: nothing is launched
   const int rc = prepare(M, N, segs, nseg, transA, transX, 1.f, 0.f, nullptr, LH_ACT_NONE, M,
                          nullptr, &dummy, M, workspace_bytes ? (void *)(uintptr_t)256 : nullptr,
-                         workspace_bytes, &p);
+                         workspace_bytes, max_planes, &p);
   if (rc != LH_OK) return rc;
   const Config &k = kConfigs[p.config];
   if (p.vec)

@@ -377,6 +377,11 @@ class NeuralMachineTranslation {
   void Gemm(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg, int trans_a, int trans_x,
             float beta, const float *bias, int act, const int *colmask, float *C, int ldc,
             const char *what);
+  // The plain product for a consumer that adds partial sums itself (the LSTM cell kernel takes
+  // three addends).  Returns the number of addends n and fills addend[0..n): either {C} with
+  // C = beta * C + product, or the partial planes of a split product preceded by C when beta = 1.
+  int GemmAddends(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg, float beta,
+                  float *C, int ldc, const float *addend[3], const char *what);
 
   LstmLayer input_layer_source_, input_layer_target_;
   std::vector<std::unique_ptr<LstmLayer>> v_hidden_layers_source_, v_hidden_layers_target_;

@@ -253,11 +253,14 @@ void LstmNode::ForwardProp() {
   }
   segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
   if (feed) segs[nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
-  M.Gemm(kTagGateGemm, 4 * H, B, segs, nseg, 0, 0, beta, nullptr, LH_ACT_NONE, nullptr, pre, 4 * H,
-         "LstmNode::ForwardPropGpu stacked gate product");
+  // a split product stays in partial planes: the cell kernel adds them up (no reduction pass)
+  const float *addend[3];
+  const int n_add = M.GemmAddends(kTagGateGemm, 4 * H, B, segs, nseg, beta, pre, 4 * H, addend,
+                                  "LstmNode::ForwardPropGpu stacked gate product");
   const bool drop_out = M.apply_dropout_ && L.out_dropout_;
-  ProfileScope pc(M.profiler_, kTagLstmCell, ((p_device_gates_ ? 44.0 : 28.0) + (drop_out ? 8.0 : 0.0)) * H * B);
-  LhErrorWrapper(lh_lstm_cell_fwd_f32(H, B, pre, nullptr, nullptr,
+  ProfileScope pc(M.profiler_, kTagLstmCell,
+                  ((p_device_gates_ ? 44.0 : 28.0) + (drop_out ? 8.0 : 0.0) + 16.0 * (n_add - 1)) * H * B);
+  LhErrorWrapper(lh_lstm_cell_fwd_f32(H, B, addend[0], addend[1], addend[2],
                                       L.p_device_b_stack_.get(), p_device_c_t_prev_,
                                       p_device_input_vocab_indices_01_, feed ? 1 : 0,
                                       M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f,

@@ -18,7 +18,7 @@ NeuralMachineTranslation::NeuralMachineTranslation(const GlobalConfiguration &cf
 void NeuralMachineTranslation::Gemm(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg,
                                     int trans_a, int trans_x, float beta, const float *bias, int act,
                                     const int *colmask, float *C, int ldc, const char *what) {
-  ProfileScope ps(profiler_, tag, gemm_workspace_.size(), rows, cols, segs, nseg, trans_a, trans_x);
+  ProfileScope ps(profiler_, tag, gemm_workspace_.size(), 0, rows, cols, segs, nseg, trans_a, trans_x);
   LhErrorWrapper(lh_gemm_ws_f32(rows, cols, segs, nseg, trans_a, trans_x, 1.f, beta, bias, act, rows,
                                 colmask, C, ldc, gemm_workspace_.get(), gemm_workspace_.size(),
                                 stream_),
@@ -128,6 +128,28 @@ void NeuralMachineTranslation::InitModelDecoding(int n_sent, int beam_size) {
   if (cfg_.attention_mode_) attention_layer_.p_device_hs_col_.Upload(sent.data(), B, stream_);
   decoder_.Init(beam_size, n_sent, T);
   Synchronize();
+}
+
+int NeuralMachineTranslation::GemmAddends(int tag, int rows, int cols, const lh_gemm_seg *segs,
+                                          int nseg, float beta, float *C, int ldc,
+                                          const float *addend[3], const char *what) {
+  if (beta != 0.f && beta != 1.f) throw LinmtError("GemmAddends: beta must be 0 or 1");
+  // planes can only replace C when they have C's leading dimension
+  const bool can_split = ldc == rows && rows % 4 == 0;
+  const int max_planes = !can_split ? 1 : (beta == 0.f ? 3 : 2);
+  ProfileScope ps(profiler_, tag, gemm_workspace_.size(), max_planes, rows, cols, segs, nseg, 0, 0);
+  int planes = 1;
+  LhErrorWrapper(lh_gemm_planes_f32(rows, cols, segs, nseg, 0, 0, beta, C, ldc, gemm_workspace_.get(),
+                                    gemm_workspace_.size(), max_planes, &planes, stream_),
+                 what);
+  int n = 0;
+  if (planes == 1 || beta != 0.f) addend[n++] = C;
+  if (planes > 1) {
+    const float *ws = reinterpret_cast<const float *>(gemm_workspace_.get());
+    for (int p = 0; p < planes; ++p) addend[n++] = ws + (size_t)p * rows * cols;
+  }
+  for (int i = n; i < 3; ++i) addend[i] = nullptr;
+  return n;
 }
 
 bool NeuralMachineTranslation::SetParam(const std::string &name, const float *host, size_t n) {

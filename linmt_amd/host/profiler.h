@@ -120,14 +120,14 @@ class ProfileScope {
     if (on_) slot_ = p_.Begin(ProfileTagName(tag), work);
   }
   // Matrix product: the key carries the kernel instance lh_gemm_f32 will launch for this problem.
-  ProfileScope(Profiler &p, int tag, size_t workspace_bytes, int M, int N, const lh_gemm_seg *segs,
-               int nseg, int transA,
+  ProfileScope(Profiler &p, int tag, size_t workspace_bytes, int max_planes, int M, int N,
+               const lh_gemm_seg *segs, int nseg, int transA,
                int transX)
       : p_(p), on_(p.Wants(tag)) {
     if (!on_) return;
     char name[160] = {0};
-    LhErrorWrapper(lh_gemm_kernel_name(M, N, segs, nseg, transA, transX, workspace_bytes, name,
-                                       sizeof(name)),
+    LhErrorWrapper(lh_gemm_kernel_name(M, N, segs, nseg, transA, transX, workspace_bytes, max_planes,
+                                       name, sizeof(name)),
                    "lh_gemm_kernel_name");
     double k = 0;
     for (int s = 0; s < nseg; ++s) k += segs[s].K;

@@ -43,8 +43,11 @@ SIGNATURES = {
     "lh_gemm_ws_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int, C.c_int,
                                  C.c_float, C.c_float, c_f32p, C.c_int, C.c_int, c_i32p, c_f32p,
                                  C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "lh_gemm_planes_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
+                                     C.c_int, C.c_float, c_f32p, C.c_int, C.c_void_p, C.c_size_t,
+                                     C.c_int, C.POINTER(C.c_int), C.c_void_p]),
     "lh_gemm_kernel_name": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
-                                      C.c_int, C.c_size_t, C.c_char_p, C.c_int]),
+                                      C.c_int, C.c_size_t, C.c_int, C.c_char_p, C.c_int]),
     "lh_gemm_set_config_override": (C.c_int, [C.c_int]),
     "lh_gemm_set_splits_override": (C.c_int, [C.c_int]),
     "lh_gemm_config_info": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int * 8)]),
@@ -188,11 +191,23 @@ def gemm(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0
               "lh_gemm_act_rows_f32")
 
 
-def gemm_kernel_name(M, N, segs, transA=False, transX=False, workspace_bytes=0):
+def gemm_kernel_name(M, N, segs, transA=False, transX=False, workspace_bytes=0, max_planes=0):
     buf = C.create_string_buffer(128)
     check(load().lh_gemm_kernel_name(M, N, _segs(segs), len(segs), int(transA), int(transX),
-                                     workspace_bytes, buf, 128), "lh_gemm_kernel_name")
+                                     workspace_bytes, max_planes, buf, 128), "lh_gemm_kernel_name")
     return buf.value.decode()
+
+
+def gemm_planes(M, N, segs, C_out, ldc, workspace, max_planes, transA=False, transX=False, beta=0.0,
+                stream=None):
+    """lh_gemm_planes_f32: returns the number of planes S; for S > 1 the planes are the
+    ((M+3)&~3) x N blocks at the start of `workspace` (a float tensor) and C_out is untouched."""
+    planes = C.c_int()
+    check(load().lh_gemm_planes_f32(M, N, _segs(segs), len(segs), int(transA), int(transX), beta,
+                                    _ptr(C_out), ldc, workspace.data_ptr(),
+                                    workspace.numel() * workspace.element_size(), max_planes,
+                                    C.byref(planes), _stream(stream)), "lh_gemm_planes_f32")
+    return planes.value
 
 
 def gemm_config_info(config, transA=False, transX=False):

@@ -153,6 +153,41 @@ def test_gemm_split_k(lh):
         lh.check(L.lh_gemm_set_splits_override(10 ** 6), "override")
 
 
+def test_gemm_planes(lh):
+    """lh_gemm_planes_f32: S == 1 writes beta * C + product; S > 1 leaves C alone and the planes
+    in the workspace add up to the product.  Forced and freely chosen splits."""
+    rng = np.random.default_rng(23)
+    L = lh.load()
+    ws = torch.full((4 << 20,), float("nan"), device="cuda")
+    try:
+        for forced in (0, 1, 2, 3):
+            L.lh_gemm_set_splits_override(forced)
+            for M, N, Ks, beta, max_planes in ((4000, 96, (1000, 1000), 0.0, 3), (400, 64, (520,), 1.0, 2),
+                                               (132, 36, (40, 24), 0.0, 3), (64, 8, (16,), 1.0, 1)):
+                As = [uni(rng, M, K, s=0.1) for K in Ks]
+                Xs = [uni(rng, K, N) for K in Ks]
+                want = sum(A.astype(np.float64) @ X for A, X in zip(As, Xs))
+                segs = [(dev(A), M, dev(X), K, K) for A, X, K in zip(As, Xs, Ks)]
+                C0 = uni(rng, M, N)
+                out = dev(C0)
+                S = lh.gemm_planes(M, N, segs, out, M, ws, max_planes, beta=beta)
+                what = f"forced {forced} shape {(M, N, Ks)} beta {beta}: {S} planes"
+                assert 1 <= S <= max_planes, what
+                if forced in (2, 3) and max_planes >= forced and sum(Ks) >= 512:
+                    assert S == forced, what
+                if S == 1:
+                    assert_close(host(out, (M, N)), want + beta * C0, what)
+                else:
+                    assert np.array_equal(host(out, (M, N)), C0), what + ": C was written"
+                    ld = (M + 3) & ~3
+                    planes = ws[: S * ld * N].cpu().numpy().reshape(S, N, ld)[:, :, :M]
+                    assert_close(planes.sum(axis=0).T, want, what)
+    finally:
+        L.lh_gemm_set_splits_override(0)
+    with pytest.raises(lh.LinmtHipError):
+        lh.gemm_planes(8, 8, [(ws, 8, ws, 8, 8)], ws, 8, ws, 0)
+
+
 def test_gemm_every_tile_configuration(lh):
     """Each tile configuration (incl. the intra-workgroup split-K ones) on shapes with ragged edges,
     several K segments and both transposes; also the row-limited activation and the kernel name."""
