@@ -198,9 +198,12 @@ int lh_lstm_cell_fwd_f32(int H, int B, const float *pre1, const float *pre2, con
  * viterbi (B, optional).  max_len (= the W of the global variant) is ignored for D >= 0.
  * hs_steps = number of encoder timesteps held in hs; a slot whose tau falls outside [0,hs_steps)
  * reads as a zero vector instead of touching memory outside the buffer.
+ * proj_col_stride = distance in floats between the columns of tanh1 and of wa (0 = H): both may be
+ * halves of one 2H x B product of row-stacked [W_p ; W_a^T] (lh_gemm_act_rows_f32).
  */
 int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_steps, const float *tanh1,
-                         const float *v_p, const float *wa, const float *hs, long long hs_step_stride,
+                         const float *v_p, const float *wa, long long proj_col_stride,
+                         const float *hs, long long hs_step_stride,
                          long long hs_col_stride, const int *hs_col, const int *batch_info,
                          const int *mask01, float *p_t, float *sigma, int *indices, float *align,
                          float *cached_exp, float *ctx, int *viterbi, lh_stream_t stream);

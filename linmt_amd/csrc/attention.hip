@@ -18,6 +18,7 @@ constexpr int kWaves = kThreads / lh::kWave;
 struct AttnArgs {
   int H, B, D, W;
   const float *tanh1, *v_p, *wa, *hs;
+  long long proj_col_stride;  // distance between columns of tanh1 and of wa (>= H)
   long long step_stride, col_stride;
   int hs_steps;
   const int *hs_col, *batch_info, *mask01;
@@ -58,14 +59,14 @@ __global__ __launch_bounds__(kThreads) void attn_core_kernel(const AttnArgs a) {
   const int off = a.batch_info[B + b];
   const int m = a.mask01[b];
   const int col = a.hs_col ? a.hs_col[b] : b;
-  const float *wa = a.wa + (size_t)b * H;
+  const float *wa = a.wa + (size_t)b * a.proj_col_stride;
   const float *hs_c = a.hs + (size_t)col * a.col_stride;
 
   float p = 0.f;
   int lo = 0, hi = len - 1;
   if (D >= 0) {
     float part = 0.f;
-    const float *t1 = a.tanh1 + (size_t)b * H;
+    const float *t1 = a.tanh1 + (size_t)b * a.proj_col_stride;
     for (int r = tid; r < H; r += kThreads) part += a.v_p[r] * t1[r];
     const float dot = lh::block_sum<kWaves>(part, s_red);
     const float sig = (float)(1.0 / (1.0 + exp(-1.0 * (double)dot)));
@@ -173,7 +174,8 @@ __global__ __launch_bounds__(kThreads) void attn_core_kernel(const AttnArgs a) {
 
 extern "C" int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_steps,
                                     const float *tanh1, const float *v_p, const float *wa,
-                                    const float *hs, long long hs_step_stride,
+                                    long long proj_col_stride, const float *hs,
+                                    long long hs_step_stride,
                                     long long hs_col_stride, const int *hs_col,
                                     const int *batch_info, const int *mask01, float *p_t,
                                     float *sigma, int *indices, float *align, float *cached_exp,
@@ -189,11 +191,14 @@ extern "C" int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_ste
     return lh::fail_arg("lh_attn_core_fwd_f32: local-p needs tanh1, v_p, p_t and sigma");
   if (hs_step_stride < 0 || hs_col_stride < 0)
     return lh::fail_arg("lh_attn_core_fwd_f32: negative stride");
+  if (proj_col_stride == 0) proj_col_stride = H;
+  if (proj_col_stride < H)
+    return lh::fail_arg("lh_attn_core_fwd_f32: proj_col_stride %lld < H", proj_col_stride);
 
-  AttnArgs a{H, B, D, W, tanh1, v_p, wa, hs, hs_step_stride, hs_col_stride, hs_steps, hs_col,
+  AttnArgs a{H, B, D, W, tanh1, v_p, wa, hs, proj_col_stride, hs_step_stride, hs_col_stride, hs_steps, hs_col,
              batch_info, mask01, p_t, sigma, indices, align, cached_exp, ctx, viterbi};
   const bool vec = H % 4 == 0 && lh::aligned16(wa) && lh::aligned16(hs) && lh::aligned16(ctx) &&
-                   hs_step_stride % 4 == 0 && hs_col_stride % 4 == 0;
+                   hs_step_stride % 4 == 0 && hs_col_stride % 4 == 0 && proj_col_stride % 4 == 0;
   hipStream_t st = lh::as_stream(stream);
   if (vec) hipLaunchKernelGGL(attn_core_kernel<true>, dim3(B), dim3(kThreads), 0, st, a);
   else hipLaunchKernelGGL(attn_core_kernel<false>, dim3(B), dim3(kThreads), 0, st, a);

@@ -237,6 +237,12 @@ class AttentionLayer {
   int hs_steps_ = 0;       // timesteps currently held
   bool use_hs_col_ = false;  // decode: beam columns share their sentence's states
   std::vector<AttentionNode> v_nodes_;
+  // Outside training the two projections of h_t share one launch: [W_p ; W_a^T] (2H x H) * h_t
+  // with tanh on the upper half (src/layer_attention.h:272-275 and :327).  The stack is rebuilt
+  // when W_p or W_a is set; training updates them on the device and keeps the two products apart.
+  DeviceArray<float> p_device_w_pa_stack_, proj_out_;
+  bool pa_stack_dirty_ = true;
+  void BuildProjectionStack();
 
   // ---- training --------------------------------------------------------------------------------
   DeviceArray<float> p_device_w_a_grad_, p_device_w_p_grad_, p_device_v_p_grad_,
@@ -376,7 +382,7 @@ class NeuralMachineTranslation {
   // Every dense product of the model: profiling key, workspace, error text.
   void Gemm(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg, int trans_a, int trans_x,
             float beta, const float *bias, int act, const int *colmask, float *C, int ldc,
-            const char *what);
+            const char *what, int act_rows = -1);  // act_rows < 0: the activation covers every row
   // The plain product for a consumer that adds partial sums itself (the LSTM cell kernel takes
   // three addends).  Returns the number of addends n and fills addend[0..n): either {C} with
   // C = beta * C + product, or the partial planes of a split product preceded by C when beta = 1.

@@ -368,6 +368,7 @@ void AttentionLayer::PreprocessMinibatchInformation(const int *p_host_batch_info
 
 bool AttentionLayer::SetParam(const std::string &name, const float *host, size_t n) {
   hipStream_t s = p_neural_mt_->stream_;
+  if (name == "W_a" || name == "W_p") pa_stack_dirty_ = true;
   if (name == "W_a") return SetFlat(p_device_w_a_, host, n, s);
   if (name == "W_p") return SetFlat(p_device_w_p_, host, n, s);
   if (name == "v_p") return SetFlat(p_device_v_p_, host, n, s);
@@ -375,6 +376,26 @@ bool AttentionLayer::SetParam(const std::string &name, const float *host, size_t
   if (name == "W_c1") return SetFlat(p_device_w_c_p1_, host, n, s);
   if (name == "W_c2") return SetFlat(p_device_w_c_p2_, host, n, s);
   return false;
+}
+
+void AttentionLayer::BuildProjectionStack() {
+  const size_t H = lstm_size_;
+  hipStream_t s = p_neural_mt_->stream_;
+  std::vector<float> wa, wp, stack(2 * H * H);
+  if (!GetFlat(p_device_w_a_, &wa, s) || !GetFlat(p_device_w_p_, &wp, s))
+    throw LinmtError("AttentionLayer::BuildProjectionStack: cannot read W_a / W_p");
+  for (size_t k = 0; k < H; ++k)      // column k of the 2H x H stack
+    for (size_t i = 0; i < H; ++i) {  // W_p[i,k] above W_a^T[i,k] = W_a[k,i]
+      stack[i + k * 2 * H] = wp[i + k * H];
+      stack[H + i + k * 2 * H] = wa[k + i * H];
+    }
+  if (p_device_w_pa_stack_.size() == 0) {
+    p_device_w_pa_stack_.Alloc(2 * H * H);
+    proj_out_.Alloc(2 * H * (size_t)minibatch_size_);
+  }
+  p_device_w_pa_stack_.Upload(stack.data(), stack.size(), s);
+  HipErrorWrapper(hipStreamSynchronize(s), "projection stack upload failed");  // `stack` is a local
+  pa_stack_dirty_ = false;
 }
 
 bool AttentionLayer::GetParam(const std::string &name, std::vector<float> *out) {
@@ -397,12 +418,22 @@ void AttentionNode::ForwardProp() {
   const int H = A.lstm_size_, B = minibatch_size_;
   const float *ha = p_device_h_t_;  // no dropout outside training
   Profiler &prof = A.p_neural_mt_->profiler_;
-  if (!A.global_mode_) {
-    lh_gemm_seg seg{A.p_device_w_p_.get(), H, ha, H, H};
-    A.p_neural_mt_->Gemm(kTagAttnProjGemm, H, B, &seg, 1, 0, 0, 0.f, nullptr, LH_ACT_TANH, nullptr,
-                         p_device_tanh_1_, H, "AttentionNode::ForwardProp p_device_tanh_1_");
-  }
-  {
+  const float *tanh1 = p_device_tanh_1_, *wa = p_device_h_t_wa_cache_;
+  long long proj_col_stride = H;
+  if (!A.global_mode_ && !A.p_neural_mt_->cfg_.train_mode_) {
+    if (A.pa_stack_dirty_) A.BuildProjectionStack();
+    lh_gemm_seg seg{A.p_device_w_pa_stack_.get(), 2 * H, ha, H, H};
+    A.p_neural_mt_->Gemm(kTagAttnProjGemm, 2 * H, B, &seg, 1, 0, 0, 0.f, nullptr, LH_ACT_TANH, nullptr,
+                         A.proj_out_.get(), 2 * H, "AttentionNode::ForwardProp [W_p ; W_a^T] h_t", H);
+    tanh1 = A.proj_out_.get();
+    wa = A.proj_out_.get() + H;
+    proj_col_stride = 2 * H;
+  } else {
+    if (!A.global_mode_) {
+      lh_gemm_seg seg{A.p_device_w_p_.get(), H, ha, H, H};
+      A.p_neural_mt_->Gemm(kTagAttnProjGemm, H, B, &seg, 1, 0, 0, 0.f, nullptr, LH_ACT_TANH, nullptr,
+                           p_device_tanh_1_, H, "AttentionNode::ForwardProp p_device_tanh_1_");
+    }
     lh_gemm_seg seg{A.p_device_w_a_.get(), H, ha, H, H};
     A.p_neural_mt_->Gemm(kTagAttnProjGemm, H, B, &seg, 1, 1, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
                          p_device_h_t_wa_cache_, H,
@@ -412,7 +443,7 @@ void AttentionNode::ForwardProp() {
   ProfileScope ps(prof, kTagAttnCore, 4.0 * B * ((double)A.window_ * H + 2.0 * H + 2.0 * A.window_));
   LhErrorWrapper(
       lh_attn_core_fwd_f32(H, B, A.global_mode_ ? -1 : A.d_, A.window_, A.hs_steps_,
-                           p_device_tanh_1_, A.p_device_v_p_.get(), p_device_h_t_wa_cache_,
+                           tanh1, A.p_device_v_p_.get(), wa, proj_col_stride,
                            A.p_device_total_hs_, A.hs_step_stride_, A.hs_col_stride_,
                            A.use_hs_col_ ? A.p_device_hs_col_.get() : nullptr,
                            A.p_device_batch_information_.get(), p_device_indices_mask_,

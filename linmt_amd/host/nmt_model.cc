@@ -17,9 +17,11 @@ NeuralMachineTranslation::NeuralMachineTranslation(const GlobalConfiguration &cf
 
 void NeuralMachineTranslation::Gemm(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg,
                                     int trans_a, int trans_x, float beta, const float *bias, int act,
-                                    const int *colmask, float *C, int ldc, const char *what) {
+                                    const int *colmask, float *C, int ldc, const char *what,
+                                    int act_rows) {
   ProfileScope ps(profiler_, tag, gemm_workspace_.size(), 0, rows, cols, segs, nseg, trans_a, trans_x);
-  LhErrorWrapper(lh_gemm_ws_f32(rows, cols, segs, nseg, trans_a, trans_x, 1.f, beta, bias, act, rows,
+  LhErrorWrapper(lh_gemm_ws_f32(rows, cols, segs, nseg, trans_a, trans_x, 1.f, beta, bias, act,
+                                act_rows < 0 ? rows : act_rows,
                                 colmask, C, ldc, gemm_workspace_.get(), gemm_workspace_.size(),
                                 stream_),
                  what);

@@ -55,7 +55,8 @@ SIGNATURES = {
                                        c_i32p, C.c_int, C.c_float, c_f32p, c_f32p, c_f32p, c_f32p,
                                        C.c_float, c_f32p, C.c_void_p]),
     "lh_attn_core_fwd_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, c_f32p, c_f32p,
-                                       c_f32p, c_f32p, C.c_longlong, C.c_longlong, c_i32p, c_i32p,
+                                       c_f32p, C.c_longlong, c_f32p, C.c_longlong, C.c_longlong,
+                                       c_i32p, c_i32p,
                                        c_i32p, c_f32p, c_f32p, c_i32p, c_f32p, c_f32p, c_f32p,
                                        c_i32p, C.c_void_p]),
     "lh_softmax_fwd_f32": (C.c_int, [c_f32p, C.c_int, c_f32p, C.c_int, C.c_int, c_f32p, C.c_int,
@@ -229,9 +230,11 @@ def lstm_cell_fwd(H, B, pre1, bias4h, c_prev, mask01, c, h, pre2=None, pre3=None
 
 def attn_core_fwd(H, B, D, max_len, hs_steps, tanh1, v_p, wa, hs, hs_step_stride, hs_col_stride,
                   hs_col, batch_info, mask01, p_t, sigma, indices, align, cached_exp, ctx,
-                  viterbi=None, stream=None):
+                  viterbi=None, proj_col_stride=0, stream=None):
+    """proj_col_stride: distance between the columns of tanh1 / wa (0 = H)."""
     check(load().lh_attn_core_fwd_f32(H, B, D, max_len, hs_steps, _ptr(tanh1), _ptr(v_p), _ptr(wa),
-                                      _ptr(hs), hs_step_stride, hs_col_stride, _ptr(hs_col),
+                                      proj_col_stride, _ptr(hs), hs_step_stride, hs_col_stride,
+                                      _ptr(hs_col),
                                       _ptr(batch_info), _ptr(mask01), _ptr(p_t), _ptr(sigma),
                                       _ptr(indices), _ptr(align), _ptr(cached_exp), _ptr(ctx),
                                       _ptr(viterbi), _stream(stream)), "lh_attn_core_fwd_f32")

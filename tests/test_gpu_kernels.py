@@ -288,18 +288,25 @@ def _attn_case(rng, H, B, S, lens, n_cols=None):
     return hs, tanh1.astype(np.float32), v_p, wa
 
 
-def _run_attn(lh, H, B, D, max_len, S, tanh1, v_p, wa, hs, step, colstride, hs_col, bi, mask):
+def _run_attn(lh, H, B, D, max_len, S, tanh1, v_p, wa, hs, step, colstride, hs_col, bi, mask,
+              stacked=False):
+    """stacked: tanh1 and wa are handed over as the two halves of one 2H x B matrix."""
     W = 2 * D + 1 if D >= 0 else max_len
+    d_tanh1, d_wa, stride = None if tanh1 is None else dev(tanh1), dev(wa), 0
+    if stacked:
+        both = dev(np.concatenate([tanh1, wa], axis=0))  # (2H, B), column-major on the device
+        d_tanh1, d_wa, stride = both, both[H:], 2 * H
     o = dict(p_t=torch.zeros(B, device="cuda"), sigma=torch.zeros(B, device="cuda"),
              indices=torch.empty(B * W, dtype=torch.int32, device="cuda"),
              align=torch.empty(B * W, device="cuda"), cached_exp=torch.empty(B * W, device="cuda"),
              ctx=torch.empty(H * B, device="cuda"),
              viterbi=torch.empty(B, dtype=torch.int32, device="cuda"))
-    lh.attn_core_fwd(H, B, D, max_len, S, None if tanh1 is None else dev(tanh1),
-                     None if v_p is None else dev(v_p), dev(wa),
+    lh.attn_core_fwd(H, B, D, max_len, S, d_tanh1,
+                     None if v_p is None else dev(v_p), d_wa,
                      torch.from_numpy(hs).cuda(), step, colstride,
                      None if hs_col is None else dev(hs_col), dev(bi), dev(mask), o["p_t"],
-                     o["sigma"], o["indices"], o["align"], o["cached_exp"], o["ctx"], o["viterbi"])
+                     o["sigma"], o["indices"], o["align"], o["cached_exp"], o["ctx"], o["viterbi"],
+                     proj_col_stride=stride)
     return dict(p_t=host(o["p_t"], (B,)), sigma=host(o["sigma"], (B,)),
                 indices=host(o["indices"], (B, W)), align=host(o["align"], (B, W)),
                 cached_exp=host(o["cached_exp"], (W, B)), ctx=host(o["ctx"], (H, B)),
@@ -327,6 +334,10 @@ def test_attn_core_local_p(lh, orc, H, B, S, D):
     assert_close(got["cached_exp"][:, same], want["cached_exp"][:, same], "gaussian cache")
     assert_close(got["ctx"][:, same], want["ctx"][:, same], "context")
     assert np.all(got["ctx"][:, mask == 0] == 0)
+    # the projections as halves of one row-stacked product: same bits
+    again = _run_attn(lh, H, B, D, 0, S, tanh1, v_p, wa, hs, B * H, H, None, bi, mask, stacked=True)
+    for key in got:
+        assert np.array_equal(got[key], again[key]), key
 
 
 def test_attn_core_shared_sentence_states(lh, orc):
