@@ -36,6 +36,8 @@ typedef struct lnmt_config {
 typedef struct lnmt_decode_options {
   int beam_size;
   float max_decoding_ratio, min_decoding_ratio, penalty, diversity, lp_alpha, cp_beta;
+  int unk_replacement_mode; /* the reference's unk_replacement_mode__: export alignment scores per
+                               step, Viterbi alignments per token, coverage penalty on the scores */
 } lnmt_decode_options;
 
 /* Training options (src/global_configuration.h:107-123, src/utility_cu.cu:82-96). */
@@ -104,11 +106,13 @@ int lnmt_get_state(lnmt_model *m, int kind, int side, int layer, int timestep, f
 /* Batched EnsembleFactory::DecodeFile.  sentences: concatenated source ids in ORIGINAL order,
  * lengths[n].  Outputs: best (n x cap, row-major), best_len[n], best_score[n], steps[n]; if
  * hyp_tokens != NULL also every finished hypothesis: hyp_tokens (n x hyp_cap x cap), hyp_len and
- * hyp_score (n x hyp_cap), n_hyp[n]. */
+ * hyp_score (n x hyp_cap), n_hyp[n].  best_viterbi (n x cap, may be NULL; filled when
+ * o->unk_replacement_mode is set): the source position (original order) aligned to each token of
+ * the 1-best, -1 where no alignment score was positive. */
 int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int *lengths, int n,
                       const lnmt_decode_options *o, int *best, int cap, int *best_len,
                       float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
-                      float *hyp_score, int hyp_cap, int *n_hyp);
+                      float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi);
 
 /* The model's HIP stream (hipStream_t as void*), for callers that time with HIP events. */
 void *lnmt_model_stream(lnmt_model *m);

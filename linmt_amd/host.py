@@ -50,7 +50,8 @@ class TuningEvent(C.Structure):
 class DecodeOptions(C.Structure):
     _fields_ = [("beam_size", C.c_int), ("max_decoding_ratio", C.c_float),
                 ("min_decoding_ratio", C.c_float), ("penalty", C.c_float),
-                ("diversity", C.c_float), ("lp_alpha", C.c_float), ("cp_beta", C.c_float)]
+                ("diversity", C.c_float), ("lp_alpha", C.c_float), ("cp_beta", C.c_float),
+                ("unk_replacement_mode", C.c_int)]
 
 
 def load():
@@ -307,13 +308,17 @@ class Model:
         return out.reshape((rows, cols), order="F")
 
     def decode_batch(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0,
-                     diversity=0.0, lp_alpha=0.65, cp_beta=0.20, with_hyps=False, hyp_cap=256):
+                     diversity=0.0, lp_alpha=0.65, cp_beta=0.20, with_hyps=False, hyp_cap=256,
+                     alignments=False):
+        """alignments=True: the reference's unk_replacement_mode__; results gain best_viterbi."""
         n = len(sentences)
         lengths = np.array([len(s) for s in sentences], np.int32)
         flat = np.ascontiguousarray(np.concatenate([np.asarray(s, np.int32) for s in sentences]))
         cap = self.cfg.longest_sentence + 2
-        o = DecodeOptions(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta)
+        o = DecodeOptions(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta,
+                          int(alignments))
         best = np.zeros((n, cap), np.int32)
+        vit = np.full((n, cap), -1, np.int32) if alignments else None
         blen = np.zeros(n, np.int32)
         bscore = np.zeros(n, np.float32)
         steps = np.zeros(n, np.int32)
@@ -325,7 +330,7 @@ class Model:
             hs = np.zeros((n, hyp_cap), np.float32)
         _check(load().lnmt_decode_batch(self.handle, _p(flat), _p(lengths), n, C.byref(o), _p(best),
                                         cap, _p(blen), _p(bscore), _p(steps), _p(ht), _p(hl),
-                                        _p(hs), hyp_cap, _p(nh)), "decode_batch")
+                                        _p(hs), hyp_cap, _p(nh), _p(vit)), "decode_batch")
         res = []
         for i in range(n):
             r = dict(best=best[i, :blen[i]].copy(), best_score=float(bscore[i]),
@@ -333,6 +338,8 @@ class Model:
             if with_hyps:
                 k = min(int(nh[i]), hyp_cap)
                 r["hyps"] = [(ht[i, j, :hl[i, j]].copy(), float(hs[i, j])) for j in range(k)]
+            if alignments:
+                r["best_viterbi"] = vit[i, :blen[i]].copy()
             res.append(r)
         return res
 

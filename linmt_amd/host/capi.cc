@@ -215,7 +215,7 @@ extern "C" int lnmt_get_state(lnmt_model *m, int kind, int side, int layer, int 
 extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int *lengths, int n,
                                  const lnmt_decode_options *o, int *best, int cap, int *best_len,
                                  float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
-                                 float *hyp_score, int hyp_cap, int *n_hyp) {
+                                 float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi) {
   return Guard([&] {
     std::vector<std::vector<int>> sents(n);
     size_t off = 0;
@@ -232,12 +232,16 @@ extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int 
     d.diversity_ = o->diversity;
     d.lp_alpha_ = o->lp_alpha;
     d.cp_beta_ = o->cp_beta;
+    d.unk_replacement_mode_ = o->unk_replacement_mode != 0;
     std::vector<SentenceResult> res;
     m->nmt->DecodeBatch(sents, d, &res);
     for (int i = 0; i < n; ++i) {
       const SentenceResult &r = res[i];
       const int bl = std::min((int)r.best.size(), cap);
       for (int j = 0; j < bl; ++j) best[(size_t)i * cap + j] = r.best[j];
+      if (best_viterbi)
+        for (int j = 0; j < bl; ++j)
+          best_viterbi[(size_t)i * cap + j] = j < (int)r.best_viterbi.size() ? r.best_viterbi[j] : -1;
       best_len[i] = bl;
       best_score[i] = r.best_score;
       if (steps) steps[i] = r.steps;

@@ -330,16 +330,26 @@ class SoftmaxLayer : public BaseLossLayer {
 struct Hypothesis {
   std::vector<int> tokens;  // <START> ... <EOF>
   float score = 0.f;        // log-probability (+ penalties), before length / coverage rescoring
+  // unk_replacement_mode_ only (decoder.h:129-130): per token the source position with the largest
+  // alignment score (-20 at <START>) and the alignment scores over the source positions
+  std::vector<int> viterbi;
+  std::vector<std::vector<float>> alignments_scores;
 };
 
 struct DecodeOptions {
   int beam_size_ = 12;
   float max_decoding_ratio_ = 1.5f, min_decoding_ratio_ = 0.5f;
   float penalty_ = 0.f, diversity_ = 0.f, lp_alpha_ = 0.65f, cp_beta_ = 0.20f;
+  // the reference's unk_replacement_mode__ (layer_attention.h:342-386): export the alignment
+  // scores of every step; hypotheses carry Viterbi alignments and the coverage penalty is computed
+  // from the exported scores instead of zeros
+  bool unk_replacement_mode_ = false;
 };
 
 struct SentenceResult {
   std::vector<int> best;  // 1-best without <START>/<EOF>
+  std::vector<int> best_viterbi;  // unk_replacement_mode_: source position aligned to each token
+  int best_index = -1;            // index of the 1-best in hypotheses
   float best_score = 0.f;
   std::vector<Hypothesis> hypotheses;  // in the order the reference's v_hypotheses_ would hold them
   int steps = 0;                       // decoder forward passes this sentence took part in
@@ -360,9 +370,13 @@ class Decoder {
   DeviceArray<float> cand_logp_, logp_eof_, score_[2], fin_score_hist_, score_hist_;
   DeviceArray<int> cand_id_, limit_, tok_hist_, backptr_hist_, fin_count_hist_, fin_beam_hist_,
       current_indices_;
+  // unk_replacement_mode_: the attention core's alignments / window indices of every step
+  // ([step][column + columns_of_that_step * slot]), allocated on first use
+  DeviceArray<float> align_hist_;
+  DeviceArray<int> index_hist_;
   void Init(int beam_size, int n_sent, int max_steps);
   // OutputKBestHypotheses (decoder.h:529-699) for one sentence, num_hypotheses = 1.
-  static void OutputKBestHypotheses(const std::vector<Hypothesis> &hyps, int source_length,
+  static void OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_length,
                                     const DecodeOptions &o, SentenceResult *out);
 };
 

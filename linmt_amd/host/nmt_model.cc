@@ -400,10 +400,11 @@ void Decoder::Init(int beam_size, int n_sent, int max_steps) {
   fin_score_hist_.Alloc(T * B);
 }
 
-// Length normalisation, coverage penalty, minimum-ratio filter, best-first (decoder.h:529-600);
-// with alignment export off every alignment-score row is the all-zero vector the reference starts
-// from (decoder.h:364-370), which is what the coverage term is computed from here too.
-void Decoder::OutputKBestHypotheses(const std::vector<Hypothesis> &hyps, int source_length,
+// Length normalisation, coverage penalty, minimum-ratio filter, best-first (decoder.h:529-600).
+// With alignment export off every alignment-score row is the all-zero vector the reference starts
+// from (decoder.h:364-370); with it on the rows are the exported scores, smoothed and normalised in
+// place as the reference does (so a later print shows the normalised values).
+void Decoder::OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_length,
                                     const DecodeOptions &o, SentenceResult *out) {
   int best = -1;
   float best_score = 0.f;
@@ -415,14 +416,31 @@ void Decoder::OutputKBestHypotheses(const std::vector<Hypothesis> &hyps, int sou
       s /= lp;
     }
     if (0 != o.cp_beta_) {
-      float sum = 0;
-      for (int k = 0; k < source_length; ++k) sum += 0.01f;
-      const float unit = 0.01f / sum;
       float cp_x_y = 0;
-      for (int k = 0; k < source_length; ++k) {
-        float col = 0;
-        for (int j = 1; j < size - 1; ++j) col += unit;
-        cp_x_y += std::log(std::min(col, 1.0f));
+      if (!hyps[i].alignments_scores.empty()) {
+        std::vector<std::vector<float>> &as = hyps[i].alignments_scores;
+        for (int j = 1; j < size - 1; ++j) {
+          float sum = 0;
+          for (int k = 0; k < source_length; ++k) {
+            as[j][k] += 0.01f;
+            sum += as[j][k];
+          }
+          for (int k = 0; k < source_length; ++k) as[j][k] /= sum;
+        }
+        for (int k = 0; k < source_length; ++k) {
+          float col = 0;
+          for (int j = 1; j < size - 1; ++j) col += as[j][k];
+          cp_x_y += std::log(std::min(col, 1.0f));
+        }
+      } else {
+        float sum = 0;
+        for (int k = 0; k < source_length; ++k) sum += 0.01f;
+        const float unit = 0.01f / sum;
+        for (int k = 0; k < source_length; ++k) {
+          float col = 0;
+          for (int j = 1; j < size - 1; ++j) col += unit;
+          cp_x_y += std::log(std::min(col, 1.0f));
+        }
       }
       cp_x_y *= o.cp_beta_;
       if (cp_x_y < -20) cp_x_y = -20;
@@ -435,17 +453,18 @@ void Decoder::OutputKBestHypotheses(const std::vector<Hypothesis> &hyps, int sou
     }
   }
   out->best.clear();
+  out->best_viterbi.clear();
+  out->best_index = best;
   out->best_score = 0.f;
   if (best >= 0) {
     const std::vector<int> &t = hyps[best].tokens;
     out->best.assign(t.begin() + 1, t.end() - 1);
+    if (!hyps[best].viterbi.empty())
+      out->best_viterbi.assign(hyps[best].viterbi.begin() + 1, hyps[best].viterbi.end() - 1);
     out->best_score = best_score;
   }
 }
 
-// Batched EnsembleFactory::DecodeFile (decoder.h:1702-1776), one model.  Sentences are processed
-// longest first so that at every step the still-active sentences are a prefix of the columns and
-// the kernels simply run on fewer columns as sentences reach their length limit.
 void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &sentences,
                                            const DecodeOptions &o,
                                            std::vector<SentenceResult> *results) {
@@ -519,6 +538,19 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
                    "TransferDecodingStatesGpu");
   }
 
+  // unk_replacement_mode_: the attention node writes every step's alignments and window indices
+  // into its own slice of a history instead of the one reused buffer
+  const bool capture = o.unk_replacement_mode_ && cfg_.attention_mode_;
+  const int W = cfg_.attention_mode_ ? attention_layer_.window_ : 0;
+  AttentionNode *an = cfg_.attention_mode_ ? &attention_layer_.v_nodes_[0] : nullptr;
+  float *const node_alignments = an ? an->p_device_alignments_ : nullptr;
+  int *const node_indices = an ? an->p_device_indices_ : nullptr;
+  const size_t hist_slice = (size_t)n_sent_ * beam * W;
+  if (capture && d.align_hist_.size() < hist_slice * d.max_steps_) {
+    d.align_hist_.Alloc(hist_slice * d.max_steps_);
+    d.index_hist_.Alloc(hist_slice * d.max_steps_);
+  }
+
   int cur = 0;
   std::vector<int> active_at(max_limit + 1);
   std::vector<std::vector<int>> bi_keep;
@@ -538,6 +570,10 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
         bi[(size_t)Ba + b] = binfo[(size_t)B + b];
       }
       attention_layer_.PreprocessMinibatchInformation(bi.data(), Ba);
+    }
+    if (capture) {
+      an->p_device_alignments_ = d.align_hist_.get() + hist_slice * step;
+      an->p_device_indices_ = d.index_hist_.get() + hist_slice * step;
     }
     ForwardPropTarget(step, p_device_step_indices, Ba);
     {
@@ -576,6 +612,16 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   d.fin_count_hist_.Download(fcount.data(), fcount.size(), stream_);
   d.fin_beam_hist_.Download(fbeam.data(), fbeam.size(), stream_);
   d.fin_score_hist_.Download(fscore.data(), fscore.size(), stream_);
+  std::vector<float> ahist;
+  std::vector<int> ihist;
+  if (capture) {
+    an->p_device_alignments_ = node_alignments;
+    an->p_device_indices_ = node_indices;
+    ahist.resize(hist_slice * steps);
+    ihist.resize(hist_slice * steps);
+    d.align_hist_.Download(ahist.data(), ahist.size(), stream_);
+    d.index_hist_.Download(ihist.data(), ihist.size(), stream_);
+  }
   Synchronize();
   profiler_.Collect();
 
@@ -586,26 +632,60 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
     SentenceResult &r = (*results)[order[k]];
     r.steps = limit[k] + 1;
     const int c0 = k * beam;
-    auto prefix = [&](int step, int column, std::vector<int> *out) {
-      // tokens chosen at steps 0..step-1 along the path that ends in `column` before step `step`
-      out->assign(step + 1, Decoder::start_symbol_);
+    const int source_length = (int)sentences[order[k]].size();
+    // alignment scores over the source positions of `column` at step t, and their arg-max as
+    // EnsemblesModels takes it (decoder.h:1946-1961): first strictly largest score above 0
+    auto alignment_row = [&](int t, int column, std::vector<float> *scores, int *viterbi) {
+      // (the reference's rows have longest_sentence_ entries; those past the sentence stay zero
+      // and are never read)
+      scores->assign(source_length, 0.f);
+      const size_t Ba_t = (size_t)active_at[t] * beam;
+      for (int j = 0; j < W; ++j) {
+        const size_t at = hist_slice * t + column + Ba_t * j;
+        const int idx = ihist[at];
+        if (idx >= 0 && idx < source_length) (*scores)[idx] = ahist[at];
+      }
+      float max_val = 0;
+      *viterbi = -1;
+      for (int j = 0; j < source_length; ++j)
+        if ((*scores)[j] > max_val) {
+          max_val = (*scores)[j];
+          *viterbi = j;
+        }
+    };
+    auto prefix = [&](int step, int column, Hypothesis *h) {
+      // tokens chosen at steps 0..step-1 along the path that ends in `column` before step `step`;
+      // token t+1 was produced by the forward pass of its PARENT column at step t, whose
+      // alignments it carries (decoder.h:452-456)
+      h->tokens.assign(step + 1, Decoder::start_symbol_);
+      if (capture) {
+        h->viterbi.assign(step + 2, -20);
+        h->alignments_scores.assign(step + 2, std::vector<float>());
+      }
       int col = column;
       for (int t = step - 1; t >= 0; --t) {
-        (*out)[t + 1] = tok[(size_t)t * B + col];
+        h->tokens[t + 1] = tok[(size_t)t * B + col];
         col = bp[(size_t)t * B + col];
+        if (capture) alignment_row(t, col, &h->alignments_scores[t + 1], &h->viterbi[t + 1]);
       }
     };
     for (int step = 0; step <= limit[k]; ++step) {
       const int nf = fcount[(size_t)step * n + k];
       for (int f = 0; f < nf; ++f) {
         Hypothesis h;
-        prefix(step, c0 + fbeam[(size_t)step * B + c0 + f], &h.tokens);
+        const int parent = c0 + fbeam[(size_t)step * B + c0 + f];
+        prefix(step, parent, &h);
         h.tokens.push_back(Decoder::end_symbol_);
+        if (capture)  // <EOF> itself comes out of the parent's forward pass at this step
+          alignment_row(step, parent, &h.alignments_scores[step + 1], &h.viterbi[step + 1]);
         h.score = fscore[(size_t)step * B + c0 + f];
         r.hypotheses.push_back(std::move(h));
       }
     }
-    Decoder::OutputKBestHypotheses(r.hypotheses, (int)sentences[order[k]].size(), o, &r);
+    Decoder::OutputKBestHypotheses(r.hypotheses, source_length, o, &r);
+    if (capture)  // only the 1-best keeps its score rows (they are what a printout shows)
+      for (size_t h = 0; h < r.hypotheses.size(); ++h)
+        if ((int)h != r.best_index) std::vector<std::vector<float>>().swap(r.hypotheses[h].alignments_scores);
   }
 }
 

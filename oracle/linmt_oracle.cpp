@@ -629,7 +629,8 @@ namespace {
 // Attention node on top of the decoder stack (ha = h_t, no dropout), writing h_tild.
 void attention_step(orc_model *m, int B, const float *h_t, const float *hs, long long step_stride,
                     long long col_stride, const int *hs_col, int hs_steps, const int *batch_info,
-                    const int *mask01, int max_len, float *h_tild) {
+                    const int *mask01, int max_len, float *h_tild, std::vector<int> *out_indices = nullptr,
+                    std::vector<float> *out_align = nullptr) {
   const int H = m->cfg.H;
   const int D = m->cfg.attention == 1 ? m->cfg.D : -1;
   const int W = D >= 0 ? 2 * D + 1 : max_len;
@@ -644,6 +645,8 @@ void attention_step(orc_model *m, int B, const float *h_t, const float *hs, long
   orc_attn_core_fwd(H, B, D, max_len, hs_steps, tanh1.data(), m->params["attn.v_p"].data(),
                     wa.data(), hs, step_stride, col_stride, hs_col, batch_info, mask01, pt.data(),
                     sig.data(), ind.data(), al.data(), ce.data(), cx.data(), nullptr);
+  if (out_indices) *out_indices = ind;
+  if (out_align) *out_align = al;
   mat_apply(m, "attn.W_c1", H, H, cx.data(), B, t1.data());
   mat_apply(m, "attn.W_c2", H, H, h_t, B, t2.data());
   const float *b_out = m->params["attn.b_out"].data();
@@ -659,7 +662,15 @@ void attention_step(orc_model *m, int B, const float *h_t, const float *hs, long
 struct Hyp {
   std::vector<int> tokens;  // with <START> ... <EOF>
   float score;
+  // unk_replacement_mode__ only: per token the source position with the largest alignment score
+  // and the alignment scores over the source positions (decoder.h:129-130)
+  std::vector<int> viterbi;
+  std::vector<std::vector<float>> align_scores;
 };
+
+int decode_impl(orc_model *m, const int *src_ids, int S, const orc_decode_opts *o, bool unk_mode,
+                int *best_tokens, int cap, int *best_len, float *best_score, int *hyp_tokens,
+                int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi);
 
 }  // namespace
 
@@ -673,6 +684,27 @@ extern "C" int orc_decode_sentence(orc_model *m, const int *src_ids, int S,
                                    const orc_decode_opts *o, int *best_tokens, int cap,
                                    int *best_len, float *best_score, int *hyp_tokens, int *hyp_len,
                                    float *hyp_score, int hyp_cap, int *n_hyp) {
+  return decode_impl(m, src_ids, S, o, false, best_tokens, cap, best_len, best_score, hyp_tokens,
+                     hyp_len, hyp_score, hyp_cap, n_hyp, nullptr);
+}
+
+// The same with unk_replacement_mode__ on (layer_attention.h:342-386, decoder.h:1930-1962): every
+// step exports the alignment scores over the source positions, the Viterbi alignment is their
+// arg-max, both travel with the hypotheses, and the coverage penalty of OutputKBestHypotheses sees
+// real scores.  best_viterbi (capacity cap) receives the alignments of the 1-best's tokens.
+extern "C" int orc_decode_sentence_alignments(orc_model *m, const int *src_ids, int S,
+                                              const orc_decode_opts *o, int *best_tokens, int cap,
+                                              int *best_len, float *best_score, int *best_viterbi,
+                                              int *hyp_tokens, int *hyp_len, float *hyp_score,
+                                              int hyp_cap, int *n_hyp) {
+  return decode_impl(m, src_ids, S, o, m->cfg.attention != 0, best_tokens, cap, best_len, best_score,
+                     hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, best_viterbi);
+}
+
+namespace {
+int decode_impl(orc_model *m, const int *src_ids, int S, const orc_decode_opts *o, bool unk_mode,
+                int *best_tokens, int cap, int *best_len, float *best_score, int *hyp_tokens,
+                int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi) {
 #ifdef _OPENMP
   if (o->num_threads > 0) omp_set_num_threads(o->num_threads);
 #endif
@@ -734,6 +766,15 @@ extern "C" int orc_decode_sentence(orc_model *m, const int *src_ids, int S,
   std::vector<float> top_scores(B, 0.f), top_scores_tmp(B, 0.f);
   std::vector<int> current_indices(B, start_symbol), new_indices_changes(B, 0);
   std::vector<Hyp> hyps;
+  // viterbi_alignments__ / alignment_scores__ (utility_cu.h:91-93) and the per-beam histories
+  // eigen_top_sentences_viterbi_ (initialised to -20, decoder.h:347) / _alignments_scores_
+  std::vector<int> vit(B, -1), top_vit((size_t)B * longest, -20), top_vit_tmp;
+  std::vector<float> ascore((size_t)longest * B, 0.f);
+  std::vector<std::vector<float>> top_as((size_t)B * longest), top_as_tmp;
+  auto column_scores = [&](int b) {
+    return std::vector<float>(ascore.begin() + (size_t)longest * b,
+                              ascore.begin() + (size_t)longest * (b + 1));
+  };
 
   std::vector<float> xb((size_t)H * B), logits((size_t)V * B), dist((size_t)V * B);
   std::vector<int> tok(B), bp(B), fin_beam(B);
@@ -754,9 +795,34 @@ extern "C" int orc_decode_sentence(orc_model *m, const int *src_ids, int S,
     }
     const float *top = cur[L - 1].h.data();
     if (cfg.attention) {
+      std::vector<int> ind;
+      std::vector<float> al;
       attention_step(m, B, top, top_states.data(), H, 0, hs_col.data(), S, batch_info.data(),
-                     ones.data(), S, h_tild.data());
+                     ones.data(), S, h_tild.data(), &ind, &al);
       top = h_tild.data();
+      if (unk_mode) {
+        // layer_attention.h:360-385: scores of the window's valid slots, zero elsewhere
+        std::fill(ascore.begin(), ascore.end(), 0.f);
+        const int W = (int)(ind.size() / B);
+        for (int j = 0; j < W; ++j)
+          for (int b = 0; b < B; ++b) {
+            const int idx = ind[idx2c(b, j, B)];
+            if (idx != -1) ascore[(size_t)idx + (size_t)longest * b] = al[idx2c(b, j, B)];
+          }
+        // EnsemblesModels (decoder.h:1946-1961): first strictly largest score above 0
+        for (int b = 0; b < B; ++b) {
+          float max_val = 0;
+          int max_index = -1;
+          for (int j = 0; j < longest; ++j) {
+            const float v = ascore[(size_t)j + (size_t)longest * b];
+            if (v > max_val) {
+              max_val = v;
+              max_index = j;
+            }
+          }
+          vit[b] = max_index;
+        }
+      }
     }
     mat_apply(m, "softmax.D", V, H, top, B, logits.data());
     orc_softmax_fwd(logits.data(), V, m->params["softmax.b_d"].data(), V, B, dist.data(), V);
@@ -780,7 +846,28 @@ extern "C" int orc_decode_sentence(orc_model *m, const int *src_ids, int S,
         h.tokens[j] = top_sentences[(size_t)fin_beam[f] * longest + j];
       h.tokens[current_index + 1] = end_symbol;
       h.score = fin_score[f];
+      if (unk_mode) {
+        const size_t row = (size_t)fin_beam[f] * longest;
+        h.viterbi.assign(top_vit.begin() + row, top_vit.begin() + row + current_index + 2);
+        h.viterbi[current_index + 1] = vit[fin_beam[f]];
+        h.align_scores.assign(top_as.begin() + row, top_as.begin() + row + current_index + 2);
+        h.align_scores[current_index + 1] = column_scores(fin_beam[f]);
+      }
       hyps.push_back(h);
+    }
+    if (unk_mode) {
+      top_vit_tmp = top_vit;
+      top_as_tmp = top_as;
+      for (int i = 0; i < B; ++i) {
+        for (int j = 0; j < longest; ++j) {
+          top_vit_tmp[(size_t)i * longest + j] = top_vit[(size_t)bp[i] * longest + j];
+          top_as_tmp[(size_t)i * longest + j] = top_as[(size_t)bp[i] * longest + j];
+        }
+        top_vit_tmp[(size_t)i * longest + current_index + 1] = vit[bp[i]];
+        top_as_tmp[(size_t)i * longest + current_index + 1] = column_scores(bp[i]);
+      }
+      top_vit.swap(top_vit_tmp);
+      top_as.swap(top_as_tmp);
     }
     for (int i = 0; i < B; ++i) {
       memcpy(&top_tmp[(size_t)i * longest], &top_sentences[(size_t)bp[i] * longest],
@@ -816,6 +903,13 @@ extern "C" int orc_decode_sentence(orc_model *m, const int *src_ids, int S,
       h.tokens.assign(top_sentences.begin() + (size_t)i * longest,
                       top_sentences.begin() + (size_t)i * longest + current_index + 2);
       h.score = top_scores[i];
+      if (unk_mode) {
+        const size_t row = (size_t)i * longest;
+        h.viterbi.assign(top_vit.begin() + row, top_vit.begin() + row + current_index + 2);
+        h.viterbi[current_index + 1] = vit[i];
+        h.align_scores.assign(top_as.begin() + row, top_as.begin() + row + current_index + 2);
+        h.align_scores[current_index + 1] = column_scores(i);
+      }
       hyps.push_back(h);
     }
     current_index += 1;
@@ -840,7 +934,28 @@ extern "C" int orc_decode_sentence(orc_model *m, const int *src_ids, int S,
       const float lp = powf((float)(5 + size), o->lp_alpha) / powf((float)(5 + 1), o->lp_alpha);
       s /= lp;
     }
-    if (0 != o->cp_beta) {
+    if (0 != o->cp_beta && unk_mode) {
+      // decoder.h:541-583 on the exported scores: +0.01, rows normalised over the source, then
+      // the log of each source position's capped total
+      std::vector<std::vector<float>> &as = hyps[i].align_scores;
+      for (int j = 1; j < size - 1; ++j) {
+        float sum = 0;
+        for (int k = 0; k < S; ++k) {
+          as[j][k] += 0.01f;
+          sum += as[j][k];
+        }
+        for (int k = 0; k < S; ++k) as[j][k] /= sum;
+      }
+      float cp = 0;
+      for (int k = 0; k < S; ++k) {
+        float sum = 0;
+        for (int j = 1; j < size - 1; ++j) sum += as[j][k];
+        cp += std::log(std::min(sum, 1.0f));
+      }
+      cp *= o->cp_beta;
+      if (cp < -20) cp = -20;
+      s += cp;
+    } else if (0 != o->cp_beta) {
       // alignment-score rows are all zero: +0.01 each, normalised to 0.01/sum(0.01 x S)
       float unit;
       {
@@ -876,12 +991,16 @@ extern "C" int orc_decode_sentence(orc_model *m, const int *src_ids, int S,
   if (best >= 0) {
     const auto &t = hyps[best].tokens;
     int n = 0;
-    for (size_t j = 1; j + 1 < t.size() && n < cap; ++j) best_tokens[n++] = t[j];
+    for (size_t j = 1; j + 1 < t.size() && n < cap; ++j) {
+      if (best_viterbi) best_viterbi[n] = unk_mode ? hyps[best].viterbi[j] : -1;
+      best_tokens[n++] = t[j];
+    }
     *best_len = n;
     *best_score = rs[best];
   }
   return steps_run;
 }
+}  // namespace
 
 // NeuralMachineTranslation::GetError (src/deep_rnn.h:2173-2317) with SoftmaxLayer::ComputeLossGpu.
 extern "C" double orc_forward_xent(orc_model *m, const int *src, int S, const int *tgt_in,

@@ -105,6 +105,14 @@ int orc_decode_sentence(orc_model *m, const int *src_ids, int S, const orc_decod
                         int *best_tokens, int cap, int *best_len, float *best_score,
                         int *hyp_tokens, int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp);
 
+/* The same with the reference's unk_replacement_mode__ on: alignment scores exported at every
+ * step, Viterbi alignments carried by the hypotheses, coverage penalty on the real scores.
+ * best_viterbi (capacity cap) receives the source position aligned to each token of the 1-best. */
+int orc_decode_sentence_alignments(orc_model *m, const int *src_ids, int S, const orc_decode_opts *o,
+                                   int *best_tokens, int cap, int *best_len, float *best_score,
+                                   int *best_viterbi, int *hyp_tokens, int *hyp_len,
+                                   float *hyp_score, int hyp_cap, int *n_hyp);
+
 /* Teacher-forced forward + cross-entropy (GetError): src B x S and tgt_in/tgt_out B x T, all
  * column-major with -1 padding (source reversed + left-padded, target right-padded).
  * Returns sum over non-pad target positions of log p(target) (natural log, double). */

@@ -286,7 +286,10 @@ class Model:
         lib().orc_model_commit(self.handle)
 
     def decode_sentence(self, src_ids, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0,
-                        diversity=0.0, lp_alpha=0.65, cp_beta=0.20, num_threads=0, hyp_cap=4096):
+                        diversity=0.0, lp_alpha=0.65, cp_beta=0.20, num_threads=0, hyp_cap=4096,
+                        alignments=False):
+        """alignments=True: the reference's unk_replacement_mode__ (exported alignment scores,
+        coverage penalty on them); the result then holds best_viterbi."""
         src_ids = i32(src_ids)
         cap = self.cfg.longest_sent + 2
         o = DecodeOpts(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta,
@@ -298,13 +301,22 @@ class Model:
         hl = np.zeros(hyp_cap, np.int32)
         hs = np.zeros(hyp_cap, np.float32)
         nh = C.c_int(0)
-        steps = lib().orc_decode_sentence(self.handle, _p(src_ids), src_ids.size, C.byref(o),
-                                          _p(best), cap, C.byref(blen), C.byref(bscore), _p(ht),
-                                          _p(hl), _p(hs), hyp_cap, C.byref(nh))
+        vit = np.full(cap, -1, np.int32)
+        if alignments:
+            steps = lib().orc_decode_sentence_alignments(
+                self.handle, _p(src_ids), src_ids.size, C.byref(o), _p(best), cap, C.byref(blen),
+                C.byref(bscore), _p(vit), _p(ht), _p(hl), _p(hs), hyp_cap, C.byref(nh))
+        else:
+            steps = lib().orc_decode_sentence(self.handle, _p(src_ids), src_ids.size, C.byref(o),
+                                              _p(best), cap, C.byref(blen), C.byref(bscore),
+                                              _p(ht), _p(hl), _p(hs), hyp_cap, C.byref(nh))
         n = min(nh.value, hyp_cap)
         hyps = [(ht[i, :hl[i]].copy(), float(hs[i])) for i in range(n)]
-        return dict(best=best[:blen.value].copy(), best_score=float(bscore.value), hyps=hyps,
-                    steps=steps)
+        out = dict(best=best[:blen.value].copy(), best_score=float(bscore.value), hyps=hyps,
+                   steps=steps)
+        if alignments:
+            out["best_viterbi"] = vit[:blen.value].copy()
+        return out
 
     def forward_xent(self, src, tgt_in, tgt_out, batch_info, num_threads=0):
         """src (B,S), tgt_in/tgt_out (B,T) int arrays with -1 padding (column t = timestep t)."""

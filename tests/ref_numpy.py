@@ -113,10 +113,14 @@ def encode(P, layers, H, src_ids):
 
 def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=True, max_ratio=1.5,
                 min_ratio=0.5, penalty=0.0, diversity=0.0, lp_alpha=0.65, cp_beta=0.2,
-                longest=104, margins=None):
+                longest=104, margins=None, alignments=False):
     """Sort-based beam search with the reference's rules (src/decoder.h:355-699).  Returns
     (best_tokens, best_score, hyps); margins (list) collects the smallest score gaps seen, so a test
-    can skip seeds whose decisions are closer than fp32 can resolve."""
+    can skip seeds whose decisions are closer than fp32 can resolve.
+    alignments=True (the reference's unk_replacement_mode__): every token carries the attention
+    weights over the source positions of the step that produced it; the coverage penalty is computed
+    from them and a fourth result holds, per 1-best token, the source position of the largest
+    weight (-1 if none is positive)."""
     S = len(src_ids)
     beam = min(beam, int(np.sqrt(V)))
     he, ce, top = encode(P, layers, H, src_ids)
@@ -126,7 +130,8 @@ def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=Tr
     tokens = np.zeros(beam, int)
     scores = np.zeros(beam)
     hist = [[0] for _ in range(beam)]
-    hyps = []
+    ahist = [[] for _ in range(beam)]  # per token: dict source position -> attention weight
+    hyps, hyp_align = [], []
     D64 = P["softmax.D"].astype(np.float64)
     bd = P["softmax.b_d"].astype(np.float64)
     Wt = P["tgt.0.W"].astype(np.float64)
@@ -144,14 +149,14 @@ def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=Tr
             nc.append(b_)
             x = a
         topv = x
-        ht_new = None
+        ht_new, al = None, [{} for _ in range(beam)]
         if attention:
-            ht_new, _ = attention_local_p(P, topv, lambda b, s: top[s], [S] * beam, ones, D)
+            ht_new, al = attention_local_p(P, topv, lambda b, s: top[s], [S] * beam, ones, D)
             topv = ht_new
-        return nh, nc, ht_new, log_softmax(D64 @ topv + bd[:, None])
+        return nh, nc, ht_new, log_softmax(D64 @ topv + bd[:, None]), al
 
     for step in range(limit):
-        nh, nc, ht_new, lp = forward(step)
+        nh, nc, ht_new, lp, al = forward(step)
         cands = []
         for i in range(1 if step == 0 else beam):
             order = np.lexsort((np.arange(V), -lp[:, i]))[: beam + 1]
@@ -172,33 +177,54 @@ def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=Tr
                 continue
             if v == 1:
                 hyps.append((hist[i] + [1], s_ + penalty))
+                hyp_align.append(ahist[i] + [al[i]])
                 continue
             new_tok.append(v)
             new_bp.append(i)
             new_sc.append(s_ + penalty)
         assert len(new_tok) == beam
         hist = [hist[i] + [v] for i, v in zip(new_bp, new_tok)]
+        ahist = [ahist[i] + [al[i]] for i in new_bp]
         tokens = np.array(new_tok)
         scores = np.array(new_sc)
         h = [x[:, new_bp] for x in nh]
         c = [x[:, new_bp] for x in nc]
         if attention:
             h_tild = ht_new[:, new_bp]
-    _, _, _, lp = forward(limit if limit > 0 else 1)
+    _, _, _, lp, al = forward(limit if limit > 0 else 1)
     for i in range(beam):
         hyps.append((hist[i] + [1], scores[i] + lp[1, i] + penalty))
+        hyp_align.append(ahist[i] + [al[i]])
 
-    best, best_s = None, None
-    for toks, s_ in hyps:
+    best, best_s, best_al = None, None, None
+    for (toks, s_), al_h in zip(hyps, hyp_align):
         n = len(toks)
         r = s_
         if lp_alpha != 0:
             r = r / (((5.0 + n) ** lp_alpha) / (6.0 ** lp_alpha))
-        if cp_beta != 0:
+        if cp_beta != 0 and alignments:
+            # rows = the n-2 real tokens (al_h[j] belongs to token j+1; <EOF>'s row is left out),
+            # smoothed by 0.01 and normalised over the source; coverage = capped column sums
+            rows = np.zeros((max(n - 2, 0), S))
+            for j in range(n - 2):
+                for pos, a in al_h[j].items():
+                    rows[j, pos] = a
+            rows = rows + 0.01
+            rows = rows / rows.sum(axis=1, keepdims=True) if n > 2 else rows
+            cp = cp_beta * np.sum(np.log(np.minimum(rows.sum(axis=0), 1.0))) if n > 2 else -np.inf
+            r = r + max(cp, -20.0)
+        elif cp_beta != 0:
             cp = cp_beta * S * np.log(min((n - 2) / S, 1.0)) if n > 2 else -np.inf
             r = r + max(cp, -20.0)
         if n / S > min_ratio and (best is None or r > best_s):
-            best, best_s = toks, r
+            best, best_s, best_al = toks, r, al_h
+    if alignments:
+        vit = []
+        for j in range(len(best) - 2 if best is not None else 0):
+            pos = sorted(best_al[j].items())
+            top_a = max([a for _, a in pos], default=0.0)
+            vit.append(next((p for p, a in pos if a == top_a), -1) if top_a > 0 else -1)
+        return (best[1:-1] if best is not None else []), best_s, hyps, vit
     return (best[1:-1] if best is not None else []), best_s, hyps
 
 

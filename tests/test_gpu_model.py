@@ -91,6 +91,29 @@ def test_decode_options_vs_oracle(orc, host):
     gm.close()
 
 
+def test_decode_with_exported_alignments_vs_oracle(orc, host):
+    """unk_replacement_mode__: alignment scores exported at every step (a ragged batch, so the
+    number of live columns changes between steps), Viterbi alignment per 1-best token and the
+    coverage penalty computed from the scores -- against the oracle's single-sentence search,
+    which is pinned on the numpy model (tests/test_oracle_pins.py)."""
+    rng = np.random.default_rng(14)
+    for layers, H, Vs, Vt, D, beam, lens in ((2, 48, 60, 70, 2, 4, (11, 4, 7, 1, 9)),
+                                             (1, 32, 40, 90, 10, 5, (6, 14, 3))):
+        P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 30, 0.5, decoding=(len(lens), beam))
+        sents = [rng.integers(0, Vs, size=n) for n in lens]
+        for kw in (dict(), dict(cp_beta=0.6, lp_alpha=0.3)):
+            got = gm.decode_batch(sents, beam=beam, with_hyps=True, alignments=True, **kw)
+            plain = gm.decode_batch(sents, beam=beam, with_hyps=True, **kw)
+            for i, s in enumerate(sents):
+                want = om.decode_sentence(s, beam=beam, alignments=True, **kw)
+                _compare_decode(want, got[i], f"{kw} sentence {i} (len {len(s)})")
+                assert got[i]["best_viterbi"].tolist() == want["best_viterbi"].tolist(), (i, kw)
+                assert all(-1 <= v < len(s) for v in got[i]["best_viterbi"])
+                # the search itself is the same with and without the export
+                assert len(plain[i]["hyps"]) == len(got[i]["hyps"])
+        gm.close()
+
+
 def test_decode_no_attention_and_no_feed(orc, host):
     rng = np.random.default_rng(5)
     for attention, feed in ((0, False), (1, False)):

@@ -302,6 +302,33 @@ def test_decode_sentence_vs_numpy_beam_search(orc):
     assert checked >= 3
 
 
+def test_decode_sentence_with_exported_alignments_vs_numpy(orc):
+    """The unk_replacement_mode__ variant: alignment scores exported per step, coverage penalty on
+    them, Viterbi alignment per 1-best token -- against the numpy model, which carries the float64
+    attention weights of every token and applies the definition of the penalty directly."""
+    rng = np.random.default_rng(13)
+    checked = differs = 0
+    for trial in range(10):
+        P, m = _tiny_model(orc, rng)
+        S = int(rng.integers(3, 9))
+        src = rng.integers(0, 30, size=S)
+        margins = []
+        best, best_s, hyps, vit = R.beam_decode(P, 2, 12, 37, src, beam=3, D=2, longest=40,
+                                                margins=margins, alignments=True)
+        if min(margins) < 1e-4:
+            continue
+        got = m.decode_sentence(src, beam=3, alignments=True)
+        assert got["best"].tolist() == list(best)
+        assert_close(got["best_score"], best_s, "rescored 1-best", rtol=1e-4, atol=1e-4)
+        assert got["best_viterbi"].tolist() == vit
+        assert all(-1 <= v < S for v in vit)
+        plain = m.decode_sentence(src, beam=3)
+        assert len(plain["hyps"]) == len(got["hyps"])  # the search itself does not change
+        differs += int(abs(plain["best_score"] - got["best_score"]) > 1e-3)
+        checked += 1
+    assert checked >= 5 and differs >= 3  # the penalty really is computed from the scores
+
+
 def test_forward_xent_vs_numpy(orc):
     """Teacher-forced forward + CE on a ragged minibatch (reversed, left-padded source; right-padded
     target; -1 padding) against the float64 numpy model run sentence by sentence."""
