@@ -196,6 +196,37 @@ int lnmt_tuning(lnmt_model *m, const lnmt_tuning_options *o, lnmt_tuning_event *
 /* NeuralMachineTranslation::GetPerplexity (src/deep_rnn.h:1490-1568) over an integerised file. */
 int lnmt_get_perplexity(lnmt_model *m, const char *file_name, double *perplexity);
 
+/* Dispatcher::Decoding (src/dispatcher.cu:387-436): translate a text file with a reference model
+ * file.  Source lines -> ids with the model's source vocabulary (IntegerizeFileDecoding,
+ * src/input_file_preprocess.cc:1312-1482; sentences with length + 1 >= longest_sentence - 2 are
+ * thrown away as the reference does), batched beam search, one line of ids per sentence in the
+ * format of Decoder::OutputKBestHypotheses (src/decoder.h:602-681; with print_decoding_information:
+ * " |||| score |||| Viterbi alignments |||| alignments of the <UNK> tokens", with
+ * print_alignments_scores also the alignment scores), then ids -> words (UnintFile,
+ * src/input_file_preprocess.cc:1485-1581).  seconds covers the search only. */
+typedef struct lnmt_decoding_options {
+  const char *model_file, *source_file;
+  const char *ids_file;   /* NULL: final_file + ".ids" */
+  const char *final_file;
+  int beam_size;
+  float penalty, max_decoding_ratio, min_decoding_ratio, lp_alpha, cp_beta, diversity;
+  int longest_sentence;
+  int attention_width; /* D of the local-p window (not stored in the model file); <= 0: 10 */
+  int print_decoding_information, print_alignments_scores, unk_replacement_mode;
+  int sentences_per_batch;
+} lnmt_decoding_options;
+int lnmt_decoding(const lnmt_decoding_options *o, int *sentences, int *sentences_thrown_away,
+                  long long *source_words, long long *target_words, double *seconds);
+/* The two file conversions on their own (host only, no GPU).  lnmt_integerize_file_decoding:
+ * ids (concatenated, reading order) / lengths / input line numbers of the sentences kept;
+ * *n_sentences receives their number, which may exceed max_sentences (then call again). */
+int lnmt_integerize_file_decoding(const char *model_file, const char *source_file,
+                                  int max_sent_cutoff, int *ids, long long ids_cap, int *lengths,
+                                  int *lines, int max_sentences, int *n_sentences,
+                                  int *target_vocab_size);
+int lnmt_unint_file(const char *model_file, const char *unint_file, const char *final_file,
+                    int sequence_to_sequence, int decoder_mode);
+
 #ifdef __cplusplus
 }
 #endif

@@ -47,6 +47,17 @@ class TuningEvent(C.Structure):
                 ("value", C.c_double)]
 
 
+class DecodingOptions(C.Structure):
+    _fields_ = [("model_file", C.c_char_p), ("source_file", C.c_char_p), ("ids_file", C.c_char_p),
+                ("final_file", C.c_char_p), ("beam_size", C.c_int), ("penalty", C.c_float),
+                ("max_decoding_ratio", C.c_float), ("min_decoding_ratio", C.c_float),
+                ("lp_alpha", C.c_float), ("cp_beta", C.c_float), ("diversity", C.c_float),
+                ("longest_sentence", C.c_int), ("attention_width", C.c_int),
+                ("print_decoding_information", C.c_int),
+                ("print_alignments_scores", C.c_int), ("unk_replacement_mode", C.c_int),
+                ("sentences_per_batch", C.c_int)]
+
+
 class DecodeOptions(C.Structure):
     _fields_ = [("beam_size", C.c_int), ("max_decoding_ratio", C.c_float),
                 ("min_decoding_ratio", C.c_float), ("penalty", C.c_float),
@@ -108,6 +119,13 @@ def load():
     lib.lnmt_file_helper_read_minibatch.argtypes = [C.c_void_p]
     lib.lnmt_file_helper_get.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_longlong]
     lib.lnmt_file_helper_info.argtypes = [C.c_void_p, C.POINTER(C.c_int * 8)]
+    lib.lnmt_decoding.argtypes = [C.POINTER(DecodingOptions), C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                  C.POINTER(C.c_longlong), C.POINTER(C.c_longlong),
+                                  C.POINTER(C.c_double)]
+    lib.lnmt_integerize_file_decoding.argtypes = [C.c_char_p, C.c_char_p, C.c_int, C.c_void_p,
+                                                  C.c_longlong, C.c_void_p, C.c_void_p, C.c_int,
+                                                  C.POINTER(C.c_int), C.POINTER(C.c_int)]
+    lib.lnmt_unint_file.argtypes = [C.c_char_p, C.c_char_p, C.c_char_p, C.c_int, C.c_int]
     lib.lnmt_tuning.argtypes = [C.c_void_p, C.POINTER(TuningOptions), C.POINTER(TuningEvent),
                                 C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_longlong),
                                 C.POINTER(C.c_double), C.POINTER(C.c_float)]
@@ -342,6 +360,48 @@ class Model:
                 r["best_viterbi"] = vit[i, :blen[i]].copy()
             res.append(r)
         return res
+
+
+def decoding(model_file, source_file, final_file, ids_file=None, beam=12, penalty=0.0,
+             max_ratio=1.5, min_ratio=0.5, lp_alpha=0.65, cp_beta=0.20, diversity=0.0,
+             longest_sentence=200, attention_width=10, print_decoding_information=False,
+             print_alignments_scores=False, unk_replacement_mode=False, sentences_per_batch=64):
+    """Dispatcher::Decoding: translate a text file with a reference model file."""
+    enc = lambda p: None if p is None else os.fsencode(p)  # noqa: E731
+    o = DecodingOptions(enc(model_file), enc(source_file), enc(ids_file), enc(final_file), beam,
+                        penalty, max_ratio, min_ratio, lp_alpha, cp_beta, diversity,
+                        longest_sentence, attention_width, int(print_decoding_information),
+                        int(print_alignments_scores), int(unk_replacement_mode),
+                        sentences_per_batch)
+    n, thrown, sw, tw, secs = C.c_int(), C.c_int(), C.c_longlong(), C.c_longlong(), C.c_double()
+    _check(load().lnmt_decoding(C.byref(o), C.byref(n), C.byref(thrown), C.byref(sw), C.byref(tw),
+                                C.byref(secs)), "decoding")
+    return dict(sentences=n.value, sentences_thrown_away=thrown.value, source_words=sw.value,
+                target_words=tw.value, seconds=secs.value)
+
+
+def integerize_file_decoding(model_file, source_file, max_sent_cutoff):
+    """IntegerizeFileDecoding: (list of id arrays in reading order, input line of each, target
+    vocabulary size)."""
+    lib = load()
+    n, v = C.c_int(), C.c_int()
+    cap_s, cap_i = 1 << 16, 1 << 22
+    ids, lens, lines = np.empty(cap_i, np.int32), np.empty(cap_s, np.int32), np.empty(cap_s, np.int32)
+    _check(lib.lnmt_integerize_file_decoding(os.fsencode(model_file), os.fsencode(source_file),
+                                             max_sent_cutoff, _p(ids), cap_i, _p(lens), _p(lines),
+                                             cap_s, C.byref(n), C.byref(v)),
+           "integerize_file_decoding")
+    out, at = [], 0
+    for i in range(min(n.value, cap_s)):
+        out.append(ids[at:at + lens[i]].copy())
+        at += lens[i]
+    return out, lines[:len(out)].tolist(), v.value
+
+
+def unint_file(model_file, unint_path, final_path, sequence_to_sequence=True, decoder_mode=True):
+    _check(load().lnmt_unint_file(os.fsencode(model_file), os.fsencode(unint_path),
+                                  os.fsencode(final_path), int(sequence_to_sequence),
+                                  int(decoder_mode)), "unint_file")
 
 
 def read_model_information(path):

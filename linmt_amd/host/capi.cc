@@ -6,6 +6,7 @@
 #include "../../include/linmt_host.h"
 #include "dispatcher.h"
 #include "file_helper.h"
+#include "input_file_preprocess.h"
 #include "nmt.h"
 
 using namespace linmt;
@@ -415,4 +416,66 @@ extern "C" int lnmt_tuning(lnmt_model *m, const lnmt_tuning_options *o, lnmt_tun
 
 extern "C" int lnmt_get_perplexity(lnmt_model *m, const char *file_name, double *perplexity) {
   return Guard([&] { *perplexity = m->nmt->GetPerplexity(file_name); });
+}
+
+extern "C" int lnmt_decoding(const lnmt_decoding_options *o, int *sentences, int *sentences_thrown_away,
+                             long long *source_words, long long *target_words, double *seconds) {
+  return Guard([&] {
+    if (!o || !o->model_file || !o->source_file || !o->final_file)
+      throw LinmtError("lnmt_decoding: model_file, source_file and final_file are required");
+    DecodingConfiguration c;
+    c.model_name_ = o->model_file;
+    c.decode_user_file_ = o->source_file;
+    c.decoder_output_file_ = o->ids_file ? o->ids_file : "";
+    c.decoder_final_file_ = o->final_file;
+    c.beam_size_ = o->beam_size;
+    c.penalty_ = o->penalty;
+    c.max_decoding_ratio_ = o->max_decoding_ratio;
+    c.min_decoding_ratio_ = o->min_decoding_ratio;
+    c.decoding_lp_alpha_ = o->lp_alpha;
+    c.decoding_cp_beta_ = o->cp_beta;
+    c.decoding_diversity_ = o->diversity;
+    if (o->longest_sentence > 0) c.longest_sentence_ = o->longest_sentence;
+    if (o->attention_width > 0) c.attention_width_ = o->attention_width;
+    c.print_decoding_information_mode_ = o->print_decoding_information != 0;
+    c.print_alignments_scores_mode_ = o->print_alignments_scores != 0;
+    c.unk_replacement_mode_ = o->unk_replacement_mode != 0;
+    if (o->sentences_per_batch > 0) c.sentences_per_batch_ = o->sentences_per_batch;
+    const DecodingReport r = Dispatcher::Decoding(c);
+    if (sentences) *sentences = r.sentences;
+    if (sentences_thrown_away) *sentences_thrown_away = r.sentences_thrown_away;
+    if (source_words) *source_words = r.source_words;
+    if (target_words) *target_words = r.target_words;
+    if (seconds) *seconds = r.seconds;
+  });
+}
+
+extern "C" int lnmt_integerize_file_decoding(const char *model_file, const char *source_file,
+                                             int max_sent_cutoff, int *ids, long long ids_cap,
+                                             int *lengths, int *lines, int max_sentences,
+                                             int *n_sentences, int *target_vocab_size) {
+  return Guard([&] {
+    InputFilePreprocess helper;
+    std::vector<std::vector<int>> sentences;
+    std::vector<int> kept;
+    const int v = helper.IntegerizeFileDecoding(model_file, source_file, max_sent_cutoff, &sentences, &kept);
+    if (target_vocab_size) *target_vocab_size = v;
+    if (n_sentences) *n_sentences = (int)sentences.size();
+    long long at = 0;
+    for (size_t i = 0; i < sentences.size() && (int)i < max_sentences; ++i) {
+      if (at + (long long)sentences[i].size() > ids_cap) throw LinmtError("lnmt_integerize_file_decoding: ids buffer too small");
+      std::copy(sentences[i].begin(), sentences[i].end(), ids + at);
+      at += (long long)sentences[i].size();
+      lengths[i] = (int)sentences[i].size();
+      if (lines) lines[i] = kept[i];
+    }
+  });
+}
+
+extern "C" int lnmt_unint_file(const char *model_file, const char *unint_file, const char *final_file,
+                               int sequence_to_sequence, int decoder_mode) {
+  return Guard([&] {
+    InputFilePreprocess helper;
+    helper.UnintFile(model_file, unint_file, final_file, sequence_to_sequence != 0, decoder_mode != 0);
+  });
 }

@@ -5,6 +5,7 @@
 #include <fstream>
 
 #include "file_helper.h"
+#include "input_file_preprocess.h"
 
 namespace linmt {
 
@@ -57,6 +58,117 @@ void NeuralMachineTranslation::DumpBestModel(const std::string &best_model_name,
       }
   }
   DumpWeights(best_model_name);
+}
+
+// One line of Decoder::OutputKBestHypotheses (src/decoder.h:602-681) for num_hypotheses = 1.
+static void WriteHypothesisLine(std::ostream &out, const SentenceResult &r, int source_length,
+                                const DecodingConfiguration &c) {
+  for (size_t j = 0; j < r.best.size(); ++j) out << (j ? " " : "") << r.best[j];
+  if (r.best_index >= 0 && c.print_decoding_information_mode_) {
+    const Hypothesis &h = r.hypotheses[r.best_index];
+    auto viterbi = [&](size_t j) { return h.viterbi.empty() ? -1 : h.viterbi[j]; };
+    const size_t size = h.tokens.size();
+    out << " |||| " << r.best_score << " ||||";
+    for (size_t j = 1; j + 1 < size; ++j) out << " " << viterbi(j);
+    if (size <= 2) out << " ";
+    out << " ||||";
+    int unk_number = 0;
+    for (size_t j = 1; j + 1 < size; ++j)
+      if (h.tokens[j] == 2) {
+        ++unk_number;
+        out << " " << viterbi(j);
+      }
+    if (0 == unk_number) out << " -1";
+    if (c.print_alignments_scores_mode_) {
+      out << " ||||";
+      for (size_t j = 1; j + 1 < size; ++j) {
+        out << " ";
+        for (int k = 0; k < source_length; ++k) {
+          if (k) out << "/";
+          out << (h.alignments_scores.empty() ? 0.f : h.alignments_scores[j][k]);
+        }
+      }
+      if (size <= 2) out << " ";
+    }
+  }
+  out << "\n";
+}
+
+DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
+  DecodingReport report;
+  const ModelInformation info = ReadModelInformation(c.model_name_);
+  GlobalConfiguration g;
+  g.num_layers_ = info.num_layers;
+  g.lstm_size_ = info.lstm_size;
+  g.embedding_size_ = info.lstm_size;
+  g.source_vocab_size_ = info.source_vocab_size;
+  g.target_vocab_size_ = info.target_vocab_size;
+  g.longest_sentence_ = c.longest_sentence_;
+  g.attention_mode_ = info.attention_model ? 1 : 0;
+  g.attention_width_ = c.attention_width_;
+  g.feed_input_mode_ = info.feed_input != 0;
+  g.sequence_to_sequence_mode_ = true;
+
+  InputFilePreprocess input_helper;
+  std::vector<std::vector<int>> sentences;
+  std::vector<int> kept;
+  input_helper.IntegerizeFileDecoding(c.model_name_, c.decode_user_file_, c.longest_sentence_, &sentences,
+                                      &kept);
+  {
+    std::ifstream count(c.decode_user_file_.c_str());
+    std::string line;
+    int lines = 0;
+    while (std::getline(count, line)) ++lines;
+    report.sentences_thrown_away = lines - (int)sentences.size();
+  }
+  report.sentences = (int)sentences.size();
+
+  int beam = c.beam_size_;
+  if (beam > (int)std::sqrt((double)g.target_vocab_size_)) beam = (int)std::sqrt((double)g.target_vocab_size_);
+  const int n_sent = std::max(1, std::min(c.sentences_per_batch_, (int)sentences.size()));
+  NeuralMachineTranslation neural(g);
+  neural.InitModelDecoding(n_sent, beam);
+  neural.LoadWeights(c.model_name_);
+
+  DecodeOptions o;
+  o.beam_size_ = c.beam_size_;
+  o.max_decoding_ratio_ = c.max_decoding_ratio_;
+  o.min_decoding_ratio_ = c.min_decoding_ratio_;
+  o.penalty_ = c.penalty_;
+  o.diversity_ = c.decoding_diversity_;
+  o.lp_alpha_ = c.decoding_lp_alpha_;
+  o.cp_beta_ = c.decoding_cp_beta_;
+  o.unk_replacement_mode_ = c.unk_replacement_mode_ && g.attention_mode_;
+
+  const std::string ids_file =
+      c.decoder_output_file_.empty() ? c.decoder_final_file_ + ".ids" : c.decoder_output_file_;
+  {
+    std::ofstream output(ids_file.c_str());
+    if (!output) throw LinmtError("Decoding: cannot open " + ids_file);
+    const auto begin = std::chrono::steady_clock::now();
+    for (size_t first = 0; first < sentences.size(); first += n_sent) {
+      // an empty source line cannot be encoded: it translates to an empty line
+      std::vector<std::vector<int>> batch;
+      std::vector<size_t> where;
+      const size_t last = std::min(sentences.size(), first + n_sent);
+      for (size_t i = first; i < last; ++i)
+        if (!sentences[i].empty()) {
+          batch.push_back(sentences[i]);
+          where.push_back(i - first);
+        }
+      std::vector<SentenceResult> results, ordered(last - first);
+      if (!batch.empty()) neural.DecodeBatch(batch, o, &results);
+      for (size_t b = 0; b < batch.size(); ++b) ordered[where[b]] = std::move(results[b]);
+      for (size_t i = first; i < last; ++i) {
+        WriteHypothesisLine(output, ordered[i - first], (int)sentences[i].size(), c);
+        report.source_words += (long long)sentences[i].size();
+        report.target_words += (long long)ordered[i - first].best.size();
+      }
+    }
+    report.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - begin).count();
+  }
+  input_helper.UnintFile(c.model_name_, ids_file, c.decoder_final_file_, true, true);
+  return report;
 }
 
 TuningReport Dispatcher::Tuning(NeuralMachineTranslation &neural, TuningConfiguration &configuration,

@@ -47,8 +47,39 @@ struct TuningReport {
   std::vector<TuningEvent> events;
 };
 
+// The fields of GlobalConfiguration that Decoding reads (src/global_configuration.h:228-262,298),
+// same names and defaults, plus the batch size of this implementation.
+struct DecodingConfiguration {
+  std::string model_name_;           // the reference's text model file
+  std::string decode_user_file_;     // source sentences, one per line, tokenised text
+  std::string decoder_output_file_;  // ids of the translations ("" = decoder_final_file_ + ".ids")
+  std::string decoder_final_file_;   // the translations as words
+  int beam_size_ = 12;
+  float penalty_ = 0.f, max_decoding_ratio_ = 1.5f, min_decoding_ratio_ = 0.5f;
+  float decoding_lp_alpha_ = 0.65f, decoding_cp_beta_ = 0.20f, decoding_diversity_ = 0.f;
+  int longest_sentence_ = 200;  // src/global_configuration.h:298: 100, doubled for translation
+  int attention_width_ = 10;    // D of the local-p window: not stored in the model file, the
+                                // reference takes it from its configuration too
+  bool print_decoding_information_mode_ = false;  // " |||| score |||| alignments |||| <UNK> alignments"
+  bool print_alignments_scores_mode_ = false;     // ... " |||| " alignment scores per token
+  bool unk_replacement_mode_ = false;             // export alignments (what the two prints show)
+  int sentences_per_batch_ = 64;  // no counterpart: the reference decodes one sentence at a time
+};
+
+struct DecodingReport {
+  int sentences = 0, sentences_thrown_away = 0;
+  long long source_words = 0, target_words = 0;
+  double seconds = 0.0;  // decoding only (model loading and file conversion excluded)
+};
+
 class Dispatcher {
  public:
+  // Dispatcher::Decoding (src/dispatcher.cu:387-436): model file -> decoder, source text -> ids
+  // (InputFilePreprocess::IntegerizeFileDecoding), beam search (EnsembleFactory::DecodeFile with
+  // one model), id output (Decoder::OutputKBestHypotheses, one hypothesis per sentence) -> words
+  // (UnintFile).
+  static DecodingReport Decoding(const DecodingConfiguration &configuration);
+
   // `neural` must have been created for training with cfg.minibatch_size_ columns.  `log`
   // (optional) receives every event as it happens.
   static TuningReport Tuning(NeuralMachineTranslation &neural, TuningConfiguration &configuration,

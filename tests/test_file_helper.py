@@ -95,3 +95,26 @@ def test_model_information():
                         attention_model=1, feed_input=1, multi_source=0, combine_lstm=0, char_cnn=0)
     with pytest.raises(host.HostError):
         host.read_model_information(os.path.join(GOLDEN, "no_such_model.nmt"))
+
+
+def test_integerize_source_text_and_unintegerize_output(tmp_path):
+    """IntegerizeFileDecoding / UnintFile (src/input_file_preprocess.cc:1312-1581) with the
+    vocabularies of tests/golden/tiny_model.nmt (source: <UNK> s1..s4; target: <START> <EOF> <UNK>
+    t3..t5).  Expected values written out by hand from the rules: text before " |||| ", unknown
+    words -> <UNK> (id 0), a sentence with length + 1 >= cutoff - 2 is dropped, ids up to the first
+    "||||" become words, separator lines and the rest of a line are copied."""
+    from linmt_amd import host
+    model = os.path.join(GOLDEN, "tiny_model.nmt")
+    src = tmp_path / "src.txt"
+    src.write_text("s1 s2 s3\ns4 nope s1 |||| ignored tail\n\ns2 s2 s2 s2 s2 s2 s2 s2 s2\n  s3  \n")
+    sents, lines, vt = host.integerize_file_decoding(model, str(src), 12)
+    assert [x.tolist() for x in sents] == [[1, 2, 3], [4, 0, 1], [], [3]]
+    assert lines == [0, 1, 2, 4] and vt == 6   # the nine-word line is thrown away (9 + 1 >= 10)
+    ids = tmp_path / "out.ids"
+    ids.write_text("3 4 5\n2 |||| -1.5 |||| 0 |||| 0\n\n================\n5 ||||\n1 0\n")
+    final = tmp_path / "final.txt"
+    host.unint_file(model, str(ids), str(final))
+    assert final.read_text() == ("t3 t4 t5\n<UNK> |||| -1.5 |||| 0 |||| 0\n\n================\n"
+                                 "t5 |||| \n<EOF> <START>\n")
+    with pytest.raises(host.HostError):
+        host.integerize_file_decoding(os.path.join(GOLDEN, "nope.nmt"), str(src), 12)

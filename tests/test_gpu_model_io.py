@@ -78,3 +78,59 @@ def test_dump_then_load_round_trip(host, tmp_path, layers, attention, feed, s2s)
     c = host.Model(layers + 1, H, Vs, Vt, **kw)
     with pytest.raises(host.HostError):
         c.load_weights(path)
+
+
+def test_decoding_a_text_file(host, tmp_path):
+    """Dispatcher::Decoding end to end: model file + source text -> ids file -> words, in batches,
+    with the decoding-information fields; the ids and alignments must be the ones DecodeBatch gives
+    for the same sentences on a model loaded from the same file."""
+    rng = np.random.default_rng(8)
+    layers, H, Vs, Vt, D, beam = 2, 24, 30, 40, 2, 4
+    P = R.make_params(rng, layers, H, Vs, Vt, attention=True, feed_input=True, scale=0.5)
+    kw = dict(longest_sentence=24, attention_mode=1, attention_width=D, feed_input=True)
+    a = host.Model(layers, H, Vs, Vt, minibatch_size=1, **kw)
+    a.set_params(P)
+    model = str(tmp_path / "model.nmt")
+    a.dump_model(model)  # placeholder vocabularies: source <UNK> w1.., target <START> <EOF> <UNK> w3..
+
+    lens = [5, 1, 9, 3, 7, 2, 6]
+    sents = [rng.integers(0, Vs, size=n) for n in lens]
+    word = lambda i: "<UNK>" if i == 0 else f"w{i}"  # noqa: E731
+    lines = [" ".join(word(i) for i in s_) for s_ in sents]
+    lines[3] = lines[3].replace(word(sents[3][1]), "never-seen")  # an out-of-vocabulary word
+    sents[3][1] = 0
+    lines.insert(2, "")                                            # an empty line
+    lines.insert(5, " ".join(["w1"] * 30))                         # too long: thrown away
+    src = tmp_path / "src.txt"
+    src.write_text("\n".join(lines) + "\n")
+    final, ids = str(tmp_path / "out.txt"), str(tmp_path / "out.ids")
+    rep = host.decoding(model, str(src), final, ids_file=ids, beam=beam, longest_sentence=24,
+                        attention_width=D, print_decoding_information=True, unk_replacement_mode=True,
+                        sentences_per_batch=3)
+    assert rep["sentences"] == len(lens) + 1 and rep["sentences_thrown_away"] == 1
+    assert rep["source_words"] == sum(lens)
+
+    # the same groups the driver forms (three kept lines at a time, the empty one not decoded), so
+    # that every product has the same shape and the comparison can be exact
+    b = host.Model(layers, H, Vs, Vt, decoding=(3, beam), **kw)
+    b.load_weights(model)
+    want = []
+    for group in (sents[0:2], sents[2:5], sents[5:7]):
+        want += b.decode_batch(group, beam=beam, alignments=True)
+    got_ids = open(ids).read().split("\n")[:-1]
+    got_txt = open(final).read().split("\n")[:-1]
+    assert len(got_ids) == len(lens) + 1 and got_ids[2] == "" and got_txt[2] == ""
+    del got_ids[2], got_txt[2]
+    tword = lambda i: ["<START>", "<EOF>", "<UNK>"][i] if i < 3 else f"w{i}"  # noqa: E731
+    for k, (line, text, w) in enumerate(zip(got_ids, got_txt, want)):
+        fields = line.split(" |||| ")
+        assert len(fields) == 4, line
+        toks = [int(x) for x in fields[0].split()]
+        assert toks == w["best"].tolist(), k
+        assert np.isclose(float(fields[1]), w["best_score"], rtol=1e-4, atol=1e-5)
+        assert [int(x) for x in fields[2].split()] == w["best_viterbi"].tolist(), k
+        unk = [v for t, v in zip(toks, w["best_viterbi"].tolist()) if t == 2]
+        assert [int(x) for x in fields[3].split()] == (unk if unk else [-1]), k
+        assert text.split(" |||| ")[0].split() == [tword(t) for t in toks]
+        assert text.split(" |||| ")[1:] == fields[1:]
+    assert rep["target_words"] == sum(len(w["best"]) for w in want)
