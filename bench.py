@@ -254,7 +254,8 @@ def main():
                     help="sentences of the same workload decoded by the CPU oracle for cpu_baseline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-level", type=int, default=1,
-                    help="1: HIP events around the matrix products during the timed steps; "
+                    help="1: HIP events around the output projection (the dominant kernel) during "
+                         "the timed steps; "
                          "2: one extra untimed pass with every launch bracketed (kernel table)")
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the decode benchmark, time the fused HBM-bound kernels alone "

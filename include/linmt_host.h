@@ -117,9 +117,9 @@ int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int *lengths, i
 /* The model's HIP stream (hipStream_t as void*), for callers that time with HIP events. */
 void *lnmt_model_stream(lnmt_model *m);
 
-/* Live kernel timing with HIP events on the model's stream.  level 0 = off, 1 = the matrix products,
- * 2 = every launch of the path.  Totals accumulate over lnmt_decode_batch / lnmt_get_error calls
- * until the level is set again.  Entries are keyed "<call site>" or, for matrix products,
+/* Live kernel timing with HIP events on the model's stream.  level 0 = off, 1 = the output
+ * projection (the dominant matrix product), 2 = every launch of the path.  Totals accumulate
+ * over lnmt_decode_batch / lnmt_get_error calls until the level is set again.  Entries are keyed "<call site>" or, for matrix products,
  * "<call site>|<kernel instance>"; work = algorithmic flop (matrix products) or bytes (others). */
 int lnmt_profile_set_level(lnmt_model *m, int level);
 int lnmt_profile_count(lnmt_model *m);

@@ -152,6 +152,7 @@ class LstmLayer {
   bool input_hoisted_ = false;    // this pass uses them
   bool mw_fold_dirty_ = true;
   void ForwardPropInputAllSteps(int steps);
+  void ForwardPropInputSteps(int first, int steps);
   void BuildEmbeddingFold();
   DeviceArray<float> p_device_h_t_previous_, p_device_c_t_previous_;  // decode: PreviousTargetState
   DeviceArray<int> p_device_input_vocab_indices_full_, p_device_input_vocab_indices_01_full_;
@@ -393,6 +394,16 @@ class NeuralMachineTranslation {
   // stream_, which is the ordering that sharing it requires.
   static constexpr size_t kGemmWorkspaceBytes = size_t(64) << 20;
   DeviceArray<char> gemm_workspace_;
+  // the part of it the products launched right now may use (all of it on the single stream; one
+  // slice per layer while the encoder's layers run side by side)
+  char *gemm_ws_ptr_ = nullptr;
+  size_t gemm_ws_bytes_ = 0;
+  // Encoder of a decoding batch: layer l+1 can start on a block of timesteps as soon as layer l
+  // has finished it, so every layer gets a stream of its own (layer 0: stream_) and the L
+  // recurrences overlap instead of queueing 2*L*S small launches behind each other.
+  std::vector<hipStream_t> lane_streams_;
+  std::vector<hipEvent_t> lane_events_;
+  static constexpr int kLaneChunkSteps = 8;
   // Every dense product of the model: profiling key, workspace, error text.
   void Gemm(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg, int trans_a, int trans_x,
             float beta, const float *bias, int act, const int *colmask, float *C, int ldc,
@@ -491,6 +502,7 @@ class NeuralMachineTranslation {
   // encoder + decoder + attention of a teacher-forced minibatch (shared by GetError and
   // ComputeGradients); per_step_loss: also run the loss of every step as GetError does.
   void RunSourceSide(int source_length, int minibatch_size);
+  void RunSourceSideLanes(int source_length, int minibatch_size);
   void ForwardTeacherForced(const int *p_host_source, int source_length,
                             const int *p_host_target_in, const int *p_host_target_out,
                             int target_length, const int *p_host_batch_information,

@@ -295,6 +295,17 @@ void LstmLayer::ForwardPropInputAllSteps(int steps) {
          4 * H, "LstmLayer input products, all steps");
 }
 
+// The same for the timesteps [first, first + steps) of a layer above the input layer.
+void LstmLayer::ForwardPropInputSteps(int first, int steps) {
+  NeuralMachineTranslation &M = *p_neural_mt_;
+  if (input_layer_mode_) throw LinmtError("ForwardPropInputSteps: not for the input layer");
+  const int H = lstm_size_, N = minibatch_size_ * steps;
+  lh_gemm_seg seg{p_device_m_stack_.get(), 4 * H, v_nodes_[first].p_device_h_t_below_, input_size_,
+                  input_size_};
+  M.Gemm(kTagGateGemm, 4 * H, N, &seg, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
+         v_nodes_[first].p_device_pre_x_, 4 * H, "LstmLayer input products, a block of steps");
+}
+
 // mw_fold_ = M_stack * W (4H x V): the input product of every vocabulary entry, for decoding.
 void LstmLayer::BuildEmbeddingFold() {
   NeuralMachineTranslation &M = *p_neural_mt_;

@@ -4,6 +4,8 @@
 #include <cstring>
 #include <numeric>
 
+#include <cstdlib>
+
 #include "nmt.h"
 
 namespace linmt {
@@ -13,21 +15,29 @@ NeuralMachineTranslation::NeuralMachineTranslation(const GlobalConfiguration &cf
   HipErrorWrapper(hipStreamCreate(&stream_), "stream creation failed");
   profiler_.stream_ = stream_;
   gemm_workspace_.Alloc(kGemmWorkspaceBytes);
+  gemm_ws_ptr_ = gemm_workspace_.get();
+  gemm_ws_bytes_ = gemm_workspace_.size();
 }
 
 void NeuralMachineTranslation::Gemm(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg,
                                     int trans_a, int trans_x, float beta, const float *bias, int act,
                                     const int *colmask, float *C, int ldc, const char *what,
                                     int act_rows) {
-  ProfileScope ps(profiler_, tag, gemm_workspace_.size(), 0, rows, cols, segs, nseg, trans_a, trans_x);
+  ProfileScope ps(profiler_, tag, gemm_ws_bytes_, 0, rows, cols, segs, nseg, trans_a, trans_x);
   LhErrorWrapper(lh_gemm_ws_f32(rows, cols, segs, nseg, trans_a, trans_x, 1.f, beta, bias, act,
                                 act_rows < 0 ? rows : act_rows,
-                                colmask, C, ldc, gemm_workspace_.get(), gemm_workspace_.size(),
+                                colmask, C, ldc, gemm_ws_ptr_, gemm_ws_bytes_,
                                 stream_),
                  what);
 }
 
 NeuralMachineTranslation::~NeuralMachineTranslation() {
+  if (stream_) (void)hipStreamSynchronize(stream_);
+  for (hipEvent_t e : lane_events_) (void)hipEventDestroy(e);
+  for (size_t l = 1; l < lane_streams_.size(); ++l) {  // lane 0 is stream_
+    (void)hipStreamSynchronize(lane_streams_[l]);
+    (void)hipStreamDestroy(lane_streams_[l]);
+  }
   if (stream_) {
     (void)hipStreamSynchronize(stream_);
     (void)hipStreamDestroy(stream_);
@@ -139,15 +149,15 @@ int NeuralMachineTranslation::GemmAddends(int tag, int rows, int cols, const lh_
   // planes can only replace C when they have C's leading dimension
   const bool can_split = ldc == rows && rows % 4 == 0;
   const int max_planes = !can_split ? 1 : (beta == 0.f ? 3 : 2);
-  ProfileScope ps(profiler_, tag, gemm_workspace_.size(), max_planes, rows, cols, segs, nseg, 0, 0);
+  ProfileScope ps(profiler_, tag, gemm_ws_bytes_, max_planes, rows, cols, segs, nseg, 0, 0);
   int planes = 1;
-  LhErrorWrapper(lh_gemm_planes_f32(rows, cols, segs, nseg, 0, 0, beta, C, ldc, gemm_workspace_.get(),
-                                    gemm_workspace_.size(), max_planes, &planes, stream_),
+  LhErrorWrapper(lh_gemm_planes_f32(rows, cols, segs, nseg, 0, 0, beta, C, ldc, gemm_ws_ptr_,
+                                    gemm_ws_bytes_, max_planes, &planes, stream_),
                  what);
   int n = 0;
   if (planes == 1 || beta != 0.f) addend[n++] = C;
   if (planes > 1) {
-    const float *ws = reinterpret_cast<const float *>(gemm_workspace_.get());
+    const float *ws = reinterpret_cast<const float *>(gemm_ws_ptr_);
     for (int p = 0; p < planes; ++p) addend[n++] = ws + (size_t)p * rows * cols;
   }
   for (int i = n; i < 3; ++i) addend[i] = nullptr;
@@ -294,6 +304,79 @@ void NeuralMachineTranslation::ForwardTeacherForced(const int *p_host_source, in
 // Encoder for n_sent sentences at once; ids are n_sent x source_length column-major, reversed and
 // left-padded with -1, so that every sentence ends at the last step and padded prefixes keep the
 // state at exactly zero (deep_rnn.h:1572-1646 runs one sentence with B = 1).
+// Layer l on lane l.  The work is issued layer by layer (so every event is recorded before the
+// wait that names it is issued); on the GPU layer l+1 follows layer l one block of timesteps behind.
+void NeuralMachineTranslation::RunSourceSideLanes(int source_length, int B) {
+  const int L = cfg_.num_layers_, C = kLaneChunkSteps;
+  const int chunks = (source_length + C - 1) / C;
+  if (lane_streams_.empty()) {
+    lane_streams_.assign(L, stream_);
+    for (int l = 1; l < L; ++l)
+      HipErrorWrapper(hipStreamCreate(&lane_streams_[l]), "encoder lane stream creation failed");
+  }
+  while (lane_events_.size() < (size_t)L * (chunks + 1) + 1) {
+    hipEvent_t e;
+    HipErrorWrapper(hipEventCreateWithFlags(&e, hipEventDisableTiming), "encoder lane event creation failed");
+    lane_events_.push_back(e);
+  }
+  auto event = [&](int l, int c) { return lane_events_[1 + (size_t)l * (chunks + 1) + c]; };
+
+  // everything queued so far (index upload, the previous batch) precedes every lane
+  HipErrorWrapper(hipEventRecord(lane_events_[0], stream_), "encoder lane fork failed");
+  for (int l = 1; l < L; ++l)
+    HipErrorWrapper(hipStreamWaitEvent(lane_streams_[l], lane_events_[0], 0), "encoder lane fork failed");
+
+  hipStream_t const main_stream = stream_;
+  char *const ws = gemm_workspace_.get();
+  const size_t ws_slice = (gemm_workspace_.size() / L) & ~size_t(255);
+  struct Restore {
+    NeuralMachineTranslation &m;
+    hipStream_t s;
+    ~Restore() {
+      m.stream_ = s;
+      m.profiler_.stream_ = s;
+      m.gemm_ws_ptr_ = m.gemm_workspace_.get();
+      m.gemm_ws_bytes_ = m.gemm_workspace_.size();
+    }
+  } restore{*this, main_stream};
+
+  for (int l = 0; l < L; ++l) {
+    LstmLayer &Ls = SourceLayer(l);
+    stream_ = lane_streams_[l];
+    profiler_.stream_ = stream_;
+    gemm_ws_ptr_ = ws + ws_slice * l;
+    gemm_ws_bytes_ = ws_slice;
+    for (int t = 0; t < source_length; ++t) {
+      const size_t step = (size_t)t * B;
+      LstmNode &n = Ls.v_nodes_[t];
+      n.minibatch_size_ = B;
+      float *hp = t == 0 ? Ls.p_device_init_hidden_vec_.get() : Ls.v_nodes_[t - 1].p_device_h_t_;
+      float *cp = t == 0 ? Ls.p_device_init_cell_vec_.get() : Ls.v_nodes_[t - 1].p_device_c_t_;
+      if (l == 0) {
+        n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_full_.get() + step,
+                                  Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+      } else {
+        n.UpdateVectorsForwardGpu(Ls.p_device_input_vocab_indices_01_full_.get() + step, hp, cp);
+        n.p_device_h_t_below_ = UpwardState(SourceLayer(l - 1), t);
+      }
+    }
+    Ls.input_hoisted_ = true;
+    if (l == 0) Ls.ForwardPropInputAllSteps(source_length);  // embeddings: no layer below to wait for
+    for (int c = 0; c < chunks; ++c) {
+      const int t0 = c * C, nt = std::min(C, source_length - t0);
+      if (l > 0) {
+        HipErrorWrapper(hipStreamWaitEvent(stream_, event(l - 1, c), 0), "encoder lane wait failed");
+        Ls.ForwardPropInputSteps(t0, nt);
+      }
+      for (int t = t0; t < t0 + nt; ++t) Ls.v_nodes_[t].ForwardProp();
+      HipErrorWrapper(hipEventRecord(event(l, c), stream_), "encoder lane record failed");
+    }
+  }
+  // join: the caller's stream continues after the last block of every layer
+  for (int l = 1; l < L; ++l)
+    HipErrorWrapper(hipStreamWaitEvent(main_stream, event(l, chunks - 1), 0), "encoder lane join failed");
+}
+
 void NeuralMachineTranslation::ForwardPropSource(const int *p_host_source, int source_length,
                                                  int n_sent) {
   const int L = cfg_.num_layers_;
@@ -305,6 +388,15 @@ void NeuralMachineTranslation::ForwardPropSource(const int *p_host_source, int s
 // one layer at a time: the layer's input products for all steps in one GEMM, then the recurrence.
 void NeuralMachineTranslation::RunSourceSide(int source_length, int B) {
   const int L = cfg_.num_layers_;
+  static const bool lanes_off = getenv("LINMT_NO_LANES") != nullptr;  // measurement aid
+  bool lanes = !lanes_off && decode_mode_ && L > 1 && L <= 4 && profiler_.level_ < 2 &&
+               source_length > kLaneChunkSteps;
+  for (int l = 0; l < L && lanes; ++l)
+    lanes = SourceLayer(l).input_hoistable_ && B == SourceLayer(l).minibatch_size_;
+  if (lanes) {
+    RunSourceSideLanes(source_length, B);
+    return;
+  }
   for (int l = 0; l < L; ++l) {
     LstmLayer &Ls = SourceLayer(l);
     for (int t = 0; t < source_length; ++t) {
