@@ -579,13 +579,18 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
     sx.store(sb + kAF, tid);  \
   } while (0)
 
+  // Software pipeline, two slabs deep: LDS holds slab s (being consumed) and slab s+1, the
+  // staging registers hold slab s+2 in flight.  A slab goes to LDS at the START of the iteration
+  // before it is consumed -- its buffer was released by the barrier that ended the previous
+  // iteration -- so neither the global loads nor the LDS stores sit between two slabs of MFMAs.
   LH_ISSUE();
   LH_STASH(smem);
+  if (total > 1) LH_ISSUE();
   __syncthreads();
   int cur = 0;  // float offset of the slab buffer being consumed
   for (int s = 0; s < total; ++s) {
-    const bool has_next = s + 1 < total;
-    if (has_next) LH_ISSUE();
+    if (s + 1 < total) LH_STASH(smem + (kSlab - cur));
+    if (s + 2 < total) LH_ISSUE();
     {
       const float *as = smem + cur + fa_off;
       const float *xs = smem + cur + fx_off;
@@ -615,7 +620,6 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
                                                                acc[a][b], 0, 0, 0);
       }
     }
-    if (has_next) LH_STASH(smem + (kSlab - cur));
     __syncthreads();
     cur = kSlab - cur;
   }
