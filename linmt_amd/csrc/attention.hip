@@ -170,6 +170,157 @@ __global__ __launch_bounds__(kThreads) void attn_core_kernel(const AttnArgs a) {
   }
 }
 
+// The same computation for windows of at most WCAP slots (local-p with D <= 10) and 16-byte
+// aligned operands: the whole W x H window of the column is read ONCE, straight into registers
+// (thread t holds rows 4t..4t+3 -- and 4(t+256).. when H > 1024 -- of every slot, all loads in
+// flight together), the scores are block-reduced from per-thread partial dot products, and the
+// context vector is accumulated from the same registers.
+template <int NQ, int WCAP>
+__global__ __launch_bounds__(kThreads) void attn_core_regs_kernel(const AttnArgs a) {
+  __shared__ float s_part[kWaves][WCAP];
+  __shared__ float s_val[WCAP];
+  __shared__ int s_tau[WCAP];
+  __shared__ int s_idx[WCAP];
+  __shared__ float s_red[kWaves];
+
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x, wave = tid / lh::kWave, lane = tid % lh::kWave;
+  const int H = a.H, B = a.B, W = a.W, D = a.D;
+  const int len = a.batch_info[b];
+  const int off = a.batch_info[B + b];
+  const int m = a.mask01[b];
+  const int col = a.hs_col ? a.hs_col[b] : b;
+  const float *wa = a.wa + (size_t)b * a.proj_col_stride;
+  const float *hs_c = a.hs + (size_t)col * a.col_stride;
+
+  float p = 0.f;
+  int lo = 0, hi = len - 1;
+  if (D >= 0) {
+    float part = 0.f;
+    const float *t1 = a.tanh1 + (size_t)b * a.proj_col_stride;
+    for (int r = tid; r < H; r += kThreads) part += a.v_p[r] * t1[r];
+    const float dot = lh::block_sum<kWaves>(part, s_red);
+    const float sig = (float)(1.0 / (1.0 + exp(-1.0 * (double)dot)));
+    p = (float)len * sig;
+    lo = (0 > (int)p - D) ? 0 : ((int)p - D);
+    hi = ((len - 1) < (int)p + D) ? (len - 1) : ((int)p + D);
+    if (tid == 0) {
+      a.p_t[b] = p;
+      a.sigma[b] = sig;
+    }
+  }
+  for (int j = tid; j < WCAP; j += kThreads) {
+    int idx = -1, tau = -1;
+    if (j < W) {
+      if (m == 1 && lo + j <= hi) idx = lo + j;
+      a.indices[b + (size_t)B * j] = idx;
+      if (idx >= 0) {
+        tau = len - 1 - idx + off;
+        if (tau < 0 || tau >= a.hs_steps) tau = -1;
+      }
+    }
+    s_idx[j] = idx;
+    s_tau[j] = tau;
+  }
+  __syncthreads();
+
+  // the window, once
+  float4 h[WCAP][NQ];
+  float4 w4[NQ];
+  bool row_ok[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    const int r = (tid + q * kThreads) * 4;
+    row_ok[q] = r < H;
+    w4[q] = row_ok[q] ? *reinterpret_cast<const float4 *>(wa + r) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+#pragma unroll
+  for (int j = 0; j < WCAP; ++j) {
+    const int tau = s_tau[j];  // the same for every thread: a scalar branch
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      h[j][q] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (tau >= 0 && row_ok[q])
+        h[j][q] = *reinterpret_cast<const float4 *>(hs_c + (size_t)tau * a.step_stride +
+                                                    (size_t)(tid + q * kThreads) * 4);
+    }
+  }
+  // scores: per-thread partial dot products, wavefront sums, then the four wavefronts in order
+#pragma unroll
+  for (int j = 0; j < WCAP; ++j) {
+    float sc = 0.f;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q)
+      sc += h[j][q].x * w4[q].x + h[j][q].y * w4[q].y + h[j][q].z * w4[q].z + h[j][q].w * w4[q].w;
+    sc = lh::wave_sum(sc);
+    if (lane == 0) s_part[wave][j] = sc;
+  }
+  __syncthreads();
+  for (int j = tid; j < WCAP; j += kThreads) {
+    float sc = s_part[0][j];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) sc += s_part[w][j];
+    s_val[j] = s_tau[j] >= 0 ? sc : 0.f;
+  }
+  __syncthreads();
+
+  float mx = D >= 0 ? 0.f : -FLT_MAX;
+  for (int j = 0; j < W; ++j) {
+    if (s_idx[j] != -1 && s_val[j] > mx) mx = s_val[j];
+  }
+  float Z = 0.f;
+  for (int j = 0; j < W; ++j) {
+    if (s_idx[j] != -1) Z += expf(s_val[j] - mx);
+  }
+  __syncthreads();
+  const float sigma_sq = (float)((D * D) / 4.0);
+  for (int j = tid; j < WCAP; j += kThreads) {
+    float al = 0.f, g = 1.f;
+    if (j < W) {
+      const int idx = s_idx[j];
+      if (idx != -1) {
+        const float e = expf(s_val[j] - mx);
+        if (D >= 0) {
+          const float dlt = p - (float)idx;
+          g = expf((-1.f * (dlt * dlt)) / (2.f * sigma_sq));
+        }
+        al = (Z != 0.f) ? (e / Z) * g : e;
+      }
+      a.align[b + (size_t)B * j] = al;
+      a.cached_exp[j + (size_t)W * b] = g;
+    }
+    s_val[j] = al;
+  }
+  __syncthreads();
+
+  if (a.viterbi && tid == 0) {
+    float best = -1.f;
+    int best_idx = -1;
+    for (int j = 0; j < W; ++j) {
+      if (best < s_val[j]) {
+        best = s_val[j];
+        best_idx = s_idx[j];
+      }
+    }
+    a.viterbi[b] = best_idx;
+  }
+
+  float *ctx = a.ctx + (size_t)b * H;
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int j = 0; j < WCAP; ++j) {
+      if (s_tau[j] < 0) continue;  // the general kernel skips these slots too
+      const float w = s_val[j];
+      acc.x += w * h[j][q].x; acc.y += w * h[j][q].y; acc.z += w * h[j][q].z; acc.w += w * h[j][q].w;
+    }
+    if (row_ok[q]) *reinterpret_cast<float4 *>(ctx + (size_t)(tid + q * kThreads) * 4) = acc;
+  }
+}
+
+constexpr int kRegsSlots = 21;  // the reference's default window: D = 10
+
 }  // namespace
 
 extern "C" int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_steps,
@@ -200,7 +351,11 @@ extern "C" int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_ste
   const bool vec = H % 4 == 0 && lh::aligned16(wa) && lh::aligned16(hs) && lh::aligned16(ctx) &&
                    hs_step_stride % 4 == 0 && hs_col_stride % 4 == 0 && proj_col_stride % 4 == 0;
   hipStream_t st = lh::as_stream(stream);
-  if (vec) hipLaunchKernelGGL(attn_core_kernel<true>, dim3(B), dim3(kThreads), 0, st, a);
+  if (vec && W <= kRegsSlots && H <= 4 * kThreads)
+    hipLaunchKernelGGL((attn_core_regs_kernel<1, kRegsSlots>), dim3(B), dim3(kThreads), 0, st, a);
+  else if (vec && W <= kRegsSlots && H <= 8 * kThreads)
+    hipLaunchKernelGGL((attn_core_regs_kernel<2, kRegsSlots>), dim3(B), dim3(kThreads), 0, st, a);
+  else if (vec) hipLaunchKernelGGL(attn_core_kernel<true>, dim3(B), dim3(kThreads), 0, st, a);
   else hipLaunchKernelGGL(attn_core_kernel<false>, dim3(B), dim3(kThreads), 0, st, a);
   return lh::check_launch("lh_attn_core_fwd_f32");
 }

@@ -314,7 +314,11 @@ def _run_attn(lh, H, B, D, max_len, S, tanh1, v_p, wa, hs, step, colstride, hs_c
 
 
 @pytest.mark.parametrize("H,B,S,D", [(1000, 64, 100, 10), (256, 32, 30, 10), (1000, 128, 50, 3),
-                                     (12, 5, 9, 2)])
+                                     (12, 5, 9, 2),
+                                     (2000, 16, 40, 10),   # two row quads per thread
+                                     (1000, 16, 60, 12),   # window wider than the register path holds
+                                     (1002, 8, 30, 10),    # rows not a multiple of four
+                                     (4100, 4, 30, 10)])   # more rows than the register path holds
 def test_attn_core_local_p(lh, orc, H, B, S, D):
     rng = np.random.default_rng(5)
     lens = rng.integers(1, S + 1, size=B).astype(np.int32)
