@@ -13,6 +13,8 @@
 #ifndef LINMT_HOST_H_
 #define LINMT_HOST_H_
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -226,6 +228,37 @@ int lnmt_integerize_file_decoding(const char *model_file, const char *source_fil
                                   int *target_vocab_size);
 int lnmt_unint_file(const char *model_file, const char *unint_file, const char *final_file,
                     int sequence_to_sequence, int decoder_mode);
+
+/* ---- one sentence at a time: the decoder of the translation service ---------------------------
+ * DecoderSentence (src/decoder_sentence.h:22-52, src/decoder_sentence.cu:14-391).  create reads a
+ * configuration file of lines `param="--key" value="..."` (keys: --nmt-model (required, one
+ * file), --beam-size, --longest-sent, --attention-width, --decoding-ratio "min max", --lp-alpha,
+ * --cp-beta, --diversity, --print-decoding-info, --print-align-scores, --nbest (1), --multi-gpu),
+ * the vocabularies and, with load_model != 0, the weights (GPU).  NULL on error.  process
+ * translates one tokenised sentence (text after " |||| " is ignored): words of the best
+ * hypothesis, then with --print-decoding-info " |||| score |||| alignments |||| <UNK> alignments".
+ * *needed receives the size of the text including its terminator; a buffer that is too small is
+ * an error.  integerize / unint are the two text conversions alone (host only; integerize returns
+ * the ids reversed, the order the reference's encoder reads them in).  settings reports what
+ * create read (file names in *o are NULL; the model file goes to model_file). */
+typedef struct lnmt_decoder_sentence lnmt_decoder_sentence;
+lnmt_decoder_sentence *lnmt_decoder_sentence_create(const char *config_file, int load_model);
+void lnmt_decoder_sentence_destroy(lnmt_decoder_sentence *d);
+int lnmt_decoder_sentence_process(lnmt_decoder_sentence *d, const char *sentence, char *out,
+                                  size_t cap, size_t *needed);
+int lnmt_decoder_sentence_integerize(lnmt_decoder_sentence *d, const char *sentence, int *ids,
+                                     int cap, int *n);
+int lnmt_decoder_sentence_unint(lnmt_decoder_sentence *d, const char *sentence, char *out,
+                                size_t cap, size_t *needed);
+int lnmt_decoder_sentence_settings(lnmt_decoder_sentence *d, lnmt_decoding_options *o,
+                                   char *model_file, size_t cap);
+
+/* The C interface the reference's Python server binds (src/decoder_sentence.h:94-97,
+ * src/decoder_sentence.cu:844-874), same names and behaviour: one decoder per process, msg is the
+ * path of the configuration file, the returned text belongs to the library until the next call,
+ * "" for an empty sentence, an error prints a message and ends the process.  Not re-entrant. */
+void python_decoder_init(char *msg);
+char *python_decoder_do_job(char *sentence);
 
 #ifdef __cplusplus
 }

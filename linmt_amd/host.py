@@ -72,6 +72,9 @@ def load():
     if not os.path.exists(LIB_PATH):
         raise HostError(f"{LIB_PATH} is missing: build it with __graft_entry__.build(); "
                         "there is no CPU fallback")
+    # torch brings a HIP runtime of its own: whichever runtime a process loads first has to be the
+    # one that initialises the device, so torch goes first wherever both end up in one process
+    import torch  # noqa: F401
     lib = C.CDLL(LIB_PATH)
     lib.lnmt_last_error.restype = C.c_char_p
     lib.lnmt_model_create_scoring.restype = C.c_void_p
@@ -130,6 +133,21 @@ def load():
                                 C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_longlong),
                                 C.POINTER(C.c_double), C.POINTER(C.c_float)]
     lib.lnmt_get_perplexity.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_double)]
+    lib.lnmt_decoder_sentence_create.restype = C.c_void_p
+    lib.lnmt_decoder_sentence_create.argtypes = [C.c_char_p, C.c_int]
+    lib.lnmt_decoder_sentence_destroy.restype = None
+    lib.lnmt_decoder_sentence_destroy.argtypes = [C.c_void_p]
+    lib.lnmt_decoder_sentence_process.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t,
+                                                  C.POINTER(C.c_size_t)]
+    lib.lnmt_decoder_sentence_unint.argtypes = lib.lnmt_decoder_sentence_process.argtypes
+    lib.lnmt_decoder_sentence_integerize.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int,
+                                                     C.POINTER(C.c_int)]
+    lib.lnmt_decoder_sentence_settings.argtypes = [C.c_void_p, C.POINTER(DecodingOptions),
+                                                   C.c_char_p, C.c_size_t]
+    lib.python_decoder_init.restype = None
+    lib.python_decoder_init.argtypes = [C.c_char_p]
+    lib.python_decoder_do_job.restype = C.c_char_p
+    lib.python_decoder_do_job.argtypes = [C.c_char_p]
     _lib = lib
     return lib
 
@@ -402,6 +420,68 @@ def unint_file(model_file, unint_path, final_path, sequence_to_sequence=True, de
     _check(load().lnmt_unint_file(os.fsencode(model_file), os.fsencode(unint_path),
                                   os.fsencode(final_path), int(sequence_to_sequence),
                                   int(decoder_mode)), "unint_file")
+
+
+class DecoderSentence:
+    """The reference's one-sentence decoder (DecoderSentence, src/decoder_sentence.h:22-52):
+    configuration file -> model; process(sentence) -> translation text.  load_model=False reads
+    the configuration and the vocabularies only (no GPU): integerize / unint / settings work."""
+
+    def __init__(self, config_file, load_model=True):
+        self._h = load().lnmt_decoder_sentence_create(os.fsencode(config_file), int(load_model))
+        if not self._h:
+            raise HostError("DecoderSentence: " + load().lnmt_last_error().decode("utf-8", "replace"))
+
+    def close(self):
+        if self._h:
+            load().lnmt_decoder_sentence_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def _text(self, fn, sentence, what):
+        cap = 1 << 16
+        while True:
+            buf, need = C.create_string_buffer(cap), C.c_size_t(0)
+            rc = fn(self._h, sentence.encode("utf-8"), buf, cap, C.byref(need))
+            if rc != 0 and need.value > cap:
+                cap = need.value
+                continue
+            _check(rc, what)
+            return buf.value.decode("utf-8", "replace")
+
+    def process(self, sentence):
+        return self._text(load().lnmt_decoder_sentence_process, sentence, "DecoderSentence.process")
+
+    def unint(self, sentence):
+        return self._text(load().lnmt_decoder_sentence_unint, sentence, "DecoderSentence.unint")
+
+    def integerize(self, sentence):
+        """ids in the order the encoder reads them (reversed)."""
+        cap = max(16, len(sentence))
+        ids, n = np.empty(cap, np.int32), C.c_int(0)
+        _check(load().lnmt_decoder_sentence_integerize(self._h, sentence.encode("utf-8"), _p(ids), cap,
+                                                       C.byref(n)), "DecoderSentence.integerize")
+        return ids[:n.value].copy()
+
+    def settings(self):
+        o, name = DecodingOptions(), C.create_string_buffer(4096)
+        _check(load().lnmt_decoder_sentence_settings(self._h, C.byref(o), name, 4096),
+               "DecoderSentence.settings")
+        out = {f: getattr(o, f) for f, _ in DecodingOptions._fields_
+               if f not in ("model_file", "source_file", "ids_file", "final_file")}
+        out["model_file"] = os.fsdecode(name.value)
+        return out
+
+
+def python_decoder_init(config_file):
+    """python_decoder_init of the reference's server library (src/decoder_sentence.cu:847-850)."""
+    load().python_decoder_init(os.fsencode(config_file))
+
+
+def python_decoder_do_job(sentence):
+    """python_decoder_do_job (src/decoder_sentence.cu:852-874): bytes in, translation text out."""
+    return load().python_decoder_do_job(sentence.encode("utf-8")).decode("utf-8", "replace")
 
 
 def read_model_information(path):

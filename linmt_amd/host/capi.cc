@@ -1,9 +1,12 @@
 // C facade over the C++ layer classes (declared in include/linmt_host.h).
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 
 #include "../../include/linmt_host.h"
+#include "decoder_sentence.h"
 #include "dispatcher.h"
 #include "file_helper.h"
 #include "input_file_preprocess.h"
@@ -478,4 +481,121 @@ extern "C" int lnmt_unint_file(const char *model_file, const char *unint_file, c
     InputFilePreprocess helper;
     helper.UnintFile(model_file, unint_file, final_file, sequence_to_sequence != 0, decoder_mode != 0);
   });
+}
+
+struct lnmt_decoder_sentence {
+  DecoderSentence decoder;
+};
+
+extern "C" lnmt_decoder_sentence *lnmt_decoder_sentence_create(const char *config_file, int load_model) {
+  lnmt_decoder_sentence *d = nullptr;
+  if (Guard([&] {
+        if (!config_file) throw LinmtError("lnmt_decoder_sentence_create: config_file is required");
+        std::unique_ptr<lnmt_decoder_sentence> p(new lnmt_decoder_sentence());
+        p->decoder.Init(config_file, load_model != 0);
+        d = p.release();
+      }) != 0)
+    return nullptr;
+  return d;
+}
+
+extern "C" void lnmt_decoder_sentence_destroy(lnmt_decoder_sentence *d) { delete d; }
+
+namespace {
+void CopyText(const std::string &text, char *out, size_t cap, size_t *needed) {
+  if (needed) *needed = text.size() + 1;
+  if (text.size() + 1 > cap) throw LinmtError("output buffer too small");
+  std::memcpy(out, text.c_str(), text.size() + 1);
+}
+}  // namespace
+
+extern "C" int lnmt_decoder_sentence_process(lnmt_decoder_sentence *d, const char *sentence, char *out,
+                                             size_t cap, size_t *needed) {
+  return Guard([&] {
+    std::string output;
+    d->decoder.Process(sentence, output);
+    CopyText(output, out, cap, needed);
+  });
+}
+
+extern "C" int lnmt_decoder_sentence_integerize(lnmt_decoder_sentence *d, const char *sentence, int *ids,
+                                                int cap, int *n) {
+  return Guard([&] {
+    std::vector<int> v;
+    d->decoder.IntegerizeSentence(sentence, v);
+    if (n) *n = (int)v.size();
+    if ((int)v.size() > cap) throw LinmtError("lnmt_decoder_sentence_integerize: ids buffer too small");
+    std::copy(v.begin(), v.end(), ids);
+  });
+}
+
+extern "C" int lnmt_decoder_sentence_unint(lnmt_decoder_sentence *d, const char *sentence, char *out,
+                                           size_t cap, size_t *needed) {
+  return Guard([&] {
+    std::string text(sentence);
+    d->decoder.UnintSentence(text);
+    CopyText(text, out, cap, needed);
+  });
+}
+
+extern "C" int lnmt_decoder_sentence_settings(lnmt_decoder_sentence *d, lnmt_decoding_options *o,
+                                              char *model_file, size_t cap) {
+  return Guard([&] {
+    const DecodingConfiguration &c = d->decoder.configuration();
+    std::memset(o, 0, sizeof(*o));
+    o->beam_size = c.beam_size_;
+    o->penalty = c.penalty_;
+    o->max_decoding_ratio = c.max_decoding_ratio_;
+    o->min_decoding_ratio = c.min_decoding_ratio_;
+    o->lp_alpha = c.decoding_lp_alpha_;
+    o->cp_beta = c.decoding_cp_beta_;
+    o->diversity = c.decoding_diversity_;
+    o->longest_sentence = c.longest_sentence_;
+    o->attention_width = c.attention_width_;
+    o->print_decoding_information = c.print_decoding_information_mode_;
+    o->print_alignments_scores = c.print_alignments_scores_mode_;
+    o->unk_replacement_mode = c.unk_replacement_mode_;
+    o->sentences_per_batch = c.sentences_per_batch_;
+    if (model_file) CopyText(c.model_name_, model_file, cap, nullptr);
+  });
+}
+
+// The process-wide decoder of the reference's translation server (src/decoder_sentence.cu:844-874):
+// one instance, the returned text is owned by the library and released by the next call, errors
+// end the process as the reference's do.
+namespace {
+char *decoder_result__ = nullptr;
+DecoderSentence *decoder_sentence__ = nullptr;
+
+[[noreturn]] void Fatal(const char *where, const std::exception &e) {
+  std::fprintf(stderr, "   Error: %s: %s\n", where, e.what());
+  std::exit(EXIT_FAILURE);
+}
+}  // namespace
+
+extern "C" void python_decoder_init(char *msg) {
+  try {
+    std::unique_ptr<DecoderSentence> fresh(new DecoderSentence());
+    fresh->Init(msg ? msg : "");
+    delete decoder_sentence__;
+    decoder_sentence__ = fresh.release();
+  } catch (const std::exception &e) {
+    Fatal("python_decoder_init", e);
+  }
+}
+
+extern "C" char *python_decoder_do_job(char *sentence) {
+  delete[] decoder_result__;
+  decoder_result__ = nullptr;
+  std::string output_sentence;
+  try {
+    if (!decoder_sentence__) throw LinmtError("python_decoder_init has not been called");
+    const std::string input_sentence(sentence ? sentence : "");
+    if (!input_sentence.empty()) decoder_sentence__->Process(input_sentence, output_sentence);
+  } catch (const std::exception &e) {
+    Fatal("python_decoder_do_job", e);
+  }
+  decoder_result__ = new char[output_sentence.size() + 1];
+  std::memcpy(decoder_result__, output_sentence.c_str(), output_sentence.size() + 1);
+  return decoder_result__;
 }

@@ -60,11 +60,12 @@ void NeuralMachineTranslation::DumpBestModel(const std::string &best_model_name,
   DumpWeights(best_model_name);
 }
 
-// One line of Decoder::OutputKBestHypotheses (src/decoder.h:602-681) for num_hypotheses = 1.
-static void WriteHypothesisLine(std::ostream &out, const SentenceResult &r, int source_length,
-                                const DecodingConfiguration &c) {
+// One line of Decoder::OutputKBestHypotheses (src/decoder.h:602-681) for num_hypotheses = 1;
+// Decoder::ObtainOneBestHypothesis (src/decoder.h:788-856) builds the same text as a string.
+void WriteHypothesis(std::ostream &out, const SentenceResult &r, int source_length,
+                     bool print_decoding_information, bool print_alignments_scores) {
   for (size_t j = 0; j < r.best.size(); ++j) out << (j ? " " : "") << r.best[j];
-  if (r.best_index >= 0 && c.print_decoding_information_mode_) {
+  if (r.best_index >= 0 && print_decoding_information) {
     const Hypothesis &h = r.hypotheses[r.best_index];
     auto viterbi = [&](size_t j) { return h.viterbi.empty() ? -1 : h.viterbi[j]; };
     const size_t size = h.tokens.size();
@@ -79,7 +80,7 @@ static void WriteHypothesisLine(std::ostream &out, const SentenceResult &r, int 
         out << " " << viterbi(j);
       }
     if (0 == unk_number) out << " -1";
-    if (c.print_alignments_scores_mode_) {
+    if (print_alignments_scores) {
       out << " ||||";
       for (size_t j = 1; j + 1 < size; ++j) {
         out << " ";
@@ -91,6 +92,11 @@ static void WriteHypothesisLine(std::ostream &out, const SentenceResult &r, int 
       if (size <= 2) out << " ";
     }
   }
+}
+
+static void WriteHypothesisLine(std::ostream &out, const SentenceResult &r, int source_length,
+                                const DecodingConfiguration &c) {
+  WriteHypothesis(out, r, source_length, c.print_decoding_information_mode_, c.print_alignments_scores_mode_);
   out << "\n";
 }
 

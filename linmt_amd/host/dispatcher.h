@@ -7,6 +7,7 @@
 
 #include <cfloat>
 #include <functional>
+#include <ostream>
 #include <string>
 #include <vector>
 
@@ -71,6 +72,12 @@ struct DecodingReport {
   long long source_words = 0, target_words = 0;
   double seconds = 0.0;  // decoding only (model loading and file conversion excluded)
 };
+
+// The text of one translation as the reference prints it: ids, then (print_decoding_information)
+// " |||| score |||| Viterbi alignments |||| <UNK> alignments" and (print_alignments_scores)
+// " |||| " the alignment scores of every token; no line end (src/decoder.h:602-681, 788-856).
+void WriteHypothesis(std::ostream &out, const SentenceResult &r, int source_length,
+                     bool print_decoding_information, bool print_alignments_scores);
 
 class Dispatcher {
  public:

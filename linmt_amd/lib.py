@@ -113,6 +113,9 @@ def load():
         raise LinmtHipError(
             f"{LIB_PATH} is missing: build it with `make -C linmt_amd/csrc` "
             "(or __graft_entry__.build()); there is no CPU fallback")
+    # torch brings a HIP runtime of its own; the callers here hand over torch tensors, so its
+    # runtime has to be the first one the process loads
+    import torch  # noqa: F401
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
