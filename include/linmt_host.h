@@ -40,6 +40,8 @@ typedef struct lnmt_decode_options {
   float max_decoding_ratio, min_decoding_ratio, penalty, diversity, lp_alpha, cp_beta;
   int unk_replacement_mode; /* the reference's unk_replacement_mode__: export alignment scores per
                                step, Viterbi alignments per token, coverage penalty on the scores */
+  int num_hypotheses;       /* the reference's hypotheses_number_: hypotheses kept per sentence
+                               (<= 0: 1) */
 } lnmt_decode_options;
 
 /* Training options (src/global_configuration.h:107-123, src/utility_cu.cu:82-96). */
@@ -110,11 +112,15 @@ int lnmt_get_state(lnmt_model *m, int kind, int side, int layer, int timestep, f
  * hyp_tokens != NULL also every finished hypothesis: hyp_tokens (n x hyp_cap x cap), hyp_len and
  * hyp_score (n x hyp_cap), n_hyp[n].  best_viterbi (n x cap, may be NULL; filled when
  * o->unk_replacement_mode is set): the source position (original order) aligned to each token of
- * the 1-best, -1 where no alignment score was positive. */
+ * the 1-best, -1 where no alignment score was positive.  kbest_index / kbest_score (n x
+ * o->num_hypotheses, may be NULL): the hypotheses Decoder::OutputKBestHypotheses keeps
+ * (src/decoder.h:587-607), best first, as indices into the sentence's finished hypotheses (the
+ * order of hyp_tokens) with their final scores; -1 / 0 where fewer pass the length filter. */
 int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int *lengths, int n,
                       const lnmt_decode_options *o, int *best, int cap, int *best_len,
                       float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
-                      float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi);
+                      float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi,
+                      int *kbest_index, float *kbest_score);
 
 /* The model's HIP stream (hipStream_t as void*), for callers that time with HIP events. */
 void *lnmt_model_stream(lnmt_model *m);
@@ -216,6 +222,7 @@ typedef struct lnmt_decoding_options {
   int attention_width; /* D of the local-p window (not stored in the model file); <= 0: 10 */
   int print_decoding_information, print_alignments_scores, unk_replacement_mode;
   int sentences_per_batch;
+  int num_hypotheses; /* k-best list per sentence, closed by a line of '=' when != 1; <= 0: 1 */
 } lnmt_decoding_options;
 int lnmt_decoding(const lnmt_decoding_options *o, int *sentences, int *sentences_thrown_away,
                   long long *source_words, long long *target_words, double *seconds);

@@ -55,14 +55,14 @@ class DecodingOptions(C.Structure):
                 ("longest_sentence", C.c_int), ("attention_width", C.c_int),
                 ("print_decoding_information", C.c_int),
                 ("print_alignments_scores", C.c_int), ("unk_replacement_mode", C.c_int),
-                ("sentences_per_batch", C.c_int)]
+                ("sentences_per_batch", C.c_int), ("num_hypotheses", C.c_int)]
 
 
 class DecodeOptions(C.Structure):
     _fields_ = [("beam_size", C.c_int), ("max_decoding_ratio", C.c_float),
                 ("min_decoding_ratio", C.c_float), ("penalty", C.c_float),
                 ("diversity", C.c_float), ("lp_alpha", C.c_float), ("cp_beta", C.c_float),
-                ("unk_replacement_mode", C.c_int)]
+                ("unk_replacement_mode", C.c_int), ("num_hypotheses", C.c_int)]
 
 
 def load():
@@ -102,7 +102,7 @@ def load():
     lib.lnmt_decode_batch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
                                       C.POINTER(DecodeOptions), C.c_void_p, C.c_int, C.c_void_p,
                                       C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
-                                      C.c_int, C.c_void_p]
+                                      C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.lnmt_model_stream.restype = C.c_void_p
     lib.lnmt_model_stream.argtypes = [C.c_void_p]
     lib.lnmt_profile_set_level.argtypes = [C.c_void_p, C.c_int]
@@ -345,14 +345,18 @@ class Model:
 
     def decode_batch(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0,
                      diversity=0.0, lp_alpha=0.65, cp_beta=0.20, with_hyps=False, hyp_cap=256,
-                     alignments=False):
-        """alignments=True: the reference's unk_replacement_mode__; results gain best_viterbi."""
+                     alignments=False, num_hypotheses=1):
+        """alignments=True: the reference's unk_replacement_mode__; results gain best_viterbi.
+        num_hypotheses > 1: results gain kbest = [(index into the finished hypotheses, final
+        score)], best first."""
         n = len(sentences)
         lengths = np.array([len(s) for s in sentences], np.int32)
         flat = np.ascontiguousarray(np.concatenate([np.asarray(s, np.int32) for s in sentences]))
         cap = self.cfg.longest_sentence + 2
         o = DecodeOptions(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta,
-                          int(alignments))
+                          int(alignments), int(num_hypotheses))
+        kidx = np.full((n, max(1, num_hypotheses)), -1, np.int32)
+        kscore = np.zeros((n, max(1, num_hypotheses)), np.float32)
         best = np.zeros((n, cap), np.int32)
         vit = np.full((n, cap), -1, np.int32) if alignments else None
         blen = np.zeros(n, np.int32)
@@ -366,7 +370,8 @@ class Model:
             hs = np.zeros((n, hyp_cap), np.float32)
         _check(load().lnmt_decode_batch(self.handle, _p(flat), _p(lengths), n, C.byref(o), _p(best),
                                         cap, _p(blen), _p(bscore), _p(steps), _p(ht), _p(hl),
-                                        _p(hs), hyp_cap, _p(nh), _p(vit)), "decode_batch")
+                                        _p(hs), hyp_cap, _p(nh), _p(vit), _p(kidx), _p(kscore)),
+               "decode_batch")
         res = []
         for i in range(n):
             r = dict(best=best[i, :blen[i]].copy(), best_score=float(bscore[i]),
@@ -376,6 +381,7 @@ class Model:
                 r["hyps"] = [(ht[i, j, :hl[i, j]].copy(), float(hs[i, j])) for j in range(k)]
             if alignments:
                 r["best_viterbi"] = vit[i, :blen[i]].copy()
+            r["kbest"] = [(int(a), float(b)) for a, b in zip(kidx[i], kscore[i]) if a >= 0]
             res.append(r)
         return res
 
@@ -383,14 +389,15 @@ class Model:
 def decoding(model_file, source_file, final_file, ids_file=None, beam=12, penalty=0.0,
              max_ratio=1.5, min_ratio=0.5, lp_alpha=0.65, cp_beta=0.20, diversity=0.0,
              longest_sentence=200, attention_width=10, print_decoding_information=False,
-             print_alignments_scores=False, unk_replacement_mode=False, sentences_per_batch=64):
+             print_alignments_scores=False, unk_replacement_mode=False, sentences_per_batch=64,
+             num_hypotheses=1):
     """Dispatcher::Decoding: translate a text file with a reference model file."""
     enc = lambda p: None if p is None else os.fsencode(p)  # noqa: E731
     o = DecodingOptions(enc(model_file), enc(source_file), enc(ids_file), enc(final_file), beam,
                         penalty, max_ratio, min_ratio, lp_alpha, cp_beta, diversity,
                         longest_sentence, attention_width, int(print_decoding_information),
                         int(print_alignments_scores), int(unk_replacement_mode),
-                        sentences_per_batch)
+                        sentences_per_batch, num_hypotheses)
     n, thrown, sw, tw, secs = C.c_int(), C.c_int(), C.c_longlong(), C.c_longlong(), C.c_double()
     _check(load().lnmt_decoding(C.byref(o), C.byref(n), C.byref(thrown), C.byref(sw), C.byref(tw),
                                 C.byref(secs)), "decoding")

@@ -219,7 +219,8 @@ extern "C" int lnmt_get_state(lnmt_model *m, int kind, int side, int layer, int 
 extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int *lengths, int n,
                                  const lnmt_decode_options *o, int *best, int cap, int *best_len,
                                  float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
-                                 float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi) {
+                                 float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi,
+                                 int *kbest_index, float *kbest_score) {
   return Guard([&] {
     std::vector<std::vector<int>> sents(n);
     size_t off = 0;
@@ -237,6 +238,7 @@ extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int 
     d.lp_alpha_ = o->lp_alpha;
     d.cp_beta_ = o->cp_beta;
     d.unk_replacement_mode_ = o->unk_replacement_mode != 0;
+    d.hypotheses_number_ = std::max(1, o->num_hypotheses);
     std::vector<SentenceResult> res;
     m->nmt->DecodeBatch(sents, d, &res);
     for (int i = 0; i < n; ++i) {
@@ -250,6 +252,11 @@ extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int 
       best_score[i] = r.best_score;
       if (steps) steps[i] = r.steps;
       if (n_hyp) n_hyp[i] = (int)r.hypotheses.size();
+      for (int k = 0; k < d.hypotheses_number_; ++k) {
+        const bool have = k < (int)r.kbest.size();
+        if (kbest_index) kbest_index[(size_t)i * d.hypotheses_number_ + k] = have ? r.kbest[k] : -1;
+        if (kbest_score) kbest_score[(size_t)i * d.hypotheses_number_ + k] = have ? r.kbest_score[k] : 0.f;
+      }
       if (hyp_tokens) {
         const int nh = std::min((int)r.hypotheses.size(), hyp_cap);
         for (int h = 0; h < nh; ++h) {
@@ -444,6 +451,7 @@ extern "C" int lnmt_decoding(const lnmt_decoding_options *o, int *sentences, int
     c.print_alignments_scores_mode_ = o->print_alignments_scores != 0;
     c.unk_replacement_mode_ = o->unk_replacement_mode != 0;
     if (o->sentences_per_batch > 0) c.sentences_per_batch_ = o->sentences_per_batch;
+    if (o->num_hypotheses > 0) c.hypotheses_number_ = o->num_hypotheses;
     const DecodingReport r = Dispatcher::Decoding(c);
     if (sentences) *sentences = r.sentences;
     if (sentences_thrown_away) *sentences_thrown_away = r.sentences_thrown_away;
@@ -556,6 +564,7 @@ extern "C" int lnmt_decoder_sentence_settings(lnmt_decoder_sentence *d, lnmt_dec
     o->print_alignments_scores = c.print_alignments_scores_mode_;
     o->unk_replacement_mode = c.unk_replacement_mode_;
     o->sentences_per_batch = c.sentences_per_batch_;
+    o->num_hypotheses = c.hypotheses_number_;
     if (model_file) CopyText(c.model_name_, model_file, cap, nullptr);
   });
 }

@@ -60,16 +60,17 @@ void NeuralMachineTranslation::DumpBestModel(const std::string &best_model_name,
   DumpWeights(best_model_name);
 }
 
-// One line of Decoder::OutputKBestHypotheses (src/decoder.h:602-681) for num_hypotheses = 1;
+// One line of Decoder::OutputKBestHypotheses (src/decoder.h:609-681) without its line end;
 // Decoder::ObtainOneBestHypothesis (src/decoder.h:788-856) builds the same text as a string.
 void WriteHypothesis(std::ostream &out, const SentenceResult &r, int source_length,
-                     bool print_decoding_information, bool print_alignments_scores) {
-  for (size_t j = 0; j < r.best.size(); ++j) out << (j ? " " : "") << r.best[j];
-  if (r.best_index >= 0 && print_decoding_information) {
-    const Hypothesis &h = r.hypotheses[r.best_index];
+                     bool print_decoding_information, bool print_alignments_scores, int rank) {
+  if (rank < 0 || rank >= (int)r.kbest.size()) return;  // nothing passed the length filter
+  const Hypothesis &h = r.hypotheses[r.kbest[rank]];
+  const size_t size = h.tokens.size();
+  for (size_t j = 1; j + 1 < size; ++j) out << (j > 1 ? " " : "") << h.tokens[j];
+  if (print_decoding_information) {
     auto viterbi = [&](size_t j) { return h.viterbi.empty() ? -1 : h.viterbi[j]; };
-    const size_t size = h.tokens.size();
-    out << " |||| " << r.best_score << " ||||";
+    out << " |||| " << r.kbest_score[rank] << " ||||";
     for (size_t j = 1; j + 1 < size; ++j) out << " " << viterbi(j);
     if (size <= 2) out << " ";
     out << " ||||";
@@ -94,10 +95,21 @@ void WriteHypothesis(std::ostream &out, const SentenceResult &r, int source_leng
   }
 }
 
-static void WriteHypothesisLine(std::ostream &out, const SentenceResult &r, int source_length,
-                                const DecodingConfiguration &c) {
-  WriteHypothesis(out, r, source_length, c.print_decoding_information_mode_, c.print_alignments_scores_mode_);
-  out << "\n";
+// What OutputKBestHypotheses writes for one sentence (src/decoder.h:609-696): a line per kept
+// hypothesis, best first, and a rule after the list unless a single hypothesis was asked for.  A
+// sentence without a hypothesis that passes the length filter writes no line in the reference;
+// an empty line stands for it here, so that line k of the output is always sentence k when one
+// hypothesis is asked for.
+static void WriteHypothesisLines(std::ostream &out, const SentenceResult &r, int source_length,
+                                 const DecodingConfiguration &c) {
+  const int n = (int)r.kbest.size();
+  for (int rank = 0; rank < n; ++rank) {
+    WriteHypothesis(out, r, source_length, c.print_decoding_information_mode_,
+                    c.print_alignments_scores_mode_, rank);
+    out << "\n";
+  }
+  if (1 != c.hypotheses_number_) out << "================\n";
+  else if (n == 0) out << "\n";
 }
 
 DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
@@ -145,6 +157,7 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
   o.lp_alpha_ = c.decoding_lp_alpha_;
   o.cp_beta_ = c.decoding_cp_beta_;
   o.unk_replacement_mode_ = c.unk_replacement_mode_ && g.attention_mode_;
+  o.hypotheses_number_ = std::max(1, c.hypotheses_number_);
 
   const std::string ids_file =
       c.decoder_output_file_.empty() ? c.decoder_final_file_ + ".ids" : c.decoder_output_file_;
@@ -166,7 +179,7 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
       if (!batch.empty()) neural.DecodeBatch(batch, o, &results);
       for (size_t b = 0; b < batch.size(); ++b) ordered[where[b]] = std::move(results[b]);
       for (size_t i = first; i < last; ++i) {
-        WriteHypothesisLine(output, ordered[i - first], (int)sentences[i].size(), c);
+        WriteHypothesisLines(output, ordered[i - first], (int)sentences[i].size(), c);
         report.source_words += (long long)sentences[i].size();
         report.target_words += (long long)ordered[i - first].best.size();
       }

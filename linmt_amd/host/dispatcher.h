@@ -56,6 +56,7 @@ struct DecodingConfiguration {
   std::string decoder_output_file_;  // ids of the translations ("" = decoder_final_file_ + ".ids")
   std::string decoder_final_file_;   // the translations as words
   int beam_size_ = 12;
+  int hypotheses_number_ = 1;  // k-best list per sentence, closed by a line of '=' when != 1
   float penalty_ = 0.f, max_decoding_ratio_ = 1.5f, min_decoding_ratio_ = 0.5f;
   float decoding_lp_alpha_ = 0.65f, decoding_cp_beta_ = 0.20f, decoding_diversity_ = 0.f;
   int longest_sentence_ = 200;  // src/global_configuration.h:298: 100, doubled for translation
@@ -76,14 +77,15 @@ struct DecodingReport {
 // The text of one translation as the reference prints it: ids, then (print_decoding_information)
 // " |||| score |||| Viterbi alignments |||| <UNK> alignments" and (print_alignments_scores)
 // " |||| " the alignment scores of every token; no line end (src/decoder.h:602-681, 788-856).
+// rank: which of the kept hypotheses (0 = best).
 void WriteHypothesis(std::ostream &out, const SentenceResult &r, int source_length,
-                     bool print_decoding_information, bool print_alignments_scores);
+                     bool print_decoding_information, bool print_alignments_scores, int rank = 0);
 
 class Dispatcher {
  public:
   // Dispatcher::Decoding (src/dispatcher.cu:387-436): model file -> decoder, source text -> ids
   // (InputFilePreprocess::IntegerizeFileDecoding), beam search (EnsembleFactory::DecodeFile with
-  // one model), id output (Decoder::OutputKBestHypotheses, one hypothesis per sentence) -> words
+  // one model), id output (Decoder::OutputKBestHypotheses) -> words
   // (UnintFile).
   static DecodingReport Decoding(const DecodingConfiguration &configuration);
 

@@ -345,6 +345,9 @@ struct DecodeOptions {
   // scores of every step; hypotheses carry Viterbi alignments and the coverage penalty is computed
   // from the exported scores instead of zeros
   bool unk_replacement_mode_ = false;
+  // the reference's hypotheses_number_ (global_configuration.h:229): how many of the finished
+  // hypotheses OutputKBestHypotheses keeps, best first
+  int hypotheses_number_ = 1;
 };
 
 struct SentenceResult {
@@ -352,6 +355,10 @@ struct SentenceResult {
   std::vector<int> best_viterbi;  // unk_replacement_mode_: source position aligned to each token
   int best_index = -1;            // index of the 1-best in hypotheses
   float best_score = 0.f;
+  // the hypotheses_number_ best (fewer when fewer pass the length filter): indices into
+  // hypotheses, best first, with their final scores; kbest[0] == best_index
+  std::vector<int> kbest;
+  std::vector<float> kbest_score;
   std::vector<Hypothesis> hypotheses;  // in the order the reference's v_hypotheses_ would hold them
   int steps = 0;                       // decoder forward passes this sentence took part in
 };
@@ -376,7 +383,7 @@ class Decoder {
   DeviceArray<float> align_hist_;
   DeviceArray<int> index_hist_;
   void Init(int beam_size, int n_sent, int max_steps);
-  // OutputKBestHypotheses (decoder.h:529-699) for one sentence, num_hypotheses = 1.
+  // OutputKBestHypotheses (decoder.h:529-699) for one sentence: the selection, not the printing.
   static void OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_length,
                                     const DecodeOptions &o, SentenceResult *out);
 };

@@ -498,8 +498,14 @@ void Decoder::Init(int beam_size, int n_sent, int max_steps) {
 // place as the reference does (so a later print shows the normalised values).
 void Decoder::OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_length,
                                     const DecodeOptions &o, SentenceResult *out) {
-  int best = -1;
-  float best_score = 0.f;
+  // the kept set, worst first: a hypothesis enters while there is room, afterwards only by beating
+  // the worst kept one strictly (decoder.h:589-600; which of two exactly equal scores the
+  // reference's heap drops first is not defined by its source)
+  const size_t keep = (size_t)std::max(1, o.hypotheses_number_);
+  std::vector<std::pair<float, int>> kept;
+  auto worse = [](const std::pair<float, int> &a, const std::pair<float, int> &b) {
+    return a.first != b.first ? a.first < b.first : a.second > b.second;
+  };
   for (size_t i = 0; i < hyps.size(); ++i) {
     float s = hyps[i].score;
     const int size = (int)hyps[i].tokens.size();
@@ -539,11 +545,26 @@ void Decoder::OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_le
       s += cp_x_y;
     }
     const float len_ratio = ((float)size) / source_length;
-    if (len_ratio > o.min_decoding_ratio_ && (best < 0 || best_score < s)) {
-      best = (int)i;
-      best_score = s;
+    if (len_ratio > o.min_decoding_ratio_) {
+      if (kept.size() < keep) {
+        kept.emplace_back(s, (int)i);
+      } else {
+        auto lowest = std::min_element(kept.begin(), kept.end(), worse);
+        if (lowest->first < s) *lowest = std::make_pair(s, (int)i);
+      }
     }
   }
+  std::sort(kept.begin(), kept.end(), [&](const std::pair<float, int> &a, const std::pair<float, int> &b) {
+    return worse(b, a);
+  });
+  out->kbest.clear();
+  out->kbest_score.clear();
+  for (const auto &k : kept) {
+    out->kbest.push_back(k.second);
+    out->kbest_score.push_back(k.first);
+  }
+  const int best = kept.empty() ? -1 : kept[0].second;
+  const float best_score = kept.empty() ? 0.f : kept[0].first;
   out->best.clear();
   out->best_viterbi.clear();
   out->best_index = best;
@@ -775,9 +796,10 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
       }
     }
     Decoder::OutputKBestHypotheses(r.hypotheses, source_length, o, &r);
-    if (capture)  // only the 1-best keeps its score rows (they are what a printout shows)
+    if (capture)  // only the hypotheses kept hold on to their score rows (what a printout shows)
       for (size_t h = 0; h < r.hypotheses.size(); ++h)
-        if ((int)h != r.best_index) std::vector<std::vector<float>>().swap(r.hypotheses[h].alignments_scores);
+        if (std::find(r.kbest.begin(), r.kbest.end(), (int)h) == r.kbest.end())
+          std::vector<std::vector<float>>().swap(r.hypotheses[h].alignments_scores);
   }
 }
 

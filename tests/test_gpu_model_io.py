@@ -134,3 +134,63 @@ def test_decoding_a_text_file(host, tmp_path):
         assert text.split(" |||| ")[0].split() == [tword(t) for t in toks]
         assert text.split(" |||| ")[1:] == fields[1:]
     assert rep["target_words"] == sum(len(w["best"]) for w in want)
+
+
+def test_k_best_lists(host, tmp_path):
+    """Decoder::OutputKBestHypotheses with hypotheses_number_ > 1 (src/decoder.h:529-607, 692-694):
+    the kept hypotheses are the k best final scores among those that pass the length filter, best
+    first; a decoded file holds them line by line with a rule of '=' after every sentence.  The
+    final scores are recomputed here from the raw hypotheses: length normalisation
+    ((5+|Y|)/6)^alpha and, without exported alignments, the coverage penalty of uniform rows."""
+    rng = np.random.default_rng(21)
+    layers, H, Vs, Vt, D, beam, k = 2, 24, 30, 40, 2, 5, 3
+    P = R.make_params(rng, layers, H, Vs, Vt, attention=True, feed_input=True, scale=0.8)
+    kw = dict(longest_sentence=24, attention_mode=1, attention_width=D, feed_input=True)
+    m = host.Model(layers, H, Vs, Vt, decoding=(2, beam), **kw)
+    m.set_params(P)
+    sents = [rng.integers(0, Vs, size=n) for n in (7, 4)]
+    alpha, beta, min_ratio = np.float32(0.65), np.float32(0.2), 0.5
+    res = m.decode_batch(sents, beam=beam, with_hyps=True, num_hypotheses=k)
+    one = m.decode_batch(sents, beam=beam)
+    for sent, r, r1 in zip(sents, res, one):
+        S = len(sent)
+        final = []
+        for toks, raw in r["hyps"]:
+            size = len(toks)
+            s_ = np.float32(raw) / (np.float32(5 + size) ** alpha / np.float32(6) ** alpha)
+            col = np.float32(0)
+            for _ in range(1, size - 1):
+                col += np.float32(0.01) / np.float32(S * 0.01)
+            cp = max(np.float32(beta * S * np.log(min(col, np.float32(1)))), np.float32(-20)) if size > 2 \
+                else np.float32(-20)
+            final.append((float(s_ + cp), size / S > min_ratio))
+        order = sorted((i for i, f in enumerate(final) if f[1]), key=lambda i: -final[i][0])[:k]
+        assert len(order) == k                        # the case is sized so that k survive
+        assert [i for i, _ in r["kbest"]] == order
+        assert np.allclose([s_ for _, s_ in r["kbest"]], [final[i][0] for i in order], rtol=1e-4, atol=1e-5)
+        # the head of the list is the single hypothesis of the default call
+        assert r["hyps"][order[0]][0][1:-1].tolist() == r1["best"].tolist() == r["best"].tolist()
+
+    a = host.Model(layers, H, Vs, Vt, minibatch_size=1, **kw)
+    a.set_params(P)
+    model = str(tmp_path / "model.nmt")
+    a.dump_model(model)
+    word = lambda i: "<UNK>" if i == 0 else f"w{i}"  # noqa: E731
+    src = tmp_path / "src.txt"
+    src.write_text("".join(" ".join(word(i) for i in s_) + "\n" for s_ in sents))
+    final_file, ids = str(tmp_path / "out.txt"), str(tmp_path / "out.ids")
+    host.decoding(model, str(src), final_file, ids_file=ids, beam=beam, longest_sentence=24,
+                  attention_width=D, print_decoding_information=True, sentences_per_batch=2,
+                  num_hypotheses=k)
+    lines = open(ids).read().split("\n")[:-1]
+    assert len(lines) == 2 * (k + 1) and lines[k] == lines[2 * k + 1] == "================"
+    b = host.Model(layers, H, Vs, Vt, decoding=(2, beam), **kw)
+    b.load_weights(model)
+    want = b.decode_batch(sents, beam=beam, with_hyps=True, num_hypotheses=k)
+    for sidx, w in enumerate(want):
+        for rank, (hyp, score) in enumerate(w["kbest"]):
+            fields = lines[sidx * (k + 1) + rank].split(" |||| ")
+            assert [int(x) for x in fields[0].split()] == w["hyps"][hyp][0][1:-1].tolist()
+            assert np.isclose(float(fields[1]), score, rtol=1e-4, atol=1e-5)
+    words = open(final_file).read().split("\n")[:-1]
+    assert len(words) == len(lines) and words[k] == "================"
