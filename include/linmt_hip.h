@@ -123,6 +123,33 @@ int lh_gemm_ws_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, 
 int lh_gemm_planes_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
                        float beta, float *C, int ldc, void *workspace, size_t workspace_bytes,
                        int max_planes, int *planes, lh_stream_t stream);
+/* The stacked gate product of one LSTM step AND the cell, in one kernel (inference form: no gate
+ * values kept, no dropout):
+ *   pre = sum_s A_s X_s (+ addend[:, addend_col ? addend_col[b] : b]) + bias4h     (4H x B, never stored)
+ *   c, h = cell(pre, c_prev, mask01)                        exactly as lh_lstm_cell_fwd_f32 computes them
+ * Replaces, for one node, the 8-12 SGEMMs and the gate / cell / hidden-state kernels of
+ * LstmInputHiddenNode::ForwardPropGpu (src/node_input_to_hidden.h:218-636) and
+ * LstmHiddenHiddenNode::ForwardPropGpu (src/node_hidden_to_hidden.h:194-444).  A_s are the stacked
+ * 4H x K_s gate matrices (rows g*H .. g*H+H-1 = gate g in the order i, f, c', o), X_s the K_s x B
+ * inputs, all as stored (no transposes).  addend (4H x anything, leading dimension ld_addend, may
+ * be NULL) holds pre-activation terms computed elsewhere: the input product of every step done
+ * ahead of the recurrence, or -- with addend_col = the token of each column -- a table of input
+ * products per vocabulary entry (addend_ncols of them; ids are clamped into that range like
+ * lh_embed_lookup_f32 does), which makes the embedding lookup part of this kernel.
+ * c may be c_prev; c and h must not overlap an X operand.
+ * Only products that lh_gemm_planes_f32 would run as one unsplit launch of a tile whose LDS can
+ * hold the whole tile are run this way: lh_gate_gemm_lstm_cell_plan says whether that is so
+ * (*fusable) and names the kernel instance; when it is not, lh_gate_gemm_lstm_cell_f32 fails and
+ * the caller uses lh_gemm_planes_f32 + lh_lstm_cell_fwd_f32.  workspace_bytes is what the caller
+ * would hand lh_gemm_planes_f32 (it only steers the choice; no workspace is used). */
+int lh_gate_gemm_lstm_cell_plan(int H, int B, const lh_gemm_seg *segs, int nseg, int has_addend,
+                                size_t workspace_bytes, int *fusable, char *name, int name_cap);
+int lh_gate_gemm_lstm_cell_f32(int H, int B, const lh_gemm_seg *segs, int nseg, const float *addend,
+                               int ld_addend, const int *addend_col, int addend_ncols,
+                               const float *bias4h,
+                               const float *c_prev, const int *mask01, int sigmoid_f64,
+                               float cell_clip, float *c, float *h, size_t workspace_bytes,
+                               lh_stream_t stream);
 /* Name of the kernel instance lh_gemm_ws_f32 (max_planes = 0) or lh_gemm_planes_f32 would launch
  * for this problem (tile shape and operand flags), as profilers print it; no counterpart in the
  * reference.  Pointers in `segs` are only inspected for alignment; workspace_bytes = 0 describes

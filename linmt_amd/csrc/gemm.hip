@@ -50,6 +50,17 @@ struct GemmArgs {
   float *ws_part;
   int ws_ld;
   int leave_partial;  // host only: the caller sums the planes itself, no reduction launch
+  // Gate product with the LSTM cell in its epilogue (gate_gemm_cell_kernel): M = 4 * cell_H rows
+  // in gate order i, f, c', o; C (ldc) is a read-only addend to the pre-activations when beta = 1,
+  // taken from column addend_col[n] when that is given; bias and colmask are the stacked gate bias
+  // and the 0/1 column mask; the kernel writes c_out and h_out (cell_H x N) and nothing else.
+  int cell_H;
+  const float *c_prev;
+  float *c_out, *h_out;
+  float cell_clip;
+  int sigmoid_f64;
+  const int *addend_col;
+  int addend_ncols;  // entries of addend_col are clamped to [0, addend_ncols)
 };
 
 // Stages one BK x BD operand slab: global -> registers (load), registers -> LDS [BK][BD+PAD] (store).
@@ -419,6 +430,19 @@ struct Stage {
       goff[i] = d < dn ? off : 0u;
     }
   }
+  // The same for a tile of a stacked gate matrix that holds BD/4 rows of each of the four gates:
+  // tile row d is row (d % (BD/4)) of gate d / (BD/4); gates are H rows apart; rows_left = rows of
+  // a gate that exist from the tile origin on.
+  __device__ __forceinline__ void set_ld_gates(int ld, int tid, int H, int rows_left) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int u = tid + i * NT;
+      const int d = unit_d(u), k = unit_k(u);
+      const int r = d % (BD / 4), row = (d / (BD / 4)) * H + r;
+      const unsigned off = KC ? (unsigned)(row * ld + k) * 4u : (unsigned)(k * ld + row) * 4u;
+      goff[i] = r < rows_left ? off : 0u;
+    }
+  }
   // kn (< BK) = k values left in the segment: units past it re-read the slab origin and are
   // zeroed before they reach LDS.
   __device__ __forceinline__ void clamp_tail(int tid, int kn) {
@@ -471,8 +495,9 @@ constexpr int smem2_floats() {
               (WK - 1) * BM * BN);
 }
 
-template <int BM, int BN, int WM, int WN, int WK, int BK, bool TA, bool TX>
-__global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs g) {
+// CELL: the rows of a tile are BM/4 rows of each LSTM gate and the epilogue is the LSTM cell.
+template <int BM, int BN, int WM, int WN, int WK, int BK, bool TA, bool TX, bool CELL>
+__device__ __forceinline__ void gemm_body(const GemmArgs &g) {
   constexpr int NT = 64 * WM * WN * WK;
   constexpr int TM = BM / WM, TN = BN / WN;
   constexpr int FM = TM / 32, FN = TN / 32;
@@ -495,7 +520,8 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
   const int splits = g.splits;
   const int tile = splits == 1 ? logical : logical / splits;
   const int split = splits == 1 ? 0 : logical % splits;
-  const int m0 = (tile / g.tiles_n) * BM;
+  // CELL: m0 counts rows of ONE gate
+  const int m0 = (tile / g.tiles_n) * (CELL ? BM / 4 : BM);
   const int n0 = (tile % g.tiles_n) * BN;
 
   const int tid = threadIdx.x;
@@ -549,7 +575,8 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
     const int lx = lseg == 0 ? ldx0 : (lseg == 1 ? ldx1 : ldx2);                     \
     const int Ks = lseg == 0 ? K0 : (lseg == 1 ? K1 : K2);                           \
     if (new_seg) {                                                                   \
-      sa.set_ld(la, tid, M - m0);                                                    \
+      if constexpr (CELL) sa.set_ld_gates(la, tid, g.cell_H, g.cell_H - m0);         \
+      else sa.set_ld(la, tid, M - m0);                                               \
       sx.set_ld(lx, tid, N - n0);                                                    \
     }                                                                                \
     const float *pa = TA ? Ab + (size_t)m0 * la + lk0 : Ab + (size_t)lk0 * la + m0;  \
@@ -653,6 +680,54 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
     }
   }
 
+  if constexpr (CELL) {
+    // The four gates of a cell sit in different wavefronts: the tile goes through LDS as
+    // S[n][m] (the slab buffers and the partial tiles are dead), then every thread of the
+    // workgroup takes cells.
+    constexpr int GQ = BM / 4;
+    static_assert(smem2_floats<BM, BN, WM, WN, WK, BK, TA, TX>() >= BM * BN, "tile does not fit LDS");
+    if constexpr (WK > 1) __syncthreads();  // the partial tiles have been read
+    if (wk == 0) {
+#pragma unroll
+      for (int a = 0; a < FN; ++a)
+#pragma unroll
+        for (int b = 0; b < FM; ++b)
+#pragma unroll
+          for (int j = 0; j < 16; ++j)
+            smem[(wn * TN + a * 32 + lhi * 4 + (j / 4) * 8 + (j % 4)) * BM + wm * TM + b * 32 + l32] =
+                acc[a][b][j];
+    }
+    __syncthreads();
+    const int H = g.cell_H;
+    const bool add = g.beta != 0.f;
+    for (int idx = tid; idx < GQ * BN; idx += NT) {
+      const int rl = idx % GQ, nl = idx / GQ;
+      const int r = m0 + rl, n = n0 + nl;
+      if (r >= H || n >= g.N) continue;
+      float pre[4];
+      int col = n;
+      if (g.addend_col) col = min(max(g.addend_col[n], 0), g.addend_ncols - 1);
+      const float *ad = add ? g.C + (size_t)col * g.ldc + r : nullptr;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float v = smem[nl * BM + q * GQ + rl];
+        if (add) v += ad[(size_t)q * H];
+        pre[q] = v + g.bias[q * H + r];
+      }
+      const size_t o = (size_t)n * H + r;
+      float c, h;
+      if (g.sigmoid_f64)
+        lh::lstm_cell_point<true>(pre[0], pre[1], pre[2], pre[3], g.c_prev[o], (float)g.colmask[n],
+                                  g.cell_clip, c, h);
+      else
+        lh::lstm_cell_point<false>(pre[0], pre[1], pre[2], pre[3], g.c_prev[o], (float)g.colmask[n],
+                                   g.cell_clip, c, h);
+      g.c_out[o] = c;
+      g.h_out[o] = h;
+    }
+    return;
+  }
+
   if (wk > 0) return;
 
   // Epilogue: accumulator register j of lane l is C[m = .. + l%32][n = .. + 8*(j/4) + 4*(l/32) + j%4].
@@ -688,6 +763,23 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs 
       }
     }
   }
+}
+
+template <int BM, int BN, int WM, int WN, int WK, int BK, bool TA, bool TX>
+__global__ __launch_bounds__(64 * WM * WN * WK) void gemm_kernel(const GemmArgs g) {
+  gemm_body<BM, BN, WM, WN, WK, BK, TA, TX, false>(g);
+}
+
+// Stacked gate product W*[x; h; h~] (both operands as stored, no transposes) + LSTM cell.
+template <int BM, int BN, int WM, int WN, int WK, int BK>
+__global__ __launch_bounds__(64 * WM * WN * WK) void gate_gemm_cell_kernel(const GemmArgs g) {
+  gemm_body<BM, BN, WM, WN, WK, BK, false, false, true>(g);
+}
+
+// Whether a configuration's LDS holds a whole tile, which the cell epilogue needs.
+template <int BM, int BN, int WM, int WN, int WK, int BK>
+constexpr bool cell_capable() {
+  return smem2_floats<BM, BN, WM, WN, WK, BK, false, false>() >= BM * BN;
 }
 
 // Second half of a split product: C = epilogue(sum of the partial planes, in split order).
@@ -825,6 +917,43 @@ int launch_index(int c, const GemmArgs &g, bool ta, bool tx, bool vec, hipStream
 }
 
 template <int BM, int BN, int WM, int WN, int WK, int BK>
+int launch_cell_cfg(const GemmArgs &g0, hipStream_t st) {
+  if constexpr (cell_capable<BM, BN, WM, WN, WK, BK>()) {
+    GemmArgs g = g0;
+    g.tiles_m = (g.cell_H + BM / 4 - 1) / (BM / 4);
+    g.tiles_n = (g.N + BN - 1) / BN;
+    g.splits = 1;
+    g.slabs_per_split = 0;
+    for (int s = 0; s < g.nseg; ++s) g.slabs_per_split += (g.K[s] + BK - 1) / BK;
+    const dim3 grid(g.tiles_m * g.tiles_n), block(64 * WM * WN * WK);
+    return launch_kernel(gate_gemm_cell_kernel<BM, BN, WM, WN, WK, BK>,
+                         smem2_floats<BM, BN, WM, WN, WK, BK, false, false>() * 4, grid, block, st, g);
+  } else {
+    return lh::fail_arg("lh_gate_gemm_lstm_cell_f32: internal error, tile %dx%d cannot hold the cell", BM, BN);
+  }
+}
+
+int launch_cell_index(int c, const GemmArgs &g, hipStream_t st) {
+  switch (c) {
+#define LH_CFG_CASE(I, BM, BN, WM, WN, WK, BK) \
+  case I: return launch_cell_cfg<BM, BN, WM, WN, WK, BK>(g, st);
+    LH_GEMM_CONFIGS(LH_CFG_CASE)
+#undef LH_CFG_CASE
+    default: return lh::fail_arg("lh_gate_gemm_lstm_cell_f32: configuration %d does not exist", c);
+  }
+}
+
+bool cell_capable_index(int c) {
+  switch (c) {
+#define LH_CFG_CASE(I, BM, BN, WM, WN, WK, BK) \
+  case I: return cell_capable<BM, BN, WM, WN, WK, BK>();
+    LH_GEMM_CONFIGS(LH_CFG_CASE)
+#undef LH_CFG_CASE
+    default: return false;
+  }
+}
+
+template <int BM, int BN, int WM, int WN, int WK, int BK>
 int occupancy_cfg(bool ta, bool tx, int *blocks_per_cu, int *lds_bytes) {
   constexpr int block = 64 * WM * WN * WK;
   hipError_t e;
@@ -888,6 +1017,7 @@ struct Tuning {
 #include "gemm_tuning.inc"
 constexpr int kCUs = 256;
 constexpr float kReduceFixedUs = 2.5f, kReduceBytesPerUs = 3.0e6f;
+constexpr float kCellFixedUs = 4.0f;  // a launch of the LSTM cell kernel behind its product
 
 float predict_us(const Tuning &t, const Config &k, int M, int N, const int *K, int nseg, int want,
                  bool reduce_free, int *splits) {
@@ -916,9 +1046,15 @@ float predict_us(const Tuning &t, const Config &k, int M, int N, const int *K, i
 }
 
 // max_planes > 0: the caller consumes up to that many partial planes itself (no reduction pass).
+
+// only_cell: restrict the choice to unsplit launches of configurations whose LDS holds a whole
+// tile (what the gate product with the cell in its epilogue can use).  *us (optional) receives
+// the predicted time of the choice.
 void pick_config(int M, int N, const int *K, int nseg, bool ta, bool tx, bool vec,
-                 size_t workspace_bytes, int max_planes, int *config, int *splits) {
+                 size_t workspace_bytes, int max_planes, int *config, int *splits,
+                 bool only_cell = false, float *us_out = nullptr) {
   *splits = 1;
+  if (us_out) *us_out = 0.f;
   if (!vec) {
     *config = kUnalignedConfig;
     return;
@@ -927,10 +1063,11 @@ void pick_config(int M, int N, const int *K, int nseg, bool ta, bool tx, bool ve
   struct Memo {
     int M, N, K[LH_GEMM_MAX_SEGS], flags, config, splits;
     size_t workspace_bytes;
+    float us;
   };
   static thread_local Memo memo[64];
   const int flags = 1 + (ta ? 2 : 0) + (tx ? 4 : 0) + 8 * nseg + 64 * (g_config_override + 1) +
-                    4096 * g_splits_override + 131072 * max_planes;
+                    4096 * g_splits_override + 131072 * max_planes + (only_cell ? 1048576 : 0);
   int Kk[LH_GEMM_MAX_SEGS] = {0, 0, 0};
   for (int s = 0; s < nseg; ++s) Kk[s] = K[s];
   const unsigned h = ((unsigned)M * 2654435761u) ^ ((unsigned)N * 40503u) ^ ((unsigned)Kk[0] * 97u) ^
@@ -940,6 +1077,7 @@ void pick_config(int M, int N, const int *K, int nseg, bool ta, bool tx, bool ve
       e.K[2] == Kk[2] && e.workspace_bytes == workspace_bytes) {
     *config = e.config;
     *splits = e.splits;
+    if (us_out) *us_out = e.us;
     return;
   }
   static const int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
@@ -948,8 +1086,10 @@ void pick_config(int M, int N, const int *K, int nseg, bool ta, bool tx, bool ve
   *config = kUnalignedConfig;
   for (int c = 0; c < kNumConfigs; ++c) {
     if (g_config_override >= 0 && c != g_config_override) continue;
+    if (only_cell && !cell_capable_index(c)) continue;
     for (int want : kSplitChoices) {
-      if (g_splits_override > 0) want = fit_splits(M, N, g_splits_override, workspace_bytes);
+      if (only_cell && want > 1) break;
+      if (!only_cell && g_splits_override > 0) want = fit_splits(M, N, g_splits_override, workspace_bytes);
       if (max_planes > 0 && want > max_planes) want = max_planes;
       if (want > 1 && fit_splits(M, N, want, workspace_bytes) < want) break;
       int S;
@@ -962,7 +1102,9 @@ void pick_config(int M, int N, const int *K, int nseg, bool ta, bool tx, bool ve
       if (g_splits_override > 0 || (max_planes > 0 && want >= max_planes)) break;
     }
   }
-  e = Memo{M, N, {Kk[0], Kk[1], Kk[2]}, flags, *config, *splits, workspace_bytes};
+  if (best > 2.9e38f) *config = -1;  // only_cell: the override names a configuration that cannot
+  if (us_out) *us_out = best;
+  e = Memo{M, N, {Kk[0], Kk[1], Kk[2]}, flags, *config, *splits, workspace_bytes, best};
 }
 
 struct Prepared {
@@ -1069,6 +1211,100 @@ extern "C" int lh_gemm_planes_f32(int M, int N, const lh_gemm_seg *segs, int nse
   const int share = (slabs + want - 1) / want;
   *planes = (slabs + share - 1) / share;
   return launch_index(p.config, p.g, p.ta, p.tx, p.vec, lh::as_stream(stream));
+}
+
+namespace {
+// The choice lh_gemm_planes_f32 makes for the stacked gate product of an LSTM cell, and whether
+// that choice can carry the cell in its epilogue: aligned operands, no K split, a tile that fits LDS.
+int plan_cell(int H, int B, const lh_gemm_seg *segs, int nseg, bool has_addend, const float *addend,
+              int ld_addend, size_t workspace_bytes, Prepared *p, bool *fusable) {
+  if (H <= 0 || B <= 0) return lh::fail_arg("lh_gate_gemm_lstm_cell: H=%d B=%d", H, B);
+  float dummy;
+  const int rc = prepare(4 * H, B, segs, nseg, 0, 0, 1.f, has_addend ? 1.f : 0.f, nullptr, LH_ACT_NONE,
+                         4 * H, nullptr, has_addend && addend ? const_cast<float *>(addend) : &dummy,
+                         has_addend && addend ? ld_addend : 4 * H,
+                         workspace_bytes ? (void *)(uintptr_t)256 : nullptr, workspace_bytes,
+                         has_addend ? 2 : 3, p);
+  if (rc != LH_OK) return rc;
+  *fusable = false;
+  if (!p->vec || H % 4 != 0) return LH_OK;
+  // Best unsplit launch that can carry the cell against the best launch of any kind followed by
+  // the cell kernel (a launch of its own that reads the pre-activations, or S planes of them, back).
+  int cfg_any, splits_any, cfg_cell, splits_cell;
+  float us_any, us_cell;
+  const size_t ws = workspace_bytes;
+  pick_config(4 * H, B, p->g.K, nseg, false, false, true, ws, has_addend ? 2 : 3, &cfg_any, &splits_any,
+              false, &us_any);
+  pick_config(4 * H, B, p->g.K, nseg, false, false, true, ws, has_addend ? 2 : 3, &cfg_cell,
+              &splits_cell, true, &us_cell);
+  if (cfg_cell < 0) return LH_OK;
+  const float cell_us = kCellFixedUs + 28.f * (float)H * (float)B / kReduceBytesPerUs;
+  if (us_cell <= us_any + cell_us) {
+    *fusable = true;
+    p->config = cfg_cell;
+    p->g.splits = 1;
+  }
+  return LH_OK;
+}
+}  // namespace
+
+extern "C" int lh_gate_gemm_lstm_cell_plan(int H, int B, const lh_gemm_seg *segs, int nseg,
+                                           int has_addend, size_t workspace_bytes, int *fusable,
+                                           char *name, int name_cap) {
+  if (!fusable) return lh::fail_arg("lh_gate_gemm_lstm_cell_plan: fusable is NULL");
+  Prepared p;
+  bool f = false;
+  const int rc = plan_cell(H, B, segs, nseg, has_addend != 0, nullptr, 0, workspace_bytes, &p, &f);
+  if (rc != LH_OK) return rc;
+  *fusable = f ? 1 : 0;
+  if (name && name_cap > 0) {
+    const Config &k = kConfigs[p.config];
+    if (f) snprintf(name, name_cap, "gate_gemm_cell_kernel<%d, %d, %d, %d, %d, %d>", k.bm, k.bn, k.wm, k.wn, k.wk, k.bk);
+    else name[0] = 0;
+  }
+  return LH_OK;
+}
+
+extern "C" int lh_gate_gemm_lstm_cell_f32(int H, int B, const lh_gemm_seg *segs, int nseg,
+                                          const float *addend, int ld_addend, const int *addend_col,
+                                          int addend_ncols, const float *bias4h, const float *c_prev,
+                                          const int *mask01, int sigmoid_f64, float cell_clip,
+                                          float *c, float *h, size_t workspace_bytes,
+                                          lh_stream_t stream) {
+  if (!bias4h || !c_prev || !mask01 || !c || !h)
+    return lh::fail_arg("lh_gate_gemm_lstm_cell_f32: a required pointer is NULL");
+  if (addend && ld_addend < 4 * H)
+    return lh::fail_arg("lh_gate_gemm_lstm_cell_f32: ld_addend=%d < 4H=%d", ld_addend, 4 * H);
+  if (addend_col && (!addend || addend_ncols < 1))
+    return lh::fail_arg("lh_gate_gemm_lstm_cell_f32: addend_col needs addend and addend_ncols >= 1");
+  Prepared p;
+  bool f = false;
+  const int rc = plan_cell(H, B, segs, nseg, addend != nullptr, addend, ld_addend, workspace_bytes, &p, &f);
+  if (rc != LH_OK) return rc;
+  if (!f)
+    return lh::fail_arg("lh_gate_gemm_lstm_cell_f32: this product does not run fused "
+                        "(ask lh_gate_gemm_lstm_cell_plan first)");
+  // Other workgroups still read the operands while one writes its cells: the outputs must not
+  // overlap any X operand (c may be c_prev: a cell is read and written by one thread).
+  for (int s = 0; s < nseg; ++s) {
+    const float *x0 = segs[s].X, *x1 = x0 + (size_t)segs[s].ldx * B;
+    const float *outs[2] = {c, h};
+    for (const float *o : outs)
+      if (o < x1 && x0 < o + (size_t)H * B)
+        return lh::fail_arg("lh_gate_gemm_lstm_cell_f32: an output overlaps operand X of segment %d", s);
+  }
+  GemmArgs &g = p.g;
+  g.bias = bias4h;
+  g.colmask = mask01;
+  g.cell_H = H;
+  g.c_prev = c_prev;
+  g.c_out = c;
+  g.h_out = h;
+  g.cell_clip = cell_clip;
+  g.sigmoid_f64 = sigmoid_f64;
+  g.addend_col = addend_col;
+  g.addend_ncols = addend_ncols;
+  return launch_cell_index(p.config, g, lh::as_stream(stream));
 }
 
 extern "C" int lh_gemm_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,

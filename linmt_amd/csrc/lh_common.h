@@ -69,4 +69,33 @@ __device__ __forceinline__ T block_max(T v, T *lds) {
   return r;
 }
 
+// The LSTM cell at one (row, column): gates from the four pre-activations (bias included), the new
+// cell state (optionally clipped) and hidden state, both zeroed in padded columns (m = 0/1).
+// F64 evaluates the logistic function in double as the reference's feed-input kernels do
+// (src/deep_rnn_kernel.h:64-80).  Shared by the cell kernel and the matrix product that applies
+// the cell in its epilogue, so that both give the same bits.
+template <bool F64>
+__device__ __forceinline__ float sigmoid_ref(float x) {
+  if constexpr (F64) {
+    return (float)(1.0 / (1.0 + exp(-1.0 * (double)x)));
+  } else {
+    return 1.0f / (1.0f + expf(-1.0f * x));
+  }
+}
+template <bool F64>
+__device__ __forceinline__ void lstm_cell_point(float &s0, float &s1, float &s2, float &s3,
+                                                float c_prev, float m, float cell_clip, float &c,
+                                                float &h) {
+  const float it = sigmoid_ref<F64>(s0);
+  const float ft = sigmoid_ref<F64>(s1);
+  const float gt = tanhf(s2);
+  const float ot = sigmoid_ref<F64>(s3);
+  s0 = it, s1 = ft, s2 = gt, s3 = ot;
+  float ct = ft * c_prev + it * gt;
+  if (cell_clip > 0.f) ct = fminf(fmaxf(ct, -cell_clip), cell_clip);
+  const float ht = ot * tanhf(ct);
+  c = ct * m;
+  h = ht * m;
+}
+
 }  // namespace lh

@@ -36,15 +36,6 @@ struct Vec<1> {
   __device__ __forceinline__ void store(float *p) const { *p = v[0]; }
 };
 
-template <bool F64>
-__device__ __forceinline__ float sigmoid_ref(float x) {
-  if constexpr (F64) {
-    return (float)(1.0 / (1.0 + exp(-1.0 * (double)x)));
-  } else {
-    return 1.0f / (1.0f + expf(-1.0f * x));
-  }
-}
-
 template <int VW, bool F64>
 __global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(const CellFwdArgs a) {
   const int HQ = a.H / VW;
@@ -83,16 +74,8 @@ __global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(const CellFwdArgs a)
   Vec<VW> c, h;
 #pragma unroll
   for (int i = 0; i < VW; ++i) {
-    const float it = sigmoid_ref<F64>(s[0].v[i]);
-    const float ft = sigmoid_ref<F64>(s[1].v[i]);
-    const float gt = tanhf(s[2].v[i]);
-    const float ot = sigmoid_ref<F64>(s[3].v[i]);
-    s[0].v[i] = it; s[1].v[i] = ft; s[2].v[i] = gt; s[3].v[i] = ot;
-    float ct = ft * cp.v[i] + it * gt;
-    if (a.cell_clip > 0.f) ct = fminf(fmaxf(ct, -a.cell_clip), a.cell_clip);
-    const float ht = ot * tanhf(ct);
-    c.v[i] = ct * m;
-    h.v[i] = ht * m;
+    lh::lstm_cell_point<F64>(s[0].v[i], s[1].v[i], s[2].v[i], s[3].v[i], cp.v[i], m, a.cell_clip,
+                             c.v[i], h.v[i]);
   }
   if (a.gates) {
 #pragma unroll

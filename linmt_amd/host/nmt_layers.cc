@@ -223,6 +223,7 @@ void LstmNode::ForwardProp() {
   lh_gemm_seg segs[3];
   int nseg = 0;
   float beta = 0.f;
+  const float *x = nullptr;  // input operand of the product, when the input term is not an addend
   if (L.input_hoisted_) {
     // M*x of every step is already in pre_x_all_: this step only adds the recurrent products
     pre = p_device_pre_x_;
@@ -230,40 +231,62 @@ void LstmNode::ForwardProp() {
   } else if (folded) {
     // M*W[:,token] is a column of the precomputed 4H x V product
     if (L.mw_fold_dirty_) L.BuildEmbeddingFold();
+    beta = 1.f;
+  } else if (L.input_layer_mode_) {
+    const bool drop = M.apply_dropout_ && p_device_dropout_mask_;
+    ProfileScope ps(M.profiler_, kTagEmbedLookup, (drop ? 12.0 : 8.0) * L.input_size_ * B);
+    LhErrorWrapper(lh_embed_lookup_f32(L.p_device_w_.get(), L.input_size_, L.vocab_size_,
+                                       p_device_input_vocab_indices_, B,
+                                       drop ? p_device_dropout_mask_ : nullptr,
+                                       drop ? M.cfg_.dropout_rate_ : 1.f, p_device_sparse_lookup_, s),
+                   "LstmInputHiddenNode::ForwardPropGpu sparse lookup");
+    x = p_device_sparse_lookup_;
+  } else {
+    x = p_device_h_t_below_;
+  }
+  if (x) segs[nseg++] = {L.p_device_m_stack_.get(), 4 * H, x, L.input_size_, L.input_size_};
+  segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
+  if (feed) segs[nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
+  const bool drop_out = M.apply_dropout_ && L.out_dropout_;
+  const float cell_clip = M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f;
+
+  // Inference form (no gate values kept, no dropout): product and cell in ONE kernel whenever the
+  // product runs unsplit; the folded embedding table is then read by that kernel too.
+  if (!p_device_gates_ && !drop_out) {
+    int fusable = 0;
+    char name[160] = {0};
+    LhErrorWrapper(lh_gate_gemm_lstm_cell_plan(H, B, segs, nseg, beta != 0.f, M.gemm_ws_bytes_, &fusable,
+                                               name, sizeof(name)),
+                   "lh_gate_gemm_lstm_cell_plan");
+    if (fusable) {
+      double k = 0;
+      for (int i = 0; i < nseg; ++i) k += segs[i].K;
+      ProfileScope ps(M.profiler_, kTagGateGemm, name, 2.0 * 4 * H * (double)B * k);
+      LhErrorWrapper(lh_gate_gemm_lstm_cell_f32(
+                         H, B, segs, nseg, beta != 0.f ? (folded ? L.mw_fold_.get() : pre) : nullptr,
+                         4 * H, folded ? p_device_input_vocab_indices_ : nullptr,
+                         folded ? L.vocab_size_ : 0, L.p_device_b_stack_.get(), p_device_c_t_prev_,
+                         p_device_input_vocab_indices_01_, feed ? 1 : 0, cell_clip, p_device_c_t_,
+                         p_device_h_t_, M.gemm_ws_bytes_, s),
+                     "LstmNode::ForwardPropGpu gate product with cell");
+      return;
+    }
+  }
+  if (folded) {
     ProfileScope ps(M.profiler_, kTagEmbedLookup, 8.0 * 4 * H * B);
     LhErrorWrapper(lh_embed_lookup_f32(L.mw_fold_.get(), 4 * H, L.vocab_size_,
                                        p_device_input_vocab_indices_, B, nullptr, 1.f, pre, s),
                    "LstmInputHiddenNode::ForwardPropGpu folded lookup");
-    beta = 1.f;
-  } else {
-    const float *x = nullptr;
-    if (L.input_layer_mode_) {
-      const bool drop = M.apply_dropout_ && p_device_dropout_mask_;
-      ProfileScope ps(M.profiler_, kTagEmbedLookup, (drop ? 12.0 : 8.0) * L.input_size_ * B);
-      LhErrorWrapper(lh_embed_lookup_f32(L.p_device_w_.get(), L.input_size_, L.vocab_size_,
-                                         p_device_input_vocab_indices_, B,
-                                         drop ? p_device_dropout_mask_ : nullptr,
-                                         drop ? M.cfg_.dropout_rate_ : 1.f, p_device_sparse_lookup_, s),
-                     "LstmInputHiddenNode::ForwardPropGpu sparse lookup");
-      x = p_device_sparse_lookup_;
-    } else {
-      x = p_device_h_t_below_;
-    }
-    segs[nseg++] = {L.p_device_m_stack_.get(), 4 * H, x, L.input_size_, L.input_size_};
   }
-  segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
-  if (feed) segs[nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
   // a split product stays in partial planes: the cell kernel adds them up (no reduction pass)
   const float *addend[3];
   const int n_add = M.GemmAddends(kTagGateGemm, 4 * H, B, segs, nseg, beta, pre, 4 * H, addend,
                                   "LstmNode::ForwardPropGpu stacked gate product");
-  const bool drop_out = M.apply_dropout_ && L.out_dropout_;
   ProfileScope pc(M.profiler_, kTagLstmCell,
                   ((p_device_gates_ ? 44.0 : 28.0) + (drop_out ? 8.0 : 0.0) + 16.0 * (n_add - 1)) * H * B);
   LhErrorWrapper(lh_lstm_cell_fwd_f32(H, B, addend[0], addend[1], addend[2],
                                       L.p_device_b_stack_.get(), p_device_c_t_prev_,
-                                      p_device_input_vocab_indices_01_, feed ? 1 : 0,
-                                      M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f,
+                                      p_device_input_vocab_indices_01_, feed ? 1 : 0, cell_clip,
                                       p_device_gates_, p_device_c_t_, p_device_h_t_,
                                       drop_out ? p_device_out_dropout_mask_ : nullptr,
                                       drop_out ? M.cfg_.dropout_rate_ : 1.f,

@@ -131,6 +131,10 @@ class ProfileScope {
     for (int s = 0; s < nseg; ++s) k += segs[s].K;
     slot_ = p_.Begin(std::string(ProfileTagName(tag)) + "|" + name, 2.0 * M * (double)N * k);
   }
+  // Matrix product whose kernel instance the caller already knows.
+  ProfileScope(Profiler &p, int tag, const char *kernel_name, double flop) : p_(p), on_(p.Wants(tag)) {
+    if (on_) slot_ = p_.Begin(std::string(ProfileTagName(tag)) + "|" + kernel_name, flop);
+  }
   ~ProfileScope() noexcept(false) {
     if (on_) p_.End(slot_);
   }

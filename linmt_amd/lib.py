@@ -48,6 +48,11 @@ SIGNATURES = {
                                      C.c_int, C.POINTER(C.c_int), C.c_void_p]),
     "lh_gemm_kernel_name": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
                                       C.c_int, C.c_size_t, C.c_int, C.c_char_p, C.c_int]),
+    "lh_gate_gemm_lstm_cell_plan": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
+                                              C.c_size_t, C.POINTER(C.c_int), C.c_char_p, C.c_int]),
+    "lh_gate_gemm_lstm_cell_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, c_f32p,
+                                             C.c_int, c_i32p, C.c_int, c_f32p, c_f32p, c_i32p, C.c_int,
+                                             C.c_float, c_f32p, c_f32p, C.c_size_t, C.c_void_p]),
     "lh_gemm_set_config_override": (C.c_int, [C.c_int]),
     "lh_gemm_set_splits_override": (C.c_int, [C.c_int]),
     "lh_gemm_config_info": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int * 8)]),
@@ -200,6 +205,25 @@ def gemm_kernel_name(M, N, segs, transA=False, transX=False, workspace_bytes=0, 
     check(load().lh_gemm_kernel_name(M, N, _segs(segs), len(segs), int(transA), int(transX),
                                      workspace_bytes, max_planes, buf, 128), "lh_gemm_kernel_name")
     return buf.value.decode()
+
+
+def gate_gemm_lstm_cell_plan(H, B, segs, has_addend=False, workspace_bytes=0):
+    """(fusable, kernel instance name) for lh_gate_gemm_lstm_cell_f32 on this problem."""
+    f, buf = C.c_int(), C.create_string_buffer(128)
+    check(load().lh_gate_gemm_lstm_cell_plan(H, B, _segs(segs), len(segs), int(has_addend),
+                                             workspace_bytes, C.byref(f), buf, 128),
+          "lh_gate_gemm_lstm_cell_plan")
+    return bool(f.value), buf.value.decode()
+
+
+def gate_gemm_lstm_cell(H, B, segs, bias4h, c_prev, mask01, c, h, addend=None, ld_addend=0,
+                        addend_col=None, addend_ncols=0, sigmoid_f64=False, cell_clip=0.0, workspace_bytes=0,
+                        stream=None):
+    check(load().lh_gate_gemm_lstm_cell_f32(H, B, _segs(segs), len(segs), _ptr(addend), ld_addend,
+                                            _ptr(addend_col), addend_ncols, _ptr(bias4h), _ptr(c_prev),
+                                            _ptr(mask01), int(sigmoid_f64), cell_clip, _ptr(c),
+                                            _ptr(h), workspace_bytes, _stream(stream)),
+          "lh_gate_gemm_lstm_cell_f32")
 
 
 def gemm_planes(M, N, segs, C_out, ldc, workspace, max_planes, transA=False, transX=False, beta=0.0,

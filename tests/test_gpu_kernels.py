@@ -279,6 +279,90 @@ def test_lstm_cell_fwd(lh, orc, H, B, feed):
     assert_close(host(h, (H, B)), wh2, "h clip")
 
 
+def test_gate_gemm_with_the_cell_in_its_epilogue(lh, orc):
+    """lh_gate_gemm_lstm_cell_f32 for every tile configuration that can carry the cell: against the
+    oracle's cell on float64 pre-activations (tolerance), and bit for bit against the two-call
+    path (lh_gemm_planes_f32 + lh_lstm_cell_fwd_f32) under the same configuration.  Ragged H and B,
+    one to three K segments, the addend read straight or through a column index (the folded
+    embedding table), masked columns, in-place cell state, clip, double-precision logistic."""
+    rng = np.random.default_rng(31)
+    L = lh.load()
+    n_cfg = L.lh_gemm_set_config_override(-1)
+    cases = [  # H, B, Ks, addend: None / "plain" / "table", f64, clip
+        (100, 76, (100, 36), None, False, 0.0),
+        (36, 37, (68,), "plain", True, 0.0),
+        (72, 132, (20, 12, 136), "table", False, 0.5),
+        (248, 40, (64, 64), "table", True, 0.0),
+    ]
+    fused_runs = 0
+    try:
+        for cfg in range(n_cfg):
+            L.lh_gemm_set_config_override(cfg)
+            for H, B, Ks, addend, f64, clip in cases:
+                As = [uni(rng, 4 * H, K, s=0.3) for K in Ks]
+                Xs = [uni(rng, K, B) for K in Ks]
+                bias, c_prev = uni(rng, 4 * H, s=0.5), uni(rng, H, B)
+                mask = (rng.uniform(size=B) < 0.8).astype(np.int32)
+                segs = [(dev(A), 4 * H, dev(X), K, K) for A, X, K in zip(As, Xs, Ks)]
+                table = cols = add_np = None
+                ld, V = 4 * H, 0
+                if addend == "plain":
+                    add_np = uni(rng, 4 * H, B)
+                    table = dev(add_np)
+                elif addend == "table":
+                    V = 23
+                    full = uni(rng, 4 * H + 4, V)[: 4 * H + 4]      # leading dimension > 4H
+                    ld = 4 * H + 4
+                    cols_np = rng.integers(0, V, size=B).astype(np.int32)
+                    cols_np[0], cols_np[-1] = -3, V + 5          # clamped like the embedding lookup
+                    table, cols = dev(full), dev(cols_np)
+                    add_np = full[: 4 * H, np.clip(cols_np, 0, V - 1)]
+                ok, name = lh.gate_gemm_lstm_cell_plan(H, B, segs, has_addend=addend is not None)
+                what = f"config {cfg} H={H} B={B} K={Ks} addend={addend}: {name}"
+                if not ok:
+                    assert name == ""
+                    c = dev(c_prev)
+                    with pytest.raises(lh.LinmtHipError):
+                        lh.gate_gemm_lstm_cell(H, B, segs, dev(bias), c, dev(mask), c,
+                                               torch.empty(H * B, device="cuda"))
+                    continue
+                assert name.startswith("gate_gemm_cell_kernel<"), what
+                fused_runs += 1
+                c = dev(c_prev)                                      # in place
+                h = torch.full((H * B,), float("nan"), device="cuda")
+                lh.gate_gemm_lstm_cell(H, B, segs, dev(bias), c, dev(mask), c, h, addend=table,
+                                       ld_addend=ld if table is not None else 0, addend_col=cols,
+                                       addend_ncols=V, sigmoid_f64=f64, cell_clip=clip)
+                pre = sum(A.astype(np.float64) @ X for A, X in zip(As, Xs))
+                if add_np is not None:
+                    pre = pre + add_np
+                _, wc, wh = orc.lstm_cell_fwd(pre.astype(np.float32), bias, c_prev, mask, feed=f64, cell_clip=clip)
+                assert_close(host(c, (H, B)), wc, what + " c")
+                assert_close(host(h, (H, B)), wh, what + " h")
+                assert np.all(host(h, (H, B))[:, mask == 0] == 0), what
+                # the two-call path under the same configuration: the same bits
+                pre_buf = dev(add_np) if add_np is not None else torch.empty(4 * H * B, device="cuda")
+                S = lh.gemm_planes(4 * H, B, segs, pre_buf, 4 * H, torch.empty(16, device="cuda"),
+                                   2 if add_np is not None else 3, beta=1.0 if add_np is not None else 0.0)
+                assert S == 1, what
+                c2, h2 = dev(c_prev), torch.empty(H * B, device="cuda")
+                lh.lstm_cell_fwd(H, B, pre_buf, dev(bias), c2, dev(mask), c2, h2, cell_clip=clip,
+                                 sigmoid_f64=f64)
+                assert np.array_equal(host(c, (H, B)), host(c2, (H, B))), what + ": c differs from the two-call path"
+                assert np.array_equal(host(h, (H, B)), host(h2, (H, B))), what + ": h differs from the two-call path"
+    finally:
+        L.lh_gemm_set_config_override(-1)
+    assert fused_runs >= 4 * 15
+    # an output on top of an operand is refused
+    H, B, K = 32, 32, 32
+    A, X = dev(uni(rng, 4 * H, K)), dev(uni(rng, K, B))
+    ok, _ = lh.gate_gemm_lstm_cell_plan(H, B, [(A, 4 * H, X, K, K)])
+    if ok:
+        z, m = torch.zeros(4 * H * B, device="cuda"), torch.ones(B, dtype=torch.int32, device="cuda")
+        with pytest.raises(lh.LinmtHipError):
+            lh.gate_gemm_lstm_cell(H, B, [(A, 4 * H, X, K, K)], z, z, m, z, X)
+
+
 def _attn_case(rng, H, B, S, lens, n_cols=None):
     n_cols = n_cols or B
     hs = uni(rng, S, n_cols, H, s=0.9)          # [tau][col][H], like tanh-bounded states
