@@ -52,7 +52,7 @@ __global__ __launch_bounds__(kThreads) void attn_core_kernel(const AttnArgs a) {
   __shared__ float s_red[kWaves];
   __shared__ float s_scalar[2];
 
-  const int b = blockIdx.x;
+  const int b = lh::xcd_contiguous(blockIdx.x, gridDim.x);  // a sentence's columns on one XCD
   const int tid = threadIdx.x, wave = tid / lh::kWave, lane = tid % lh::kWave;
   const int H = a.H, B = a.B, W = a.W, D = a.D;
   const int len = a.batch_info[b];
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(kThreads) void attn_core_regs_kernel(const AttnArgs
   __shared__ int s_idx[WCAP];
   __shared__ float s_red[kWaves];
 
-  const int b = blockIdx.x;
+  const int b = lh::xcd_contiguous(blockIdx.x, gridDim.x);  // a sentence's columns on one XCD
   const int tid = threadIdx.x, wave = tid / lh::kWave, lane = tid % lh::kWave;
   const int H = a.H, B = a.B, W = a.W, D = a.D;
   const int len = a.batch_info[b];

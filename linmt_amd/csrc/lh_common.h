@@ -69,6 +69,15 @@ __device__ __forceinline__ T block_max(T v, T *lds) {
   return r;
 }
 
+// Workgroups of a launch are dealt to the 8 XCDs (each with its own L2) round-robin.  Maps a
+// workgroup id to a work item so that every XCD owns one contiguous range of the n items: items
+// that read the same data (the beam columns of a sentence) then share an L2.
+__device__ __forceinline__ int xcd_contiguous(int id, int n) {
+  const int xcd = id % 8, within = id / 8;
+  const int per = n / 8, rem = n % 8;
+  return xcd * per + (xcd < rem ? xcd : rem) + within;
+}
+
 // The LSTM cell at one (row, column): gates from the four pre-activations (bias included), the new
 // cell state (optionally clipped) and hidden state, both zeroed in padded columns (m = 0/1).
 // F64 evaluates the logistic function in double as the reference's feed-input kernels do
