@@ -235,6 +235,32 @@ int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_steps, const f
                          const int *mask01, float *p_t, float *sigma, int *indices, float *align,
                          float *cached_exp, float *ctx, int *viterbi, lh_stream_t stream);
 
+/* The same attention step over a PROJECTED memory, for decoding, where one sentence's encoder
+ * states serve every step of its beam: with score_mem = W_a * hs and ctx_mem = W_c1 * hs computed
+ * once per sentence (two plain lh_gemm_f32 calls over all source positions),
+ *   score_j = h_t . score_mem_j            (= (W_a^T h_t) . hs_j of AttentionNode::ForwardProp)
+ *   h~      = tanh(sum_j a_j ctx_mem_j + out_add + out_bias) * mask01
+ *           (= tanh(W_c1 c_t + W_c2 h_t + b) with out_add = W_c2 h_t, src/layer_attention.h:447-478),
+ * so the per-step products W_a^T h_t and W_c1 c_t are gone and the context vector never exists.
+ * tanh1 = tanh(W_p h_t) as in lh_attn_core_fwd_f32; tanh1, h_t and out_add are H x B with the given
+ * column strides (0 = H); the memories are addressed like hs there (mem_col = hs_col).  Everything
+ * else (p_t, sigma, indices, align, cached_exp, viterbi) is written exactly as
+ * lh_attn_core_fwd_f32 writes it.  Local-p only, window 2D+1 <= LH_ATTN_PROJECTED_MAX_WINDOW,
+ * H <= LH_ATTN_PROJECTED_MAX_H and a multiple of 4, 16-byte aligned operands: other cases use
+ * lh_attn_core_fwd_f32 and the two products.  No counterpart in the reference (an algebraic
+ * regrouping of its step). */
+#define LH_ATTN_PROJECTED_MAX_WINDOW 21
+#define LH_ATTN_PROJECTED_MAX_H 2048
+int lh_attn_core_projected_fwd_f32(int H, int B, int D, int hs_steps, const float *tanh1,
+                                   long long tanh1_col_stride, const float *v_p, const float *h_t,
+                                   long long h_t_col_stride, const float *score_mem,
+                                   const float *ctx_mem, long long mem_step_stride,
+                                   long long mem_col_stride, const int *mem_col,
+                                   const int *batch_info, const int *mask01, const float *out_add,
+                                   long long out_add_col_stride, const float *out_bias, float *p_t,
+                                   float *sigma, int *indices, float *align, float *cached_exp,
+                                   float *h_tild, int *viterbi, lh_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * a8 / a9. Vocabulary softmax and log-likelihood, one pass over the V x B logits.
  *

@@ -26,6 +26,14 @@ struct AttnArgs {
   int *indices;
   float *align, *cached_exp, *ctx;
   int *viterbi;
+  // Projected memory (register kernel only).  ctx_mem != NULL: the context sum runs over ctx_mem
+  // (laid out like hs) instead of hs.  out_add / out_bias != NULL are added to that sum (out_add
+  // per column, out_add_col_stride apart) and out_tanh applies tanh and the column mask: the
+  // output is then the attention layer's h~ rather than the context vector.
+  long long wa_col_stride;  // distance between columns of wa
+  const float *ctx_mem, *out_add, *out_bias;
+  long long out_add_col_stride;
+  int out_tanh;
 };
 
 template <bool VEC>
@@ -190,7 +198,7 @@ __global__ __launch_bounds__(kThreads) void attn_core_regs_kernel(const AttnArgs
   const int off = a.batch_info[B + b];
   const int m = a.mask01[b];
   const int col = a.hs_col ? a.hs_col[b] : b;
-  const float *wa = a.wa + (size_t)b * a.proj_col_stride;
+  const float *wa = a.wa + (size_t)b * a.wa_col_stride;
   const float *hs_c = a.hs + (size_t)col * a.col_stride;
 
   float p = 0.f;
@@ -255,6 +263,22 @@ __global__ __launch_bounds__(kThreads) void attn_core_regs_kernel(const AttnArgs
     sc = lh::wave_sum(sc);
     if (lane == 0) s_part[wave][j] = sc;
   }
+  if (a.ctx_mem) {
+    // the scores are done with the window: the same registers take the window of ctx_mem, whose
+    // loads fly while the scores are normalised
+    const float *cm = a.ctx_mem + (size_t)col * a.col_stride;
+#pragma unroll
+    for (int j = 0; j < WCAP; ++j) {
+      const int tau = s_tau[j];
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        h[j][q] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (tau >= 0 && row_ok[q])
+          h[j][q] = *reinterpret_cast<const float4 *>(cm + (size_t)tau * a.step_stride +
+                                                      (size_t)(tid + q * kThreads) * 4);
+      }
+    }
+  }
   __syncthreads();
   for (int j = tid; j < WCAP; j += kThreads) {
     float sc = s_part[0][j];
@@ -315,7 +339,22 @@ __global__ __launch_bounds__(kThreads) void attn_core_regs_kernel(const AttnArgs
       const float w = s_val[j];
       acc.x += w * h[j][q].x; acc.y += w * h[j][q].y; acc.z += w * h[j][q].z; acc.w += w * h[j][q].w;
     }
-    if (row_ok[q]) *reinterpret_cast<float4 *>(ctx + (size_t)(tid + q * kThreads) * 4) = acc;
+    if (!row_ok[q]) continue;
+    const size_t r = (size_t)(tid + q * kThreads) * 4;
+    if (a.out_add) {
+      const float4 t = *reinterpret_cast<const float4 *>(a.out_add + (size_t)b * a.out_add_col_stride + r);
+      acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+    }
+    if (a.out_bias) {
+      const float4 t = *reinterpret_cast<const float4 *>(a.out_bias + r);
+      acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+    }
+    if (a.out_tanh) {
+      const float mf = (float)m;
+      acc.x = tanhf(acc.x) * mf; acc.y = tanhf(acc.y) * mf;
+      acc.z = tanhf(acc.z) * mf; acc.w = tanhf(acc.w) * mf;
+    }
+    *reinterpret_cast<float4 *>(ctx + r) = acc;
   }
 }
 
@@ -347,7 +386,8 @@ extern "C" int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_ste
     return lh::fail_arg("lh_attn_core_fwd_f32: proj_col_stride %lld < H", proj_col_stride);
 
   AttnArgs a{H, B, D, W, tanh1, v_p, wa, hs, proj_col_stride, hs_step_stride, hs_col_stride, hs_steps, hs_col,
-             batch_info, mask01, p_t, sigma, indices, align, cached_exp, ctx, viterbi};
+             batch_info, mask01, p_t, sigma, indices, align, cached_exp, ctx, viterbi,
+             proj_col_stride, nullptr, nullptr, nullptr, 0, 0};
   const bool vec = H % 4 == 0 && lh::aligned16(wa) && lh::aligned16(hs) && lh::aligned16(ctx) &&
                    hs_step_stride % 4 == 0 && hs_col_stride % 4 == 0 && proj_col_stride % 4 == 0;
   hipStream_t st = lh::as_stream(stream);
@@ -358,4 +398,50 @@ extern "C" int lh_attn_core_fwd_f32(int H, int B, int D, int max_len, int hs_ste
   else if (vec) hipLaunchKernelGGL(attn_core_kernel<true>, dim3(B), dim3(kThreads), 0, st, a);
   else hipLaunchKernelGGL(attn_core_kernel<false>, dim3(B), dim3(kThreads), 0, st, a);
   return lh::check_launch("lh_attn_core_fwd_f32");
+}
+
+extern "C" int lh_attn_core_projected_fwd_f32(int H, int B, int D, int hs_steps, const float *tanh1,
+                                              long long tanh1_col_stride, const float *v_p,
+                                              const float *h_t, long long h_t_col_stride,
+                                              const float *score_mem, const float *ctx_mem,
+                                              long long mem_step_stride, long long mem_col_stride,
+                                              const int *mem_col, const int *batch_info,
+                                              const int *mask01, const float *out_add,
+                                              long long out_add_col_stride, const float *out_bias,
+                                              float *p_t, float *sigma, int *indices, float *align,
+                                              float *cached_exp, float *h_tild, int *viterbi,
+                                              lh_stream_t stream) {
+  if (H <= 0 || B <= 0 || hs_steps <= 0)
+    return lh::fail_arg("lh_attn_core_projected_fwd_f32: H=%d B=%d hs_steps=%d", H, B, hs_steps);
+  const int W = 2 * D + 1;
+  if (D < 0 || W > LH_ATTN_PROJECTED_MAX_WINDOW || H > LH_ATTN_PROJECTED_MAX_H || H % 4 != 0)
+    return lh::fail_arg("lh_attn_core_projected_fwd_f32: D=%d H=%d outside what the kernel holds in "
+                        "registers (window <= %d, H <= %d, H %% 4 == 0)", D, H,
+                        LH_ATTN_PROJECTED_MAX_WINDOW, LH_ATTN_PROJECTED_MAX_H);
+  if (!tanh1 || !v_p || !h_t || !score_mem || !ctx_mem || !batch_info || !mask01 || !out_add ||
+      !out_bias || !p_t || !sigma || !indices || !align || !cached_exp || !h_tild)
+    return lh::fail_arg("lh_attn_core_projected_fwd_f32: a required pointer is NULL");
+  if (tanh1_col_stride == 0) tanh1_col_stride = H;
+  if (h_t_col_stride == 0) h_t_col_stride = H;
+  if (out_add_col_stride == 0) out_add_col_stride = H;
+  if (tanh1_col_stride < H || h_t_col_stride < H || out_add_col_stride < H || mem_step_stride < 0 ||
+      mem_col_stride < 0)
+    return lh::fail_arg("lh_attn_core_projected_fwd_f32: a stride is too small");
+  if (!lh::aligned16(h_t) || !lh::aligned16(score_mem) || !lh::aligned16(ctx_mem) ||
+      !lh::aligned16(out_add) || !lh::aligned16(out_bias) || !lh::aligned16(h_tild) ||
+      h_t_col_stride % 4 != 0 || out_add_col_stride % 4 != 0 || mem_step_stride % 4 != 0 ||
+      mem_col_stride % 4 != 0)
+    return lh::fail_arg("lh_attn_core_projected_fwd_f32: operands must be 16-byte aligned with "
+                        "strides that are multiples of 4");
+  static_assert(LH_ATTN_PROJECTED_MAX_WINDOW == kRegsSlots && LH_ATTN_PROJECTED_MAX_H == 8 * kThreads,
+                "limits published in the header");
+  AttnArgs a{H, B, D, W, tanh1, v_p, h_t, score_mem, tanh1_col_stride, mem_step_stride, mem_col_stride,
+             hs_steps, mem_col, batch_info, mask01, p_t, sigma, indices, align, cached_exp, h_tild,
+             viterbi, h_t_col_stride, ctx_mem, out_add, out_bias, out_add_col_stride, 1};
+  hipStream_t st = lh::as_stream(stream);
+  if (H <= 4 * kThreads)
+    hipLaunchKernelGGL((attn_core_regs_kernel<1, kRegsSlots>), dim3(B), dim3(kThreads), 0, st, a);
+  else
+    hipLaunchKernelGGL((attn_core_regs_kernel<2, kRegsSlots>), dim3(B), dim3(kThreads), 0, st, a);
+  return lh::check_launch("lh_attn_core_projected_fwd_f32");
 }

@@ -244,6 +244,19 @@ class AttentionLayer {
   DeviceArray<float> p_device_w_pa_stack_, proj_out_;
   bool pa_stack_dirty_ = true;
   void BuildProjectionStack();
+  // Decoding: a sentence's encoder states serve every step of its beam, so the two products that
+  // involve them are taken out of the step.  Once per batch score_mem_ = W_a * hs and
+  // ctx_mem_ = W_c1 * hs over all source positions (laid out like the states); per step one
+  // product [W_p ; W_c2] (2H x H) * h_t and one kernel that scores against score_mem_, sums
+  // ctx_mem_ with the alignment weights and finishes h~ = tanh(. + W_c2 h_t + b).  The context
+  // vector itself is never formed.  Local-p attention with a window the kernel holds in registers.
+  DeviceArray<float> score_mem_, ctx_mem_, p_device_w_pc_stack_, pc_out_;
+  bool pc_stack_dirty_ = true;
+  bool projected_memory_ = false;  // the two memories hold this batch's states
+  bool ProjectedMemoryPossible() const;
+  // capacity = floats of the encoder's state slab (the memories are allocated once, that large)
+  void BuildProjectedMemory(int source_length, size_t capacity);
+  void BuildOutputStack();
 
   // ---- training --------------------------------------------------------------------------------
   DeviceArray<float> p_device_w_a_grad_, p_device_w_p_grad_, p_device_v_p_grad_,

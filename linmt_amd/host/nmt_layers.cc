@@ -1,5 +1,7 @@
 // LSTM, attention and softmax layer classes: parameter storage and the per-node forward bodies,
 // each a short ordered list of launches into liblinmt_hip.so on the model's single stream.
+#include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 #include "nmt.h"
@@ -403,6 +405,7 @@ void AttentionLayer::PreprocessMinibatchInformation(const int *p_host_batch_info
 bool AttentionLayer::SetParam(const std::string &name, const float *host, size_t n) {
   hipStream_t s = p_neural_mt_->stream_;
   if (name == "W_a" || name == "W_p") pa_stack_dirty_ = true;
+  if (name == "W_p" || name == "W_c2") pc_stack_dirty_ = true;
   if (name == "W_a") return SetFlat(p_device_w_a_, host, n, s);
   if (name == "W_p") return SetFlat(p_device_w_p_, host, n, s);
   if (name == "v_p") return SetFlat(p_device_v_p_, host, n, s);
@@ -432,6 +435,55 @@ void AttentionLayer::BuildProjectionStack() {
   pa_stack_dirty_ = false;
 }
 
+bool AttentionLayer::ProjectedMemoryPossible() const {
+  return use_hs_col_ && !global_mode_ && !p_neural_mt_->cfg_.train_mode_ &&
+         window_ <= LH_ATTN_PROJECTED_MAX_WINDOW && lstm_size_ <= LH_ATTN_PROJECTED_MAX_H &&
+         lstm_size_ % 4 == 0 && hs_col_stride_ == lstm_size_ && hs_step_stride_ % lstm_size_ == 0 &&
+         !std::getenv("LINMT_NO_PROJECTED_MEMORY");  // measurement aid: the step's own products
+}
+
+void AttentionLayer::BuildOutputStack() {
+  const size_t H = lstm_size_;
+  hipStream_t s = p_neural_mt_->stream_;
+  std::vector<float> wp, wc2, stack(2 * H * H);
+  if (!GetFlat(p_device_w_p_, &wp, s) || !GetFlat(p_device_w_c_p2_, &wc2, s))
+    throw LinmtError("AttentionLayer::BuildOutputStack: cannot read W_p / W_c2");
+  for (size_t k = 0; k < H; ++k) {  // column k of the 2H x H stack: W_p above W_c2
+    std::copy(wp.begin() + k * H, wp.begin() + (k + 1) * H, stack.begin() + k * 2 * H);
+    std::copy(wc2.begin() + k * H, wc2.begin() + (k + 1) * H, stack.begin() + k * 2 * H + H);
+  }
+  if (p_device_w_pc_stack_.size() == 0) {
+    p_device_w_pc_stack_.Alloc(2 * H * H);
+    pc_out_.Alloc(2 * H * (size_t)minibatch_size_);
+  }
+  p_device_w_pc_stack_.Upload(stack.data(), stack.size(), s);
+  HipErrorWrapper(hipStreamSynchronize(s), "output stack upload failed");  // `stack` is a local
+  pc_stack_dirty_ = false;
+}
+
+// W_a * hs and W_c1 * hs for the source_length timesteps the encoder has just written, every
+// allocated column (columns beyond the batch hold older, finite states nobody reads).
+void AttentionLayer::BuildProjectedMemory(int source_length, size_t capacity) {
+  projected_memory_ = false;
+  if (!ProjectedMemoryPossible()) return;
+  const int H = lstm_size_;
+  const long long cols = hs_step_stride_ / H * source_length;
+  if ((size_t)cols * H > capacity)
+    throw LinmtError("AttentionLayer::BuildProjectedMemory: more states than the encoder holds");
+  if (score_mem_.size() < capacity) {
+    score_mem_.Alloc(capacity);
+    ctx_mem_.Alloc(capacity);
+  }
+  NeuralMachineTranslation &M = *p_neural_mt_;
+  lh_gemm_seg sa{p_device_w_a_.get(), H, p_device_total_hs_, H, H};
+  M.Gemm(kTagAttnProjGemm, H, (int)cols, &sa, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
+         score_mem_.get(), H, "AttentionLayer::BuildProjectedMemory W_a hs");
+  lh_gemm_seg sc{p_device_w_c_p1_.get(), H, p_device_total_hs_, H, H};
+  M.Gemm(kTagAttnOutGemm, H, (int)cols, &sc, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
+         ctx_mem_.get(), H, "AttentionLayer::BuildProjectedMemory W_c1 hs");
+  projected_memory_ = true;
+}
+
 bool AttentionLayer::GetParam(const std::string &name, std::vector<float> *out) {
   hipStream_t s = p_neural_mt_->stream_;
   if (name == "W_a") return GetFlat(p_device_w_a_, out, s);
@@ -454,6 +506,24 @@ void AttentionNode::ForwardProp() {
   Profiler &prof = A.p_neural_mt_->profiler_;
   const float *tanh1 = p_device_tanh_1_, *wa = p_device_h_t_wa_cache_;
   long long proj_col_stride = H;
+  if (A.projected_memory_) {
+    // decoding over the projected memory: one product, one kernel, h~ out
+    if (A.pc_stack_dirty_) A.BuildOutputStack();
+    lh_gemm_seg seg{A.p_device_w_pc_stack_.get(), 2 * H, ha, H, H};
+    A.p_neural_mt_->Gemm(kTagAttnProjGemm, 2 * H, B, &seg, 1, 0, 0, 0.f, nullptr, LH_ACT_TANH, nullptr,
+                         A.pc_out_.get(), 2 * H, "AttentionNode::ForwardProp [W_p ; W_c2] h_t", H);
+    ProfileScope ps(prof, kTagAttnCore, 4.0 * B * (2.0 * A.window_ * H + 4.0 * H + 2.0 * A.window_));
+    LhErrorWrapper(lh_attn_core_projected_fwd_f32(
+                       H, B, A.d_, A.hs_steps_, A.pc_out_.get(), 2 * H, A.p_device_v_p_.get(), ha, H,
+                       A.score_mem_.get(), A.ctx_mem_.get(), A.hs_step_stride_, A.hs_col_stride_,
+                       A.p_device_hs_col_.get(), A.p_device_batch_information_.get(),
+                       p_device_indices_mask_, A.pc_out_.get() + H, 2 * H,
+                       A.p_device_output_bias_.get(), p_device_p_t_, p_device_sigma_1_,
+                       p_device_indices_, p_device_alignments_, p_device_cached_exp_,
+                       p_device_final_tmp_2_, nullptr, s),
+                   "AttentionNode::ForwardProp attention over the projected memory");
+    return;
+  }
   if (!A.global_mode_ && !A.p_neural_mt_->cfg_.train_mode_) {
     if (A.pa_stack_dirty_) A.BuildProjectionStack();
     lh_gemm_seg seg{A.p_device_w_pa_stack_.get(), 2 * H, ha, H, H};

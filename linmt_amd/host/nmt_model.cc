@@ -236,6 +236,7 @@ void NeuralMachineTranslation::ForwardTeacherForced(const int *p_host_source, in
     // the batch information is uploaded for B columns: lengths at [0,B), offsets at [B,2B)
     attention_layer_.hs_step_stride_ = (long long)cfg_.lstm_size_ * SourceLayer(L - 1).minibatch_size_;
     attention_layer_.hs_steps_ = source_length;
+    attention_layer_.projected_memory_ = false;  // a decoding batch's memory is not this pass's
   }
   softmax_layer_.p_device_loss_.Zero(stream_);
 
@@ -388,7 +389,7 @@ void NeuralMachineTranslation::ForwardPropSource(const int *p_host_source, int s
 // one layer at a time: the layer's input products for all steps in one GEMM, then the recurrence.
 void NeuralMachineTranslation::RunSourceSide(int source_length, int B) {
   const int L = cfg_.num_layers_;
-  static const bool lanes_off = getenv("LINMT_NO_LANES") != nullptr;  // measurement aid
+  const bool lanes_off = getenv("LINMT_NO_LANES") != nullptr;  // measurement and test aid
   bool lanes = !lanes_off && decode_mode_ && L > 1 && L <= 4 && profiler_.level_ < 2 &&
                source_length > kLaneChunkSteps;
   for (int l = 0; l < L && lanes; ++l)
@@ -634,6 +635,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   if (n != n_sent_ && cfg_.attention_mode_)
     attention_layer_.hs_step_stride_ = (long long)H * n_sent_;
   ForwardPropSource(src.data(), S, n);
+  if (cfg_.attention_mode_) attention_layer_.BuildProjectedMemory(S, SourceLayer(L - 1).h_all_.size());
 
   // TransferDecodingStatesGpu (layer_input_to_hidden.h:1536-1545): encoder's final (h, c) of layer
   // l, sentence s -> every beam column of s.

@@ -53,6 +53,11 @@ SIGNATURES = {
     "lh_gate_gemm_lstm_cell_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, c_f32p,
                                              C.c_int, c_i32p, C.c_int, c_f32p, c_f32p, c_i32p, C.c_int,
                                              C.c_float, c_f32p, c_f32p, C.c_size_t, C.c_void_p]),
+    "lh_attn_core_projected_fwd_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, c_f32p,
+                                                 C.c_longlong, c_f32p, c_f32p, C.c_longlong, c_f32p,
+                                                 c_f32p, C.c_longlong, C.c_longlong, c_i32p, c_i32p,
+                                                 c_i32p, c_f32p, C.c_longlong, c_f32p, c_f32p, c_f32p,
+                                                 c_i32p, c_f32p, c_f32p, c_f32p, c_i32p, C.c_void_p]),
     "lh_gemm_set_config_override": (C.c_int, [C.c_int]),
     "lh_gemm_set_splits_override": (C.c_int, [C.c_int]),
     "lh_gemm_config_info": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int * 8)]),
@@ -205,6 +210,18 @@ def gemm_kernel_name(M, N, segs, transA=False, transX=False, workspace_bytes=0, 
     check(load().lh_gemm_kernel_name(M, N, _segs(segs), len(segs), int(transA), int(transX),
                                      workspace_bytes, max_planes, buf, 128), "lh_gemm_kernel_name")
     return buf.value.decode()
+
+
+def attn_core_projected_fwd(H, B, D, hs_steps, tanh1, tanh1_col_stride, v_p, h_t, h_t_col_stride,
+                            score_mem, ctx_mem, mem_step_stride, mem_col_stride, mem_col, batch_info,
+                            mask01, out_add, out_add_col_stride, out_bias, p_t, sigma, indices, align,
+                            cached_exp, h_tild, viterbi=None, stream=None):
+    check(load().lh_attn_core_projected_fwd_f32(
+        H, B, D, hs_steps, _ptr(tanh1), tanh1_col_stride, _ptr(v_p), _ptr(h_t), h_t_col_stride,
+        _ptr(score_mem), _ptr(ctx_mem), mem_step_stride, mem_col_stride, _ptr(mem_col),
+        _ptr(batch_info), _ptr(mask01), _ptr(out_add), out_add_col_stride, _ptr(out_bias), _ptr(p_t),
+        _ptr(sigma), _ptr(indices), _ptr(align), _ptr(cached_exp), _ptr(h_tild), _ptr(viterbi),
+        _stream(stream)), "lh_attn_core_projected_fwd_f32")
 
 
 def gate_gemm_lstm_cell_plan(H, B, segs, has_addend=False, workspace_bytes=0):

@@ -449,6 +449,63 @@ def test_attn_core_shared_sentence_states(lh, orc):
     assert_close(got["ctx"][:, same], want["ctx"][:, same], "context")
 
 
+@pytest.mark.parametrize("H,n_sent,beam,S,D", [(1000, 8, 12, 60, 10), (2000, 3, 4, 30, 10), (64, 5, 3, 17, 2)])
+def test_attn_core_over_projected_memory(lh, orc, H, n_sent, beam, S, D):
+    """lh_attn_core_projected_fwd_f32: scores against W_a*hs, context sum over W_c1*hs, h~ out.
+    Expected values from the oracle's attention step on the plain memory (with W_a^T h_t as its
+    score operand) followed by tanh(W_c1 c_t + W_c2 h_t + b) in float64 -- the reference's order of
+    operations (src/layer_attention.h:243-483), which the regrouped kernel has to reproduce."""
+    rng = np.random.default_rng(33)
+    B = n_sent * beam
+    lens_s = rng.integers(max(1, S // 4), S + 1, size=n_sent)
+    lens_s[0] = S
+    lens = np.repeat(lens_s, beam).astype(np.int32)
+    hs_col = np.repeat(np.arange(n_sent), beam).astype(np.int32)
+    bi = np.concatenate([lens, S - lens]).astype(np.int32)
+    mask = (rng.uniform(size=B) < 0.9).astype(np.int32)
+    hs = uni(rng, S, n_sent, H, s=0.9)
+    sc = 1.0 / np.sqrt(H)
+    W_a, W_c1, W_c2 = (uni(rng, H, H, s=2 * sc) for _ in range(3))
+    W_p, v_p, b_out = uni(rng, H, H, s=2 * sc), uni(rng, H, s=0.3), uni(rng, H, s=0.2)
+    h_t = uni(rng, H, B, s=0.9)
+    f64 = np.float64
+    tanh1 = np.tanh(W_p.astype(f64) @ h_t).astype(np.float32)
+    wa = (W_a.astype(f64).T @ h_t).astype(np.float32)
+    want = orc.attn_core_fwd(H, B, D, 0, S, tanh1, v_p, wa, hs, n_sent * H, H, hs_col, bi, mask)
+    want_ht = np.tanh(W_c1.astype(f64) @ want["ctx"] + W_c2.astype(f64) @ h_t + b_out[:, None]) * mask
+    score_mem = (hs.astype(f64) @ W_a.astype(f64).T).astype(np.float32)    # [tau][col][H] = W_a hs
+    ctx_mem = (hs.astype(f64) @ W_c1.astype(f64).T).astype(np.float32)
+    # tanh1 and W_c2 h_t as the halves of one stacked 2H x B product, as the decoder hands them over
+    both = dev(np.concatenate([tanh1, (W_c2.astype(f64) @ h_t).astype(np.float32)], axis=0))
+    W = 2 * D + 1
+    o = dict(p_t=torch.zeros(B, device="cuda"), sigma=torch.zeros(B, device="cuda"),
+             indices=torch.empty(B * W, dtype=torch.int32, device="cuda"),
+             align=torch.empty(B * W, device="cuda"), cached_exp=torch.empty(B * W, device="cuda"),
+             h_tild=torch.full((H * B,), float("nan"), device="cuda"),
+             viterbi=torch.empty(B, dtype=torch.int32, device="cuda"))
+    lh.attn_core_projected_fwd(H, B, D, S, both, 2 * H, dev(v_p), dev(h_t), H,
+                               torch.from_numpy(score_mem).cuda(), torch.from_numpy(ctx_mem).cuda(),
+                               n_sent * H, H, dev(hs_col), dev(bi), dev(mask), both[H:], 2 * H,
+                               dev(b_out), o["p_t"], o["sigma"], o["indices"], o["align"],
+                               o["cached_exp"], o["h_tild"], o["viterbi"])
+    got_p = host(o["p_t"], (B,))
+    assert_close(got_p, want["p_t"], "p_t")
+    same = got_p.astype(np.int64) == want["p_t"].astype(np.int64)
+    assert same.mean() > 0.95
+    assert np.array_equal(host(o["indices"], (B, W))[same], want["indices"][same])
+    assert np.array_equal(host(o["viterbi"], (B,))[same], want["viterbi"][same])
+    assert_close(host(o["align"], (B, W))[same], want["align"][same], "alignments")
+    got_ht = host(o["h_tild"], (H, B))
+    assert_close(got_ht[:, same], want_ht[:, same], "h~", rtol=2e-4, atol=2e-5)
+    assert np.all(got_ht[:, mask == 0] == 0)
+    with pytest.raises(lh.LinmtHipError):   # a window the registers do not hold
+        lh.attn_core_projected_fwd(H, B, 11, S, both, 2 * H, dev(v_p), dev(h_t), H,
+                                   torch.from_numpy(score_mem).cuda(), torch.from_numpy(ctx_mem).cuda(),
+                                   n_sent * H, H, dev(hs_col), dev(bi), dev(mask), both[H:], 2 * H,
+                                   dev(b_out), o["p_t"], o["sigma"], o["indices"], o["align"],
+                                   o["cached_exp"], o["h_tild"], o["viterbi"])
+
+
 def test_attn_core_global(lh, orc):
     rng = np.random.default_rng(7)
     H, B, S = 1000, 128, 50

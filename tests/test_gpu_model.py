@@ -140,6 +140,31 @@ def test_decode_config3_architecture(orc, host):
     gm.close()
 
 
+def test_decode_same_with_and_without_the_regrouped_step(orc, host, monkeypatch):
+    """Decoding regroups the step (encoder lanes; gate product with the cell in its epilogue;
+    attention over W_a*hs / W_c1*hs computed once per batch).  With the switches that turn the
+    lanes and the projected memory off, the plain step must give the same translations, with
+    scores inside the floating-point tolerance, and both must match the oracle."""
+    rng = np.random.default_rng(16)
+    layers, H, Vs, Vt, D, beam = 3, 96, 200, 260, 4, 6
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 40, 0.35, decoding=(5, beam))
+    sents = [rng.integers(0, Vs, size=n) for n in (17, 9, 12, 3, 21)]
+    fast = gm.decode_batch(sents, beam=beam, with_hyps=True, alignments=True)
+    monkeypatch.setenv("LINMT_NO_PROJECTED_MEMORY", "1")
+    monkeypatch.setenv("LINMT_NO_LANES", "1")
+    plain = gm.decode_batch(sents, beam=beam, with_hyps=True, alignments=True)
+    monkeypatch.delenv("LINMT_NO_PROJECTED_MEMORY")
+    monkeypatch.delenv("LINMT_NO_LANES")
+    for i, (a, b) in enumerate(zip(fast, plain)):
+        assert a["best"].tolist() == b["best"].tolist(), i
+        assert a["best_viterbi"].tolist() == b["best_viterbi"].tolist(), i
+        assert np.isclose(a["best_score"], b["best_score"], rtol=1e-4, atol=1e-5), i
+        assert a["n_hyp"] == b["n_hyp"], i
+        _compare_decode(om.decode_sentence(sents[i], beam=beam, alignments=True), a,
+                        f"regrouped step, sentence {i}")
+    gm.close()
+
+
 def _ragged_minibatch(rng, B, S, T, Vs, Vt, min_len=1):
     lens_s = rng.integers(min_len, S + 1, size=B)
     lens_t = rng.integers(max(min_len, 2), T + 1, size=B)
