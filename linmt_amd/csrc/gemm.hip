@@ -495,6 +495,12 @@ constexpr int smem2_floats() {
               (WK - 1) * BM * BN);
 }
 
+// The rare paths of the K loop (a new K segment, a short last slab) are a few dozen selects each.
+// Left alone the compiler turns those branches into straight-line selects that every iteration
+// executes, and vector ALU instructions take issue time from the matrix pipe; an empty statement
+// the optimiser must keep makes each of them a real, normally untaken, branch.
+#define LH_KEEP_BRANCH() asm volatile("" ::: "memory")
+
 // CELL: the rows of a tile are BM/4 rows of each LSTM gate and the epilogue is the LSTM cell.
 template <int BM, int BN, int WM, int WN, int WK, int BK, bool TA, bool TX, bool CELL>
 __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
@@ -575,6 +581,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
     const int lx = lseg == 0 ? ldx0 : (lseg == 1 ? ldx1 : ldx2);                     \
     const int Ks = lseg == 0 ? K0 : (lseg == 1 ? K1 : K2);                           \
     if (new_seg) {                                                                   \
+      LH_KEEP_BRANCH();                                                              \
       if constexpr (CELL) sa.set_ld_gates(la, tid, g.cell_H, g.cell_H - m0);         \
       else sa.set_ld(la, tid, M - m0);                                               \
       sx.set_ld(lx, tid, N - n0);                                                    \
@@ -583,6 +590,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
     const float *px = !TX ? Xb + (size_t)n0 * lx + lk0 : Xb + (size_t)lk0 * lx + n0; \
     tail = Ks - lk0 < BK;                                                            \
     if (tail) {                                                                      \
+      LH_KEEP_BRANCH();                                                              \
       sa.clamp_tail(tid, Ks - lk0);                                                  \
       sx.clamp_tail(tid, Ks - lk0);                                                  \
     }                                                                                \
@@ -599,6 +607,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
   do {                        \
     float *sb = (BUF);        \
     if (tail) {               \
+      LH_KEEP_BRANCH();       \
       sa.zero_tail();         \
       sx.zero_tail();         \
     }                         \
@@ -615,40 +624,68 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
   if (total > 1) LH_ISSUE();
   __syncthreads();
   int cur = 0;  // float offset of the slab buffer being consumed
+  // Fragments are read one group (8 k) ahead of the MFMAs that use them.  Deep slabs (one
+  // workgroup per CU, nobody else to cover a stall) keep that up across slab boundaries: the
+  // barrier that releases a slab sits BEFORE the MFMAs of its last group, whose fragments are in
+  // registers by then, and the first group of the next slab is read right behind it, under those
+  // MFMAs.  Shallow slabs run several workgroups per CU, which hide the one exposed read per slab
+  // better than the dozen registers the carried fragments cost would (they lower the occupancy).
+  constexpr bool kCarry = BK >= 64 && NG % 2 == 0;
+  float fa[2][FM][4], fx[2][FN][4];
+  if constexpr (kCarry) {
+#pragma unroll
+    for (int b = 0; b < FM; ++b) SA::read_frag(smem + fa_off, 0, b, fa[0][b]);
+#pragma unroll
+    for (int a = 0; a < FN; ++a) SX::read_frag(smem + fx_off, 0, a, fx[0][a]);
+  }
   for (int s = 0; s < total; ++s) {
     if (s + 1 < total) LH_STASH(smem + (kSlab - cur));
     if (s + 2 < total) LH_ISSUE();
-    {
-      const float *as = smem + cur + fa_off;
-      const float *xs = smem + cur + fx_off;
-      float fa[2][FM][4], fx[2][FN][4];
+    const float *as = smem + cur + fa_off;
+    const float *xs = smem + cur + fx_off;
+    if constexpr (!kCarry) {
 #pragma unroll
       for (int b = 0; b < FM; ++b) SA::read_frag(as, 0, b, fa[0][b]);
 #pragma unroll
       for (int a = 0; a < FN; ++a) SX::read_frag(xs, 0, a, fx[0][a]);
-#pragma unroll
-      for (int grp = 0; grp < NG; ++grp) {
-        const int c = grp & 1, n = c ^ 1;
-        if (grp + 1 < NG) {
-#pragma unroll
-          for (int b = 0; b < FM; ++b) SA::read_frag(as, grp + 1, b, fa[n][b]);
-#pragma unroll
-          for (int a = 0; a < FN; ++a) SX::read_frag(xs, grp + 1, a, fx[n][a]);
-        }
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-          for (int a = 0; a < FN; ++a)
-#pragma unroll
-            for (int b = 0; b < FM; ++b)
-              // operands swapped on purpose: the transposed product puts consecutive m in
-              // consecutive lanes of every accumulator register
-              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fx[c][a][q], fa[c][b][q],
-                                                               acc[a][b], 0, 0, 0);
-      }
     }
-    __syncthreads();
-    cur = kSlab - cur;
+#pragma unroll
+    for (int grp = 0; grp < NG; ++grp) {
+      const int c = grp & 1, n = c ^ 1;
+      if (grp + 1 < NG) {
+#pragma unroll
+        for (int b = 0; b < FM; ++b) SA::read_frag(as, grp + 1, b, fa[n][b]);
+#pragma unroll
+        for (int a = 0; a < FN; ++a) SX::read_frag(xs, grp + 1, a, fx[n][a]);
+      } else if constexpr (kCarry) {
+        // nothing moves across: the MFMAs of the groups before stay ahead of the barrier, where
+        // they cover the latency of the fragment reads the barrier has to wait for
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        cur = kSlab - cur;
+        if (s + 1 < total) {
+#pragma unroll
+          for (int b = 0; b < FM; ++b) SA::read_frag(smem + cur + fa_off, 0, b, fa[n][b]);
+#pragma unroll
+          for (int a = 0; a < FN; ++a) SX::read_frag(smem + cur + fx_off, 0, a, fx[n][a]);
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int a = 0; a < FN; ++a)
+#pragma unroll
+          for (int b = 0; b < FM; ++b)
+            // operands swapped on purpose: the transposed product puts consecutive m in
+            // consecutive lanes of every accumulator register
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fx[c][a][q], fa[c][b][q],
+                                                             acc[a][b], 0, 0, 0);
+    }
+    if constexpr (!kCarry) {
+      __syncthreads();
+      cur = kSlab - cur;
+    }
   }
 #undef LH_ISSUE
 #undef LH_STASH
