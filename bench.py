@@ -4,7 +4,10 @@
 
 One "step" = one pass of the hot path over one batch: a full batched beam search (encoder, every
 decoder step with on-device top-k / merge / state gather, hypothesis read-back) over 64 synthetic
-source sentences.  Prints ONE JSON line (see README / DESIGN.md for the fields).
+source sentences.  Prints ONE JSON line: metric / value / unit (whole-job target tokens per second,
+inputs resident on the device), ms_per_step, the workload in `config`, `roofline` for the dominant
+kernel (live HIP-event timing of its launches against the fp32 MFMA peak, measured HBM traffic),
+`cpu_baseline` (the CPU restatement on the host cores, same sentences) and `parity` (1-best of both).
 
   python bench.py --gpus 1 --steps K --warmup W
 
