@@ -407,6 +407,8 @@ struct Stage {
   static constexpr int kFloats = KC ? KQ * LDQ * 4 : BK * LDD;
   static constexpr int kUnits = KQ * BD;  // 16-byte units in a slab
   static constexpr int NU = (kUnits + NT - 1) / NT;
+  // every thread owns NU whole units: no per-unit guard (and no exec-mask bookkeeping in the K loop)
+  static constexpr bool kExact = kUnits % NT == 0;
   static_assert(NU <= 32, "validity mask is 32 bits");
   static_assert(BD % 16 == 0 && BK % 16 == 0, "tile extents");
 
@@ -458,7 +460,7 @@ struct Stage {
     const char *b = reinterpret_cast<const char *>(base);
 #pragma unroll
     for (int i = 0; i < NU; ++i)
-      if (tid + i * NT < kUnits) v[i] = *reinterpret_cast<const float4 *>(b + goff[i]);
+      if (kExact || tid + i * NT < kUnits) v[i] = *reinterpret_cast<const float4 *>(b + goff[i]);
   }
   __device__ __forceinline__ void zero_tail() {
 #pragma unroll
@@ -468,7 +470,7 @@ struct Stage {
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int u = tid + i * NT;
-      if (u < kUnits) *reinterpret_cast<float4 *>(buf + unit_lds(u)) = v[i];
+      if (kExact || u < kUnits) *reinterpret_cast<float4 *>(buf + unit_lds(u)) = v[i];
     }
   }
   // Fragment reads.  origin = float offset for (first k of the wavefront's share, lane half, row d).
@@ -571,37 +573,50 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
     }
   }
   lk0 *= BK;
-  bool new_seg = true;  // the per-thread offsets must be rebuilt for the segment's leading dimension
+  // The K loop's scalar work is a few additions: the origin of the next slab in each operand
+  // advances by a fixed step, and everything that depends on the segment (base pointers, leading
+  // dimensions, the per-thread offsets) is set up only when a segment begins.  Both wavefronts of
+  // a SIMD run this code at the same time, right behind the barrier, so every scalar instruction
+  // here is time the matrix pipe stands still.
+  bool new_seg = true;  // the next slab opens a segment (or the first one of this share)
   bool tail = false;    // the slab in the staging registers ends its segment short of BK
-#define LH_ISSUE()                                                                   \
-  do {                                                                               \
-    const float *Ab = lseg == 0 ? A0 : (lseg == 1 ? A1 : A2);                        \
-    const float *Xb = lseg == 0 ? X0 : (lseg == 1 ? X1 : X2);                        \
-    const int la = lseg == 0 ? lda0 : (lseg == 1 ? lda1 : lda2);                     \
-    const int lx = lseg == 0 ? ldx0 : (lseg == 1 ? ldx1 : ldx2);                     \
-    const int Ks = lseg == 0 ? K0 : (lseg == 1 ? K1 : K2);                           \
-    if (new_seg) {                                                                   \
-      LH_KEEP_BRANCH();                                                              \
-      if constexpr (CELL) sa.set_ld_gates(la, tid, g.cell_H, g.cell_H - m0);         \
-      else sa.set_ld(la, tid, M - m0);                                               \
-      sx.set_ld(lx, tid, N - n0);                                                    \
-    }                                                                                \
-    const float *pa = TA ? Ab + (size_t)m0 * la + lk0 : Ab + (size_t)lk0 * la + m0;  \
-    const float *px = !TX ? Xb + (size_t)n0 * lx + lk0 : Xb + (size_t)lk0 * lx + n0; \
-    tail = Ks - lk0 < BK;                                                            \
-    if (tail) {                                                                      \
-      LH_KEEP_BRANCH();                                                              \
-      sa.clamp_tail(tid, Ks - lk0);                                                  \
-      sx.clamp_tail(tid, Ks - lk0);                                                  \
-    }                                                                                \
-    sa.load(pa, tid);                                                                \
-    sx.load(px, tid);                                                                \
-    lk0 += BK;                                                                       \
-    new_seg = tail || lk0 >= Ks; /* a clamped tail also dirtied the offsets */       \
-    if (lk0 >= Ks) {                                                                 \
-      ++lseg;                                                                        \
-      lk0 = 0;                                                                       \
-    }                                                                                \
+  const float *pa = nullptr, *px = nullptr;  // origin of the next slab inside A / X
+  int step_a = 0, step_x = 0;                // floats from one slab to the next
+  int kleft = 0;                             // k values of the segment not yet loaded
+#define LH_ISSUE()                                                                 \
+  do {                                                                             \
+    if (new_seg) {                                                                 \
+      LH_KEEP_BRANCH();                                                            \
+      const float *Ab = lseg == 0 ? A0 : (lseg == 1 ? A1 : A2);                    \
+      const float *Xb = lseg == 0 ? X0 : (lseg == 1 ? X1 : X2);                    \
+      const int la = lseg == 0 ? lda0 : (lseg == 1 ? lda1 : lda2);                 \
+      const int lx = lseg == 0 ? ldx0 : (lseg == 1 ? ldx1 : ldx2);                 \
+      const int Ks = lseg == 0 ? K0 : (lseg == 1 ? K1 : K2);                       \
+      if constexpr (CELL) sa.set_ld_gates(la, tid, g.cell_H, g.cell_H - m0);       \
+      else sa.set_ld(la, tid, M - m0);                                             \
+      sx.set_ld(lx, tid, N - n0);                                                  \
+      pa = TA ? Ab + (size_t)m0 * la + lk0 : Ab + (size_t)lk0 * la + m0;           \
+      px = !TX ? Xb + (size_t)n0 * lx + lk0 : Xb + (size_t)lk0 * lx + n0;          \
+      step_a = TA ? BK : BK * la;                                                  \
+      step_x = !TX ? BK : BK * lx;                                                 \
+      kleft = Ks - lk0;                                                            \
+    }                                                                              \
+    tail = kleft < BK;                                                             \
+    if (tail) {                                                                    \
+      LH_KEEP_BRANCH();                                                            \
+      sa.clamp_tail(tid, kleft);                                                   \
+      sx.clamp_tail(tid, kleft);                                                   \
+    }                                                                              \
+    sa.load(pa, tid);                                                              \
+    sx.load(px, tid);                                                              \
+    pa += step_a;                                                                  \
+    px += step_x;                                                                  \
+    kleft -= BK;                                                                   \
+    new_seg = kleft <= 0; /* a short last slab has clamped the offsets as well */  \
+    if (new_seg) {                                                                 \
+      ++lseg;                                                                      \
+      lk0 = 0;                                                                     \
+    }                                                                              \
   } while (0)
 #define LH_STASH(BUF)         \
   do {                        \
