@@ -654,8 +654,6 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
     for (int a = 0; a < FN; ++a) SX::read_frag(smem + fx_off, 0, a, fx[0][a]);
   }
   for (int s = 0; s < total; ++s) {
-    if (s + 1 < total) LH_STASH(smem + (kSlab - cur));
-    if (s + 2 < total) LH_ISSUE();
     const float *as = smem + cur + fa_off;
     const float *xs = smem + cur + fx_off;
     if constexpr (!kCarry) {
@@ -687,7 +685,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
         }
       }
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
+      for (int q = 0; q < 4; ++q) {
 #pragma unroll
         for (int a = 0; a < FN; ++a)
 #pragma unroll
@@ -696,6 +694,11 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
             // consecutive lanes of every accumulator register
             acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fx[c][a][q], fa[c][b][q],
                                                              acc[a][b], 0, 0, 0);
+        // the staging work of the slab rides behind MFMAs that are already in the pipe instead
+        // of standing between two groups of them
+        if (grp == 0 && q == 0 && s + 1 < total) LH_STASH(smem + (kSlab - cur));
+        if (grp == 0 && q == 1 && s + 2 < total) LH_ISSUE();
+      }
     }
     if constexpr (!kCarry) {
       __syncthreads();
