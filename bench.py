@@ -160,7 +160,15 @@ def bench_fused_kernels(torch, steps, warmup):
             4.0 * B * (W * H + 2 * H + 2 * W),
             lambda: lh.attn_core_fwd(H, B, D, 0, S, tanh1, v_p, wa, hs, ncol * H, H, col, bi, m,
                                      o[0], o[1], o[2], o[3], o[4], o[5]))
-        del hs, tanh1, wa
+        # the decoding form: scores against W_a*hs, context sum over W_c1*hs, h~ out
+        hs2, both, b_out = f(S * ncol * H), f(2 * H * B), f(H) * 0.1
+        add("attn_core_projected_fwd (local-p, decoding)",
+            f"H={H} B={B} S={S} D={D} ({per} columns/sentence)",
+            4.0 * B * (2 * W * H + 4 * H + 2 * W),
+            lambda: lh.attn_core_projected_fwd(H, B, D, S, both, 2 * H, v_p, wa, H, hs, hs2, ncol * H,
+                                               H, col, bi, m, both[H:], 2 * H, b_out, o[0], o[1],
+                                               o[2], o[3], o[4], o[5]))
+        del hs, hs2, both, tanh1, wa
     for H, B, n_t in ((1000, 768, 9), (1000, 768 * 16, 9)):
         srcs = [f(H * B) for _ in range(n_t)]
         dsts = [torch.empty(H * B, device=dev) for _ in range(n_t)]
