@@ -755,30 +755,51 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &g) {
     __syncthreads();
     const int H = g.cell_H;
     const bool add = g.beta != 0.f;
-    for (int idx = tid; idx < GQ * BN; idx += NT) {
+    // A thread's cells: everything they read from memory is fetched first, with independent
+    // loads (the outputs may alias c_prev, so loads interleaved with the stores would wait for
+    // one another, a memory latency per cell), then the arithmetic, then the stores.
+    constexpr int kCells = GQ * BN, kPer = (kCells + NT - 1) / NT;
+    float cprev[kPer], mask[kPer], pre[kPer][4];
+    bool ok[kPer];
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int idx = tid + i * NT;
       const int rl = idx % GQ, nl = idx / GQ;
       const int r = m0 + rl, n = n0 + nl;
-      if (r >= H || n >= g.N) continue;
-      float pre[4];
-      int col = n;
-      if (g.addend_col) col = min(max(g.addend_col[n], 0), g.addend_ncols - 1);
-      const float *ad = add ? g.C + (size_t)col * g.ldc + r : nullptr;
+      ok[i] = idx < kCells && r < H && n < g.N;
+      cprev[i] = 0.f, mask[i] = 0.f;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        float v = smem[nl * BM + q * GQ + rl];
-        if (add) v += ad[(size_t)q * H];
-        pre[q] = v + g.bias[q * H + r];
+      for (int q = 0; q < 4; ++q) pre[i][q] = 0.f;
+      if (ok[i]) {
+        int col = n;
+        if (g.addend_col) col = min(max(g.addend_col[n], 0), g.addend_ncols - 1);
+        const float *ad = g.C + (size_t)col * g.ldc + r;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float v = smem[nl * BM + q * GQ + rl];
+          const float t = add ? ad[(size_t)q * H] : 0.f;
+          pre[i][q] = (add ? v + t : v) + g.bias[q * H + r];
+        }
+        cprev[i] = g.c_prev[(size_t)n * H + r];
+        mask[i] = (float)g.colmask[n];
       }
-      const size_t o = (size_t)n * H + r;
+    }
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int idx = tid + i * NT;
+      const int r = m0 + idx % GQ, n = n0 + idx / GQ;
       float c, h;
       if (g.sigmoid_f64)
-        lh::lstm_cell_point<true>(pre[0], pre[1], pre[2], pre[3], g.c_prev[o], (float)g.colmask[n],
+        lh::lstm_cell_point<true>(pre[i][0], pre[i][1], pre[i][2], pre[i][3], cprev[i], mask[i],
                                   g.cell_clip, c, h);
       else
-        lh::lstm_cell_point<false>(pre[0], pre[1], pre[2], pre[3], g.c_prev[o], (float)g.colmask[n],
+        lh::lstm_cell_point<false>(pre[i][0], pre[i][1], pre[i][2], pre[i][3], cprev[i], mask[i],
                                    g.cell_clip, c, h);
-      g.c_out[o] = c;
-      g.h_out[o] = h;
+      if (ok[i]) {
+        const size_t o = (size_t)n * H + r;
+        g.c_out[o] = c;
+        g.h_out[o] = h;
+      }
     }
     return;
   }
