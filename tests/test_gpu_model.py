@@ -165,6 +165,39 @@ def test_decode_same_with_and_without_the_regrouped_step(orc, host, monkeypatch)
     gm.close()
 
 
+def test_decode_random_architectures_vs_oracle(orc, host):
+    """A seeded sweep over architectures and batch shapes the fixed cases do not hit: 1-4 layers,
+    hidden sizes that land on different tile configurations (and on the one- and two-quad attention
+    kernels), windows from 3 to 21 slots, beams 2-12, partly filled batches, attention / feed input
+    / alignment export on and off.  Weight scales stay where fp32 rounding is not amplified: with
+    uniform(-0.8, 0.8) weights at H = 256 two GPU runs that differ only in the tile configuration
+    of their products already disagree by 1e-3 after one step, so that regime says nothing."""
+    rng = np.random.default_rng(2024)
+    for trial in range(14):
+        layers = int(rng.integers(1, 5))
+        H = int(rng.choice([32, 48, 100, 128, 256, 1100]))
+        Vs, Vt = int(rng.integers(30, 300)), int(rng.integers(40, 500))
+        D, n_sent = int(rng.integers(1, 11)), int(rng.integers(1, 9))
+        att = int(rng.choice([0, 1, 1, 1]))
+        feed = bool(att and rng.integers(0, 2))
+        align = bool(att and rng.integers(0, 2))
+        beam = min(int(rng.integers(2, 13)), int(np.sqrt(Vt)))
+        scale = float(rng.choice([0.2, 0.4])) * (0.25 if H > 256 else (0.5 if H == 256 else 1.0))
+        P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 44, scale, decoding=(n_sent, beam),
+                          attention=att, feed=feed)
+        n = int(rng.integers(1, n_sent + 1))
+        sents = [rng.integers(0, Vs, size=int(rng.integers(1, 25))) for _ in range(n)]
+        got = gm.decode_batch(sents, beam=beam, with_hyps=True, alignments=align)
+        what = (f"trial {trial}: layers={layers} H={H} V={Vs}/{Vt} D={D} beam={beam} batch {n}/{n_sent} "
+                f"attention={att} feed={feed} alignments={align} scale={scale}")
+        for i, s_ in enumerate(sents):
+            want = om.decode_sentence(s_, beam=beam, alignments=align)
+            _compare_decode(want, got[i], f"{what}, sentence {i} (len {len(s_)})")
+            if align:
+                assert got[i]["best_viterbi"].tolist() == want["best_viterbi"].tolist(), what
+        gm.close()
+
+
 def _ragged_minibatch(rng, B, S, T, Vs, Vt, min_len=1):
     lens_s = rng.integers(min_len, S + 1, size=B)
     lens_t = rng.integers(max(min_len, 2), T + 1, size=B)
