@@ -201,12 +201,37 @@ __global__ __launch_bounds__(kThreads) void attn_core_regs_kernel(const AttnArgs
   const float *wa = a.wa + (size_t)b * a.wa_col_stride;
   const float *hs_c = a.hs + (size_t)col * a.col_stride;
 
+  // everything that does not depend on the window position is requested first
+  float4 w4[NQ], oadd[NQ], obias[NQ];
+  bool row_ok[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    const int r = (tid + q * kThreads) * 4;
+    row_ok[q] = r < H;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    w4[q] = row_ok[q] ? *reinterpret_cast<const float4 *>(wa + r) : zero;
+    oadd[q] = (row_ok[q] && a.out_add)
+                  ? *reinterpret_cast<const float4 *>(a.out_add + (size_t)b * a.out_add_col_stride + r)
+                  : zero;
+    obias[q] = (row_ok[q] && a.out_bias) ? *reinterpret_cast<const float4 *>(a.out_bias + r) : zero;
+  }
+
   float p = 0.f;
   int lo = 0, hi = len - 1;
   if (D >= 0) {
     float part = 0.f;
     const float *t1 = a.tanh1 + (size_t)b * a.proj_col_stride;
-    for (int r = tid; r < H; r += kThreads) part += a.v_p[r] * t1[r];
+    // rows tid, tid + 256, ... in that order (H <= NQ * 1024), all loads in flight together
+    float vv[4 * NQ], tt[4 * NQ];
+#pragma unroll
+    for (int k = 0; k < 4 * NQ; ++k) {
+      const int r = tid + k * kThreads;
+      vv[k] = r < H ? a.v_p[r] : 0.f;
+      tt[k] = r < H ? t1[r] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < 4 * NQ; ++k)
+      if (tid + k * kThreads < H) part += vv[k] * tt[k];
     const float dot = lh::block_sum<kWaves>(part, s_red);
     const float sig = (float)(1.0 / (1.0 + exp(-1.0 * (double)dot)));
     p = (float)len * sig;
@@ -234,14 +259,6 @@ __global__ __launch_bounds__(kThreads) void attn_core_regs_kernel(const AttnArgs
 
   // the window, once
   float4 h[WCAP][NQ];
-  float4 w4[NQ];
-  bool row_ok[NQ];
-#pragma unroll
-  for (int q = 0; q < NQ; ++q) {
-    const int r = (tid + q * kThreads) * 4;
-    row_ok[q] = r < H;
-    w4[q] = row_ok[q] ? *reinterpret_cast<const float4 *>(wa + r) : make_float4(0.f, 0.f, 0.f, 0.f);
-  }
 #pragma unroll
   for (int j = 0; j < WCAP; ++j) {
     const int tau = s_tau[j];  // the same for every thread: a scalar branch
@@ -292,18 +309,23 @@ __global__ __launch_bounds__(kThreads) void attn_core_regs_kernel(const AttnArgs
   for (int j = 0; j < W; ++j) {
     if (s_idx[j] != -1 && s_val[j] > mx) mx = s_val[j];
   }
+  // one exponential per slot, taken by the slot's thread; the sum then runs over the slots in
+  // order as before
+  __shared__ float s_exp[WCAP];
+  for (int j = tid; j < WCAP; j += kThreads)
+    s_exp[j] = (j < W && s_idx[j] != -1) ? expf(s_val[j] - mx) : 0.f;
+  __syncthreads();
   float Z = 0.f;
   for (int j = 0; j < W; ++j) {
-    if (s_idx[j] != -1) Z += expf(s_val[j] - mx);
+    if (s_idx[j] != -1) Z += s_exp[j];
   }
-  __syncthreads();
   const float sigma_sq = (float)((D * D) / 4.0);
   for (int j = tid; j < WCAP; j += kThreads) {
     float al = 0.f, g = 1.f;
     if (j < W) {
       const int idx = s_idx[j];
       if (idx != -1) {
-        const float e = expf(s_val[j] - mx);
+        const float e = s_exp[j];
         if (D >= 0) {
           const float dlt = p - (float)idx;
           g = expf((-1.f * (dlt * dlt)) / (2.f * sigma_sq));
@@ -342,12 +364,10 @@ __global__ __launch_bounds__(kThreads) void attn_core_regs_kernel(const AttnArgs
     if (!row_ok[q]) continue;
     const size_t r = (size_t)(tid + q * kThreads) * 4;
     if (a.out_add) {
-      const float4 t = *reinterpret_cast<const float4 *>(a.out_add + (size_t)b * a.out_add_col_stride + r);
-      acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+      acc.x += oadd[q].x; acc.y += oadd[q].y; acc.z += oadd[q].z; acc.w += oadd[q].w;
     }
     if (a.out_bias) {
-      const float4 t = *reinterpret_cast<const float4 *>(a.out_bias + r);
-      acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+      acc.x += obias[q].x; acc.y += obias[q].y; acc.z += obias[q].z; acc.w += obias[q].w;
     }
     if (a.out_tanh) {
       const float mf = (float)m;
