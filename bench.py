@@ -33,7 +33,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3
 # known size gives).  A counter run cannot happen inside the timed run, so the figure is carried
 # here; its algorithmic counterpart is 30000*1000*4 + 768*1000*4 read + 30000*768*4 written.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_kernel<64, 64, 2, 2, 1, 16, false, false>": int((232646 + 92729) * 1024),
+    "gemm_kernel<64, 64, 2, 2, 1, 16, false, false>": int((235759 + 92723) * 1024),
     "gemm_kernel<128, 96, 4, 1, 1, 16, false, false>": int((240671 + 89778) * 1024),
     "gemm_kernel<128, 64, 2, 2, 1, 16, false, false>": int((232112 + 101329) * 1024),
 }
