@@ -48,6 +48,9 @@ int Guard(F &&f) {
   } catch (const std::exception &e) {
     g_error = e.what();
     return -1;
+  } catch (...) {  // nothing may unwind into a C caller
+    g_error = "unknown C++ exception";
+    return -1;
   }
 }
 
