@@ -319,6 +319,17 @@ int lh_logsoftmax_xent_f32(const float *logits, int ldl, const float *bias, int 
 int lh_beam_topk_f32(const float *logits, int ldl, const float *bias, int V, int B, int K,
                      int eof_id, float *cand_logp, int *cand_id, float *logp_eof,
                      lh_stream_t stream);
+/* The same selection over the combined distribution of several models.  Replaces
+ * EnsembleFactory::EnsemblesModels (src/decoder.h:1910-1931) in front of ExpandHypothesis:
+ *   q[v,b] = (float)((sum over models, in double, of p[m][v + ldp*b]) / n_models),
+ *   cand_logp = log(q / sum_v q[v,b]) for the K largest q of column b (ties: lowest id), likewise
+ *   logp_eof.  p[m] are the models' probabilities (lh_softmax_fwd_f32), V x B each with leading
+ *   dimension ldp.  Needs V % 4 == 0, ldp % 4 == 0, 16-byte aligned p[m], V <= 65536,
+ *   n_models <= LH_ENSEMBLE_MAX_MODELS.  p is a HOST array of device pointers. */
+#define LH_ENSEMBLE_MAX_MODELS 8
+int lh_beam_topk_ensemble_f32(const float *const *p, int n_models, int ldp, int V, int B, int K,
+                              int eof_id, float *cand_logp, int *cand_id, float *logp_eof,
+                              lh_stream_t stream);
 int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const int *limit,
                       const float *cand_logp, const int *cand_id, const float *logp_eof,
                       const float *prev_score, float diversity, float penalty, int start_id,

@@ -121,6 +121,17 @@ int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int *lengths, i
                       float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
                       float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi,
                       int *kbest_index, float *kbest_score);
+/* The same with an ensemble of n_models models decoded in lockstep (EnsembleFactory::DecodeFile
+ * with several models, src/decoder.h:1778-1931): before every beam step the models' distributions
+ * are averaged and renormalised (EnsemblesModels, :1910-1931), and with o->unk_replacement_mode
+ * their alignment scores are added up (:1933-1962).  models[0] runs the beam search; all were
+ * created by lnmt_model_create_decoding with the same n_sent and beam_size and have the same target
+ * vocabulary (a multiple of 4) and longest sentence.  n_models = 1 is lnmt_decode_batch. */
+int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_models, const int *sentences,
+                               const int *lengths, int n, const lnmt_decode_options *o, int *best,
+                               int cap, int *best_len, float *best_score, int *steps,
+                               int *hyp_tokens, int *hyp_len, float *hyp_score, int hyp_cap,
+                               int *n_hyp, int *best_viterbi, int *kbest_index, float *kbest_score);
 
 /* The model's HIP stream (hipStream_t as void*), for callers that time with HIP events. */
 void *lnmt_model_stream(lnmt_model *m);

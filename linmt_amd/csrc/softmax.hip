@@ -313,13 +313,20 @@ __device__ __forceinline__ void collect(const float4 (&x)[NV], int tid, int V, f
   }
 }
 
-// Up to NV = 8 the register budget is held to 64 per thread so that two workgroups share a CU and
-// one column's selection overlaps the other's loads.
-template <int NV>
-__global__ __launch_bounds__(kT, (NV <= 8 ? 8 : 4)) void beam_topk_kernel(
-    const float *__restrict__ logits, int ldl, const float *__restrict__ bias, int V, int K,
-    int eof_id, float *__restrict__ cand_logp, int *__restrict__ cand_id,
-    float *__restrict__ logp_eof) {
+// The distributions of several models, for EnsembleFactory::EnsemblesModels (src/decoder.h:1910-1931).
+struct EnsembleArgs {
+  const float *p[LH_ENSEMBLE_MAX_MODELS];
+  int n_models;
+};
+
+// ENS = false: the column is logits (+bias) of one model and a candidate's score is its
+// log-softmax.  ENS = true: the column is the mean over the models of their probabilities (summed
+// in double, like the reference) and a candidate's score is log(mean / sum of the column's means).
+template <int NV, bool ENS>
+__device__ __forceinline__ void beam_topk_body(
+    const float *__restrict__ logits, int ldl, const float *__restrict__ bias,
+    const EnsembleArgs &ens, int V, int K, int eof_id, float *__restrict__ cand_logp,
+    int *__restrict__ cand_id, float *__restrict__ logp_eof) {
   __shared__ float red[kNW];
   __shared__ float s_v[kT];
   __shared__ int s_id[kT];
@@ -332,14 +339,40 @@ __global__ __launch_bounds__(kT, (NV <= 8 ? 8 : 4)) void beam_topk_kernel(
   const int b = blockIdx.x, tid = threadIdx.x;
   const int wave = tid / lh::kWave;
   float4 x[NV];
-  load_column<NV>(x, logits + (size_t)b * ldl, bias, V, tid);
-  const float tmax = local_max<NV>(x);
-  const float mx = lh::block_max<kNW>(tmax, red);
-  float part = 0.f;
+  float tmax, mx = 0.f, lse = 0.f, norm = 1.f;
+  if constexpr (!ENS) {
+    load_column<NV>(x, logits + (size_t)b * ldl, bias, V, tid);
+    tmax = local_max<NV>(x);
+    mx = lh::block_max<kNW>(tmax, red);
+    float part = 0.f;
 #pragma unroll
-  for (int i = 0; i < NV; ++i)
-    part += (exp_neg(x[i].x - mx) + exp_neg(x[i].y - mx)) + (exp_neg(x[i].z - mx) + exp_neg(x[i].w - mx));
-  const float lse = logf(lh::block_sum<kNW>(part, red));
+    for (int i = 0; i < NV; ++i)
+      part += (exp_neg(x[i].x - mx) + exp_neg(x[i].y - mx)) + (exp_neg(x[i].z - mx) + exp_neg(x[i].w - mx));
+    lse = logf(lh::block_sum<kNW>(part, red));
+  } else {
+    const int V4 = V / 4;
+    const double n = (double)ens.n_models;
+    float part = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int f = tid + i * kT;
+      float4 v = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);  // rows >= V are never candidates
+      if (f < V4) {
+        double s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+        for (int m = 0; m < ens.n_models; ++m) {
+          const float4 t = reinterpret_cast<const float4 *>(ens.p[m] + (size_t)b * ldl)[f];
+          s0 += t.x, s1 += t.y, s2 += t.z, s3 += t.w;
+        }
+        v = make_float4((float)(s0 / n), (float)(s1 / n), (float)(s2 / n), (float)(s3 / n));
+        part += (v.x + v.y) + (v.z + v.w);
+      }
+      x[i] = v;
+    }
+    tmax = local_max<NV>(x);
+    norm = lh::block_sum<kNW>(part, red);
+  }
+  // a candidate's score from its value in x
+  auto score_of = [&](float v) { return ENS ? logf(v / norm) : (v - mx) - lse; };
 
   if (eof_id >= 0 && eof_id < V && (eof_id / 4) % kT == tid) {
     const int i = (eof_id / 4) / kT, c = eof_id % 4;
@@ -347,7 +380,7 @@ __global__ __launch_bounds__(kT, (NV <= 8 ? 8 : 4)) void beam_topk_kernel(
 #pragma unroll
     for (int k = 0; k < NV; ++k)
       if (k == i) z = comp(x[k], c);
-    logp_eof[b] = (z - mx) - lse;
+    logp_eof[b] = score_of(z);
   }
 
   // ---- fast path: threshold from group maxima ----------------------------------------------
@@ -430,10 +463,28 @@ __global__ __launch_bounds__(kT, (NV <= 8 ? 8 : 4)) void beam_topk_kernel(
 #pragma unroll 4
     for (int q = 0; q < n; ++q) rank += beats(l_v[q], l_id[q], v, id) ? 1 : 0;
     if (rank < K) {
-      cand_logp[(size_t)b * K + rank] = (v - mx) - lse;
+      cand_logp[(size_t)b * K + rank] = score_of(v);
       cand_id[(size_t)b * K + rank] = id;
     }
   }
+}
+
+// Up to NV = 8 the register budget is held to 64 per thread so that two workgroups share a CU and
+// one column's selection overlaps the other's loads.
+template <int NV>
+__global__ __launch_bounds__(kT, (NV <= 8 ? 8 : 4)) void beam_topk_kernel(
+    const float *__restrict__ logits, int ldl, const float *__restrict__ bias, int V, int K,
+    int eof_id, float *__restrict__ cand_logp, int *__restrict__ cand_id,
+    float *__restrict__ logp_eof) {
+  beam_topk_body<NV, false>(logits, ldl, bias, EnsembleArgs{}, V, K, eof_id, cand_logp, cand_id,
+                            logp_eof);
+}
+
+template <int NV>
+__global__ __launch_bounds__(kT, 4) void beam_topk_ensemble_kernel(
+    const EnsembleArgs ens, int ldp, int V, int K, int eof_id, float *__restrict__ cand_logp,
+    int *__restrict__ cand_id, float *__restrict__ logp_eof) {
+  beam_topk_body<NV, true>(nullptr, ldp, nullptr, ens, V, K, eof_id, cand_logp, cand_id, logp_eof);
 }
 
 // Generic fallback for the fused top-K: K sweeps over the column with an exclusion threshold.
@@ -560,6 +611,40 @@ extern "C" int lh_softmax_xent_grad_f32(const float *logits, int ldl, const floa
   if (rc != LH_OK) return rc;
   hipLaunchKernelGGL(masked_sum_kernel, dim3(1), dim3(kT), 0, st, logp_tgt, mask01, B, loss_accum);
   return lh::check_launch("lh_softmax_xent_grad_f32 (sum)");
+}
+
+extern "C" int lh_beam_topk_ensemble_f32(const float *const *p, int n_models, int ldp, int V, int B,
+                                         int K, int eof_id, float *cand_logp, int *cand_id,
+                                         float *logp_eof, lh_stream_t stream) {
+  if (V <= 0 || B <= 0 || !p || !cand_logp || !cand_id || !logp_eof || ldp < V)
+    return lh::fail_arg("lh_beam_topk_ensemble_f32: V=%d B=%d ldp=%d or NULL pointer", V, B, ldp);
+  if (n_models < 1 || n_models > LH_ENSEMBLE_MAX_MODELS)
+    return lh::fail_arg("lh_beam_topk_ensemble_f32: n_models=%d outside [1,%d]", n_models,
+                        LH_ENSEMBLE_MAX_MODELS);
+  if (K < 1 || K > LH_BEAM_MAX_K || K > V)
+    return lh::fail_arg("lh_beam_topk_ensemble_f32: K=%d outside [1,min(%d,V=%d)]", K,
+                        LH_BEAM_MAX_K, V);
+  EnsembleArgs ens{};
+  ens.n_models = n_models;
+  int nv = -1;
+  for (int m = 0; m < n_models; ++m) {
+    if (!p[m]) return lh::fail_arg("lh_beam_topk_ensemble_f32: distribution %d is NULL", m);
+    ens.p[m] = p[m];
+    const int nv_m = pick_nv(p[m], ldp, nullptr, V);
+    nv = m == 0 ? nv_m : (nv_m == nv ? nv : 0);
+  }
+  if (nv != 2 && nv != 4 && nv != 8 && nv != 16)
+    return lh::fail_arg("lh_beam_topk_ensemble_f32: needs V %% 4 == 0, ldp %% 4 == 0, 16-byte "
+                        "aligned distributions and V <= %d (V=%d ldp=%d)", 16 * 4 * kT, V, ldp);
+  hipStream_t st = lh::as_stream(stream);
+  const dim3 grid(B), block(kT);
+  switch (nv) {
+    case 2: hipLaunchKernelGGL(beam_topk_ensemble_kernel<2>, grid, block, 0, st, ens, ldp, V, K, eof_id, cand_logp, cand_id, logp_eof); break;
+    case 4: hipLaunchKernelGGL(beam_topk_ensemble_kernel<4>, grid, block, 0, st, ens, ldp, V, K, eof_id, cand_logp, cand_id, logp_eof); break;
+    case 8: hipLaunchKernelGGL(beam_topk_ensemble_kernel<8>, grid, block, 0, st, ens, ldp, V, K, eof_id, cand_logp, cand_id, logp_eof); break;
+    default: hipLaunchKernelGGL(beam_topk_ensemble_kernel<16>, grid, block, 0, st, ens, ldp, V, K, eof_id, cand_logp, cand_id, logp_eof); break;
+  }
+  return lh::check_launch("lh_beam_topk_ensemble_f32");
 }
 
 extern "C" int lh_beam_topk_f32(const float *logits, int ldl, const float *bias, int V, int B, int K,

@@ -103,6 +103,8 @@ def load():
                                       C.POINTER(DecodeOptions), C.c_void_p, C.c_int, C.c_void_p,
                                       C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.lnmt_decode_batch_ensemble.argtypes = [C.POINTER(C.c_void_p), C.c_int] + \
+        lib.lnmt_decode_batch.argtypes[1:]
     lib.lnmt_model_stream.restype = C.c_void_p
     lib.lnmt_model_stream.argtypes = [C.c_void_p]
     lib.lnmt_profile_set_level.argtypes = [C.c_void_p, C.c_int]
@@ -345,10 +347,11 @@ class Model:
 
     def decode_batch(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0,
                      diversity=0.0, lp_alpha=0.65, cp_beta=0.20, with_hyps=False, hyp_cap=256,
-                     alignments=False, num_hypotheses=1):
+                     alignments=False, num_hypotheses=1, ensemble=()):
         """alignments=True: the reference's unk_replacement_mode__; results gain best_viterbi.
         num_hypotheses > 1: results gain kbest = [(index into the finished hypotheses, final
-        score)], best first."""
+        score)], best first.  ensemble: further decoding models whose distributions are averaged
+        with this one's before every beam step (EnsembleFactory with several models)."""
         n = len(sentences)
         lengths = np.array([len(s) for s in sentences], np.int32)
         flat = np.ascontiguousarray(np.concatenate([np.asarray(s, np.int32) for s in sentences]))
@@ -368,9 +371,11 @@ class Model:
             ht = np.zeros((n, hyp_cap, cap), np.int32)
             hl = np.zeros((n, hyp_cap), np.int32)
             hs = np.zeros((n, hyp_cap), np.float32)
-        _check(load().lnmt_decode_batch(self.handle, _p(flat), _p(lengths), n, C.byref(o), _p(best),
-                                        cap, _p(blen), _p(bscore), _p(steps), _p(ht), _p(hl),
-                                        _p(hs), hyp_cap, _p(nh), _p(vit), _p(kidx), _p(kscore)),
+        handles = (C.c_void_p * (1 + len(ensemble)))(self.handle, *[m.handle for m in ensemble])
+        _check(load().lnmt_decode_batch_ensemble(handles, len(handles), _p(flat), _p(lengths), n,
+                                                 C.byref(o), _p(best), cap, _p(blen), _p(bscore),
+                                                 _p(steps), _p(ht), _p(hl), _p(hs), hyp_cap, _p(nh),
+                                                 _p(vit), _p(kidx), _p(kscore)),
                "decode_batch")
         res = []
         for i in range(n):

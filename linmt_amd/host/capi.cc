@@ -224,7 +224,27 @@ extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int 
                                  float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
                                  float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi,
                                  int *kbest_index, float *kbest_score) {
+  lnmt_model *one[1] = {m};
+  return lnmt_decode_batch_ensemble(one, 1, sentences, lengths, n, o, best, cap, best_len,
+                                    best_score, steps, hyp_tokens, hyp_len, hyp_score, hyp_cap,
+                                    n_hyp, best_viterbi, kbest_index, kbest_score);
+}
+
+extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_models,
+                                          const int *sentences, const int *lengths, int n,
+                                          const lnmt_decode_options *o, int *best, int cap,
+                                          int *best_len, float *best_score, int *steps,
+                                          int *hyp_tokens, int *hyp_len, float *hyp_score,
+                                          int hyp_cap, int *n_hyp, int *best_viterbi,
+                                          int *kbest_index, float *kbest_score) {
   return Guard([&] {
+    if (!models || n_models < 1 || !models[0]) throw LinmtError("no model");
+    lnmt_model *m = models[0];
+    std::vector<NeuralMachineTranslation *> others;
+    for (int k = 1; k < n_models; ++k) {
+      if (!models[k]) throw LinmtError("ensemble model is NULL");
+      others.push_back(models[k]->nmt.get());
+    }
     std::vector<std::vector<int>> sents(n);
     size_t off = 0;
     for (int i = 0; i < n; ++i) {
@@ -243,7 +263,7 @@ extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int 
     d.unk_replacement_mode_ = o->unk_replacement_mode != 0;
     d.hypotheses_number_ = std::max(1, o->num_hypotheses);
     std::vector<SentenceResult> res;
-    m->nmt->DecodeBatch(sents, d, &res);
+    m->nmt->DecodeBatch(sents, d, &res, others);
     for (int i = 0; i < n; ++i) {
       const SentenceResult &r = res[i];
       const int bl = std::min((int)r.best.size(), cap);

@@ -441,6 +441,8 @@ class NeuralMachineTranslation {
   BaseLossLayer *p_softmax_layer_ = &softmax_layer_;
   Decoder decoder_;
   DeviceArray<float> p_device_h_tild_previous_;  // decode: gathered h~ of the previous step
+  DeviceArray<float> p_device_ensemble_dist_;    // decode in an ensemble: this model's probabilities
+  std::vector<hipEvent_t> ensemble_events_;      // owned by the model that runs the beam search
   DeviceArray<int> p_device_ones_, p_device_sentence_of_column_;
 
   explicit NeuralMachineTranslation(const GlobalConfiguration &cfg);
@@ -465,8 +467,13 @@ class NeuralMachineTranslation {
   void SwapDecodingStates(const int *p_device_backptr, int minibatch);
   // EnsembleFactory::DecodeFile (decoder.h:1702-1776) for a batch of sentences (ids in ORIGINAL
   // order, ragged).  Results come back in input order.
+  // `ensemble`: further models decoded in lockstep with this one (EnsembleFactory,
+  // decoder.h:1778-1931): their distributions are averaged with this model's before every beam
+  // step.  They must be initialised for decoding with the same n_sent, beam, target vocabulary
+  // and longest sentence; hidden size, depth and attention may differ.
   void DecodeBatch(const std::vector<std::vector<int>> &sentences, const DecodeOptions &o,
-                   std::vector<SentenceResult> *results);
+                   std::vector<SentenceResult> *results,
+                   const std::vector<NeuralMachineTranslation *> &ensemble = {});
 
   // ---- training --------------------------------------------------------------------------------
   DeviceArray<double> p_device_norm_workspace_, p_device_norms_;

@@ -34,6 +34,7 @@ void NeuralMachineTranslation::Gemm(int tag, int rows, int cols, const lh_gemm_s
 NeuralMachineTranslation::~NeuralMachineTranslation() {
   if (stream_) (void)hipStreamSynchronize(stream_);
   for (hipEvent_t e : lane_events_) (void)hipEventDestroy(e);
+  for (hipEvent_t e : ensemble_events_) (void)hipEventDestroy(e);
   for (size_t l = 1; l < lane_streams_.size(); ++l) {  // lane 0 is stream_
     (void)hipStreamSynchronize(lane_streams_[l]);
     (void)hipStreamDestroy(lane_streams_[l]);
@@ -581,8 +582,26 @@ void Decoder::OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_le
 
 void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &sentences,
                                            const DecodeOptions &o,
-                                           std::vector<SentenceResult> *results) {
+                                           std::vector<SentenceResult> *results,
+                                           const std::vector<NeuralMachineTranslation *> &ensemble) {
   if (!decode_mode_) throw LinmtError("DecodeBatch: call InitModelDecoding first");
+  // EnsembleFactory (decoder.h:1702-1931): every model runs the same columns in lockstep, each on
+  // its own stream; this model owns the beam search, the others hand it their distributions.
+  std::vector<NeuralMachineTranslation *> models{this};
+  for (NeuralMachineTranslation *m : ensemble) {
+    if (!m || m == this) throw LinmtError("DecodeBatch: ensemble entries must be other models");
+    if (!m->decode_mode_ || m->n_sent_ != n_sent_ || m->beam_size_ != beam_size_ ||
+        m->cfg_.target_vocab_size_ != cfg_.target_vocab_size_ ||
+        m->cfg_.longest_sentence_ != cfg_.longest_sentence_ ||
+        m->cfg_.num_layers_ > LH_GATHER_MAX_TENSORS / 2 - 1)
+      throw LinmtError("DecodeBatch: ensemble models must be initialised for decoding with the same "
+                       "n_sent, beam, target vocabulary and longest sentence");
+    models.push_back(m);
+  }
+  const int n_models = (int)models.size();
+  if (n_models > LH_ENSEMBLE_MAX_MODELS) throw LinmtError("DecodeBatch: too many models");
+  if (n_models > 1 && cfg_.target_vocab_size_ % 4 != 0)
+    throw LinmtError("DecodeBatch: an ensemble needs a target vocabulary that is a multiple of 4");
   const int n = (int)sentences.size();
   int beam = o.beam_size_;
   if (beam > (int)std::sqrt((double)cfg_.target_vocab_size_))  // decoder.h:1662-1664
@@ -613,7 +632,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
       binfo[(size_t)n * beam + (size_t)k * beam + j] = S - len;
     }
   }
-  const int B = n * beam, K = beam + 1, H = cfg_.lstm_size_, L = cfg_.num_layers_;
+  const int B = n * beam, K = beam + 1;
   Decoder &d = decoder_;
   if (max_limit + 1 > d.max_steps_) throw LinmtError("DecodeBatch: too many decoding steps");
 
@@ -622,48 +641,91 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   d.current_indices_.Upload(start.data(), B, stream_);
   d.score_[0].Zero(stream_);
   d.limit_.Upload(limit.data(), n, stream_);
-  if (cfg_.attention_mode_) {
-    attention_layer_.PreprocessMinibatchInformation(binfo.data(), B);
-    attention_layer_.hs_step_stride_ = (long long)H * SourceLayer(L - 1).minibatch_size_;
-    attention_layer_.hs_steps_ = S;
-    if (attention_layer_.global_mode_ && S > attention_layer_.window_)
-      throw LinmtError("DecodeBatch: source longer than the attention window");
-  }
-
-  // the encoder layers were allocated for n_sent_ columns; run them on n (ld is lstm_size_, so a
-  // smaller batch simply uses the first n columns of every step's buffer)
-  if (n != n_sent_ && cfg_.attention_mode_)
-    attention_layer_.hs_step_stride_ = (long long)H * n_sent_;
-  ForwardPropSource(src.data(), S, n);
-  if (cfg_.attention_mode_) attention_layer_.BuildProjectedMemory(S, SourceLayer(L - 1).h_all_.size());
-
-  // TransferDecodingStatesGpu (layer_input_to_hidden.h:1536-1545): encoder's final (h, c) of layer
-  // l, sentence s -> every beam column of s.
-  {
-    const float *gs[LH_GATHER_MAX_TENSORS];
-    float *gd[LH_GATHER_MAX_TENSORS];
-    int g = 0;
-    for (int l = 0; l < L; ++l) {
-      gs[g] = SourceLayer(l).v_nodes_[S - 1].p_device_h_t_;
-      gd[g++] = TargetLayer(l).p_device_h_t_previous_.get();
-      gs[g] = SourceLayer(l).v_nodes_[S - 1].p_device_c_t_;
-      gd[g++] = TargetLayer(l).p_device_c_t_previous_.get();
-    }
-    LhErrorWrapper(lh_beam_gather_f32(gs, gd, g, H, B, n, p_device_sentence_of_column_.get(), stream_),
-                   "TransferDecodingStatesGpu");
-  }
 
   // unk_replacement_mode_: the attention node writes every step's alignments and window indices
-  // into its own slice of a history instead of the one reused buffer
-  const bool capture = o.unk_replacement_mode_ && cfg_.attention_mode_;
-  const int W = cfg_.attention_mode_ ? attention_layer_.window_ : 0;
-  AttentionNode *an = cfg_.attention_mode_ ? &attention_layer_.v_nodes_[0] : nullptr;
-  float *const node_alignments = an ? an->p_device_alignments_ : nullptr;
-  int *const node_indices = an ? an->p_device_indices_ : nullptr;
-  const size_t hist_slice = (size_t)n_sent_ * beam * W;
-  if (capture && d.align_hist_.size() < hist_slice * d.max_steps_) {
-    d.align_hist_.Alloc(hist_slice * d.max_steps_);
-    d.index_hist_.Alloc(hist_slice * d.max_steps_);
+  // into its own slice of a history instead of the one reused buffer.  (With several models the
+  // scores of all of them are added up, decoder.h:1933-1945, so all of them must have attention.)
+  bool capture = o.unk_replacement_mode_;
+  for (NeuralMachineTranslation *m : models) capture = capture && m->cfg_.attention_mode_;
+  struct NodeBuffers {
+    float *alignments;
+    int *indices;
+  };
+  std::vector<NodeBuffers> node_buffers(n_models, NodeBuffers{nullptr, nullptr});
+  std::vector<size_t> hist_slices(n_models, 0);
+
+  for (int k = 0; k < n_models; ++k) {
+    NeuralMachineTranslation &M = *models[k];
+    const int H = M.cfg_.lstm_size_, L = M.cfg_.num_layers_;
+    if (M.cfg_.attention_mode_) {
+      M.attention_layer_.PreprocessMinibatchInformation(binfo.data(), B);
+      M.attention_layer_.hs_step_stride_ = (long long)H * M.SourceLayer(L - 1).minibatch_size_;
+      M.attention_layer_.hs_steps_ = S;
+      if (M.attention_layer_.global_mode_ && S > M.attention_layer_.window_)
+        throw LinmtError("DecodeBatch: source longer than the attention window");
+    }
+    // the encoder layers were allocated for n_sent_ columns; run them on n (ld is lstm_size_, so a
+    // smaller batch simply uses the first n columns of every step's buffer)
+    if (n != n_sent_ && M.cfg_.attention_mode_)
+      M.attention_layer_.hs_step_stride_ = (long long)H * n_sent_;
+    M.ForwardPropSource(src.data(), S, n);
+    if (M.cfg_.attention_mode_)
+      M.attention_layer_.BuildProjectedMemory(S, M.SourceLayer(L - 1).h_all_.size());
+
+    // TransferDecodingStatesGpu (layer_input_to_hidden.h:1536-1545): encoder's final (h, c) of
+    // layer l, sentence s -> every beam column of s.
+    {
+      const float *gs[LH_GATHER_MAX_TENSORS];
+      float *gd[LH_GATHER_MAX_TENSORS];
+      int g = 0;
+      for (int l = 0; l < L; ++l) {
+        gs[g] = M.SourceLayer(l).v_nodes_[S - 1].p_device_h_t_;
+        gd[g++] = M.TargetLayer(l).p_device_h_t_previous_.get();
+        gs[g] = M.SourceLayer(l).v_nodes_[S - 1].p_device_c_t_;
+        gd[g++] = M.TargetLayer(l).p_device_c_t_previous_.get();
+      }
+      LhErrorWrapper(lh_beam_gather_f32(gs, gd, g, H, B, n, M.p_device_sentence_of_column_.get(),
+                                        M.stream_),
+                     "TransferDecodingStatesGpu");
+    }
+    if (M.cfg_.attention_mode_) {
+      AttentionNode &node = M.attention_layer_.v_nodes_[0];
+      node_buffers[k] = NodeBuffers{node.p_device_alignments_, node.p_device_indices_};
+      hist_slices[k] = (size_t)n_sent_ * beam * M.attention_layer_.window_;
+      Decoder &dm = M.decoder_;
+      if (capture && dm.align_hist_.size() < hist_slices[k] * d.max_steps_) {
+        dm.align_hist_.Alloc(hist_slices[k] * d.max_steps_);
+        dm.index_hist_.Alloc(hist_slices[k] * d.max_steps_);
+      }
+    }
+    if (n_models > 1 && M.p_device_ensemble_dist_.size() < (size_t)M.cfg_.target_vocab_size_ * B)
+      M.p_device_ensemble_dist_.Alloc((size_t)M.cfg_.target_vocab_size_ * n_sent_ * beam);
+  }
+  // the nodes get their own buffers back however this function is left
+  struct RestoreNodes {
+    std::vector<NeuralMachineTranslation *> &models;
+    std::vector<NodeBuffers> &buffers;
+    ~RestoreNodes() {
+      for (size_t k = 0; k < models.size(); ++k)
+        if (buffers[k].alignments) {
+          AttentionNode &node = models[k]->attention_layer_.v_nodes_[0];
+          node.p_device_alignments_ = buffers[k].alignments;
+          node.p_device_indices_ = buffers[k].indices;
+        }
+    }
+  } restore_nodes{models, node_buffers};
+  // ordering between the models' streams: one event per model ("distribution of this step is
+  // ready") and one for the beam step ("tokens and back-pointers of this step are ready")
+  if (n_models > 1) {
+    while (ensemble_events_.size() < (size_t)n_models + 1) {
+      hipEvent_t e;
+      HipErrorWrapper(hipEventCreateWithFlags(&e, hipEventDisableTiming), "ensemble event creation failed");
+      ensemble_events_.push_back(e);
+    }
+    // the uploads above (start tokens, scores) precede every model's first step
+    HipErrorWrapper(hipEventRecord(ensemble_events_[0], stream_), "ensemble event record failed");
+    for (int k = 1; k < n_models; ++k)
+      HipErrorWrapper(hipStreamWaitEvent(models[k]->stream_, ensemble_events_[0], 0), "ensemble wait failed");
   }
 
   int cur = 0;
@@ -675,28 +737,52 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
     while (n_active < n && limit[n_active] >= step) ++n_active;  // limits are non-increasing
     active_at[step] = n_active;
     const int Ba = n_active * beam;
-    if (cfg_.attention_mode_ && (step == 0 || n_active != active_at[step - 1])) {
+    if (step == 0 || n_active != active_at[step - 1]) {
       // the batch information is [len_0..len_{Ba-1}, off_0..off_{Ba-1}] for the columns in use, so
       // it is laid out again whenever the number of active columns changes
-      bi_keep.emplace_back(2 * (size_t)Ba);  // kept alive until the stream has been synchronised
+      bi_keep.emplace_back(2 * (size_t)Ba);  // kept alive until the streams have been synchronised
       std::vector<int> &bi = bi_keep.back();
       for (int b = 0; b < Ba; ++b) {
         bi[b] = binfo[b];
         bi[(size_t)Ba + b] = binfo[(size_t)B + b];
       }
-      attention_layer_.PreprocessMinibatchInformation(bi.data(), Ba);
+      for (NeuralMachineTranslation *m : models)
+        if (m->cfg_.attention_mode_) m->attention_layer_.PreprocessMinibatchInformation(bi.data(), Ba);
     }
-    if (capture) {
-      an->p_device_alignments_ = d.align_hist_.get() + hist_slice * step;
-      an->p_device_indices_ = d.index_hist_.get() + hist_slice * step;
+    const int V = cfg_.target_vocab_size_;
+    for (int k = n_models - 1; k >= 0; --k) {  // the other models first: this one's stream waits for them
+      NeuralMachineTranslation &M = *models[k];
+      if (capture) {
+        AttentionNode &node = M.attention_layer_.v_nodes_[0];
+        node.p_device_alignments_ = M.decoder_.align_hist_.get() + hist_slices[k] * step;
+        node.p_device_indices_ = M.decoder_.index_hist_.get() + hist_slices[k] * step;
+      }
+      M.ForwardPropTarget(step, p_device_step_indices, Ba);
+      if (n_models > 1) {
+        LhErrorWrapper(lh_softmax_fwd_f32(M.softmax_layer_.GetDistPtr(), V, nullptr, V, Ba,
+                                          M.p_device_ensemble_dist_.get(), V, M.stream_),
+                       "ensemble: model distribution");
+        if (k > 0) {
+          HipErrorWrapper(hipEventRecord(ensemble_events_[k], M.stream_), "ensemble event record failed");
+          HipErrorWrapper(hipStreamWaitEvent(stream_, ensemble_events_[k], 0), "ensemble wait failed");
+        }
+      }
     }
-    ForwardPropTarget(step, p_device_step_indices, Ba);
-    {
+    if (n_models == 1) {
       ProfileScope ps(profiler_, kTagBeamTopK, 4.0 * cfg_.target_vocab_size_ * Ba);
       LhErrorWrapper(lh_beam_topk_f32(softmax_layer_.GetDistPtr(), cfg_.target_vocab_size_, nullptr,
                                     cfg_.target_vocab_size_, Ba, K, Decoder::end_symbol_,
                                     d.cand_logp_.get(), d.cand_id_.get(), d.logp_eof_.get(), stream_),
                    "beam top-k");
+    } else {
+      // EnsemblesModels (decoder.h:1910-1931) + the per-column selection of ExpandHypothesis
+      const float *dist[LH_ENSEMBLE_MAX_MODELS];
+      for (int k = 0; k < n_models; ++k) dist[k] = models[k]->p_device_ensemble_dist_.get();
+      ProfileScope ps(profiler_, kTagBeamTopK, 4.0 * n_models * V * Ba);
+      LhErrorWrapper(lh_beam_topk_ensemble_f32(dist, n_models, V, V, Ba, K, Decoder::end_symbol_,
+                                               d.cand_logp_.get(), d.cand_id_.get(),
+                                               d.logp_eof_.get(), stream_),
+                     "ensemble beam top-k");
     }
     const size_t off = (size_t)step * B;
     {
@@ -712,7 +798,12 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
     }
     cur ^= 1;
     if (step < max_limit) {
-      SwapDecodingStates(d.backptr_hist_.get() + off, Ba);
+      if (n_models > 1) {
+        HipErrorWrapper(hipEventRecord(ensemble_events_[0], stream_), "ensemble event record failed");
+        for (int k = 1; k < n_models; ++k)
+          HipErrorWrapper(hipStreamWaitEvent(models[k]->stream_, ensemble_events_[0], 0), "ensemble wait failed");
+      }
+      for (NeuralMachineTranslation *m : models) m->SwapDecodingStates(d.backptr_hist_.get() + off, Ba);
       // the tokens just chosen are the next step's input ids, read in place from the history
       p_device_step_indices = d.tok_hist_.get() + off;
     }
@@ -727,15 +818,20 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   d.fin_count_hist_.Download(fcount.data(), fcount.size(), stream_);
   d.fin_beam_hist_.Download(fbeam.data(), fbeam.size(), stream_);
   d.fin_score_hist_.Download(fscore.data(), fscore.size(), stream_);
-  std::vector<float> ahist;
-  std::vector<int> ihist;
-  if (capture) {
-    an->p_device_alignments_ = node_alignments;
-    an->p_device_indices_ = node_indices;
-    ahist.resize(hist_slice * steps);
-    ihist.resize(hist_slice * steps);
-    d.align_hist_.Download(ahist.data(), ahist.size(), stream_);
-    d.index_hist_.Download(ihist.data(), ihist.size(), stream_);
+  std::vector<std::vector<float>> ahists(n_models);
+  std::vector<std::vector<int>> ihists(n_models);
+  for (int k = 0; k < n_models; ++k) {
+    NeuralMachineTranslation &M = *models[k];
+    if (capture) {
+      ahists[k].resize(hist_slices[k] * steps);
+      ihists[k].resize(hist_slices[k] * steps);
+      M.decoder_.align_hist_.Download(ahists[k].data(), ahists[k].size(), M.stream_);
+      M.decoder_.index_hist_.Download(ihists[k].data(), ihists[k].size(), M.stream_);
+    } else if (k > 0) {
+      // nothing of this model is read back: wait for its stream so that the host arrays it was
+      // handed (batch information) and the shared device buffers can be reused
+      HipErrorWrapper(hipStreamSynchronize(M.stream_), "ensemble stream synchronisation failed");
+    }
   }
   Synchronize();
   profiler_.Collect();
@@ -755,10 +851,13 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
       // and are never read)
       scores->assign(source_length, 0.f);
       const size_t Ba_t = (size_t)active_at[t] * beam;
-      for (int j = 0; j < W; ++j) {
-        const size_t at = hist_slice * t + column + Ba_t * j;
-        const int idx = ihist[at];
-        if (idx >= 0 && idx < source_length) (*scores)[idx] = ahist[at];
+      for (int k = 0; k < n_models; ++k) {  // the models' scores are added up (decoder.h:1933-1945)
+        const int Wk = models[k]->attention_layer_.window_;
+        for (int j = 0; j < Wk; ++j) {
+          const size_t at = hist_slices[k] * t + column + Ba_t * j;
+          const int idx = ihists[k][at];
+          if (idx >= 0 && idx < source_length) (*scores)[idx] += ahists[k][at];
+        }
       }
       float max_val = 0;
       *viterbi = -1;

@@ -77,6 +77,9 @@ SIGNATURES = {
                                          c_f64p, c_f64p, C.c_void_p]),
     "lh_beam_topk_f32": (C.c_int, [c_f32p, C.c_int, c_f32p, C.c_int, C.c_int, C.c_int, C.c_int,
                                    c_f32p, c_i32p, c_f32p, C.c_void_p]),
+    "lh_beam_topk_ensemble_f32": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_int,
+                                            C.c_int, C.c_int, C.c_int, c_f32p, c_i32p, c_f32p,
+                                            C.c_void_p]),
     "lh_beam_merge_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, c_i32p, c_f32p, c_i32p,
                                     c_f32p, c_f32p, C.c_float, C.c_float, C.c_int, C.c_int, c_i32p,
                                     c_i32p, c_f32p, c_i32p, c_i32p, c_f32p, C.c_void_p]),
@@ -304,6 +307,14 @@ def beam_topk(logits, ldl, bias, V, B, K, eof_id, cand_logp, cand_id, logp_eof, 
     check(load().lh_beam_topk_f32(_ptr(logits), ldl, _ptr(bias), V, B, K, eof_id, _ptr(cand_logp),
                                   _ptr(cand_id), _ptr(logp_eof), _stream(stream)),
           "lh_beam_topk_f32")
+
+
+def beam_topk_ensemble(ps, ldp, V, B, K, eof_id, cand_logp, cand_id, logp_eof, stream=None):
+    """ps: the models' V x B probability tensors (lh_softmax_fwd_f32)."""
+    arr = (C.c_void_p * len(ps))(*[p.data_ptr() for p in ps])
+    check(load().lh_beam_topk_ensemble_f32(arr, len(ps), ldp, V, B, K, eof_id, _ptr(cand_logp),
+                                           _ptr(cand_id), _ptr(logp_eof), _stream(stream)),
+          "lh_beam_topk_ensemble_f32")
 
 
 def beam_merge(n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof, prev_score, diversity,

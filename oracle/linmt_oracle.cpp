@@ -419,15 +419,16 @@ struct GlobCmp {
   bool operator()(const GlobObj &a, const GlobObj &b) const { return a.val < b.val; }
 };
 
-// p (V x cols, col-major) -> renormalised row-major copy, as CopyDistToEigen + EnsemblesModels do.
-void renormalise(const float *p, int V, int cols, std::vector<float> &out) {
+// p[k] (V x cols, col-major, one per model) -> averaged, renormalised row-major copy, as
+// CopyDistToEigen + EnsemblesModels (src/decoder.h:1910-1931) do.
+void renormalise(const float *const *p, int num_models, int V, int cols, std::vector<float> &out) {
   out.resize((size_t)V * cols);
   std::vector<float> norm(cols, 0.f);
   for (int i = 0; i < V; ++i)
     for (int j = 0; j < cols; ++j) {
       double tmp_sum = 0;
-      tmp_sum += p[idx2c(i, j, V)];
-      out[(size_t)i * cols + j] = (float)(tmp_sum / 1);
+      for (int k = 0; k < num_models; ++k) tmp_sum += p[k][idx2c(i, j, V)];
+      out[(size_t)i * cols + j] = (float)(tmp_sum / num_models);
     }
   for (int i = 0; i < V; ++i)
     for (int j = 0; j < cols; ++j) norm[j] += out[(size_t)i * cols + j];
@@ -440,8 +441,17 @@ extern "C" void orc_beam_expand(const float *p, int V, int beam, int step, const
                                 float diversity, float penalty, int start_id, int eof_id, int *tok,
                                 int *backptr, float *score, int *fin_count, int *fin_beam,
                                 float *fin_score) {
+  orc_beam_expand_ensemble(&p, 1, V, beam, step, prev_score, diversity, penalty, start_id, eof_id,
+                           tok, backptr, score, fin_count, fin_beam, fin_score);
+}
+
+extern "C" void orc_beam_expand_ensemble(const float *const *p, int num_models, int V, int beam,
+                                         int step, const float *prev_score, float diversity,
+                                         float penalty, int start_id, int eof_id, int *tok,
+                                         int *backptr, float *score, int *fin_count, int *fin_beam,
+                                         float *fin_score) {
   std::vector<float> dist;
-  renormalise(p, V, beam, dist);
+  renormalise(p, num_models, V, beam, dist);
   int cols = beam;
   if (step == 0) cols = 1;
   std::priority_queue<DecObj, std::vector<DecObj>, DecCmp> pq;
@@ -668,9 +678,10 @@ struct Hyp {
   std::vector<std::vector<float>> align_scores;
 };
 
-int decode_impl(orc_model *m, const int *src_ids, int S, const orc_decode_opts *o, bool unk_mode,
-                int *best_tokens, int cap, int *best_len, float *best_score, int *hyp_tokens,
-                int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi);
+int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
+                const orc_decode_opts *o, bool unk_mode, int *best_tokens, int cap, int *best_len,
+                float *best_score, int *hyp_tokens, int *hyp_len, float *hyp_score, int hyp_cap,
+                int *n_hyp, int *best_viterbi);
 
 }  // namespace
 
@@ -684,8 +695,8 @@ extern "C" int orc_decode_sentence(orc_model *m, const int *src_ids, int S,
                                    const orc_decode_opts *o, int *best_tokens, int cap,
                                    int *best_len, float *best_score, int *hyp_tokens, int *hyp_len,
                                    float *hyp_score, int hyp_cap, int *n_hyp) {
-  return decode_impl(m, src_ids, S, o, false, best_tokens, cap, best_len, best_score, hyp_tokens,
-                     hyp_len, hyp_score, hyp_cap, n_hyp, nullptr);
+  return decode_impl(&m, 1, src_ids, S, o, false, best_tokens, cap, best_len, best_score,
+                     hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, nullptr);
 }
 
 // The same with unk_replacement_mode__ on (layer_attention.h:342-386, decoder.h:1930-1962): every
@@ -697,67 +708,101 @@ extern "C" int orc_decode_sentence_alignments(orc_model *m, const int *src_ids, 
                                               int *best_len, float *best_score, int *best_viterbi,
                                               int *hyp_tokens, int *hyp_len, float *hyp_score,
                                               int hyp_cap, int *n_hyp) {
-  return decode_impl(m, src_ids, S, o, m->cfg.attention != 0, best_tokens, cap, best_len, best_score,
-                     hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, best_viterbi);
+  return decode_impl(&m, 1, src_ids, S, o, m->cfg.attention != 0, best_tokens, cap, best_len,
+                     best_score, hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, best_viterbi);
+}
+
+// The same for an ensemble (EnsembleFactory with several models, src/decoder.h:1778-1931): every
+// model runs every step, EnsemblesModels averages their distributions (and, with alignments, adds
+// up their alignment scores) before ExpandHypothesis.  All models share the target vocabulary and
+// the longest sentence; ms[0]'s configuration supplies them.
+extern "C" int orc_decode_sentence_ensemble(orc_model *const *ms, int num_models, const int *src_ids,
+                                            int S, const orc_decode_opts *o, int alignments,
+                                            int *best_tokens, int cap, int *best_len,
+                                            float *best_score, int *best_viterbi, int *hyp_tokens,
+                                            int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp) {
+  bool unk = alignments != 0;
+  for (int k = 0; k < num_models; ++k) unk = unk && ms[k]->cfg.attention != 0;
+  return decode_impl(ms, num_models, src_ids, S, o, unk, best_tokens, cap, best_len, best_score,
+                     hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, unk ? best_viterbi : nullptr);
 }
 
 namespace {
-int decode_impl(orc_model *m, const int *src_ids, int S, const orc_decode_opts *o, bool unk_mode,
+int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
+                const orc_decode_opts *o, bool unk_mode,
                 int *best_tokens, int cap, int *best_len, float *best_score, int *hyp_tokens,
                 int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi) {
 #ifdef _OPENMP
   if (o->num_threads > 0) omp_set_num_threads(o->num_threads);
 #endif
-  const orc_model_config &cfg = m->cfg;
-  const int H = cfg.H, L = cfg.layers, V = cfg.V_tgt;
+  const int V = ms[0]->cfg.V_tgt;
   int beam = o->beam;
   if (beam > (int)std::sqrt((double)V)) beam = (int)std::sqrt((double)V);  // decoder.h:1662-1664
   const int start_symbol = 0, end_symbol = 1;
-  const int longest = cfg.longest_sent;
-
-  // ---- ForwardPropSource: B = 1, source reversed (input_file_preprocess.cc:633) -----------------
-  std::vector<LayerState> enc(L);
-  for (auto &s : enc) {
-    s.h.assign(H, 0.f);
-    s.c.assign(H, 0.f);
-  }
-  std::vector<float> top_states((size_t)S * H);
-  std::vector<float> x(H), hn(H), cn(H);
-  const int one = 1;
-  for (int t = 0; t < S; ++t) {
-    int id = src_ids[S - 1 - t];
-    int id0, m01;
-    orc_preprocess_indices(&id, 1, &id0, &m01, nullptr);
-    orc_embed_lookup(m->params["src.0.W"].data(), H, cfg.V_src, &id0, 1, nullptr, 1.f, x.data());
-    for (int l = 0; l < L; ++l) {
-      const std::string pfx = "src." + std::to_string(l) + ".";
-      lstm_layer_step(m, pfx, 1, x.data(), enc[l].h.data(), enc[l].c.data(), nullptr, &one,
-                      hn.data(), cn.data());
-      enc[l].h = hn;
-      enc[l].c = cn;
-      x = hn;
-    }
-    memcpy(&top_states[(size_t)t * H], enc[L - 1].h.data(), sizeof(float) * H);
-  }
-
-  // ---- decoder state: TransferDecodingStatesGpu broadcasts the encoder's final (h,c) -------------
+  const int longest = ms[0]->cfg.longest_sent;
   const int B = beam;
-  std::vector<LayerState> prev(L), cur(L);
-  for (int l = 0; l < L; ++l) {
-    prev[l].h.resize((size_t)H * B);
-    prev[l].c.resize((size_t)H * B);
-    cur[l].h.resize((size_t)H * B);
-    cur[l].c.resize((size_t)H * B);
-    for (int b = 0; b < B; ++b) {
-      memcpy(&prev[l].h[(size_t)b * H], enc[l].h.data(), sizeof(float) * H);
-      memcpy(&prev[l].c[(size_t)b * H], enc[l].c.data(), sizeof(float) * H);
-    }
-  }
-  std::vector<float> h_tild((size_t)H * B, 0.f), h_tild_prev((size_t)H * B, 0.f);
+  const int one = 1;
+
+  // what one model of the ensemble carries through the sentence
+  struct Run {
+    orc_model *m;
+    int H, L;
+    std::vector<LayerState> enc, prev, cur;
+    std::vector<float> top_states, h_tild, h_tild_prev, xb, logits, dist, ascore;
+  };
+  std::vector<Run> runs(num_models);
   std::vector<int> ones(B, 1), batch_info(2 * B), hs_col(B, 0);
   for (int b = 0; b < B; ++b) {
     batch_info[b] = S;      // decoder.h:1277-1291: (len, 0) replicated over the beam
     batch_info[B + b] = 0;
+  }
+  for (int k = 0; k < num_models; ++k) {
+    Run &r = runs[k];
+    orc_model *m = r.m = ms[k];
+    const orc_model_config &cfg = m->cfg;
+    const int H = r.H = cfg.H, L = r.L = cfg.layers;
+    // ---- ForwardPropSource: B = 1, source reversed (input_file_preprocess.cc:633) ---------------
+    r.enc.resize(L);
+    for (auto &s : r.enc) {
+      s.h.assign(H, 0.f);
+      s.c.assign(H, 0.f);
+    }
+    r.top_states.resize((size_t)S * H);
+    std::vector<float> x(H), hn(H), cn(H);
+    for (int t = 0; t < S; ++t) {
+      int id = src_ids[S - 1 - t];
+      int id0, m01;
+      orc_preprocess_indices(&id, 1, &id0, &m01, nullptr);
+      orc_embed_lookup(m->params["src.0.W"].data(), H, cfg.V_src, &id0, 1, nullptr, 1.f, x.data());
+      for (int l = 0; l < L; ++l) {
+        const std::string pfx = "src." + std::to_string(l) + ".";
+        lstm_layer_step(m, pfx, 1, x.data(), r.enc[l].h.data(), r.enc[l].c.data(), nullptr, &one,
+                        hn.data(), cn.data());
+        r.enc[l].h = hn;
+        r.enc[l].c = cn;
+        x = hn;
+      }
+      memcpy(&r.top_states[(size_t)t * H], r.enc[L - 1].h.data(), sizeof(float) * H);
+    }
+    // ---- decoder state: TransferDecodingStatesGpu broadcasts the encoder's final (h,c) ----------
+    r.prev.resize(L);
+    r.cur.resize(L);
+    for (int l = 0; l < L; ++l) {
+      r.prev[l].h.resize((size_t)H * B);
+      r.prev[l].c.resize((size_t)H * B);
+      r.cur[l].h.resize((size_t)H * B);
+      r.cur[l].c.resize((size_t)H * B);
+      for (int b = 0; b < B; ++b) {
+        memcpy(&r.prev[l].h[(size_t)b * H], r.enc[l].h.data(), sizeof(float) * H);
+        memcpy(&r.prev[l].c[(size_t)b * H], r.enc[l].c.data(), sizeof(float) * H);
+      }
+    }
+    r.h_tild.assign((size_t)H * B, 0.f);
+    r.h_tild_prev.assign((size_t)H * B, 0.f);
+    r.xb.resize((size_t)H * B);
+    r.logits.resize((size_t)V * B);
+    r.dist.resize((size_t)V * B);
+    r.ascore.assign((size_t)longest * B, 0.f);
   }
 
   // ---- Decoder::InitDecoder -----------------------------------------------------------------------
@@ -776,56 +821,70 @@ int decode_impl(orc_model *m, const int *src_ids, int S, const orc_decode_opts *
                               ascore.begin() + (size_t)longest * (b + 1));
   };
 
-  std::vector<float> xb((size_t)H * B), logits((size_t)V * B), dist((size_t)V * B);
   std::vector<int> tok(B), bp(B), fin_beam(B);
   std::vector<float> sc(B), fin_score(B);
+  std::vector<const float *> dists(num_models);
+  for (int k = 0; k < num_models; ++k) dists[k] = runs[k].dist.data();
 
   auto forward_target = [&](int curr_index) {
-    std::vector<int> id0(B), m01(B);
-    orc_preprocess_indices(current_indices.data(), B, id0.data(), m01.data(), nullptr);
-    orc_embed_lookup(m->params["tgt.0.W"].data(), H, V, id0.data(), B, nullptr, 1.f, xb.data());
-    const float *below = xb.data();
-    for (int l = 0; l < L; ++l) {
-      const std::string pfx = "tgt." + std::to_string(l) + ".";
-      const bool feed = l == 0 && cfg.feed_input && cfg.attention && curr_index != 0;
-      lstm_layer_step(m, pfx, B, below, prev[l].h.data(), prev[l].c.data(),
-                      feed ? h_tild_prev.data() : nullptr, ones.data(), cur[l].h.data(),
-                      cur[l].c.data());
-      below = cur[l].h.data();
-    }
-    const float *top = cur[L - 1].h.data();
-    if (cfg.attention) {
-      std::vector<int> ind;
-      std::vector<float> al;
-      attention_step(m, B, top, top_states.data(), H, 0, hs_col.data(), S, batch_info.data(),
-                     ones.data(), S, h_tild.data(), &ind, &al);
-      top = h_tild.data();
-      if (unk_mode) {
-        // layer_attention.h:360-385: scores of the window's valid slots, zero elsewhere
-        std::fill(ascore.begin(), ascore.end(), 0.f);
-        const int W = (int)(ind.size() / B);
-        for (int j = 0; j < W; ++j)
-          for (int b = 0; b < B; ++b) {
-            const int idx = ind[idx2c(b, j, B)];
-            if (idx != -1) ascore[(size_t)idx + (size_t)longest * b] = al[idx2c(b, j, B)];
-          }
-        // EnsemblesModels (decoder.h:1946-1961): first strictly largest score above 0
-        for (int b = 0; b < B; ++b) {
-          float max_val = 0;
-          int max_index = -1;
-          for (int j = 0; j < longest; ++j) {
-            const float v = ascore[(size_t)j + (size_t)longest * b];
-            if (v > max_val) {
-              max_val = v;
-              max_index = j;
+    for (Run &r : runs) {
+      orc_model *m = r.m;
+      const orc_model_config &cfg = m->cfg;
+      const int H = r.H, L = r.L;
+      std::vector<int> id0(B), m01(B);
+      orc_preprocess_indices(current_indices.data(), B, id0.data(), m01.data(), nullptr);
+      orc_embed_lookup(m->params["tgt.0.W"].data(), H, V, id0.data(), B, nullptr, 1.f, r.xb.data());
+      const float *below = r.xb.data();
+      for (int l = 0; l < L; ++l) {
+        const std::string pfx = "tgt." + std::to_string(l) + ".";
+        const bool feed = l == 0 && cfg.feed_input && cfg.attention && curr_index != 0;
+        lstm_layer_step(m, pfx, B, below, r.prev[l].h.data(), r.prev[l].c.data(),
+                        feed ? r.h_tild_prev.data() : nullptr, ones.data(), r.cur[l].h.data(),
+                        r.cur[l].c.data());
+        below = r.cur[l].h.data();
+      }
+      const float *top = r.cur[L - 1].h.data();
+      if (cfg.attention) {
+        std::vector<int> ind;
+        std::vector<float> al;
+        attention_step(m, B, top, r.top_states.data(), H, 0, hs_col.data(), S, batch_info.data(),
+                       ones.data(), S, r.h_tild.data(), &ind, &al);
+        top = r.h_tild.data();
+        if (unk_mode) {
+          // layer_attention.h:360-385: scores of the window's valid slots, zero elsewhere
+          std::fill(r.ascore.begin(), r.ascore.end(), 0.f);
+          const int W = (int)(ind.size() / B);
+          for (int j = 0; j < W; ++j)
+            for (int b = 0; b < B; ++b) {
+              const int idx = ind[idx2c(b, j, B)];
+              if (idx != -1) r.ascore[(size_t)idx + (size_t)longest * b] = al[idx2c(b, j, B)];
             }
-          }
-          vit[b] = max_index;
         }
       }
+      mat_apply(m, "softmax.D", V, H, top, B, r.logits.data());
+      orc_softmax_fwd(r.logits.data(), V, m->params["softmax.b_d"].data(), V, B, r.dist.data(), V);
     }
-    mat_apply(m, "softmax.D", V, H, top, B, logits.data());
-    orc_softmax_fwd(logits.data(), V, m->params["softmax.b_d"].data(), V, B, dist.data(), V);
+    if (unk_mode) {
+      // EnsemblesModels (decoder.h:1933-1961): the models' scores added up, then the first
+      // strictly largest score above 0
+      for (size_t i = 0; i < ascore.size(); ++i) {
+        float tmp_sum = 0;
+        for (const Run &r : runs) tmp_sum += r.ascore[i];
+        ascore[i] = tmp_sum;
+      }
+      for (int b = 0; b < B; ++b) {
+        float max_val = 0;
+        int max_index = -1;
+        for (int j = 0; j < longest; ++j) {
+          const float v = ascore[(size_t)j + (size_t)longest * b];
+          if (v > max_val) {
+            max_val = v;
+            max_index = j;
+          }
+        }
+        vit[b] = max_index;
+      }
+    }
   };
 
   int steps_run = 0;
@@ -835,9 +894,9 @@ int decode_impl(orc_model *m, const int *src_ids, int S, const orc_decode_opts *
     forward_target(curr_index);
     ++steps_run;
     int nfin = 0;
-    orc_beam_expand(dist.data(), V, B, curr_index, top_scores.data(), o->diversity, o->penalty,
-                    start_symbol, end_symbol, tok.data(), bp.data(), sc.data(), &nfin,
-                    fin_beam.data(), fin_score.data());
+    orc_beam_expand_ensemble(dists.data(), num_models, V, B, curr_index, top_scores.data(),
+                             o->diversity, o->penalty, start_symbol, end_symbol, tok.data(),
+                             bp.data(), sc.data(), &nfin, fin_beam.data(), fin_score.data());
     // bookkeeping of decoder.h:436-479
     for (int f = 0; f < nfin; ++f) {
       Hyp h;
@@ -881,12 +940,14 @@ int decode_impl(orc_model *m, const int *src_ids, int S, const orc_decode_opts *
     top_scores = top_scores_tmp;
     current_index += 1;
     // SwapDecodingStates + TargetCopyPrevStates
-    for (int l = 0; l < L; ++l) {
-      orc_beam_gather(cur[l].h.data(), prev[l].h.data(), H, B, new_indices_changes.data());
-      orc_beam_gather(cur[l].c.data(), prev[l].c.data(), H, B, new_indices_changes.data());
+    for (Run &r : runs) {
+      for (int l = 0; l < r.L; ++l) {
+        orc_beam_gather(r.cur[l].h.data(), r.prev[l].h.data(), r.H, B, new_indices_changes.data());
+        orc_beam_gather(r.cur[l].c.data(), r.prev[l].c.data(), r.H, B, new_indices_changes.data());
+      }
+      if (r.m->cfg.attention && r.m->cfg.feed_input)
+        orc_beam_gather(r.h_tild.data(), r.h_tild_prev.data(), r.H, B, new_indices_changes.data());
     }
-    if (cfg.attention && cfg.feed_input)
-      orc_beam_gather(h_tild.data(), h_tild_prev.data(), H, B, new_indices_changes.data());
     last_index = curr_index;
   }
   forward_target(last_index + 1);
@@ -895,7 +956,7 @@ int decode_impl(orc_model *m, const int *src_ids, int S, const orc_decode_opts *
   // the host renormalisation.
   {
     std::vector<float> rn;
-    renormalise(dist.data(), V, B, rn);
+    renormalise(dists.data(), num_models, V, B, rn);
     for (int i = 0; i < B; ++i) {
       top_sentences[(size_t)i * longest + current_index + 1] = end_symbol;
       top_scores[i] += std::log(rn[(size_t)1 * B + i]) + o->penalty;

@@ -66,6 +66,14 @@ void orc_logsoftmax_xent(const float *logits, int ldl, const float *bias, int V,
 void orc_beam_expand(const float *p, int V, int beam, int step, const float *prev_score,
                      float diversity, float penalty, int start_id, int eof_id, int *tok,
                      int *backptr, float *score, int *fin_count, int *fin_beam, float *fin_score);
+/* The same from the distributions of several models: EnsemblesModels (src/decoder.h:1910-1931)
+ * averages them in double, rounds to float and renormalises each column in float before the
+ * expansion.  pin: equals orc_beam_expand for num_models identical distributions; the averaged
+ * distribution against numpy (tests/test_oracle_pins.py). */
+void orc_beam_expand_ensemble(const float *const *p, int num_models, int V, int beam, int step,
+                              const float *prev_score, float diversity, float penalty, int start_id,
+                              int eof_id, int *tok, int *backptr, float *score, int *fin_count,
+                              int *fin_beam, float *fin_score);
 void orc_beam_gather(const float *src, float *dst, int H, int B, const int *backptr);
 
 /* ---- whole model ----------------------------------------------------------------------------- */
@@ -112,6 +120,18 @@ int orc_decode_sentence_alignments(orc_model *m, const int *src_ids, int S, cons
                                    int *best_tokens, int cap, int *best_len, float *best_score,
                                    int *best_viterbi, int *hyp_tokens, int *hyp_len,
                                    float *hyp_score, int hyp_cap, int *n_hyp);
+/* EnsembleFactory::DecodeFile with several models (src/decoder.h:1778-1931): every model runs every
+ * step on the shared hypotheses; their distributions are averaged before the expansion and, with
+ * alignments != 0 (and attention in every model), their alignment scores added up.  ms[0] supplies
+ * the target vocabulary size and the longest sentence.  Outputs as orc_decode_sentence_alignments
+ * (best_viterbi may be NULL).  pin: two copies of one model decode exactly like the model alone;
+ * two different models against the numpy beam search on the averaged distribution
+ * (tests/test_oracle_pins.py). */
+int orc_decode_sentence_ensemble(orc_model *const *ms, int num_models, const int *src_ids, int S,
+                                 const orc_decode_opts *o, int alignments, int *best_tokens, int cap,
+                                 int *best_len, float *best_score, int *best_viterbi,
+                                 int *hyp_tokens, int *hyp_len, float *hyp_score, int hyp_cap,
+                                 int *n_hyp);
 
 /* Teacher-forced forward + cross-entropy (GetError): src B x S and tgt_in/tgt_out B x T, all
  * column-major with -1 padding (source reversed + left-padded, target right-padded).

@@ -200,6 +200,24 @@ def beam_expand(p, step, prev_score, diversity=0.0, penalty=0.0, start_id=0, eof
     return dict(tok=tok, backptr=bp, score=sc, fin_beam=fb[:n].copy(), fin_score=fs[:n].copy())
 
 
+def beam_expand_ensemble(ps, step, prev_score, diversity=0.0, penalty=0.0, start_id=0, eof_id=1):
+    """ps: the models' (V, beam) probabilities.  Result as beam_expand."""
+    ps = [np.asfortranarray(p, np.float32) for p in ps]
+    V, beam = ps[0].shape
+    tok = np.empty(beam, np.int32)
+    bp = np.empty(beam, np.int32)
+    sc = np.empty(beam, np.float32)
+    fc = np.zeros(1, np.int32)
+    fb = np.zeros(max(beam, 1) * 2 + 4, np.int32)
+    fs = np.zeros(max(beam, 1) * 2 + 4, np.float32)
+    arr = (C.c_void_p * len(ps))(*[p.ctypes.data for p in ps])
+    lib().orc_beam_expand_ensemble(arr, len(ps), V, beam, step, _p(f32(prev_score)), _f(diversity),
+                                   _f(penalty), start_id, eof_id, _p(tok), _p(bp), _p(sc), _p(fc),
+                                   _p(fb), _p(fs))
+    n = int(fc[0])
+    return dict(tok=tok, backptr=bp, score=sc, fin_beam=fb[:n].copy(), fin_score=fs[:n].copy())
+
+
 def beam_gather(src, backptr):
     src = np.asfortranarray(src, np.float32)
     H, B = src.shape
@@ -287,9 +305,10 @@ class Model:
 
     def decode_sentence(self, src_ids, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0,
                         diversity=0.0, lp_alpha=0.65, cp_beta=0.20, num_threads=0, hyp_cap=4096,
-                        alignments=False):
+                        alignments=False, ensemble=()):
         """alignments=True: the reference's unk_replacement_mode__ (exported alignment scores,
-        coverage penalty on them); the result then holds best_viterbi."""
+        coverage penalty on them); the result then holds best_viterbi.  ensemble: further models
+        whose distributions are averaged with this one's before every beam step."""
         src_ids = i32(src_ids)
         cap = self.cfg.longest_sent + 2
         o = DecodeOpts(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta,
@@ -302,7 +321,17 @@ class Model:
         hs = np.zeros(hyp_cap, np.float32)
         nh = C.c_int(0)
         vit = np.full(cap, -1, np.int32)
-        if alignments:
+        if ensemble:
+            handles = (C.c_void_p * (1 + len(ensemble)))(self.handle, *[m.handle for m in ensemble])
+            f = lib().orc_decode_sentence_ensemble
+            f.restype = C.c_int
+            f.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int] + \
+                [C.c_void_p, C.c_int] + [C.c_void_p] * 6 + [C.c_int, C.c_void_p]
+            alignments = alignments and all(m.cfg.attention for m in (self,) + tuple(ensemble))
+            steps = f(handles, len(handles), _p(src_ids), src_ids.size, C.byref(o), int(alignments),
+                      _p(best), cap, C.byref(blen), C.byref(bscore), _p(vit), _p(ht), _p(hl), _p(hs),
+                      hyp_cap, C.byref(nh))
+        elif alignments:
             steps = lib().orc_decode_sentence_alignments(
                 self.handle, _p(src_ids), src_ids.size, C.byref(o), _p(best), cap, C.byref(blen),
                 C.byref(bscore), _p(vit), _p(ht), _p(hl), _p(hs), hyp_cap, C.byref(nh))

@@ -113,38 +113,51 @@ def encode(P, layers, H, src_ids):
 
 def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=True, max_ratio=1.5,
                 min_ratio=0.5, penalty=0.0, diversity=0.0, lp_alpha=0.65, cp_beta=0.2,
-                longest=104, margins=None, alignments=False):
+                longest=104, margins=None, alignments=False, ensemble=()):
     """Sort-based beam search with the reference's rules (src/decoder.h:355-699).  Returns
     (best_tokens, best_score, hyps); margins (list) collects the smallest score gaps seen, so a test
     can skip seeds whose decisions are closer than fp32 can resolve.
     alignments=True (the reference's unk_replacement_mode__): every token carries the attention
     weights over the source positions of the step that produced it; the coverage penalty is computed
     from them and a fourth result holds, per 1-best token, the source position of the largest
-    weight (-1 if none is positive)."""
+    weight (-1 if none is positive).
+    ensemble: parameter sets of further models of the same shape (EnsembleFactory with several
+    models): the step's distribution is the mean of the models' distributions, a token's alignment
+    weights are the sum of the models' weights."""
+    if ensemble:
+        return _beam_decode_ensemble([P] + list(ensemble), layers, H, V, src_ids, beam, D, attention,
+                                     feed_input, max_ratio, min_ratio, penalty, diversity, lp_alpha,
+                                     cp_beta, longest, margins, alignments)
+    return _beam_decode_ensemble([P], layers, H, V, src_ids, beam, D, attention, feed_input,
+                                 max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta, longest,
+                                 margins, alignments)
+
+
+def _beam_decode_ensemble(Ps, layers, H, V, src_ids, beam, D, attention, feed_input, max_ratio,
+                          min_ratio, penalty, diversity, lp_alpha, cp_beta, longest, margins,
+                          alignments):
     S = len(src_ids)
     beam = min(beam, int(np.sqrt(V)))
-    he, ce, top = encode(P, layers, H, src_ids)
-    h = [np.repeat(he[l], beam, axis=1) for l in range(layers)]
-    c = [np.repeat(ce[l], beam, axis=1) for l in range(layers)]
-    h_tild = np.zeros((H, beam))
+    M = len(Ps)
+    enc = [encode(P, layers, H, src_ids) for P in Ps]
+    hs = [[np.repeat(enc[k][0][l], beam, axis=1) for l in range(layers)] for k in range(M)]
+    cs = [[np.repeat(enc[k][1][l], beam, axis=1) for l in range(layers)] for k in range(M)]
+    h_tilds = [np.zeros((H, beam)) for _ in range(M)]
     tokens = np.zeros(beam, int)
     scores = np.zeros(beam)
     hist = [[0] for _ in range(beam)]
     ahist = [[] for _ in range(beam)]  # per token: dict source position -> attention weight
     hyps, hyp_align = [], []
-    D64 = P["softmax.D"].astype(np.float64)
-    bd = P["softmax.b_d"].astype(np.float64)
-    Wt = P["tgt.0.W"].astype(np.float64)
     ones = np.ones(beam, int)
     limit = min(int(np.float32(max_ratio) * S), longest - 2)
 
-    def forward(step):
-        nonlocal h, c
-        x = Wt[:, tokens]
+    def forward_one(k, step):
+        P, top = Ps[k], enc[k][2]
+        x = P["tgt.0.W"].astype(np.float64)[:, tokens]
         nh, nc = [], []
         for l in range(layers):
-            ht = h_tild if (l == 0 and feed_input and attention and step != 0) else None
-            a, b_, _ = lstm_step(P, f"tgt.{l}.", x, h[l], c[l], ht)
+            ht = h_tilds[k] if (l == 0 and feed_input and attention and step != 0) else None
+            a, b_, _ = lstm_step(P, f"tgt.{l}.", x, hs[k][l], cs[k][l], ht)
             nh.append(a)
             nc.append(b_)
             x = a
@@ -153,7 +166,21 @@ def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=Tr
         if attention:
             ht_new, al = attention_local_p(P, topv, lambda b, s: top[s], [S] * beam, ones, D)
             topv = ht_new
-        return nh, nc, ht_new, log_softmax(D64 @ topv + bd[:, None]), al
+        lp = log_softmax(P["softmax.D"].astype(np.float64) @ topv + P["softmax.b_d"].astype(np.float64)[:, None])
+        return nh, nc, ht_new, lp, al
+
+    def forward(step):
+        outs = [forward_one(k, step) for k in range(M)]
+        if M == 1:
+            lp, al = outs[0][3], outs[0][4]
+        else:
+            lp = np.log(np.mean([np.exp(o[3]) for o in outs], axis=0))
+            al = [{} for _ in range(beam)]
+            for o in outs:
+                for b in range(beam):
+                    for pos, a in o[4][b].items():
+                        al[b][pos] = al[b].get(pos, 0.0) + a
+        return [o[0] for o in outs], [o[1] for o in outs], [o[2] for o in outs], lp, al
 
     for step in range(limit):
         nh, nc, ht_new, lp, al = forward(step)
@@ -187,10 +214,11 @@ def beam_decode(P, layers, H, V, src_ids, beam, D, attention=True, feed_input=Tr
         ahist = [ahist[i] + [al[i]] for i in new_bp]
         tokens = np.array(new_tok)
         scores = np.array(new_sc)
-        h = [x[:, new_bp] for x in nh]
-        c = [x[:, new_bp] for x in nc]
-        if attention:
-            h_tild = ht_new[:, new_bp]
+        for k in range(M):
+            hs[k] = [x[:, new_bp] for x in nh[k]]
+            cs[k] = [x[:, new_bp] for x in nc[k]]
+            if attention:
+                h_tilds[k] = ht_new[k][:, new_bp]
     _, _, _, lp, al = forward(limit if limit > 0 else 1)
     for i in range(beam):
         hyps.append((hist[i] + [1], scores[i] + lp[1, i] + penalty))

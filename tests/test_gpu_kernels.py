@@ -650,6 +650,48 @@ def test_beam_topk_ties_take_lowest_id(lh):
     assert_close(host(cl, (K, B))[:, 0], np.full(K, -np.log(V)), "uniform log-prob")
 
 
+@pytest.mark.parametrize("V,B,K,n_models", [(30000, 24, 13, 3), (5000, 7, 13, 2), (50000, 5, 64, 8),
+                                            (1004, 12, 5, 1)])
+def test_beam_topk_ensemble(lh, V, B, K, n_models):
+    """lh_beam_topk_ensemble_f32 against EnsemblesModels' arithmetic in numpy: mean of the models'
+    probabilities taken in float64 and rounded to float32, divided by the float32 column sum of
+    those means, log.  Candidate ids bit for bit (value desc, id asc), scores within tolerance.
+    With n identical models the mean is the model's own distribution exactly."""
+    rng = np.random.default_rng(91)
+    ld = V + 4
+    ps = []
+    for _ in range(n_models):
+        z = uni(rng, V, B, s=4.0).astype(np.float64)
+        p = np.exp(z - z.max(axis=0)) / np.exp(z - z.max(axis=0)).sum(axis=0)
+        full = np.zeros((ld, B), np.float32)
+        full[:V] = p.astype(np.float32)
+        ps.append(full)
+    ps[0][[3, 900], 1] = ps[0][[17, 901], 1]                              # some exact ties
+    q = (sum(p[:V].astype(np.float64) for p in ps) / n_models).astype(np.float32)
+    norm = q.sum(axis=0, dtype=np.float64).astype(np.float32)
+    want_logp = np.log((q / norm).astype(np.float64))
+    cl = torch.empty(K * B, device="cuda")
+    ci = torch.empty(K * B, dtype=torch.int32, device="cuda")
+    le = torch.empty(B, device="cuda")
+    dps = [dev(p) for p in ps]
+    lh.beam_topk_ensemble(dps, ld, V, B, K, 1, cl, ci, le)
+    gi, gl = host(ci, (K, B)), host(cl, (K, B))
+    for b in range(B):
+        order = np.lexsort((np.arange(V), -q[:, b]))[:K]
+        assert np.array_equal(gi[:, b], order), f"column {b}"
+        assert_close(gl[:, b], want_logp[order, b], f"column {b} scores")
+    assert_close(host(le, (B,)), want_logp[1], "log p(<EOF>)")
+    # n copies of one model: exactly that model's own selection
+    lh.beam_topk_ensemble([dps[0]] * n_models, ld, V, B, K, 1, cl, ci, le)
+    one_i, one_l = host(ci, (K, B)).copy(), host(cl, (K, B)).copy()
+    lh.beam_topk_ensemble([dps[0]], ld, V, B, K, 1, cl, ci, le)
+    assert np.array_equal(one_i, host(ci, (K, B))) and np.array_equal(one_l, host(cl, (K, B)))
+    with pytest.raises(lh.LinmtHipError):                                  # unaligned leading dimension
+        lh.beam_topk_ensemble(dps, ld + 1, V, B, K, 1, cl, ci, le)
+    with pytest.raises(lh.LinmtHipError):
+        lh.beam_topk_ensemble(dps * 9, ld, V, B, K, 1, cl, ci, le)
+
+
 @pytest.mark.parametrize("V,K", [(30000, 13), (50000, 64), (5000, 13), (300, 64), (37, 5)])
 def test_beam_topk_adversarial_layouts(lh, V, K):
     """Layouts that stress the selection: the winners packed into the rows one thread owns (ids

@@ -114,6 +114,51 @@ def test_decode_with_exported_alignments_vs_oracle(orc, host):
         gm.close()
 
 
+def test_decode_ensemble_vs_oracle(orc, host):
+    """EnsembleFactory with several models: models of different width, depth and attention window
+    decode a ragged batch in lockstep, their distributions averaged before every beam step
+    (lh_beam_topk_ensemble_f32) -- against the oracle's ensemble search (pinned on the numpy model),
+    with and without exported alignments, whose scores are added up over the models.  An ensemble
+    of a model with itself gives the model's own translations."""
+    rng = np.random.default_rng(15)
+    Vs, Vt, beam, lens = 60, 72, 4, (9, 4, 12, 2, 7)
+    shapes = ((2, 48, 2), (1, 32, 3), (3, 40, 10))           # layers, H, D
+    pairs = [_pair(orc, host, rng, L, H, Vs, Vt, D, 30, 0.5, decoding=(len(lens), beam))
+             for L, H, D in shapes]
+    oms, gms = [p[1] for p in pairs], [p[2] for p in pairs]
+    sents = [rng.integers(0, Vs, size=n) for n in lens]
+    for n_models in (2, 3):
+        for kw in (dict(), dict(alignments=True, cp_beta=0.6, lp_alpha=0.3)):
+            got = gms[0].decode_batch(sents, beam=beam, with_hyps=True, ensemble=gms[1:n_models], **kw)
+            for i, s in enumerate(sents):
+                want = oms[0].decode_sentence(s, beam=beam, ensemble=tuple(oms[1:n_models]), **kw)
+                _compare_decode(want, got[i], f"{n_models} models {kw} sentence {i} (len {len(s)})")
+                if kw:
+                    assert got[i]["best_viterbi"].tolist() == want["best_viterbi"].tolist(), (i, n_models)
+    alone = gms[0].decode_batch(sents, beam=beam, with_hyps=True)
+    # a second model with the same parameters
+    L0, H0, D0 = shapes[0]
+    twin = host.Model(L0, H0, Vs, Vt, longest_sentence=30, attention_mode=1, attention_width=D0,
+                      feed_input=True, minibatch_size=1, decoding=(len(lens), beam))
+    twin.set_params(pairs[0][0])
+    both = gms[0].decode_batch(sents, beam=beam, with_hyps=True, ensemble=[twin])
+    for a, b in zip(alone, both):
+        assert a["best"].tolist() == b["best"].tolist()
+        assert len(a["hyps"]) == len(b["hyps"])
+        for (at, as_), (bt, bs) in zip(a["hyps"], b["hyps"]):
+            assert at.tolist() == bt.tolist()
+            assert abs(as_ - bs) <= 1e-4 * max(1.0, abs(as_))
+    # and afterwards every model still decodes on its own
+    again = gms[0].decode_batch(sents, beam=beam, with_hyps=True)
+    for a, b in zip(alone, again):
+        assert a["best"].tolist() == b["best"].tolist() and a["best_score"] == b["best_score"]
+    with pytest.raises(host.HostError):
+        gms[0].decode_batch(sents, beam=beam, ensemble=[gms[0]])
+    twin.close()
+    for g in gms:
+        g.close()
+
+
 def test_decode_no_attention_and_no_feed(orc, host):
     rng = np.random.default_rng(5)
     for attention, feed in ((0, False), (1, False)):

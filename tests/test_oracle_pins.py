@@ -329,6 +329,76 @@ def test_decode_sentence_with_exported_alignments_vs_numpy(orc):
     assert checked >= 5 and differs >= 3  # the penalty really is computed from the scores
 
 
+def test_beam_expand_ensemble_pins(orc):
+    """EnsemblesModels in front of the expansion: n copies of one distribution expand exactly like
+    the distribution alone; different distributions expand exactly like their float64 mean rounded
+    to float32 (the averaging restated in numpy), and like the brute-force expansion of that mean."""
+    rng = np.random.default_rng(41)
+    V, beam = 53, 4
+    for step in (0, 3):
+        ps = []
+        for _ in range(3):
+            z = rng.normal(size=(V, beam)) * 2
+            ps.append((np.exp(z) / np.exp(z).sum(axis=0)).astype(np.float32))
+        prev = rng.uniform(-3, 0, size=beam).astype(np.float32)
+        alone = orc.beam_expand(ps[0], step, prev, diversity=0.1, penalty=0.2)
+        copies = orc.beam_expand_ensemble([ps[0]] * 3, step, prev, diversity=0.1, penalty=0.2)
+        mixed = orc.beam_expand_ensemble(ps, step, prev, diversity=0.1, penalty=0.2)
+        mean = (sum(p.astype(np.float64) for p in ps) / 3).astype(np.float32)
+        of_mean = orc.beam_expand(mean, step, prev, diversity=0.1, penalty=0.2)
+        for key in ("tok", "backptr", "score", "fin_beam", "fin_score"):
+            assert np.array_equal(alone[key], copies[key]), key
+            assert np.array_equal(mixed[key], of_mean[key]), key
+        tok, bp, sc, fb, fs = _bruteforce_expand(mean, step, prev, 0.1, 0.2, beam)
+        if len(tok) == beam:
+            assert mixed["tok"].tolist() == tok and mixed["backptr"].tolist() == bp
+            assert_close(mixed["score"], sc, "beam scores", rtol=1e-6, atol=1e-6)
+
+
+def test_decode_sentence_ensemble_pins(orc):
+    """Two copies of one model decode exactly like the model alone (tokens, hypotheses, scores,
+    alignments); two different models decode like the numpy beam search over the mean of their
+    distributions, with and without exported alignments."""
+    rng = np.random.default_rng(43)
+    checked = 0
+    for trial in range(12):
+        P1, m1 = _tiny_model(orc, rng)
+        P2, m2 = _tiny_model(orc, rng)
+        S = int(rng.integers(3, 9))
+        src = rng.integers(0, 30, size=S)
+        for al in (False, True):
+            alone = m1.decode_sentence(src, beam=3, alignments=al)
+            twice = m1.decode_sentence(src, beam=3, alignments=al, ensemble=(m1,))
+            assert alone["best"].tolist() == twice["best"].tolist()
+            assert len(alone["hyps"]) == len(twice["hyps"])
+            for (at, as_), (tt, ts) in zip(alone["hyps"], twice["hyps"]):
+                assert at.tolist() == tt.tolist() and as_ == ts
+            if not al:
+                assert alone["best_score"] == twice["best_score"]
+            else:
+                # the summed alignment scores are twice the model's own: same arg-max
+                assert alone["best_viterbi"].tolist() == twice["best_viterbi"].tolist()
+        margins = []
+        best, best_s, hyps, vit = R.beam_decode(P1, 2, 12, 37, src, beam=3, D=2, longest=40,
+                                                margins=margins, alignments=True, ensemble=[P2])
+        if min(margins) < 1e-4:
+            continue
+        got = m1.decode_sentence(src, beam=3, alignments=True, ensemble=(m2,))
+        assert got["best"].tolist() == list(best)
+        assert_close(got["best_score"], best_s, "rescored 1-best", rtol=1e-4, atol=1e-4)
+        assert got["best_viterbi"].tolist() == vit
+        assert len(got["hyps"]) == len(hyps)
+        for (gt, gs), (wt, ws) in zip(got["hyps"], hyps):
+            assert gt.tolist() == list(wt)
+            assert_close(gs, ws, "hypothesis score", rtol=1e-4, atol=1e-4)
+        best0, s0, hyps0 = R.beam_decode(P1, 2, 12, 37, src, beam=3, D=2, longest=40, ensemble=[P2])
+        got0 = m1.decode_sentence(src, beam=3, ensemble=(m2,))
+        assert got0["best"].tolist() == list(best0)
+        assert_close(got0["best_score"], s0, "rescored 1-best", rtol=1e-4, atol=1e-4)
+        checked += 1
+    assert checked >= 5
+
+
 def test_forward_xent_vs_numpy(orc):
     """Teacher-forced forward + CE on a ragged minibatch (reversed, left-padded source; right-padded
     target; -1 padding) against the float64 numpy model run sentence by sentence."""
