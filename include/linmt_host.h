@@ -234,6 +234,11 @@ typedef struct lnmt_decoding_options {
   int print_decoding_information, print_alignments_scores, unk_replacement_mode;
   int sentences_per_batch;
   int num_hypotheses; /* k-best list per sentence, closed by a line of '=' when != 1; <= 0: 1 */
+  /* further model files of an ensemble (the reference's several --decoding models,
+   * src/global_configuration.cc:964-1005): the source text is integerised once per model with
+   * the model's own source vocabulary; the target vocabulary must be model_file's.  NULL / 0: none */
+  const char *const *ensemble_model_files;
+  int n_ensemble_models;
 } lnmt_decoding_options;
 int lnmt_decoding(const lnmt_decoding_options *o, int *sentences, int *sentences_thrown_away,
                   long long *source_words, long long *target_words, double *seconds);

@@ -55,7 +55,8 @@ class DecodingOptions(C.Structure):
                 ("longest_sentence", C.c_int), ("attention_width", C.c_int),
                 ("print_decoding_information", C.c_int),
                 ("print_alignments_scores", C.c_int), ("unk_replacement_mode", C.c_int),
-                ("sentences_per_batch", C.c_int), ("num_hypotheses", C.c_int)]
+                ("sentences_per_batch", C.c_int), ("num_hypotheses", C.c_int),
+                ("ensemble_model_files", C.POINTER(C.c_char_p)), ("n_ensemble_models", C.c_int)]
 
 
 class DecodeOptions(C.Structure):
@@ -395,14 +396,16 @@ def decoding(model_file, source_file, final_file, ids_file=None, beam=12, penalt
              max_ratio=1.5, min_ratio=0.5, lp_alpha=0.65, cp_beta=0.20, diversity=0.0,
              longest_sentence=200, attention_width=10, print_decoding_information=False,
              print_alignments_scores=False, unk_replacement_mode=False, sentences_per_batch=64,
-             num_hypotheses=1):
-    """Dispatcher::Decoding: translate a text file with a reference model file."""
+             num_hypotheses=1, ensemble_model_files=()):
+    """Dispatcher::Decoding: translate a text file with a reference model file (or with an
+    ensemble: model_file plus ensemble_model_files)."""
     enc = lambda p: None if p is None else os.fsencode(p)  # noqa: E731
+    more = (C.c_char_p * max(1, len(ensemble_model_files)))(*[enc(f) for f in ensemble_model_files])
     o = DecodingOptions(enc(model_file), enc(source_file), enc(ids_file), enc(final_file), beam,
                         penalty, max_ratio, min_ratio, lp_alpha, cp_beta, diversity,
                         longest_sentence, attention_width, int(print_decoding_information),
                         int(print_alignments_scores), int(unk_replacement_mode),
-                        sentences_per_batch, num_hypotheses)
+                        sentences_per_batch, num_hypotheses, more, len(ensemble_model_files))
     n, thrown, sw, tw, secs = C.c_int(), C.c_int(), C.c_longlong(), C.c_longlong(), C.c_double()
     _check(load().lnmt_decoding(C.byref(o), C.byref(n), C.byref(thrown), C.byref(sw), C.byref(tw),
                                 C.byref(secs)), "decoding")

@@ -475,6 +475,11 @@ extern "C" int lnmt_decoding(const lnmt_decoding_options *o, int *sentences, int
     c.unk_replacement_mode_ = o->unk_replacement_mode != 0;
     if (o->sentences_per_batch > 0) c.sentences_per_batch_ = o->sentences_per_batch;
     if (o->num_hypotheses > 0) c.hypotheses_number_ = o->num_hypotheses;
+    for (int k = 0; k < o->n_ensemble_models; ++k) {
+      if (!o->ensemble_model_files || !o->ensemble_model_files[k])
+        throw LinmtError("lnmt_decoding: ensemble model file is NULL");
+      c.ensemble_model_names_.push_back(o->ensemble_model_files[k]);
+    }
     const DecodingReport r = Dispatcher::Decoding(c);
     if (sentences) *sentences = r.sentences;
     if (sentences_thrown_away) *sentences_thrown_away = r.sentences_thrown_away;

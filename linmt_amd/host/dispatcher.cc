@@ -112,9 +112,9 @@ static void WriteHypothesisLines(std::ostream &out, const SentenceResult &r, int
   else if (n == 0) out << "\n";
 }
 
-DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
-  DecodingReport report;
-  const ModelInformation info = ReadModelInformation(c.model_name_);
+static GlobalConfiguration DecodingModelConfiguration(const std::string &model_name,
+                                                      const DecodingConfiguration &c) {
+  const ModelInformation info = ReadModelInformation(model_name);
   GlobalConfiguration g;
   g.num_layers_ = info.num_layers;
   g.lstm_size_ = info.lstm_size;
@@ -126,6 +126,12 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
   g.attention_width_ = c.attention_width_;
   g.feed_input_mode_ = info.feed_input != 0;
   g.sequence_to_sequence_mode_ = true;
+  return g;
+}
+
+DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
+  DecodingReport report;
+  const GlobalConfiguration g = DecodingModelConfiguration(c.model_name_, c);
 
   InputFilePreprocess input_helper;
   std::vector<std::vector<int>> sentences;
@@ -147,6 +153,26 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
   NeuralMachineTranslation neural(g);
   neural.InitModelDecoding(n_sent, beam);
   neural.LoadWeights(c.model_name_);
+  // the other models of an ensemble, each with its own integerised copy of the text
+  std::vector<std::unique_ptr<NeuralMachineTranslation>> others;
+  std::vector<NeuralMachineTranslation *> ensemble;
+  std::vector<std::vector<std::vector<int>>> other_sentences;
+  bool all_attention = g.attention_mode_ != 0;
+  for (const std::string &name : c.ensemble_model_names_) {
+    const GlobalConfiguration gk = DecodingModelConfiguration(name, c);
+    if (gk.target_vocab_size_ != g.target_vocab_size_)
+      throw LinmtError("Decoding: the models of an ensemble must share the target vocabulary");
+    all_attention = all_attention && gk.attention_mode_ != 0;
+    other_sentences.emplace_back();
+    std::vector<int> kept_k;
+    input_helper.IntegerizeFileDecoding(name, c.decode_user_file_, c.longest_sentence_,
+                                        &other_sentences.back(), &kept_k);
+    if (kept_k != kept) throw LinmtError("Decoding: the models of an ensemble keep different sentences");
+    others.emplace_back(new NeuralMachineTranslation(gk));
+    others.back()->InitModelDecoding(n_sent, beam);
+    others.back()->LoadWeights(name);
+    ensemble.push_back(others.back().get());
+  }
 
   DecodeOptions o;
   o.beam_size_ = c.beam_size_;
@@ -156,7 +182,7 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
   o.diversity_ = c.decoding_diversity_;
   o.lp_alpha_ = c.decoding_lp_alpha_;
   o.cp_beta_ = c.decoding_cp_beta_;
-  o.unk_replacement_mode_ = c.unk_replacement_mode_ && g.attention_mode_;
+  o.unk_replacement_mode_ = c.unk_replacement_mode_ && all_attention;
   o.hypotheses_number_ = std::max(1, c.hypotheses_number_);
 
   const std::string ids_file =
@@ -168,15 +194,17 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
     for (size_t first = 0; first < sentences.size(); first += n_sent) {
       // an empty source line cannot be encoded: it translates to an empty line
       std::vector<std::vector<int>> batch;
+      std::vector<std::vector<std::vector<int>>> other_batches(ensemble.size());
       std::vector<size_t> where;
       const size_t last = std::min(sentences.size(), first + n_sent);
       for (size_t i = first; i < last; ++i)
         if (!sentences[i].empty()) {
           batch.push_back(sentences[i]);
+          for (size_t k = 0; k < ensemble.size(); ++k) other_batches[k].push_back(other_sentences[k][i]);
           where.push_back(i - first);
         }
       std::vector<SentenceResult> results, ordered(last - first);
-      if (!batch.empty()) neural.DecodeBatch(batch, o, &results);
+      if (!batch.empty()) neural.DecodeBatch(batch, o, &results, ensemble, other_batches);
       for (size_t b = 0; b < batch.size(); ++b) ordered[where[b]] = std::move(results[b]);
       for (size_t i = first; i < last; ++i) {
         WriteHypothesisLines(output, ordered[i - first], (int)sentences[i].size(), c);

@@ -52,6 +52,10 @@ struct TuningReport {
 // same names and defaults, plus the batch size of this implementation.
 struct DecodingConfiguration {
   std::string model_name_;           // the reference's text model file
+  // further models of an ensemble (the reference's model_names_[1..]): the source text is
+  // integerised once per model with the model's own source vocabulary; the target vocabulary and
+  // the un-integerisation are the first model's
+  std::vector<std::string> ensemble_model_names_;
   std::string decode_user_file_;     // source sentences, one per line, tokenised text
   std::string decoder_output_file_;  // ids of the translations ("" = decoder_final_file_ + ".ids")
   std::string decoder_final_file_;   // the translations as words

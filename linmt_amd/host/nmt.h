@@ -470,10 +470,14 @@ class NeuralMachineTranslation {
   // `ensemble`: further models decoded in lockstep with this one (EnsembleFactory,
   // decoder.h:1778-1931): their distributions are averaged with this model's before every beam
   // step.  They must be initialised for decoding with the same n_sent, beam, target vocabulary
-  // and longest sentence; hidden size, depth and attention may differ.
+  // and longest sentence; hidden size, depth and attention may differ.  ensemble_sentences: the
+  // same sentences integerised with the source vocabulary of each further model (the reference
+  // integerises the text once per model, global_configuration.cc:985); empty = they share this
+  // model's source ids.
   void DecodeBatch(const std::vector<std::vector<int>> &sentences, const DecodeOptions &o,
                    std::vector<SentenceResult> *results,
-                   const std::vector<NeuralMachineTranslation *> &ensemble = {});
+                   const std::vector<NeuralMachineTranslation *> &ensemble = {},
+                   const std::vector<std::vector<std::vector<int>>> &ensemble_sentences = {});
 
   // ---- training --------------------------------------------------------------------------------
   DeviceArray<double> p_device_norm_workspace_, p_device_norms_;

@@ -583,7 +583,8 @@ void Decoder::OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_le
 void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &sentences,
                                            const DecodeOptions &o,
                                            std::vector<SentenceResult> *results,
-                                           const std::vector<NeuralMachineTranslation *> &ensemble) {
+                                           const std::vector<NeuralMachineTranslation *> &ensemble,
+                                           const std::vector<std::vector<std::vector<int>>> &ensemble_sentences) {
   if (!decode_mode_) throw LinmtError("DecodeBatch: call InitModelDecoding first");
   // EnsembleFactory (decoder.h:1702-1931): every model runs the same columns in lockstep, each on
   // its own stream; this model owns the beam search, the others hand it their distributions.
@@ -600,6 +601,16 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   }
   const int n_models = (int)models.size();
   if (n_models > LH_ENSEMBLE_MAX_MODELS) throw LinmtError("DecodeBatch: too many models");
+  if (!ensemble_sentences.empty()) {
+    if (ensemble_sentences.size() != ensemble.size())
+      throw LinmtError("DecodeBatch: one set of source ids per ensemble model");
+    for (const auto &set : ensemble_sentences) {
+      if (set.size() != sentences.size()) throw LinmtError("DecodeBatch: ensemble source ids: sentence count differs");
+      for (size_t i = 0; i < set.size(); ++i)
+        if (set[i].size() != sentences[i].size())
+          throw LinmtError("DecodeBatch: ensemble source ids: sentence length differs");
+    }
+  }
   if (n_models > 1 && cfg_.target_vocab_size_ % 4 != 0)
     throw LinmtError("DecodeBatch: an ensemble needs a target vocabulary that is a multiple of 4");
   const int n = (int)sentences.size();
@@ -652,6 +663,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
     int *indices;
   };
   std::vector<NodeBuffers> node_buffers(n_models, NodeBuffers{nullptr, nullptr});
+  std::vector<std::vector<int>> src_own;
   std::vector<size_t> hist_slices(n_models, 0);
 
   for (int k = 0; k < n_models; ++k) {
@@ -668,7 +680,19 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
     // smaller batch simply uses the first n columns of every step's buffer)
     if (n != n_sent_ && M.cfg_.attention_mode_)
       M.attention_layer_.hs_step_stride_ = (long long)H * n_sent_;
-    M.ForwardPropSource(src.data(), S, n);
+    if (k > 0 && !ensemble_sentences.empty()) {
+      // this model's own ids of the same words, laid out like `src`
+      src_own.emplace_back((size_t)n * S, -1);  // kept alive until the streams have been synchronised
+      std::vector<int> &own = src_own.back();
+      for (int q = 0; q < n; ++q) {
+        const std::vector<int> &w = ensemble_sentences[k - 1][order[q]];
+        const int len = (int)w.size();
+        for (int t = 0; t < len; ++t) own[(size_t)(S - len + t) * n + q] = w[len - 1 - t];
+      }
+      M.ForwardPropSource(own.data(), S, n);
+    } else {
+      M.ForwardPropSource(src.data(), S, n);
+    }
     if (M.cfg_.attention_mode_)
       M.attention_layer_.BuildProjectedMemory(S, M.SourceLayer(L - 1).h_all_.size());
 

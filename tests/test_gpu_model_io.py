@@ -136,6 +136,62 @@ def test_decoding_a_text_file(host, tmp_path):
     assert rep["target_words"] == sum(len(w["best"]) for w in want)
 
 
+def test_decoding_a_text_file_with_an_ensemble(host, tmp_path):
+    """Dispatcher::Decoding with two model files: the text is integerised once per model, with the
+    model's own source vocabulary (the second model knows fewer words, so some of them are <UNK>
+    for it only), the models decode in lockstep and the first model's target vocabulary spells the
+    output.  Expected: DecodeBatch on the shared ids with a stand-in for the second model whose
+    embedding table repeats the <UNK> column for the words it does not know."""
+    rng = np.random.default_rng(18)
+    Vt, D, beam = 40, 2, 4
+    kw = dict(longest_sentence=24, attention_mode=1, attention_width=D, feed_input=True)
+    PA = R.make_params(rng, 2, 24, 30, Vt, attention=True, feed_input=True, scale=0.5)
+    PB30 = R.make_params(rng, 1, 16, 30, Vt, attention=True, feed_input=True, scale=0.5)
+    PB30["src.0.W"][:, 20:] = PB30["src.0.W"][:, [0]]
+    PB20 = dict(PB30)
+    PB20["src.0.W"] = np.ascontiguousarray(PB30["src.0.W"][:, :20])
+    files = []
+    for name, (L, H, Vs, P) in dict(a=(2, 24, 30, PA), b=(1, 16, 20, PB20)).items():
+        m = host.Model(L, H, Vs, Vt, minibatch_size=1, **kw)
+        m.set_params(P)
+        files.append(str(tmp_path / f"{name}.nmt"))
+        m.dump_model(files[-1])
+        m.close()
+    lens = [5, 8, 3, 6, 2]
+    sents = [rng.integers(1, 30, size=n) for n in lens]
+    assert any((s_ >= 20).any() for s_ in sents)
+    src = tmp_path / "src.txt"
+    src.write_text("\n".join(" ".join(f"w{i}" for i in s_) for s_ in sents) + "\n")
+    final, ids = str(tmp_path / "out.txt"), str(tmp_path / "out.ids")
+    rep = host.decoding(files[0], str(src), final, ids_file=ids, beam=beam, longest_sentence=24,
+                        attention_width=D, print_decoding_information=True, unk_replacement_mode=True,
+                        sentences_per_batch=3, ensemble_model_files=files[1:])
+    assert rep["sentences"] == len(lens) and rep["sentences_thrown_away"] == 0
+
+    a = host.Model(2, 24, 30, Vt, decoding=(3, beam), **kw)
+    a.load_weights(files[0])
+    b = host.Model(1, 16, 30, Vt, decoding=(3, beam), **kw)
+    b.set_params(PB30)
+    want = []
+    for group in (sents[0:3], sents[3:5]):
+        want += a.decode_batch(group, beam=beam, alignments=True, ensemble=[b])
+    alone = []
+    for group in (sents[0:3], sents[3:5]):
+        alone += a.decode_batch(group, beam=beam, alignments=True)
+    got_ids = open(ids).read().split("\n")[:-1]
+    assert len(got_ids) == len(lens)
+    for k, (line, w) in enumerate(zip(got_ids, want)):
+        fields = line.split(" |||| ")
+        assert [int(x) for x in fields[0].split()] == w["best"].tolist(), k
+        assert np.isclose(float(fields[1]), w["best_score"], rtol=1e-4, atol=1e-5)
+        assert [int(x) for x in fields[2].split()] == w["best_viterbi"].tolist(), k
+    # the second model really takes part
+    assert any(x["best"].tolist() != y["best"].tolist() or abs(x["best_score"] - y["best_score"]) > 1e-3
+               for x, y in zip(want, alone))
+    a.close()
+    b.close()
+
+
 def test_k_best_lists(host, tmp_path):
     """Decoder::OutputKBestHypotheses with hypotheses_number_ > 1 (src/decoder.h:529-607, 692-694):
     the kept hypotheses are the k best final scores among those that pass the length filter, best
