@@ -75,9 +75,11 @@ bool DecoderSentence::GeneralSettings(std::map<std::string, std::string> &m_para
 
   if (!has("--nmt-model")) throw LinmtError("you must assign --nmt-model in config file!");
   const std::vector<std::string> model_names = SplitAt(m_parameters["--nmt-model"], ' ');
-  if (model_names.size() != 1)
-    throw LinmtError("--nmt-model: exactly one model file (ensembles are not part of this library)");
+  if (model_names.empty()) throw LinmtError("you must assign --nmt-model in config file!");
+  // several files: an ensemble; sentences are integerised with the first model's vocabulary
+  // (src/decoder_sentence.cu:21)
   c.model_name_ = model_names[0];
+  c.ensemble_model_names_.assign(model_names.begin() + 1, model_names.end());
   if (has("--nbest") && std::stoi(m_parameters["--nbest"]) != 1)
     throw LinmtError("--nbest: only the best hypothesis is returned by this library");
   if (has("--multi-gpu") && SplitAt(m_parameters["--multi-gpu"], ' ').size() != model_names.size())
@@ -175,25 +177,42 @@ bool DecoderSentence::Init(const std::string &config, bool load_model) {
   GeneralSettings(m_parameters);
   LoadParallelVocabulary(configuration_.model_name_, target_vocab_size_);
 
-  const ModelInformation info = ReadModelInformation(configuration_.model_name_);
-  attention_model_mode_ = info.attention_model != 0;
+  std::vector<std::string> names(1, configuration_.model_name_);
+  names.insert(names.end(), configuration_.ensemble_model_names_.begin(),
+               configuration_.ensemble_model_names_.end());
+  attention_model_mode_ = true;
+  std::vector<GlobalConfiguration> configs;
+  for (const std::string &name : names) {
+    const ModelInformation info = ReadModelInformation(name);
+    attention_model_mode_ = attention_model_mode_ && info.attention_model != 0;
+    GlobalConfiguration g;
+    g.num_layers_ = info.num_layers;
+    g.lstm_size_ = info.lstm_size;
+    g.embedding_size_ = info.lstm_size;
+    g.source_vocab_size_ = info.source_vocab_size;
+    g.target_vocab_size_ = info.target_vocab_size;
+    g.longest_sentence_ = configuration_.longest_sentence_;
+    g.attention_mode_ = info.attention_model ? 1 : 0;
+    g.attention_width_ = configuration_.attention_width_;
+    g.feed_input_mode_ = info.feed_input != 0;
+    g.sequence_to_sequence_mode_ = true;
+    if (!configs.empty() && (g.target_vocab_size_ != configs[0].target_vocab_size_ ||
+                             g.source_vocab_size_ != configs[0].source_vocab_size_))
+      throw LinmtError("--nmt-model: the models of an ensemble must share both vocabularies");
+    configs.push_back(g);
+  }
   if (!load_model) return true;
-  GlobalConfiguration g;
-  g.num_layers_ = info.num_layers;
-  g.lstm_size_ = info.lstm_size;
-  g.embedding_size_ = info.lstm_size;
-  g.source_vocab_size_ = info.source_vocab_size;
-  g.target_vocab_size_ = info.target_vocab_size;
-  g.longest_sentence_ = configuration_.longest_sentence_;
-  g.attention_mode_ = info.attention_model ? 1 : 0;
-  g.attention_width_ = configuration_.attention_width_;
-  g.feed_input_mode_ = info.feed_input != 0;
-  g.sequence_to_sequence_mode_ = true;
   int beam = configuration_.beam_size_;
-  if (beam > (int)std::sqrt((double)g.target_vocab_size_)) beam = (int)std::sqrt((double)g.target_vocab_size_);
-  neural_.reset(new NeuralMachineTranslation(g));
-  neural_->InitModelDecoding(1, beam);
-  neural_->LoadWeights(configuration_.model_name_);
+  const int Vt = configs[0].target_vocab_size_;
+  if (beam > (int)std::sqrt((double)Vt)) beam = (int)std::sqrt((double)Vt);
+  ensemble_.clear();
+  for (size_t k = 0; k < names.size(); ++k) {
+    std::unique_ptr<NeuralMachineTranslation> m(new NeuralMachineTranslation(configs[k]));
+    m->InitModelDecoding(1, beam);
+    m->LoadWeights(names[k]);
+    if (k == 0) neural_ = std::move(m);
+    else ensemble_.push_back(std::move(m));
+  }
   return true;
 }
 
@@ -221,7 +240,9 @@ bool DecoderSentence::Process(const std::string &input_sentence, std::string &ou
   // DecodeBatch takes reading order and reverses by itself
   std::vector<std::vector<int>> batch(1, std::vector<int>(v_input_sentence_int.rbegin(), v_input_sentence_int.rend()));
   std::vector<SentenceResult> results;
-  neural_->DecodeBatch(batch, o, &results);
+  std::vector<NeuralMachineTranslation *> others;
+  for (auto &m : ensemble_) others.push_back(m.get());
+  neural_->DecodeBatch(batch, o, &results, others);
   std::ostringstream ids;
   WriteHypothesis(ids, results[0], source_length, c.print_decoding_information_mode_,
                   c.print_alignments_scores_mode_);

@@ -44,6 +44,7 @@ class DecoderSentence {
   int target_vocab_size_ = 0;
   bool attention_model_mode_ = false;
   std::unique_ptr<NeuralMachineTranslation> neural_;
+  std::vector<std::unique_ptr<NeuralMachineTranslation>> ensemble_;  // --nmt-model files 2..n
 };
 
 }  // namespace linmt

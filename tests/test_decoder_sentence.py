@@ -59,7 +59,7 @@ def test_config_file_and_settings(tmp_path):
     ('param="--nmt-model" value="{m}"\nparam="--beam-size" value="0"\n', "beam 0"),
     ('param="--nmt-model" value="{m}"\nparam="--decoding-ratio" value="1"\n', "one ratio"),
     ('param="--nmt-model" value="{m}"\nparam="--decoding-ratio" value="2 1"\n', "min >= max"),
-    ('param="--nmt-model" value="{m} {m}"\n', "an ensemble"),
+    ('param="--nmt-model" value="{m} /no/such/second.nmt"\n', "an ensemble with a missing file"),
     ('param="--nmt-model" value="{m}"\nparam="--nbest" value="3"\n', "n-best list"),
     ('param="--nmt-model" value="{m}"\nparam="--multi-gpu" value="0 1"\n', "gpus != models"),
     ('param="--nmt-model" value="/no/such/model.nmt"\n', "missing model file"),
@@ -110,12 +110,28 @@ def test_translations_match_decode_batch(tmp_path):
     d = host.DecoderSentence(str(cfg))
     b = host.Model(layers, H, Vs, Vt, decoding=(1, beam), **kw)
     b.load_weights(model)
+    # a second model file: the service then decodes with the ensemble of the two
+    P2 = R.make_params(rng, 1, 16, Vs, Vt, attention=True, feed_input=True, scale=0.5)
+    a2 = host.Model(1, 16, Vs, Vt, minibatch_size=1, **kw)
+    a2.set_params(P2)
+    model2 = str(tmp_path / "model2.nmt")
+    a2.dump_model(model2)
+    cfg2 = tmp_path / "ensemble.config"
+    cfg2.write_text(cfg.read_text().replace(f'value="{model}"', f'value="{model} {model2}"'))
+    d2 = host.DecoderSentence(str(cfg2))
+    b2 = host.Model(1, 16, Vs, Vt, decoding=(1, beam), **kw)
+    b2.load_weights(model2)
     word = lambda i: "<UNK>" if i == 0 else f"w{i}"  # noqa: E731
     tword = lambda i: ["<START>", "<EOF>", "<UNK>"][i] if i < 3 else f"w{i}"  # noqa: E731
     for n in (6, 1, 11, 3):
         sent = rng.integers(0, Vs, size=n)
         text = d.process(" ".join(word(i) for i in sent) + " |||| not part of the sentence")
         w = b.decode_batch([sent], beam=beam, alignments=True, min_ratio=0.0, max_ratio=2.0)[0]
+        text2 = d2.process(" ".join(word(i) for i in sent))
+        w2 = b.decode_batch([sent], beam=beam, alignments=True, min_ratio=0.0, max_ratio=2.0,
+                            ensemble=[b2])[0]
+        assert text2.split(" |||| ")[0].split() == [tword(t) for t in w2["best"].tolist()]
+        assert np.isclose(float(text2.split(" |||| ")[1]), w2["best_score"], rtol=1e-4, atol=1e-5)
         fields = text.split(" |||| ")
         assert len(fields) == 5, text
         assert fields[0].split() == [tword(t) for t in w["best"].tolist()]
