@@ -144,6 +144,13 @@ def bench_fused_kernels(torch, steps, warmup):
             lambda: lh.logsoftmax_xent(z, V, None, V, B, tgt, m, lp, loss))
         add("beam_topk (log-softmax + top-13)", f"V={V} B={B}", 4.0 * V * B,
             lambda: lh.beam_topk(z, V, None, V, B, K, 1, cl, ci, le))
+        if B == 768:
+            # an ensemble of two models: both distributions are read once
+            p2 = torch.empty(V * B, device=dev)
+            lh.softmax_fwd(f(V * B), V, None, V, B, p2, V)
+            add("beam_topk_ensemble (2 models, mean + top-13)", f"V={V} B={B}", 8.0 * V * B,
+                lambda: lh.beam_topk_ensemble([p, p2], V, V, B, K, 1, cl, ci, le))
+            del p2
         del z, p
     for H, B, S, D, per in ((1000, 768, 60, 10, 12), (1000, 768 * 16, 60, 10, 1)):
         ncol = B // per
