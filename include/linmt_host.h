@@ -257,7 +257,8 @@ int lnmt_unint_file(const char *model_file, const char *unint_file, const char *
  * configuration file of lines `param="--key" value="..."` (keys: --nmt-model (required; several
  * files separated by blanks are decoded as an ensemble, the first one's vocabularies serving all,
  * src/decoder_sentence.cu:21-28), --beam-size, --longest-sent, --attention-width, --decoding-ratio "min max", --lp-alpha,
- * --cp-beta, --diversity, --print-decoding-info, --print-align-scores, --nbest (1), --multi-gpu),
+ * --cp-beta, --diversity, --print-decoding-info, --print-align-scores, --nbest (accepted, a sentence always comes back as its one best hypothesis,
+ * src/decoder.h:703), --multi-gpu),
  * the vocabularies and, with load_model != 0, the weights (GPU).  NULL on error.  process
  * translates one tokenised sentence (text after " |||| " is ignored): words of the best
  * hypothesis, then with --print-decoding-info " |||| score |||| alignments |||| <UNK> alignments".

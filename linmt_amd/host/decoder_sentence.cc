@@ -80,8 +80,9 @@ bool DecoderSentence::GeneralSettings(std::map<std::string, std::string> &m_para
   // (src/decoder_sentence.cu:21)
   c.model_name_ = model_names[0];
   c.ensemble_model_names_.assign(model_names.begin() + 1, model_names.end());
-  if (has("--nbest") && std::stoi(m_parameters["--nbest"]) != 1)
-    throw LinmtError("--nbest: only the best hypothesis is returned by this library");
+  // --nbest is read by the reference and handed to its decoder, but a sentence always comes back
+  // as its one best hypothesis (Decoder::ObtainOneBestHypothesis, src/decoder.h:703): accepted,
+  // without effect
   if (has("--multi-gpu") && SplitAt(m_parameters["--multi-gpu"], ' ').size() != model_names.size())
     throw LinmtError("for decoding, each model must be specified a gpu");
 

@@ -60,7 +60,6 @@ def test_config_file_and_settings(tmp_path):
     ('param="--nmt-model" value="{m}"\nparam="--decoding-ratio" value="1"\n', "one ratio"),
     ('param="--nmt-model" value="{m}"\nparam="--decoding-ratio" value="2 1"\n', "min >= max"),
     ('param="--nmt-model" value="{m} /no/such/second.nmt"\n', "an ensemble with a missing file"),
-    ('param="--nmt-model" value="{m}"\nparam="--nbest" value="3"\n', "n-best list"),
     ('param="--nmt-model" value="{m}"\nparam="--multi-gpu" value="0 1"\n', "gpus != models"),
     ('param="--nmt-model" value="/no/such/model.nmt"\n', "missing model file"),
 ])
