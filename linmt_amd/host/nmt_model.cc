@@ -644,11 +644,21 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
     }
   }
   const int B = n * beam, K = beam + 1;
+  // Host arrays that asynchronous uploads read (together with src, limit and binfo above).  They
+  // are declared before the guard below, so however this function is left, every model's stream
+  // has drained before any of them is destroyed.
+  std::vector<std::vector<int>> src_own, bi_keep;
+  std::vector<int> start(B, Decoder::start_symbol_);
+  struct DrainStreams {
+    std::vector<NeuralMachineTranslation *> &models;
+    ~DrainStreams() {
+      for (NeuralMachineTranslation *m : models) (void)hipStreamSynchronize(m->stream_);
+    }
+  } drain_streams{models};
   Decoder &d = decoder_;
   if (max_limit + 1 > d.max_steps_) throw LinmtError("DecodeBatch: too many decoding steps");
 
   // InitDecoder (decoder.h:334-350): <START> everywhere, scores 0
-  std::vector<int> start(B, Decoder::start_symbol_);
   d.current_indices_.Upload(start.data(), B, stream_);
   d.score_[0].Zero(stream_);
   d.limit_.Upload(limit.data(), n, stream_);
@@ -663,7 +673,6 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
     int *indices;
   };
   std::vector<NodeBuffers> node_buffers(n_models, NodeBuffers{nullptr, nullptr});
-  std::vector<std::vector<int>> src_own;
   std::vector<size_t> hist_slices(n_models, 0);
 
   for (int k = 0; k < n_models; ++k) {
@@ -754,7 +763,6 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
 
   int cur = 0;
   std::vector<int> active_at(max_limit + 1);
-  std::vector<std::vector<int>> bi_keep;
   int *p_device_step_indices = d.current_indices_.get();  // <START> for every column
   for (int step = 0; step <= max_limit; ++step) {
     int n_active = 0;
