@@ -112,6 +112,21 @@ int lh_gemm_ws_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, 
                    float alpha, float beta, const float *bias, int act, int act_rows,
                    const int *colmask, float *C, int ldc, void *workspace, size_t workspace_bytes,
                    lh_stream_t stream);
+/* lh_gemm_ws_f32 for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc) and so have no workspace to hand over.  It
+ * has no counterpart in the reference.  The partial planes go into an array of
+ * LH_GEMM_NOALLOC_WS_BYTES that is part of the library's device code: each GPU the library runs
+ * on holds its own copy until the process ends.  Same arguments, same choice of tile and split and
+ * bit for bit the same result as lh_gemm_ws_f32 with a workspace of LH_GEMM_NOALLOC_WS_BYTES.  No
+ * hipMalloc / hipFree and no allocating library routine is called.  A product of which two
+ * partial planes (((M + 3) & ~3) x N floats each) do not fit the array is rejected with
+ * LH_ERR_ARG.  Every call on a GPU shares that GPU's array (its contents between calls mean
+ * nothing, nothing in it has to be cleared): calls that overlap in time on one GPU -- from
+ * different streams or threads -- race on it; order them on one stream. */
+#define LH_GEMM_NOALLOC_WS_BYTES (32u << 20)
+int lh_gemm_noalloc_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
+                        float alpha, float beta, const float *bias, int act, int act_rows,
+                        const int *colmask, float *C, int ldc, lh_stream_t stream);
 /* The plain product for a consumer that can add up partial sums itself (the LSTM cell kernel takes
  * three addends): like lh_gemm_ws_f32 with alpha = 1 and no bias / activation / mask, but a split
  * product is left unreduced.  *planes receives S, 1 <= S <= max_planes:

@@ -43,6 +43,9 @@ SIGNATURES = {
     "lh_gemm_ws_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int, C.c_int,
                                  C.c_float, C.c_float, c_f32p, C.c_int, C.c_int, c_i32p, c_f32p,
                                  C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "lh_gemm_noalloc_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
+                                      C.c_int, C.c_float, C.c_float, c_f32p, C.c_int, C.c_int,
+                                      c_i32p, c_f32p, C.c_int, C.c_void_p]),
     "lh_gemm_planes_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
                                      C.c_int, C.c_float, c_f32p, C.c_int, C.c_void_p, C.c_size_t,
                                      C.c_int, C.POINTER(C.c_int), C.c_void_p]),
@@ -206,6 +209,18 @@ def gemm(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0
                                           beta, _ptr(bias), act, act_rows, _ptr(colmask),
                                           _ptr(C_out), ldc, _stream(stream)),
               "lh_gemm_act_rows_f32")
+
+
+LH_GEMM_NOALLOC_WS_BYTES = 32 << 20
+
+
+def gemm_noalloc(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0,
+                 bias=None, act=LH_ACT_NONE, colmask=None, act_rows=None, stream=None):
+    """lh_gemm_noalloc_f32: the K-split product over the library's own scratch array."""
+    check(load().lh_gemm_noalloc_f32(M, N, _segs(segs), len(segs), int(transA), int(transX), alpha,
+                                     beta, _ptr(bias), act, M if act_rows is None else act_rows,
+                                     _ptr(colmask), _ptr(C_out), ldc, _stream(stream)),
+          "lh_gemm_noalloc_f32")
 
 
 def gemm_kernel_name(M, N, segs, transA=False, transX=False, workspace_bytes=0, max_planes=0):
