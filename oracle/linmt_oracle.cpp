@@ -12,6 +12,8 @@
 //     (undefined behaviour in the reference; this restatement stops popping instead).
 #include "linmt_oracle.h"
 
+#include <immintrin.h>
+
 #include <algorithm>
 #include <cfloat>
 #include <cmath>
@@ -33,59 +35,89 @@ inline size_t idx2c(size_t i, size_t j, size_t ld) { return j * ld + i; }  // sr
 
 // Dot products with 8 independent fp32 partial sums (vectorisable, deterministic).
 inline float dot8(const float *a, const float *b, int n) {
-  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  __m256 acc = _mm256_setzero_ps();
   int k = 0;
   for (; k + 8 <= n; k += 8)
-    for (int u = 0; u < 8; ++u) acc[u] += a[k + u] * b[k + u];
+    acc = _mm256_fmadd_ps(_mm256_loadu_ps(a + k), _mm256_loadu_ps(b + k), acc);
+  float q[8];
+  _mm256_storeu_ps(q, acc);
   float tail = 0.f;
-  for (; k < n; ++k) tail += a[k] * b[k];
-  return ((acc[0] + acc[4]) + (acc[1] + acc[5])) + ((acc[2] + acc[6]) + (acc[3] + acc[7])) + tail;
+  for (; k < n; ++k) tail = std::fma(a[k], b[k], tail);
+  return ((q[0] + q[4]) + (q[1] + q[5])) + ((q[2] + q[6]) + (q[3] + q[7])) + tail;
 }
 
 // C (col-major M x N) = alpha * At (row-major M x K, row stride lda) * X (col-major K x N) + beta*C.
+// Every element is one dot product with the summation order of dot8; the two loop nests below
+// differ only in which elements a thread visits in which order.
 void gemm_rowA(int M, int N, int K, const float *At, int lda, const float *X, int ldx, float alpha,
                float beta, float *C, int ldc) {
+  if (K <= 64 && N >= 64) {
+    // Short dot products into a large C (weight gradients d x^T over a small minibatch): walk C
+    // column by column so that the read-modify-write of C is contiguous.
 #pragma omp parallel for schedule(static)
-  for (int m = 0; m < M; ++m) {
-    const float *a = At + (size_t)m * lda;
-    int n = 0;
-    for (; n + 4 <= N; n += 4) {
-      float acc[4][8];
-      for (int j = 0; j < 4; ++j)
-        for (int u = 0; u < 8; ++u) acc[j][u] = 0.f;
-      const float *x0 = X + (size_t)n * ldx, *x1 = x0 + ldx, *x2 = x1 + ldx, *x3 = x2 + ldx;
-      int k = 0;
-      for (; k + 8 <= K; k += 8)
-        for (int u = 0; u < 8; ++u) {
-          const float av = a[k + u];
-          acc[0][u] += av * x0[k + u];
-          acc[1][u] += av * x1[k + u];
-          acc[2][u] += av * x2[k + u];
-          acc[3][u] += av * x3[k + u];
-        }
-      float t[4] = {0, 0, 0, 0};
-      for (; k < K; ++k) {
-        t[0] += a[k] * x0[k]; t[1] += a[k] * x1[k]; t[2] += a[k] * x2[k]; t[3] += a[k] * x3[k];
-      }
-      for (int j = 0; j < 4; ++j) {
-        const float *q = acc[j];
-        const float d = ((q[0] + q[4]) + (q[1] + q[5])) + ((q[2] + q[6]) + (q[3] + q[7])) + t[j];
-        float *c = C + idx2c(m, n + j, ldc);
-        *c = beta == 0.f ? alpha * d : alpha * d + beta * *c;
+    for (int n = 0; n < N; ++n) {
+      const float *x = X + (size_t)n * ldx;
+      float *c = C + (size_t)n * ldc;
+      for (int m = 0; m < M; ++m) {
+        const float d = dot8(At + (size_t)m * lda, x, K);
+        c[m] = beta == 0.f ? alpha * d : alpha * d + beta * c[m];
       }
     }
-    for (; n < N; ++n) {
-      const float d = dot8(a, X + (size_t)n * ldx, K);
-      float *c = C + idx2c(m, n, ldc);
-      *c = beta == 0.f ? alpha * d : alpha * d + beta * *c;
+    return;
+  }
+  // Register tile of 4 rows x 4 columns: each element keeps the 8 lane sums of dot8 in one
+  // vector register, so a loaded piece of a row serves 4 columns and a piece of a column 4 rows.
+  const int Mb = (M + 3) / 4;
+#pragma omp parallel for schedule(static)
+  for (int mb = 0; mb < Mb; ++mb) {
+    const int m0 = mb * 4, mr = std::min(4, M - m0);
+    const float *a[4];
+    for (int i = 0; i < 4; ++i) a[i] = At + (size_t)(m0 + (i < mr ? i : 0)) * lda;
+    for (int n0 = 0; n0 < N; n0 += 4) {
+      const int nr = std::min(4, N - n0);
+      const float *x[4];
+      for (int j = 0; j < 4; ++j) x[j] = X + (size_t)(n0 + (j < nr ? j : 0)) * ldx;
+      __m256 acc[4][4];
+      for (int i = 0; i < 4; ++i)
+        for (int j = 0; j < 4; ++j) acc[i][j] = _mm256_setzero_ps();
+      int k = 0;
+      for (; k + 8 <= K; k += 8) {
+        const __m256 x0 = _mm256_loadu_ps(x[0] + k), x1 = _mm256_loadu_ps(x[1] + k),
+                     x2 = _mm256_loadu_ps(x[2] + k), x3 = _mm256_loadu_ps(x[3] + k);
+        for (int i = 0; i < 4; ++i) {
+          const __m256 av = _mm256_loadu_ps(a[i] + k);
+          acc[i][0] = _mm256_fmadd_ps(av, x0, acc[i][0]);
+          acc[i][1] = _mm256_fmadd_ps(av, x1, acc[i][1]);
+          acc[i][2] = _mm256_fmadd_ps(av, x2, acc[i][2]);
+          acc[i][3] = _mm256_fmadd_ps(av, x3, acc[i][3]);
+        }
+      }
+      for (int i = 0; i < mr; ++i)
+        for (int j = 0; j < nr; ++j) {
+          float q[8];
+          _mm256_storeu_ps(q, acc[i][j]);
+          float tail = 0.f;
+          for (int kk = k; kk < K; ++kk) tail = std::fma(a[i][kk], x[j][kk], tail);
+          const float d = ((q[0] + q[4]) + (q[1] + q[5])) + ((q[2] + q[6]) + (q[3] + q[7])) + tail;
+          float *c = C + idx2c(m0 + i, n0 + j, ldc);
+          *c = beta == 0.f ? alpha * d : alpha * d + beta * *c;
+        }
     }
   }
 }
 
 void transpose_to(const float *src, int rows, int cols, int ld, float *dst) {
-  // src col-major rows x cols (ld) -> dst row-major rows x cols (i.e. col-major cols x rows)
-  for (int j = 0; j < cols; ++j)
-    for (int i = 0; i < rows; ++i) dst[(size_t)i * cols + j] = src[idx2c(i, j, ld)];
+  // src col-major rows x cols (ld) -> dst row-major rows x cols (i.e. col-major cols x rows),
+  // in 32 x 32 blocks so that both sides stay in cache
+  constexpr int T = 32;
+  const int bi = (rows + T - 1) / T, bj = (cols + T - 1) / T;
+#pragma omp parallel for schedule(static) if ((size_t)rows * cols > 65536)
+  for (int blk = 0; blk < bi * bj; ++blk) {
+    const int i0 = (blk / bj) * T, j0 = (blk % bj) * T;
+    const int i1 = std::min(rows, i0 + T), j1 = std::min(cols, j0 + T);
+    for (int i = i0; i < i1; ++i)
+      for (int j = j0; j < j1; ++j) dst[(size_t)i * cols + j] = src[idx2c(i, j, ld)];
+  }
 }
 
 inline float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-1.0f * x)); }          // deep_rnn_kernel.cu:83
@@ -520,6 +552,13 @@ namespace {
 
 const char *kGateNames[4] = {"i", "f", "c", "o"};  // stacked order i,f,g(=c'),o
 
+// Embedding size.  The reference fixes it to the LSTM size (src/global_configuration.h:220); a
+// configuration with E > 0 generalises the two places that touch an embedding: the tables W are
+// E x V and the first layer's input matrices M_* are H x E.
+inline int emb_size(const orc_model_config &cfg) { return cfg.E > 0 ? cfg.E : cfg.H; }
+// rows of the vector a layer reads from below
+inline int in_size(const orc_model_config &cfg, int layer) { return layer == 0 ? emb_size(cfg) : cfg.H; }
+
 void add_param(orc_model *m, const std::string &name, size_t n) { m->params[name].assign(n, 0.f); }
 
 // y (rows x B) = P (rows x K, named parameter) * x (K x B)
@@ -537,9 +576,9 @@ struct LayerState {
   std::vector<float> h, c;
 };
 
-// One LSTM layer step (node ForwardPropGpu): x is H x B (already looked up / from below).
+// One LSTM layer step (node ForwardPropGpu): x is K x B (looked up: K = E; from below: K = H).
 // Writes the stacked 4H x B products per operand and runs the cell.
-void lstm_layer_step(orc_model *m, const std::string &pfx, int B, const float *x,
+void lstm_layer_step(orc_model *m, const std::string &pfx, int K, int B, const float *x,
                      const float *h_prev, const float *c_prev, const float *h_tild,
                      const int *mask01, float *h, float *c) {
   const int H = m->cfg.H;
@@ -550,7 +589,7 @@ void lstm_layer_step(orc_model *m, const std::string &pfx, int B, const float *x
   std::vector<float> bias((size_t)4 * H);
   for (int g = 0; g < 4; ++g) {
     const std::string gn = kGateNames[g];
-    mat_apply(m, pfx + "M_" + gn, H, H, x, B, tmp.data());
+    mat_apply(m, pfx + "M_" + gn, H, K, x, B, tmp.data());
     for (int b = 0; b < B; ++b)
       memcpy(&p1[idx2c((size_t)g * H, b, (size_t)4 * H)], &tmp[(size_t)b * H], sizeof(float) * H);
     mat_apply(m, pfx + "W_h" + gn, H, H, h_prev, B, tmp.data());
@@ -572,7 +611,7 @@ void lstm_layer_step(orc_model *m, const std::string &pfx, int B, const float *x
 extern "C" orc_model *orc_model_create(const orc_model_config *cfg) {
   orc_model *m = new orc_model();
   m->cfg = *cfg;
-  const size_t H = cfg->H;
+  const size_t H = cfg->H, E = emb_size(*cfg);
   for (int side = 0; side < 2; ++side) {
     const std::string s = side == 0 ? "src." : "tgt.";
     const size_t V = side == 0 ? cfg->V_src : cfg->V_tgt;
@@ -581,12 +620,12 @@ extern "C" orc_model *orc_model_create(const orc_model_config *cfg) {
       for (int g = 0; g < 4; ++g) {
         const std::string gn = kGateNames[g];
         add_param(m, pfx + "W_h" + gn, H * H);
-        add_param(m, pfx + "M_" + gn, H * H);
+        add_param(m, pfx + "M_" + gn, H * (l == 0 ? E : H));
         add_param(m, pfx + "b_" + gn, H);
         if (side == 1 && l == 0 && cfg->feed_input && cfg->attention)
           add_param(m, pfx + "Q_" + gn, H * H);
       }
-      if (l == 0) add_param(m, pfx + "W", H * V);
+      if (l == 0) add_param(m, pfx + "W", E * V);
     }
   }
   if (cfg->attention) {
@@ -611,6 +650,18 @@ extern "C" float *orc_model_param(orc_model *m, const char *name, long long *n_e
   return it->second.data();
 }
 
+// Internal to the oracle (used by linmt_oracle_train.cpp): the row-major copy orc_model_commit
+// keeps of a matrix parameter, or NULL when none is kept under that name.
+const float *orc_model_rowmajor(orc_model *m, const char *name) {
+  const auto it = m->rowmajor.find(name);
+  if (it == m->rowmajor.end() || std::string(name) == "attn.W_a") return nullptr;
+  return it->second.data();
+}
+void orc_gemm_rowmajor_a(int M, int N, int K, const float *At, const float *X, int ldx, float alpha,
+                         float beta, float *C, int ldc) {
+  gemm_rowA(M, N, K, At, K, X, ldx, alpha, beta, C, ldc);
+}
+
 extern "C" void orc_model_commit(orc_model *m) {
   const int H = m->cfg.H;
   m->rowmajor.clear();
@@ -622,7 +673,8 @@ extern "C" void orc_model_commit(orc_model *m) {
         leaf == "W_p" || leaf == "W_c1" || leaf == "W_c2") {
       auto &dst = m->rowmajor[n];
       dst.resize(kv.second.size());
-      transpose_to(kv.second.data(), H, H, H, dst.data());
+      const int cols = (int)(kv.second.size() / (size_t)H);  // H, or E for the first layer's M_*
+      transpose_to(kv.second.data(), H, cols, H, dst.data());
     } else if (leaf == "W_a") {
       m->rowmajor[n] = kv.second;  // used transposed: W_a^T row-major == W_a column-major
     } else if (leaf == "D") {
@@ -768,16 +820,18 @@ int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
       s.c.assign(H, 0.f);
     }
     r.top_states.resize((size_t)S * H);
-    std::vector<float> x(H), hn(H), cn(H);
+    const int E = emb_size(cfg);
+    std::vector<float> x(std::max(E, H)), hn(H), cn(H);
     for (int t = 0; t < S; ++t) {
       int id = src_ids[S - 1 - t];
       int id0, m01;
       orc_preprocess_indices(&id, 1, &id0, &m01, nullptr);
-      orc_embed_lookup(m->params["src.0.W"].data(), H, cfg.V_src, &id0, 1, nullptr, 1.f, x.data());
+      x.resize(E);
+      orc_embed_lookup(m->params["src.0.W"].data(), E, cfg.V_src, &id0, 1, nullptr, 1.f, x.data());
       for (int l = 0; l < L; ++l) {
         const std::string pfx = "src." + std::to_string(l) + ".";
-        lstm_layer_step(m, pfx, 1, x.data(), r.enc[l].h.data(), r.enc[l].c.data(), nullptr, &one,
-                        hn.data(), cn.data());
+        lstm_layer_step(m, pfx, in_size(cfg, l), 1, x.data(), r.enc[l].h.data(), r.enc[l].c.data(),
+                        nullptr, &one, hn.data(), cn.data());
         r.enc[l].h = hn;
         r.enc[l].c = cn;
         x = hn;
@@ -799,7 +853,7 @@ int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
     }
     r.h_tild.assign((size_t)H * B, 0.f);
     r.h_tild_prev.assign((size_t)H * B, 0.f);
-    r.xb.resize((size_t)H * B);
+    r.xb.resize((size_t)E * B);
     r.logits.resize((size_t)V * B);
     r.dist.resize((size_t)V * B);
     r.ascore.assign((size_t)longest * B, 0.f);
@@ -833,12 +887,13 @@ int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
       const int H = r.H, L = r.L;
       std::vector<int> id0(B), m01(B);
       orc_preprocess_indices(current_indices.data(), B, id0.data(), m01.data(), nullptr);
-      orc_embed_lookup(m->params["tgt.0.W"].data(), H, V, id0.data(), B, nullptr, 1.f, r.xb.data());
+      orc_embed_lookup(m->params["tgt.0.W"].data(), emb_size(cfg), V, id0.data(), B, nullptr, 1.f,
+                       r.xb.data());
       const float *below = r.xb.data();
       for (int l = 0; l < L; ++l) {
         const std::string pfx = "tgt." + std::to_string(l) + ".";
         const bool feed = l == 0 && cfg.feed_input && cfg.attention && curr_index != 0;
-        lstm_layer_step(m, pfx, B, below, r.prev[l].h.data(), r.prev[l].c.data(),
+        lstm_layer_step(m, pfx, in_size(cfg, l), B, below, r.prev[l].h.data(), r.prev[l].c.data(),
                         feed ? r.h_tild_prev.data() : nullptr, ones.data(), r.cur[l].h.data(),
                         r.cur[l].c.data());
         below = r.cur[l].h.data();
@@ -1071,22 +1126,23 @@ extern "C" double orc_forward_xent(orc_model *m, const int *src, int S, const in
   if (num_threads > 0) omp_set_num_threads(num_threads);
 #endif
   const orc_model_config &cfg = m->cfg;
-  const int H = cfg.H, L = cfg.layers, V = cfg.V_tgt;
+  const int H = cfg.H, L = cfg.layers, V = cfg.V_tgt, E = emb_size(cfg);
   std::vector<LayerState> st(L);
   for (auto &s : st) {
     s.h.assign((size_t)H * B, 0.f);
     s.c.assign((size_t)H * B, 0.f);
   }
   std::vector<float> hs((size_t)S * H * B);
-  std::vector<float> x((size_t)H * B), hn((size_t)H * B), cn((size_t)H * B);
+  std::vector<float> x((size_t)std::max(E, H) * B), hn((size_t)H * B), cn((size_t)H * B);
   std::vector<int> id0(B), m01(B);
   for (int t = 0; t < S; ++t) {
     orc_preprocess_indices(src + (size_t)t * B, B, id0.data(), m01.data(), nullptr);
-    orc_embed_lookup(m->params["src.0.W"].data(), H, cfg.V_src, id0.data(), B, nullptr, 1.f,
+    x.resize((size_t)E * B);
+    orc_embed_lookup(m->params["src.0.W"].data(), E, cfg.V_src, id0.data(), B, nullptr, 1.f,
                      x.data());
     for (int l = 0; l < L; ++l) {
       const std::string pfx = "src." + std::to_string(l) + ".";
-      lstm_layer_step(m, pfx, B, x.data(), st[l].h.data(), st[l].c.data(), nullptr, m01.data(),
+      lstm_layer_step(m, pfx, in_size(cfg, l), B, x.data(), st[l].h.data(), st[l].c.data(), nullptr, m01.data(),
                       hn.data(), cn.data());
       st[l].h = hn;
       st[l].c = cn;
@@ -1099,11 +1155,12 @@ extern "C" double orc_forward_xent(orc_model *m, const int *src, int S, const in
   std::vector<int> t0(B), tm(B);
   for (int t = 0; t < T; ++t) {
     orc_preprocess_indices(tgt_in + (size_t)t * B, B, id0.data(), m01.data(), nullptr);
-    orc_embed_lookup(m->params["tgt.0.W"].data(), H, V, id0.data(), B, nullptr, 1.f, x.data());
+    x.resize((size_t)E * B);
+    orc_embed_lookup(m->params["tgt.0.W"].data(), E, V, id0.data(), B, nullptr, 1.f, x.data());
     for (int l = 0; l < L; ++l) {
       const std::string pfx = "tgt." + std::to_string(l) + ".";
       const bool feed = l == 0 && cfg.feed_input && cfg.attention && t != 0;
-      lstm_layer_step(m, pfx, B, x.data(), st[l].h.data(), st[l].c.data(),
+      lstm_layer_step(m, pfx, in_size(cfg, l), B, x.data(), st[l].h.data(), st[l].c.data(),
                       feed ? h_tild.data() : nullptr, m01.data(), hn.data(), cn.data());
       st[l].h = hn;
       st[l].c = cn;

@@ -79,12 +79,17 @@ void orc_beam_gather(const float *src, float *dst, int H, int B, const int *back
 /* ---- whole model ----------------------------------------------------------------------------- */
 typedef struct orc_model_config {
   int layers;        /* LSTM layers per side */
-  int H;             /* lstm_size == embedding size */
+  int H;             /* lstm_size (and the embedding size when E == 0) */
   int V_src, V_tgt;
   int attention;     /* 0 none, 1 local-p, 2 global-general (build-defined) */
   int D;             /* attention window half-width */
   int feed_input;
   int longest_sent;  /* longest_sentence_ of the reference (already including its +4) */
+  int E;             /* embedding size; 0 = H, the reference's only case
+                        (src/global_configuration.h:220).  E != H is a generalisation: "*.0.W" is
+                        E x V and "*.0.M_*" are H x E.  pin: E == H gives the same bits as E = 0,
+                        and the gradients at E != H agree with central differences of the
+                        independent numpy model (tests/test_oracle_train_pins.py). */
 } orc_model_config;
 
 typedef struct orc_model orc_model;

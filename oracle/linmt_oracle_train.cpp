@@ -23,6 +23,12 @@
 
 #include "linmt_oracle.h"
 
+// from linmt_oracle.cpp: the transposed copy the model keeps of a matrix after orc_model_commit,
+// and the product on such a copy (what orc_gemm does after transposing A itself)
+const float *orc_model_rowmajor(orc_model *m, const char *name);
+void orc_gemm_rowmajor_a(int M, int N, int K, const float *At, const float *X, int ldx, float alpha,
+                         float beta, float *C, int ldc);
+
 namespace {
 
 inline size_t idx2c(size_t i, size_t j, size_t ld) { return j * ld + i; }
@@ -73,18 +79,37 @@ Vec &G(orc_trainer *t, const std::string &name, size_t n) {
   return g;
 }
 
-// y = P x for the H x H parameter `name` (col-major), optionally transposed.
-void apply(orc_trainer *t, const std::string &name, int transA, const float *x, int B, float beta,
-           float *y) {
-  const int H = t->cfg.H;
-  orc_gemm(H, B, H, P(t, name), H, transA, x, H, 0, 1.f, beta, y, H);
+// Embedding size: the LSTM size unless the configuration names another (a generalisation, the
+// reference has E == H, src/global_configuration.h:220).  Only the first layer of a side reads
+// an embedding: its x is E x B and its M_* are H x E.
+int emb(const orc_trainer *t) { return t->cfg.E > 0 ? t->cfg.E : t->cfg.H; }
+int in_rows(const orc_trainer *t, const std::string &pfx) {
+  return pfx == "src.0." || pfx == "tgt.0." ? emb(t) : t->cfg.H;
 }
 
-// grad(name) += a b^T  (a, b: H x B)
-void outer_acc(orc_trainer *t, const std::string &name, const float *a, const float *b, int B) {
+// y = P x for the H x K parameter `name` (col-major): y is H x B, x is K x B; transposed: y is
+// K x B, x is H x B.  K = H for every matrix but the first layer's M_*.
+void apply(orc_trainer *t, const std::string &name, int transA, const float *x, int B, float beta,
+           float *y, int K = 0) {
   const int H = t->cfg.H;
-  Vec &g = G(t, name, (size_t)H * H);
-  orc_gemm(H, H, B, a, H, 0, b, H, 1, 1.f, 1.f, g.data(), H);
+  if (K <= 0) K = H;
+  if (transA) {
+    orc_gemm(K, B, H, P(t, name), H, 1, x, H, 0, 1.f, beta, y, K);
+    return;
+  }
+  // same arithmetic as orc_gemm, without transposing the matrix again on every call
+  const float *rm = orc_model_rowmajor(t->m, name.c_str());
+  if (rm) orc_gemm_rowmajor_a(H, B, K, rm, x, K, 1.f, beta, y, H);
+  else orc_gemm(H, B, K, P(t, name), H, 0, x, K, 0, 1.f, beta, y, H);
+}
+
+// grad(name) += a b^T  (a: H x B, b: K x B)
+void outer_acc(orc_trainer *t, const std::string &name, const float *a, const float *b, int B,
+               int K = 0) {
+  const int H = t->cfg.H;
+  if (K <= 0) K = H;
+  Vec &g = G(t, name, (size_t)H * K);
+  orc_gemm(H, K, B, a, H, 0, b, K, 1, 1.f, 1.f, g.data(), H);
 }
 
 // grad(name) += a 1
@@ -108,7 +133,7 @@ void cell_forward(orc_trainer *t, const std::string &pfx, int B, CellTape &tp) {
       for (int b = 0; b < B; ++b)
         memcpy(&dst[idx2c((size_t)g * H, b, (size_t)4 * H)], &tmp[(size_t)b * H], sizeof(float) * H);
     };
-    apply(t, pfx + "M_" + gn, 0, tp.x.data(), B, 0.f, tmp.data());
+    apply(t, pfx + "M_" + gn, 0, tp.x.data(), B, 0.f, tmp.data(), in_rows(t, pfx));
     put(p1);
     apply(t, pfx + "W_h" + gn, 0, tp.h_prev.data(), B, 0.f, tmp.data());
     put(p2);
@@ -127,7 +152,8 @@ void cell_forward(orc_trainer *t, const std::string &pfx, int B, CellTape &tp) {
 }
 
 // Backward of one LSTM node.  dh_above may be NULL (zero).  dh_next / dc_next are the errors handed
-// back by node t+1 and are replaced by the ones for node t-1.  dx receives M^T d (H x B);
+// back by node t+1 and are replaced by the ones for node t-1.  dx receives M^T d (H x B, E x B in
+// a first layer);
 // dh_tild_below (feed input, t > 0) receives Q^T d.
 void cell_backward(orc_trainer *t, const std::string &pfx, int B, const CellTape &tp,
                    const float *dh_above, const float *above_drop_mask, Vec &dh_next, Vec &dc_next,
@@ -145,11 +171,12 @@ void cell_backward(orc_trainer *t, const std::string &pfx, int B, const CellTape
       memcpy(&d[g][(size_t)b * H], &dg[idx2c((size_t)g * H, b, (size_t)4 * H)], sizeof(float) * H);
   }
   Vec dh_prev(n, 0.f);
-  dx.assign(n, 0.f);
+  const int Kx = in_rows(t, pfx);
+  dx.assign((size_t)Kx * B, 0.f);
   for (int g = 0; g < 4; ++g) {
     const std::string gn = kGate[g];
     apply(t, pfx + "W_h" + gn, 1, d[g].data(), B, 1.f, dh_prev.data());
-    apply(t, pfx + "M_" + gn, 1, d[g].data(), B, 1.f, dx.data());
+    apply(t, pfx + "M_" + gn, 1, d[g].data(), B, 1.f, dx.data(), Kx);
   }
   if (tp.feed && dh_tild_below) {
     dh_tild_below->assign(n, 0.f);
@@ -160,7 +187,7 @@ void cell_backward(orc_trainer *t, const std::string &pfx, int B, const CellTape
   for (int g = 0; g < 4; ++g) {
     const std::string gn = kGate[g];
     outer_acc(t, pfx + "W_h" + gn, d[g].data(), tp.h_prev.data(), B);
-    outer_acc(t, pfx + "M_" + gn, d[g].data(), tp.x.data(), B);
+    outer_acc(t, pfx + "M_" + gn, d[g].data(), tp.x.data(), B, Kx);
     if (tp.feed) outer_acc(t, pfx + "Q_" + gn, d[g].data(), tp.h_tild_prev.data(), B);
     rowsum_acc(t, pfx + "b_" + gn, d[g].data(), H, B);
   }
@@ -171,7 +198,7 @@ void cell_backward(orc_trainer *t, const std::string &pfx, int B, const CellTape
 // WSmallGradientKernel: small_grad[:, rev[idx0_b]] += dx[:, b].  Pad columns carry dx = 0.
 void scatter_embedding(orc_trainer *t, const std::string &name, int side, const Vec &dx,
                        const CellTape &tp, int B, const float *drop_mask) {
-  const int H = t->cfg.H;
+  const int H = emb(t);  // rows of an embedding
   const std::vector<int> &u = t->uniq[side];
   Vec &g = G(t, name, (size_t)H * u.size());
   for (int b = 0; b < B; ++b) {
@@ -338,10 +365,10 @@ extern "C" void orc_trainer_set_dropout(orc_trainer *t, float keep, const float 
                                         const float *tgt_embed, const float *src_out,
                                         const float *tgt_out, int S, int T, int B) {
   t->keep = keep;
-  const size_t n = (size_t)t->cfg.H * B, L = t->cfg.layers;
+  const size_t n = (size_t)t->cfg.H * B, ne = (size_t)emb(t) * B, L = t->cfg.layers;
   if (!(keep > 0.f)) return;
-  t->drop_embed[0].assign(src_embed, src_embed + n * S);
-  t->drop_embed[1].assign(tgt_embed, tgt_embed + n * T);
+  t->drop_embed[0].assign(src_embed, src_embed + ne * S);
+  t->drop_embed[1].assign(tgt_embed, tgt_embed + ne * T);
   t->drop_out[0].assign(src_out, src_out + n * S * L);
   t->drop_out[1].assign(tgt_out, tgt_out + n * T * L);
 }
@@ -358,8 +385,8 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
                                         const int *src_unique, int n_src_unique,
                                         const int *tgt_unique, int n_tgt_unique) {
   const orc_model_config &cfg = t->cfg;
-  const int H = cfg.H, L = cfg.layers, V = cfg.V_tgt;
-  const size_t n = (size_t)H * B;
+  const int H = cfg.H, L = cfg.layers, V = cfg.V_tgt, E = emb(t);
+  const size_t n = (size_t)H * B, ne = (size_t)E * B;
   const bool attn = cfg.attention != 0;
   const bool feed_cfg = attn && cfg.feed_input;
   const int D = cfg.attention == 1 ? cfg.D : -1;
@@ -367,11 +394,11 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
   t->uniq[0].assign(src_unique, src_unique + n_src_unique);
   t->uniq[1].assign(tgt_unique, tgt_unique + n_tgt_unique);
   for (auto &kv : t->grads) std::fill(kv.second.begin(), kv.second.end(), 0.f);
-  G(t, "src.0.W", (size_t)H * n_src_unique);
-  G(t, "tgt.0.W", (size_t)H * n_tgt_unique);
+  G(t, "src.0.W", (size_t)E * n_src_unique);
+  G(t, "tgt.0.W", (size_t)E * n_tgt_unique);
 
   const bool drop = t->keep > 0.f;
-  if (drop && (t->drop_embed[0].size() != n * S || t->drop_embed[1].size() != n * T ||
+  if (drop && (t->drop_embed[0].size() != ne * S || t->drop_embed[1].size() != ne * T ||
                t->drop_out[0].size() != n * S * L || t->drop_out[1].size() != n * T * L)) {
     fprintf(stderr, "orc_trainer: dropout masks do not match this minibatch\n");
     exit(EXIT_FAILURE);
@@ -382,7 +409,7 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
     return t->drop_out[side].data() + ((size_t)l * steps + s) * n;
   };
   auto embed_mask = [&](int side, int s) -> const float * {
-    return drop ? t->drop_embed[side].data() + (size_t)s * n : nullptr;
+    return drop ? t->drop_embed[side].data() + (size_t)s * ne : nullptr;
   };
   auto dropped = [&](const Vec &h, const float *mask) {
     Vec r = h;
@@ -402,9 +429,9 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
       tp.idx0.resize(B);
       tp.mask.resize(B);
       orc_preprocess_indices(src + (size_t)s * B, B, tp.idx0.data(), tp.mask.data(), nullptr);
-      tp.x.assign(n, 0.f);
+      tp.x.assign(l == 0 ? ne : n, 0.f);
       if (l == 0)
-        orc_embed_lookup(P(t, "src.0.W"), H, cfg.V_src, tp.idx0.data(), B, embed_mask(0, s),
+        orc_embed_lookup(P(t, "src.0.W"), E, cfg.V_src, tp.idx0.data(), B, embed_mask(0, s),
                          drop ? t->keep : 1.f, tp.x.data());
       else
         tp.x = dropped(enc[s][l - 1].h, out_mask(0, l - 1, s));
@@ -422,9 +449,9 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
       tp.idx0.resize(B);
       tp.mask.resize(B);
       orc_preprocess_indices(tgt_in + (size_t)s * B, B, tp.idx0.data(), tp.mask.data(), nullptr);
-      tp.x.assign(n, 0.f);
+      tp.x.assign(l == 0 ? ne : n, 0.f);
       if (l == 0)
-        orc_embed_lookup(P(t, "tgt.0.W"), H, V, tp.idx0.data(), B, embed_mask(1, s),
+        orc_embed_lookup(P(t, "tgt.0.W"), E, V, tp.idx0.data(), B, embed_mask(1, s),
                          drop ? t->keep : 1.f, tp.x.data());
       else
         tp.x = dropped(dec[s][l - 1].h, out_mask(1, l - 1, s));
@@ -471,7 +498,8 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
     }
     // softmax: p, log-likelihood, and the output error (onehot - p) * mask of GetHTGradientGpu
     Vec logits((size_t)V * B);
-    orc_gemm(V, B, H, P(t, "softmax.D"), V, 0, top, H, 0, 1.f, 0.f, logits.data(), V);
+    orc_gemm_rowmajor_a(V, B, H, orc_model_rowmajor(t->m, "softmax.D"), top, H, 1.f, 0.f,
+                        logits.data(), V);
     std::vector<int> t0(B);
     tgt_mask[s].resize(B);
     orc_preprocess_indices(tgt_out + (size_t)s * B, B, t0.data(), tgt_mask[s].data(), nullptr);
@@ -568,7 +596,7 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
 // are cleared.  Returns the global norm (clip_mode 2) or 0.
 extern "C" float orc_update_weights(orc_trainer *t, float learning_rate, int clip_mode,
                                     float norm_clip, float individual_clip, int minibatch_size) {
-  const int H = t->cfg.H;
+  const int H = emb(t);  // only the embedding columns are addressed by row below
   for (auto &kv : t->grads)
     for (auto &v : kv.second) v = (1.0f / minibatch_size) * v;
   float global = 0.f;

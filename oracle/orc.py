@@ -23,7 +23,7 @@ def build():
 class ModelConfig(C.Structure):
     _fields_ = [("layers", C.c_int), ("H", C.c_int), ("V_src", C.c_int), ("V_tgt", C.c_int),
                 ("attention", C.c_int), ("D", C.c_int), ("feed_input", C.c_int),
-                ("longest_sent", C.c_int)]
+                ("longest_sent", C.c_int), ("E", C.c_int)]
 
 
 class DecodeOpts(C.Structure):
@@ -283,8 +283,11 @@ def attn_core_bwd(H, B, D, max_len, hs_steps, dctx, tanh1, v_p, wa, hs, step_str
 class Model:
     """Host model of the oracle; parameters are numpy views into the oracle's own buffers."""
 
-    def __init__(self, layers, H, V_src, V_tgt, attention=1, D=10, feed_input=1, longest_sent=104):
-        self.cfg = ModelConfig(layers, H, V_src, V_tgt, attention, D, feed_input, longest_sent)
+    def __init__(self, layers, H, V_src, V_tgt, attention=1, D=10, feed_input=1, longest_sent=104,
+                 E=0):
+        """E: embedding size, 0 = H (the reference's only case)."""
+        self.cfg = ModelConfig(layers, H, V_src, V_tgt, attention, D, feed_input, longest_sent, E)
+        self.E = E if E > 0 else H
         self.handle = C.c_void_p(lib().orc_model_create(C.byref(self.cfg)))
 
     def param(self, name):
@@ -372,13 +375,13 @@ class Model:
             return
         H, L = self.cfg.H, self.cfg.layers
         se, te, so, to = (f32(a).ravel() for a in (src_embed, tgt_embed, src_out, tgt_out))
-        S, T = se.size // (H * B), te.size // (H * B)
+        S, T = se.size // (self.E * B), te.size // (self.E * B)
         assert so.size == L * S * H * B and to.size == L * T * H * B
         lib().orc_trainer_set_dropout(t, _f(keep), _p(se), _p(te), _p(so), _p(to), S, T, B)
 
     def compute_gradients(self, src, tgt_in, tgt_out, batch_info, src_unique, tgt_unique):
         """Forward + backward (no update).  Returns (sum log p, {name: gradient}); matrices come back
-        as Fortran-ordered 2-D arrays, the embedding gradients as (H, n_unique)."""
+        as Fortran-ordered 2-D arrays, the embedding gradients as (E, n_unique)."""
         self._trainer()
         src = np.asfortranarray(src, np.int32)
         tgt_in = np.asfortranarray(tgt_in, np.int32)
@@ -407,18 +410,23 @@ class Model:
                 names += ["attn.W_p", "attn.v_p"]
         return names + ["softmax.D", "softmax.b_d"]
 
+    def _shape(self, name, flat):
+        H = self.cfg.H
+        if name == "softmax.D":
+            return flat.reshape((self.cfg.V_tgt, H), order="F")
+        if name.endswith(".W"):  # embedding table or its small gradient: E rows
+            return flat.reshape((self.E, flat.size // self.E), order="F")
+        if flat.size % H == 0 and flat.size > H and not name.endswith("b_d"):
+            return flat.reshape((H, flat.size // H), order="F")
+        return flat
+
     def grad(self, name):
         n = C.c_longlong(0)
         ptr = lib().orc_trainer_grad(self.trainer, name.encode(), C.byref(n))
         if not ptr:
             raise KeyError(name)
         flat = np.frombuffer((C.c_float * n.value).from_address(ptr), dtype=np.float32).copy()
-        H = self.cfg.H
-        if name == "softmax.D":
-            return flat.reshape((self.cfg.V_tgt, H), order="F")
-        if flat.size % H == 0 and flat.size > H and not name.endswith("b_d"):
-            return flat.reshape((H, flat.size // H), order="F")
-        return flat
+        return self._shape(name, flat)
 
     def update_weights(self, learning_rate, clip_mode, norm_clip, individual_clip, minibatch_size):
         return float(lib().orc_update_weights(self.trainer, _f(learning_rate), clip_mode,
@@ -426,12 +434,7 @@ class Model:
 
     def get_param(self, name):
         flat = self.param(name).copy()
-        H = self.cfg.H
-        if name == "softmax.D":
-            return flat.reshape((self.cfg.V_tgt, H), order="F")
-        if flat.size % H == 0 and flat.size > H and not name.endswith("b_d"):
-            return flat.reshape((H, flat.size // H), order="F")
-        return flat
+        return self._shape(name, flat)
 
     def __del__(self):
         try:

@@ -11,10 +11,12 @@ def sigmoid(x):
     return 1.0 / (1.0 + np.exp(-x))
 
 
-def make_params(rng, layers, H, V_src, V_tgt, attention=True, feed_input=True, scale=0.08):
+def make_params(rng, layers, H, V_src, V_tgt, attention=True, feed_input=True, scale=0.08, E=None):
     """Reference initialisation: uniform[-scale, scale], forget-gate bias 1
-    (src/utility_cu.cu:77-78, src/layer_input_to_hidden.h:651-655)."""
+    (src/utility_cu.cu:77-78, src/layer_input_to_hidden.h:651-655).  E: embedding size (default H,
+    the reference's only case); the tables are E x V and the first layer's M_* are H x E."""
     P = {}
+    E = H if E is None else E
 
     def u(*shape):
         return rng.uniform(-scale, scale, size=shape).astype(np.float32)
@@ -24,13 +26,13 @@ def make_params(rng, layers, H, V_src, V_tgt, attention=True, feed_input=True, s
             pfx = f"{side}.{l}."
             for g in GATES:
                 P[pfx + "W_h" + g] = u(H, H)
-                P[pfx + "M_" + g] = u(H, H)
+                P[pfx + "M_" + g] = u(H, E if l == 0 else H)
                 P[pfx + "b_" + g] = u(H)
                 if side == "tgt" and l == 0 and attention and feed_input:
                     P[pfx + "Q_" + g] = u(H, H)
             P[pfx + "b_f"] = np.ones(H, np.float32)
             if l == 0:
-                P[pfx + "W"] = u(H, V)
+                P[pfx + "W"] = u(E, V)
     if attention:
         for n in ("W_a", "W_p", "W_c1", "W_c2"):
             P["attn." + n] = u(H, H)

@@ -15,10 +15,11 @@ def _sentences(rng, Vs, Vt, lens_s, lens_t):
     return [(rng.integers(0, Vs, size=a), rng.integers(3, Vt, size=b)) for a, b in zip(lens_s, lens_t)]
 
 
-def _model(orc, rng, layers, H, Vs, Vt, attention, feed, D, scale=0.5):
+def _model(orc, rng, layers, H, Vs, Vt, attention, feed, D, scale=0.5, E=None):
     P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(attention), feed_input=bool(feed),
-                      scale=scale)
-    m = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=feed, longest_sent=40)
+                      scale=scale, E=E)
+    m = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=feed, longest_sent=40,
+                  E=E or 0)
     m.set_params(P)
     return P, m
 
@@ -29,14 +30,19 @@ CASES = [
     dict(layers=2, attention=0, feed=0, D=2, seed=23),
     dict(layers=3, attention=1, feed=1, D=3, seed=24),
     dict(layers=2, attention=2, feed=1, D=-1, seed=25),  # global attention: no window, no Gaussian
+    # embedding size != LSTM size (a generalisation of the reference, which has E == H): a
+    # narrower and a wider embedding
+    dict(layers=2, attention=1, feed=1, D=2, seed=26, E=4),
+    dict(layers=1, attention=2, feed=1, D=-1, seed=27, E=10),
 ]
 
 
-@pytest.mark.parametrize("case", CASES, ids=lambda c: f"L{c['layers']}a{c['attention']}f{c['feed']}")
+@pytest.mark.parametrize("case", CASES,
+                         ids=lambda c: f"L{c['layers']}a{c['attention']}f{c['feed']}E{c.get('E', 0)}")
 def test_gradients_vs_central_differences(orc, case):
     rng = np.random.default_rng(case["seed"])
     layers, H, Vs, Vt, D = case["layers"], 7, 13, 11, case["D"]
-    P, m = _model(orc, rng, layers, H, Vs, Vt, case["attention"], case["feed"], D)
+    P, m = _model(orc, rng, layers, H, Vs, Vt, case["attention"], case["feed"], D, E=case.get("E"))
     sents = _sentences(rng, Vs, Vt, [5, 3, 7, 4], [4, 6, 2, 5])
     src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
     ll, grads = m.compute_gradients(src, tin, tout, bi, su, tu)
@@ -72,18 +78,19 @@ def test_gradients_vs_central_differences(orc, case):
     assert checked == 2 * len(m.param_names())
 
 
-@pytest.mark.parametrize("attention", [1, 0])
-def test_gradients_with_dropout_vs_central_differences(orc, attention):
+@pytest.mark.parametrize("attention,E", [(1, None), (0, None), (1, 5)])
+def test_gradients_with_dropout_vs_central_differences(orc, attention, E):
     """Same check with dropout masks: embeddings, every layer's upward output, the attention /
-    softmax input.  keep = 0.6 so that many elements are dropped."""
-    rng = np.random.default_rng(27 + attention)
+    softmax input.  keep = 0.6 so that many elements are dropped.  The last case has an embedding
+    narrower than the LSTM (embedding masks of E rows)."""
+    rng = np.random.default_rng(27 + attention + (E or 0))
     layers, H, Vs, Vt, D, keep = 2, 7, 13, 11, 2, 0.6
-    P, m = _model(orc, rng, layers, H, Vs, Vt, attention, attention, D)
+    P, m = _model(orc, rng, layers, H, Vs, Vt, attention, attention, D, E=E)
     sents = _sentences(rng, Vs, Vt, [5, 3, 7, 4], [4, 6, 2, 5])
     src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
     B, S, T = len(sents), src.shape[1], tin.shape[1]
-    drop = dict(keep=keep, src_embed=rng.random((S, B, H)).astype(np.float32),
-                tgt_embed=rng.random((T, B, H)).astype(np.float32),
+    drop = dict(keep=keep, src_embed=rng.random((S, B, E or H)).astype(np.float32),
+                tgt_embed=rng.random((T, B, E or H)).astype(np.float32),
                 src_out=rng.random((layers, S, B, H)).astype(np.float32),
                 tgt_out=rng.random((layers, T, B, H)).astype(np.float32))
     m.set_dropout(keep, B, drop["src_embed"], drop["tgt_embed"], drop["src_out"], drop["tgt_out"])
@@ -139,11 +146,53 @@ def test_embedding_rows_outside_the_minibatch_get_no_gradient(orc):
                 assert abs(grads[name][r, k] - fd) <= 2e-3 * max(1.0, abs(fd)), (name, vid, r)
 
 
-@pytest.mark.parametrize("mode", [0, 1, 2, 3])
-def test_update_closed_form(orc, mode):
+def test_explicit_embedding_size_equal_to_lstm_size_changes_nothing(orc):
+    """E == H reduction of the embedding-size generalisation: a model created with E = H gives the
+    bits of a model created the reference's way (E = 0): log-likelihood, every gradient, the
+    update, a beam decode and the scoring pass."""
+    layers, H, Vs, Vt, D = 2, 8, 13, 30, 2
+    outs = []
+    for E in (None, H):
+        rng = np.random.default_rng(61)
+        P, m = _model(orc, rng, layers, H, Vs, Vt, 1, 1, D, E=E)
+        sents = _sentences(rng, Vs, Vt, [5, 3, 7, 4], [4, 6, 2, 5])
+        src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
+        xent = m.forward_xent(src, tin, tout, bi)
+        dec = m.decode_sentence(sents[2][0], beam=3)
+        ll, grads = m.compute_gradients(src, tin, tout, bi, su, tu)
+        norm = m.update_weights(0.3, 2, 0.01, 0.0, len(sents))
+        outs.append((xent, dec["best"].tolist(), dec["best_score"], ll, grads, norm,
+                     {k: m.get_param(k) for k in m.param_names()}))
+    a, b = outs
+    assert a[0] == b[0] and a[1] == b[1] and a[2] == b[2] and a[3] == b[3] and a[5] == b[5]
+    for k in a[4]:
+        assert np.array_equal(a[4][k], b[4][k]), k
+        assert np.array_equal(a[6][k], b[6][k]), k
+
+
+def test_forward_with_other_embedding_size_vs_numpy(orc):
+    """Scoring pass and beam decode at E != H against the independent numpy model."""
+    rng = np.random.default_rng(62)
+    layers, H, E, Vs, Vt, D = 2, 8, 5, 13, 30, 2
+    P, m = _model(orc, rng, layers, H, Vs, Vt, 1, 1, D, E=E)
+    sents = _sentences(rng, Vs, Vt, [5, 3, 7, 4], [4, 6, 2, 5])
+    src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
+    P64 = {k: v.astype(np.float64) for k, v in P.items()}
+    want = R.minibatch_loglik(P64, layers, H, D, sents)
+    assert abs(m.forward_xent(src, tin, tout, bi) - want) < 1e-4 * max(1.0, abs(want))
+    margins = []
+    best, score, _ = R.beam_decode(P, layers, H, Vt, sents[0][0], 3, D, margins=margins, longest=40)
+    assert min(margins) > 1e-4  # no decision closer than fp32 resolves
+    got = m.decode_sentence(sents[0][0], beam=3)
+    assert got["best"].tolist() == list(best)
+    assert abs(got["best_score"] - score) <= 1e-4 * max(1.0, abs(score))
+
+
+@pytest.mark.parametrize("mode,E", [(0, None), (1, None), (2, None), (3, None), (2, 4)])
+def test_update_closed_form(orc, mode, E):
     rng = np.random.default_rng(41 + mode)
     layers, H, Vs, Vt, D = 2, 6, 9, 10, 1
-    P, m = _model(orc, rng, layers, H, Vs, Vt, 1, 1, D, scale=0.8)
+    P, m = _model(orc, rng, layers, H, Vs, Vt, 1, 1, D, scale=0.8, E=E)
     sents = _sentences(rng, Vs, Vt, [5, 3, 4], [4, 3, 5])
     src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
     _, grads = m.compute_gradients(src, tin, tout, bi, su, tu)
