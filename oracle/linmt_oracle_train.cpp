@@ -600,10 +600,40 @@ extern "C" float orc_update_weights(orc_trainer *t, float learning_rate, int cli
   for (auto &kv : t->grads)
     for (auto &v : kv.second) v = (1.0f / minibatch_size) * v;
   float global = 0.f;
-  auto sumsq = [](const Vec &g) {
-    float s = 0.f;
-    for (float v : g) s += v * v;
-    return s;
+  // BasicComputeNormP1 <<<256, 256>>> + BasicComputeNormP2 (src/deep_rnn_kernel.h:616-676): thread
+  // (block, tid) sums the squares of elements block*256 + tid, + 65536, ... in fp32; every block
+  // folds its 256 sums with the shared-memory tree (strides 128, 64, then WarpReduceSum's 32 ... 1,
+  // src/deep_rnn_kernel.h:313-320), and one more such tree folds the 256 block results.
+  auto tree256 = [](std::vector<float> &buf) {
+    for (int stride = 128; stride > 32; stride >>= 1)
+      for (int tid = 0; tid < stride; ++tid) buf[tid] += buf[stride + tid];
+    // WarpReduceSum runs on 32 lanes in lockstep: every lane adds the value the lane 32, 16, ...
+    // above it held BEFORE this step (lanes >= the step width read stale sums that never reach
+    // lane 0; the buffer is padded so that those reads stay in range)
+    for (int off = 32; off >= 1; off >>= 1) {
+      float next[32];
+      for (int tid = 0; tid < 32; ++tid) next[tid] = buf[tid] + buf[tid + off];
+      for (int tid = 0; tid < 32; ++tid) buf[tid] = next[tid];
+    }
+    return buf[0];
+  };
+  auto sumsq = [&](const Vec &g) {
+    constexpr int NT = 256;
+    std::vector<float> part((size_t)NT * NT, 0.f);
+    const size_t n = g.size();
+#pragma omp parallel for schedule(static)
+    for (int t = 0; t < NT * NT; ++t) {
+      float acc = 0.f;
+      for (size_t i = (size_t)t; i < n; i += (size_t)NT * NT) acc += g[i] * g[i];
+      part[t] = acc;
+    }
+    std::vector<float> blocks(NT + 64, 0.f), buf(NT + 64, 0.f);
+    for (int b = 0; b < NT; ++b) {
+      std::fill(buf.begin(), buf.end(), 0.f);
+      std::copy(part.begin() + (size_t)b * NT, part.begin() + (size_t)(b + 1) * NT, buf.begin());
+      blocks[b] = tree256(buf);
+    }
+    return tree256(blocks);
   };
   if (clip_mode == 2) {
     for (auto &kv : t->grads)

@@ -21,15 +21,15 @@ def host():
 
 
 def _pair(orc, host, rng, layers, H, Vs, Vt, D, longest, scale, decoding=None, minibatch=1,
-          attention=1, feed=True):
+          attention=1, feed=True, E=None):
     P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(attention), feed_input=feed,
-                      scale=scale)
+                      scale=scale, E=E)
     om = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=int(feed),
-                   longest_sent=longest)
+                   longest_sent=longest, E=E or 0)
     om.set_params(P)
     gm = host.Model(layers, H, Vs, Vt, longest_sentence=longest, attention_mode=attention,
                     attention_width=D, feed_input=feed, minibatch_size=minibatch,
-                    decoding=decoding)
+                    decoding=decoding, embedding_size=E or 0)
     gm.set_params(P)
     return P, om, gm
 
@@ -172,6 +172,31 @@ def test_decode_no_attention_and_no_feed(orc, host):
         gm.close()
 
 
+@pytest.mark.parametrize("layers,H,E,Vs,Vt,beam,lens,attention,feed",
+                         [(2, 64, None, 120, 150, 4, (9, 4, 12, 1, 6), 2, True),   # global attention
+                          (3, 48, None, 80, 200, 6, (14, 3, 8), 2, False),
+                          (2, 64, 40, 120, 150, 4, (9, 4, 12, 1, 6), 1, True),     # E != H (folded table)
+                          (2, 48, 96, 80, 200, 6, (14, 3, 8), 2, True)])
+def test_decode_global_attention_and_other_embedding_size(orc, host, layers, H, E, Vs, Vt, beam,
+                                                          lens, attention, feed):
+    """Beam decoding with Luong global attention (attention_mode 2: the window is the whole
+    sentence, no projected memory) and with an embedding narrower / wider than the LSTM (the
+    decoder's folded table M*W is then 4H x V from an H x E and an E x V factor), ragged batches,
+    against the oracle's single-sentence searches."""
+    rng = np.random.default_rng(33)
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, 3, 40, 0.4, decoding=(len(lens), beam),
+                      attention=attention, feed=feed, E=E)
+    sents = [rng.integers(0, Vs, size=n) for n in lens]
+    for align in (False, True):
+        got = gm.decode_batch(sents, beam=beam, with_hyps=True, alignments=align)
+        for i, s in enumerate(sents):
+            want = om.decode_sentence(s, beam=beam, alignments=align)
+            _compare_decode(want, got[i], f"attention {attention} E={E} sentence {i} (len {len(s)})")
+            if align:
+                assert got[i]["best_viterbi"].tolist() == want["best_viterbi"].tolist(), i
+    gm.close()
+
+
 def test_decode_config3_architecture(orc, host):
     """The headline architecture at full width (4+4 layers, H=1000, V=30000, beam 12, local-p D=10,
     feed input) on a few short sentences the CPU oracle finishes in seconds."""
@@ -260,15 +285,17 @@ def _ragged_minibatch(rng, B, S, T, Vs, Vt, min_len=1):
     return src, tin, tout, bi, int(lens_t.sum())
 
 
-@pytest.mark.parametrize("layers,H,Vs,Vt,D,B,S,T,attention,feed",
-                         [(2, 64, 90, 110, 3, 9, 12, 10, 1, True),
-                          (4, 128, 300, 500, 10, 16, 20, 18, 1, True),
-                          (2, 64, 90, 110, 3, 9, 12, 10, 2, True),   # global general (build-defined)
-                          (2, 64, 90, 110, 3, 9, 12, 10, 0, False)])
-def test_get_error_vs_oracle(orc, host, layers, H, Vs, Vt, D, B, S, T, attention, feed):
+@pytest.mark.parametrize("layers,H,Vs,Vt,D,B,S,T,attention,feed,E",
+                         [(2, 64, 90, 110, 3, 9, 12, 10, 1, True, None),
+                          (4, 128, 300, 500, 10, 16, 20, 18, 1, True, None),
+                          (2, 64, 90, 110, 3, 9, 12, 10, 2, True, None),   # global general (build-defined)
+                          (2, 64, 90, 110, 3, 9, 12, 10, 0, False, None),
+                          (2, 64, 90, 110, 3, 9, 12, 10, 1, True, 40),     # embedding size != LSTM size
+                          (3, 96, 90, 110, 10, 9, 12, 10, 2, True, 128)])
+def test_get_error_vs_oracle(orc, host, layers, H, Vs, Vt, D, B, S, T, attention, feed, E):
     rng = np.random.default_rng(7)
     P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 30, 0.3, minibatch=B,
-                      attention=attention, feed=feed)
+                      attention=attention, feed=feed, E=E)
     src, tin, tout, bi, n_words = _ragged_minibatch(rng, B, S, T, Vs, Vt)
     want = om.forward_xent(src, tin, tout, bi)
     got = gm.get_error(src, tin, tout, bi)

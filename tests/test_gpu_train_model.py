@@ -27,14 +27,16 @@ def _minibatch(rng, Vs, Vt, lens_s, lens_t):
     return sents, R.pack_minibatch(sents)
 
 
-def _pair(orc, host, rng, layers, H, Vs, Vt, D, attention, feed, B, training, scale=0.5, clip_cell=False):
+def _pair(orc, host, rng, layers, H, Vs, Vt, D, attention, feed, B, training, scale=0.5, clip_cell=False,
+          E=None):
     P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(attention), feed_input=bool(feed),
-                      scale=scale)
-    om = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=int(feed), longest_sent=40)
+                      scale=scale, E=E)
+    om = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=int(feed), longest_sent=40,
+                   E=E or 0)
     om.set_params(P)
     gm = host.Model(layers, H, Vs, Vt, longest_sentence=40, attention_mode=attention,
                     attention_width=D, feed_input=bool(feed), minibatch_size=B, training=training,
-                    clip_cell=clip_cell)
+                    clip_cell=clip_cell, embedding_size=E or 0)
     gm.set_params(P)
     return P, om, gm
 
@@ -53,17 +55,23 @@ CASES = [
     dict(layers=2, H=16, attention=0, feed=0, D=2, seed=63),
     dict(layers=3, H=32, attention=1, feed=1, D=10, seed=64),  # window wider than the sentences
     dict(layers=2, H=16, attention=2, feed=1, D=2, seed=65),   # global attention
+    # embedding size != LSTM size (the reference has E == H; the oracle's generalisation is pinned
+    # by central differences): a wider, a narrower and an unaligned embedding
+    dict(layers=2, H=32, E=24, attention=1, feed=1, D=2, seed=66),
+    dict(layers=2, H=16, E=40, attention=1, feed=1, D=3, seed=67),
+    dict(layers=1, H=16, E=13, attention=2, feed=0, D=2, seed=68),
 ]
 
 
-@pytest.mark.parametrize("case", CASES, ids=lambda c: f"L{c['layers']}H{c['H']}a{c['attention']}f{c['feed']}")
+@pytest.mark.parametrize("case", CASES,
+                         ids=lambda c: f"L{c['layers']}H{c['H']}E{c.get('E', 0)}a{c['attention']}f{c['feed']}")
 def test_compute_gradients_vs_oracle(orc, host, case):
     rng = np.random.default_rng(case["seed"])
     Vs, Vt = 29, 41
     lens_s, lens_t = [5, 3, 9, 4, 7, 1], [4, 6, 2, 8, 5, 3]
     B = len(lens_s)
     P, om, gm = _pair(orc, host, rng, case["layers"], case["H"], Vs, Vt, case["D"],
-                      case["attention"], case["feed"], B, dict(grad_clip_mode=0))
+                      case["attention"], case["feed"], B, dict(grad_clip_mode=0), E=case.get("E"))
     sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
     want_ll, want = om.compute_gradients(src, tin, tout, bi, su, tu)
     got_ll = gm.compute_gradients(src, tin, tout, bi, su, tu)
@@ -85,8 +93,8 @@ def test_compute_gradients_vs_oracle(orc, host, case):
     gm.close()
 
 
-@pytest.mark.parametrize("mode", [0, 1, 2, 3])
-def test_update_weights_vs_oracle(orc, host, mode):
+@pytest.mark.parametrize("mode,E", [(0, None), (1, None), (2, None), (3, None), (2, 24), (1, 8)])
+def test_update_weights_vs_oracle(orc, host, mode, E):
     rng = np.random.default_rng(70 + mode)
     layers, H, Vs, Vt, D = 2, 16, 29, 41, 2
     lens_s, lens_t = [5, 3, 9, 4], [4, 6, 2, 8]
@@ -94,7 +102,7 @@ def test_update_weights_vs_oracle(orc, host, mode):
     lr = 0.7
     # thresholds low enough that every clip is active on these gradients
     opts = dict(learning_rate=lr, grad_clip_mode=mode, norm_clip=0.05, individual_clip=0.002)
-    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 1, 1, B, opts, scale=0.8)
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 1, 1, B, opts, scale=0.8, E=E)
     for it in range(2):  # the second minibatch starts from cleared gradients and updated weights
         sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
         want_ll, _ = om.compute_gradients(src, tin, tout, bi, su, tu)
@@ -134,8 +142,8 @@ def test_gradients_with_error_clip(orc, host):
     assert not np.allclose(outs[0], outs[2], rtol=1e-3, atol=1e-7)
 
 
-@pytest.mark.parametrize("attention", [1, 0])
-def test_compute_gradients_with_dropout_vs_oracle(orc, host, attention):
+@pytest.mark.parametrize("attention,E", [(1, None), (0, None), (1, 24)])
+def test_compute_gradients_with_dropout_vs_oracle(orc, host, attention, E):
     """The model draws its own masks (one uniform tensor per layer and minibatch); the test reads
     them back and hands the very same masks to the oracle."""
     rng = np.random.default_rng(95 + attention)
@@ -143,14 +151,14 @@ def test_compute_gradients_with_dropout_vs_oracle(orc, host, attention):
     lens_s, lens_t = [5, 3, 9, 4, 7, 1], [4, 6, 2, 8, 5, 3]
     B = len(lens_s)
     P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, attention, attention, B,
-                      dict(grad_clip_mode=0, dropout_keep=keep, dropout_seed=7))
+                      dict(grad_clip_mode=0, dropout_keep=keep, dropout_seed=7), E=E)
     sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
     S, T = src.shape[1], tin.shape[1]
     lls = []
     for it in range(2):  # a second minibatch draws new masks
         got_ll = gm.compute_gradients(src, tin, tout, bi, su, tu)
-        se = gm.get_dropout_mask(0, 0, 0, H, B, S)
-        te = gm.get_dropout_mask(0, 1, 0, H, B, T)
+        se = gm.get_dropout_mask(0, 0, 0, E or H, B, S)
+        te = gm.get_dropout_mask(0, 1, 0, E or H, B, T)
         so = np.stack([gm.get_dropout_mask(1, 0, l, H, B, S) if l < layers - 1
                        else np.ones((S, B, H), np.float32) for l in range(layers)])
         to = np.stack([gm.get_dropout_mask(1, 1, l, H, B, T) for l in range(layers)])
