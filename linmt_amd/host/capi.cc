@@ -230,6 +230,23 @@ extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int 
                                     n_hyp, best_viterbi, kbest_index, kbest_score);
 }
 
+extern "C" int lnmt_decode_history(lnmt_model *m, int sentence, int *tok, int *backptr,
+                                   int cap_steps, int *steps) {
+  return Guard([&] {
+    if (!m || !tok || !backptr || !steps) throw LinmtError("lnmt_decode_history: NULL argument");
+    const auto &h = m->nmt->last_history_;
+    if (sentence < 0 || sentence >= h.n) throw LinmtError("lnmt_decode_history: no such sentence in the last batch");
+    const int k = h.slot_of_sentence[sentence], B = h.n * h.beam;
+    const int n_steps = std::min(h.limit[k], cap_steps);  // expansion steps 0 .. limit-1
+    for (int t = 0; t < n_steps; ++t)
+      for (int j = 0; j < h.beam; ++j) {
+        tok[(size_t)t * h.beam + j] = h.tok[(size_t)t * B + (size_t)k * h.beam + j];
+        backptr[(size_t)t * h.beam + j] = h.backptr[(size_t)t * B + (size_t)k * h.beam + j] - k * h.beam;
+      }
+    *steps = n_steps;
+  });
+}
+
 extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_models,
                                           const int *sentences, const int *lengths, int n,
                                           const lnmt_decode_options *o, int *best, int cap,

@@ -440,6 +440,14 @@ class NeuralMachineTranslation {
   SoftmaxLayer softmax_layer_;
   BaseLossLayer *p_softmax_layer_ = &softmax_layer_;
   Decoder decoder_;
+  // Host copy of the beam histories of the last DecodeBatch (what the reference keeps in
+  // eigen_top_sentences_ / new_indices_changes_, src/decoder.h:128-199, step by step): token and
+  // GLOBAL back-pointer column of beam entry (step, column), columns in the batch's internal
+  // order (sentences longest first); slot_of_sentence maps a caller's sentence to its column block.
+  struct DecodeHistory {
+    int n = 0, beam = 0, steps = 0;
+    std::vector<int> slot_of_sentence, limit, tok, backptr;
+  } last_history_;
   DeviceArray<float> p_device_h_tild_previous_;  // decode: gathered h~ of the previous step
   DeviceArray<float> p_device_ensemble_dist_;    // decode in an ensemble: this model's probabilities
   std::vector<hipEvent_t> ensemble_events_;      // owned by the model that runs the beam search

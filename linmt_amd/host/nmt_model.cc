@@ -649,6 +649,11 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   // has drained before any of them is destroyed.
   std::vector<std::vector<int>> src_own, bi_keep;
   std::vector<int> start(B, Decoder::start_symbol_);
+  // ... and the host arrays that asynchronous downloads write at the end
+  std::vector<int> tok, bp, fcount, fbeam;
+  std::vector<float> fscore;
+  std::vector<std::vector<float>> ahists(n_models);
+  std::vector<std::vector<int>> ihists(n_models);
   struct DrainStreams {
     std::vector<NeuralMachineTranslation *> &models;
     ~DrainStreams() {
@@ -843,15 +848,13 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
 
   // one read-back for the whole batch
   const size_t steps = (size_t)max_limit + 1;
-  std::vector<int> tok(steps * B), bp(steps * B), fcount(steps * n), fbeam(steps * B);
-  std::vector<float> fscore(steps * B);
+  tok.resize(steps * B), bp.resize(steps * B), fcount.resize(steps * n), fbeam.resize(steps * B);
+  fscore.resize(steps * B);
   d.tok_hist_.Download(tok.data(), tok.size(), stream_);
   d.backptr_hist_.Download(bp.data(), bp.size(), stream_);
   d.fin_count_hist_.Download(fcount.data(), fcount.size(), stream_);
   d.fin_beam_hist_.Download(fbeam.data(), fbeam.size(), stream_);
   d.fin_score_hist_.Download(fscore.data(), fscore.size(), stream_);
-  std::vector<std::vector<float>> ahists(n_models);
-  std::vector<std::vector<int>> ihists(n_models);
   for (int k = 0; k < n_models; ++k) {
     NeuralMachineTranslation &M = *models[k];
     if (capture) {
@@ -934,6 +937,15 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
         if (std::find(r.kbest.begin(), r.kbest.end(), (int)h) == r.kbest.end())
           std::vector<std::vector<float>>().swap(r.hypotheses[h].alignments_scores);
   }
+  // the streams have been synchronised: the histories are complete and no copy is in flight
+  last_history_.n = n;
+  last_history_.beam = beam;
+  last_history_.steps = (int)steps;
+  last_history_.slot_of_sentence.assign(n, 0);
+  for (int k = 0; k < n; ++k) last_history_.slot_of_sentence[order[k]] = k;
+  last_history_.limit = limit;
+  last_history_.tok = std::move(tok);
+  last_history_.backptr = std::move(bp);
 }
 
 }  // namespace linmt

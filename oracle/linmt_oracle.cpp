@@ -533,6 +533,50 @@ extern "C" void orc_beam_expand_ensemble(const float *const *p, int num_models, 
   *fin_count = nfin;
 }
 
+// How close the decisions of one orc_beam_expand_ensemble call were, on the fp32 numbers it
+// compared: the smallest gap, in log-probability, between
+//   - the last kept (rank beam+1) and the first dropped probability of a live column, and
+//   - two neighbours of the score-ordered candidate list, from its head down to the first
+//     candidate that no longer found a slot (<START> drops and <EOF> finishes included).
+// A step whose margin is 0 holds an exact fp32 tie; one whose margin is below the rounding
+// difference between two summation orders can come out differently on another fp32
+// implementation of the same mathematics.  Not part of the reference: test infrastructure that
+// tells a near-tie from a real difference.  pin: brute force by full sort (this is one).
+extern "C" float orc_beam_step_margin(const float *const *p, int num_models, int V, int beam,
+                                      int step, const float *prev_score, float diversity,
+                                      int start_id, int eof_id) {
+  std::vector<float> dist;
+  renormalise(p, num_models, V, beam, dist);
+  const int cols = step == 0 ? 1 : beam;
+  const int K = beam + 1;
+  float margin = FLT_MAX;
+  std::vector<GlobObj> cands;
+  std::vector<std::pair<float, int>> col(V);
+  for (int i = 0; i < cols; ++i) {
+    for (int j = 0; j < V; ++j) col[j] = {dist[(size_t)j * beam + i], j};
+    const int keep = std::min(K + 1, V);
+    std::partial_sort(col.begin(), col.begin() + keep, col.end(),
+                      [](const std::pair<float, int> &a, const std::pair<float, int> &b) {
+                        return a.first != b.first ? a.first > b.first : a.second < b.second;
+                      });
+    if (V > K) margin = std::min(margin, std::log(col[K - 1].first) - std::log(col[K].first));
+    for (int r = 0; r < std::min(K, V); ++r)
+      cands.push_back(GlobObj{std::log(col[r].first) + prev_score[i] - (float)(r + 1) * diversity, i,
+                              col[r].second});
+  }
+  std::stable_sort(cands.begin(), cands.end(),
+                   [](const GlobObj &a, const GlobObj &b) { return a.val > b.val; });
+  int slots = 0;
+  for (size_t q = 0; q < cands.size(); ++q) {
+    if (q + 1 < cands.size()) margin = std::min(margin, cands[q].val - cands[q + 1].val);
+    if (cands[q].vocab != start_id && cands[q].vocab != eof_id && ++slots == beam) {
+      // the neighbour below the last slot was compared too (it is the first one left out)
+      break;
+    }
+  }
+  return margin;
+}
+
 // SwapStatesDecoding, src/layer_input_to_hidden.h:1517-1531.
 extern "C" void orc_beam_gather(const float *src, float *dst, int H, int B, const int *backptr) {
   for (int k = 0; k < B; ++k)
@@ -730,10 +774,18 @@ struct Hyp {
   std::vector<std::vector<float>> align_scores;
 };
 
+// Per-step record of the search for orc_decode_sentence_trace: the beam after every expansion
+// (tokens, LOCAL back-pointers, scores; beam entries per step) and the step's margin.
+struct DecodeTrace {
+  int *tok, *backptr;
+  float *score, *margin;
+  int cap_steps, steps;
+};
+
 int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
                 const orc_decode_opts *o, bool unk_mode, int *best_tokens, int cap, int *best_len,
                 float *best_score, int *hyp_tokens, int *hyp_len, float *hyp_score, int hyp_cap,
-                int *n_hyp, int *best_viterbi);
+                int *n_hyp, int *best_viterbi, DecodeTrace *trace = nullptr);
 
 }  // namespace
 
@@ -749,6 +801,22 @@ extern "C" int orc_decode_sentence(orc_model *m, const int *src_ids, int S,
                                    float *hyp_score, int hyp_cap, int *n_hyp) {
   return decode_impl(&m, 1, src_ids, S, o, false, best_tokens, cap, best_len, best_score,
                      hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, nullptr);
+}
+
+// orc_decode_sentence that also records the beam after every expansion step and how close that
+// step's decisions were (orc_beam_step_margin): trace_tok / trace_backptr / trace_score hold beam
+// entries per step (back-pointers are beam-local), trace_margin one value per step; *n_steps
+// receives the number of expansion steps recorded (at most cap_steps).
+extern "C" int orc_decode_sentence_trace(orc_model *m, const int *src_ids, int S,
+                                         const orc_decode_opts *o, int *best_tokens, int cap,
+                                         int *best_len, float *best_score, int *trace_tok,
+                                         int *trace_backptr, float *trace_score,
+                                         float *trace_margin, int cap_steps, int *n_steps) {
+  DecodeTrace tr{trace_tok, trace_backptr, trace_score, trace_margin, cap_steps, 0};
+  const int rc = decode_impl(&m, 1, src_ids, S, o, false, best_tokens, cap, best_len, best_score,
+                             nullptr, nullptr, nullptr, 0, nullptr, nullptr, &tr);
+  *n_steps = tr.steps;
+  return rc;
 }
 
 // The same with unk_replacement_mode__ on (layer_attention.h:342-386, decoder.h:1930-1962): every
@@ -783,7 +851,8 @@ namespace {
 int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
                 const orc_decode_opts *o, bool unk_mode,
                 int *best_tokens, int cap, int *best_len, float *best_score, int *hyp_tokens,
-                int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi) {
+                int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi,
+                DecodeTrace *trace) {
 #ifdef _OPENMP
   if (o->num_threads > 0) omp_set_num_threads(o->num_threads);
 #endif
@@ -952,6 +1021,17 @@ int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
     orc_beam_expand_ensemble(dists.data(), num_models, V, B, curr_index, top_scores.data(),
                              o->diversity, o->penalty, start_symbol, end_symbol, tok.data(),
                              bp.data(), sc.data(), &nfin, fin_beam.data(), fin_score.data());
+    if (trace && curr_index < trace->cap_steps) {
+      for (int i = 0; i < B; ++i) {
+        trace->tok[(size_t)curr_index * B + i] = tok[i];
+        trace->backptr[(size_t)curr_index * B + i] = bp[i];
+        trace->score[(size_t)curr_index * B + i] = sc[i];
+      }
+      trace->margin[curr_index] =
+          orc_beam_step_margin(dists.data(), num_models, V, B, curr_index, top_scores.data(),
+                               o->diversity, start_symbol, end_symbol);
+      trace->steps = curr_index + 1;
+    }
     // bookkeeping of decoder.h:436-479
     for (int f = 0; f < nfin; ++f) {
       Hyp h;

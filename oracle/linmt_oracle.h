@@ -118,6 +118,20 @@ int orc_decode_sentence(orc_model *m, const int *src_ids, int S, const orc_decod
                         int *best_tokens, int cap, int *best_len, float *best_score,
                         int *hyp_tokens, int *hyp_len, float *hyp_score, int hyp_cap, int *n_hyp);
 
+/* How close the decisions of one orc_beam_expand_ensemble call were: the smallest gap (in
+ * log-probability, on the fp32 values the expansion compared) between the last kept and the first
+ * dropped probability of a live column, and between neighbours of the score-ordered candidate
+ * list down to the first candidate left without a slot.  0 = an exact tie.  Test infrastructure
+ * (no counterpart in the reference): it tells a near-tie from a real difference. */
+float orc_beam_step_margin(const float *const *p, int num_models, int V, int beam, int step,
+                           const float *prev_score, float diversity, int start_id, int eof_id);
+/* orc_decode_sentence that also records the beam after every expansion step (beam tokens,
+ * beam-local back-pointers and scores per step) and the step's orc_beam_step_margin. */
+int orc_decode_sentence_trace(orc_model *m, const int *src_ids, int S, const orc_decode_opts *o,
+                              int *best_tokens, int cap, int *best_len, float *best_score,
+                              int *trace_tok, int *trace_backptr, float *trace_score,
+                              float *trace_margin, int cap_steps, int *n_steps);
+
 /* The same with the reference's unk_replacement_mode__ on: alignment scores exported at every
  * step, Viterbi alignments carried by the hypotheses, coverage penalty on the real scores.
  * best_viterbi (capacity cap) receives the source position aligned to each token of the 1-best. */

@@ -218,6 +218,17 @@ def beam_expand_ensemble(ps, step, prev_score, diversity=0.0, penalty=0.0, start
     return dict(tok=tok, backptr=bp, score=sc, fin_beam=fb[:n].copy(), fin_score=fs[:n].copy())
 
 
+def beam_step_margin(ps, step, prev_score, diversity=0.0, start_id=0, eof_id=1):
+    """ps: the models' (V, beam) probabilities; the smallest gap the expansion had to resolve."""
+    ps = [np.asfortranarray(p, np.float32) for p in ps]
+    V, beam = ps[0].shape
+    arr = (C.c_void_p * len(ps))(*[p.ctypes.data for p in ps])
+    f = lib().orc_beam_step_margin
+    f.restype = C.c_float
+    return float(f(arr, len(ps), V, beam, step, _p(f32(prev_score)), _f(diversity), start_id,
+                   eof_id))
+
+
 def beam_gather(src, backptr):
     src = np.asfortranarray(src, np.float32)
     H, B = src.shape
@@ -349,6 +360,34 @@ class Model:
         if alignments:
             out["best_viterbi"] = vit[:blen.value].copy()
         return out
+
+    def decode_sentence_trace(self, src_ids, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0,
+                              diversity=0.0, lp_alpha=0.65, cp_beta=0.20, num_threads=0):
+        """decode_sentence plus the beam after every expansion step: dict(best, best_score, steps,
+        tok (n, beam), backptr (n, beam; beam-local), score (n, beam), margin (n,)) where margin is
+        the smallest gap between two candidates the step had to order (orc_beam_step_margin)."""
+        src_ids = i32(src_ids)
+        cap = self.cfg.longest_sent + 2
+        b = min(beam, int(np.sqrt(self.cfg.V_tgt)))
+        o = DecodeOpts(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta,
+                       num_threads)
+        best = np.zeros(cap, np.int32)
+        blen, bscore, nst = C.c_int(0), C.c_float(0), C.c_int(0)
+        tok = np.zeros((cap, b), np.int32)
+        bp = np.zeros((cap, b), np.int32)
+        sc = np.zeros((cap, b), np.float32)
+        mg = np.zeros(cap, np.float32)
+        f = lib().orc_decode_sentence_trace
+        f.restype = C.c_int
+        f.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int,
+                      C.c_void_p, C.c_void_p] + [C.c_void_p] * 4 + [C.c_int, C.c_void_p]
+        steps = f(self.handle, _p(src_ids), src_ids.size, C.byref(o), _p(best), cap,
+                  C.byref(blen), C.byref(bscore), _p(tok), _p(bp), _p(sc), _p(mg), cap,
+                  C.byref(nst))
+        n = nst.value
+        return dict(best=best[:blen.value].copy(), best_score=float(bscore.value), steps=steps,
+                    tok=tok[:n].copy(), backptr=bp[:n].copy(), score=sc[:n].copy(),
+                    margin=mg[:n].copy())
 
     def forward_xent(self, src, tgt_in, tgt_out, batch_info, num_threads=0):
         """src (B,S), tgt_in/tgt_out (B,T) int arrays with -1 padding (column t = timestep t)."""

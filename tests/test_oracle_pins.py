@@ -260,6 +260,75 @@ def test_beam_expand_vs_bruteforce(orc, step, diversity, penalty):
         assert 0 not in got["tok"] and 1 not in got["tok"]
 
 
+def test_beam_step_margin_planted_gaps(orc):
+    """orc_beam_step_margin on distributions whose gaps are planted: two columns with the same
+    logits 0, -0.5, -0.9, -1.0, ... (beam 2, so three candidates per column) and previous scores
+    0 and -0.3 give candidate scores c + {0, -0.3, -0.5, -0.8, -0.9, -1.2}; the two slots are filled
+    by the first two, so the list is compared down to the third."""
+    V, beam = 12, 2
+
+    def dist(z_col):
+        z = np.full((V, beam), -9.0)
+        for b in range(beam):
+            z[2:2 + len(z_col[b]), b] = z_col[b]
+        return scipy.special.softmax(z, axis=0).astype(np.float32)
+
+    prev = np.array([0.0, -0.3], np.float32)
+    base = [0.0, -0.5, -0.9, -1.0]
+    # the closest decision is rank 3 against rank 4 inside a column: 0.1
+    assert abs(orc.beam_step_margin([dist([base, base])], 3, prev) - 0.1) < 1e-5
+    # with the fourth entry far away the closest one is between list neighbours 2 and 3: 0.2
+    far = [0.0, -0.5, -0.9, -4.0]
+    assert abs(orc.beam_step_margin([dist([far, far])], 3, prev) - 0.2) < 1e-5
+    # at step 0 only column 0 is expanded: neighbours 0 / -0.5 / -0.9 -> 0.4 (the third is compared
+    # because it is the first candidate left without a slot)
+    assert abs(orc.beam_step_margin([dist([far, far])], 0, prev) - 0.4) < 1e-5
+    # <EOF> on top of column 0 takes no slot, so the walk goes one candidate further:
+    # c + {0 (EOF), -0.3, -0.5, -0.8, ...}: gaps 0.3, 0.2, 0.3 -> still 0.2, but with the third
+    # real candidate close to the fourth (-0.8 against -0.82) the margin drops to 0.02
+    z = np.full((V, beam), -9.0)
+    z[1, 0], z[2, 0], z[3, 0], z[4, 0] = 0.0, -0.5, -0.9, -4.0
+    z[2, 1], z[3, 1], z[4, 1], z[5, 1] = 0.0, -0.52, -0.9, -4.0
+    c0 = scipy.special.logsumexp(z[:, 0]) - scipy.special.logsumexp(z[:, 1])
+    prev2 = np.array([0.0, -0.3 - c0], np.float32)  # makes both columns' constants equal
+    p = scipy.special.softmax(z, axis=0).astype(np.float32)
+    # list: EOF 0, col1 -0.3, col0 -0.5, col1 -0.82, col0 -0.9 ...; slots = -0.3 and -0.5; compared
+    # down to -0.82: gaps 0.3, 0.2, 0.32 -> 0.2
+    assert abs(orc.beam_step_margin([p], 3, prev2) - 0.2) < 1e-4
+    # an exact tie between the last kept and the first dropped probability of a column
+    tie = [0.0, -0.5, -0.9, -0.9]
+    assert orc.beam_step_margin([dist([tie, far])], 3, prev) == 0.0
+    # invariant on random inputs: never larger than the gap between two neighbouring slots
+    rng = np.random.default_rng(77)
+    for _ in range(20):
+        zz = rng.standard_normal((40, 4)) * 2
+        pp = scipy.special.softmax(zz, axis=0).astype(np.float32)
+        pv = (rng.standard_normal(4) * 0.5).astype(np.float32)
+        out = orc.beam_expand(pp, 2, pv)
+        m = orc.beam_step_margin([pp], 2, pv)
+        assert m >= 0 and m <= np.min(out["score"][:-1] - out["score"][1:]) + 1e-6
+
+
+def test_decode_sentence_trace_matches_plain_decode(orc):
+    """The traced decode is the plain decode plus a record: same 1-best; following the recorded
+    back-pointers from the recorded tokens rebuilds a finished hypothesis of the plain decode."""
+    rng = np.random.default_rng(78)
+    P, m = _tiny_model(orc, rng)
+    src = rng.integers(0, 30, size=7)
+    plain = m.decode_sentence(src, beam=4)
+    tr = m.decode_sentence_trace(src, beam=4)
+    assert tr["best"].tolist() == plain["best"].tolist() and tr["best_score"] == plain["best_score"]
+    n = tr["tok"].shape[0]
+    assert n == plain["steps"] - 1 and tr["margin"].shape == (n,) and np.all(tr["margin"] >= 0)
+    # path of beam entry 0 after the last expansion
+    col, toks = 0, []
+    for t in range(n - 1, -1, -1):
+        toks.append(int(tr["tok"][t, col]))
+        col = int(tr["backptr"][t, col])
+    want = [0] + toks[::-1] + [1]
+    assert any(h.tolist() == want for h, _ in plain["hyps"])
+
+
 def test_beam_gather_composition(orc):
     rng = np.random.default_rng(10)
     x = rng.standard_normal((5, 6)).astype(np.float32)
