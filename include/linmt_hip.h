@@ -171,9 +171,10 @@ int lh_gate_gemm_lstm_cell_f32(int H, int B, const lh_gemm_seg *segs, int nseg, 
  * lh_gemm_f32 / lh_gemm_act_rows_f32. */
 int lh_gemm_kernel_name(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
                         size_t workspace_bytes, int max_planes, char *name, int name_cap);
-/* Tuning and test aids (no counterpart in the reference).
+/* Tuning and test aids (no counterpart in the reference).  Both overrides belong to the CALLING
+ * THREAD: they change nothing for lh_gemm_* calls made from other host threads.
  * lh_gemm_set_config_override: forces tile configuration `config` for every later lh_gemm_* call
- * of the process, config < 0 restores the built-in choice.  Returns the number of configurations
+ * of this thread, config < 0 restores the built-in choice.  Returns the number of configurations
  * (so 0 <= config < return value), LH_ERR_ARG if config is too large.
  * lh_gemm_set_splits_override: likewise forces the K split of lh_gemm_ws_f32 (as far as the
  * workspace allows), splits <= 0 restores the built-in choice; returns the largest split.
@@ -289,9 +290,11 @@ int lh_attn_core_projected_fwd_f32(int H, int B, int D, int hs_steps, const floa
  *
  * lh_logsoftmax_xent_f32 replaces OutputdistPerplexityKernel (src/deep_rnn_kernel.h:433-519) and
  * the host loop of SoftmaxLayer::ComputeLossGpu (src/layer_loss.h:693-701) without the V x B
- * double buffer: in double, logp_tgt[b] = log(exp(z_t - mx)) - log(sum_v exp(z_v - mx)) with
- * z = (double)(logits + bias); *loss_accum += sum_{b: mask01[b]==1} logp_tgt[b] (summed in
- * column order by one thread, like the reference's host loop).  logp_tgt may be NULL.
+ * double buffer: logp_tgt[b] = log(exp(z_t - mx)) - log(sum_v exp(z_v - mx)) in double with
+ * z = logits + bias, where the V exponentials under the sum are single-precision values added up
+ * in double (the reference takes them in double too; the result differs by ~1e-7, against a
+ * tolerance of 1e-5 on a log-probability); *loss_accum += sum_{b: mask01[b]==1} logp_tgt[b].
+ * logp_tgt may be NULL.
  */
 int lh_softmax_fwd_f32(const float *logits, int ldl, const float *bias, int V, int B, float *p,
                        int ldp, lh_stream_t stream);
@@ -433,7 +436,8 @@ int lh_rowsum_acc_f32(const float *A, long long lda, int rows, long long cols, f
  * atomicAdd scatter makes the sum order vary from run to run: here the caller lists, per unique
  * id k, the dx columns that carry that id (seg_cols[seg_start[k] .. seg_start[k+1])), and
  *   small_grad[:,k] = beta*small_grad[:,k] + sum_{s} dx[:, seg_cols[s]]       (E rows)
- * in list order.  Padding columns are simply not listed.  drop_mask (laid out like dx, optional):
+ * added up in an order that the list alone fixes (16 interleaved partial sums, then those in
+ * order), so the result does not vary from run to run.  Padding columns are simply not listed.  drop_mask (laid out like dx, optional):
  * every dx element is first multiplied by (drop_mask < keep) * (1/keep), the embedding dropout of
  * WSmallGradientKernelDropout (src/deep_rnn_kernel.h:288-303).
  */

@@ -134,35 +134,69 @@ __global__ __launch_bounds__(256) void rowsum_kernel(const float *__restrict__ A
 
 // ---------------------------------------------------------------------------------------------
 // Embedding gradient: small_grad[:, k] (+)= sum over the dx columns listed for unique id k.
-// One workgroup per (unique id, 1024-row slab); columns are added in list order.
+// Token frequencies are Zipfian: a few ids own thousands of columns, most own one.  A workgroup
+// takes one id and a slab of 16 * VW rows; its 256 threads are 16 row lanes x 16 column phases,
+// phase p adding up columns p, p + 16, ... of the id's list (four loads in flight per thread), and
+// the 16 partial sums meet in LDS in phase order.  The order of the additions is fixed by the
+// list alone (no atomics), so the result is the same from run to run.
+constexpr int kEgLanes = 16, kEgPhases = 16;
 template <int VW>
 __global__ __launch_bounds__(256) void embed_gather_grad_kernel(
     const float *__restrict__ dx, long long ldx, int E, const int *__restrict__ seg_start,
     const int *__restrict__ seg_cols, const float *__restrict__ drop_mask, float keep, float beta,
     float *__restrict__ small_grad, long long ldg) {
+  __shared__ float part[kEgPhases][kEgLanes * VW + 1];
   const int k = blockIdx.x;
-  const int r = (blockIdx.y * 256 + threadIdx.x) * VW;
-  if (r >= E) return;
+  const int lane = threadIdx.x % kEgLanes, ph = threadIdx.x / kEgLanes;
+  const int r = (blockIdx.y * kEgLanes + lane) * VW;
+  const bool row_ok = r < E;
   const int s0 = seg_start[k], s1 = seg_start[k + 1];
-  Vec<VW> acc, t;
+  const float inv = drop_mask ? 1.0f / keep : 1.0f;
+  Vec<VW> acc;
 #pragma unroll
   for (int i = 0; i < VW; ++i) acc.v[i] = 0.f;
-  const float inv = drop_mask ? 1.0f / keep : 1.0f;
-  for (int s = s0; s < s1; ++s) {
-    const long long o = (long long)seg_cols[s] * ldx + r;
-    t.load(dx + o);
-    if (drop_mask) {
-      Vec<VW> u;
-      u.load(drop_mask + o);
+  if (row_ok) {
+    auto add = [&](const Vec<VW> &t, const Vec<VW> &u) {
 #pragma unroll
-      for (int i = 0; i < VW; ++i) acc.v[i] += t.v[i] * (float)(keep > u.v[i]) * inv;
-    } else {
+      for (int i = 0; i < VW; ++i)
+        acc.v[i] += drop_mask ? t.v[i] * (float)(keep > u.v[i]) * inv : t.v[i];
+    };
+    int s = s0 + ph;
+    for (; s + 3 * kEgPhases < s1; s += 4 * kEgPhases) {
+      long long o[4];
+      Vec<VW> t[4], u[4];
 #pragma unroll
-      for (int i = 0; i < VW; ++i) acc.v[i] += t.v[i];
+      for (int q = 0; q < 4; ++q) o[q] = (long long)seg_cols[s + q * kEgPhases] * ldx + r;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        t[q].load(dx + o[q]);
+        if (drop_mask) u[q].load(drop_mask + o[q]);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) add(t[q], u[q]);
     }
+    for (; s < s1; s += kEgPhases) {
+      const long long o = (long long)seg_cols[s] * ldx + r;
+      Vec<VW> t, u;
+      t.load(dx + o);
+      if (drop_mask) u.load(drop_mask + o);
+      add(t, u);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < VW; ++i) part[ph][lane * VW + i] = acc.v[i];
+  __syncthreads();
+  if (ph != 0 || !row_ok) return;
+#pragma unroll
+  for (int i = 0; i < VW; ++i) {
+    float t = 0.f;
+#pragma unroll
+    for (int q = 0; q < kEgPhases; ++q) t += part[q][lane * VW + i];
+    acc.v[i] = t;
   }
   float *o = small_grad + (long long)k * ldg + r;
   if (beta != 0.f) {
+    Vec<VW> t;
     t.load(o);
 #pragma unroll
     for (int i = 0; i < VW; ++i) acc.v[i] += beta * t.v[i];
@@ -473,11 +507,11 @@ extern "C" int lh_embed_gather_grad_f32(const float *dx, long long ldx, int E, i
                    lh::aligned16(small_grad) && lh::aligned16(drop_mask);
   hipStream_t st = lh::as_stream(stream);
   if (vec)
-    hipLaunchKernelGGL(embed_gather_grad_kernel<4>, dim3(n_unique, (E / 4 + 255) / 256), dim3(256),
-                       0, st, dx, ldx, E, seg_start, seg_cols, drop_mask, keep, beta, small_grad, ldg);
+    hipLaunchKernelGGL(embed_gather_grad_kernel<4>, dim3(n_unique, (E / 4 + kEgLanes - 1) / kEgLanes),
+                       dim3(256), 0, st, dx, ldx, E, seg_start, seg_cols, drop_mask, keep, beta, small_grad, ldg);
   else
-    hipLaunchKernelGGL(embed_gather_grad_kernel<1>, dim3(n_unique, (E + 255) / 256), dim3(256), 0,
-                       st, dx, ldx, E, seg_start, seg_cols, drop_mask, keep, beta, small_grad, ldg);
+    hipLaunchKernelGGL(embed_gather_grad_kernel<1>, dim3(n_unique, (E + kEgLanes - 1) / kEgLanes),
+                       dim3(256), 0, st, dx, ldx, E, seg_start, seg_cols, drop_mask, keep, beta, small_grad, ldg);
   return lh::check_launch("lh_embed_gather_grad_f32");
 }
 

@@ -554,8 +554,10 @@ def test_softmax_xent_loglik(lh, orc, V, B):
     loss = torch.tensor([0.25], dtype=torch.float64, device="cuda")
     lh.logsoftmax_xent(dz, V, db, V, B, dev(tgt), dev(mask), lp, loss)
     wlp, wloss = orc.logsoftmax_xent(z, bias, tgt, mask)
-    assert_close(host(lp, (B,)), wlp, "log p(target)", rtol=1e-9, atol=1e-9)
-    assert_close(loss.item(), wloss + 0.25, "masked loss", rtol=1e-9, atol=1e-9)
+    # the kernel takes the exponentials under the sum in single precision and adds them in
+    # double: |d log p| ~ 1e-7 per column, stated here as 1e-6 (the task's bound is 1e-5)
+    assert_close(host(lp, (B,)), wlp, "log p(target)", rtol=0, atol=1e-6)
+    assert_close(loss.item(), wloss + 0.25, "masked loss", rtol=0, atol=1e-6 * B)
 
 
 def _oracle_beam_step(orc, z, bias, n_sent, beam, step, limit, prev, diversity, penalty):

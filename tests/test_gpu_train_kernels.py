@@ -80,12 +80,20 @@ def test_rowsum_acc(lh, rows, cols, lda):
         assert_close(host(out, (rows,)), want, "row sums", rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("E,U,N", [(1000, 300, 2000), (6, 3, 10), (512, 1, 40)])
-def test_embed_gather_grad(lh, E, U, N):
-    """Against the dense per-id sum in float64 (the definition of the scatter)."""
+@pytest.mark.parametrize("E,U,N,zipf", [(1000, 300, 2000, False), (6, 3, 10, False),
+                                        (512, 1, 40, False), (1024, 400, 9000, True),
+                                        (37, 50, 3000, True)])
+def test_embed_gather_grad(lh, E, U, N, zipf):
+    """Against the dense per-id sum in float64 (the definition of the scatter).  zipf: token
+    frequencies as in text, a few ids own thousands of columns and most own one or two."""
     rng = np.random.default_rng(53)
     dx = uni(rng, E, N)
-    owner = rng.integers(-1, U, size=N)  # -1: padding column, listed nowhere
+    if zipf:
+        p = np.arange(1, U + 1, dtype=np.float64) ** -1.1
+        owner = rng.choice(U, size=N, p=p / p.sum())
+        owner[rng.random(N) < 0.1] = -1
+    else:
+        owner = rng.integers(-1, U, size=N)  # -1: padding column, listed nowhere
     owner[:U] = np.arange(U)
     cols = [np.flatnonzero(owner == k) for k in range(U)]
     seg_start = np.concatenate([[0], np.cumsum([len(c) for c in cols])]).astype(np.int32)
@@ -96,6 +104,9 @@ def test_embed_gather_grad(lh, E, U, N):
         lh.embed_gather_grad(dev(dx), E, E, U, dev(seg_start), dev(seg_cols), g, E, beta)
         want = np.stack([dx[:, c].astype(np.float64).sum(axis=1) for c in cols], axis=1) + beta * g0
         assert_close(host(g, (E, U)), want, "small gradient", rtol=1e-4, atol=1e-5)
+        g2 = dev(g0)
+        lh.embed_gather_grad(dev(dx), E, E, U, dev(seg_start), dev(seg_cols), g2, E, beta)
+        assert torch.equal(g, g2), "the sum must not depend on scheduling"
     # embedding dropout: each dx element passes through (mask < keep) / keep first
     u, keep = rng.random((E, N)).astype(np.float32), 0.8
     g = dev(g0)
