@@ -165,6 +165,44 @@ int lh_gate_gemm_lstm_cell_f32(int H, int B, const lh_gemm_seg *segs, int nseg, 
                                const float *c_prev, const int *mask01, int sigmoid_f64,
                                float cell_clip, float *c, float *h, size_t workspace_bytes,
                                lh_stream_t stream);
+/* Several stacked gate products of one step in ONE launch (no counterpart in the reference, which
+ * issues every layer's 8-12 SGEMMs one after the other, src/node_input_to_hidden.h:297-556,
+ * src/node_hidden_to_hidden.h:248-386).  While decoding, what a step needs from the previous one is
+ * known when the step starts: every layer's recurrent product W_h h_{t-1} and, for the first
+ * target layer, the whole pre-activation (W_h h_{t-1} + Q h~_{t-1} + the folded embedding column).
+ * Handing all of them over together gives the GPU a few thousand tiles at once; the products
+ * that do depend on the step (M h_t of the layer below) then run with half the depth and take the
+ * stored product as their addend (lh_gate_gemm_lstm_cell_f32).
+ * Each problem is sum_s A_s X_s over the 4H x K_s stacked gate matrices and K_s x B inputs, as
+ * stored.  cell != 0: the problem's pre-activations are complete and it ends in the LSTM cell,
+ * fields as the arguments of the same name of lh_gate_gemm_lstm_cell_f32.  cell == 0: the 4H x B
+ * product is stored to out (leading dimension ld_out >= 4H, 16-byte aligned).  No output may
+ * overlap an X operand of any problem of the group.  lh_gate_gemm_group_plan says whether the group
+ * runs this way (*runnable; aligned operands, H a multiple of 4) and names the kernel instance;
+ * when it does not, lh_gate_gemm_group_f32 fails and the caller issues the products one by one. */
+#define LH_GATE_GROUP_MAX 8
+typedef struct lh_gate_problem {
+  lh_gemm_seg segs[LH_GEMM_MAX_SEGS];
+  int nseg;
+  int cell;
+  const float *addend;
+  int ld_addend;
+  const int *addend_col;
+  int addend_ncols;
+  const float *bias4h;
+  const float *c_prev;
+  const int *mask01;
+  int sigmoid_f64;
+  float cell_clip;
+  float *c;
+  float *h;
+  float *out;
+  int ld_out;
+} lh_gate_problem;
+int lh_gate_gemm_group_plan(int H, int B, const lh_gate_problem *problems, int n_problems,
+                            int *runnable, char *name, int name_cap);
+int lh_gate_gemm_group_f32(int H, int B, const lh_gate_problem *problems, int n_problems,
+                           lh_stream_t stream);
 /* Name of the kernel instance lh_gemm_ws_f32 (max_planes = 0) or lh_gemm_planes_f32 would launch
  * for this problem (tile shape and operand flags), as profilers print it; no counterpart in the
  * reference.  Pointers in `segs` are only inspected for alignment; workspace_bytes = 0 describes

@@ -85,6 +85,9 @@ class LstmNode {
   // buffers owned by the layer, one slice per node
   float *p_device_sparse_lookup_ = nullptr;  // layer 1: E x B embedding columns
   float *p_device_pre_x_ = nullptr;  // 4H x B: M*x of this step when the layer computed it for all steps
+  // decoding: W_h*h_{t-1} of this step already sits in the layer's preact_ (the step's grouped
+  // launch put it there); ForwardProp only adds M*x of the layer below
+  bool recurrent_hoisted_ = false;
   float *p_device_gates_ = nullptr;          // 4H x B: i_t, f_t, c_prime_t_tanh, o_t (NULL when not kept)
   float *p_device_c_t_ = nullptr;
   float *p_device_h_t_ = nullptr;
@@ -111,6 +114,10 @@ class LstmNode {
                                float *p_device_c_t_prev);
   // ForwardPropGpu of both node kinds (node_input_to_hidden.h:218-636, node_hidden_to_hidden.h:194-444).
   void ForwardProp();
+  // The node's step as one problem of a grouped launch (lh_gate_gemm_group_f32): complete = the
+  // whole pre-activation with the cell (first target layer while decoding: nothing in it depends
+  // on this step), otherwise only W_h*h_{t-1} into the layer's preact_.
+  void DescribeRecurrentProblem(bool complete, lh_gate_problem *q);
 };
 
 // InputToHiddenLayer (src/layer_input_to_hidden.h:37-378) / HiddenToHiddenLayer

@@ -226,7 +226,13 @@ void LstmNode::ForwardProp() {
   int nseg = 0;
   float beta = 0.f;
   const float *x = nullptr;  // input operand of the product, when the input term is not an addend
-  if (L.input_hoisted_) {
+  if (recurrent_hoisted_) {
+    // W_h*h_{t-1} is already in preact_ (grouped launch at the start of the step): add M*x
+    if (L.input_layer_mode_ || feed || !p_device_h_t_below_)
+      throw LinmtError("LstmNode::ForwardProp: a hoisted recurrent product needs an upper layer");
+    beta = 1.f;
+    x = p_device_h_t_below_;
+  } else if (L.input_hoisted_) {
     // M*x of every step is already in pre_x_all_: this step only adds the recurrent products
     pre = p_device_pre_x_;
     beta = 1.f;
@@ -247,7 +253,7 @@ void LstmNode::ForwardProp() {
     x = p_device_h_t_below_;
   }
   if (x) segs[nseg++] = {L.p_device_m_stack_.get(), 4 * H, x, L.input_size_, L.input_size_};
-  segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
+  if (!recurrent_hoisted_) segs[nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
   if (feed) segs[nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
   const bool drop_out = M.apply_dropout_ && L.out_dropout_;
   const float cell_clip = M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f;
@@ -294,6 +300,36 @@ void LstmNode::ForwardProp() {
                                       drop_out ? M.cfg_.dropout_rate_ : 1.f,
                                       drop_out ? p_device_h_t_dropped_ : nullptr, s),
                  "LstmNode::ForwardPropGpu fused cell");
+}
+
+void LstmNode::DescribeRecurrentProblem(bool complete, lh_gate_problem *q) {
+  LstmLayer &L = *p_layer_;
+  NeuralMachineTranslation &M = *L.p_neural_mt_;
+  const int H = L.lstm_size_;
+  *q = lh_gate_problem{};
+  q->segs[q->nseg++] = {L.p_device_w_h_stack_.get(), 4 * H, p_device_h_t_prev_, H, H};
+  if (!complete) {
+    q->out = L.preact_.get();
+    q->ld_out = 4 * H;
+    return;
+  }
+  const bool feed = L.feed_input_mode_ && 0 != index_;
+  if (!(M.decode_mode_ && L.input_layer_mode_ && !L.source_side_mode_))
+    throw LinmtError("DescribeRecurrentProblem: only the first target layer is complete at step start");
+  if (L.mw_fold_dirty_) L.BuildEmbeddingFold();
+  if (feed) q->segs[q->nseg++] = {L.p_device_q_stack_.get(), 4 * H, p_device_h_tild_, H, H};
+  q->cell = 1;
+  q->addend = L.mw_fold_.get();
+  q->ld_addend = 4 * H;
+  q->addend_col = p_device_input_vocab_indices_;
+  q->addend_ncols = L.vocab_size_;
+  q->bias4h = L.p_device_b_stack_.get();
+  q->c_prev = p_device_c_t_prev_;
+  q->mask01 = p_device_input_vocab_indices_01_;
+  q->sigmoid_f64 = feed ? 1 : 0;
+  q->cell_clip = M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f;
+  q->c = p_device_c_t_;
+  q->h = p_device_h_t_;
 }
 
 // M*[x_0 .. x_{steps-1}] in one GEMM (input layer: after ONE lookup of all steps' embeddings).

@@ -26,6 +26,14 @@ class GemmSeg(C.Structure):
                 ("K", C.c_int)]
 
 
+class GateProblem(C.Structure):
+    _fields_ = [("segs", GemmSeg * LH_GEMM_MAX_SEGS), ("nseg", C.c_int), ("cell", C.c_int),
+                ("addend", C.c_void_p), ("ld_addend", C.c_int), ("addend_col", C.c_void_p),
+                ("addend_ncols", C.c_int), ("bias4h", C.c_void_p), ("c_prev", C.c_void_p),
+                ("mask01", C.c_void_p), ("sigmoid_f64", C.c_int), ("cell_clip", C.c_float),
+                ("c", C.c_void_p), ("h", C.c_void_p), ("out", C.c_void_p), ("ld_out", C.c_int)]
+
+
 # name -> (restype, argtypes); mirrors include/linmt_hip.h one to one.
 SIGNATURES = {
     "lh_abi_version": (C.c_int, []),
@@ -56,6 +64,10 @@ SIGNATURES = {
     "lh_gate_gemm_lstm_cell_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, c_f32p,
                                              C.c_int, c_i32p, C.c_int, c_f32p, c_f32p, c_i32p, C.c_int,
                                              C.c_float, c_f32p, c_f32p, C.c_size_t, C.c_void_p]),
+    "lh_gate_gemm_group_plan": (C.c_int, [C.c_int, C.c_int, C.POINTER(GateProblem), C.c_int,
+                                          C.POINTER(C.c_int), C.c_char_p, C.c_int]),
+    "lh_gate_gemm_group_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GateProblem), C.c_int,
+                                         C.c_void_p]),
     "lh_attn_core_projected_fwd_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, c_f32p,
                                                  C.c_longlong, c_f32p, c_f32p, C.c_longlong, c_f32p,
                                                  c_f32p, C.c_longlong, C.c_longlong, c_i32p, c_i32p,
@@ -259,6 +271,40 @@ def gate_gemm_lstm_cell(H, B, segs, bias4h, c_prev, mask01, c, h, addend=None, l
                                             _ptr(mask01), int(sigmoid_f64), cell_clip, _ptr(c),
                                             _ptr(h), workspace_bytes, _stream(stream)),
           "lh_gate_gemm_lstm_cell_f32")
+
+
+def _gate_problems(problems):
+    """problems: dicts with segs=[(A, lda, X, ldx, K)] and either out/ld_out (plain product) or the
+    cell fields bias4h, c_prev, mask01, c, h (+ addend, ld_addend, addend_col, addend_ncols,
+    sigmoid_f64, cell_clip)."""
+    arr = (GateProblem * len(problems))()
+    d = lambda t: None if t is None else t.data_ptr()  # noqa: E731
+    for q, p in zip(arr, problems):
+        for i, (A, lda, X, ldx, K) in enumerate(p["segs"]):
+            q.segs[i].A, q.segs[i].lda, q.segs[i].X, q.segs[i].ldx, q.segs[i].K = (
+                A.data_ptr(), lda, X.data_ptr(), ldx, K)
+        q.nseg = len(p["segs"])
+        q.cell = int("c" in p)
+        q.addend, q.ld_addend = d(p.get("addend")), p.get("ld_addend", 0)
+        q.addend_col, q.addend_ncols = d(p.get("addend_col")), p.get("addend_ncols", 0)
+        q.bias4h, q.c_prev, q.mask01 = d(p.get("bias4h")), d(p.get("c_prev")), d(p.get("mask01"))
+        q.sigmoid_f64, q.cell_clip = int(p.get("sigmoid_f64", False)), p.get("cell_clip", 0.0)
+        q.c, q.h = d(p.get("c")), d(p.get("h"))
+        q.out, q.ld_out = d(p.get("out")), p.get("ld_out", 0)
+    return arr
+
+
+def gate_gemm_group_plan(H, B, problems):
+    """(runnable, kernel instance name) of lh_gate_gemm_group_f32 on these problems."""
+    r, buf = C.c_int(), C.create_string_buffer(128)
+    check(load().lh_gate_gemm_group_plan(H, B, _gate_problems(problems), len(problems), C.byref(r),
+                                         buf, 128), "lh_gate_gemm_group_plan")
+    return bool(r.value), buf.value.decode()
+
+
+def gate_gemm_group(H, B, problems, stream=None):
+    check(load().lh_gate_gemm_group_f32(H, B, _gate_problems(problems), len(problems),
+                                        _stream(stream)), "lh_gate_gemm_group_f32")
 
 
 def gemm_planes(M, N, segs, C_out, ldc, workspace, max_planes, transA=False, transX=False, beta=0.0,

@@ -279,6 +279,97 @@ def test_lstm_cell_fwd(lh, orc, H, B, feed):
     assert_close(host(h, (H, B)), wh2, "h clip")
 
 
+def test_gate_gemm_group(lh, orc):
+    """lh_gate_gemm_group_f32: one launch holding a cell problem (two K segments, the addend read
+    through a column index, in-place cell state) and plain problems of another depth.  Under a
+    forced tile configuration the group gives the bits of the single launches of the same
+    configuration (lh_gate_gemm_lstm_cell_f32, lh_gemm_f32); under the library's own choice it is
+    checked against float64.  Ragged H and B, a group of one, an unaligned group is refused."""
+    rng = np.random.default_rng(131)
+    L = lh.load()
+    n_cfg = L.lh_gemm_set_config_override(-1)
+
+    def build(H, B, Kcell, Kplain, n_plain):
+        As = [uni(rng, 4 * H, K, s=0.3) for K in Kcell]
+        Xs = [uni(rng, K, B) for K in Kcell]
+        bias, c_prev = uni(rng, 4 * H, s=0.5), uni(rng, H, B)
+        mask = (rng.uniform(size=B) < 0.8).astype(np.int32)
+        V = 19
+        table = uni(rng, 4 * H, V)
+        cols = rng.integers(0, V, size=B).astype(np.int32)
+        plain = [(uni(rng, 4 * H, Kplain, s=0.3), uni(rng, Kplain, B)) for _ in range(n_plain)]
+        dv = dict(segs=[(dev(A), 4 * H, dev(X), K, K) for A, X, K in zip(As, Xs, Kcell)],
+                  bias=dev(bias), mask=dev(mask), table=dev(table), cols=dev(cols),
+                  plain=[[(dev(A), 4 * H, dev(X), Kplain, Kplain)] for A, X in plain])
+        pre = sum(A.astype(np.float64) @ X for A, X in zip(As, Xs)) + table[:, cols]
+        _, wc, wh = orc.lstm_cell_fwd(pre.astype(np.float32), bias, c_prev, mask, feed=True)
+        want_plain = [A.astype(np.float64) @ X for A, X in plain]
+        return dv, c_prev, V, wc, wh, want_plain
+
+    def run_group(H, B, dv, c_prev, V):
+        c = dev(c_prev)
+        h = torch.full((H * B,), float("nan"), device="cuda")
+        outs = [torch.full((4 * H * B,), float("nan"), device="cuda") for _ in dv["plain"]]
+        problems = [dict(segs=dv["segs"], bias4h=dv["bias"], c_prev=c, mask01=dv["mask"], c=c, h=h,
+                         addend=dv["table"], ld_addend=4 * H, addend_col=dv["cols"], addend_ncols=V,
+                         sigmoid_f64=True)]
+        problems += [dict(segs=sg, out=o, ld_out=4 * H) for sg, o in zip(dv["plain"], outs)]
+        ok, name = lh.gate_gemm_group_plan(H, B, problems)
+        if not ok:
+            with pytest.raises(lh.LinmtHipError):
+                lh.gate_gemm_group(H, B, problems)
+            return None
+        assert name.startswith("gate_gemm_group_kernel<")
+        lh.gate_gemm_group(H, B, problems)
+        return host(c, (H, B)), host(h, (H, B)), [host(o, (4 * H, B)) for o in outs], name
+
+    shapes = [(100, 76, (100, 36), 52, 2), (36, 40, (68,), 68, 3), (248, 132, (64, 64), 128, 1),
+              (64, 8, (32,), 32, 0)]
+    try:
+        groups_run = 0
+        for cfg in list(range(n_cfg)) + [-1]:
+            L.lh_gemm_set_config_override(cfg)
+            for H, B, Kc, Kp, n_plain in shapes:
+                dv, c_prev, V, wc, wh, want_plain = build(H, B, Kc, Kp, n_plain)
+                got = run_group(H, B, dv, c_prev, V)
+                if got is None:
+                    assert cfg >= 0  # the library's own choice always finds a tile
+                    continue
+                groups_run += 1
+                gc, gh, gouts, name = got
+                what = f"config {cfg} H={H} B={B} K={Kc}/{Kp}: {name}"
+                assert_close(gc, wc, what + " c")
+                assert_close(gh, wh, what + " h")
+                for o, w in zip(gouts, want_plain):
+                    assert_close(o, w, what + " stored product")
+                if cfg >= 0:
+                    # the same tile configuration one launch at a time: identical bits
+                    fus, _ = lh.gate_gemm_lstm_cell_plan(H, B, dv["segs"], has_addend=True)
+                    if fus:
+                        c = dev(c_prev)
+                        h = torch.empty(H * B, device="cuda")
+                        lh.gate_gemm_lstm_cell(H, B, dv["segs"], dv["bias"], c, dv["mask"], c, h,
+                                               addend=dv["table"], ld_addend=4 * H,
+                                               addend_col=dv["cols"], addend_ncols=V, sigmoid_f64=True)
+                        assert np.array_equal(host(c, (H, B)), gc), what + " c vs single launch"
+                        assert np.array_equal(host(h, (H, B)), gh), what + " h vs single launch"
+                    for sg, o in zip(dv["plain"], gouts):
+                        single = torch.empty(4 * H * B, device="cuda")
+                        lh.gemm(4 * H, B, sg, single, 4 * H)
+                        assert np.array_equal(host(single, (4 * H, B)), o), what + " product vs lh_gemm_f32"
+        assert groups_run >= len(shapes) * 4
+    finally:
+        L.lh_gemm_set_config_override(-1)
+    # H not a multiple of 4: not runnable as a group
+    H, B = 37, 8
+    a, x = dev(uni(rng, 4 * H, 16)), dev(uni(rng, 16, B))
+    o = torch.empty(4 * H * B, device="cuda")
+    ok, name = lh.gate_gemm_group_plan(H, B, [dict(segs=[(a, 4 * H, x, 16, 16)], out=o, ld_out=4 * H)])
+    assert not ok and name == ""
+    with pytest.raises(lh.LinmtHipError):  # an output on top of an operand
+        lh.gate_gemm_group(64, 8, [dict(segs=[(a, 256, x, 16, 16)], out=x, ld_out=256)])
+
+
 def test_gate_gemm_with_the_cell_in_its_epilogue(lh, orc):
     """lh_gate_gemm_lstm_cell_f32 for every tile configuration that can carry the cell: against the
     oracle's cell on float64 pre-activations (tolerance), and bit for bit against the two-call

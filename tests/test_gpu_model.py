@@ -235,6 +235,30 @@ def test_decode_same_with_and_without_the_regrouped_step(orc, host, monkeypatch)
     gm.close()
 
 
+def test_decode_same_with_grouped_gate_products(orc, host, monkeypatch):
+    """LINMT_GROUPED_GATES=1 issues what the previous step fixes of every layer's gate product as
+    one grouped launch (lh_gate_gemm_group_f32) and leaves M*h of the layer below on the chain.
+    Same arithmetic up to the order of two additions: same translations, scores inside the
+    floating-point tolerance, both equal to the oracle's."""
+    rng = np.random.default_rng(17)
+    layers, H, Vs, Vt, D, beam = 4, 96, 200, 260, 4, 6
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 40, 0.35, decoding=(5, beam))
+    sents = [rng.integers(0, Vs, size=n) for n in (17, 9, 12, 3, 21)]
+    plain = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    monkeypatch.setenv("LINMT_GROUPED_GATES", "1")
+    gm.profile(2)
+    grouped = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    assert any("gate_gemm_group_kernel" in k for k in gm.profile_totals()), "the grouped launch did not run"
+    gm.profile(0)
+    monkeypatch.delenv("LINMT_GROUPED_GATES")
+    for i, (a, b) in enumerate(zip(grouped, plain)):
+        assert a["best"].tolist() == b["best"].tolist(), i
+        assert np.isclose(a["best_score"], b["best_score"], rtol=1e-4, atol=1e-5), i
+        assert a["n_hyp"] == b["n_hyp"], i
+        _compare_decode(om.decode_sentence(sents[i], beam=beam), a, f"grouped gates, sentence {i}")
+    gm.close()
+
+
 def test_decode_random_architectures_vs_oracle(orc, host):
     """A seeded sweep over architectures and batch shapes the fixed cases do not hit: 1-4 layers,
     hidden sizes that land on different tile configurations (and on the one- and two-quad attention
