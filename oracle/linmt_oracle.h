@@ -191,6 +191,15 @@ void orc_trainer_destroy(orc_trainer *t);
 void orc_trainer_set_dropout(orc_trainer *t, float keep, const float *src_embed,
                              const float *tgt_embed, const float *src_out, const float *tgt_out,
                              int S, int T, int B);
+/* The reference's --clip-cell (cell_clip_mode__) for the following orc_compute_gradients calls:
+ * c_t clamped to +-cell_clip in the forward pass (src/node_input_to_hidden.h:599-601) and the
+ * errors a node hands on -- to step t-1, to the LSTM layer below, to the attention node through
+ * feed input -- clamped to +-error_clip (src/node_input_to_hidden.h:876-878, 950-952,
+ * src/node_hidden_to_hidden.h:774-776, 877-879).  0 switches a clamp off.
+ * pin: thresholds that never bind give the bits of the unclamped run; with binding thresholds the
+ * gradients agree with central differences of the numpy forward wherever no clamp was active
+ * (tests/test_oracle_train_pins.py). */
+void orc_trainer_set_clip(orc_trainer *t, float cell_clip, float error_clip);
 /* NeuralMachineTranslation::ComputeGradients without its final UpdateWeights: forward with stored
  * activations, then the backward pass.  Arguments as orc_forward_xent; src_unique / tgt_unique are
  * the unique non-pad input ids of the minibatch (the reference's *_wgrad lists).  Returns the summed

@@ -59,6 +59,10 @@ struct orc_trainer {
   // consumer above layer l (next layer, attention node, or softmax) reads that layer's h.
   float keep = 0.f;
   Vec drop_embed[2], drop_out[2];
+  // --clip-cell (cell_clip_mode__): c_t clamped to +-cell_clip in the forward pass
+  // (src/node_input_to_hidden.h:599-601, src/node_hidden_to_hidden.h:416-418) and the errors a node
+  // hands on clamped to +-error_clip (below).  0 = off.
+  float cell_clip = 0.f, error_clip = 0.f;
 };
 
 namespace {
@@ -147,7 +151,7 @@ void cell_forward(orc_trainer *t, const std::string &pfx, int B, CellTape &tp) {
   tp.c.assign((size_t)H * B, 0.f);
   tp.h.assign((size_t)H * B, 0.f);
   orc_lstm_cell_fwd(H, B, p1.data(), p2.data(), tp.feed ? p3.data() : nullptr, bias.data(),
-                    tp.c_prev.data(), tp.mask.data(), tp.feed ? 1 : 0, 0.f, tp.gates.data(),
+                    tp.c_prev.data(), tp.mask.data(), tp.feed ? 1 : 0, t->cell_clip, tp.gates.data(),
                     tp.c.data(), tp.h.data());
 }
 
@@ -182,6 +186,21 @@ void cell_backward(orc_trainer *t, const std::string &pfx, int B, const CellTape
     dh_tild_below->assign(n, 0.f);
     for (int g = 0; g < 4; ++g)
       apply(t, pfx + std::string("Q_") + kGate[g], 1, d[g].data(), B, 1.f, dh_tild_below->data());
+  }
+  // ClipMatKernel on the errors handed on when cell_clip_mode__ is set: d_errn_to_t_ht_m1
+  // (src/node_input_to_hidden.h:876-878, src/node_hidden_to_hidden.h:877-879), the error to the
+  // layer below of a hidden layer (src/node_hidden_to_hidden.h:774-776, before its dropout; the
+  // input layer's error to the embedding is not clamped) and the feed-input error
+  // (src/node_input_to_hidden.h:950-952).  The clamp of d_errn_to_t_ct at :974 / :898 comes after
+  // that buffer's last use and changes nothing.
+  if (t->error_clip > 0.f) {
+    const float lim = t->error_clip;
+    auto clamp_all = [lim](Vec &v) {
+      for (float &x : v) x = x > lim ? lim : (x < -lim ? -lim : x);
+    };
+    clamp_all(dh_prev);
+    if (pfx != "src.0." && pfx != "tgt.0.") clamp_all(dx);
+    if (tp.feed && dh_tild_below) clamp_all(*dh_tild_below);
   }
   // ComputeGradientsGpu
   for (int g = 0; g < 4; ++g) {
@@ -371,6 +390,11 @@ extern "C" void orc_trainer_set_dropout(orc_trainer *t, float keep, const float 
   t->drop_embed[1].assign(tgt_embed, tgt_embed + ne * T);
   t->drop_out[0].assign(src_out, src_out + n * S * L);
   t->drop_out[1].assign(tgt_out, tgt_out + n * T * L);
+}
+
+extern "C" void orc_trainer_set_clip(orc_trainer *t, float cell_clip, float error_clip) {
+  t->cell_clip = cell_clip;
+  t->error_clip = error_clip;
 }
 
 extern "C" float *orc_trainer_grad(orc_trainer *t, const char *name, long long *n_elems) {

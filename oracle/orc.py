@@ -418,6 +418,10 @@ class Model:
         assert so.size == L * S * H * B and to.size == L * T * H * B
         lib().orc_trainer_set_dropout(t, _f(keep), _p(se), _p(te), _p(so), _p(to), S, T, B)
 
+    def set_clip(self, cell_clip=0.0, error_clip=0.0):
+        """The reference's --clip-cell for the following compute_gradients calls (0 = off)."""
+        lib().orc_trainer_set_clip(self._trainer(), _f(cell_clip), _f(error_clip))
+
     def compute_gradients(self, src, tgt_in, tgt_out, batch_info, src_unique, tgt_unique):
         """Forward + backward (no update).  Returns (sum log p, {name: gradient}); matrices come back
         as Fortran-ordered 2-D arrays, the embedding gradients as (E, n_unique)."""

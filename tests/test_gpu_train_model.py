@@ -28,7 +28,7 @@ def _minibatch(rng, Vs, Vt, lens_s, lens_t):
 
 
 def _pair(orc, host, rng, layers, H, Vs, Vt, D, attention, feed, B, training, scale=0.5, clip_cell=False,
-          E=None):
+          E=None, cell_clip=50.0):
     P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(attention), feed_input=bool(feed),
                       scale=scale, E=E)
     om = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=int(feed), longest_sent=40,
@@ -36,7 +36,7 @@ def _pair(orc, host, rng, layers, H, Vs, Vt, D, attention, feed, B, training, sc
     om.set_params(P)
     gm = host.Model(layers, H, Vs, Vt, longest_sentence=40, attention_mode=attention,
                     attention_width=D, feed_input=bool(feed), minibatch_size=B, training=training,
-                    clip_cell=clip_cell, embedding_size=E or 0)
+                    clip_cell=clip_cell, embedding_size=E or 0, cell_clip_threshold=cell_clip)
     gm.set_params(P)
     return P, om, gm
 
@@ -122,20 +122,29 @@ def test_update_weights_vs_oracle(orc, host, mode, E):
 
 
 def test_gradients_with_error_clip(orc, host):
-    """--clip-cell: cell values clamped forward, the errors handed back in time clamped backward.
-    The thresholds are set low enough to be active; the oracle has no such mode, so the check is
-    the property that a clamp which never binds changes nothing, and that a binding one does."""
+    """--clip-cell: cell values clamped forward, the errors a node hands on (to step t-1, to the LSTM
+    layer below, to the attention node through feed input) clamped backward -- against the oracle's
+    restatement of those clamps (pinned by textbook BPTT in tests/test_oracle_train_pins.py).  The
+    thresholds are set low enough to bind; a clamp that never binds changes nothing."""
     rng = np.random.default_rng(81)
-    layers, H, Vs, Vt, D = 2, 16, 29, 41, 2
+    layers, H, Vs, Vt, D = 3, 16, 29, 41, 2
     lens_s, lens_t = [5, 3, 9, 4], [4, 6, 2, 8]
     B = len(lens_s)
     sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
     outs = []
-    for clip_cell, err in ((False, 1000.0), (True, 1000.0), (True, 1e-3)):
+    for clip_cell, cell, err in ((False, 50.0, 1000.0), (True, 50.0, 1000.0), (True, 0.3, 2e-3)):
         r2 = np.random.default_rng(82)
         P, om, gm = _pair(orc, host, r2, layers, H, Vs, Vt, D, 1, 1, B,
-                          dict(grad_clip_mode=0, error_clip_threshold=err), clip_cell=clip_cell)
-        gm.compute_gradients(src, tin, tout, bi, su, tu)
+                          dict(grad_clip_mode=0, error_clip_threshold=err), clip_cell=clip_cell,
+                          cell_clip=cell)
+        got_ll = gm.compute_gradients(src, tin, tout, bi, su, tu)
+        om.set_clip(cell if clip_cell else 0.0, err if clip_cell else 0.0)
+        want_ll, want = om.compute_gradients(src, tin, tout, bi, su, tu)
+        assert_close(got_ll, want_ll, "sum log p(target)", rtol=1e-5, atol=1e-4)
+        for name in om.param_names():
+            shape = _grad_shape(P, name, su, tu)
+            assert_close(gm.get_grad(name, shape), np.asarray(want[name]).reshape(shape, order="F"),
+                         f"clip_cell={clip_cell} cell={cell} err={err}: gradient of {name}", atol=2e-5)
         outs.append(gm.get_grad("src.0.M_i", (H, H)))
         gm.close()
     assert np.array_equal(outs[0], outs[1])

@@ -146,6 +146,90 @@ def test_embedding_rows_outside_the_minibatch_get_no_gradient(orc):
                 assert abs(grads[name][r, k] - fd) <= 2e-3 * max(1.0, abs(fd)), (name, vid, r)
 
 
+def test_error_clip_pins(orc):
+    """The --clip-cell clamps of the backward pass.  (i) Thresholds that never bind give the bits of
+    the unclamped run.  (ii) With a binding threshold, a two-layer model without attention is a
+    plain grid of LSTM cells through source and target, and its gradients must equal textbook
+    backpropagation through time written here in float64 with the error to step t-1 and the error
+    to the layer below clamped where the reference clamps them (src/node_input_to_hidden.h:876-878,
+    src/node_hidden_to_hidden.h:774-776, 877-879; the error to the embedding is not clamped)."""
+    rng = np.random.default_rng(71)
+    L, H, Vs, Vt = 2, 6, 9, 10
+    P, m = _model(orc, rng, L, H, Vs, Vt, 0, 0, 1, scale=0.9)
+    sents = [(np.array([4, 2, 7, 1]), np.array([5, 3, 6]))]
+    src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
+    _, base = m.compute_gradients(src, tin, tout, bi, su, tu)
+    m.set_clip(1000.0, 1000.0)
+    _, loose = m.compute_gradients(src, tin, tout, bi, su, tu)
+    for k in base:
+        assert np.array_equal(base[k], loose[k]), k
+    clip = 0.02
+    m.set_clip(0.0, clip)
+    _, got = m.compute_gradients(src, tin, tout, bi, su, tu)
+    m.set_clip(0.0, 0.0)
+    assert not np.allclose(got["src.0.W_hi"], base["src.0.W_hi"], rtol=1e-3, atol=1e-7)
+
+    # textbook BPTT, float64
+    P64 = {k: v.astype(np.float64) for k, v in P.items()}
+    s_ids, t_ids = sents[0]
+    steps = [("src", int(w)) for w in s_ids[::-1]] + [("tgt", int(w)) for w in np.concatenate([[0], t_ids])]
+    outs = [None] * len(s_ids) + [int(w) for w in np.concatenate([t_ids, [1]])]
+    h = [np.zeros((H, 1)) for _ in range(L)]
+    c = [np.zeros((H, 1)) for _ in range(L)]
+    tape = []
+    for side, w in steps:
+        x = P64[f"{side}.0.W"][:, [w]]
+        row = []
+        for l in range(L):
+            h_new, c_new, (i, f, g, o) = R.lstm_step(P64, f"{side}.{l}.", x, h[l], c[l])
+            row.append(dict(x=x, h_prev=h[l], c_prev=c[l], i=i, f=f, g=g, o=o, c=c_new, h=h_new))
+            h[l], c[l] = h_new, c_new
+            x = h_new
+        tape.append(row)
+    want = {k: np.zeros_like(v) for k, v in P64.items()}
+    dh_next = [np.zeros((H, 1)) for _ in range(L)]
+    dc_next = [np.zeros((H, 1)) for _ in range(L)]
+    for n in range(len(steps) - 1, -1, -1):
+        side, w = steps[n]
+        dh_above = np.zeros((H, 1))
+        if outs[n] is not None:
+            top = tape[n][L - 1]["h"]
+            p = np.exp(R.log_softmax(P64["softmax.D"] @ top + P64["softmax.b_d"][:, None]))
+            dz = -p
+            dz[outs[n], 0] += 1.0
+            want["softmax.D"] += dz @ top.T
+            want["softmax.b_d"] += dz[:, 0]
+            dh_above = P64["softmax.D"].T @ dz
+        for l in range(L - 1, -1, -1):
+            tp, pfx = tape[n][l], f"{side}.{l}."
+            dh = dh_next[l] + dh_above
+            tc = np.tanh(tp["c"])
+            dc = dc_next[l] + dh * tp["o"] * (1 - tc * tc)
+            d = dict(o=dh * tc * tp["o"] * (1 - tp["o"]), f=dc * tp["c_prev"] * tp["f"] * (1 - tp["f"]),
+                     i=dc * tp["g"] * tp["i"] * (1 - tp["i"]), c=dc * tp["i"] * (1 - tp["g"] ** 2))
+            dh_prev, dx = np.zeros((H, 1)), np.zeros((H, 1))
+            for gname in R.GATES:
+                want[pfx + "W_h" + gname] += d[gname] @ tp["h_prev"].T
+                want[pfx + "M_" + gname] += d[gname] @ tp["x"].T
+                want[pfx + "b_" + gname] += d[gname][:, 0]
+                dh_prev += P64[pfx + "W_h" + gname].T @ d[gname]
+                dx += P64[pfx + "M_" + gname].T @ d[gname]
+            dh_next[l] = np.clip(dh_prev, -clip, clip)       # the clamps under test
+            dc_next[l] = dc * tp["f"]
+            if l == 0:
+                want[pfx + "W"][:, [w]] += dx                 # the embedding's error: not clamped
+            else:
+                dh_above = np.clip(dx, -clip, clip)
+    for name in m.param_names():
+        g = got[name].astype(np.float64)
+        if name in ("src.0.W", "tgt.0.W"):
+            full = np.zeros_like(P64[name])
+            full[:, su if name == "src.0.W" else tu] = g
+            g = full
+        np.testing.assert_allclose(g.reshape(want[name].shape, order="F"), want[name], rtol=2e-4,
+                                   atol=2e-6, err_msg=name)
+
+
 def test_explicit_embedding_size_equal_to_lstm_size_changes_nothing(orc):
     """E == H reduction of the embedding-size generalisation: a model created with E = H gives the
     bits of a model created the reference's way (E = 0): log-likelihood, every gradient, the
