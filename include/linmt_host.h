@@ -89,6 +89,16 @@ int lnmt_compute_gradients(lnmt_model *m, const int *source, int source_length,
                            const int *source_wgrad, int len_source_wgrad, const int *target_wgrad,
                            int len_target_wgrad, const int *batch_information, int minibatch_size,
                            double *loss);
+/* The same minibatch driven node by node with the reference's own calls and in its order
+ * (src/deep_rnn.h:1137-1273): BackPropPreprocessGpu / BackProp1 / BackProp2 on the loss layer,
+ * the attention node's BackProp, BackPropPreprocessGpu + BackPropGpu(index) on every LSTM node.
+ * Same gradients as lnmt_compute_gradients up to the order of the sums over steps; not with
+ * dropout.  It exists to show (and test) that the layer classes answer to the reference's calls. */
+int lnmt_compute_gradients_stepwise(lnmt_model *m, const int *source, int source_length,
+                                    const int *target_in, const int *target_out, int target_length,
+                                    const int *source_wgrad, int len_source_wgrad,
+                                    const int *target_wgrad, int len_target_wgrad,
+                                    const int *batch_information, int minibatch_size, double *loss);
 /* Gradient by parameter name; "src.0.W" / "tgt.0.W" are E x len_wgrad (column k = id wgrad[k]). */
 int lnmt_model_get_grad(lnmt_model *m, const char *name, float *data, long long n);
 /* NeuralMachineTranslation::UpdateWeights + ClearGradients.  *global_norm (may be NULL) receives

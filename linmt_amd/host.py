@@ -87,6 +87,7 @@ def load():
     lib.lnmt_compute_gradients.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
                                            C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
                                            C.c_void_p, C.c_int, C.POINTER(C.c_double)]
+    lib.lnmt_compute_gradients_stepwise.argtypes = lib.lnmt_compute_gradients.argtypes
     lib.lnmt_model_get_grad.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
     lib.lnmt_update_weights.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
     lib.lnmt_clear_gradients.argtypes = [C.c_void_p]
@@ -304,8 +305,10 @@ class Model:
                                      C.byref(loss)), "get_error")
         return loss.value
 
-    def compute_gradients(self, src, tgt_in, tgt_out, batch_info, src_unique, tgt_unique):
-        """Forward + backward of one minibatch (no update); returns sum log p(target)."""
+    def compute_gradients(self, src, tgt_in, tgt_out, batch_info, src_unique, tgt_unique,
+                          stepwise=False):
+        """Forward + backward of one minibatch (no update); returns sum log p(target).
+        stepwise: drive the layers node by node with the reference's calls, in its order."""
         src = np.asfortranarray(src, np.int32) if src is not None else None
         tgt_in = np.asfortranarray(tgt_in, np.int32)
         tgt_out = np.asfortranarray(tgt_out, np.int32)
@@ -315,9 +318,10 @@ class Model:
         su = None if src_unique is None else np.ascontiguousarray(src_unique, np.int32)
         tu = np.ascontiguousarray(tgt_unique, np.int32)
         loss = C.c_double(0)
-        _check(load().lnmt_compute_gradients(self.handle, _p(src), S, _p(tgt_in), _p(tgt_out), T,
-                                             _p(su), 0 if su is None else su.size, _p(tu), tu.size,
-                                             _p(bi), B, C.byref(loss)), "compute_gradients")
+        fn = load().lnmt_compute_gradients_stepwise if stepwise else load().lnmt_compute_gradients
+        _check(fn(self.handle, _p(src), S, _p(tgt_in), _p(tgt_out), T,
+                  _p(su), 0 if su is None else su.size, _p(tu), tu.size,
+                  _p(bi), B, C.byref(loss)), "compute_gradients")
         return loss.value
 
     def get_grad(self, name, shape):

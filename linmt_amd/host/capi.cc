@@ -125,6 +125,20 @@ extern "C" int lnmt_compute_gradients(lnmt_model *m, const int *source, int sour
   });
 }
 
+extern "C" int lnmt_compute_gradients_stepwise(lnmt_model *m, const int *source, int source_length,
+                                               const int *target_in, const int *target_out,
+                                               int target_length, const int *source_wgrad,
+                                               int len_source_wgrad, const int *target_wgrad,
+                                               int len_target_wgrad, const int *batch_information,
+                                               int minibatch_size, double *loss) {
+  return Guard([&] {
+    *loss = m->nmt->ComputeGradientsStepwise(source, source_length, target_in, target_out,
+                                             target_length, source_wgrad, len_source_wgrad,
+                                             target_wgrad, len_target_wgrad, batch_information,
+                                             minibatch_size);
+  });
+}
+
 extern "C" int lnmt_model_get_grad(lnmt_model *m, const char *name, float *data, long long n) {
   return Guard([&] {
     std::vector<float> v;

@@ -105,6 +105,19 @@ class LstmNode {
   // GEMM over all steps (BackPropInputAllSteps).
   void BackPropGpu(const float *dh_above, bool above_is_lstm, const float *dh_next,
                    const float *dc_next, bool batched_dx);
+  // The reference's own two-call form (node_input_to_hidden.h:139-140, node_hidden_to_hidden.h:
+  // 133-134), same signatures: BackPropPreprocessGpu hands in the errors of step t+1,
+  // BackPropGpu(index) runs the node's backward step on them and on p_device_d_errt_ht_, the
+  // error from above, which the upper layer / attention node / softmax left there (a pointer the
+  // caller wires, as deep_rnn.h:470-520 does; NULL = none).  The error to the layer below is
+  // written to p_device_d_x_ (the reference's p_device_d_errn_to_t_h_below_); weight gradients
+  // are taken over all steps afterwards (LstmLayer::ComputeGradientsAllSteps), where the
+  // reference's node calls ComputeGradientsGpu per step.
+  float *p_device_d_errn_to_tp1_ht_ = nullptr;
+  float *p_device_d_errn_to_tp1_ct_ = nullptr;
+  float *p_device_d_errt_ht_ = nullptr;
+  void BackPropPreprocessGpu(float *p_device_d_errn_to_tp1_ht, float *p_device_d_errn_to_tp1_ct);
+  void BackPropGpu(int index);
 
   // InputToHidden: UpdateVectorsForwardGpu(idx0, mask01, h_prev, c_prev) (node_input_to_hidden.h:100);
   // HiddenToHidden: UpdateVectorsForwardGpu(mask01, h_prev, c_prev) (node_hidden_to_hidden.h:94).
@@ -291,6 +304,8 @@ class BaseLossLayer {
   virtual void ForwardProp(int index) = 0;
   virtual double ComputeLossGpu(int index) = 0;
   virtual void BackPropPreprocessGpu(float *p_device_h_t, int step) = 0;
+  virtual void BackProp1(int index) = 0;  // layer_loss.h:60: error to h_t of step index
+  virtual void BackProp2(int index) = 0;  // layer_loss.h:61: D and b_d gradients of step index
   virtual void GetDistributionGpuDecoderWrapper() = 0;
   virtual float *GetDistPtr() = 0;
   virtual void SetHTPtr(int index, float *p_device_h_t) = 0;
@@ -319,6 +334,16 @@ class SoftmaxLayer : public BaseLossLayer {
   void GetDistributionGpu(float *p_device_h_t);             // layer_loss.h:797-883
   double ComputeLossGpu(int index) override;                // layer_loss.h:673-704 (+ GetPerplexityGpu :708)
   void BackPropPreprocessGpu(float *p_device_h_t, int step) override;  // layer_loss.h:630-650
+  // One step at a time, as the reference drives the loss layer (deep_rnn.h:1166-1273):
+  // BackProp1 = GetHTGradientGpu (layer_loss.h:547-626): forward of step `index` on the h_t and
+  // the targets BackPropPreprocessGpu selected, log-likelihood into p_device_loss_, and the error
+  // D^T dz into step index's slice of p_device_d_errt_ht_all_; BackProp2 = ComputeDGradientGpu +
+  // ComputeBDGradientGpu (layer_loss.h:887-972) from the same dz, so it follows BackProp1 of the
+  // same index.  ForwardBackwardAllSteps is the batched form of the two.
+  void BackProp1(int index) override;
+  void BackProp2(int index) override;
+  float *p_device_h_t_step_ = nullptr;  // BackPropPreprocessGpu's h_t
+  int dz_index_ = -1;                   // step whose output error p_device_outputdist_ holds
   void GetDistributionGpuDecoderWrapper() override;
   float *GetDistPtr() override { return p_device_outputdist_.get(); }
   void SetHTPtr(int index, float *p) override { v_h_t_[index] = p; }
@@ -513,6 +538,17 @@ class NeuralMachineTranslation {
                           const int *p_host_source_wgrad, int len_source_wgrad,
                           const int *p_host_target_wgrad, int len_target_wgrad,
                           const int *p_host_batch_information, int minibatch_size);
+  // The same minibatch driven the reference's way (deep_rnn.h:1137-1273): after the forward pass,
+  // target step by target step BackPropPreprocessGpu / BackProp1 / BackProp2 on the loss layer,
+  // the attention node's BackProp, then BackPropPreprocessGpu + BackPropGpu(index) on every
+  // LSTM node from the top layer down, and the same over the source side.  Same gradients as
+  // ComputeGradients up to the order of the sums over steps.
+  double ComputeGradientsStepwise(const int *p_host_source, int source_length,
+                                  const int *p_host_target_in, const int *p_host_target_out,
+                                  int target_length, const int *p_host_source_wgrad,
+                                  int len_source_wgrad, const int *p_host_target_wgrad,
+                                  int len_target_wgrad, const int *p_host_batch_information,
+                                  int minibatch_size);
   // UpdateWeights (deep_rnn.h:1326-1412) + ClearGradients: scale, clip, theta += lr * g, zero.
   void UpdateWeights();
   void ClearGradients();
@@ -554,5 +590,17 @@ class NeuralMachineTranslation {
                             int target_length, const int *p_host_batch_information,
                             int minibatch_size, bool per_step_loss);
 };
+
+// The reference's class names.  Its layer classes are templates over the precision with float the
+// only instantiation (precision = float, src/utility_cu.h:42); both node kinds and both layer kinds
+// are one class each here, so code written against the reference's names compiles against these.
+template <typename T>
+using LstmInputHiddenNode = LstmNode;
+template <typename T>
+using LstmHiddenHiddenNode = LstmNode;
+template <typename T>
+using InputToHiddenLayer = LstmLayer;
+template <typename T>
+using HiddenToHiddenLayer = LstmLayer;
 
 }  // namespace linmt

@@ -644,7 +644,7 @@ void SoftmaxLayer::PreprocessGpuVocabIndices(const int *p_host_output_vocab_indi
 
 void SoftmaxLayer::BackPropPreprocessGpu(float *p_device_h_t, int step) {
   // layer_loss.h:630-650: select the target ids / masks of this step (step = t * minibatch)
-  (void)p_device_h_t;
+  p_device_h_t_step_ = p_device_h_t;
   p_device_output_vocab_indices_single_ = p_device_output_vocab_indices_.get() + step;
   p_device_output_vocab_indices_01_single_ = p_device_output_vocab_indices_01_.get() + step;
 }

@@ -181,6 +181,20 @@ void LstmNode::BackPropGpu(const float *dh_above, bool above_is_lstm, const floa
   }
 }
 
+void LstmNode::BackPropPreprocessGpu(float *p_device_d_errn_to_tp1_ht,
+                                     float *p_device_d_errn_to_tp1_ct) {
+  p_device_d_errn_to_tp1_ht_ = p_device_d_errn_to_tp1_ht;
+  p_device_d_errn_to_tp1_ct_ = p_device_d_errn_to_tp1_ct;
+}
+
+void LstmNode::BackPropGpu(int index) {
+  if (index != index_) throw LinmtError("LstmNode::BackPropGpu: index does not name this node");
+  LstmLayer &L = *p_layer_;
+  const bool above_is_lstm = L.layer_number_ < L.p_neural_mt_->cfg_.num_layers_ - 1;  // 0 = input layer
+  BackPropGpu(p_device_d_errt_ht_, above_is_lstm, p_device_d_errn_to_tp1_ht_,
+              p_device_d_errn_to_tp1_ct_, false);
+}
+
 void LstmLayer::BackPropInputAllSteps(int steps) {
   NeuralMachineTranslation &M = *p_neural_mt_;
   const int H = lstm_size_, N = minibatch_size_ * steps;
@@ -423,6 +437,40 @@ void SoftmaxLayer::ForwardBackwardAllSteps(const float *p_device_h_t_all, int st
   }
 }
 
+void SoftmaxLayer::BackProp1(int index) {
+  NeuralMachineTranslation &M = *p_neural_mt_;
+  const int H = lstm_size_, V = output_vocab_size_, B = current_minibatch_;
+  if (!p_device_h_t_step_ || p_device_d_errt_ht_all_.size() == 0)
+    throw LinmtError("SoftmaxLayer::BackProp1: needs InitTraining and BackPropPreprocessGpu");
+  float *dz = p_device_outputdist_.get();
+  ComputeLogits(p_device_h_t_step_, B);
+  {
+    ProfileScope ps(M.profiler_, kTagSoftmaxGrad, 8.0 * V * B);
+    LhErrorWrapper(lh_softmax_xent_grad_f32(dz, V, nullptr, V, B, p_device_output_vocab_indices_single_,
+                                            p_device_output_vocab_indices_01_single_, dz, V,
+                                            p_device_logp_tgt_.get(), p_device_loss_.get(), M.stream_),
+                   "SoftmaxLayer::BackProp1 output error");
+  }
+  lh_gemm_seg sh{p_device_d_.get(), V, dz, V, V};
+  Gemm(M, kTagErrorGemm, H, B, &sh, 1, 1, 0, 0.f,
+       p_device_d_errt_ht_all_.get() + (size_t)H * minibatch_size_ * index, H,
+       "SoftmaxLayer::GetHTGradientGpu");
+  dz_index_ = index;
+}
+
+void SoftmaxLayer::BackProp2(int index) {
+  NeuralMachineTranslation &M = *p_neural_mt_;
+  const int H = lstm_size_, V = output_vocab_size_, B = current_minibatch_;
+  if (index != dz_index_)
+    throw LinmtError("SoftmaxLayer::BackProp2: call it after BackProp1 of the same step");
+  const float *dz = p_device_outputdist_.get();
+  lh_gemm_seg sd{dz, V, p_device_h_t_step_, H, B};
+  Gemm(M, kTagWeightGradGemm, V, H, &sd, 1, 0, 1, 1.f, p_device_d_grad_.get(), V,
+       "SoftmaxLayer::ComputeDGradientGpu");
+  RowSum(M, dz, V, V, B, p_device_b_d_grad_.get());
+  dz_index_ = -1;
+}
+
 bool SoftmaxLayer::GetGrad(const std::string &name, std::vector<float> *out) {
   hipStream_t s = p_neural_mt_->stream_;
   if (name == "D") return DownloadAll(p_device_d_grad_, p_device_d_grad_.size(), out, s);
@@ -525,6 +573,89 @@ double NeuralMachineTranslation::ComputeGradients(
       Ls.ComputeGradientsAllSteps(S, nullptr, nullptr);
     }
   }
+  double loss = 0;
+  softmax_layer_.p_device_loss_.Download(&loss, 1, stream_);
+  Synchronize();
+  profiler_.Collect();
+  return loss;
+}
+
+double NeuralMachineTranslation::ComputeGradientsStepwise(
+    const int *p_host_source, int source_length, const int *p_host_target_in,
+    const int *p_host_target_out, int target_length, const int *p_host_source_wgrad,
+    int len_source_wgrad, const int *p_host_target_wgrad, int len_target_wgrad,
+    const int *p_host_batch_information, int minibatch_size) {
+  if (decode_mode_ || !cfg_.train_mode_)
+    throw LinmtError("ComputeGradientsStepwise: model was not initialised for training");
+  if (minibatch_size != cfg_.minibatch_size_)
+    throw LinmtError("ComputeGradientsStepwise: the minibatch must have exactly minibatch_size_ columns");
+  if (cfg_.dropout_mode_) throw LinmtError("ComputeGradientsStepwise: not with dropout");
+  const int L = cfg_.num_layers_, B = minibatch_size, H = cfg_.lstm_size_;
+  const int S = source_length, T = target_length;
+  const bool seq2seq = cfg_.sequence_to_sequence_mode_;
+  const bool attention = cfg_.attention_mode_ && seq2seq;
+  const bool feed = attention && cfg_.feed_input_mode_;
+  if (T < 1 || (seq2seq && S < 1)) throw LinmtError("ComputeGradientsStepwise: empty minibatch");
+  ForwardTeacherForced(p_host_source, S, p_host_target_in, p_host_target_out, T,
+                       p_host_batch_information, B, false);
+  if (seq2seq) input_layer_source_.PreprocessWGrad(p_host_source, S, B, p_host_source_wgrad, len_source_wgrad);
+  input_layer_target_.PreprocessWGrad(p_host_target_in, T, B, p_host_target_wgrad, len_target_wgrad);
+  if (attention)
+    HipErrorWrapper(hipMemsetAsync(attention_layer_.p_device_total_hs_error_.get(), 0,
+                                   sizeof(float) * (size_t)H * B * S, stream_),
+                    "ZeroAttentionError");
+  LstmLayer &top_tgt = TargetLayer(L - 1);
+  float *dht_all = softmax_layer_.p_device_d_errt_ht_all_.get();
+  // target side (deep_rnn.h:1160-1200)
+  for (int t = T - 1; t >= 0; --t) {
+    float *h_in = attention ? attention_layer_.v_nodes_[t].p_device_final_tmp_2_
+                            : top_tgt.v_nodes_[t].p_device_h_t_;
+    p_softmax_layer_->BackPropPreprocessGpu(h_in, t * B);
+    p_softmax_layer_->BackProp1(t);
+    p_softmax_layer_->BackProp2(t);
+    float *dh_top = dht_all + (size_t)H * B * t;
+    if (attention) {
+      attention_layer_.v_nodes_[t].BackProp(
+          dh_top, (feed && t < T - 1) ? input_layer_target_.p_device_errn_to_t_h_tild_.get() : nullptr);
+      dh_top = attention_layer_.p_device_errn_to_t_ht_p1_.get();
+    }
+    const bool last = t == T - 1;
+    for (int l = L - 1; l >= 0; --l) {
+      LstmLayer &Lt = TargetLayer(l);
+      LstmNode &n = Lt.v_nodes_[t];
+      n.p_device_d_errt_ht_ = l == L - 1 ? dh_top : TargetLayer(l + 1).v_nodes_[t].p_device_d_x_;
+      n.BackPropPreprocessGpu(last ? nullptr : Lt.p_device_d_errn_to_t_ht_m1_.get(),
+                              last ? nullptr : Lt.p_device_d_errn_to_t_ct_m1_.get());
+      n.BackPropGpu(t);
+    }
+  }
+  // source side (deep_rnn.h:1218-1246): the decoder's first step hands its errors to the encoder
+  if (seq2seq) {
+    for (int t = S - 1; t >= 0; --t) {
+      const bool last = t == S - 1;
+      for (int l = L - 1; l >= 0; --l) {
+        LstmLayer &Ls = SourceLayer(l);
+        LstmNode &n = Ls.v_nodes_[t];
+        n.p_device_d_errt_ht_ =
+            l == L - 1 ? (attention ? attention_layer_.p_device_total_hs_error_.get() + (size_t)H * B * t
+                                    : nullptr)
+                       : SourceLayer(l + 1).v_nodes_[t].p_device_d_x_;
+        LstmLayer &from = last ? TargetLayer(l) : Ls;
+        n.BackPropPreprocessGpu(from.p_device_d_errn_to_t_ht_m1_.get(),
+                                from.p_device_d_errn_to_t_ct_m1_.get());
+        n.BackPropGpu(t);
+      }
+    }
+  }
+  // the weight gradients of the LSTM and attention layers, which the reference accumulates node
+  // by node (ComputeGradientsGpu), are taken over all steps at once
+  const float *top_up_all = UpwardState(top_tgt, 0);
+  for (int l = 0; l < L; ++l) {
+    const float *h0 = seq2seq ? SourceLayer(l).v_nodes_[S - 1].p_device_h_t_ : nullptr;
+    TargetLayer(l).ComputeGradientsAllSteps(T, h0, attention ? attention_layer_.final_all_.get() : nullptr);
+    if (seq2seq) SourceLayer(l).ComputeGradientsAllSteps(S, nullptr, nullptr);
+  }
+  if (attention) attention_layer_.ComputeGradientsAllSteps(T, top_up_all);
   double loss = 0;
   softmax_layer_.p_device_loss_.Download(&loss, 1, stream_);
   Synchronize();

@@ -93,6 +93,38 @@ def test_compute_gradients_vs_oracle(orc, host, case):
     gm.close()
 
 
+@pytest.mark.parametrize("case", [CASES[0], CASES[2], CASES[3], CASES[4], CASES[5]],
+                         ids=lambda c: f"L{c['layers']}H{c['H']}E{c.get('E', 0)}a{c['attention']}f{c['feed']}")
+def test_stepwise_reference_calls_give_the_same_gradients(orc, host, case):
+    """The layer classes driven the reference's way -- per target and source step
+    BackPropPreprocessGpu / BackProp1 / BackProp2 on the loss layer, AttentionNode::BackProp,
+    BackPropPreprocessGpu + BackPropGpu(index) on every LSTM node, in the order of
+    NeuralMachineTranslation::ComputeGradients (src/deep_rnn.h:1137-1273) -- against the oracle,
+    and against the batched ComputeGradients of the same model."""
+    rng = np.random.default_rng(case["seed"])
+    Vs, Vt = 29, 41
+    lens_s, lens_t = [5, 3, 9, 4, 7, 1], [4, 6, 2, 8, 5, 3]
+    B = len(lens_s)
+    P, om, gm = _pair(orc, host, rng, case["layers"], case["H"], Vs, Vt, case["D"],
+                      case["attention"], case["feed"], B, dict(grad_clip_mode=0), E=case.get("E"))
+    sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
+    want_ll, want = om.compute_gradients(src, tin, tout, bi, su, tu)
+    got_ll = gm.compute_gradients(src, tin, tout, bi, su, tu, stepwise=True)
+    assert_close(got_ll, want_ll, "sum log p(target)", rtol=1e-5, atol=1e-4)
+    step = {}
+    for name in om.param_names():
+        shape = _grad_shape(P, name, su, tu)
+        step[name] = gm.get_grad(name, shape)
+        assert_close(step[name], np.asarray(want[name]).reshape(shape, order="F"),
+                     f"stepwise gradient of {name}", atol=2e-5)
+    gm.clear_gradients()
+    gm.compute_gradients(src, tin, tout, bi, su, tu)
+    for name in om.param_names():
+        assert_close(gm.get_grad(name, step[name].shape), step[name], f"batched vs stepwise {name}",
+                     atol=2e-5)
+    gm.close()
+
+
 @pytest.mark.parametrize("mode,E", [(0, None), (1, None), (2, None), (3, None), (2, 24), (1, 8)])
 def test_update_weights_vs_oracle(orc, host, mode, E):
     rng = np.random.default_rng(70 + mode)
