@@ -131,13 +131,14 @@ int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int *lengths, i
                       float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
                       float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi,
                       int *kbest_index, float *kbest_score);
-/* The beam of one sentence of the last lnmt_decode_batch call, step by step: tok / backptr hold
- * beam entries per expansion step (entry j of step t: the token chosen and the beam entry of step
- * t-1 it extends, beam-local), what the reference keeps in eigen_top_sentences_ and
- * new_indices_changes_ (src/decoder.h:128-199, 436-479).  *steps receives the number of expansion
- * steps copied (at most cap_steps).  For parity checks against a step-by-step reference. */
-int lnmt_decode_history(lnmt_model *m, int sentence, int *tok, int *backptr, int cap_steps,
-                        int *steps);
+/* The beam of one sentence of the last lnmt_decode_batch call, step by step: tok / backptr / score
+ * hold beam entries per expansion step (entry j of step t: the token chosen, the beam entry of
+ * step t-1 it extends, beam-local, and its path score), what the reference keeps in
+ * eigen_top_sentences_, new_indices_changes_ and top_sentences_scores_ (src/decoder.h:128-199,
+ * 436-479).  score may be NULL.  *steps receives the number of expansion steps copied (at most
+ * cap_steps).  For parity checks against a step-by-step reference. */
+int lnmt_decode_history(lnmt_model *m, int sentence, int *tok, int *backptr, float *score,
+                        int cap_steps, int *steps);
 
 /* The same with an ensemble of n_models models decoded in lockstep (EnsembleFactory::DecodeFile
  * with several models, src/decoder.h:1778-1931): before every beam step the models' distributions

@@ -107,8 +107,8 @@ def load():
                                       C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.lnmt_decode_batch_ensemble.argtypes = [C.POINTER(C.c_void_p), C.c_int] + \
         lib.lnmt_decode_batch.argtypes[1:]
-    lib.lnmt_decode_history.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int,
-                                        C.POINTER(C.c_int)]
+    lib.lnmt_decode_history.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                        C.c_int, C.POINTER(C.c_int)]
     lib.lnmt_model_stream.restype = C.c_void_p
     lib.lnmt_model_stream.argtypes = [C.c_void_p]
     lib.lnmt_profile_set_level.argtypes = [C.c_void_p, C.c_int]
@@ -348,14 +348,15 @@ class Model:
 
     def decode_history(self, sentence, beam):
         """Beam of sentence `sentence` of the last decode_batch call after every expansion step:
-        (tok, backptr), each (steps, beam); back-pointers are beam-local."""
+        (tok, backptr, score), each (steps, beam); back-pointers are beam-local."""
         cap = self.cfg.longest_sentence + 2
         tok = np.zeros((cap, beam), np.int32)
         bp = np.zeros((cap, beam), np.int32)
+        sc = np.zeros((cap, beam), np.float32)
         n = C.c_int(0)
-        _check(load().lnmt_decode_history(self.handle, sentence, _p(tok), _p(bp), cap, C.byref(n)),
-               "decode_history")
-        return tok[:n.value].copy(), bp[:n.value].copy()
+        _check(load().lnmt_decode_history(self.handle, sentence, _p(tok), _p(bp), _p(sc), cap,
+                                          C.byref(n)), "decode_history")
+        return tok[:n.value].copy(), bp[:n.value].copy(), sc[:n.value].copy()
 
     def get_state(self, kind, side, layer, timestep, rows, cols):
         out = np.empty(rows * cols, np.float32)

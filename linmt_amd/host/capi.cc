@@ -244,7 +244,7 @@ extern "C" int lnmt_decode_batch(lnmt_model *m, const int *sentences, const int 
                                     n_hyp, best_viterbi, kbest_index, kbest_score);
 }
 
-extern "C" int lnmt_decode_history(lnmt_model *m, int sentence, int *tok, int *backptr,
+extern "C" int lnmt_decode_history(lnmt_model *m, int sentence, int *tok, int *backptr, float *score,
                                    int cap_steps, int *steps) {
   return Guard([&] {
     if (!m || !tok || !backptr || !steps) throw LinmtError("lnmt_decode_history: NULL argument");
@@ -256,6 +256,7 @@ extern "C" int lnmt_decode_history(lnmt_model *m, int sentence, int *tok, int *b
       for (int j = 0; j < h.beam; ++j) {
         tok[(size_t)t * h.beam + j] = h.tok[(size_t)t * B + (size_t)k * h.beam + j];
         backptr[(size_t)t * h.beam + j] = h.backptr[(size_t)t * B + (size_t)k * h.beam + j] - k * h.beam;
+        if (score) score[(size_t)t * h.beam + j] = h.score[(size_t)t * B + (size_t)k * h.beam + j];
       }
     *steps = n_steps;
   });

@@ -479,6 +479,7 @@ class NeuralMachineTranslation {
   struct DecodeHistory {
     int n = 0, beam = 0, steps = 0;
     std::vector<int> slot_of_sentence, limit, tok, backptr;
+    std::vector<float> score;  // path score of beam entry (step, column)
   } last_history_;
   DeviceArray<float> p_device_h_tild_previous_;  // decode: gathered h~ of the previous step
   DeviceArray<float> p_device_ensemble_dist_;    // decode in an ensemble: this model's probabilities

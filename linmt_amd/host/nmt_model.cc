@@ -680,7 +680,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   std::vector<int> start(B, Decoder::start_symbol_);
   // ... and the host arrays that asynchronous downloads write at the end
   std::vector<int> tok, bp, fcount, fbeam;
-  std::vector<float> fscore;
+  std::vector<float> fscore, bscore;
   std::vector<std::vector<float>> ahists(n_models);
   std::vector<std::vector<int>> ihists(n_models);
   struct DrainStreams {
@@ -795,7 +795,6 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
       HipErrorWrapper(hipStreamWaitEvent(models[k]->stream_, ensemble_events_[0], 0), "ensemble wait failed");
   }
 
-  int cur = 0;
   std::vector<int> active_at(max_limit + 1);
   int *p_device_step_indices = d.current_indices_.get();  // <START> for every column
   for (int step = 0; step <= max_limit; ++step) {
@@ -855,14 +854,14 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
       ProfileScope pm(profiler_, kTagBeamMerge, 8.0 * K * Ba);
       LhErrorWrapper(
           lh_beam_merge_f32(n_active, beam, K, step, d.limit_.get(), d.cand_logp_.get(),
-                            d.cand_id_.get(), d.logp_eof_.get(), d.score_[cur].get(), o.diversity_,
+                            d.cand_id_.get(), d.logp_eof_.get(),
+                            step == 0 ? d.score_[0].get() : d.score_hist_.get() + off - B, o.diversity_,
                             o.penalty_, Decoder::start_symbol_, Decoder::end_symbol_,
                             d.tok_hist_.get() + off, d.backptr_hist_.get() + off,
-                            d.score_[cur ^ 1].get(), d.fin_count_hist_.get() + (size_t)step * n,
+                            d.score_hist_.get() + off, d.fin_count_hist_.get() + (size_t)step * n,
                             d.fin_beam_hist_.get() + off, d.fin_score_hist_.get() + off, stream_),
           "beam merge");
     }
-    cur ^= 1;
     if (step < max_limit) {
       if (n_models > 1) {
         HipErrorWrapper(hipEventRecord(ensemble_events_[0], stream_), "ensemble event record failed");
@@ -878,7 +877,8 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   // one read-back for the whole batch
   const size_t steps = (size_t)max_limit + 1;
   tok.resize(steps * B), bp.resize(steps * B), fcount.resize(steps * n), fbeam.resize(steps * B);
-  fscore.resize(steps * B);
+  fscore.resize(steps * B), bscore.resize(steps * B);
+  d.score_hist_.Download(bscore.data(), bscore.size(), stream_);
   d.tok_hist_.Download(tok.data(), tok.size(), stream_);
   d.backptr_hist_.Download(bp.data(), bp.size(), stream_);
   d.fin_count_hist_.Download(fcount.data(), fcount.size(), stream_);
@@ -975,6 +975,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
   last_history_.limit = limit;
   last_history_.tok = std::move(tok);
   last_history_.backptr = std::move(bp);
+  last_history_.score = std::move(bscore);
 }
 
 }  // namespace linmt
