@@ -113,6 +113,17 @@ def classify_beam_parity(gpu_best, gpu_tok, gpu_bp, gpu_score, trace):
     return "identical", -1, 0.0
 
 
+# HBM-side bytes per launch of the attention kernels at the decode step's size (768 columns, 12 per
+# sentence, S=60, D=10), from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` over
+# `bench.py --kernels` (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch).  Their algorithmic
+# byte count charges every beam column its own window, but the 12 columns of a sentence share one
+# in L2, so the rate against the HBM peak is quoted on the measured bytes.
+MEASURED_ATTN_BYTES = {
+    ("attn_core_fwd (local-p)", 768): int((21098 + 3195) * 1024),
+    ("attn_core_projected_fwd (local-p, decoding)", 768): int((38342 + 3195) * 1024),
+}
+
+
 def bench_fused_kernels(torch, steps, warmup, quick=False):
     from linmt_amd import lib as lh
     lh.load()
