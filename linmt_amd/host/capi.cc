@@ -650,21 +650,26 @@ extern "C" void python_decoder_init(char *msg) {
     decoder_sentence__ = fresh.release();
   } catch (const std::exception &e) {
     Fatal("python_decoder_init", e);
+  } catch (...) {  // nothing may unwind through an extern "C" frame into a ctypes caller
+    Fatal("python_decoder_init", LinmtError("unknown exception"));
   }
 }
 
 extern "C" char *python_decoder_do_job(char *sentence) {
-  delete[] decoder_result__;
-  decoder_result__ = nullptr;
-  std::string output_sentence;
+  // the previous result stays valid until the new one has been built
   try {
+    std::string output_sentence;
     if (!decoder_sentence__) throw LinmtError("python_decoder_init has not been called");
     const std::string input_sentence(sentence ? sentence : "");
     if (!input_sentence.empty()) decoder_sentence__->Process(input_sentence, output_sentence);
+    char *fresh = new char[output_sentence.size() + 1];
+    std::memcpy(fresh, output_sentence.c_str(), output_sentence.size() + 1);
+    delete[] decoder_result__;
+    decoder_result__ = fresh;
   } catch (const std::exception &e) {
     Fatal("python_decoder_do_job", e);
+  } catch (...) {
+    Fatal("python_decoder_do_job", LinmtError("unknown exception"));
   }
-  decoder_result__ = new char[output_sentence.size() + 1];
-  std::memcpy(decoder_result__, output_sentence.c_str(), output_sentence.size() + 1);
   return decoder_result__;
 }
