@@ -242,6 +242,59 @@ def bench_fused_kernels(torch, steps, warmup, quick=False):
             "launches_timed": steps, "kernels": out}
 
 
+def bench_mfma_kernels(torch, steps, warmup):
+    """The decode step's two MFMA kernels alone, at the size one step of the benchmark gives them
+    (768 columns): the output projection D*h~ + b_d and one layer's gate product with the fused
+    LSTM cell, next to a plain 1 GiB copy (the calibration point for clock counters)."""
+    from linmt_amd import lib as lh
+    lh.load()
+    steps = max(steps, 20)
+    dev = "cuda"
+    f = lambda n: (torch.rand(n, device=dev) - 0.5) * 0.16
+
+    def timed(fn):
+        for _ in range(max(warmup, 3)):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps  # us
+
+    out = []
+    n = 256 * 1024 * 1024
+    src, dst = f(n), torch.empty(n, device=dev)
+    us = timed(lambda: dst.copy_(src))
+    out.append({"kernel": "device copy (calibration)", "shape": f"{n} floats", "us": round(us, 2),
+                "GB/s": round(8.0 * n / us / 1e3, 1)})
+    del src, dst
+    H, V, B = 1000, 30000, 768
+    D, bd, x, logits = f(V * H), f(V), f(H * B), torch.empty(V * B, device=dev)
+    us = timed(lambda: lh.gemm(V, B, [(D, V, x, H, H)], logits, V, bias=bd))
+    flop = 2.0 * V * B * H
+    out.append({"kernel": "logits_gemm", "shape": f"M={V} N={B} K={H}", "flop": flop, "us": round(us, 2),
+                "TFLOP/s": round(flop / us / 1e6, 2),
+                "frac_of_peak": round(flop / us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 4)})
+    del D, logits
+    W, M4, hb, hp = f(4 * H * H), f(4 * H * H), f(H * B), f(H * B)
+    b4, cp = f(4 * H), f(H * B)
+    m = torch.ones(B, dtype=torch.int32, device=dev)
+    c, h = torch.empty(H * B, device=dev), torch.empty(H * B, device=dev)
+    segs = [(M4, 4 * H, hb, H, H), (W, 4 * H, hp, H, H)]
+    fusable, name = lh.gate_gemm_lstm_cell_plan(H, B, segs)
+    us = timed(lambda: lh.gate_gemm_lstm_cell(H, B, segs, b4, cp, m, c, h))
+    flop = 2.0 * 4 * H * B * 2 * H
+    out.append({"kernel": "gate_gemm + lstm cell", "instance": name, "fused": fusable,
+                "shape": f"M={4 * H} N={B} K={H}+{H}", "flop": flop, "us": round(us, 2),
+                "TFLOP/s": round(flop / us / 1e6, 2),
+                "frac_of_peak": round(flop / us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 4)})
+    return {"metric": "MFMA kernels alone, fp32 TFLOP/s", "unit": "TFLOP/s",
+            "peak": MFMA_FP32_PEAK_TFLOPS, "launches_timed": steps, "kernels": out}
+
+
 def bench_training(torch, host, steps, warmup, small):
     """One training minibatch (forward with stored activations, backward, global-norm clip at 5,
     SGD update) of the 8+8-layer, 2048-hidden, 1024-embedding, 50k-vocabulary model with local-p
@@ -330,6 +383,9 @@ def main():
                     help="instead of the decode benchmark, time the fused HBM-bound kernels alone "
                          "(at the benchmark's size and at a size that saturates HBM) and print "
                          "one JSON line with their achieved GB/s")
+    ap.add_argument("--mfma-kernels", action="store_true",
+                    help="instead of the decode benchmark, time the decode step's two MFMA kernels "
+                         "alone (output projection, gate product + cell) at 768 columns")
     ap.add_argument("--train", action="store_true",
                     help="instead of the decode benchmark, time one training minibatch of "
                          "BASELINE.json configs[4] and print one JSON line")
@@ -349,6 +405,9 @@ def main():
     host.load()
     if args.kernels:
         print(json.dumps(bench_fused_kernels(torch, args.steps, args.warmup)))
+        return
+    if args.mfma_kernels:
+        print(json.dumps(bench_mfma_kernels(torch, args.steps, args.warmup)))
         return
     if args.train or args.train_small:
         print(json.dumps(bench_training(torch, host, args.steps, args.warmup, args.train_small)))
