@@ -223,6 +223,66 @@ int lh_gemm_set_splits_override(int splits);
 int lh_gemm_config_info(int config, int transA, int transX, int info[8]);
 
 /* ------------------------------------------------------------------------------------------
+ * a4 (second form). The same fp32 products on the bf16 matrix pipe, for callers that opt in.  No
+ * counterpart in the reference (its products are cuBLAS SGEMM calls, src/utility_cu.h:153).
+ * Every fp32 operand value a is held as three bf16 values a1 + a2 + a3 = a (a1 = bf16(a),
+ * a2 = bf16(a - a1), a3 = bf16(a - a1 - a2)); a product a*x is formed as the six bf16 products
+ * a1x1, a1x2, a2x1, a1x3, a2x2, a3x1 -- each exact -- added into an fp32 accumulator.  What is left
+ * out is below 2^-23 |a x| per product, the size of one fp32 rounding; measured against float64 the
+ * results are as close as those of lh_gemm_f32.  v_mfma_f32_32x32x16_bf16 issues at eight times
+ * the fp32 MFMA rate, so six products take 3/8 of the matrix-pipe time.
+ *
+ * Operands are packed ahead of the product ("split planes", opaque to the caller):
+ *   - lh_split_kgroups(K): k-groups (8 k each) of a K-deep segment, K rounded up to 16;
+ *   - lh_split_bytes(D, kgroups): bytes of a packed operand with D rows (A) or columns (X);
+ *   - lh_split_gate_rows(H): the D to size a packed stacked gate matrix with (rows are padded to
+ *     whole cell tiles of 32 rows per gate);
+ *   - lh_split_pack_f32 packs up to LH_SPLIT_PACK_MAX segments in one launch.  A segment is a D x K
+ *     fp32 matrix (k_contiguous: element (d, k) at src[d * ld + k], the layout of an H x B
+ *     activation used as X; otherwise src[k * ld + d], the layout of a stored weight matrix used
+ *     as A) that becomes k-groups [kg_offset, kg_offset + lh_split_kgroups(K)) of an operand of
+ *     kgroups_total k-groups; rows / columns up to the padded extent and k beyond K are written as
+ *     zeros.  Several segments side by side give the operand of a multi-segment product
+ *     ([x; h; h~] against [M | W_h | Q]).  gate_H > 0: src is a stacked 4*gate_H x K gate matrix
+ *     (D = 4 * gate_H) whose rows are laid out in cell-tile order for
+ *     lh_gate_gemm_split_lstm_cell_f32.
+ * A packed X depends on its column count: pack and product must be given the same N / B.
+ * lh_gemm_split_f32: C = epilogue(alpha * A X + beta * C), epilogue exactly as lh_gemm_act_rows_f32.
+ * lh_gate_gemm_split_lstm_cell_f32: lh_gate_gemm_lstm_cell_f32 on packed operands; H must be a
+ * multiple of 8; addend, bias4h, c_prev, c, h 16-byte aligned.  h_planes != NULL: h is also
+ * written as k-groups [hp_kg_offset, hp_kg_offset + lh_split_kgroups(H)) of a packed X operand of
+ * hp_kgroups_total k-groups and B columns (the input of the layer above, or of the next step),
+ * which saves the separate packing launch.
+ * lh_gemm_split_set_config_override: test / tuning aid of the calling thread, like
+ * lh_gemm_set_config_override. */
+#define LH_SPLIT_PACK_MAX 8
+typedef struct lh_split_source {
+  const float *src;
+  int ld;
+  int k_contiguous;
+  int D, K;
+  int gate_H;
+  void *planes;
+  int kgroups_total;
+  int kg_offset;
+} lh_split_source;
+int lh_split_kgroups(int K);
+int lh_split_padded(int D);
+int lh_split_gate_rows(int H);
+size_t lh_split_bytes(int D, int kgroups);
+int lh_split_pack_f32(const lh_split_source *srcs, int n, lh_stream_t stream);
+int lh_gemm_split_f32(int M, int N, int kgroups, const void *A_planes, const void *X_planes,
+                      float alpha, float beta, const float *bias, int act, int act_rows,
+                      const int *colmask, float *C, int ldc, lh_stream_t stream);
+int lh_gate_gemm_split_lstm_cell_f32(int H, int B, int kgroups, const void *W_planes,
+                                     const void *X_planes, const float *addend, int ld_addend,
+                                     const int *addend_col, int addend_ncols, const float *bias4h,
+                                     const float *c_prev, const int *mask01, int sigmoid_f64,
+                                     float cell_clip, float *c, float *h, void *h_planes,
+                                     int hp_kgroups_total, int hp_kg_offset, lh_stream_t stream);
+int lh_gemm_split_set_config_override(int config);
+
+/* ------------------------------------------------------------------------------------------
  * a3. Fused LSTM cell forward: bias add, gate nonlinearities, c_t / h_t update, padding mask,
  * optional cell clip and the dropout mask of the layer above, in one pass over HBM.
  * Replaces ForwardSigmoidKernel / ForwardSigmoidKernelFeed / ForwardTanhKernel(/Feed)
