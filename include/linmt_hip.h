@@ -233,26 +233,29 @@ int lh_gemm_config_info(int config, int transA, int transX, int info[8]);
  * the fp32 MFMA rate, so six products take 3/8 of the matrix-pipe time.
  *
  * Operands are packed ahead of the product ("split planes", opaque to the caller):
- *   - lh_split_kgroups(K): k-groups (8 k each) of a K-deep segment, K rounded up to 16;
+ *   - lh_split_kgroups(K): k-groups (8 k each) a K-deep segment needs, ceil(K / 8);
+ *   - lh_split_kgroups_padded(kgroups): the k-groups of a whole operand, the sum over its segments
+ *     rounded up to whole slabs (a multiple of 8); the groups of padding must hold zeros;
  *   - lh_split_bytes(D, kgroups): bytes of a packed operand with D rows (A) or columns (X);
  *   - lh_split_gate_rows(H): the D to size a packed stacked gate matrix with (rows are padded to
  *     whole cell tiles of 32 rows per gate);
  *   - lh_split_pack_f32 packs up to LH_SPLIT_PACK_MAX segments in one launch.  A segment is a D x K
  *     fp32 matrix (k_contiguous: element (d, k) at src[d * ld + k], the layout of an H x B
  *     activation used as X; otherwise src[k * ld + d], the layout of a stored weight matrix used
- *     as A) that becomes k-groups [kg_offset, kg_offset + lh_split_kgroups(K)) of an operand of
- *     kgroups_total k-groups; rows / columns up to the padded extent and k beyond K are written as
- *     zeros.  Several segments side by side give the operand of a multi-segment product
- *     ([x; h; h~] against [M | W_h | Q]).  gate_H > 0: src is a stacked 4*gate_H x K gate matrix
+ *     as A) that becomes k-groups [kg_offset, kg_offset + kgroups) of an operand of kgroups_total
+ *     k-groups, kgroups >= lh_split_kgroups(K); rows / columns up to the padded extent and k beyond
+ *     K are written as zeros (give the last segment the operand's groups of padding as well).
+ *     Several segments side by side give the operand of a multi-segment product ([x; h; h~]
+ *     against [M | W_h | Q]; every segment but the last needs K % 8 == 0).  gate_H > 0: src is a stacked 4*gate_H x K gate matrix
  *     (D = 4 * gate_H) whose rows are laid out in cell-tile order for
  *     lh_gate_gemm_split_lstm_cell_f32.
  * A packed X depends on its column count: pack and product must be given the same N / B.
  * lh_gemm_split_f32: C = epilogue(alpha * A X + beta * C), epilogue exactly as lh_gemm_act_rows_f32.
  * lh_gate_gemm_split_lstm_cell_f32: lh_gate_gemm_lstm_cell_f32 on packed operands; H must be a
  * multiple of 8; addend, bias4h, c_prev, c, h 16-byte aligned.  h_planes != NULL: h is also
- * written as k-groups [hp_kg_offset, hp_kg_offset + lh_split_kgroups(H)) of a packed X operand of
- * hp_kgroups_total k-groups and B columns (the input of the layer above, or of the next step),
- * which saves the separate packing launch.
+ * written as k-groups [hp_kg_offset, hp_kg_offset + hp_kgroups) of a packed X operand of
+ * hp_kgroups_total k-groups and B columns (the input of the layer above, or of the next step; groups
+ * beyond H / 8 are written as zeros), which saves the separate packing launch.
  * lh_gemm_split_set_config_override: test / tuning aid of the calling thread, like
  * lh_gemm_set_config_override. */
 #define LH_SPLIT_PACK_MAX 8
@@ -265,8 +268,10 @@ typedef struct lh_split_source {
   void *planes;
   int kgroups_total;
   int kg_offset;
+  int kgroups;
 } lh_split_source;
 int lh_split_kgroups(int K);
+int lh_split_kgroups_padded(int kgroups);
 int lh_split_padded(int D);
 int lh_split_gate_rows(int H);
 size_t lh_split_bytes(int D, int kgroups);
@@ -279,7 +284,11 @@ int lh_gate_gemm_split_lstm_cell_f32(int H, int B, int kgroups, const void *W_pl
                                      const int *addend_col, int addend_ncols, const float *bias4h,
                                      const float *c_prev, const int *mask01, int sigmoid_f64,
                                      float cell_clip, float *c, float *h, void *h_planes,
-                                     int hp_kgroups_total, int hp_kg_offset, lh_stream_t stream);
+                                     int hp_kgroups_total, int hp_kg_offset, int hp_kgroups,
+                                     lh_stream_t stream);
+/* Name of the kernel instance the two products above would launch (cell != 0: M = H), as profilers
+ * print it. */
+int lh_gemm_split_kernel_name(int cell, int M, int N, char *name, int name_cap);
 int lh_gemm_split_set_config_override(int config);
 
 /* ------------------------------------------------------------------------------------------

@@ -155,6 +155,17 @@ int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_models, const in
 /* The model's HIP stream (hipStream_t as void*), for callers that time with HIP events. */
 void *lnmt_model_stream(lnmt_model *m);
 
+/* Opt-in arithmetic of a decoding model's largest matrix products (no counterpart in the
+ * reference, whose products are cuBLAS SGEMM calls).  on != 0: while at least min_columns
+ * hypotheses are alive (min_columns <= 0 keeps the current value, 160 at first), a step's stacked
+ * gate products and its output projection are formed from three-way bf16 splits of their fp32
+ * operands on the bf16 matrix pipe (lh_gemm_split_f32, lh_gate_gemm_split_lstm_cell_f32 in
+ * linmt_hip.h): every fp32 product a*x becomes six exact bf16 products added in fp32, which leaves
+ * out less than one fp32 rounding per product.  Everything else -- the encoder, attention, steps
+ * with fewer columns, scoring and training -- keeps the fp32 MFMA products, as does the default.
+ * The environment variable LINMT_SPLIT_PRODUCTS=1 switches it on when a decoding model is created. */
+int lnmt_set_split_products(lnmt_model *m, int on, int min_columns);
+
 /* Live kernel timing with HIP events on the model's stream.  level 0 = off, 1 = the output
  * projection (the dominant matrix product), 2 = every launch of the path.  Totals accumulate
  * over lnmt_decode_batch / lnmt_get_error calls until the level is set again.  Entries are keyed "<call site>" or, for matrix products,

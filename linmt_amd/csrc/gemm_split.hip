@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void split_pack_kernel(const PackArgs a) {
 // ---- the product -----------------------------------------------------------------------------
 struct SplitArgs {
   const u4v *A, *X;
-  int Mp, Np, KG;  // padded rows of A, padded columns of X, k-groups (even)
+  int Mp, Np, KG;  // padded rows of A, padded columns of X, k-groups (a multiple of 8)
   int M, N;        // CELL: M = H
   int tiles_n;
   // plain epilogue
@@ -125,27 +125,32 @@ struct SplitArgs {
   float cell_clip;
   float *c_out, *h_out;
   u4v *h_planes;   // may be null: h as split planes, k-groups hp_kg0.. of an operand with hp_KG
-  int hp_KG, hp_kg0, hp_Np;
+  int hp_KG, hp_kg0, hp_kgn, hp_Np;
 };
 
-template <int BM, int BN>
+// WK wavefront groups share a tile: a slab is 16*WK deep and group wk takes its k-groups 2wk, 2wk+1
+// (a product with few tiles is bound by the chain slab -> fragments -> MFMAs -> barrier of one
+// workgroup; WK shortens that chain).  The groups' partial tiles are added up through LDS.
+template <int BM, int BN, int WK>
 constexpr int split_lds_bytes(bool cell) {
-  const int stages = 2 * 6 * (BM + BN) * 16, tile = cell ? BN * (BM + 4) * 4 : 0;
+  const int stages = 2 * 6 * WK * (BM + BN) * 16, tile = (cell || WK > 1) ? BN * (BM + 4) * 4 : 0;
   return stages > tile ? stages : tile;
 }
 
-template <int BM, int BN, int WM, int WN, bool CELL>
-__global__ __launch_bounds__(64 * WM * WN) void gemm_split_kernel(const SplitArgs g) {
-  constexpr int NT = 64 * WM * WN, TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
+template <int BM, int BN, int WM, int WN, int WK, bool CELL>
+__global__ __launch_bounds__(64 * WM * WN * WK) void gemm_split_kernel(const SplitArgs g) {
+  constexpr int NT = 64 * WM * WN * WK, TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
   static_assert(FM >= 1 && FN >= 1 && TM % 32 == 0 && TN % 32 == 0, "wave tile = 32x32 MFMA tiles");
-  constexpr int UA = 6 * BM, UX = 6 * BN;  // 16-byte units of a slab: 3 planes x 2 k-groups x rows
+  constexpr int KGL = 2 * WK;                         // k-groups of a slab
+  constexpr int UA = 3 * KGL * BM, UX = 3 * KGL * BN;  // 16-byte units of a slab: planes x k-groups x rows
   static_assert(UA % NT == 0, "A units per thread");
   constexpr int NUA = UA / NT, NUX = (UX + NT - 1) / NT;
   constexpr bool kExactX = UX % NT == 0;
   constexpr int STAGE = UA + UX;
   static_assert(!CELL || BM == 4 * kGateRows, "a cell tile holds 32 rows of each gate");
   extern __shared__ u4v lds[];
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, wm = wave % WM, wn = wave / WM;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int wk = wave / (WM * WN), wmn = wave % (WM * WN), wm = wmn % WM, wn = wmn / WM;
   const int l32 = lane % 32, lhi = lane / 32;
   const int logical = lh::xcd_contiguous(blockIdx.x, gridDim.x);
   const int m0 = (logical / g.tiles_n) * BM, n0 = (logical % g.tiles_n) * BN;
@@ -158,17 +163,17 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_split_kernel(const SplitArg
 #pragma unroll
       for (int j = 0; j < 16; ++j) acc[a][b][j] = 0.f;
 
-  // Unit u of the A slab is (plane u / 2BM, k-group (u / BM) % 2, row u % BM); the X units follow.
+  // Unit u of the A slab is (plane u / (KGL BM), k-group (u / BM) % KGL, row u % BM); the X units follow.
   // Scalar slab origins + per-thread byte offsets that never change: no vector ALU in the loop.
   unsigned oa[NUA], ox[NUX];
 #pragma unroll
   for (int i = 0; i < NUA; ++i) {
-    const int u = tid + i * NT, p = u / (2 * BM), kgl = (u / BM) % 2, r = u % BM;
+    const int u = tid + i * NT, p = u / (KGL * BM), kgl = (u / BM) % KGL, r = u % BM;
     oa[i] = (unsigned)((p * g.KG + kgl) * g.Mp + r) * 16u;
   }
 #pragma unroll
   for (int i = 0; i < NUX; ++i) {
-    const int u = (tid + i * NT) % UX, p = u / (2 * BN), kgl = (u / BN) % 2, r = u % BN;
+    const int u = (tid + i * NT) % UX, p = u / (KGL * BN), kgl = (u / BN) % KGL, r = u % BN;
     ox[i] = (unsigned)((p * g.KG + kgl) * g.Np + r) * 16u;
   }
   // Buffer loads: the descriptor and the slab origin are scalars, the unit offset a 32-bit vector
@@ -179,8 +184,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_split_kernel(const SplitArg
       __builtin_amdgcn_make_buffer_rsrc(const_cast<u4v *>(g.A + m0), 0, bytes_a, 0x00020000);
   const __amdgpu_buffer_rsrc_t res_x =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<u4v *>(g.X + n0), 0, bytes_x, 0x00020000);
-  const unsigned step_a = 2u * g.Mp * 16u, step_x = 2u * g.Np * 16u;
-  const int slabs = g.KG / 2;
+  const unsigned step_a = (unsigned)KGL * g.Mp * 16u, step_x = (unsigned)KGL * g.Np * 16u;
+  const int slabs = g.KG / KGL;
   u4v ra[2][NUA], rx[2][NUX];
 
   auto loads = [&](u4v (&qa)[NUA], u4v (&qx)[NUX], int sn) {
@@ -200,7 +205,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_split_kernel(const SplitArg
     for (int i = 0; i < NUX; ++i)
       if (kExactX || tid + i * NT < UX) w[UA + tid + i * NT] = qx[i];
   };
-  const int fa0 = lhi * BM + wm * TM + l32, fx0 = UA + lhi * BN + wn * TN + l32;
+  const int fa0 = (2 * wk + lhi) * BM + wm * TM + l32, fx0 = UA + (2 * wk + lhi) * BN + wn * TN + l32;
   // One slab: its fragments, the next slab from the staging registers to the other LDS stage, the
   // loads of the slab after the next two, 6 MFMAs per 32x32 tile (smallest terms first), barrier.
   auto body = [&](int stage, u4v (&qa)[NUA], u4v (&qx)[NUX], int sn) {
@@ -209,9 +214,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_split_kernel(const SplitArg
 #pragma unroll
     for (int p = 0; p < 3; ++p) {
 #pragma unroll
-      for (int f = 0; f < FM; ++f) fa[p][f] = __builtin_bit_cast(bf16x8, b[fa0 + p * 2 * BM + f * 32]);
+      for (int f = 0; f < FM; ++f) fa[p][f] = __builtin_bit_cast(bf16x8, b[fa0 + p * KGL * BM + f * 32]);
 #pragma unroll
-      for (int f = 0; f < FN; ++f) fx[p][f] = __builtin_bit_cast(bf16x8, b[fx0 + p * 2 * BN + f * 32]);
+      for (int f = 0; f < FN; ++f) fx[p][f] = __builtin_bit_cast(bf16x8, b[fx0 + p * KGL * BN + f * 32]);
     }
     stores(stage ^ 1, qa, qx);
     loads(qa, qx, sn);
@@ -239,20 +244,52 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_split_kernel(const SplitArg
   }
   if (s < slabs) body(0, ra[1], rx[1], s + 3);
 
+  constexpr int LDS_M = BM + 4;
+  float *const S = reinterpret_cast<float *>(lds);  // the tile as S[n][m]; the slab stages are dead
+  if constexpr (WK > 1) {
+    // fixed order: group WK-1 stores its partial tile, the groups below add theirs one after the
+    // other, group 0 keeps the sum in its registers (plain epilogue) or leaves it in S (cell)
+#pragma unroll
+    for (int turn = WK - 1; turn >= (CELL ? 0 : 1); --turn) {
+      if (wk == turn) {
+#pragma unroll
+        for (int a = 0; a < FN; ++a)
+#pragma unroll
+          for (int b = 0; b < FM; ++b)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+              float *e = S + (wn * TN + a * 32 + lhi * 4 + (j / 4) * 8 + (j % 4)) * LDS_M + wm * TM + b * 32 + l32;
+              *e = turn == WK - 1 ? acc[a][b][j] : *e + acc[a][b][j];
+            }
+      }
+      __syncthreads();
+    }
+    if constexpr (!CELL) {
+      if (wk > 0) return;
+#pragma unroll
+      for (int a = 0; a < FN; ++a)
+#pragma unroll
+        for (int b = 0; b < FM; ++b)
+#pragma unroll
+          for (int j = 0; j < 16; ++j)
+            acc[a][b][j] += S[(wn * TN + a * 32 + lhi * 4 + (j / 4) * 8 + (j % 4)) * LDS_M + wm * TM + b * 32 + l32];
+    }
+  }
+
   if constexpr (CELL) {
-    // The four gates of a cell sit in different wavefronts: the tile goes through LDS as S[n][m]
-    // (the slab stages are dead), then every thread takes 8 consecutive rows of one column, which
-    // is also one 16-byte unit of h's split planes.
-    constexpr int LDS_M = BM + 4;
-    float *S = reinterpret_cast<float *>(lds);
+    // The four gates of a cell sit in different wavefronts: the tile goes through LDS, then every
+    // thread takes 8 consecutive rows of one column, which is also one 16-byte unit of h's split
+    // planes.
+    if constexpr (WK == 1) {
 #pragma unroll
-    for (int a = 0; a < FN; ++a)
+      for (int a = 0; a < FN; ++a)
 #pragma unroll
-      for (int b = 0; b < FM; ++b)
+        for (int b = 0; b < FM; ++b)
 #pragma unroll
-        for (int j = 0; j < 16; ++j)
-          S[(wn * TN + a * 32 + lhi * 4 + (j / 4) * 8 + (j % 4)) * LDS_M + wm * TM + b * 32 + l32] = acc[a][b][j];
-    __syncthreads();
+          for (int j = 0; j < 16; ++j)
+            S[(wn * TN + a * 32 + lhi * 4 + (j / 4) * 8 + (j % 4)) * LDS_M + wm * TM + b * 32 + l32] = acc[a][b][j];
+      __syncthreads();
+    }
     const int H = g.M;
     constexpr int kUnits = (kGateRows / 8) * BN;
     for (int idx = tid; idx < kUnits; idx += NT) {
@@ -303,12 +340,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_split_kernel(const SplitArg
 #pragma unroll
         for (int p = 0; p < 3; ++p)
           g.h_planes[((size_t)p * g.hp_KG + g.hp_kg0 + r / 8) * g.hp_Np + n] = out[p];
-        // H/8 odd: the segment ends with a k-group of padding, which must read as zeros whatever
-        // an earlier step (with another column count, hence another layout) left there
-        if ((H / 8) % 2 == 1 && r / 8 == H / 8 - 1) {
+        // k-groups of padding behind the segment must read as zeros whatever an earlier step (with
+        // another column count, hence another layout) left there
+        if (r / 8 == H / 8 - 1) {
+          for (int kg = H / 8; kg < g.hp_kgn; ++kg)
 #pragma unroll
-          for (int p = 0; p < 3; ++p)
-            g.h_planes[((size_t)p * g.hp_KG + g.hp_kg0 + H / 8) * g.hp_Np + n] = u4v{0u, 0u, 0u, 0u};
+            for (int p = 0; p < 3; ++p)
+              g.h_planes[((size_t)p * g.hp_KG + g.hp_kg0 + kg) * g.hp_Np + n] = u4v{0u, 0u, 0u, 0u};
         }
       }
     }
@@ -343,60 +381,82 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_split_kernel(const SplitArg
 }
 
 struct SplitConfig {
-  int bm, bn, wm, wn;
+  int bm, bn, wm, wn, wk;
 };
-// plain products; the built-in choice walks the table in order, 256x128 is reachable by override only
-constexpr SplitConfig kPlain[] = {{128, 128, 2, 2}, {128, 64, 2, 2}, {128, 32, 4, 1}, {256, 128, 4, 2}};
+// plain products; the built-in choice walks the first kAutoPlain in order
+constexpr SplitConfig kPlain[] = {{128, 128, 2, 2, 1}, {128, 64, 2, 2, 1}, {128, 64, 2, 2, 2},
+                                  {128, 32, 4, 1, 2}, {256, 128, 4, 2, 1}, {128, 32, 4, 1, 1}};
 constexpr int kNumPlain = sizeof(kPlain) / sizeof(kPlain[0]);
-constexpr int kAutoPlain = 3;
+constexpr int kAutoPlain = 4;
 // cell products (128 rows = 32 of each gate)
-constexpr SplitConfig kCell[] = {{128, 128, 2, 2}, {128, 64, 2, 2}, {128, 32, 4, 1}};
+constexpr SplitConfig kCell[] = {{128, 128, 2, 2, 1}, {128, 96, 4, 1, 2}, {128, 64, 2, 2, 2},
+                                 {128, 32, 4, 1, 2}, {128, 64, 2, 2, 1}, {128, 32, 4, 1, 4}};
 constexpr int kNumCell = sizeof(kCell) / sizeof(kCell[0]);
+constexpr int kAutoCell = 4;
+constexpr int kMaxKGL = 8;  // k-groups of the deepest slab: operands are padded to a multiple of it
 
 thread_local int g_split_override = -1;
 
-template <int BM, int BN, int WM, int WN, bool CELL>
+template <int BM, int BN, int WM, int WN, int WK, bool CELL>
 int launch_split(SplitArgs &g, hipStream_t s, const char *what) {
-  static_assert(split_lds_bytes<BM, BN>(CELL) <= 160 * 1024, "LDS capacity of a CU");
+  static_assert(split_lds_bytes<BM, BN, WK>(CELL) <= 160 * 1024, "LDS capacity of a CU");
+  static_assert(64 * WM * WN * WK <= 1024, "workgroup size");
   const int tiles_m = CELL ? (g.M + kGateRows - 1) / kGateRows : (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
-  // the kernel reads whole tiles of the padded operands
-  if (tiles_m * BM > g.Mp || g.tiles_n * BN > g.Np)
-    return lh::fail_arg("%s: tile grid %d x %d of %d x %d exceeds the padded operands (%d, %d)", what,
-                        tiles_m, g.tiles_n, BM, BN, g.Mp, g.Np);
-  constexpr int bytes = split_lds_bytes<BM, BN>(CELL);
+  // The kernel reads whole tiles and whole slabs.  Rows of A are padded to whole tiles; a tile of X
+  // may reach past the padded columns (BN = 96): what it reads there belongs to other k-groups or,
+  // past the end of the operand, comes back as zeros from the range-checked buffer loads, and it
+  // only feeds accumulator columns >= N, which are never stored.
+  if (tiles_m * BM > g.Mp || g.KG % (2 * WK))
+    return lh::fail_arg("%s: %d row tiles of %d exceed the %d padded rows, or %d k-groups are not whole slabs",
+                        what, tiles_m, BM, g.Mp, g.KG);
+  constexpr int bytes = split_lds_bytes<BM, BN, WK>(CELL);
   static thread_local bool raised[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return lh::fail_arg("%s: hipGetDevice", what);
   if (bytes > 64 * 1024 && !raised[dev]) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_split_kernel<BM, BN, WM, WN, CELL>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_split_kernel<BM, BN, WM, WN, WK, CELL>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
       return lh::fail_arg("%s: cannot raise the LDS limit to %d bytes", what, bytes);
     raised[dev] = true;
   }
-  gemm_split_kernel<BM, BN, WM, WN, CELL><<<tiles_m * g.tiles_n, 64 * WM * WN, bytes, s>>>(g);
+  gemm_split_kernel<BM, BN, WM, WN, WK, CELL><<<tiles_m * g.tiles_n, 64 * WM * WN * WK, bytes, s>>>(g);
   return lh::check_launch(what);
 }
 
 int launch_plain_index(int c, SplitArgs &g, hipStream_t s) {
+  const char *w = "lh_gemm_split_f32";
   switch (c) {
-    case 0: return launch_split<128, 128, 2, 2, false>(g, s, "lh_gemm_split_f32");
-    case 1: return launch_split<128, 64, 2, 2, false>(g, s, "lh_gemm_split_f32");
-    case 2: return launch_split<128, 32, 4, 1, false>(g, s, "lh_gemm_split_f32");
-    default: return launch_split<256, 128, 4, 2, false>(g, s, "lh_gemm_split_f32");
+    case 0: return launch_split<128, 128, 2, 2, 1, false>(g, s, w);
+    case 1: return launch_split<128, 64, 2, 2, 1, false>(g, s, w);
+    case 2: return launch_split<128, 64, 2, 2, 2, false>(g, s, w);
+    case 3: return launch_split<128, 32, 4, 1, 2, false>(g, s, w);
+    case 4: return launch_split<256, 128, 4, 2, 1, false>(g, s, w);
+    default: return launch_split<128, 32, 4, 1, 1, false>(g, s, w);
   }
 }
 int launch_cell_index(int c, SplitArgs &g, hipStream_t s) {
+  const char *w = "lh_gate_gemm_split_lstm_cell_f32";
   switch (c) {
-    case 0: return launch_split<128, 128, 2, 2, true>(g, s, "lh_gate_gemm_split_lstm_cell_f32");
-    case 1: return launch_split<128, 64, 2, 2, true>(g, s, "lh_gate_gemm_split_lstm_cell_f32");
-    default: return launch_split<128, 32, 4, 1, true>(g, s, "lh_gate_gemm_split_lstm_cell_f32");
+    case 0: return launch_split<128, 128, 2, 2, 1, true>(g, s, w);
+    case 1: return launch_split<128, 96, 4, 1, 2, true>(g, s, w);
+    case 2: return launch_split<128, 64, 2, 2, 2, true>(g, s, w);
+    case 3: return launch_split<128, 32, 4, 1, 2, true>(g, s, w);
+    case 4: return launch_split<128, 64, 2, 2, 1, true>(g, s, w);
+    default: return launch_split<128, 32, 4, 1, 4, true>(g, s, w);
   }
 }
 
-// The largest tile that still gives every CU a workgroup and a half; the smallest one otherwise.
+// Plain: the largest tile that still gives every CU a workgroup and a half, the smallest one
+// otherwise.  Cell (few row tiles, one workgroup per CU at a time): 128x96 while that makes three
+// quarters of the CUs busy, 128x64 down to half of them, 128x32 below (measured at H = 1000).
 int choose(const SplitConfig *table, int n_auto, int n, int rows_tiles128, int M, int N, bool cell) {
   if (g_split_override >= 0 && g_split_override < n) return g_split_override;
+  if (cell) {
+    if (4 * rows_tiles128 * ((N + 95) / 96) >= 3 * kCUs) return 1;
+    if (2 * rows_tiles128 * ((N + 63) / 64) > kCUs) return 2;
+    return 3;
+  }
   for (int c = 0; c < n_auto; ++c) {
     const int tm = cell ? rows_tiles128 : (M + table[c].bm - 1) / table[c].bm;
     const int tn = (N + table[c].bn - 1) / table[c].bn;
@@ -413,7 +473,9 @@ int check_planes(const char *what, const void *p, const char *name) {
 
 }  // namespace
 
-extern "C" int lh_split_kgroups(int K) { return K <= 0 ? 0 : (K + 15) / 16 * 2; }
+extern "C" int lh_split_kgroups(int K) { return K <= 0 ? 0 : (K + 7) / 8; }
+
+extern "C" int lh_split_kgroups_padded(int kgroups) { return kgroups <= 0 ? 0 : round_up(kgroups, kMaxKGL); }
 
 extern "C" int lh_split_padded(int D) { return D <= 0 ? 0 : round_up(D, kPadD); }
 
@@ -439,11 +501,11 @@ extern "C" int lh_split_pack_f32(const lh_split_source *srcs, int n, lh_stream_t
       return lh::fail_arg("lh_split_pack_f32: source %d: a stacked gate matrix has D = 4 * gate_H rows (D=%d, gate_H=%d)", i, q.D, q.gate_H);
     const int rc = check_planes("lh_split_pack_f32", q.planes, "planes");
     if (rc != LH_OK) return rc;
-    const int kgn = lh_split_kgroups(q.K);
-    if (q.kgroups_total < 2 || q.kgroups_total % 2 || q.kg_offset < 0 || q.kg_offset % 2 ||
+    const int kgn = q.kgroups;
+    if (kgn < lh_split_kgroups(q.K) || q.kgroups_total % kMaxKGL || q.kg_offset < 0 ||
         q.kg_offset + kgn > q.kgroups_total)
-      return lh::fail_arg("lh_split_pack_f32: source %d: k-groups [%d, %d) do not fit an operand of %d (both even)", i,
-                          q.kg_offset, q.kg_offset + kgn, q.kgroups_total);
+      return lh::fail_arg("lh_split_pack_f32: source %d: k-groups [%d, %d) must hold K=%d and fit an operand of %d "
+                          "(a multiple of %d)", i, q.kg_offset, q.kg_offset + kgn, q.K, q.kgroups_total, kMaxKGL);
     const int Dp = q.gate_H > 0 ? round_up(lh_split_gate_rows(q.gate_H), kPadD) : round_up(q.D, kPadD);
     if ((size_t)3 * q.kgroups_total * Dp * 16 >= ((size_t)1 << 32))
       return lh::fail_arg("lh_split_pack_f32: source %d: the packed operand must stay below 4 GiB", i);
@@ -465,8 +527,9 @@ extern "C" int lh_split_pack_f32(const lh_split_source *srcs, int n, lh_stream_t
 extern "C" int lh_gemm_split_f32(int M, int N, int kgroups, const void *A_planes, const void *X_planes,
                                  float alpha, float beta, const float *bias, int act, int act_rows,
                                  const int *colmask, float *C, int ldc, lh_stream_t stream) {
-  if (M < 1 || N < 1 || kgroups < 2 || kgroups % 2 || !C || ldc < M)
-    return lh::fail_arg("lh_gemm_split_f32: M=%d N=%d kgroups=%d (even) C=%p ldc=%d", M, N, kgroups, (void *)C, ldc);
+  if (M < 1 || N < 1 || kgroups < kMaxKGL || kgroups % kMaxKGL || !C || ldc < M)
+    return lh::fail_arg("lh_gemm_split_f32: M=%d N=%d kgroups=%d (a multiple of %d) C=%p ldc=%d", M, N, kgroups,
+                        kMaxKGL, (void *)C, ldc);
   if (act != LH_ACT_NONE && act != LH_ACT_TANH) return lh::fail_arg("lh_gemm_split_f32: act=%d", act);
   int rc = check_planes("lh_gemm_split_f32", A_planes, "A_planes");
   if (rc == LH_OK) rc = check_planes("lh_gemm_split_f32", X_planes, "X_planes");
@@ -489,11 +552,11 @@ extern "C" int lh_gate_gemm_split_lstm_cell_f32(int H, int B, int kgroups, const
                                                 const float *bias4h, const float *c_prev,
                                                 const int *mask01, int sigmoid_f64, float cell_clip,
                                                 float *c, float *h, void *h_planes,
-                                                int hp_kgroups_total, int hp_kg_offset,
+                                                int hp_kgroups_total, int hp_kg_offset, int hp_kgroups,
                                                 lh_stream_t stream) {
   const char *what = "lh_gate_gemm_split_lstm_cell_f32";
-  if (H < 8 || H % 8 || B < 1 || kgroups < 2 || kgroups % 2)
-    return lh::fail_arg("%s: H=%d (a multiple of 8) B=%d kgroups=%d (even)", what, H, B, kgroups);
+  if (H < 8 || H % 8 || B < 1 || kgroups < kMaxKGL || kgroups % kMaxKGL)
+    return lh::fail_arg("%s: H=%d (a multiple of 8) B=%d kgroups=%d (a multiple of %d)", what, H, B, kgroups, kMaxKGL);
   if (!bias4h || !c_prev || !mask01 || !c || !h) return lh::fail_arg("%s: a NULL operand", what);
   if (!lh::aligned16(bias4h) || !lh::aligned16(c_prev) || !lh::aligned16(c) || !lh::aligned16(h))
     return lh::fail_arg("%s: bias4h, c_prev, c and h must be 16-byte aligned", what);
@@ -514,18 +577,28 @@ extern "C" int lh_gate_gemm_split_lstm_cell_f32(int H, int B, int kgroups, const
   if (h_planes) {
     rc = check_planes(what, h_planes, "h_planes");
     if (rc != LH_OK) return rc;
-    if (hp_kgroups_total < 2 || hp_kgroups_total % 2 || hp_kg_offset < 0 || hp_kg_offset % 2 ||
-        hp_kg_offset + lh_split_kgroups(H) > hp_kgroups_total)
-      return lh::fail_arg("%s: k-groups [%d, %d) of h do not fit an operand of %d", what, hp_kg_offset,
-                          hp_kg_offset + lh_split_kgroups(H), hp_kgroups_total);
+    if (hp_kgroups < H / 8 || hp_kgroups_total % kMaxKGL || hp_kg_offset < 0 ||
+        hp_kg_offset + hp_kgroups > hp_kgroups_total)
+      return lh::fail_arg("%s: k-groups [%d, %d) of h must hold H=%d and fit an operand of %d", what, hp_kg_offset,
+                          hp_kg_offset + hp_kgroups, H, hp_kgroups_total);
     g.h_planes = reinterpret_cast<u4v *>(h_planes);
-    g.hp_KG = hp_kgroups_total, g.hp_kg0 = hp_kg_offset, g.hp_Np = round_up(B, kPadD);
+    g.hp_KG = hp_kgroups_total, g.hp_kg0 = hp_kg_offset, g.hp_kgn = hp_kgroups, g.hp_Np = round_up(B, kPadD);
   }
   const int tiles128 = (H + kGateRows - 1) / kGateRows;
-  return launch_cell_index(choose(kCell, kNumCell, kNumCell, tiles128, 4 * H, B, true), g, lh::as_stream(stream));
+  return launch_cell_index(choose(kCell, kAutoCell, kNumCell, tiles128, 4 * H, B, true), g, lh::as_stream(stream));
+}
+
+extern "C" int lh_gemm_split_kernel_name(int cell, int M, int N, char *name, int name_cap) {
+  if (!name || name_cap < 1 || M < 1 || N < 1) return lh::fail_arg("lh_gemm_split_kernel_name: M=%d N=%d", M, N);
+  const SplitConfig &k = cell ? kCell[choose(kCell, kAutoCell, kNumCell, (M + kGateRows - 1) / kGateRows, 4 * M, N, true)]
+                              : kPlain[choose(kPlain, kAutoPlain, kNumPlain, 0, M, N, false)];
+  snprintf(name, name_cap, "gemm_split_kernel<%d, %d, %d, %d, %d, %s>", k.bm, k.bn, k.wm, k.wn, k.wk,
+           cell ? "true" : "false");
+  return LH_OK;
 }
 
 extern "C" int lh_gemm_split_set_config_override(int config) {
   g_split_override = config < 0 ? -1 : config;
-  return kNumPlain;
+  return kNumPlain;  // == kNumCell
 }
+static_assert(kNumPlain == kNumCell, "one override index space");

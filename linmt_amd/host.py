@@ -111,6 +111,7 @@ def load():
                                         C.c_int, C.POINTER(C.c_int)]
     lib.lnmt_model_stream.restype = C.c_void_p
     lib.lnmt_model_stream.argtypes = [C.c_void_p]
+    lib.lnmt_set_split_products.argtypes = [C.c_void_p, C.c_int, C.c_int]
     lib.lnmt_profile_set_level.argtypes = [C.c_void_p, C.c_int]
     lib.lnmt_profile_count.argtypes = [C.c_void_p]
     lib.lnmt_profile_entry.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.c_int,
@@ -210,6 +211,11 @@ class Model:
     @property
     def stream(self):
         return load().lnmt_model_stream(self.handle)
+
+    def set_split_products(self, on=True, min_columns=0):
+        """Decoding: gate products and output projection from three-way bf16 splits on the bf16
+        matrix pipe while at least min_columns hypotheses are alive (lnmt_set_split_products)."""
+        _check(load().lnmt_set_split_products(self.handle, int(on), int(min_columns)), "set_split_products")
 
     def profile(self, level):
         """0 off, 1 output projection only, 2 every launch (HIP events on the model's stream)."""

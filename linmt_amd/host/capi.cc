@@ -338,6 +338,15 @@ extern "C" int lnmt_profile_set_level(lnmt_model *m, int level) {
   });
 }
 
+extern "C" int lnmt_set_split_products(lnmt_model *m, int on, int min_columns) {
+  return Guard([&] {
+    if (on && m->nmt->cfg_.lstm_size_ % 8)
+      throw linmt::LinmtError("lnmt_set_split_products: the hidden size must be a multiple of 8");
+    m->nmt->split_products_ = on != 0;
+    if (min_columns > 0) m->nmt->split_min_columns_ = min_columns;
+  });
+}
+
 extern "C" int lnmt_profile_count(lnmt_model *m) { return (int)m->nmt->profiler_.totals_.size(); }
 
 extern "C" int lnmt_profile_entry(lnmt_model *m, int index, char *name, int name_cap, double *ms,

@@ -171,6 +171,13 @@ class LstmLayer {
   bool input_hoistable_ = false;  // buffers exist
   bool input_hoisted_ = false;    // this pass uses them
   bool mw_fold_dirty_ = true;
+  // Decoding with split products (NeuralMachineTranslation::split_products_): the stacked gate
+  // matrices of a target step side by side, [M | W_h] (first layer: [W_h | Q]), as packed bf16
+  // planes, and the step's packed input [h_below; h_{t-1}] ([h_{t-1}; h~_{t-1}]).
+  DeviceArray<unsigned> split_w_planes_, split_x_planes_;
+  int split_kgroups_ = 0;  // k-groups of both operands, padding included
+  bool split_dirty_ = true;
+  void BuildSplitWeights();
   void ForwardPropInputAllSteps(int steps);
   void ForwardPropInputSteps(int first, int steps);
   void BuildEmbeddingFold();
@@ -322,6 +329,12 @@ class SoftmaxLayer : public BaseLossLayer {
   int current_minibatch_ = 0;
   bool training_perplexity_mode_ = false;
   DeviceArray<float> p_device_d_, p_device_b_d_;
+  // split products: D and the step's h~ as packed bf16 planes
+  DeviceArray<unsigned> split_d_planes_, split_h_planes_;
+  int split_kgroups_ = 0;
+  bool split_dirty_ = true;
+  void BuildSplitWeights();
+  void ComputeLogitsSplit(float *p_device_h_t, int minibatch);
   DeviceArray<float> p_device_outputdist_;           // V x B logits / probabilities (one step)
   DeviceArray<double> p_device_logp_tgt_, p_device_loss_, p_device_train_perplexity_;
   DeviceArray<int> p_device_output_vocab_indices_, p_device_output_vocab_indices_01_;
@@ -441,6 +454,14 @@ class NeuralMachineTranslation {
   hipStream_t stream_ = nullptr;
   bool decode_mode_ = false;
   int beam_size_ = 0, n_sent_ = 0;
+  // Opt-in (lnmt_set_split_products, or LINMT_SPLIT_PRODUCTS=1 when the model is created): a
+  // decoding step's gate products and output projection run as products of three-way bf16 splits
+  // (lh_gemm_split_f32 / lh_gate_gemm_split_lstm_cell_f32) while at least split_min_columns_
+  // hypotheses are alive; below that, and everywhere else, the fp32 MFMA products run.
+  bool split_products_ = false;
+  int split_min_columns_ = 160;
+  bool split_step_ = false;  // the step being run uses them
+  bool SplitProductsUsable(int curr_index, int minibatch) const;
   Profiler profiler_;  // live HIP-event timing on stream_, off by default
   // Scratch of lh_gemm_ws_f32 (split-K partial sums); every product of the model runs on
   // stream_, which is the ordering that sharing it requires.

@@ -142,6 +142,7 @@ bool LstmLayer::SetParam(const std::string &name, const float *host, size_t n) {
   hipStream_t s = p_neural_mt_->stream_;
   const int H = lstm_size_;
   if (name == "W" || name[0] == 'M') mw_fold_dirty_ = true;
+  split_dirty_ = true;
   if (name == "W") return input_layer_mode_ && SetFlat(p_device_w_, host, n, s);
   if (name.size() == 3 && name[0] == 'M' && name[1] == '_') {
     const int g = GateIndex(name[2]);
@@ -210,6 +211,69 @@ void LstmNode::UpdateVectorsForwardGpu(int *p_device_input_vocab_indices_01,
   p_device_c_t_prev_ = p_device_c_t_prev;
 }
 
+// ---- decoding with split products ---------------------------------------------------------------
+// The stacked gate matrices of a target step, side by side in the order of the packed input:
+// [M | W_h] for a layer that reads the layer below, [W_h | Q] (or [W_h]) for the first layer, whose
+// input product is a column of the folded embedding table.
+void LstmLayer::BuildSplitWeights() {
+  NeuralMachineTranslation &M = *p_neural_mt_;
+  const int H = lstm_size_;
+  if (source_side_mode_ || H % 8 || (!input_layer_mode_ && input_size_ != H))
+    throw LinmtError("LstmLayer::BuildSplitWeights: a target layer with H a multiple of 8");
+  const float *mat[2] = {input_layer_mode_ ? p_device_w_h_stack_.get() : p_device_m_stack_.get(),
+                         input_layer_mode_ ? p_device_q_stack_.get() : p_device_w_h_stack_.get()};
+  const int n = input_layer_mode_ && !feed_input_mode_ ? 1 : 2;
+  const int g0 = lh_split_kgroups(H);
+  split_kgroups_ = lh_split_kgroups_padded(n * g0);
+  const size_t wn = lh_split_bytes(lh_split_gate_rows(H), split_kgroups_) / sizeof(unsigned);
+  const size_t xn = lh_split_bytes(minibatch_size_, split_kgroups_) / sizeof(unsigned);
+  if (split_w_planes_.size() != wn) split_w_planes_.Alloc(wn);
+  if (split_x_planes_.size() != xn) {
+    split_x_planes_.Alloc(xn);
+    split_x_planes_.Zero(M.stream_);
+  }
+  lh_split_source src[2];
+  for (int i = 0; i < n; ++i) {
+    src[i] = lh_split_source{};
+    src[i].src = mat[i], src[i].ld = 4 * H, src[i].k_contiguous = 0, src[i].D = 4 * H, src[i].K = H;
+    src[i].gate_H = H, src[i].planes = split_w_planes_.get(), src[i].kgroups_total = split_kgroups_;
+    src[i].kg_offset = i * g0, src[i].kgroups = i == n - 1 ? split_kgroups_ - i * g0 : g0;
+  }
+  LhErrorWrapper(lh_split_pack_f32(src, n, M.stream_), "LstmLayer::BuildSplitWeights");
+  split_dirty_ = false;
+}
+
+// ForwardProp of a target node whose step runs on split products: the packed input of the layer
+// is complete (h_{t-1}, h~_{t-1} packed at the start of the step, h of the layer below written as
+// planes by that layer's kernel); one launch does the product, the cell and the planes of h for
+// the layer above.
+static void ForwardPropSplit(LstmNode &n) {
+  LstmLayer &L = *n.p_layer_;
+  NeuralMachineTranslation &M = *L.p_neural_mt_;
+  const int H = L.lstm_size_, B = n.minibatch_size_;
+  const bool feed = L.feed_input_mode_ && 0 != n.index_;
+  const float *addend = nullptr;
+  if (L.input_layer_mode_) {
+    if (L.mw_fold_dirty_) L.BuildEmbeddingFold();
+    addend = L.mw_fold_.get();
+  }
+  LstmLayer *up = L.layer_number_ + 1 < M.cfg_.num_layers_ ? &M.TargetLayer(L.layer_number_ + 1) : nullptr;
+  const float cell_clip = M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f;
+  char name[160] = {0};
+  if (M.profiler_.Wants(kTagGateGemm))
+    LhErrorWrapper(lh_gemm_split_kernel_name(1, H, B, name, sizeof(name)), "lh_gemm_split_kernel_name");
+  const double k = (L.input_layer_mode_ ? (feed ? 2.0 : 1.0) : 2.0) * H;
+  ProfileScope ps(M.profiler_, kTagGateGemm, name, 2.0 * 4 * H * (double)B * k);
+  LhErrorWrapper(lh_gate_gemm_split_lstm_cell_f32(
+                     H, B, L.split_kgroups_, L.split_w_planes_.get(), L.split_x_planes_.get(), addend,
+                     4 * H, addend ? n.p_device_input_vocab_indices_ : nullptr, addend ? L.vocab_size_ : 0,
+                     L.p_device_b_stack_.get(), n.p_device_c_t_prev_, n.p_device_input_vocab_indices_01_,
+                     feed ? 1 : 0, cell_clip, n.p_device_c_t_, n.p_device_h_t_,
+                     up ? up->split_x_planes_.get() : nullptr, up ? up->split_kgroups_ : 0, 0,
+                     lh_split_kgroups(H), M.stream_),
+                 "LstmNode::ForwardPropGpu split gate product with cell");
+}
+
 // One cell-step: [embedding lookup] -> ONE stacked multi-segment GEMM (x, h_{t-1}[, h~_{t-1}]) ->
 // ONE fused cell kernel.  The reference runs 1 + 8..12 SGEMMs + 7 elementwise kernels on 9 streams
 // here (src/node_input_to_hidden.h:218-636).
@@ -221,6 +285,10 @@ void LstmNode::ForwardProp() {
   // feed input only from the second target step on (node_input_to_hidden.h:325)
   const bool feed = L.feed_input_mode_ && 0 != index_;
   const bool folded = M.decode_mode_ && L.input_layer_mode_ && !L.source_side_mode_;
+  if (M.split_step_ && !L.source_side_mode_) {
+    ForwardPropSplit(*this);
+    return;
+  }
   float *pre = L.preact_.get();
   lh_gemm_seg segs[3];
   int nseg = 0;
@@ -657,6 +725,43 @@ void SoftmaxLayer::ComputeLogits(float *p_device_h_t, int minibatch) {
                      output_vocab_size_, "SoftmaxLayer::GetDistributionGpu p_device_outputdist");
 }
 
+void SoftmaxLayer::BuildSplitWeights() {
+  const int H = lstm_size_, V = output_vocab_size_;
+  split_kgroups_ = lh_split_kgroups_padded(lh_split_kgroups(H));
+  const size_t dn = lh_split_bytes(V, split_kgroups_) / sizeof(unsigned);
+  const size_t hn = lh_split_bytes(minibatch_size_, split_kgroups_) / sizeof(unsigned);
+  if (split_d_planes_.size() != dn) split_d_planes_.Alloc(dn);
+  if (split_h_planes_.size() != hn) split_h_planes_.Alloc(hn);
+  lh_split_source src{};
+  src.src = p_device_d_.get(), src.ld = V, src.k_contiguous = 0, src.D = V, src.K = H;
+  src.planes = split_d_planes_.get(), src.kgroups_total = split_kgroups_, src.kgroups = split_kgroups_;
+  LhErrorWrapper(lh_split_pack_f32(&src, 1, p_neural_mt_->stream_), "SoftmaxLayer::BuildSplitWeights");
+  split_dirty_ = false;
+}
+
+// ComputeLogits on split products: h~ is packed (one small launch), D was packed when it was set.
+void SoftmaxLayer::ComputeLogitsSplit(float *p_device_h_t, int minibatch) {
+  NeuralMachineTranslation &M = *p_neural_mt_;
+  const int H = lstm_size_, V = output_vocab_size_;
+  if (split_dirty_) BuildSplitWeights();
+  if (minibatch > minibatch_size_) throw LinmtError("SoftmaxLayer::ComputeLogitsSplit: more columns than allocated");
+  {
+    lh_split_source src{};
+    src.src = p_device_h_t, src.ld = H, src.k_contiguous = 1, src.D = minibatch, src.K = H;
+    src.planes = split_h_planes_.get(), src.kgroups_total = split_kgroups_, src.kgroups = split_kgroups_;
+    ProfileScope ps(M.profiler_, kTagSplitPack, 10.0 * H * minibatch);
+    LhErrorWrapper(lh_split_pack_f32(&src, 1, M.stream_), "SoftmaxLayer::ComputeLogitsSplit packing h");
+  }
+  char name[160] = {0};
+  if (M.profiler_.Wants(kTagLogitsGemm))
+    LhErrorWrapper(lh_gemm_split_kernel_name(0, V, minibatch, name, sizeof(name)), "lh_gemm_split_kernel_name");
+  ProfileScope ps(M.profiler_, kTagLogitsGemm, name, 2.0 * V * (double)minibatch * H);
+  LhErrorWrapper(lh_gemm_split_f32(V, minibatch, split_kgroups_, split_d_planes_.get(), split_h_planes_.get(),
+                                   1.f, 0.f, p_device_b_d_.get(), LH_ACT_NONE, 0, nullptr,
+                                   p_device_outputdist_.get(), V, M.stream_),
+                 "SoftmaxLayer::GetDistributionGpu p_device_outputdist (split products)");
+}
+
 void SoftmaxLayer::GetDistributionGpu(float *p_device_h_t) {
   hipStream_t s = p_neural_mt_->stream_;
   const int V = output_vocab_size_, B = current_minibatch_;
@@ -706,7 +811,10 @@ double SoftmaxLayer::GetTrainPerplexity() {
 
 bool SoftmaxLayer::SetParam(const std::string &name, const float *host, size_t n) {
   hipStream_t s = p_neural_mt_->stream_;
-  if (name == "D") return SetFlat(p_device_d_, host, n, s);
+  if (name == "D") {
+    split_dirty_ = true;
+    return SetFlat(p_device_d_, host, n, s);
+  }
   if (name == "b_d") return SetFlat(p_device_b_d_, host, n, s);
   return false;
 }

@@ -98,6 +98,7 @@ void NeuralMachineTranslation::InitModel() {
 // target side: ONE node, n_sent*beam columns, previous-state buffers (deep_rnn.h:697-922).
 void NeuralMachineTranslation::InitModelDecoding(int n_sent, int beam_size) {
   decode_mode_ = true;
+  if (const char *sp = std::getenv("LINMT_SPLIT_PRODUCTS")) split_products_ = sp[0] == '1';
   n_sent_ = n_sent;
   beam_size_ = beam_size;
   const int L = cfg_.num_layers_, T = cfg_.longest_sentence_, H = cfg_.lstm_size_;
@@ -422,10 +423,19 @@ void NeuralMachineTranslation::RunSourceSide(int source_length, int B) {
   }
 }
 
+bool NeuralMachineTranslation::SplitProductsUsable(int curr_index, int minibatch) const {
+  if (!split_products_ || !decode_mode_ || apply_dropout_ || cfg_.lstm_size_ % 8) return false;
+  if (minibatch < split_min_columns_) return false;
+  // the first step of a feed-input model has no h~_{t-1} segment: another operand shape, once per batch
+  if (cfg_.feed_input_mode_ && curr_index == 0) return false;
+  return true;
+}
+
 void NeuralMachineTranslation::ForwardPropTarget(int curr_index, int *p_device_current_indices,
                                                  int minibatch) {
   const int L = cfg_.num_layers_;
   input_layer_target_.v_nodes_[0].index_ = curr_index;  // deep_rnn.h:1760
+  split_step_ = SplitProductsUsable(curr_index, minibatch);
   for (int l = 0; l < L; ++l) {
     LstmLayer &Lt = TargetLayer(l);
     LstmNode &n = Lt.v_nodes_[0];
@@ -445,8 +455,41 @@ void NeuralMachineTranslation::ForwardPropTarget(int curr_index, int *p_device_c
   // same rate per flop as the layer-by-layer launches from 192 live columns up and 5-15% faster
   // below 128, which is under 1% of a batch: it stays off unless asked for.
   int first_on_chain = 0;
+  if (split_step_) {
+    // what the previous step fixes of every layer's packed input: h_{t-1} (and h~_{t-1} for the
+    // first layer), in launches of up to LH_SPLIT_PACK_MAX matrices
+    const int H = cfg_.lstm_size_, g0 = lh_split_kgroups(H);
+    lh_split_source src[LH_SPLIT_PACK_MAX];
+    int n = 0;
+    auto flush = [&]() {
+      if (!n) return;
+      ProfileScope ps(profiler_, kTagSplitPack, 10.0 * H * minibatch * n);
+      LhErrorWrapper(lh_split_pack_f32(src, n, stream_), "ForwardPropTarget packing the step's inputs");
+      n = 0;
+    };
+    auto add = [&](LstmLayer &Lt, const float *x, int kg_offset, bool last) {
+      if (n == LH_SPLIT_PACK_MAX) flush();
+      lh_split_source &q = src[n++];
+      q = lh_split_source{};
+      q.src = x, q.ld = H, q.k_contiguous = 1, q.D = minibatch, q.K = H;
+      q.planes = Lt.split_x_planes_.get(), q.kgroups_total = Lt.split_kgroups_;
+      q.kg_offset = kg_offset, q.kgroups = last ? Lt.split_kgroups_ - kg_offset : g0;
+    };
+    for (int l = 0; l < L; ++l) {
+      LstmLayer &Lt = TargetLayer(l);
+      if (Lt.split_dirty_) Lt.BuildSplitWeights();
+      LstmNode &nd = Lt.v_nodes_[0];
+      if (l == 0) {
+        add(Lt, nd.p_device_h_t_prev_, 0, !Lt.feed_input_mode_);
+        if (Lt.feed_input_mode_) add(Lt, nd.p_device_h_tild_, g0, true);
+      } else {
+        add(Lt, nd.p_device_h_t_prev_, g0, true);
+      }
+    }
+    flush();
+  }
   const char *grouped = std::getenv("LINMT_GROUPED_GATES");
-  if (decode_mode_ && !apply_dropout_ && L >= 2 && L <= LH_GATE_GROUP_MAX && grouped &&
+  if (!split_step_ && decode_mode_ && !apply_dropout_ && L >= 2 && L <= LH_GATE_GROUP_MAX && grouped &&
       grouped[0] == '1') {
     lh_gate_problem problems[LH_GATE_GROUP_MAX];
     for (int l = 0; l < L; ++l) TargetLayer(l).v_nodes_[0].DescribeRecurrentProblem(l == 0, &problems[l]);
@@ -477,7 +520,11 @@ void NeuralMachineTranslation::ForwardPropTarget(int curr_index, int *p_device_c
     top = an.p_device_final_tmp_2_;
   }
   softmax_layer_.SetHTPtr(0, top);
-  softmax_layer_.ComputeLogits(top, minibatch);
+  if (split_step_)
+    softmax_layer_.ComputeLogitsSplit(top, minibatch);
+  else
+    softmax_layer_.ComputeLogits(top, minibatch);
+  split_step_ = false;
 }
 
 void NeuralMachineTranslation::SwapDecodingStates(const int *p_device_backptr, int minibatch) {

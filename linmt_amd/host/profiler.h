@@ -32,6 +32,7 @@ enum ProfileTag {
   kTagRowSum,
   kTagEmbedGrad,
   kTagUpdate,
+  kTagSplitPack,  // fp32 -> three bf16 planes, for the products on the bf16 matrix pipe
   kTagCount
 };
 
@@ -41,7 +42,7 @@ inline const char *ProfileTagName(int t) {
                                          "xent", "beam_topk", "beam_merge", "beam_gather",
                                          "error_gemm", "weight_grad_gemm", "lstm_cell_bwd",
                                          "attn_bwd", "softmax_grad", "row_sum", "embed_grad",
-                                         "update"};
+                                         "update", "split_pack"};
   return t >= 0 && t < kTagCount ? names[t] : "";
 }
 

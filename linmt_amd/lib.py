@@ -37,7 +37,7 @@ class GateProblem(C.Structure):
 class SplitSource(C.Structure):
     _fields_ = [("src", C.c_void_p), ("ld", C.c_int), ("k_contiguous", C.c_int), ("D", C.c_int),
                 ("K", C.c_int), ("gate_H", C.c_int), ("planes", C.c_void_p),
-                ("kgroups_total", C.c_int), ("kg_offset", C.c_int)]
+                ("kgroups_total", C.c_int), ("kg_offset", C.c_int), ("kgroups", C.c_int)]
 
 
 # name -> (restype, argtypes); mirrors include/linmt_hip.h one to one.
@@ -83,6 +83,7 @@ SIGNATURES = {
     "lh_gemm_set_splits_override": (C.c_int, [C.c_int]),
     "lh_gemm_config_info": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int * 8)]),
     "lh_split_kgroups": (C.c_int, [C.c_int]),
+    "lh_split_kgroups_padded": (C.c_int, [C.c_int]),
     "lh_split_padded": (C.c_int, [C.c_int]),
     "lh_split_gate_rows": (C.c_int, [C.c_int]),
     "lh_split_bytes": (C.c_size_t, [C.c_int, C.c_int]),
@@ -93,7 +94,8 @@ SIGNATURES = {
     "lh_gate_gemm_split_lstm_cell_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                                    c_f32p, C.c_int, c_i32p, C.c_int, c_f32p, c_f32p,
                                                    c_i32p, C.c_int, C.c_float, c_f32p, c_f32p,
-                                                   C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+                                                   C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+    "lh_gemm_split_kernel_name": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_char_p, C.c_int]),
     "lh_gemm_split_set_config_override": (C.c_int, [C.c_int]),
     "lh_lstm_cell_fwd_f32": (C.c_int, [C.c_int, C.c_int, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p,
                                        c_i32p, C.c_int, C.c_float, c_f32p, c_f32p, c_f32p, c_f32p,
@@ -330,13 +332,18 @@ def split_kgroups(K):
     return load().lh_split_kgroups(K)
 
 
+def split_kgroups_padded(kgroups):
+    return load().lh_split_kgroups_padded(kgroups)
+
+
 def split_bytes(D, kgroups):
     return load().lh_split_bytes(D, kgroups)
 
 
 def split_pack(sources, stream=None):
-    """sources: dicts with src (tensor), ld, k_contiguous, D, K, planes (tensor), kgroups_total,
-    kg_offset and optionally gate_H (lh_split_pack_f32, up to 8 per launch)."""
+    """sources: dicts with src (tensor), ld, k_contiguous, D, K, planes (tensor), kgroups_total and
+    optionally kg_offset (0), kgroups (all from kg_offset to the operand's end when the segment is
+    alone, else ceil(K/8)) and gate_H (lh_split_pack_f32, up to 8 per launch)."""
     arr = (SplitSource * len(sources))()
     for i, q in enumerate(sources):
         arr[i].src = q["src"].data_ptr()
@@ -344,6 +351,7 @@ def split_pack(sources, stream=None):
         arr[i].D, arr[i].K, arr[i].gate_H = q["D"], q["K"], q.get("gate_H", 0)
         arr[i].planes = q["planes"].data_ptr()
         arr[i].kgroups_total, arr[i].kg_offset = q["kgroups_total"], q.get("kg_offset", 0)
+        arr[i].kgroups = q.get("kgroups", (q["K"] + 7) // 8)
     check(load().lh_split_pack_f32(arr, len(sources), _stream(stream)), "lh_split_pack_f32")
 
 
@@ -358,11 +366,11 @@ def gemm_split(M, N, kgroups, A_planes, X_planes, C_out, ldc, alpha=1.0, beta=0.
 def gate_gemm_split_lstm_cell(H, B, kgroups, W_planes, X_planes, bias4h, c_prev, mask01, c, h,
                               addend=None, ld_addend=0, addend_col=None, addend_ncols=0,
                               sigmoid_f64=False, cell_clip=0.0, h_planes=None, hp_kgroups_total=0,
-                              hp_kg_offset=0, stream=None):
+                              hp_kg_offset=0, hp_kgroups=0, stream=None):
     check(load().lh_gate_gemm_split_lstm_cell_f32(
         H, B, kgroups, _ptr(W_planes), _ptr(X_planes), _ptr(addend), ld_addend, _ptr(addend_col),
         addend_ncols, _ptr(bias4h), _ptr(c_prev), _ptr(mask01), int(sigmoid_f64), cell_clip, _ptr(c),
-        _ptr(h), _ptr(h_planes), hp_kgroups_total, hp_kg_offset, _stream(stream)),
+        _ptr(h), _ptr(h_planes), hp_kgroups_total, hp_kg_offset, hp_kgroups, _stream(stream)),
         "lh_gate_gemm_split_lstm_cell_f32")
 
 

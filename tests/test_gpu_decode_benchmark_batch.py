@@ -34,23 +34,37 @@ def host():
     return h
 
 
-def test_benchmark_batch_beams_vs_oracle_trace(orc, host):
+@pytest.fixture(scope="module")
+def workload(orc):
+    """The benchmark's model and sentences, and the oracle's traced search of every sentence."""
     layers, H, V, D, beam, n_sent, longest = 4, 1000, 30000, 10, 12, 64, 104
     rng = np.random.default_rng(bench.SEED)
     P = bench.make_params(rng, layers, H, V, V)
     sents = bench.make_sentences(rng, n_sent, V)
+    om = orc.Model(layers, H, V, V, attention=1, D=D, feed_input=1, longest_sent=longest)
+    om.set_params(P)
+    traces = [om.decode_sentence_trace(s, beam=beam) for s in sents]
+    return dict(cfg=(layers, H, V, D, beam, n_sent, longest), P=P, sents=sents, traces=traces)
+
+
+@pytest.mark.parametrize("split", [False, True], ids=["fp32_mfma", "split_bf16_products"])
+def test_benchmark_batch_beams_vs_oracle_trace(workload, host, split):
+    """split: the same demand on the opt-in arithmetic (lnmt_set_split_products), whose products
+    are as close to float64 as the fp32 MFMA ones."""
+    layers, H, V, D, beam, n_sent, longest = workload["cfg"]
+    P, sents = workload["P"], workload["sents"]
     gm = host.Model(layers, H, V, V, longest_sentence=longest, attention_mode=1, attention_width=D,
                     feed_input=True, decoding=(n_sent, beam))
     gm.set_params(P)
+    if split:
+        gm.set_split_products(True)
     res = gm.decode_batch(sents, beam=beam)
     hist = [gm.decode_history(i, beam) for i in range(n_sent)]
     gm.close()
-    om = orc.Model(layers, H, V, V, attention=1, D=D, feed_input=1, longest_sent=longest)
-    om.set_params(P)
     classes = {"identical": 0, "diverged_at_near_tie": 0, "diverged_other": 0}
     notes, steps_equal, steps_total, same_best, worst_dev = [], 0, 0, 0, 0.0
     for i, s in enumerate(sents):
-        tr = om.decode_sentence_trace(s, beam=beam)
+        tr = workload["traces"][i]
         assert hist[i][0].shape == tr["tok"].shape, f"sentence {i}: number of expansion steps"
         cls, at, eps_at = bench.classify_beam_parity(res[i]["best"], hist[i][0], hist[i][1], hist[i][2], tr)
         classes[cls] += 1
@@ -68,7 +82,7 @@ def test_benchmark_batch_beams_vs_oracle_trace(orc, host):
         if cls != "identical":
             notes.append(f"sentence {i} (len {len(s)}): {cls} at step {at}, oracle margin "
                          f"{tr['margin'][at]:.3e}, epsilon {eps_at:.3e}")
-    print(f"beam parity on the benchmark batch: {classes}; {steps_equal} of {steps_total} expansion "
+    print(f"beam parity on the benchmark batch ({'split bf16' if split else 'fp32 MFMA'} products): {classes}; {steps_equal} of {steps_total} expansion "
           f"steps identical before any divergence; largest |GPU - oracle| path score on identical "
           f"beams {worst_dev:.2e}; 1-best identical for {same_best} of {n_sent}", flush=True)
     for line in notes:

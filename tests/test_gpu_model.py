@@ -259,6 +259,39 @@ def test_decode_same_with_grouped_gate_products(orc, host, monkeypatch):
     gm.close()
 
 
+@pytest.mark.parametrize("layers,H,attention,feed,seed", [(4, 96, 1, True, 18), (1, 64, 0, False, 19),
+                                                          (2, 72, 2, True, 20)])
+def test_decode_same_with_split_products(orc, host, layers, H, attention, feed, seed):
+    """lnmt_set_split_products: the gate products and the output projection of a decoding step as
+    six exact bf16 products per term on the bf16 matrix pipe (every step here: min_columns = 1;
+    the first step of a feed-input model keeps the fp32 MFMA product).  As close to float64 as the
+    fp32 products: same translations, scores inside the floating-point tolerance, both equal to
+    the oracle's.  One to four layers, with and without attention / feed input, a ragged batch
+    whose live column count changes between steps."""
+    rng = np.random.default_rng(seed)
+    Vs, Vt, D, beam = 200, 260, 4, 6
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 40, 0.35, decoding=(5, beam),
+                      attention=attention, feed=feed)
+    sents = [rng.integers(0, Vs, size=n) for n in (17, 9, 12, 3, 21)]
+    plain = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    gm.set_split_products(True, 1)
+    gm.profile(2)
+    split = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    keys = list(gm.profile_totals())
+    assert any(k.startswith("gate_gemm|gemm_split_kernel") for k in keys), "the split gate product did not run"
+    assert any(k.startswith("logits_gemm|gemm_split_kernel") for k in keys), "the split output projection did not run"
+    gm.profile(0)
+    gm.set_split_products(False)
+    again = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    for i, (a, b, c) in enumerate(zip(split, plain, again)):
+        assert a["best"].tolist() == b["best"].tolist(), i
+        assert np.isclose(a["best_score"], b["best_score"], rtol=1e-4, atol=1e-5), i
+        assert a["n_hyp"] == b["n_hyp"], i
+        _compare_decode(om.decode_sentence(sents[i], beam=beam), a, f"split products, sentence {i}")
+        assert c["best"].tolist() == b["best"].tolist() and c["best_score"] == b["best_score"], i
+    gm.close()
+
+
 def test_decode_random_architectures_vs_oracle(orc, host):
     """A seeded sweep over architectures and batch shapes the fixed cases do not hit: 1-4 layers,
     hidden sizes that land on different tile configurations (and on the one- and two-quad attention

@@ -34,20 +34,21 @@ def test_packing_is_exact_and_zero_padded(lh):
     a = uni(rng, D, K)
     a[0, :8] = [0.0, -0.0, 1.0, -1.0, 1e38, -1e-30, 1.0 + 2.0 ** -23, 0.1]
     kg = lh.split_kgroups(K)
-    assert kg == 10 and lh.load().lh_split_padded(D) == 512
+    total = lh.split_kgroups_padded(kg + 4)
+    assert kg == 9 and total == 16 and lh.load().lh_split_padded(D) == 512
     for k_contig in (True, False):
         src = a if k_contig else a.T                      # (D, K) row-major or (K, D) row-major
         t = torch.from_numpy(np.ascontiguousarray(src)).cuda()
-        p = planes_tensor(lh, D, kg + 4)
-        p2 = planes_tensor(lh, D, kg + 4)
+        p = planes_tensor(lh, D, total)
+        p2 = planes_tensor(lh, D, total)
         lh.split_pack([dict(src=t, ld=K if k_contig else D, k_contiguous=k_contig, D=D, K=K, planes=p,
-                            kgroups_total=kg + 4, kg_offset=2),
+                            kgroups_total=total, kg_offset=2),
                        dict(src=t, ld=K if k_contig else D, k_contiguous=k_contig, D=D, K=K, planes=p2,
-                            kgroups_total=kg + 4, kg_offset=4)])
-        for planes, off in ((p, 2), (p2, 4)):
-            f = unpack(planes, 512, kg + 4)[:, off * 8:(off + kg) * 8]
-            total = f[0] + f[1] + f[2]
-            assert np.array_equal(total[:K, :D], a.T.astype(np.float64)), "a1 + a2 + a3 != a"
+                            kgroups_total=total, kg_offset=4, kgroups=total - 4)])
+        for planes, off, n in ((p, 2, kg), (p2, 4, total - 4)):
+            f = unpack(planes, 512, total)[:, off * 8:(off + n) * 8]
+            both = f[0] + f[1] + f[2]
+            assert np.array_equal(both[:K, :D], a.T.astype(np.float64)), "a1 + a2 + a3 != a"
             assert np.all(f[:, K:, :] == 0) and np.all(f[:, :, D:] == 0), "padding is not zero"
             assert np.all(np.abs(f[1, :K, :D]) <= np.abs(f[0, :K, :D]) * 2.0 ** -8 + 1e-45)
 
@@ -62,10 +63,10 @@ def test_split_product_against_float64(lh, M, N, K):
     want = A.astype(np.float64) @ X + b[:, None]
     mag = np.abs(A).astype(np.float64) @ np.abs(X) + np.abs(b)[:, None]
     Ad, Xd, bd = dev(A), dev(X), dev(b)   # column-major: A m-contiguous, X k-contiguous
-    kg = lh.split_kgroups(K)
+    kg = lh.split_kgroups_padded(lh.split_kgroups(K))
     Ap, Xp = planes_tensor(lh, M, kg), planes_tensor(lh, N, kg)
-    lh.split_pack([dict(src=Ad, ld=M, k_contiguous=False, D=M, K=K, planes=Ap, kgroups_total=kg)])
-    lh.split_pack([dict(src=Xd, ld=K, k_contiguous=True, D=N, K=K, planes=Xp, kgroups_total=kg)])
+    lh.split_pack([dict(src=Ad, ld=M, k_contiguous=False, D=M, K=K, planes=Ap, kgroups_total=kg, kgroups=kg)])
+    lh.split_pack([dict(src=Xd, ld=K, k_contiguous=True, D=N, K=K, planes=Xp, kgroups_total=kg, kgroups=kg)])
     ref = torch.empty(M * N, device="cuda")
     lh.gemm(M, N, [(Ad, M, Xd, K, K)], ref, M, bias=bd)
     ref_err = float((np.abs(host(ref, (M, N)) - want) / mag).max())
@@ -93,11 +94,11 @@ def test_split_product_against_float64(lh, M, N, K):
 
 
 def test_split_arguments_are_checked(lh):
-    kg = lh.split_kgroups(64)
+    kg = lh.split_kgroups_padded(lh.split_kgroups(64))
     P = planes_tensor(lh, 64, kg)
     out = torch.empty(64 * 64, device="cuda")
     with pytest.raises(lh.LinmtHipError):
-        lh.gemm_split(64, 64, kg + 1, P, P, out, 64)          # odd k-group count
+        lh.gemm_split(64, 64, kg + 1, P, P, out, 64)          # not whole slabs
     with pytest.raises(lh.LinmtHipError):
         lh.gemm_split(64, 64, kg, P, P, out, 32)              # ldc < M
     with pytest.raises(lh.LinmtHipError):
@@ -127,7 +128,8 @@ def test_split_gate_product_with_cell(lh, orc, H, B, Ks, addend, f64, clip):
     bias, c_prev = uni(rng, 4 * H, s=0.5), uni(rng, H, B)
     mask = (rng.uniform(size=B) < 0.8).astype(np.int32)
     kgs = [lh.split_kgroups(K) for K in Ks]
-    KG = sum(kgs)
+    KG = lh.split_kgroups_padded(sum(kgs))
+    kgs[-1] = KG - sum(kgs[:-1])                              # the last segment carries the padding
     Wp = planes_tensor(lh, L.lh_split_gate_rows(H), KG)
     Xp = planes_tensor(lh, B, KG)
     off = 0
@@ -136,9 +138,9 @@ def test_split_gate_product_with_cell(lh, orc, H, B, Ks, addend, f64, clip):
         a_d, x_d = dev(A), dev(X)
         keep += [a_d, x_d]
         lh.split_pack([dict(src=a_d, ld=4 * H, k_contiguous=False, D=4 * H, K=K, gate_H=H, planes=Wp,
-                            kgroups_total=KG, kg_offset=off),
+                            kgroups_total=KG, kg_offset=off, kgroups=kg),
                        dict(src=x_d, ld=K, k_contiguous=True, D=B, K=K, planes=Xp, kgroups_total=KG,
-                            kg_offset=off)])
+                            kg_offset=off, kgroups=kg)])
         off += kg
     table = cols = add_np = None
     ld, V = 4 * H, 0
@@ -157,29 +159,29 @@ def test_split_gate_product_with_cell(lh, orc, H, B, Ks, addend, f64, clip):
     if add_np is not None:
         pre = pre + add_np
     _, wc, wh = orc.lstm_cell_fwd(pre.astype(np.float32), bias, c_prev, mask, feed=f64, cell_clip=clip)
-    hkg = lh.split_kgroups(H)
-    n_cfg = 3
+    hkg = lh.split_kgroups_padded(H // 8 + 2)
+    n_cfg = L.lh_gemm_split_set_config_override(-1)
     try:
         for cfg in range(-1, n_cfg):
             L.lh_gemm_split_set_config_override(cfg)
             what = f"config {cfg} H={H} B={B} K={Ks} addend={addend}"
             c = dev(c_prev)                                  # in place
             h = torch.full((H * B,), float("nan"), device="cuda")
-            hp = planes_tensor(lh, B, hkg + 2)               # stale values everywhere
+            hp = planes_tensor(lh, B, hkg)                   # stale values everywhere
             lh.gate_gemm_split_lstm_cell(H, B, KG, Wp, Xp, dev(bias), c, dev(mask), c, h, addend=table,
                                          ld_addend=ld if table is not None else 0, addend_col=cols,
                                          addend_ncols=V, sigmoid_f64=f64, cell_clip=clip, h_planes=hp,
-                                         hp_kgroups_total=hkg + 2, hp_kg_offset=2)
+                                         hp_kgroups_total=hkg, hp_kg_offset=2, hp_kgroups=hkg - 2)
             assert_close(host(c, (H, B)), wc, what + " c")
             assert_close(host(h, (H, B)), wh, what + " h")
             assert np.all(host(h, (H, B))[:, mask == 0] == 0), what
             # h's planes: exactly what packing h gives, in the k-groups asked for
-            hp2 = planes_tensor(lh, B, hkg + 2)
+            hp2 = planes_tensor(lh, B, hkg)
             lh.split_pack([dict(src=h, ld=H, k_contiguous=True, D=B, K=H, planes=hp2,
-                                kgroups_total=hkg + 2, kg_offset=2)])
+                                kgroups_total=hkg, kg_offset=2, kgroups=hkg - 2)])
             Bp = L.lh_split_padded(B)
-            got = unpack(hp, Bp, hkg + 2)[:, 16:, :B]
-            exp = unpack(hp2, Bp, hkg + 2)[:, 16:, :B]
+            got = unpack(hp, Bp, hkg)[:, 16:, :B]
+            exp = unpack(hp2, Bp, hkg)[:, 16:, :B]
             assert np.array_equal(got, exp), what + ": planes of h"
     finally:
         L.lh_gemm_split_set_config_override(-1)
