@@ -27,6 +27,7 @@ sys.path.insert(0, ROOT)
 SEED = 20161030
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_FP32_PEAK_TFLOPS = 157.3
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 MFMA, MI355X
 # HBM-side bytes per launch of the dominant kernel (fetched + written beyond L2), measured with
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over this script (KiB per dispatch at the
 # grid of 768 live columns; FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a device copy of
@@ -375,6 +376,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hbm-kernels", action="store_true",
                     help="skip the stand-alone timing of the HBM-bound kernels (hbm_kernels field)")
+    ap.add_argument("--no-split-products", action="store_true",
+                    help="skip the second timing of the same batch with the opt-in arithmetic "
+                         "(lnmt_set_split_products; reported beside `value`, never as it)")
     ap.add_argument("--profile-level", type=int, default=1,
                     help="1: HIP events around the output projection (the dominant kernel) during "
                          "the timed steps; "
@@ -473,6 +477,45 @@ def main():
                                                    else (HBM_PEAK_GBS * 1e9)), 4)}
         model.profile(0)
 
+    # The same batch with the opt-in arithmetic: gate products and output projection from three-way
+    # bf16 splits of their fp32 operands (six exact products per term, fp32 accumulation).  Reported
+    # beside `value`; `value` stays the fp32 MFMA path.
+    split, split_res, split_hist = None, None, None
+    if not args.no_split_products:
+        model.set_split_products(True)
+        model.decode_batch(sents, beam=beam)  # packs the weights
+        model.profile(1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        stok = 0
+        for _ in range(args.steps):
+            split_res = model.decode_batch(sents, beam=beam)
+            stok += sum(len(r["best"]) for r in split_res)
+        torch.cuda.synchronize()
+        sdt = time.perf_counter() - t0
+        split_hist = [model.decode_history(i, beam) for i in range(n_sent)]
+        sk = {k: t for k, t in model.profile_totals().items() if k.startswith("logits_gemm|gemm_split_kernel")}
+        model.profile(0)
+        model.set_split_products(False)
+        split = {"value": round(stok / sdt, 1), "unit": "target tokens/s",
+                 "ms_per_step": round(sdt * 1e3 / args.steps, 2),
+                 "speedup_over_value": round(stok / sdt / value, 3),
+                 "arithmetic": "fp32 operands held as three bf16 terms; every product = six exact "
+                               "bf16 x bf16 products (v_mfma_f32_32x32x16_bf16) added in fp32; what "
+                               "is left out is below 2^-23 per product; used for the gate products "
+                               "and the output projection of steps with >= 160 live hypotheses",
+                 "one_best_same_as_fp32_path": int(sum(a["best"].tolist() == b["best"].tolist()
+                                                       for a, b in zip(res, split_res)))}
+        if sk:
+            kern, t = max(sk.items(), key=lambda kv: kv[1]["work"])
+            alg = t["work"] / (t["ms"] * 1e-3) / 1e12
+            split["roofline"] = {"kernel": kern.split("|", 1)[1], "call_sites": ["logits_gemm"], "bound": "mfma",
+                                 "algorithmic_TFLOP/s": round(alg, 2),
+                                 "achieved": round(6 * alg, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                                 "unit": "TFLOP/s (bf16 products issued = 6 x algorithmic)",
+                                 "frac": round(6 * alg / MFMA_BF16_PEAK_TFLOPS, 4), "launches": t["launches"],
+                                 "avg_launch_us": round(t["ms"] * 1e3 / t["launches"], 2)}
+
     # the metric's second half: the fused HBM-bound kernels alone (outside the timed region), each
     # at the size one decode step gives it (768 columns) and at a size that saturates HBM, next to
     # a plain device copy, the practical ceiling of this GPU
@@ -498,7 +541,8 @@ def main():
         om.decode_sentence(sents[by_len[0]][:3], beam=beam, num_threads=cores)  # warm-up
         cpu_tokens, cdt = 0, 0.0
         classes = {"identical": 0, "diverged_at_near_tie": 0, "diverged_other": 0}
-        same, detail = 0, []
+        sclasses = {"identical": 0, "diverged_at_near_tie": 0, "diverged_other": 0}
+        same, ssame, detail = 0, 0, []
         for i in pick:
             c0 = time.perf_counter()
             tr = om.decode_sentence_trace(sents[i], beam=beam, num_threads=cores)
@@ -508,6 +552,10 @@ def main():
             cls, at, eps = classify_beam_parity(res[i]["best"], gtok, gbp, gsc, tr)
             classes[cls] += 1
             same += int(tr["best"].tolist() == res[i]["best"].tolist())
+            if split is not None:
+                stok_h, sbp_h, ssc_h = split_hist[int(i)]
+                sclasses[classify_beam_parity(split_res[i]["best"], stok_h, sbp_h, ssc_h, tr)[0]] += 1
+                ssame += int(tr["best"].tolist() == split_res[i]["best"].tolist())
             if tr["best"].tolist() != res[i]["best"].tolist() or cls == "diverged_other":
                 detail.append({"sentence": int(i), "source_len": int(len(sents[i])), "class": cls,
                                "first_differing_step": int(at),
@@ -525,6 +573,9 @@ def main():
                                    "|GPU - oracle| path score measured on the (identical) beams "
                                    "before it + 8 ulp of the score",
                   "one_best_differs_or_unexplained": detail}
+        if split is not None:
+            split["parity"] = {"sentences_checked": int(len(pick)), "one_best_identical": int(ssame),
+                               "beam_steps": sclasses, "parity_ok": sclasses["diverged_other"] == 0}
 
     out = {
         "metric": "target tokens/sec (beam-12 decode, 1 GPU)",
@@ -549,11 +600,17 @@ def main():
         "hbm_kernels": hbm_kernels,
         "cpu_baseline": cpu_baseline,
     }
+    if split:
+        out["split_products"] = split
     if kernels:
         out["kernels"] = kernels
     if parity:
         out["parity"] = parity
     print(json.dumps(out))
+    if split and "parity" in split and not split["parity"]["parity_ok"]:
+        print("bench.py: with split products the GPU search differs from the oracle's where no "
+              "near-tie explains it", file=sys.stderr)
+        sys.exit(1)
     if parity and not parity["parity_ok"]:
         print("bench.py: the GPU search differs from the oracle's where no near-tie explains it",
               file=sys.stderr)
