@@ -235,10 +235,10 @@ int lh_gemm_config_info(int config, int transA, int transX, int info[8]);
  * Operands are packed ahead of the product ("split planes", opaque to the caller):
  *   - lh_split_kgroups(K): k-groups (8 k each) a K-deep segment needs, ceil(K / 8);
  *   - lh_split_kgroups_padded(kgroups): the k-groups of a whole operand, the sum over its segments
- *     rounded up to whole slabs (a multiple of 8); the groups of padding must hold zeros;
+ *     rounded up to whole slabs (a multiple of 16); the groups of padding must hold zeros;
  *   - lh_split_bytes(D, kgroups): bytes of a packed operand with D rows (A) or columns (X);
- *   - lh_split_gate_rows(H): the D to size a packed stacked gate matrix with (rows are padded to
- *     whole cell tiles of 32 rows per gate);
+ *   - lh_split_gate_rows(H): the D to size a packed stacked gate matrix with (its rows are stored
+ *     eight of gate i, eight of f, eight of c', eight of o, and so on);
  *   - lh_split_pack_f32 packs up to LH_SPLIT_PACK_MAX segments in one launch.  A segment is a D x K
  *     fp32 matrix (k_contiguous: element (d, k) at src[d * ld + k], the layout of an H x B
  *     activation used as X; otherwise src[k * ld + d], the layout of a stored weight matrix used

@@ -157,7 +157,7 @@ void *lnmt_model_stream(lnmt_model *m);
 
 /* Opt-in arithmetic of a decoding model's largest matrix products (no counterpart in the
  * reference, whose products are cuBLAS SGEMM calls).  on != 0: while at least min_columns
- * hypotheses are alive (min_columns <= 0 keeps the current value, 160 at first), a step's stacked
+ * hypotheses are alive (min_columns <= 0 keeps the current value, 84 at first), a step's stacked
  * gate products and its output projection are formed from three-way bf16 splits of their fp32
  * operands on the bf16 matrix pipe (lh_gemm_split_f32, lh_gate_gemm_split_lstm_cell_f32 in
  * linmt_hip.h): every fp32 product a*x becomes six exact bf16 products added in fp32, which leaves

@@ -24,7 +24,7 @@ typedef unsigned u4v __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kPadD = 256;       // rows / columns of a packed operand are padded to this
-constexpr int kGateRows = 32;    // rows of each gate in a 128-row tile of a packed gate matrix
+constexpr int kGateRows = 8;     // a packed gate matrix holds 8 rows of gate i, 8 of f, 8 of c', 8 of o, and so on
 constexpr int kCUs = 256;
 
 inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void split_pack_kernel(const PackArgs a) {
   int d = dp;
   bool have = dp < q.D;
   if (q.H > 0) {
-    // packed row t*128 + g*32 + r  <-  row g*H + t*32 + r of the stacked matrix
+    // packed row t*32 + g*8 + r  <-  row g*H + t*8 + r of the stacked matrix
     const int t = dp / (4 * kGateRows), g = (dp / kGateRows) % 4, r = t * kGateRows + dp % kGateRows;
     have = r < q.H;
     d = g * q.H + r;
@@ -137,17 +137,24 @@ constexpr int split_lds_bytes(bool cell) {
   return stages > tile ? stages : tile;
 }
 
+// Waves per SIMD the register allocation must allow: three workgroups of the plain 128x128 tile
+// per CU (its natural allocation sits at that step; a few registers more would halve the occupancy).
+template <int BM, int BN, int WK, bool CELL>
+constexpr int split_waves_per_simd() {
+  return BM == 128 && BN == 128 && WK == 1 && !CELL ? 3 : 1;
+}
+
 template <int BM, int BN, int WM, int WN, int WK, bool CELL>
-__global__ __launch_bounds__(64 * WM * WN * WK) void gemm_split_kernel(const SplitArgs g) {
+__global__ __launch_bounds__(64 * WM * WN * WK)
+__attribute__((amdgpu_waves_per_eu(split_waves_per_simd<BM, BN, WK, CELL>()))) void gemm_split_kernel(const SplitArgs g) {
   constexpr int NT = 64 * WM * WN * WK, TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
   static_assert(FM >= 1 && FN >= 1 && TM % 32 == 0 && TN % 32 == 0, "wave tile = 32x32 MFMA tiles");
   constexpr int KGL = 2 * WK;                         // k-groups of a slab
   constexpr int UA = 3 * KGL * BM, UX = 3 * KGL * BN;  // 16-byte units of a slab: planes x k-groups x rows
-  static_assert(UA % NT == 0, "A units per thread");
-  constexpr int NUA = UA / NT, NUX = (UX + NT - 1) / NT;
-  constexpr bool kExactX = UX % NT == 0;
+  constexpr int NUA = (UA + NT - 1) / NT, NUX = (UX + NT - 1) / NT;
+  constexpr bool kExactA = UA % NT == 0, kExactX = UX % NT == 0;
   constexpr int STAGE = UA + UX;
-  static_assert(!CELL || BM == 4 * kGateRows, "a cell tile holds 32 rows of each gate");
+  static_assert(!CELL || BM % (4 * kGateRows) == 0, "a cell tile holds whole groups of 8 rows per gate");
   extern __shared__ u4v lds[];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int wk = wave / (WM * WN), wmn = wave % (WM * WN), wm = wmn % WM, wn = wmn / WM;
@@ -168,7 +175,7 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_split_kernel(const Spl
   unsigned oa[NUA], ox[NUX];
 #pragma unroll
   for (int i = 0; i < NUA; ++i) {
-    const int u = tid + i * NT, p = u / (KGL * BM), kgl = (u / BM) % KGL, r = u % BM;
+    const int u = (tid + i * NT) % UA, p = u / (KGL * BM), kgl = (u / BM) % KGL, r = u % BM;
     oa[i] = (unsigned)((p * g.KG + kgl) * g.Mp + r) * 16u;
   }
 #pragma unroll
@@ -192,7 +199,8 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_split_kernel(const Spl
     const unsigned s = min(sn, slabs - 1);  // past the end: a harmless re-read of the last slab
     const unsigned sa = s * step_a, sx = s * step_x;
 #pragma unroll
-    for (int i = 0; i < NUA; ++i) qa[i] = __builtin_amdgcn_raw_buffer_load_b128(res_a, oa[i], sa, 0);
+    for (int i = 0; i < NUA; ++i)
+      if (kExactA || tid + i * NT < UA) qa[i] = __builtin_amdgcn_raw_buffer_load_b128(res_a, oa[i], sa, 0);
 #pragma unroll
     for (int i = 0; i < NUX; ++i)
       if (kExactX || tid + i * NT < UX) qx[i] = __builtin_amdgcn_raw_buffer_load_b128(res_x, ox[i], sx, 0);
@@ -200,7 +208,8 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_split_kernel(const Spl
   auto stores = [&](int stage, const u4v (&qa)[NUA], const u4v (&qx)[NUX]) {
     u4v *w = lds + stage * STAGE;
 #pragma unroll
-    for (int i = 0; i < NUA; ++i) w[tid + i * NT] = qa[i];
+    for (int i = 0; i < NUA; ++i)
+      if (kExactA || tid + i * NT < UA) w[tid + i * NT] = qa[i];
 #pragma unroll
     for (int i = 0; i < NUX; ++i)
       if (kExactX || tid + i * NT < UX) w[UA + tid + i * NT] = qx[i];
@@ -291,15 +300,16 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_split_kernel(const Spl
       __syncthreads();
     }
     const int H = g.M;
-    constexpr int kUnits = (kGateRows / 8) * BN;
+    constexpr int kGroups = BM / (4 * kGateRows);  // groups of 8 gate rows in the tile
+    constexpr int kUnits = kGroups * BN;
     for (int idx = tid; idx < kUnits; idx += NT) {
-      const int rq = idx % (kGateRows / 8), nl = idx / (kGateRows / 8);
+      const int rq = idx % kGroups, nl = idx / kGroups;
       const int r = (m0 / 4) + rq * 8, n = n0 + nl;   // first of 8 rows of every gate
       if (r >= H || n >= g.N) continue;               // H % 8 == 0: a unit is whole or absent
       float pre[4][8];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const floatx4 *sp = reinterpret_cast<const floatx4 *>(S + nl * LDS_M + q * kGateRows + rq * 8);
+        const floatx4 *sp = reinterpret_cast<const floatx4 *>(S + nl * LDS_M + rq * 4 * kGateRows + q * kGateRows);
         const floatx4 *bp = reinterpret_cast<const floatx4 *>(g.bias + (size_t)q * H + r);
         const floatx4 s0 = sp[0], s1 = sp[1], b0 = bp[0], b1 = bp[1];
         float v[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
@@ -383,17 +393,15 @@ __global__ __launch_bounds__(64 * WM * WN * WK) void gemm_split_kernel(const Spl
 struct SplitConfig {
   int bm, bn, wm, wn, wk;
 };
-// plain products; the built-in choice walks the first kAutoPlain in order
-constexpr SplitConfig kPlain[] = {{128, 128, 2, 2, 1}, {128, 64, 2, 2, 1}, {128, 64, 2, 2, 2},
-                                  {128, 32, 4, 1, 2}, {256, 128, 4, 2, 1}, {128, 32, 4, 1, 1}};
+// plain products (the last entry is reachable by override only)
+constexpr SplitConfig kPlain[] = {{128, 128, 2, 2, 1}, {128, 64, 2, 2, 1}, {128, 96, 4, 1, 2}, {128, 64, 2, 2, 2},
+                                  {64, 96, 2, 1, 4},   {64, 64, 2, 1, 4},  {64, 32, 2, 1, 4},  {256, 128, 4, 2, 1}};
 constexpr int kNumPlain = sizeof(kPlain) / sizeof(kPlain[0]);
-constexpr int kAutoPlain = 4;
-// cell products (128 rows = 32 of each gate)
-constexpr SplitConfig kCell[] = {{128, 128, 2, 2, 1}, {128, 96, 4, 1, 2}, {128, 64, 2, 2, 2},
-                                 {128, 32, 4, 1, 2}, {128, 64, 2, 2, 1}, {128, 32, 4, 1, 4}};
+// cell products (a tile of BM rows holds BM/4 rows of each gate)
+constexpr SplitConfig kCell[] = {{128, 96, 4, 1, 2}, {128, 64, 2, 2, 2}, {128, 32, 4, 1, 2}, {64, 96, 2, 1, 4},
+                                 {64, 64, 2, 1, 4},  {64, 64, 2, 2, 2},  {64, 32, 2, 1, 4},  {32, 32, 1, 1, 8}};
 constexpr int kNumCell = sizeof(kCell) / sizeof(kCell[0]);
-constexpr int kAutoCell = 4;
-constexpr int kMaxKGL = 8;  // k-groups of the deepest slab: operands are padded to a multiple of it
+constexpr int kMaxKGL = 16;  // k-groups of the deepest slab: operands are padded to a multiple of it
 
 thread_local int g_split_override = -1;
 
@@ -401,7 +409,7 @@ template <int BM, int BN, int WM, int WN, int WK, bool CELL>
 int launch_split(SplitArgs &g, hipStream_t s, const char *what) {
   static_assert(split_lds_bytes<BM, BN, WK>(CELL) <= 160 * 1024, "LDS capacity of a CU");
   static_assert(64 * WM * WN * WK <= 1024, "workgroup size");
-  const int tiles_m = CELL ? (g.M + kGateRows - 1) / kGateRows : (g.M + BM - 1) / BM;
+  const int tiles_m = CELL ? (4 * g.M + BM - 1) / BM : (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   // The kernel reads whole tiles and whole slabs.  Rows of A are padded to whole tiles; a tile of X
   // may reach past the padded columns (BN = 96): what it reads there belongs to other k-groups or,
@@ -429,40 +437,49 @@ int launch_plain_index(int c, SplitArgs &g, hipStream_t s) {
   switch (c) {
     case 0: return launch_split<128, 128, 2, 2, 1, false>(g, s, w);
     case 1: return launch_split<128, 64, 2, 2, 1, false>(g, s, w);
-    case 2: return launch_split<128, 64, 2, 2, 2, false>(g, s, w);
-    case 3: return launch_split<128, 32, 4, 1, 2, false>(g, s, w);
-    case 4: return launch_split<256, 128, 4, 2, 1, false>(g, s, w);
-    default: return launch_split<128, 32, 4, 1, 1, false>(g, s, w);
+    case 2: return launch_split<128, 96, 4, 1, 2, false>(g, s, w);
+    case 3: return launch_split<128, 64, 2, 2, 2, false>(g, s, w);
+    case 4: return launch_split<64, 96, 2, 1, 4, false>(g, s, w);
+    case 5: return launch_split<64, 64, 2, 1, 4, false>(g, s, w);
+    case 6: return launch_split<64, 32, 2, 1, 4, false>(g, s, w);
+    default: return launch_split<256, 128, 4, 2, 1, false>(g, s, w);
   }
 }
 int launch_cell_index(int c, SplitArgs &g, hipStream_t s) {
   const char *w = "lh_gate_gemm_split_lstm_cell_f32";
   switch (c) {
-    case 0: return launch_split<128, 128, 2, 2, 1, true>(g, s, w);
-    case 1: return launch_split<128, 96, 4, 1, 2, true>(g, s, w);
-    case 2: return launch_split<128, 64, 2, 2, 2, true>(g, s, w);
-    case 3: return launch_split<128, 32, 4, 1, 2, true>(g, s, w);
-    case 4: return launch_split<128, 64, 2, 2, 1, true>(g, s, w);
-    default: return launch_split<128, 32, 4, 1, 4, true>(g, s, w);
+    case 0: return launch_split<128, 96, 4, 1, 2, true>(g, s, w);
+    case 1: return launch_split<128, 64, 2, 2, 2, true>(g, s, w);
+    case 2: return launch_split<128, 32, 4, 1, 2, true>(g, s, w);
+    case 3: return launch_split<64, 96, 2, 1, 4, true>(g, s, w);
+    case 4: return launch_split<64, 64, 2, 1, 4, true>(g, s, w);
+    case 5: return launch_split<64, 64, 2, 2, 2, true>(g, s, w);
+    case 6: return launch_split<64, 32, 2, 1, 4, true>(g, s, w);
+    default: return launch_split<32, 32, 1, 1, 8, true>(g, s, w);
   }
 }
 
-// Plain: the largest tile that still gives every CU a workgroup and a half, the smallest one
-// otherwise.  Cell (few row tiles, one workgroup per CU at a time): 128x96 while that makes three
-// quarters of the CUs busy, 128x64 down to half of them, 128x32 below (measured at H = 1000).
-int choose(const SplitConfig *table, int n_auto, int n, int rows_tiles128, int M, int N, bool cell) {
+// Thresholds on the number of tiles, from sweeps over 48..768 columns (M = 30000: several
+// workgroups of a wide tile per CU; M = 4000 and 2000: few row tiles, a workgroup alone on its CU,
+// where wave groups that split K shorten the chain of slabs each workgroup walks).
+int choose(const SplitConfig *, int, int n, int rows_tiles128, int M, int N, bool cell) {
   if (g_split_override >= 0 && g_split_override < n) return g_split_override;
-  if (cell) {
-    if (4 * rows_tiles128 * ((N + 95) / 96) >= 3 * kCUs) return 1;
-    if (2 * rows_tiles128 * ((N + 63) / 64) > kCUs) return 2;
-    return 3;
+  const int t128 = cell ? rows_tiles128 : (M + 127) / 128, t64 = cell ? (M + 63) / 64 : (M + 63) / 64;
+  auto cols = [&](int bn) { return (N + bn - 1) / bn; };
+  if (cell) {  // M = 4H
+    if (4 * t128 * cols(96) >= 3 * kCUs) return 0;  // 128 x 96, 2 wave groups
+    if (t128 * cols(64) >= 224) return 1;           // 128 x 64, 2 wave groups
+    if (t64 * cols(96) >= 160) return 3;            //  64 x 96, 4 wave groups
+    if (t64 * cols(64) >= 160) return 4;            //  64 x 64, 4 wave groups
+    return 6;                                       //  64 x 32, 4 wave groups
   }
-  for (int c = 0; c < n_auto; ++c) {
-    const int tm = cell ? rows_tiles128 : (M + table[c].bm - 1) / table[c].bm;
-    const int tn = (N + table[c].bn - 1) / table[c].bn;
-    if (2 * tm * tn >= 3 * kCUs) return c;
-  }
-  return n_auto - 1;
+  if (2 * t128 * cols(128) >= 3 * kCUs) return 0;   // 128 x 128
+  if (2 * t128 * cols(64) >= 3 * kCUs) return 1;    // 128 x 64
+  if (4 * t128 * cols(96) >= 3 * kCUs) return 2;    // 128 x 96, 2 wave groups
+  if (t128 * cols(64) >= 224) return 3;             // 128 x 64, 2 wave groups
+  if (t64 * cols(96) >= 160) return 4;              //  64 x 96, 4 wave groups
+  if (t64 * cols(64) >= 160) return 5;              //  64 x 64, 4 wave groups
+  return 6;                                         //  64 x 32, 4 wave groups
 }
 
 int check_planes(const char *what, const void *p, const char *name) {
@@ -543,7 +560,7 @@ extern "C" int lh_gemm_split_f32(int M, int N, int kgroups, const void *A_planes
   g.alpha = alpha, g.beta = beta, g.bias = bias;
   g.act_rows = act == LH_ACT_TANH ? (act_rows < 0 ? M : std::min(act_rows, M)) : 0;
   g.colmask = colmask, g.C = C, g.ldc = ldc;
-  return launch_plain_index(choose(kPlain, kAutoPlain, kNumPlain, 0, M, N, false), g, lh::as_stream(stream));
+  return launch_plain_index(choose(kPlain, 0, kNumPlain, 0, M, N, false), g, lh::as_stream(stream));
 }
 
 extern "C" int lh_gate_gemm_split_lstm_cell_f32(int H, int B, int kgroups, const void *W_planes,
@@ -584,14 +601,14 @@ extern "C" int lh_gate_gemm_split_lstm_cell_f32(int H, int B, int kgroups, const
     g.h_planes = reinterpret_cast<u4v *>(h_planes);
     g.hp_KG = hp_kgroups_total, g.hp_kg0 = hp_kg_offset, g.hp_kgn = hp_kgroups, g.hp_Np = round_up(B, kPadD);
   }
-  const int tiles128 = (H + kGateRows - 1) / kGateRows;
-  return launch_cell_index(choose(kCell, kAutoCell, kNumCell, tiles128, 4 * H, B, true), g, lh::as_stream(stream));
+  const int tiles128 = (4 * H + 127) / 128;
+  return launch_cell_index(choose(kCell, 0, kNumCell, tiles128, 4 * H, B, true), g, lh::as_stream(stream));
 }
 
 extern "C" int lh_gemm_split_kernel_name(int cell, int M, int N, char *name, int name_cap) {
   if (!name || name_cap < 1 || M < 1 || N < 1) return lh::fail_arg("lh_gemm_split_kernel_name: M=%d N=%d", M, N);
-  const SplitConfig &k = cell ? kCell[choose(kCell, kAutoCell, kNumCell, (M + kGateRows - 1) / kGateRows, 4 * M, N, true)]
-                              : kPlain[choose(kPlain, kAutoPlain, kNumPlain, 0, M, N, false)];
+  const SplitConfig &k = cell ? kCell[choose(kCell, 0, kNumCell, (4 * M + 127) / 128, 4 * M, N, true)]
+                              : kPlain[choose(kPlain, 0, kNumPlain, 0, M, N, false)];
   snprintf(name, name_cap, "gemm_split_kernel<%d, %d, %d, %d, %d, %s>", k.bm, k.bn, k.wm, k.wn, k.wk,
            cell ? "true" : "false");
   return LH_OK;
@@ -599,6 +616,5 @@ extern "C" int lh_gemm_split_kernel_name(int cell, int M, int N, char *name, int
 
 extern "C" int lh_gemm_split_set_config_override(int config) {
   g_split_override = config < 0 ? -1 : config;
-  return kNumPlain;  // == kNumCell
+  return kNumPlain > kNumCell ? kNumPlain : kNumCell;  // an index past a table's end leaves that table's choice alone
 }
-static_assert(kNumPlain == kNumCell, "one override index space");

@@ -459,7 +459,7 @@ class NeuralMachineTranslation {
   // (lh_gemm_split_f32 / lh_gate_gemm_split_lstm_cell_f32) while at least split_min_columns_
   // hypotheses are alive; below that, and everywhere else, the fp32 MFMA products run.
   bool split_products_ = false;
-  int split_min_columns_ = 160;
+  int split_min_columns_ = 84;
   bool split_step_ = false;  // the step being run uses them
   bool SplitProductsUsable(int curr_index, int minibatch) const;
   Profiler profiler_;  // live HIP-event timing on stream_, off by default

@@ -258,6 +258,9 @@ static void ForwardPropSplit(LstmNode &n) {
     addend = L.mw_fold_.get();
   }
   LstmLayer *up = L.layer_number_ + 1 < M.cfg_.num_layers_ ? &M.TargetLayer(L.layer_number_ + 1) : nullptr;
+  // the layer above reads this layer's h as the first segment of its packed input
+  unsigned *h_planes = up ? up->split_x_planes_.get() : nullptr;
+  const int hp_total = up ? up->split_kgroups_ : 0, hp_groups = lh_split_kgroups(H);
   const float cell_clip = M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f;
   char name[160] = {0};
   if (M.profiler_.Wants(kTagGateGemm))
@@ -268,9 +271,8 @@ static void ForwardPropSplit(LstmNode &n) {
                      H, B, L.split_kgroups_, L.split_w_planes_.get(), L.split_x_planes_.get(), addend,
                      4 * H, addend ? n.p_device_input_vocab_indices_ : nullptr, addend ? L.vocab_size_ : 0,
                      L.p_device_b_stack_.get(), n.p_device_c_t_prev_, n.p_device_input_vocab_indices_01_,
-                     feed ? 1 : 0, cell_clip, n.p_device_c_t_, n.p_device_h_t_,
-                     up ? up->split_x_planes_.get() : nullptr, up ? up->split_kgroups_ : 0, 0,
-                     lh_split_kgroups(H), M.stream_),
+                     feed ? 1 : 0, cell_clip, n.p_device_c_t_, n.p_device_h_t_, h_planes, hp_total, 0,
+                     hp_groups, M.stream_),
                  "LstmNode::ForwardPropGpu split gate product with cell");
 }
 

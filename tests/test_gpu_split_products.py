@@ -103,7 +103,7 @@ def test_split_arguments_are_checked(lh):
         lh.gemm_split(64, 64, kg, P, P, out, 32)              # ldc < M
     with pytest.raises(lh.LinmtHipError):
         lh.split_pack([dict(src=out, ld=64, k_contiguous=True, D=64, K=64, planes=P, kgroups_total=kg,
-                            kg_offset=2)])                    # segment does not fit
+                            kg_offset=kg - 4)])               # segment does not fit
     with pytest.raises(lh.LinmtHipError):
         lh.gate_gemm_split_lstm_cell(36, 8, kg, P, P, out, out, out, out, out)   # H not a multiple of 8
 
