@@ -247,6 +247,7 @@ def bench_mfma_kernels(torch, steps, warmup):
     """The decode step's two MFMA kernels alone, at the size one step of the benchmark gives them
     (768 columns): the output projection D*h~ + b_d and one layer's gate product with the fused
     LSTM cell, next to a plain 1 GiB copy (the calibration point for clock counters)."""
+    import ctypes as C
     from linmt_amd import lib as lh
     lh.load()
     steps = max(steps, 20)
@@ -292,8 +293,49 @@ def bench_mfma_kernels(torch, steps, warmup):
                 "shape": f"M={4 * H} N={B} K={H}+{H}", "flop": flop, "us": round(us, 2),
                 "TFLOP/s": round(flop / us / 1e6, 2),
                 "frac_of_peak": round(flop / us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 4)})
+    # the same two products from three-way bf16 splits (six bf16 MFMAs per fp32 one): operands packed
+    # ahead, as the decoder does (weights once, the step's inputs per step)
+    L = lh.load()
+    kg = lh.split_kgroups_padded(lh.split_kgroups(H))
+    D = f(V * H)
+    Dp = torch.empty(lh.split_bytes(V, kg) // 4, dtype=torch.int32, device=dev)
+    xp = torch.empty(lh.split_bytes(B, kg) // 4, dtype=torch.int32, device=dev)
+    logits = torch.empty(V * B, device=dev)
+    lh.split_pack([dict(src=D, ld=V, k_contiguous=False, D=V, K=H, planes=Dp, kgroups_total=kg, kgroups=kg)])
+    src_x = [dict(src=x, ld=H, k_contiguous=True, D=B, K=H, planes=xp, kgroups_total=kg, kgroups=kg)]
+    us_pack = timed(lambda: lh.split_pack(src_x))
+    us = timed(lambda: lh.gemm_split(V, B, kg, Dp, xp, logits, V, bias=bd))
+    flop = 2.0 * V * B * H
+    name = C.create_string_buffer(160)
+    L.lh_gemm_split_kernel_name(0, V, B, name, 160)
+    out.append({"kernel": "logits_gemm, split products", "instance": name.value.decode(),
+                "shape": f"M={V} N={B} K={H}", "flop": flop, "us": round(us, 2),
+                "TFLOP/s": round(flop / us / 1e6, 2), "bf16_TFLOP/s_issued": round(6 * flop / us / 1e6, 1),
+                "frac_of_bf16_peak": round(6 * flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                "packing_h_us": round(us_pack, 2)})
+    del D, Dp, logits
+    g1 = lh.split_kgroups(H)
+    KG = lh.split_kgroups_padded(2 * g1)
+    Wp = torch.empty(lh.split_bytes(L.lh_split_gate_rows(H), KG) // 4, dtype=torch.int32, device=dev)
+    Xp = torch.empty(lh.split_bytes(B, KG) // 4, dtype=torch.int32, device=dev)
+    lh.split_pack([dict(src=M4, ld=4 * H, k_contiguous=False, D=4 * H, K=H, gate_H=H, planes=Wp,
+                        kgroups_total=KG, kg_offset=0, kgroups=g1),
+                   dict(src=W, ld=4 * H, k_contiguous=False, D=4 * H, K=H, gate_H=H, planes=Wp,
+                        kgroups_total=KG, kg_offset=g1, kgroups=KG - g1)])
+    src_g = [dict(src=hb, ld=H, k_contiguous=True, D=B, K=H, planes=Xp, kgroups_total=KG, kg_offset=0, kgroups=g1),
+             dict(src=hp, ld=H, k_contiguous=True, D=B, K=H, planes=Xp, kgroups_total=KG, kg_offset=g1,
+                  kgroups=KG - g1)]
+    lh.split_pack(src_g)
+    us = timed(lambda: lh.gate_gemm_split_lstm_cell(H, B, KG, Wp, Xp, b4, cp, m, c, h))
+    flop = 2.0 * 4 * H * B * 2 * H
+    L.lh_gemm_split_kernel_name(1, H, B, name, 160)
+    out.append({"kernel": "gate_gemm + lstm cell, split products", "instance": name.value.decode(),
+                "shape": f"M={4 * H} N={B} K={H}+{H}", "flop": flop, "us": round(us, 2),
+                "TFLOP/s": round(flop / us / 1e6, 2), "bf16_TFLOP/s_issued": round(6 * flop / us / 1e6, 1),
+                "frac_of_bf16_peak": round(6 * flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)})
     return {"metric": "MFMA kernels alone, fp32 TFLOP/s", "unit": "TFLOP/s",
-            "peak": MFMA_FP32_PEAK_TFLOPS, "launches_timed": steps, "kernels": out}
+            "peak": MFMA_FP32_PEAK_TFLOPS, "bf16_peak": MFMA_BF16_PEAK_TFLOPS, "launches_timed": steps,
+            "kernels": out}
 
 
 def bench_training(torch, host, steps, warmup, small):
@@ -379,6 +421,9 @@ def main():
     ap.add_argument("--no-split-products", action="store_true",
                     help="skip the second timing of the same batch with the opt-in arithmetic "
                          "(lnmt_set_split_products; reported beside `value`, never as it)")
+    ap.add_argument("--split-products-only", action="store_true",
+                    help="profiling aid: the whole run (timed steps, kernel table, parity) with the "
+                         "opt-in arithmetic switched on; the JSON line's metric and dtype say so")
     ap.add_argument("--profile-level", type=int, default=1,
                     help="1: HIP events around the output projection (the dominant kernel) during "
                          "the timed steps; "
@@ -424,7 +469,9 @@ def main():
     model = host.Model(layers, H, V, V, longest_sentence=longest, attention_mode=1,
                        attention_width=D, feed_input=True, decoding=(n_sent, beam))
     model.set_params(P)
-    model.set_split_products(False)  # `value` is the fp32 MFMA path whatever the environment says
+    # `value` is the fp32 MFMA path whatever the environment says (unless the run is asked to be
+    # about the opt-in arithmetic, which its metric then names)
+    model.set_split_products(bool(args.split_products_only))
 
     for _ in range(args.warmup):
         model.decode_batch(sents, beam=beam)
@@ -462,6 +509,11 @@ def main():
                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_FP32_PEAK_TFLOPS, 4),
                     "traffic": MEASURED_TRAFFIC_BYTES.get(kern), "launches": g["launches"],
                     "avg_launch_us": round(g["ms"] * 1e3 / g["launches"], 2)}
+        if kern.startswith("gemm_split_kernel"):  # six bf16 products issued per algorithmic product
+            roofline.update({"algorithmic_TFLOP/s": round(achieved, 2), "achieved": round(6 * achieved, 1),
+                             "peak": MFMA_BF16_PEAK_TFLOPS,
+                             "unit": "TFLOP/s (bf16 products issued = 6 x algorithmic)",
+                             "frac": round(6 * achieved / MFMA_BF16_PEAK_TFLOPS, 4)})
 
     histories = [model.decode_history(i, beam) for i in range(n_sent)]  # of the last timed batch
     kernels = {}
@@ -482,7 +534,7 @@ def main():
     # bf16 splits of their fp32 operands (six exact products per term, fp32 accumulation).  Reported
     # beside `value`; `value` stays the fp32 MFMA path.
     split, split_res, split_hist = None, None, None
-    if not args.no_split_products:
+    if not args.no_split_products and not args.split_products_only:
         model.set_split_products(True)
         model.decode_batch(sents, beam=beam)  # packs the weights
         model.profile(1)
@@ -591,7 +643,8 @@ def main():
                                "beam_steps": sclasses, "parity_ok": sclasses["diverged_other"] == 0}
 
     out = {
-        "metric": "target tokens/sec (beam-12 decode, 1 GPU)",
+        "metric": "target tokens/sec (beam-12 decode, 1 GPU)" +
+                  (" with split bf16 products (opt-in arithmetic)" if args.split_products_only else ""),
         "value": round(value, 1),
         "unit": "target tokens/s",
         "n_gpus": 1,
@@ -601,7 +654,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f32 operands as three bf16 terms, f32 accumulation" if args.split_products_only else "f32",
         "data": "synthetic",
         "config": {"workload": "configs[2]: beam-12 decode, 64 sentences/batch (768 live "
                                "hypotheses), 4+4 LSTM layers, hidden=emb=1000, vocab 30k/30k, "
