@@ -292,6 +292,28 @@ def test_decode_same_with_split_products(orc, host, layers, H, attention, feed, 
     gm.close()
 
 
+def test_decode_ensemble_and_alignments_with_split_products(orc, host):
+    """Split products under the other decoding features: an ensemble of two models of different
+    width (both with split products, each packing its own weights) with exported alignments and
+    the coverage penalty -- against the oracle's ensemble search."""
+    rng = np.random.default_rng(21)
+    Vs, Vt, beam, lens = 60, 72, 4, (9, 4, 12, 2, 7)
+    pairs = [_pair(orc, host, rng, L, H, Vs, Vt, D, 30, 0.5, decoding=(len(lens), beam))
+             for L, H, D in ((2, 48, 2), (3, 40, 10))]
+    oms, gms = [p[1] for p in pairs], [p[2] for p in pairs]
+    sents = [rng.integers(0, Vs, size=n) for n in lens]
+    for g in gms:
+        g.set_split_products(True, 1)
+    kw = dict(alignments=True, cp_beta=0.6, lp_alpha=0.3)
+    got = gms[0].decode_batch(sents, beam=beam, with_hyps=True, ensemble=gms[1:], **kw)
+    for i, s in enumerate(sents):
+        want = oms[0].decode_sentence(s, beam=beam, ensemble=tuple(oms[1:]), **kw)
+        _compare_decode(want, got[i], f"split products, ensemble, sentence {i} (len {len(s)})")
+        assert got[i]["best_viterbi"].tolist() == want["best_viterbi"].tolist(), i
+    for g in gms:
+        g.close()
+
+
 def test_decode_random_architectures_vs_oracle(orc, host):
     """A seeded sweep over architectures and batch shapes the fixed cases do not hit: 1-4 layers,
     hidden sizes that land on different tile configurations (and on the one- and two-quad attention
