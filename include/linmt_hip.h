@@ -250,6 +250,8 @@ int lh_gemm_config_info(int config, int transA, int transX, int info[8]);
  *     (D = 4 * gate_H) whose rows are laid out in cell-tile order for
  *     lh_gate_gemm_split_lstm_cell_f32.
  * A packed X depends on its column count: pack and product must be given the same N / B.
+ * Operand values must be finite and below 3.3e38 in magnitude: the first bf16 term of a larger one
+ * rounds to infinity, and where an fp32 product would give an infinity these give a NaN.
  * lh_gemm_split_f32: C = epilogue(alpha * A X + beta * C), epilogue exactly as lh_gemm_act_rows_f32.
  * lh_gate_gemm_split_lstm_cell_f32: lh_gate_gemm_lstm_cell_f32 on packed operands; H must be a
  * multiple of 8; addend, bias4h, c_prev, c, h 16-byte aligned.  h_planes != NULL: h is also

@@ -66,7 +66,7 @@ struct PackSrc {
   int Dp, KG, kg0, kgn;  // padded rows, k-groups of the whole operand, first k-group and count written
 };
 struct PackArgs {
-  PackSrc s[8];
+  PackSrc s[LH_SPLIT_PACK_MAX];
 };
 
 // one thread per (k-group, packed row) of source blockIdx.y
@@ -535,7 +535,7 @@ extern "C" int lh_split_pack_f32(const lh_split_source *srcs, int n, lh_stream_t
     o.Dp = Dp, o.KG = q.kgroups_total, o.kg0 = q.kg_offset, o.kgn = kgn;
     most = std::max(most, (long)Dp * kgn);
   }
-  for (int i = n; i < 8; ++i) a.s[i] = a.s[0];
+  for (int i = n; i < LH_SPLIT_PACK_MAX; ++i) a.s[i] = a.s[0];
   const dim3 grid((unsigned)((most + 255) / 256), (unsigned)n);
   split_pack_kernel<<<grid, 256, 0, lh::as_stream(stream)>>>(a);
   return lh::check_launch("lh_split_pack_f32");

@@ -79,6 +79,9 @@ GEMM_CASES = [
     (37, 13, (101,), False, False),             # nothing divisible by 4: scalar path, tails
     (37, 13, (101, 5), True, False),
     (130, 70, (19,), False, True),
+    (1001, 301, (999, 77), False, False),       # the scalar path at a size where every tile edge, K tail
+    (2047, 129, (1023,), True, False),          # and segment boundary is crossed many times
+    (513, 700, (257,), False, True),
 ]
 
 
