@@ -338,7 +338,7 @@ def bench_mfma_kernels(torch, steps, warmup):
             "kernels": out}
 
 
-def bench_training(torch, host, steps, warmup, small):
+def bench_training(torch, host, steps, warmup, small, split=False):
     """One training minibatch (forward with stored activations, backward, global-norm clip at 5,
     SGD update) of the 8+8-layer, 2048-hidden, 1024-embedding, 50k-vocabulary model with local-p
     attention and input feeding, batch 256, lengths uniform in [20,80], dropout 0.2
@@ -355,6 +355,7 @@ def bench_training(torch, host, steps, warmup, small):
                    training=dict(learning_rate=0.1, grad_clip_mode=2, norm_clip=5.0, dropout_keep=0.8,
                                  dropout_seed=SEED))
     m.set_params(make_params(rng, L, H, V, V, E=E, fast=True))
+    m.set_split_products(bool(split))
     t_init = time.time() - t0
     ls = rng.integers(lo, hi + 1, size=B)
     lt = rng.integers(lo, hi + 1, size=B)
@@ -439,6 +440,8 @@ def main():
                     help="instead of the decode benchmark, time one training minibatch of "
                          "BASELINE.json configs[4] and print one JSON line")
     ap.add_argument("--train-small", action="store_true", help="--train at a reduced size")
+    ap.add_argument("--train-split-products", action="store_true",
+                    help="--train with the opt-in arithmetic for the large batched products")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU (the path shards over sentences with no "
@@ -458,8 +461,9 @@ def main():
     if args.mfma_kernels:
         print(json.dumps(bench_mfma_kernels(torch, args.steps, args.warmup)))
         return
-    if args.train or args.train_small:
-        print(json.dumps(bench_training(torch, host, args.steps, args.warmup, args.train_small)))
+    if args.train or args.train_small or args.train_split_products:
+        print(json.dumps(bench_training(torch, host, args.steps, args.warmup, args.train_small,
+                                        args.train_split_products)))
         return
 
     layers, H, V, D, beam, n_sent, longest = 4, 1000, 30000, 10, 12, 64, 104

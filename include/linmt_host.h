@@ -163,7 +163,11 @@ void *lnmt_model_stream(lnmt_model *m);
  * linmt_hip.h): every fp32 product a*x becomes six exact bf16 products added in fp32, which leaves
  * out less than one fp32 rounding per product.  Everything else -- the encoder, attention, steps
  * with fewer columns, scoring and training -- keeps the fp32 MFMA products, as does the default.
- * The environment variable LINMT_SPLIT_PRODUCTS=1 switches it on when a decoding model is created. */
+ * On a model created for training the same switch makes the large batched products of a minibatch
+ * (weight gradients accumulated over all steps, the output projection and its two backward products,
+ * the layer-major input products) split products, both operands packed per call; the per-step
+ * products keep the fp32 MFMA path (min_columns == 1 there takes every product: a test aid).
+ * The environment variable LINMT_SPLIT_PRODUCTS=1 switches it on when a model is created. */
 int lnmt_set_split_products(lnmt_model *m, int on, int min_columns);
 
 /* Live kernel timing with HIP events on the model's stream.  level 0 = off, 1 = the output

@@ -340,8 +340,8 @@ extern "C" int lnmt_profile_set_level(lnmt_model *m, int level) {
 
 extern "C" int lnmt_set_split_products(lnmt_model *m, int on, int min_columns) {
   return Guard([&] {
-    if (on && m->nmt->cfg_.lstm_size_ % 8)
-      throw linmt::LinmtError("lnmt_set_split_products: the hidden size must be a multiple of 8");
+    if (on && m->nmt->decode_mode_ && m->nmt->cfg_.lstm_size_ % 8)
+      throw linmt::LinmtError("lnmt_set_split_products: decoding needs a hidden size that is a multiple of 8");
     m->nmt->split_products_ = on != 0;
     if (min_columns > 0) m->nmt->split_min_columns_ = min_columns;
   });

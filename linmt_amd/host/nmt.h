@@ -462,6 +462,14 @@ class NeuralMachineTranslation {
   int split_min_columns_ = 84;
   bool split_step_ = false;  // the step being run uses them
   bool SplitProductsUsable(int curr_index, int minibatch) const;
+  // The same switch on a model created for training: Gemm() forms its large batched products
+  // (weight gradients over all steps, the output projection and its backward products, the
+  // layer-major input products) this way, packing both operands on the fly into these buffers;
+  // worthwhile while the packing is a small part of the product (both extents in the thousands).
+  DeviceArray<unsigned> split_scratch_a_, split_scratch_x_;
+  bool GemmAsSplitProduct(int tag, int rows, int cols, const lh_gemm_seg *segs, int nseg, int trans_a,
+                          int trans_x, float beta, const float *bias, int act, const int *colmask,
+                          float *C, int ldc, const char *what, int act_rows);
   Profiler profiler_;  // live HIP-event timing on stream_, off by default
   // Scratch of lh_gemm_ws_f32 (split-K partial sums); every product of the model runs on
   // stream_, which is the ordering that sharing it requires.

@@ -23,12 +23,74 @@ void NeuralMachineTranslation::Gemm(int tag, int rows, int cols, const lh_gemm_s
                                     int trans_a, int trans_x, float beta, const float *bias, int act,
                                     const int *colmask, float *C, int ldc, const char *what,
                                     int act_rows) {
+  if (split_products_ && cfg_.train_mode_ &&
+      GemmAsSplitProduct(tag, rows, cols, segs, nseg, trans_a, trans_x, beta, bias, act, colmask, C, ldc,
+                         what, act_rows))
+    return;
   ProfileScope ps(profiler_, tag, gemm_ws_bytes_, 0, rows, cols, segs, nseg, trans_a, trans_x);
   LhErrorWrapper(lh_gemm_ws_f32(rows, cols, segs, nseg, trans_a, trans_x, 1.f, beta, bias, act,
                                 act_rows < 0 ? rows : act_rows,
                                 colmask, C, ldc, gemm_ws_ptr_, gemm_ws_bytes_,
                                 stream_),
                  what);
+}
+
+// A large product as a split product: both operands packed into the model's two scratch buffers by
+// one launch, then lh_gemm_split_f32.  false = not worthwhile or not expressible; the caller runs
+// the fp32 MFMA product.
+bool NeuralMachineTranslation::GemmAsSplitProduct(int tag, int rows, int cols, const lh_gemm_seg *segs,
+                                                  int nseg, int trans_a, int trans_x, float beta,
+                                                  const float *bias, int act, const int *colmask,
+                                                  float *C, int ldc, const char *what, int act_rows) {
+  if ((trans_a && trans_x) || nseg < 1 || nseg > 3) return false;
+  double k_sum = 0;
+  int groups = 0;
+  for (int i = 0; i < nseg; ++i) {
+    if (i + 1 < nseg && segs[i].K % 8) return false;  // segments sit side by side in whole k-groups
+    k_sum += segs[i].K;
+    groups += lh_split_kgroups(segs[i].K);
+  }
+  // packing costs about 10 bytes of traffic per operand element against 2*rows*cols*K flop:
+  // 160 * (1/rows + 1/cols) is its share of the product's time at the rates of this GPU
+  // (split_min_columns_ == 1, a test aid, takes every product)
+  if (split_min_columns_ != 1 &&
+      (2.0 * rows * cols * k_sum < 2e10 || 160.0 * (1.0 / rows + 1.0 / cols) > 0.2))
+    return false;
+  const int total = lh_split_kgroups_padded(groups);
+  const size_t a_bytes = lh_split_bytes(rows, total), x_bytes = lh_split_bytes(cols, total);
+  if (a_bytes >= (size_t(1) << 32) || x_bytes >= (size_t(1) << 32)) return false;
+  if (split_scratch_a_.size() * sizeof(unsigned) < a_bytes || split_scratch_x_.size() * sizeof(unsigned) < x_bytes) {
+    Synchronize();  // earlier products may still read the buffers about to be replaced
+    if (split_scratch_a_.size() * sizeof(unsigned) < a_bytes) split_scratch_a_.Alloc(a_bytes / sizeof(unsigned));
+    if (split_scratch_x_.size() * sizeof(unsigned) < x_bytes) split_scratch_x_.Alloc(x_bytes / sizeof(unsigned));
+  }
+  lh_split_source src[6];
+  int n = 0, off = 0;
+  for (int i = 0; i < nseg; ++i) {
+    const int g = lh_split_kgroups(segs[i].K), written = i + 1 == nseg ? total - off : g;
+    lh_split_source a{}, x{};
+    // A is rows x K: stored column by column (rows contiguous) unless transposed
+    a.src = segs[i].A, a.ld = segs[i].lda, a.k_contiguous = trans_a ? 1 : 0, a.D = rows, a.K = segs[i].K;
+    a.planes = split_scratch_a_.get(), a.kgroups_total = total, a.kg_offset = off, a.kgroups = written;
+    // X is K x cols: stored column by column (k contiguous) unless transposed
+    x.src = segs[i].X, x.ld = segs[i].ldx, x.k_contiguous = trans_x ? 0 : 1, x.D = cols, x.K = segs[i].K;
+    x.planes = split_scratch_x_.get(), x.kgroups_total = total, x.kg_offset = off, x.kgroups = written;
+    src[n++] = a;
+    src[n++] = x;
+    off += g;
+  }
+  {
+    ProfileScope ps(profiler_, kTagSplitPack, 10.0 * ((double)rows + cols) * k_sum);
+    LhErrorWrapper(lh_split_pack_f32(src, n, stream_), what);
+  }
+  char name[160] = {0};
+  if (profiler_.Wants(tag))
+    LhErrorWrapper(lh_gemm_split_kernel_name(0, rows, cols, name, sizeof(name)), "lh_gemm_split_kernel_name");
+  ProfileScope ps(profiler_, tag, name, 2.0 * rows * cols * k_sum);
+  LhErrorWrapper(lh_gemm_split_f32(rows, cols, total, split_scratch_a_.get(), split_scratch_x_.get(), 1.f, beta,
+                                   bias, act, act_rows < 0 ? rows : act_rows, colmask, C, ldc, stream_),
+                 what);
+  return true;
 }
 
 NeuralMachineTranslation::~NeuralMachineTranslation() {
@@ -52,6 +114,7 @@ void NeuralMachineTranslation::Synchronize() {
 // One node per timestep on both sides, minibatch = cfg.minibatch_size_ (deep_rnn.h:249-692).
 void NeuralMachineTranslation::InitModel() {
   decode_mode_ = false;
+  if (const char *sp = std::getenv("LINMT_SPLIT_PRODUCTS")) split_products_ = sp[0] == '1';
   const int B = cfg_.minibatch_size_, T = cfg_.longest_sentence_, L = cfg_.num_layers_;
   const bool seq2seq = cfg_.sequence_to_sequence_mode_;
   const bool keep = cfg_.train_mode_;  // training keeps i,f,g,o and the looked-up embeddings per step

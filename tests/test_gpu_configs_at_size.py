@@ -189,6 +189,29 @@ def test_config5_training_step_at_width(orc, host):
         worst_fro, worst_el = max(worst_fro, (fro, name)), max(worst_el, (el, name))
     print(f"gradients: largest relative Frobenius error {worst_fro[0]:.2e} ({worst_fro[1]}), largest "
           f"element error / max entry {worst_el[0]:.2e} ({worst_el[1]})", flush=True)
+
+    # the same minibatch on a second model whose matrix products are split bf16 products (size
+    # thresholds off: every product that goes through Gemm()); same seed, hence the same masks
+    gs = host.Model(layers, H, V, V, longest_sentence=16, attention_mode=1, attention_width=D,
+                    feed_input=True, minibatch_size=B, embedding_size=E,
+                    training=dict(learning_rate=lr, grad_clip_mode=2, norm_clip=clip,
+                                  dropout_keep=keep, dropout_seed=99))
+    gs.set_params(P)
+    gs.set_split_products(True, 1)
+    split_ll = gs.compute_gradients(src, tin, tout, bi, su, tu)
+    assert np.array_equal(gs.get_dropout_mask(0, 1, 0, E, B, T), te)
+    assert_close(split_ll / n_words, want_ll / n_words, "log-likelihood per word, split products",
+                 rtol=1e-4, atol=1e-5)
+    worst = (0.0, "")
+    for name in names:
+        w = np.asarray(want[name])
+        shape = w.shape if w.ndim == 2 else (w.size,)
+        fro, _ = _scaled_close(gs.get_grad(name, shape), w.reshape(shape, order="F"),
+                               f"gradient of {name}, split products")
+        worst = max(worst, (fro, name))
+    print(f"gradients with split products: largest relative Frobenius error {worst[0]:.2e} ({worst[1]})",
+          flush=True)
+    gs.close()
     del want
 
     # UpdateWeights, global-norm clip (embedding gradients outside the norm, inside the rescale)

@@ -93,6 +93,44 @@ def test_compute_gradients_vs_oracle(orc, host, case):
     gm.close()
 
 
+@pytest.mark.parametrize("case", [CASES[0], CASES[1], CASES[3], CASES[4], CASES[6]],
+                         ids=lambda c: f"L{c['layers']}H{c['H']}E{c.get('E', 0)}a{c['attention']}f{c['feed']}")
+def test_compute_gradients_with_split_products_vs_oracle(orc, host, case):
+    """lnmt_set_split_products on a training model, size thresholds off (min_columns = 1): every
+    matrix product that goes through the model's Gemm() -- error and weight-gradient products,
+    transposed operands, several K segments, accumulation into the gradient buffers, the output
+    projection, attention, unaligned sizes -- is packed into bf16 planes and formed as six exact
+    products per term.  Same tolerance against the oracle as the fp32 MFMA products."""
+    rng = np.random.default_rng(case["seed"])
+    Vs, Vt = 29, 41
+    lens_s, lens_t = [5, 3, 9, 4, 7, 1], [4, 6, 2, 8, 5, 3]
+    B = len(lens_s)
+    P, om, gm = _pair(orc, host, rng, case["layers"], case["H"], Vs, Vt, case["D"],
+                      case["attention"], case["feed"], B, dict(grad_clip_mode=0), E=case.get("E"))
+    sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
+    want_ll, want = om.compute_gradients(src, tin, tout, bi, su, tu)
+    gm.set_split_products(True, 1)
+    gm.profile(2)
+    got_ll = gm.compute_gradients(src, tin, tout, bi, su, tu)
+    keys = list(gm.profile_totals())
+    gm.profile(0)
+    # everything that goes through the model's Gemm(): only the forward gate product of a step,
+    # which hands the cell kernel up to three addends (GemmAddends), keeps the fp32 MFMA kernel
+    fp32 = sorted({k.split("|")[0] for k in keys if "|gemm_kernel" in k or "|gemm_generic_kernel" in k})
+    # (and, when H is not a multiple of 8, products of several K segments: segments are packed
+    # side by side in whole groups of 8 k)
+    allowed = {"gate_gemm"} | ({"attn_out_gemm", "error_gemm"} if case["H"] % 8 else set())
+    assert set(fp32) <= allowed, keys
+    for site in ("weight_grad_gemm", "error_gemm", "logits_gemm"):
+        assert any(k.startswith(site + "|gemm_split_kernel") for k in keys), (site, keys)
+    assert_close(got_ll, want_ll, "sum log p(target)", rtol=1e-5, atol=1e-4)
+    for name in om.param_names():
+        shape = _grad_shape(P, name, su, tu)
+        assert_close(gm.get_grad(name, shape), np.asarray(want[name]).reshape(shape, order="F"),
+                     f"gradient of {name}", atol=2e-5)
+    gm.close()
+
+
 @pytest.mark.parametrize("case", [CASES[0], CASES[2], CASES[3], CASES[4], CASES[5]],
                          ids=lambda c: f"L{c['layers']}H{c['H']}E{c.get('E', 0)}a{c['attention']}f{c['feed']}")
 def test_stepwise_reference_calls_give_the_same_gradients(orc, host, case):
