@@ -544,9 +544,11 @@ def main():
         model.profile(1)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        stok = 0
+        stok, per_batch = 0, []
         for _ in range(args.steps):
-            split_res = model.decode_batch(sents, beam=beam)
+            b0 = time.perf_counter()
+            split_res = model.decode_batch(sents, beam=beam)  # ends with a stream synchronisation
+            per_batch.append((time.perf_counter() - b0) * 1e3)
             stok += sum(len(r["best"]) for r in split_res)
         torch.cuda.synchronize()
         sdt = time.perf_counter() - t0
@@ -566,6 +568,7 @@ def main():
         model.set_split_products(False)
         split = {"value": round(stok / sdt, 1), "unit": "target tokens/s",
                  "ms_per_step": round(sdt * 1e3 / args.steps, 2),
+                 "ms_per_step_median": round(float(np.median(per_batch)), 2),
                  "speedup_over_value": round(stok / sdt / value, 3),
                  "arithmetic": "fp32 operands held as three bf16 terms; every product = six exact "
                                "bf16 x bf16 products (v_mfma_f32_32x32x16_bf16) added in fp32; what "
