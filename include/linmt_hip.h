@@ -478,6 +478,19 @@ int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const int *limit,
 int lh_beam_gather_f32(const float *const *src, float *const *dst, int n_tensors, int H, int B,
                        int B_src, const int *backptr, lh_stream_t stream);
 
+/* a10 + a11 in one launch: lh_beam_merge_f32 followed by lh_beam_gather_f32 over the n_sent*beam
+ * columns with the back-pointers just chosen (B = B_src = n_sent*beam), i.e. the tail of
+ * Decoder::ExpandHypothesis (src/decoder.h:430-480) and NeuralMachineTranslation::
+ * SwapDecodingStates (src/deep_rnn.h:1842-1857) behind it.  Same arguments, same outputs bit for
+ * bit as the two calls; several workgroups per sentence repeat the (cheap) merge so that the
+ * copies of a sentence's columns start without a second launch.  beam <= 256. */
+int lh_beam_merge_gather_f32(int n_sent, int beam, int K, int step, const int *limit,
+                             const float *cand_logp, const int *cand_id, const float *logp_eof,
+                             const float *prev_score, float diversity, float penalty, int start_id,
+                             int eof_id, int *tok, int *backptr, float *score, int *fin_count,
+                             int *fin_beam, float *fin_score, const float *const *src,
+                             float *const *dst, int n_tensors, int H, lh_stream_t stream);
+
 /* ==========================================================================================
  * Training half of the path (backward pass and update).
  * ========================================================================================== */

@@ -23,10 +23,14 @@ struct MergeArgs {
   float *fin_score;
 };
 
-// One workgroup per sentence.  Candidates are ranked by counting how many others precede them in
-// the total order (score desc, beam column asc, vocab id asc); thread 0 then walks that order the
-// way Decoder::ExpandHypothesis pops its global heap.
-__global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeArgs a) {
+// One workgroup merges one sentence.  Candidates are ranked by counting how many others precede
+// them in the total order (score desc, beam column asc, vocab id asc); slots and finished indices
+// follow from prefix counts over that order, which is what Decoder::ExpandHypothesis gets by
+// popping its global heap.  `write`: this workgroup stores the step's outputs (several workgroups
+// may merge the same sentence, each for its own use of the result).  s_bp (LDS, beam entries)
+// receives the back-pointers; valid for the whole workgroup after a barrier.
+__device__ __forceinline__ void merge_sentence(const MergeArgs &a, const int s, const bool write,
+                                               int *s_bp) {
   __shared__ float s_score[kMaxCand];
   __shared__ int s_id[kMaxCand];
   __shared__ short s_col[kMaxCand];
@@ -34,7 +38,7 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
   __shared__ unsigned char s_flag[kMaxCand];
   __shared__ int s_total[2];  // slot-taking candidates; finished hypotheses the walk reaches
 
-  const int s = blockIdx.x, tid = threadIdx.x;
+  const int tid = threadIdx.x;
   const int beam = a.beam, K = a.K;
   const int c0 = s * beam;  // first global column of this sentence
   const int limit = a.limit[s];
@@ -42,6 +46,8 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
   if (a.step >= limit) {
     // finish (== limit) or idle (> limit): no expansion.
     for (int i = tid; i < beam; i += kMergeThreads) {
+      s_bp[i] = c0 + i;
+      if (!write) continue;
       a.tok[c0 + i] = a.eof_id;
       a.backptr[c0 + i] = c0 + i;
       float sc = a.prev_score[c0 + i];
@@ -52,7 +58,7 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
       }
       a.score[c0 + i] = sc;
     }
-    if (tid == 0) a.fin_count[s] = a.step == limit ? beam : 0;
+    if (tid == 0 && write) a.fin_count[s] = a.step == limit ? beam : 0;
     return;
   }
 
@@ -114,25 +120,37 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeAr
       const float sc = s_score[e] + a.penalty;
       if (f == 2) {
         atomicAdd(&s_total[1], 1);
-        if (fins < beam) {  // at most one <EOF> candidate per column exists
+        if (fins < beam && write) {  // at most one <EOF> candidate per column exists
           a.fin_beam[c0 + fins] = s_col[e];
           a.fin_score[c0 + fins] = sc;
         }
       } else {
-        a.tok[c0 + slots] = s_id[e];
-        a.backptr[c0 + slots] = c0 + s_col[e];
-        a.score[c0 + slots] = sc;
+        s_bp[slots] = c0 + s_col[e];
+        if (write) {
+          a.tok[c0 + slots] = s_id[e];
+          a.backptr[c0 + slots] = c0 + s_col[e];
+          a.score[c0 + slots] = sc;
+        }
       }
     }
   }
   __syncthreads();
   // slots left empty when the candidates run out (the reference pops an empty heap)
   for (int i = min(s_total[0], beam) + tid; i < beam; i += kMergeThreads) {
+    s_bp[i] = c0;
+    if (!write) continue;
     a.tok[c0 + i] = a.eof_id;
     a.backptr[c0 + i] = c0;
     a.score[c0 + i] = -FLT_MAX;
   }
-  if (tid == 0) a.fin_count[s] = min(s_total[1], beam);
+  if (tid == 0 && write) a.fin_count[s] = min(s_total[1], beam);
+}
+
+constexpr int kMaxBeam = 256;  // back-pointers of a sentence kept in LDS
+
+__global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(const MergeArgs a) {
+  __shared__ int s_bp[kMaxBeam];
+  merge_sentence(a, blockIdx.x, true, s_bp);
 }
 
 struct GatherArgs {
@@ -159,6 +177,73 @@ __global__ __launch_bounds__(256) void beam_gather_kernel(const GatherArgs a) {
   }
 }
 
+// Merge + gather in one launch.  blockIdx.y = sentence, blockIdx.x = one of gridDim.x workgroups
+// that each merge the sentence (the merge reads nothing that any of them writes), the first one
+// storing the step's outputs; then the workgroups share the sentence's column copies
+// dst_t[:, s*beam + i] = src_t[:, backptr[s*beam + i]] between them, 256 threads per column.
+template <int VW>
+__global__ __launch_bounds__(kMergeThreads) void beam_merge_gather_kernel(const MergeArgs a,
+                                                                          const GatherArgs ga,
+                                                                          const int n_tensors) {
+  __shared__ int s_bp[kMaxBeam];
+  const int s = blockIdx.y;
+  merge_sentence(a, s, blockIdx.x == 0, s_bp);
+  __syncthreads();
+  const int beam = a.beam, c0 = s * beam;
+  const int HQ = ga.H / VW;
+  const int sub = threadIdx.x / 256, lane = threadIdx.x % 256;
+  constexpr int kSubs = kMergeThreads / 256;
+  for (int it = blockIdx.x * kSubs + sub; it < n_tensors * beam; it += gridDim.x * kSubs) {
+    const int t = it / beam, i = it % beam;
+    int from = s_bp[i];
+    from = from < 0 ? 0 : (from >= ga.B_src ? ga.B_src - 1 : from);
+    const float *src = ga.src[t] + (size_t)from * ga.H;
+    float *dst = ga.dst[t] + (size_t)(c0 + i) * ga.H;
+    for (int q = lane; q < HQ; q += 256) {
+      if constexpr (VW == 4)
+        reinterpret_cast<float4 *>(dst)[q] = reinterpret_cast<const float4 *>(src)[q];
+      else
+        dst[q] = src[q];
+    }
+  }
+}
+
+int check_merge_args(const char *who, int n_sent, int beam, int K, int step, const int *limit,
+                     const float *cand_logp, const int *cand_id, const float *logp_eof,
+                     const float *prev_score, const int *tok, const int *backptr, const float *score,
+                     const int *fin_count, const int *fin_beam, const float *fin_score) {
+  if (n_sent <= 0 || beam <= 0 || K <= 0 || step < 0)
+    return lh::fail_arg("%s: n_sent=%d beam=%d K=%d step=%d", who, n_sent, beam, K, step);
+  if ((long long)beam * K > kMaxCand)
+    return lh::fail_arg("%s: beam*K=%lld exceeds %d", who, (long long)beam * K, kMaxCand);
+  if (!limit || !cand_logp || !cand_id || !logp_eof || !prev_score || !tok || !backptr || !score ||
+      !fin_count || !fin_beam || !fin_score)
+    return lh::fail_arg("%s: a required pointer is NULL", who);
+  if (score == prev_score) return lh::fail_arg("%s: score aliases prev_score", who);
+  return LH_OK;
+}
+
+// fills a (tensors, H, B_src); *vec: 16-byte copies are possible
+int check_gather_args(const char *who, const float *const *src, float *const *dst, int n_tensors,
+                      int H, int B, int B_src, GatherArgs *a, bool *vec) {
+  if (n_tensors < 1 || n_tensors > LH_GATHER_MAX_TENSORS || H <= 0 || B <= 0 || B_src <= 0 ||
+      !src || !dst)
+    return lh::fail_arg("%s: n_tensors=%d H=%d B=%d B_src=%d or NULL pointer", who, n_tensors, H,
+                        B, B_src);
+  *vec = H % 4 == 0;
+  for (int t = 0; t < n_tensors; ++t) {
+    if (!src[t] || !dst[t]) return lh::fail_arg("%s: tensor %d is NULL", who, t);
+    for (int u = 0; u < n_tensors; ++u)
+      if (dst[t] == src[u]) return lh::fail_arg("%s: dst %d aliases src %d", who, t, u);
+    a->src[t] = src[t];
+    a->dst[t] = dst[t];
+    *vec = *vec && lh::aligned16(src[t]) && lh::aligned16(dst[t]);
+  }
+  a->H = H;
+  a->B_src = B_src;
+  return LH_OK;
+}
+
 }  // namespace
 
 extern "C" int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const int *limit,
@@ -167,14 +252,11 @@ extern "C" int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const in
                                  int start_id, int eof_id, int *tok, int *backptr, float *score,
                                  int *fin_count, int *fin_beam, float *fin_score,
                                  lh_stream_t stream) {
-  if (n_sent <= 0 || beam <= 0 || K <= 0 || step < 0)
-    return lh::fail_arg("lh_beam_merge_f32: n_sent=%d beam=%d K=%d step=%d", n_sent, beam, K, step);
-  if ((long long)beam * K > kMaxCand)
-    return lh::fail_arg("lh_beam_merge_f32: beam*K=%lld exceeds %d", (long long)beam * K, kMaxCand);
-  if (!limit || !cand_logp || !cand_id || !logp_eof || !prev_score || !tok || !backptr || !score ||
-      !fin_count || !fin_beam || !fin_score)
-    return lh::fail_arg("lh_beam_merge_f32: a required pointer is NULL");
-  if (score == prev_score) return lh::fail_arg("lh_beam_merge_f32: score aliases prev_score");
+  const int rc = check_merge_args("lh_beam_merge_f32", n_sent, beam, K, step, limit, cand_logp, cand_id,
+                                  logp_eof, prev_score, tok, backptr, score, fin_count, fin_beam,
+                                  fin_score);
+  if (rc != LH_OK) return rc;
+  if (beam > kMaxBeam) return lh::fail_arg("lh_beam_merge_f32: beam=%d exceeds %d", beam, kMaxBeam);
   MergeArgs a{n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof, prev_score, diversity,
               penalty, start_id, eof_id, tok, backptr, score, fin_count, fin_beam, fin_score};
   hipLaunchKernelGGL(beam_merge_kernel, dim3(n_sent), dim3(kMergeThreads), 0,
@@ -184,22 +266,11 @@ extern "C" int lh_beam_merge_f32(int n_sent, int beam, int K, int step, const in
 
 extern "C" int lh_beam_gather_f32(const float *const *src, float *const *dst, int n_tensors, int H,
                                   int B, int B_src, const int *backptr, lh_stream_t stream) {
-  if (n_tensors < 1 || n_tensors > LH_GATHER_MAX_TENSORS || H <= 0 || B <= 0 || B_src <= 0 ||
-      !src || !dst || !backptr)
-    return lh::fail_arg("lh_beam_gather_f32: n_tensors=%d H=%d B=%d B_src=%d or NULL pointer",
-                        n_tensors, H, B, B_src);
+  if (!backptr) return lh::fail_arg("lh_beam_gather_f32: backptr is NULL");
   GatherArgs a{};
-  bool vec = H % 4 == 0;
-  for (int t = 0; t < n_tensors; ++t) {
-    if (!src[t] || !dst[t]) return lh::fail_arg("lh_beam_gather_f32: tensor %d is NULL", t);
-    for (int u = 0; u < n_tensors; ++u)
-      if (dst[t] == src[u]) return lh::fail_arg("lh_beam_gather_f32: dst %d aliases src %d", t, u);
-    a.src[t] = src[t];
-    a.dst[t] = dst[t];
-    vec = vec && lh::aligned16(src[t]) && lh::aligned16(dst[t]);
-  }
-  a.H = H;
-  a.B_src = B_src;
+  bool vec;
+  const int rc = check_gather_args("lh_beam_gather_f32", src, dst, n_tensors, H, B, B_src, &a, &vec);
+  if (rc != LH_OK) return rc;
   a.backptr = backptr;
   const int hq = vec ? H / 4 : H;
   const dim3 grid((hq + 255) / 256, B, n_tensors), block(256);
@@ -207,4 +278,35 @@ extern "C" int lh_beam_gather_f32(const float *const *src, float *const *dst, in
   if (vec) hipLaunchKernelGGL(beam_gather_kernel<4>, grid, block, 0, lh::as_stream(stream), a);
   else hipLaunchKernelGGL(beam_gather_kernel<1>, grid, block, 0, lh::as_stream(stream), a);
   return lh::check_launch("lh_beam_gather_f32");
+}
+
+extern "C" int lh_beam_merge_gather_f32(int n_sent, int beam, int K, int step, const int *limit,
+                                        const float *cand_logp, const int *cand_id,
+                                        const float *logp_eof, const float *prev_score,
+                                        float diversity, float penalty, int start_id, int eof_id,
+                                        int *tok, int *backptr, float *score, int *fin_count,
+                                        int *fin_beam, float *fin_score, const float *const *src,
+                                        float *const *dst, int n_tensors, int H,
+                                        lh_stream_t stream) {
+  const char *who = "lh_beam_merge_gather_f32";
+  int rc = check_merge_args(who, n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof,
+                            prev_score, tok, backptr, score, fin_count, fin_beam, fin_score);
+  if (rc != LH_OK) return rc;
+  if (beam > kMaxBeam) return lh::fail_arg("%s: beam=%d exceeds %d", who, beam, kMaxBeam);
+  if (n_sent > 65535) return lh::fail_arg("%s: n_sent=%d exceeds 65535", who, n_sent);
+  GatherArgs ga{};
+  bool vec;
+  rc = check_gather_args(who, src, dst, n_tensors, H, n_sent * beam, n_sent * beam, &ga, &vec);
+  if (rc != LH_OK) return rc;
+  MergeArgs a{n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof, prev_score, diversity,
+              penalty, start_id, eof_id, tok, backptr, score, fin_count, fin_beam, fin_score};
+  // enough workgroups per sentence to give every CU one (each of them repeats the merge)
+  int per = (256 + n_sent - 1) / n_sent;
+  per = per < 1 ? 1 : (per > 16 ? 16 : per);
+  const dim3 grid(per, n_sent), block(kMergeThreads);
+  if (vec)
+    hipLaunchKernelGGL(beam_merge_gather_kernel<4>, grid, block, 0, lh::as_stream(stream), a, ga, n_tensors);
+  else
+    hipLaunchKernelGGL(beam_merge_gather_kernel<1>, grid, block, 0, lh::as_stream(stream), a, ga, n_tensors);
+  return lh::check_launch(who);
 }

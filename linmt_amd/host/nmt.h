@@ -535,6 +535,10 @@ class NeuralMachineTranslation {
   void ForwardPropTarget(int curr_index, int *p_device_current_indices, int minibatch);
   // SwapDecodingStates + TargetCopyPrevStates (deep_rnn.h:1842-1872) in one gather launch.
   void SwapDecodingStates(const int *p_device_backptr, int minibatch);
+  // the (source, destination) pairs SwapDecodingStates moves: h and c of every target layer and,
+  // with input feeding, h~; returns their number
+  int DecodingStateTensors(const float **src, float **dst);
+  bool separate_beam_launches_ = false;  // measurement and test aid (LINMT_SEPARATE_BEAM_LAUNCHES)
   // EnsembleFactory::DecodeFile (decoder.h:1702-1776) for a batch of sentences (ids in ORIGINAL
   // order, ragged).  Results come back in input order.
   // `ensemble`: further models decoded in lockstep with this one (EnsembleFactory,

@@ -162,6 +162,7 @@ void NeuralMachineTranslation::InitModel() {
 void NeuralMachineTranslation::InitModelDecoding(int n_sent, int beam_size) {
   decode_mode_ = true;
   if (const char *sp = std::getenv("LINMT_SPLIT_PRODUCTS")) split_products_ = sp[0] == '1';
+  separate_beam_launches_ = std::getenv("LINMT_SEPARATE_BEAM_LAUNCHES") != nullptr;
   n_sent_ = n_sent;
   beam_size_ = beam_size;
   const int L = cfg_.num_layers_, T = cfg_.longest_sentence_, H = cfg_.lstm_size_;
@@ -590,10 +591,8 @@ void NeuralMachineTranslation::ForwardPropTarget(int curr_index, int *p_device_c
   split_step_ = false;
 }
 
-void NeuralMachineTranslation::SwapDecodingStates(const int *p_device_backptr, int minibatch) {
+int NeuralMachineTranslation::DecodingStateTensors(const float **src, float **dst) {
   const int L = cfg_.num_layers_;
-  const float *src[LH_GATHER_MAX_TENSORS];
-  float *dst[LH_GATHER_MAX_TENSORS];
   int n = 0;
   for (int l = 0; l < L; ++l) {
     LstmLayer &Lt = TargetLayer(l);
@@ -606,6 +605,13 @@ void NeuralMachineTranslation::SwapDecodingStates(const int *p_device_backptr, i
     src[n] = attention_layer_.v_nodes_[0].p_device_final_tmp_2_;
     dst[n++] = p_device_h_tild_previous_.get();
   }
+  return n;
+}
+
+void NeuralMachineTranslation::SwapDecodingStates(const int *p_device_backptr, int minibatch) {
+  const float *src[LH_GATHER_MAX_TENSORS];
+  float *dst[LH_GATHER_MAX_TENSORS];
+  const int n = DecodingStateTensors(src, dst);
   ProfileScope ps(profiler_, kTagBeamGather, 8.0 * n * cfg_.lstm_size_ * minibatch);
   LhErrorWrapper(lh_beam_gather_f32(src, dst, n, cfg_.lstm_size_, minibatch, minibatch,
                                     p_device_backptr, stream_),
@@ -960,6 +966,27 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
                      "ensemble beam top-k");
     }
     const size_t off = (size_t)step * B;
+    // One model: the merge and the move of the surviving hypotheses' states are one launch.
+    const bool merge_and_swap = n_models == 1 && step < max_limit && beam <= 256 && !separate_beam_launches_;
+    if (merge_and_swap) {
+      const float *gs[LH_GATHER_MAX_TENSORS];
+      float *gd[LH_GATHER_MAX_TENSORS];
+      const int g = DecodingStateTensors(gs, gd);
+      ProfileScope pm(profiler_, kTagBeamMergeGather, 8.0 * K * Ba + 8.0 * g * cfg_.lstm_size_ * Ba);
+      LhErrorWrapper(
+          lh_beam_merge_gather_f32(n_active, beam, K, step, d.limit_.get(), d.cand_logp_.get(),
+                                   d.cand_id_.get(), d.logp_eof_.get(),
+                                   step == 0 ? d.score_[0].get() : d.score_hist_.get() + off - B,
+                                   o.diversity_, o.penalty_, Decoder::start_symbol_,
+                                   Decoder::end_symbol_, d.tok_hist_.get() + off,
+                                   d.backptr_hist_.get() + off, d.score_hist_.get() + off,
+                                   d.fin_count_hist_.get() + (size_t)step * n,
+                                   d.fin_beam_hist_.get() + off, d.fin_score_hist_.get() + off, gs, gd,
+                                   g, cfg_.lstm_size_, stream_),
+          "beam merge and state swap");
+      p_device_step_indices = d.tok_hist_.get() + off;
+      continue;
+    }
     {
       ProfileScope pm(profiler_, kTagBeamMerge, 8.0 * K * Ba);
       LhErrorWrapper(

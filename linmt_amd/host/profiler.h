@@ -33,6 +33,7 @@ enum ProfileTag {
   kTagEmbedGrad,
   kTagUpdate,
   kTagSplitPack,  // fp32 -> three bf16 planes, for the products on the bf16 matrix pipe
+  kTagBeamMergeGather,  // merge and state gather of a step in one launch
   kTagCount
 };
 
@@ -42,7 +43,7 @@ inline const char *ProfileTagName(int t) {
                                          "xent", "beam_topk", "beam_merge", "beam_gather",
                                          "error_gemm", "weight_grad_gemm", "lstm_cell_bwd",
                                          "attn_bwd", "softmax_grad", "row_sum", "embed_grad",
-                                         "update", "split_pack"};
+                                         "update", "split_pack", "beam_merge_gather"};
   return t >= 0 && t < kTagCount ? names[t] : "";
 }
 

@@ -121,6 +121,11 @@ SIGNATURES = {
                                     c_i32p, c_f32p, c_i32p, c_i32p, c_f32p, C.c_void_p]),
     "lh_beam_gather_f32": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int,
                                      C.c_int, C.c_int, C.c_int, c_i32p, C.c_void_p]),
+    "lh_beam_merge_gather_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, c_i32p, c_f32p, c_i32p,
+                                           c_f32p, c_f32p, C.c_float, C.c_float, C.c_int, C.c_int,
+                                           c_i32p, c_i32p, c_f32p, c_i32p, c_i32p, c_f32p,
+                                           C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int,
+                                           C.c_int, C.c_void_p]),
     "lh_softmax_xent_grad_f32": (C.c_int, [c_f32p, C.c_int, c_f32p, C.c_int, C.c_int, c_i32p,
                                            c_i32p, c_f32p, C.c_int, c_f64p, c_f64p, C.c_void_p]),
     "lh_uniform_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_ulonglong, C.c_void_p]),
@@ -462,6 +467,20 @@ def beam_gather(src, dst, H, B, backptr, B_src=None, stream=None):
     d = (C.c_void_p * n)(*[t.data_ptr() for t in dst])
     check(load().lh_beam_gather_f32(s, d, n, H, B, B_src, _ptr(backptr), _stream(stream)),
           "lh_beam_gather_f32")
+
+
+def beam_merge_gather(n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof, prev_score,
+                      diversity, penalty, start_id, eof_id, tok, backptr, score, fin_count, fin_beam,
+                      fin_score, src, dst, H, stream=None):
+    n = len(src)
+    s = (C.c_void_p * n)(*[t.data_ptr() for t in src])
+    d = (C.c_void_p * n)(*[t.data_ptr() for t in dst])
+    check(load().lh_beam_merge_gather_f32(n_sent, beam, K, step, _ptr(limit), _ptr(cand_logp),
+                                          _ptr(cand_id), _ptr(logp_eof), _ptr(prev_score), diversity,
+                                          penalty, start_id, eof_id, _ptr(tok), _ptr(backptr),
+                                          _ptr(score), _ptr(fin_count), _ptr(fin_beam),
+                                          _ptr(fin_score), s, d, n, H, _stream(stream)),
+          "lh_beam_merge_gather_f32")
 
 
 # ---- training half ------------------------------------------------------------------------------

@@ -736,7 +736,7 @@ namespace {
 void attention_step(orc_model *m, int B, const float *h_t, const float *hs, long long step_stride,
                     long long col_stride, const int *hs_col, int hs_steps, const int *batch_info,
                     const int *mask01, int max_len, float *h_tild, std::vector<int> *out_indices = nullptr,
-                    std::vector<float> *out_align = nullptr) {
+                    std::vector<float> *out_align = nullptr, std::vector<float> *out_pt = nullptr) {
   const int H = m->cfg.H;
   const int D = m->cfg.attention == 1 ? m->cfg.D : -1;
   const int W = D >= 0 ? 2 * D + 1 : max_len;
@@ -753,6 +753,7 @@ void attention_step(orc_model *m, int B, const float *h_t, const float *hs, long
                     sig.data(), ind.data(), al.data(), ce.data(), cx.data(), nullptr);
   if (out_indices) *out_indices = ind;
   if (out_align) *out_align = al;
+  if (out_pt) *out_pt = pt;
   mat_apply(m, "attn.W_c1", H, H, cx.data(), B, t1.data());
   mat_apply(m, "attn.W_c2", H, H, h_t, B, t2.data());
   const float *b_out = m->params["attn.b_out"].data();
@@ -780,6 +781,11 @@ struct DecodeTrace {
   int *tok, *backptr;
   float *score, *margin;
   int cap_steps, steps;
+  // optional, one value per step: how far the closest window position p_t of the step's live
+  // columns was from an integer (the window is cut at (int)p_t, LowerUpperKernel
+  // deep_rnn_kernel.h:1095-1098, so two fp32 evaluations of a p_t that close to an integer may
+  // read different windows); 0.5 when the model has no local-p attention
+  float *window_margin = nullptr;
 };
 
 int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
@@ -811,8 +817,10 @@ extern "C" int orc_decode_sentence_trace(orc_model *m, const int *src_ids, int S
                                          const orc_decode_opts *o, int *best_tokens, int cap,
                                          int *best_len, float *best_score, int *trace_tok,
                                          int *trace_backptr, float *trace_score,
-                                         float *trace_margin, int cap_steps, int *n_steps) {
+                                         float *trace_margin, int cap_steps, int *n_steps,
+                                         float *trace_window_margin) {
   DecodeTrace tr{trace_tok, trace_backptr, trace_score, trace_margin, cap_steps, 0};
+  tr.window_margin = trace_window_margin;
   const int rc = decode_impl(&m, 1, src_ids, S, o, false, best_tokens, cap, best_len, best_score,
                              nullptr, nullptr, nullptr, 0, nullptr, nullptr, &tr);
   *n_steps = tr.steps;
@@ -948,8 +956,10 @@ int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
   std::vector<float> sc(B), fin_score(B);
   std::vector<const float *> dists(num_models);
   for (int k = 0; k < num_models; ++k) dists[k] = runs[k].dist.data();
+  float step_window_margin = 0.5f;  // of the last forward_target call
 
   auto forward_target = [&](int curr_index) {
+    step_window_margin = 0.5f;
     for (Run &r : runs) {
       orc_model *m = r.m;
       const orc_model_config &cfg = m->cfg;
@@ -970,10 +980,13 @@ int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
       const float *top = r.cur[L - 1].h.data();
       if (cfg.attention) {
         std::vector<int> ind;
-        std::vector<float> al;
+        std::vector<float> al, pt;
         attention_step(m, B, top, r.top_states.data(), H, 0, hs_col.data(), S, batch_info.data(),
-                       ones.data(), S, r.h_tild.data(), &ind, &al);
+                       ones.data(), S, r.h_tild.data(), &ind, &al, &pt);
         top = r.h_tild.data();
+        if (cfg.attention == 1)
+          for (int b = 0; b < (curr_index == 0 ? 1 : B); ++b)  // step 0: the columns are copies
+            step_window_margin = std::min(step_window_margin, std::fabs(pt[b] - std::nearbyint(pt[b])));
         if (unk_mode) {
           // layer_attention.h:360-385: scores of the window's valid slots, zero elsewhere
           std::fill(r.ascore.begin(), r.ascore.end(), 0.f);
@@ -1030,6 +1043,7 @@ int decode_impl(orc_model *const *ms, int num_models, const int *src_ids, int S,
       trace->margin[curr_index] =
           orc_beam_step_margin(dists.data(), num_models, V, B, curr_index, top_scores.data(),
                                o->diversity, start_symbol, end_symbol);
+      if (trace->window_margin) trace->window_margin[curr_index] = step_window_margin;
       trace->steps = curr_index + 1;
     }
     // bookkeeping of decoder.h:436-479

@@ -126,11 +126,17 @@ int orc_decode_sentence(orc_model *m, const int *src_ids, int S, const orc_decod
 float orc_beam_step_margin(const float *const *p, int num_models, int V, int beam, int step,
                            const float *prev_score, float diversity, int start_id, int eof_id);
 /* orc_decode_sentence that also records the beam after every expansion step (beam tokens,
- * beam-local back-pointers and scores per step) and the step's orc_beam_step_margin. */
+ * beam-local back-pointers and scores per step) and the step's orc_beam_step_margin.
+ * trace_window_margin (may be NULL), one value per step: the smallest distance of a live column's
+ * window position p_t from an integer -- the local-p window is cut at (int)p_t
+ * (LowerUpperKernel, src/deep_rnn_kernel.h:1095-1098), so two fp32 evaluations of a p_t that
+ * close to an integer may read windows one position apart; 0.5 for models without local-p
+ * attention. */
 int orc_decode_sentence_trace(orc_model *m, const int *src_ids, int S, const orc_decode_opts *o,
                               int *best_tokens, int cap, int *best_len, float *best_score,
                               int *trace_tok, int *trace_backptr, float *trace_score,
-                              float *trace_margin, int cap_steps, int *n_steps);
+                              float *trace_margin, int cap_steps, int *n_steps,
+                              float *trace_window_margin);
 
 /* The same with the reference's unk_replacement_mode__ on: alignment scores exported at every
  * step, Viterbi alignments carried by the hypotheses, coverage penalty on the real scores.

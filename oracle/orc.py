@@ -365,7 +365,9 @@ class Model:
                               diversity=0.0, lp_alpha=0.65, cp_beta=0.20, num_threads=0):
         """decode_sentence plus the beam after every expansion step: dict(best, best_score, steps,
         tok (n, beam), backptr (n, beam; beam-local), score (n, beam), margin (n,)) where margin is
-        the smallest gap between two candidates the step had to order (orc_beam_step_margin)."""
+        the smallest gap between two candidates the step had to order (orc_beam_step_margin) and
+        window_margin (n,) the smallest distance of a live column's local-p window position from
+        an integer."""
         src_ids = i32(src_ids)
         cap = self.cfg.longest_sent + 2
         b = min(beam, int(np.sqrt(self.cfg.V_tgt)))
@@ -377,17 +379,18 @@ class Model:
         bp = np.zeros((cap, b), np.int32)
         sc = np.zeros((cap, b), np.float32)
         mg = np.zeros(cap, np.float32)
+        wm = np.zeros(cap, np.float32)
         f = lib().orc_decode_sentence_trace
         f.restype = C.c_int
         f.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int,
-                      C.c_void_p, C.c_void_p] + [C.c_void_p] * 4 + [C.c_int, C.c_void_p]
+                      C.c_void_p, C.c_void_p] + [C.c_void_p] * 4 + [C.c_int, C.c_void_p, C.c_void_p]
         steps = f(self.handle, _p(src_ids), src_ids.size, C.byref(o), _p(best), cap,
                   C.byref(blen), C.byref(bscore), _p(tok), _p(bp), _p(sc), _p(mg), cap,
-                  C.byref(nst))
+                  C.byref(nst), _p(wm))
         n = nst.value
         return dict(best=best[:blen.value].copy(), best_score=float(bscore.value), steps=steps,
                     tok=tok[:n].copy(), backptr=bp[:n].copy(), score=sc[:n].copy(),
-                    margin=mg[:n].copy())
+                    margin=mg[:n].copy(), window_margin=wm[:n].copy())
 
     def forward_xent(self, src, tgt_in, tgt_out, batch_info, num_threads=0):
         """src (B,S), tgt_in/tgt_out (B,T) int arrays with -1 padding (column t = timestep t)."""

@@ -832,6 +832,47 @@ def test_beam_gather(lh, orc):
         lh.beam_gather(ds, ds, H, B, dev(bp))  # in place is rejected
 
 
+@pytest.mark.parametrize("n_sent,beam,H,n", [(64, 12, 1000, 9), (5, 12, 1000, 9), (300, 4, 36, 3),
+                                            (3, 7, 130, 24), (1, 1, 8, 1)])
+def test_beam_merge_gather_equals_the_two_calls(lh, n_sent, beam, H, n):
+    """lh_beam_merge_gather_f32 against lh_beam_merge_f32 + lh_beam_gather_f32, bit for bit, at
+    step 0 (one live column per sentence), on expanding, finishing and idle sentences, with
+    <START> / <EOF> among the candidates; unaligned tensors take the scalar copy."""
+    rng = np.random.default_rng(n_sent * 131 + beam)
+    B, K = n_sent * beam, beam + 1
+    for step in (0, 3):
+        limit = rng.integers(2, 6, size=n_sent).astype(np.int32)          # < , == and > step 3
+        cl = np.sort(uni(rng, K, B, s=3.0), axis=0)[::-1]                  # (K, B): best first per column
+        ci = rng.integers(0, 50, size=(K, B)).astype(np.int32)             # 0 = <START>, 1 = <EOF>
+        prev = uni(rng, B, s=5.0)
+        le = uni(rng, B, s=2.0)
+        srcs = [dev(uni(rng, H, B)) for _ in range(n)]
+        if H % 4:                                                          # and one unaligned base
+            srcs[0] = dev(uni(rng, H * B + 1, 1))[1:]
+        args = (n_sent, beam, K, step, dev(limit), dev(cl), dev(ci), dev(le), dev(prev), 0.1, 0.05, 0, 1)
+
+        def outputs():
+            return [torch.full((B,), -7, dtype=torch.int32, device="cuda"),
+                    torch.full((B,), -7, dtype=torch.int32, device="cuda"),
+                    torch.full((B,), 7.0, device="cuda"),
+                    torch.full((n_sent,), -7, dtype=torch.int32, device="cuda"),
+                    torch.full((B,), -7, dtype=torch.int32, device="cuda"),
+                    torch.full((B,), 7.0, device="cuda")]
+        o1, o2 = outputs(), outputs()
+        d1 = [torch.full((H * B,), 3.0, device="cuda") for _ in range(n)]
+        d2 = [torch.full((H * B,), 3.0, device="cuda") for _ in range(n)]
+        lh.beam_merge(*args, *o1)
+        lh.beam_gather(srcs, d1, H, B, o1[1])
+        lh.beam_merge_gather(*args, *o2, srcs, d2, H)
+        torch.cuda.synchronize()
+        for a, b, what in zip(o1, o2, ("tok", "backptr", "score", "fin_count", "fin_beam", "fin_score")):
+            assert torch.equal(a, b), f"step {step}: {what}"
+        for t, (a, b) in enumerate(zip(d1, d2)):
+            assert torch.equal(a, b), f"step {step}: tensor {t}"
+    with pytest.raises(lh.LinmtHipError):
+        lh.beam_merge_gather(*args, *o2, srcs, srcs, H)                    # in place is rejected
+
+
 def test_full_size_softmax_properties(lh):
     """Config-3 size (V=30000, B=768): too large for the CPU oracle in a unit test, so checked
     through size-independent properties: columns sum to 1, shift invariance, argmax preserved,

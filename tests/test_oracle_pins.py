@@ -329,6 +329,29 @@ def test_decode_sentence_trace_matches_plain_decode(orc):
     assert any(h.tolist() == want for h, _ in plain["hyps"])
 
 
+def test_decode_trace_window_margin_closed_form(orc):
+    """The traced decode's window margin against a closed form: with v_p = 0 every window position
+    is p_t = S * sigmoid(0) = S / 2, so the margin is 0 for an even source length and 0.5 for an odd
+    one at every step; with real weights it lies in [0, 0.5] and differs between steps; a model
+    without local-p attention reports 0.5."""
+    rng = np.random.default_rng(79)
+    P, m = _tiny_model(orc, rng)
+    P0 = dict(P)
+    P0["attn.v_p"] = np.zeros_like(P["attn.v_p"])
+    m.set_params(P0)
+    for S, want in ((6, 0.0), (7, 0.5)):
+        tr = m.decode_sentence_trace(rng.integers(0, 30, size=S), beam=4)
+        assert tr["window_margin"].shape == tr["margin"].shape
+        assert np.all(tr["window_margin"] == want), (S, tr["window_margin"])
+    m.set_params(P)
+    tr = m.decode_sentence_trace(rng.integers(0, 30, size=9), beam=4)
+    wm = tr["window_margin"]
+    assert np.all((wm >= 0) & (wm <= 0.5)) and len(set(wm.tolist())) > 1
+    g = orc.Model(2, 12, 30, 37, attention=2, D=0, feed_input=1, longest_sent=40)
+    g.set_params(P)
+    assert np.all(g.decode_sentence_trace(rng.integers(0, 30, size=5), beam=4)["window_margin"] == 0.5)
+
+
 def test_beam_gather_composition(orc):
     rng = np.random.default_rng(10)
     x = rng.standard_normal((5, 6)).astype(np.float32)
