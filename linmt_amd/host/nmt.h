@@ -538,7 +538,6 @@ class NeuralMachineTranslation {
   // the (source, destination) pairs SwapDecodingStates moves: h and c of every target layer and,
   // with input feeding, h~; returns their number
   int DecodingStateTensors(const float **src, float **dst);
-  bool separate_beam_launches_ = false;  // measurement and test aid (LINMT_SEPARATE_BEAM_LAUNCHES)
   // EnsembleFactory::DecodeFile (decoder.h:1702-1776) for a batch of sentences (ids in ORIGINAL
   // order, ragged).  Results come back in input order.
   // `ensemble`: further models decoded in lockstep with this one (EnsembleFactory,

@@ -162,7 +162,6 @@ void NeuralMachineTranslation::InitModel() {
 void NeuralMachineTranslation::InitModelDecoding(int n_sent, int beam_size) {
   decode_mode_ = true;
   if (const char *sp = std::getenv("LINMT_SPLIT_PRODUCTS")) split_products_ = sp[0] == '1';
-  separate_beam_launches_ = std::getenv("LINMT_SEPARATE_BEAM_LAUNCHES") != nullptr;
   n_sent_ = n_sent;
   beam_size_ = beam_size;
   const int L = cfg_.num_layers_, T = cfg_.longest_sentence_, H = cfg_.lstm_size_;
@@ -913,6 +912,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
 
   std::vector<int> active_at(max_limit + 1);
   int *p_device_step_indices = d.current_indices_.get();  // <START> for every column
+  const bool separate_beam_launches = getenv("LINMT_SEPARATE_BEAM_LAUNCHES") != nullptr;  // measurement and test aid
   for (int step = 0; step <= max_limit; ++step) {
     int n_active = 0;
     while (n_active < n && limit[n_active] >= step) ++n_active;  // limits are non-increasing
@@ -967,7 +967,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
     }
     const size_t off = (size_t)step * B;
     // One model: the merge and the move of the surviving hypotheses' states are one launch.
-    const bool merge_and_swap = n_models == 1 && step < max_limit && beam <= 256 && !separate_beam_launches_;
+    const bool merge_and_swap = n_models == 1 && step < max_limit && beam <= 256 && !separate_beam_launches;
     if (merge_and_swap) {
       const float *gs[LH_GATHER_MAX_TENSORS];
       float *gd[LH_GATHER_MAX_TENSORS];

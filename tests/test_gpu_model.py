@@ -235,6 +235,31 @@ def test_decode_same_with_and_without_the_regrouped_step(orc, host, monkeypatch)
     gm.close()
 
 
+def test_decode_same_with_separate_beam_launches(orc, host, monkeypatch):
+    """The merge and the state swap of a step as one launch (lh_beam_merge_gather_f32, the default
+    with one model) and as the two launches it replaces (LINMT_SEPARATE_BEAM_LAUNCHES=1): the same
+    kernels' arithmetic, so every token, score and hypothesis is equal bit for bit."""
+    rng = np.random.default_rng(23)
+    layers, H, Vs, Vt, D, beam = 2, 64, 150, 170, 3, 5
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 40, 0.35, decoding=(6, beam))
+    sents = [rng.integers(0, Vs, size=n) for n in (14, 3, 9, 20, 6, 11)]
+    gm.profile(2)
+    one = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    assert "beam_merge_gather" in gm.profile_totals(), "the single launch did not run"
+    monkeypatch.setenv("LINMT_SEPARATE_BEAM_LAUNCHES", "1")
+    gm.profile(2)
+    two = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    assert "beam_gather" in gm.profile_totals() and "beam_merge_gather" not in gm.profile_totals()
+    monkeypatch.delenv("LINMT_SEPARATE_BEAM_LAUNCHES")
+    gm.profile(0)
+    for i, (a, b) in enumerate(zip(one, two)):
+        assert a["best"].tolist() == b["best"].tolist() and a["best_score"] == b["best_score"], i
+        assert a["n_hyp"] == b["n_hyp"] and a["steps"] == b["steps"], i
+        for (ta, sa), (tb, sb) in zip(a["hyps"], b["hyps"]):
+            assert ta.tolist() == tb.tolist() and sa == sb, i
+    gm.close()
+
+
 def test_decode_same_with_grouped_gate_products(orc, host, monkeypatch):
     """LINMT_GROUPED_GATES=1 issues what the previous step fixes of every layer's gate product as
     one grouped launch (lh_gate_gemm_group_f32) and leaves M*h of the layer below on the chain.
