@@ -165,6 +165,20 @@ int lh_gate_gemm_lstm_cell_f32(int H, int B, const lh_gemm_seg *segs, int nseg, 
                                const float *c_prev, const int *mask01, int sigmoid_f64,
                                float cell_clip, float *c, float *h, size_t workspace_bytes,
                                lh_stream_t stream);
+/* The same kernel in the training form of the same reference code (the forward half of
+ * src/node_input_to_hidden.h:218-636 and src/node_hidden_to_hidden.h:194-444 with train on): it also
+ * stores what the backward pass and the layer above need, exactly as lh_lstm_cell_fwd_f32 does:
+ *   gates  (4H x B, ld 4H, optional) receives i, f, g, o
+ *   h_drop (H x B, optional)  = (next_drop_mask < keep) * (1/keep) * h
+ * No addend_col (training looks embeddings up).  Same condition on when it runs
+ * (lh_gate_gemm_lstm_cell_plan), same aliasing rules; gates and h_drop must not overlap an X
+ * operand either. */
+int lh_gate_gemm_lstm_cell_train_f32(int H, int B, const lh_gemm_seg *segs, int nseg,
+                                     const float *addend, int ld_addend, const float *bias4h,
+                                     const float *c_prev, const int *mask01, int sigmoid_f64,
+                                     float cell_clip, float *gates, float *c, float *h,
+                                     const float *next_drop_mask, float keep, float *h_drop,
+                                     size_t workspace_bytes, lh_stream_t stream);
 /* Several stacked gate products of one step in ONE launch (no counterpart in the reference, which
  * issues every layer's 8-12 SGEMMs one after the other, src/node_input_to_hidden.h:297-556,
  * src/node_hidden_to_hidden.h:248-386).  While decoding, what a step needs from the previous one is

@@ -328,15 +328,30 @@ void LstmNode::ForwardProp() {
   const bool drop_out = M.apply_dropout_ && L.out_dropout_;
   const float cell_clip = M.cfg_.clip_cell_mode_ ? M.cfg_.cell_clip_threshold_ : 0.f;
 
-  // Inference form (no gate values kept, no dropout): product and cell in ONE kernel whenever the
-  // product runs unsplit; the folded embedding table is then read by that kernel too.
-  if (!p_device_gates_ && !drop_out) {
+  // Product and cell in ONE kernel whenever the product runs unsplit; in the inference form (no
+  // gate values kept, no dropout) the folded embedding table is read by that kernel too, the
+  // training form also stores the gate values and the dropped copy of h for the layer above.
+  {
     int fusable = 0;
     char name[160] = {0};
     LhErrorWrapper(lh_gate_gemm_lstm_cell_plan(H, B, segs, nseg, beta != 0.f, M.gemm_ws_bytes_, &fusable,
                                                name, sizeof(name)),
                    "lh_gate_gemm_lstm_cell_plan");
-    if (fusable) {
+    if (fusable && (p_device_gates_ || drop_out) && !folded) {
+      double k = 0;
+      for (int i = 0; i < nseg; ++i) k += segs[i].K;
+      ProfileScope ps(M.profiler_, kTagGateGemm, name, 2.0 * 4 * H * (double)B * k);
+      LhErrorWrapper(lh_gate_gemm_lstm_cell_train_f32(
+                         H, B, segs, nseg, beta != 0.f ? pre : nullptr, 4 * H, L.p_device_b_stack_.get(),
+                         p_device_c_t_prev_, p_device_input_vocab_indices_01_, feed ? 1 : 0, cell_clip,
+                         p_device_gates_, p_device_c_t_, p_device_h_t_,
+                         drop_out ? p_device_out_dropout_mask_ : nullptr,
+                         drop_out ? M.cfg_.dropout_rate_ : 1.f, drop_out ? p_device_h_t_dropped_ : nullptr,
+                         M.gemm_ws_bytes_, s),
+                     "LstmNode::ForwardPropGpu gate product with cell (training form)");
+      return;
+    }
+    if (fusable && !p_device_gates_ && !drop_out) {
       double k = 0;
       for (int i = 0; i < nseg; ++i) k += segs[i].K;
       ProfileScope ps(M.profiler_, kTagGateGemm, name, 2.0 * 4 * H * (double)B * k);

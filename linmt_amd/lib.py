@@ -70,6 +70,10 @@ SIGNATURES = {
     "lh_gate_gemm_lstm_cell_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, c_f32p,
                                              C.c_int, c_i32p, C.c_int, c_f32p, c_f32p, c_i32p, C.c_int,
                                              C.c_float, c_f32p, c_f32p, C.c_size_t, C.c_void_p]),
+    "lh_gate_gemm_lstm_cell_train_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int,
+                                                   c_f32p, C.c_int, c_f32p, c_f32p, c_i32p, C.c_int,
+                                                   C.c_float, c_f32p, c_f32p, c_f32p, c_f32p,
+                                                   C.c_float, c_f32p, C.c_size_t, C.c_void_p]),
     "lh_gate_gemm_group_plan": (C.c_int, [C.c_int, C.c_int, C.POINTER(GateProblem), C.c_int,
                                           C.POINTER(C.c_int), C.c_char_p, C.c_int]),
     "lh_gate_gemm_group_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GateProblem), C.c_int,
@@ -297,6 +301,17 @@ def gate_gemm_lstm_cell(H, B, segs, bias4h, c_prev, mask01, c, h, addend=None, l
                                             _ptr(mask01), int(sigmoid_f64), cell_clip, _ptr(c),
                                             _ptr(h), workspace_bytes, _stream(stream)),
           "lh_gate_gemm_lstm_cell_f32")
+
+
+def gate_gemm_lstm_cell_train(H, B, segs, bias4h, c_prev, mask01, c, h, gates=None, addend=None,
+                              ld_addend=0, sigmoid_f64=False, cell_clip=0.0, next_drop_mask=None,
+                              keep=1.0, h_drop=None, workspace_bytes=0, stream=None):
+    check(load().lh_gate_gemm_lstm_cell_train_f32(H, B, _segs(segs), len(segs), _ptr(addend), ld_addend,
+                                                  _ptr(bias4h), _ptr(c_prev), _ptr(mask01),
+                                                  int(sigmoid_f64), cell_clip, _ptr(gates), _ptr(c),
+                                                  _ptr(h), _ptr(next_drop_mask), keep, _ptr(h_drop),
+                                                  workspace_bytes, _stream(stream)),
+          "lh_gate_gemm_lstm_cell_train_f32")
 
 
 def _gate_problems(problems):

@@ -282,6 +282,72 @@ def test_lstm_cell_fwd(lh, orc, H, B, feed):
     assert_close(host(h, (H, B)), wh2, "h clip")
 
 
+@pytest.mark.parametrize("H,B,Ks,addend,f64,clip,keep", [
+    (100, 76, (100, 36), False, False, 0.0, 0.8),
+    (36, 40, (68,), True, True, 0.0, 1.0),
+    (248, 132, (64, 64, 32), True, False, 0.4, 0.7),
+    (2048, 256, (256, 128), True, True, 0.0, 0.8),
+])
+def test_gate_gemm_lstm_cell_training_form(lh, orc, H, B, Ks, addend, f64, clip, keep):
+    """lh_gate_gemm_lstm_cell_train_f32 for every tile configuration that can carry the cell:
+    gates, c, h against the oracle's cell on float64 pre-activations, h_drop against its closed
+    form, and everything bit for bit against lh_gemm_f32 + lh_lstm_cell_fwd_f32 under the same
+    configuration."""
+    rng = np.random.default_rng(H + B)
+    L = lh.load()
+    As = [uni(rng, 4 * H, K, s=0.3) for K in Ks]
+    Xs = [uni(rng, K, B) for K in Ks]
+    bias, c_prev = uni(rng, 4 * H, s=0.5), uni(rng, H, B)
+    mask = (rng.uniform(size=B) < 0.8).astype(np.int32)
+    add_np = uni(rng, 4 * H, B) if addend else None
+    drop = rng.uniform(size=(H, B)).astype(np.float32) if keep < 1.0 else None
+    segs = [(dev(A), 4 * H, dev(X), K, K) for A, X, K in zip(As, Xs, Ks)]
+    pre = sum(A.astype(np.float64) @ X for A, X in zip(As, Xs))
+    if addend:
+        pre = pre + add_np
+    wg, wc, wh = orc.lstm_cell_fwd(pre.astype(np.float32), bias, c_prev, mask, feed=f64, cell_clip=clip)
+    d_bias, d_mask = dev(bias), dev(mask)
+    d_drop = None if drop is None else dev(drop)
+    n_cfg = L.lh_gemm_set_config_override(-1)
+    ran = 0
+    try:
+        for cfg in list(range(n_cfg)) + [-1]:
+            L.lh_gemm_set_config_override(cfg)
+            ok, name = lh.gate_gemm_lstm_cell_plan(H, B, segs, has_addend=addend)
+            if not ok:
+                continue
+            ran += 1
+            what = f"config {cfg} ({name}) H={H} B={B} K={Ks}"
+            c = dev(c_prev)                                    # in place
+            h = torch.full((H * B,), float("nan"), device="cuda")
+            g = torch.full((4 * H * B,), float("nan"), device="cuda")
+            hd = None if drop is None else torch.full((H * B,), float("nan"), device="cuda")
+            lh.gate_gemm_lstm_cell_train(H, B, segs, d_bias, c, d_mask, c, h, gates=g,
+                                         addend=None if not addend else dev(add_np), ld_addend=4 * H,
+                                         sigmoid_f64=f64, cell_clip=clip, next_drop_mask=d_drop,
+                                         keep=keep, h_drop=hd)
+            assert_close(host(g, (4 * H, B)), wg, what + " gates")
+            assert_close(host(c, (H, B)), wc, what + " c")
+            assert_close(host(h, (H, B)), wh, what + " h")
+            if drop is not None:
+                want = ((drop < np.float32(keep)).astype(np.float32) * (np.float32(1.0) / np.float32(keep))) * host(h, (H, B))
+                assert np.array_equal(host(hd, (H, B)), want), what + " h_drop"
+            # the two-call path under the same configuration
+            p2 = dev(add_np) if addend else torch.empty(4 * H * B, device="cuda")
+            lh.gemm(4 * H, B, segs, p2, 4 * H, beta=1.0 if addend else 0.0)
+            c2, h2 = dev(c_prev), torch.empty(H * B, device="cuda")
+            g2 = torch.empty(4 * H * B, device="cuda")
+            hd2 = None if drop is None else torch.empty(H * B, device="cuda")
+            lh.lstm_cell_fwd(H, B, p2, d_bias, c2, d_mask, c2, h2, sigmoid_f64=f64, cell_clip=clip,
+                             gates=g2, next_drop_mask=d_drop, keep=keep, h_drop=hd2)
+            if cfg >= 0 or lh.gemm_kernel_name(4 * H, B, segs).split("<")[1] == name.split("<")[1]:
+                for a, b, w in ((g, g2, "gates"), (c, c2, "c"), (h, h2, "h")) + (((hd, hd2, "h_drop"),) if hd is not None else ()):
+                    assert torch.equal(a, b), what + f" {w} vs the two calls"
+    finally:
+        L.lh_gemm_set_config_override(-1)
+    assert ran >= 5
+
+
 def test_gate_gemm_group(lh, orc):
     """lh_gate_gemm_group_f32: one launch holding a cell problem (two K segments, the addend read
     through a column index, in-place cell state) and plain problems of another depth.  Under a
