@@ -395,14 +395,21 @@ def bench_training(torch, host, steps, warmup, small, split=False):
 
     for _ in range(warmup):
         step()
-    m.profile(2)
+    m.profile(0)
     torch.cuda.synchronize()
     t0 = time.time()
     for _ in range(steps):
         ll, nrm = step()
     torch.cuda.synchronize()
     dt = (time.time() - t0) / steps
+    # the per-site table comes from further, untimed minibatches with every launch bracketed by
+    # events (the brackets cost about 10 us of idle GPU per launch, 6-8% of such a minibatch)
+    m.profile(2)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
     tot = m.profile_totals()
+    m.profile(0)
     rows = []
     for k, v in sorted(tot.items(), key=lambda kv: -kv[1]["ms"]):
         is_gemm = "|" in k
