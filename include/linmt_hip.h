@@ -326,7 +326,13 @@ int lh_gemm_split_set_config_override(int config);
  *   gates  (4H x B, optional) receives i,f,g,o for the backward pass
  *   h_drop (H x B, optional)  = (next_drop_mask < keep) * (1/keep) * h
  * ld of every 4H x B operand is 4H, of every H x B operand H.  c may alias c_prev.
+ * mask01[b] is 0 or 1; with LH_MASK_F32_GATES added to it, column b takes the fp32 sigmoids even
+ * when sigmoid_f64 != 0 (a decoder that runs columns at different steps in one launch: the
+ * reference evaluates the first step of a sentence with the plain kernels and every later one with
+ * the Feed kernels, src/node_input_to_hidden.h:350-621).  lh_gate_gemm_lstm_cell_f32 reads its mask
+ * the same way.
  */
+#define LH_MASK_F32_GATES 2
 int lh_lstm_cell_fwd_f32(int H, int B, const float *pre1, const float *pre2, const float *pre3,
                          const float *bias4h, const float *c_prev, const int *mask01,
                          int sigmoid_f64, float cell_clip, float *gates, float *c, float *h,
@@ -504,6 +510,39 @@ int lh_beam_merge_gather_f32(int n_sent, int beam, int K, int step, const int *l
                              int eof_id, int *tok, int *backptr, float *score, int *fin_count,
                              int *fin_beam, float *fin_score, const float *const *src,
                              float *const *dst, int n_tensors, int H, lh_stream_t stream);
+
+/* A decoder that keeps every beam column busy (no counterpart in the reference, whose
+ * Decoder works on one sentence at a time): the beam columns of a sentence ("slot") are handed to
+ * the next sentence of the input as soon as the sentence has taken its last step, so the sentences
+ * in flight are at different steps.
+ *
+ * lh_beam_merge_gather_stream_f32 is lh_beam_merge_gather_f32 with sentence s at step
+ * tick - start[s] (limit[s] counts from the sentence's own first step; a slot without a sentence
+ * has limit -1 and idles).
+ *
+ * lh_stream_admit_f32 puts n_adm <= LH_STREAM_ADMIT_MAX sentences into slots, in one launch.  For
+ * admission q (a HOST array): start[slot] = tick, limit[slot] = limit; for the slot's beam columns
+ * c: hs_col[c] = hs_col_value, batch_info[c] = len, batch_info[B + c] = off (either array may be
+ * NULL), tok_prev[c] = start_id, score_prev[c] = 0; dst_t[:, c] = src_t[:, sentence_col] for the
+ * n_tensors state tensors (src_t is H x n_src: the encoder's final states, what
+ * TransferDecodingStatesGpu broadcasts, src/layer_input_to_hidden.h:1536-1545) and zero_t[:, c] = 0
+ * for the n_zero tensors that start a sentence at zero (h~ of the step before).  src / dst / zero
+ * are HOST arrays of device pointers. */
+#define LH_STREAM_ADMIT_MAX 16
+typedef struct {
+  int slot, sentence_col, hs_col_value, len, off, limit, tick;
+} lh_stream_admission;
+int lh_beam_merge_gather_stream_f32(int n_sent, int beam, int K, int tick, const int *start,
+                                    const int *limit, const float *cand_logp, const int *cand_id,
+                                    const float *logp_eof, const float *prev_score, float diversity,
+                                    float penalty, int start_id, int eof_id, int *tok, int *backptr,
+                                    float *score, int *fin_count, int *fin_beam, float *fin_score,
+                                    const float *const *src, float *const *dst, int n_tensors, int H,
+                                    lh_stream_t stream);
+int lh_stream_admit_f32(const lh_stream_admission *adm, int n_adm, int beam, int B, int *start,
+                        int *limit, int *hs_col, int *batch_info, const float *const *src,
+                        float *const *dst, int n_tensors, float *const *zero, int n_zero, int H,
+                        int n_src, int *tok_prev, int start_id, float *score_prev, lh_stream_t stream);
 
 /* ==========================================================================================
  * Training half of the path (backward pass and update).

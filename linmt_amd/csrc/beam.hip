@@ -21,6 +21,9 @@ struct MergeArgs {
   float *score;
   int *fin_count, *fin_beam;
   float *fin_score;
+  // optional: sentence s is at step `step - start[s]` (a decoder whose sentences start at different
+  // ticks); NULL = every sentence is at `step`
+  const int *start;
 };
 
 // One workgroup merges one sentence.  Candidates are ranked by counting how many others precede
@@ -42,8 +45,9 @@ __device__ __forceinline__ void merge_sentence(const MergeArgs &a, const int s, 
   const int beam = a.beam, K = a.K;
   const int c0 = s * beam;  // first global column of this sentence
   const int limit = a.limit[s];
+  const int step = a.start ? a.step - a.start[s] : a.step;
 
-  if (a.step >= limit) {
+  if (step >= limit) {
     // finish (== limit) or idle (> limit): no expansion.
     for (int i = tid; i < beam; i += kMergeThreads) {
       s_bp[i] = c0 + i;
@@ -51,18 +55,18 @@ __device__ __forceinline__ void merge_sentence(const MergeArgs &a, const int s, 
       a.tok[c0 + i] = a.eof_id;
       a.backptr[c0 + i] = c0 + i;
       float sc = a.prev_score[c0 + i];
-      if (a.step == limit) {
+      if (step == limit) {
         sc = sc + (a.logp_eof[c0 + i] + a.penalty);  // decoder.h:506 adds (log p + penalty)
         a.fin_beam[c0 + i] = i;
         a.fin_score[c0 + i] = sc;
       }
       a.score[c0 + i] = sc;
     }
-    if (tid == 0 && write) a.fin_count[s] = a.step == limit ? beam : 0;
+    if (tid == 0 && write) a.fin_count[s] = step == limit ? beam : 0;
     return;
   }
 
-  const int cols = a.step == 0 ? 1 : beam;
+  const int cols = step == 0 ? 1 : beam;
   const int C = cols * K;
   if (tid < 2) s_total[tid] = 0;
   for (int e = tid; e < C; e += kMergeThreads) {
@@ -208,6 +212,51 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_gather_kernel(const 
   }
 }
 
+// A decoder that keeps its beam columns busy: a finished sentence's columns ("slot") are handed to
+// the next sentence.  One launch admits up to LH_STREAM_ADMIT_MAX sentences: blockIdx.y = admission,
+// blockIdx.x = (tensor, beam column) -- the encoder's final state of the sentence into every column
+// of the slot, zeros into the tensors that start at zero -- and the first block of an admission also
+// writes the slot's entries of the small arrays.
+struct AdmitArgs {
+  lh_stream_admission adm[LH_STREAM_ADMIT_MAX];
+  int beam, B, H, n_src, n_tensors, n_zero, start_id;
+  int *start, *limit, *hs_col, *batch_info, *tok_prev;
+  float *score_prev;
+  const float *src[LH_GATHER_MAX_TENSORS];
+  float *dst[LH_GATHER_MAX_TENSORS];
+  float *zero[LH_GATHER_MAX_TENSORS];
+};
+
+__global__ __launch_bounds__(256) void stream_admit_kernel(const AdmitArgs a) {
+  const lh_stream_admission q = a.adm[blockIdx.y];
+  const int t = blockIdx.x / a.beam, j = blockIdx.x % a.beam;
+  const int c = q.slot * a.beam + j;  // the column
+  if (t < a.n_tensors) {
+    const float *src = a.src[t] + (size_t)q.sentence_col * a.H;
+    float *dst = a.dst[t] + (size_t)c * a.H;
+    for (int i = threadIdx.x; i < a.H; i += 256) dst[i] = src[i];
+  } else {
+    float *dst = a.zero[t - a.n_tensors] + (size_t)c * a.H;
+    for (int i = threadIdx.x; i < a.H; i += 256) dst[i] = 0.f;
+  }
+  if (blockIdx.x == 0) {
+    if (threadIdx.x == 0) {
+      a.start[q.slot] = q.tick;
+      a.limit[q.slot] = q.limit;
+    }
+    for (int i = threadIdx.x; i < a.beam; i += 256) {
+      const int cc = q.slot * a.beam + i;
+      if (a.hs_col) a.hs_col[cc] = q.hs_col_value;
+      if (a.batch_info) {
+        a.batch_info[cc] = q.len;
+        a.batch_info[a.B + cc] = q.off;
+      }
+      a.tok_prev[cc] = a.start_id;
+      a.score_prev[cc] = 0.f;
+    }
+  }
+}
+
 int check_merge_args(const char *who, int n_sent, int beam, int K, int step, const int *limit,
                      const float *cand_logp, const int *cand_id, const float *logp_eof,
                      const float *prev_score, const int *tok, const int *backptr, const float *score,
@@ -280,6 +329,15 @@ extern "C" int lh_beam_gather_f32(const float *const *src, float *const *dst, in
   return lh::check_launch("lh_beam_gather_f32");
 }
 
+namespace {
+int merge_gather(const char *who, int n_sent, int beam, int K, int step, const int *start,
+                 const int *limit, const float *cand_logp, const int *cand_id, const float *logp_eof,
+                 const float *prev_score, float diversity, float penalty, int start_id, int eof_id,
+                 int *tok, int *backptr, float *score, int *fin_count, int *fin_beam,
+                 float *fin_score, const float *const *src, float *const *dst, int n_tensors, int H,
+                 lh_stream_t stream);
+}
+
 extern "C" int lh_beam_merge_gather_f32(int n_sent, int beam, int K, int step, const int *limit,
                                         const float *cand_logp, const int *cand_id,
                                         const float *logp_eof, const float *prev_score,
@@ -288,7 +346,70 @@ extern "C" int lh_beam_merge_gather_f32(int n_sent, int beam, int K, int step, c
                                         int *fin_beam, float *fin_score, const float *const *src,
                                         float *const *dst, int n_tensors, int H,
                                         lh_stream_t stream) {
-  const char *who = "lh_beam_merge_gather_f32";
+  return merge_gather("lh_beam_merge_gather_f32", n_sent, beam, K, step, nullptr, limit, cand_logp,
+                      cand_id, logp_eof, prev_score, diversity, penalty, start_id, eof_id, tok, backptr,
+                      score, fin_count, fin_beam, fin_score, src, dst, n_tensors, H, stream);
+}
+
+extern "C" int lh_beam_merge_gather_stream_f32(int n_sent, int beam, int K, int tick, const int *start,
+                                               const int *limit, const float *cand_logp,
+                                               const int *cand_id, const float *logp_eof,
+                                               const float *prev_score, float diversity,
+                                               float penalty, int start_id, int eof_id, int *tok,
+                                               int *backptr, float *score, int *fin_count,
+                                               int *fin_beam, float *fin_score,
+                                               const float *const *src, float *const *dst,
+                                               int n_tensors, int H, lh_stream_t stream) {
+  if (!start) return lh::fail_arg("lh_beam_merge_gather_stream_f32: start is NULL");
+  return merge_gather("lh_beam_merge_gather_stream_f32", n_sent, beam, K, tick, start, limit, cand_logp,
+                      cand_id, logp_eof, prev_score, diversity, penalty, start_id, eof_id, tok, backptr,
+                      score, fin_count, fin_beam, fin_score, src, dst, n_tensors, H, stream);
+}
+
+extern "C" int lh_stream_admit_f32(const lh_stream_admission *adm, int n_adm, int beam, int B,
+                                   int *start, int *limit, int *hs_col, int *batch_info,
+                                   const float *const *src, float *const *dst, int n_tensors,
+                                   float *const *zero, int n_zero, int H, int n_src, int *tok_prev,
+                                   int start_id, float *score_prev, lh_stream_t stream) {
+  const char *who = "lh_stream_admit_f32";
+  if (!adm || n_adm < 1 || n_adm > LH_STREAM_ADMIT_MAX || beam < 1 || B < beam || H < 1 || n_src < 1)
+    return lh::fail_arg("%s: n_adm=%d beam=%d B=%d H=%d n_src=%d", who, n_adm, beam, B, H, n_src);
+  if (n_tensors < 0 || n_tensors > LH_GATHER_MAX_TENSORS || n_zero < 0 || n_zero > LH_GATHER_MAX_TENSORS ||
+      n_tensors + n_zero < 1)
+    return lh::fail_arg("%s: n_tensors=%d n_zero=%d", who, n_tensors, n_zero);
+  if (!start || !limit || !tok_prev || !score_prev || (n_tensors && (!src || !dst)) || (n_zero && !zero))
+    return lh::fail_arg("%s: a required pointer is NULL", who);
+  AdmitArgs a{};
+  for (int i = 0; i < n_adm; ++i) {
+    const lh_stream_admission &q = adm[i];
+    if (q.slot < 0 || (q.slot + 1) * beam > B || q.sentence_col < 0 || q.sentence_col >= n_src)
+      return lh::fail_arg("%s: admission %d: slot %d / sentence column %d out of range", who, i, q.slot,
+                          q.sentence_col);
+    a.adm[i] = q;
+  }
+  a.beam = beam, a.B = B, a.H = H, a.n_src = n_src, a.n_tensors = n_tensors, a.n_zero = n_zero;
+  a.start_id = start_id, a.start = start, a.limit = limit, a.hs_col = hs_col, a.batch_info = batch_info;
+  a.tok_prev = tok_prev, a.score_prev = score_prev;
+  for (int t = 0; t < n_tensors; ++t) {
+    if (!src[t] || !dst[t]) return lh::fail_arg("%s: tensor %d is NULL", who, t);
+    a.src[t] = src[t], a.dst[t] = dst[t];
+  }
+  for (int t = 0; t < n_zero; ++t) {
+    if (!zero[t]) return lh::fail_arg("%s: zero tensor %d is NULL", who, t);
+    a.zero[t] = zero[t];
+  }
+  hipLaunchKernelGGL(stream_admit_kernel, dim3((n_tensors + n_zero) * beam, n_adm), dim3(256), 0,
+                     lh::as_stream(stream), a);
+  return lh::check_launch(who);
+}
+
+namespace {
+int merge_gather(const char *who, int n_sent, int beam, int K, int step, const int *start,
+                 const int *limit, const float *cand_logp, const int *cand_id, const float *logp_eof,
+                 const float *prev_score, float diversity, float penalty, int start_id, int eof_id,
+                 int *tok, int *backptr, float *score, int *fin_count, int *fin_beam,
+                 float *fin_score, const float *const *src, float *const *dst, int n_tensors, int H,
+                 lh_stream_t stream) {
   int rc = check_merge_args(who, n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof,
                             prev_score, tok, backptr, score, fin_count, fin_beam, fin_score);
   if (rc != LH_OK) return rc;
@@ -299,7 +420,7 @@ extern "C" int lh_beam_merge_gather_f32(int n_sent, int beam, int K, int step, c
   rc = check_gather_args(who, src, dst, n_tensors, H, n_sent * beam, n_sent * beam, &ga, &vec);
   if (rc != LH_OK) return rc;
   MergeArgs a{n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof, prev_score, diversity,
-              penalty, start_id, eof_id, tok, backptr, score, fin_count, fin_beam, fin_score};
+              penalty, start_id, eof_id, tok, backptr, score, fin_count, fin_beam, fin_score, start};
   // enough workgroups per sentence to give every CU one (each of them repeats the merge)
   int per = (256 + n_sent - 1) / n_sent;
   per = per < 1 ? 1 : (per > 16 ? 16 : per);
@@ -310,3 +431,4 @@ extern "C" int lh_beam_merge_gather_f32(int n_sent, int beam, int K, int step, c
     hipLaunchKernelGGL(beam_merge_gather_kernel<1>, grid, block, 0, lh::as_stream(stream), a, ga, n_tensors);
   return lh::check_launch(who);
 }
+}  // namespace

@@ -329,11 +329,13 @@ __attribute__((amdgpu_waves_per_eu(split_waves_per_simd<BM, BN, WK, CELL>()))) v
       const floatx4 *cp = reinterpret_cast<const floatx4 *>(g.c_prev + (size_t)n * H + r);
       const floatx4 c0 = cp[0], c1 = cp[1];
       const float cprev[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-      const float mask = (float)g.colmask[n];
+      const int cm = g.colmask[n];
+      const float mask = (float)(cm & 1);
+      const bool f64 = g.sigmoid_f64 && !(cm & LH_MASK_F32_GATES);
       float c[8], h[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        if (g.sigmoid_f64)
+        if (f64)
           lh::lstm_cell_point<true>(pre[0][j], pre[1][j], pre[2][j], pre[3][j], cprev[j], mask, g.cell_clip, c[j], h[j]);
         else
           lh::lstm_cell_point<false>(pre[0][j], pre[1][j], pre[2][j], pre[3][j], cprev[j], mask, g.cell_clip, c[j], h[j]);

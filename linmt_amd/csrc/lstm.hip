@@ -69,13 +69,19 @@ __global__ __launch_bounds__(256) void lstm_cell_fwd_kernel(const CellFwdArgs a)
   }
   Vec<VW> cp;
   cp.load(a.c_prev + o1);
-  const float m = (float)a.mask01[b];
+  const int cm = a.mask01[b];
+  const float m = (float)(cm & 1);
+  const bool f32_gates = (cm & LH_MASK_F32_GATES) != 0;
 
   Vec<VW> c, h;
 #pragma unroll
   for (int i = 0; i < VW; ++i) {
-    lh::lstm_cell_point<F64>(s[0].v[i], s[1].v[i], s[2].v[i], s[3].v[i], cp.v[i], m, a.cell_clip,
-                             c.v[i], h.v[i]);
+    if (F64 && f32_gates)
+      lh::lstm_cell_point<false>(s[0].v[i], s[1].v[i], s[2].v[i], s[3].v[i], cp.v[i], m, a.cell_clip,
+                                 c.v[i], h.v[i]);
+    else
+      lh::lstm_cell_point<F64>(s[0].v[i], s[1].v[i], s[2].v[i], s[3].v[i], cp.v[i], m, a.cell_clip,
+                               c.v[i], h.v[i]);
   }
   if (a.gates) {
 #pragma unroll

@@ -109,6 +109,10 @@ def load():
         lib.lnmt_decode_batch.argtypes[1:]
     lib.lnmt_decode_history.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
                                         C.c_int, C.POINTER(C.c_int)]
+    lib.lnmt_decode_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                       C.POINTER(DecodeOptions), C.c_void_p, C.c_int, C.c_void_p,
+                                       C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.c_int, C.c_void_p, C.POINTER(C.c_int)]
     lib.lnmt_model_stream.restype = C.c_void_p
     lib.lnmt_model_stream.argtypes = [C.c_void_p]
     lib.lnmt_set_split_products.argtypes = [C.c_void_p, C.c_int, C.c_int]
@@ -414,6 +418,45 @@ class Model:
             r["kbest"] = [(int(a), float(b)) for a, b in zip(kidx[i], kscore[i]) if a >= 0]
             res.append(r)
         return res
+
+
+def _decode_stream(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0, diversity=0.0,
+                   lp_alpha=0.65, cp_beta=0.20, with_hyps=False, hyp_cap=256):
+    """DecodeStream: any number of sentences through the model's n_sent slots of beam columns, a
+    finished sentence's slot going to the next sentence.  Results as decode_batch, in the order of
+    `sentences`; self.stream_ticks = steps taken in all."""
+    n = len(sentences)
+    lengths = np.array([len(s) for s in sentences], np.int32)
+    flat = np.ascontiguousarray(np.concatenate([np.asarray(s, np.int32) for s in sentences]))
+    cap = self.cfg.longest_sentence + 2
+    o = DecodeOptions(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta, 0, 1)
+    best = np.zeros((n, cap), np.int32)
+    blen = np.zeros(n, np.int32)
+    bscore = np.zeros(n, np.float32)
+    steps = np.zeros(n, np.int32)
+    nh = np.zeros(n, np.int32)
+    ht = hl = hs = None
+    if with_hyps:
+        ht = np.zeros((n, hyp_cap, cap), np.int32)
+        hl = np.zeros((n, hyp_cap), np.int32)
+        hs = np.zeros((n, hyp_cap), np.float32)
+    ticks = C.c_int(0)
+    _check(load().lnmt_decode_stream(self.handle, _p(flat), _p(lengths), n, C.byref(o), _p(best), cap,
+                                     _p(blen), _p(bscore), _p(steps), _p(ht), _p(hl), _p(hs), hyp_cap,
+                                     _p(nh), C.byref(ticks)), "decode_stream")
+    self.stream_ticks = ticks.value
+    res = []
+    for i in range(n):
+        r = dict(best=best[i, :blen[i]].copy(), best_score=float(bscore[i]), steps=int(steps[i]),
+                 n_hyp=int(nh[i]))
+        if with_hyps:
+            k = min(int(nh[i]), hyp_cap)
+            r["hyps"] = [(ht[i, j, :hl[i, j]].copy(), float(hs[i, j])) for j in range(k)]
+        res.append(r)
+    return res
+
+
+Model.decode_stream = _decode_stream
 
 
 def decoding(model_file, source_file, final_file, ids_file=None, beam=12, penalty=0.0,

@@ -270,7 +270,7 @@ extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_model
                                           int hyp_cap, int *n_hyp, int *best_viterbi,
                                           int *kbest_index, float *kbest_score) {
   return Guard([&] {
-    if (!models || n_models < 1 || !models[0]) throw LinmtError("no model");
+    if (!models || (n_models < 1 && n_models != -1) || !models[0]) throw LinmtError("no model");
     lnmt_model *m = models[0];
     std::vector<NeuralMachineTranslation *> others;
     for (int k = 1; k < n_models; ++k) {
@@ -295,7 +295,10 @@ extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_model
     d.unk_replacement_mode_ = o->unk_replacement_mode != 0;
     d.hypotheses_number_ = std::max(1, o->num_hypotheses);
     std::vector<SentenceResult> res;
-    m->nmt->DecodeBatch(sents, d, &res, others);
+    if (n_models == -1)  // lnmt_decode_stream
+      m->nmt->DecodeStream(sents, d, &res);
+    else
+      m->nmt->DecodeBatch(sents, d, &res, others);
     for (int i = 0; i < n; ++i) {
       const SentenceResult &r = res[i];
       const int bl = std::min((int)r.best.size(), cap);
@@ -325,6 +328,18 @@ extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_model
       }
     }
   });
+}
+
+extern "C" int lnmt_decode_stream(lnmt_model *m, const int *sentences, const int *lengths, int n,
+                                  const lnmt_decode_options *o, int *best, int cap, int *best_len,
+                                  float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
+                                  float *hyp_score, int hyp_cap, int *n_hyp, int *ticks) {
+  // n_models = -1 selects DecodeStream inside the shared marshalling
+  const int rc = lnmt_decode_batch_ensemble(&m, -1, sentences, lengths, n, o, best, cap, best_len, best_score,
+                                            steps, hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, nullptr,
+                                            nullptr, nullptr);
+  if (rc == 0 && ticks) *ticks = m->nmt->stream_ticks_;
+  return rc;
 }
 
 extern "C" void *lnmt_model_stream(lnmt_model *m) { return m->nmt->stream_; }

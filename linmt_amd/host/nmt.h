@@ -551,6 +551,14 @@ class NeuralMachineTranslation {
                    std::vector<SentenceResult> *results,
                    const std::vector<NeuralMachineTranslation *> &ensemble = {},
                    const std::vector<std::vector<std::vector<int>>> &ensemble_sentences = {});
+  // The same search over any number of sentences with every beam column kept busy: a sentence
+  // that has taken its last step hands its beam columns to the next sentence of the list, so the
+  // sentences in flight are at different steps (nmt_stream.cc).  One model, local-p attention,
+  // no alignment export.  Every sentence goes through the steps DecodeBatch takes it through.
+  void DecodeStream(const std::vector<std::vector<int>> &sentences, const DecodeOptions &o,
+                    std::vector<SentenceResult> *results);
+  const int *stream_layer0_mask_ = nullptr;  // DecodeStream: the first target layer's column mask of this tick
+  int stream_ticks_ = 0;                     // steps the last DecodeStream took
 
   // ---- training --------------------------------------------------------------------------------
   DeviceArray<double> p_device_norm_workspace_, p_device_norms_;

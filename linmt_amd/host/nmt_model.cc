@@ -505,7 +505,8 @@ void NeuralMachineTranslation::ForwardPropTarget(int curr_index, int *p_device_c
     n.minibatch_size_ = minibatch;
     n.recurrent_hoisted_ = false;
     if (l == 0)
-      n.UpdateVectorsForwardGpu(p_device_current_indices, p_device_ones_.get(),
+      n.UpdateVectorsForwardGpu(p_device_current_indices,
+                                stream_layer0_mask_ ? const_cast<int *>(stream_layer0_mask_) : p_device_ones_.get(),
                                 Lt.p_device_h_t_previous_.get(), Lt.p_device_c_t_previous_.get());
     else
       n.UpdateVectorsForwardGpu(p_device_ones_.get(), Lt.p_device_h_t_previous_.get(),

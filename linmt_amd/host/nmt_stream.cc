@@ -1,0 +1,310 @@
+// NeuralMachineTranslation::DecodeStream: beam search over a list of sentences with every beam
+// column kept busy.  DecodeBatch starts a batch's sentences together and lets them end one by
+// one, so its products shrink from n_sent*beam columns to beam columns over a batch; here a
+// sentence that has taken its last step hands its beam columns ("slot") to the next sentence of
+// the list, so every step runs n_sent*beam columns until the list runs out.  Every sentence goes
+// through exactly the steps DecodeBatch (and Decoder::ExpandHypothesis, src/decoder.h:355-525)
+// takes it through; only which sentences share a launch differs.
+//
+// The number of steps of a sentence is fixed by its length (decoder.h:1734), so the whole
+// schedule -- which sentence enters which slot at which tick, and when a group of sentences has
+// to be encoded -- is laid out on the host before the first launch, and nothing is read back
+// until the end.  Sentences are encoded in groups of up to n_sent (ForwardPropSource as in
+// DecodeBatch); what decoding needs of a group -- the projected attention memories W_a*hs and
+// W_c1*hs and the encoder's final states -- is kept in one of kRing slabs until the group's last
+// sentence has finished.
+#include <algorithm>
+#include <cmath>
+#include <numeric>
+
+#include "nmt.h"
+
+namespace linmt {
+
+namespace {
+constexpr int kRing = 4;  // groups whose encoder outputs are held at once
+
+struct Admission {
+  int sentence, group, column, slot, tick, limit;
+};
+}  // namespace
+
+void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> &sentences,
+                                            const DecodeOptions &o,
+                                            std::vector<SentenceResult> *results) {
+  if (!decode_mode_) throw LinmtError("DecodeStream: call InitModelDecoding first");
+  if (!cfg_.attention_mode_ || !attention_layer_.ProjectedMemoryPossible())
+    throw LinmtError("DecodeStream: needs local-p attention over a projected memory");
+  if (o.unk_replacement_mode_) throw LinmtError("DecodeStream: alignment export is not supported");
+  const int n = (int)sentences.size(), L = cfg_.num_layers_, H = cfg_.lstm_size_;
+  int beam = o.beam_size_;
+  if (beam > (int)std::sqrt((double)cfg_.target_vocab_size_))  // decoder.h:1662-1664
+    beam = (int)std::sqrt((double)cfg_.target_vocab_size_);
+  if (n < 1 || beam != beam_size_) throw LinmtError("DecodeStream: beam does not match InitModelDecoding");
+  if (2 * L + 1 > LH_GATHER_MAX_TENSORS) throw LinmtError("DecodeStream: too many layers");
+  const int longest = cfg_.longest_sentence_, slots = n_sent_, B = slots * beam, K = beam + 1;
+  for (const auto &w : sentences)
+    if (w.empty() || (int)w.size() > longest) throw LinmtError("DecodeStream: source sentence length out of range");
+
+  // ---- groups: n_sent sentences each, in input order; inside a group longest first ---------------
+  const int G = (n + slots - 1) / slots;
+  std::vector<std::vector<int>> group_order(G);  // encoder column -> sentence
+  std::vector<int> group_S(G), limit(n);
+  for (int g = 0; g < G; ++g) {
+    std::vector<int> &ord = group_order[g];
+    for (int i = g * slots; i < std::min(n, (g + 1) * slots); ++i) ord.push_back(i);
+    std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return sentences[a].size() > sentences[b].size(); });
+    group_S[g] = (int)sentences[ord[0]].size();
+  }
+  for (int i = 0; i < n; ++i)
+    limit[i] = std::min((int)(o.max_decoding_ratio_ * (int)sentences[i].size()), longest - 2);  // decoder.h:1734
+
+  // ---- the schedule -----------------------------------------------------------------------------------
+  std::vector<Admission> adm;                       // in admission order
+  std::vector<std::vector<int>> adm_at, encode_at;  // per tick: indices into adm / groups to encode
+  std::vector<int> free_at(slots, 0), group_done(G, 0), start_of(n, 0), slot_of(n, 0);
+  {
+    int g = 0, k = 0, tick = 0, encoded = 0;
+    while (g < G) {
+      if ((int)adm_at.size() <= tick) adm_at.resize(tick + 1), encode_at.resize(tick + 1);
+      for (int s = 0; s < slots && g < G; ++s) {
+        if (free_at[s] > tick) continue;
+        if (g >= encoded) {
+          // the group's slab is free once the group that held it has finished completely (all of
+          // that group's sentences were admitted before this one, so its last tick is known)
+          if (g >= kRing && group_done[g - kRing] > tick) break;
+          encode_at[tick].push_back(g);
+          encoded = g + 1;
+        }
+        const int i = group_order[g][k];
+        adm_at[tick].push_back((int)adm.size());
+        adm.push_back(Admission{i, g, k, s, tick, limit[i]});
+        start_of[i] = tick, slot_of[i] = s;
+        free_at[s] = tick + limit[i] + 1;  // steps 0 .. limit
+        group_done[g] = std::max(group_done[g], free_at[s]);
+        if (++k == (int)group_order[g].size()) ++g, k = 0;
+      }
+      ++tick;
+    }
+  }
+  const int ticks = *std::max_element(free_at.begin(), free_at.end());
+  adm_at.resize(ticks), encode_at.resize(ticks);
+
+  // ---- device state of the stream ------------------------------------------------------------------
+  // rows of the histories: row t+1 is written by tick t, row t holds what tick t reads (tokens
+  // chosen and path scores of the tick before; a fresh slot's entries are set by its admission)
+  DeviceArray<int> tok_hist, bp_hist, fcount_hist, fbeam_hist, start_dev, limit_dev, mask_table;
+  DeviceArray<float> score_hist, fscore_hist, finals;
+  const size_t rows = (size_t)ticks + 1;
+  tok_hist.Alloc(rows * B), bp_hist.Alloc(rows * B), score_hist.Alloc(rows * B);
+  fcount_hist.Alloc((size_t)ticks * slots), fbeam_hist.Alloc((size_t)ticks * B), fscore_hist.Alloc((size_t)ticks * B);
+  start_dev.Alloc(slots), limit_dev.Alloc(slots);
+  const size_t final_slab = (size_t)2 * L * H * slots;  // [layer][h, c][H x n_sent]
+  finals.Alloc(final_slab * kRing);
+  // what the first target layer reads as its column mask: 1, and for a feed-input model
+  // 1 + LH_MASK_F32_GATES on a sentence's first step (the reference runs that step through the
+  // kernels without the feed terms, node_input_to_hidden.h:325-621)
+  std::vector<int> mask_host((size_t)ticks * B, 1), minus_one(slots, -1), zeros(slots, 0);
+  if (cfg_.feed_input_mode_)
+    for (const Admission &a : adm)
+      for (int j = 0; j < beam; ++j) mask_host[(size_t)a.tick * B + (size_t)a.slot * beam + j] = 1 + LH_MASK_F32_GATES;
+  mask_table.Alloc(mask_host.size());
+  // host arrays that asynchronous copies read or write: declared before the guard, so however this
+  // function is left the stream has drained before any of them is destroyed
+  std::vector<std::vector<int>> src_blocks(G);  // the encoder's id block of every group
+  std::vector<int> tok, bp, fcount, fbeam, binfo0(2 * (size_t)B, 0);
+  std::vector<float> fscore, bscore;
+  std::fill(binfo0.begin(), binfo0.begin() + B, 1);  // length 1, offset 0: a column without a sentence
+  struct Restore {
+    NeuralMachineTranslation &m;
+    int B;
+    ~Restore() {
+      // DecodeBatch reads the encoder states of column b's sentence through hs_col[b] = b / beam
+      (void)hipMemcpyAsync(m.attention_layer_.p_device_hs_col_.get(), m.p_device_sentence_of_column_.get(),
+                           sizeof(int) * B, hipMemcpyDeviceToDevice, m.stream_);
+      (void)hipStreamSynchronize(m.stream_);
+      m.stream_layer0_mask_ = nullptr;
+    }
+  } restore{*this, B};
+  mask_table.Upload(mask_host.data(), mask_host.size(), stream_);
+  start_dev.Upload(zeros.data(), slots, stream_);
+  limit_dev.Upload(minus_one.data(), slots, stream_);
+  tok_hist.Zero(stream_);  // a slot that never held a sentence feeds <START> = 0
+  score_hist.Zero(stream_);
+
+  // the attention memories of kRing groups side by side: slab r starts T_cap * n_sent columns
+  // after slab 0, which an entry of hs_col can express
+  AttentionLayer &A = attention_layer_;
+  const size_t slab_floats = SourceLayer(L - 1).h_all_.size();
+  const long long T_cap = (long long)(slab_floats / ((size_t)H * slots));
+  if (A.score_mem_.size() < slab_floats * kRing) {
+    A.score_mem_.Alloc(slab_floats * kRing);
+    A.ctx_mem_.Alloc(slab_floats * kRing);
+  }
+  A.hs_step_stride_ = (long long)H * slots;
+  A.hs_steps_ = (int)T_cap;
+  A.projected_memory_ = true;
+  // every column points at valid memory from the first tick on, sentence or not
+  A.PreprocessMinibatchInformation(binfo0.data(), B);
+  HipErrorWrapper(hipMemcpyAsync(A.p_device_hs_col_.get(), p_device_sentence_of_column_.get(), sizeof(int) * B,
+                                 hipMemcpyDeviceToDevice, stream_),
+                  "DecodeStream: hs_col initialisation failed");
+  if (p_device_h_tild_previous_.size()) p_device_h_tild_previous_.Zero(stream_);
+
+  const float *state_src[LH_GATHER_MAX_TENSORS];
+  float *state_dst[LH_GATHER_MAX_TENSORS], *zero_dst[1];
+  const float *swap_src[LH_GATHER_MAX_TENSORS];
+  float *swap_dst[LH_GATHER_MAX_TENSORS];
+  const int n_swap = DecodingStateTensors(swap_src, swap_dst);
+  for (int l = 0; l < L; ++l) {
+    state_dst[2 * l] = TargetLayer(l).p_device_h_t_previous_.get();
+    state_dst[2 * l + 1] = TargetLayer(l).p_device_c_t_previous_.get();
+  }
+  const bool has_tild = cfg_.feed_input_mode_ && p_device_h_tild_previous_.size();
+  zero_dst[0] = has_tild ? p_device_h_tild_previous_.get() : nullptr;
+
+  for (int t = 0; t < ticks; ++t) {
+    // ---- groups whose first sentence enters at this tick: encode them ---------------------------
+    for (int g : encode_at[t]) {
+      const std::vector<int> &ord = group_order[g];
+      const int ng = (int)ord.size(), S = group_S[g], r = g % kRing;
+      std::vector<int> &src_block = src_blocks[g];
+      src_block.assign((size_t)ng * S, -1);  // reversed, left-padded (input_file_preprocess.cc:633)
+      for (int k = 0; k < ng; ++k) {
+        const std::vector<int> &w = sentences[ord[k]];
+        const int len = (int)w.size();
+        for (int q = 0; q < len; ++q) src_block[(size_t)(S - len + q) * ng + k] = w[len - 1 - q];
+      }
+      ForwardPropSource(src_block.data(), S, ng);
+      const int cols = slots * S;  // the encoder's slices hold n_sent columns per step
+      lh_gemm_seg sa{A.p_device_w_a_.get(), H, A.p_device_total_hs_, H, H};
+      Gemm(kTagAttnProjGemm, H, cols, &sa, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
+           A.score_mem_.get() + slab_floats * r, H, "DecodeStream W_a hs");
+      lh_gemm_seg sc{A.p_device_w_c_p1_.get(), H, A.p_device_total_hs_, H, H};
+      Gemm(kTagAttnOutGemm, H, cols, &sc, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
+           A.ctx_mem_.get() + slab_floats * r, H, "DecodeStream W_c1 hs");
+      for (int l = 0; l < L; ++l) {
+        const LstmNode &last = SourceLayer(l).v_nodes_[S - 1];
+        float *dst = finals.get() + final_slab * r + (size_t)2 * l * H * slots;
+        HipErrorWrapper(hipMemcpyAsync(dst, last.p_device_h_t_, sizeof(float) * H * ng, hipMemcpyDeviceToDevice, stream_),
+                        "DecodeStream: copy of the encoder's final h failed");
+        HipErrorWrapper(hipMemcpyAsync(dst + (size_t)H * slots, last.p_device_c_t_, sizeof(float) * H * ng,
+                                       hipMemcpyDeviceToDevice, stream_),
+                        "DecodeStream: copy of the encoder's final c failed");
+      }
+    }
+    // ---- sentences that enter at this tick --------------------------------------------------------
+    const std::vector<int> &now = adm_at[t];
+    for (size_t at = 0; at < now.size();) {
+      // one launch per group of the ring (the state tensors of a launch come from one slab)
+      lh_stream_admission q[LH_STREAM_ADMIT_MAX];
+      const int r = adm[now[at]].group % kRing;
+      int m = 0;
+      while (at < now.size() && m < LH_STREAM_ADMIT_MAX && adm[now[at]].group % kRing == r) {
+        const Admission &a = adm[now[at++]];
+        const int len = (int)sentences[a.sentence].size();
+        q[m++] = lh_stream_admission{a.slot, a.column, (int)(a.column + r * T_cap * slots), len,
+                                     group_S[a.group] - len, a.limit, a.tick};
+      }
+      for (int l = 0; l < L; ++l) {
+        state_src[2 * l] = finals.get() + final_slab * r + (size_t)2 * l * H * slots;
+        state_src[2 * l + 1] = state_src[2 * l] + (size_t)H * slots;
+      }
+      LhErrorWrapper(lh_stream_admit_f32(q, m, beam, B, start_dev.get(), limit_dev.get(),
+                                         A.p_device_hs_col_.get(), A.p_device_batch_information_.get(),
+                                         state_src, state_dst, 2 * L, zero_dst, has_tild ? 1 : 0, H, slots,
+                                         tok_hist.get() + (size_t)t * B, Decoder::start_symbol_,
+                                         score_hist.get() + (size_t)t * B, stream_),
+                     "DecodeStream admission");
+    }
+    // ---- one step of every slot ------------------------------------------------------------------------
+    stream_layer0_mask_ = mask_table.get() + (size_t)t * B;
+    ForwardPropTarget(1, tok_hist.get() + (size_t)t * B, B);
+    stream_layer0_mask_ = nullptr;
+    {
+      ProfileScope ps(profiler_, kTagBeamTopK, 4.0 * cfg_.target_vocab_size_ * B);
+      LhErrorWrapper(lh_beam_topk_f32(softmax_layer_.GetDistPtr(), cfg_.target_vocab_size_, nullptr,
+                                      cfg_.target_vocab_size_, B, K, Decoder::end_symbol_,
+                                      decoder_.cand_logp_.get(), decoder_.cand_id_.get(),
+                                      decoder_.logp_eof_.get(), stream_),
+                     "DecodeStream beam top-k");
+    }
+    {
+      ProfileScope pm(profiler_, kTagBeamMergeGather, 8.0 * K * B + 8.0 * n_swap * H * B);
+      LhErrorWrapper(lh_beam_merge_gather_stream_f32(
+                         slots, beam, K, t, start_dev.get(), limit_dev.get(), decoder_.cand_logp_.get(),
+                         decoder_.cand_id_.get(), decoder_.logp_eof_.get(), score_hist.get() + (size_t)t * B,
+                         o.diversity_, o.penalty_, Decoder::start_symbol_, Decoder::end_symbol_,
+                         tok_hist.get() + (size_t)(t + 1) * B, bp_hist.get() + (size_t)(t + 1) * B,
+                         score_hist.get() + (size_t)(t + 1) * B, fcount_hist.get() + (size_t)t * slots,
+                         fbeam_hist.get() + (size_t)t * B, fscore_hist.get() + (size_t)t * B, swap_src,
+                         swap_dst, n_swap, H, stream_),
+                     "DecodeStream beam merge and state swap");
+    }
+  }
+
+  // ---- one read-back -----------------------------------------------------------------------------------
+  tok.resize(rows * B), bp.resize(rows * B), bscore.resize(rows * B);
+  fcount.resize((size_t)ticks * slots), fbeam.resize((size_t)ticks * B), fscore.resize((size_t)ticks * B);
+  tok_hist.Download(tok.data(), tok.size(), stream_);
+  bp_hist.Download(bp.data(), bp.size(), stream_);
+  score_hist.Download(bscore.data(), bscore.size(), stream_);
+  fcount_hist.Download(fcount.data(), fcount.size(), stream_);
+  fbeam_hist.Download(fbeam.data(), fbeam.size(), stream_);
+  fscore_hist.Download(fscore.data(), fscore.size(), stream_);
+  Synchronize();
+  profiler_.Collect();
+
+  // ---- hypotheses by walking the back-pointers, as DecodeBatch does ---------------------------------
+  results->assign(n, SentenceResult());
+  int max_limit = 0;
+  for (int i = 0; i < n; ++i) {
+    SentenceResult &r = (*results)[i];
+    const int t0 = start_of[i], c0 = slot_of[i] * beam, s = slot_of[i];
+    r.steps = limit[i] + 1;
+    max_limit = std::max(max_limit, limit[i]);
+    auto prefix = [&](int step, int column, Hypothesis *h) {
+      h->tokens.assign(step + 1, Decoder::start_symbol_);
+      int col = column;
+      for (int q = step - 1; q >= 0; --q) {
+        h->tokens[q + 1] = tok[(size_t)(t0 + q + 1) * B + col];
+        col = bp[(size_t)(t0 + q + 1) * B + col];
+      }
+    };
+    for (int step = 0; step <= limit[i]; ++step) {
+      const int nf = fcount[(size_t)(t0 + step) * slots + s];
+      for (int f = 0; f < nf; ++f) {
+        Hypothesis h;
+        const int parent = c0 + fbeam[(size_t)(t0 + step) * B + c0 + f];
+        prefix(step, parent, &h);
+        h.tokens.push_back(Decoder::end_symbol_);
+        h.score = fscore[(size_t)(t0 + step) * B + c0 + f];
+        r.hypotheses.push_back(std::move(h));
+      }
+    }
+    Decoder::OutputKBestHypotheses(r.hypotheses, (int)sentences[i].size(), o, &r);
+  }
+  // the search of every sentence in the layout lnmt_decode_history reads: [step][sentence * beam + j]
+  DecodeHistory &hist = last_history_;
+  hist.n = n, hist.beam = beam, hist.steps = max_limit + 1;
+  hist.slot_of_sentence.resize(n);
+  std::iota(hist.slot_of_sentence.begin(), hist.slot_of_sentence.end(), 0);
+  hist.limit = limit;
+  const size_t Bn = (size_t)n * beam;
+  hist.tok.assign((size_t)hist.steps * Bn, Decoder::end_symbol_);
+  hist.backptr.assign((size_t)hist.steps * Bn, 0);
+  hist.score.assign((size_t)hist.steps * Bn, 0.f);
+  for (int i = 0; i < n; ++i) {
+    const int t0 = start_of[i], c0 = slot_of[i] * beam;
+    for (int step = 0; step <= limit[i]; ++step)
+      for (int j = 0; j < beam; ++j) {
+        const size_t from = (size_t)(t0 + step + 1) * B + c0 + j, to = (size_t)step * Bn + (size_t)i * beam + j;
+        hist.tok[to] = tok[from];
+        hist.backptr[to] = bp[from] - c0 + i * beam;
+        hist.score[to] = bscore[from];
+      }
+  }
+  stream_ticks_ = ticks;
+}
+
+}  // namespace linmt

@@ -21,6 +21,11 @@ c_i32p = C.c_void_p
 c_f64p = C.c_void_p
 
 
+class StreamAdmission(C.Structure):
+    _fields_ = [("slot", C.c_int), ("sentence_col", C.c_int), ("hs_col_value", C.c_int),
+                ("len", C.c_int), ("off", C.c_int), ("limit", C.c_int), ("tick", C.c_int)]
+
+
 class GemmSeg(C.Structure):
     _fields_ = [("A", C.c_void_p), ("lda", C.c_int), ("X", C.c_void_p), ("ldx", C.c_int),
                 ("K", C.c_int)]
@@ -130,6 +135,15 @@ SIGNATURES = {
                                            c_i32p, c_i32p, c_f32p, c_i32p, c_i32p, c_f32p,
                                            C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int,
                                            C.c_int, C.c_void_p]),
+    "lh_beam_merge_gather_stream_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, c_i32p, c_i32p,
+                                                  c_f32p, c_i32p, c_f32p, c_f32p, C.c_float, C.c_float,
+                                                  C.c_int, C.c_int, c_i32p, c_i32p, c_f32p, c_i32p,
+                                                  c_i32p, c_f32p, C.POINTER(C.c_void_p),
+                                                  C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_void_p]),
+    "lh_stream_admit_f32": (C.c_int, [C.POINTER(StreamAdmission), C.c_int, C.c_int, C.c_int, c_i32p,
+                                      c_i32p, c_i32p, c_i32p, C.POINTER(C.c_void_p),
+                                      C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_void_p), C.c_int,
+                                      C.c_int, C.c_int, c_i32p, C.c_int, c_f32p, C.c_void_p]),
     "lh_softmax_xent_grad_f32": (C.c_int, [c_f32p, C.c_int, c_f32p, C.c_int, C.c_int, c_i32p,
                                            c_i32p, c_f32p, C.c_int, c_f64p, c_f64p, C.c_void_p]),
     "lh_uniform_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_ulonglong, C.c_void_p]),
@@ -496,6 +510,31 @@ def beam_merge_gather(n_sent, beam, K, step, limit, cand_logp, cand_id, logp_eof
                                           _ptr(score), _ptr(fin_count), _ptr(fin_beam),
                                           _ptr(fin_score), s, d, n, H, _stream(stream)),
           "lh_beam_merge_gather_f32")
+
+
+def beam_merge_gather_stream(n_sent, beam, K, tick, start, limit, cand_logp, cand_id, logp_eof,
+                             prev_score, diversity, penalty, start_id, eof_id, tok, backptr, score,
+                             fin_count, fin_beam, fin_score, src, dst, H, stream=None):
+    n = len(src)
+    s = (C.c_void_p * n)(*[t.data_ptr() for t in src])
+    d = (C.c_void_p * n)(*[t.data_ptr() for t in dst])
+    check(load().lh_beam_merge_gather_stream_f32(n_sent, beam, K, tick, _ptr(start), _ptr(limit),
+                                                 _ptr(cand_logp), _ptr(cand_id), _ptr(logp_eof),
+                                                 _ptr(prev_score), diversity, penalty, start_id, eof_id,
+                                                 _ptr(tok), _ptr(backptr), _ptr(score), _ptr(fin_count),
+                                                 _ptr(fin_beam), _ptr(fin_score), s, d, n, H,
+                                                 _stream(stream)), "lh_beam_merge_gather_stream_f32")
+
+
+def stream_admit(admissions, beam, B, start, limit, hs_col, batch_info, src, dst, zero, H, n_src,
+                 tok_prev, start_id, score_prev, stream=None):
+    """admissions: dicts with slot, sentence_col, hs_col_value, len, off, limit, tick."""
+    arr = (StreamAdmission * len(admissions))(*[StreamAdmission(**a) for a in admissions])
+    ptrs = lambda ts: (C.c_void_p * max(1, len(ts)))(*[t.data_ptr() for t in ts])  # noqa: E731
+    check(load().lh_stream_admit_f32(arr, len(admissions), beam, B, _ptr(start), _ptr(limit),
+                                     _ptr(hs_col), _ptr(batch_info), ptrs(src), ptrs(dst), len(src),
+                                     ptrs(zero), len(zero), H, n_src, _ptr(tok_prev), start_id,
+                                     _ptr(score_prev), _stream(stream)), "lh_stream_admit_f32")
 
 
 # ---- training half ------------------------------------------------------------------------------
