@@ -442,6 +442,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hbm-kernels", action="store_true",
                     help="skip the stand-alone timing of the HBM-bound kernels (hbm_kernels field)")
+    ap.add_argument("--no-stream", action="store_true",
+                    help="skip the extra leg that decodes the same sentences with every beam column "
+                         "kept busy (lnmt_decode_stream; reported beside `value`, never as it)")
     ap.add_argument("--no-split-products", action="store_true",
                     help="skip the second timing of the same batch with the opt-in arithmetic "
                          "(lnmt_set_split_products; reported beside `value`, never as it)")
@@ -557,6 +560,35 @@ def main():
                                                    else (HBM_PEAK_GBS * 1e9)), 4)}
         model.profile(0)
 
+    # The same sentences, `steps` times over, as ONE list decoded with every beam column kept busy: a
+    # sentence that has taken its last step hands its 12 columns to the next sentence of the list
+    # (lnmt_decode_stream), so every step runs 768 hypotheses instead of a batch's shrinking set.
+    # Reported beside `value`; `value` stays one batch after the other.
+    stream, stream_hist = None, None
+    if not args.no_stream and not args.split_products_only:
+        model.profile(0)
+        model.decode_stream(sents * max(args.warmup, 1), beam=beam)
+        torch.cuda.synchronize()
+        s0 = time.perf_counter()
+        stream_res = model.decode_stream(sents * args.steps, beam=beam)  # ends with a stream synchronisation
+        sdt0 = time.perf_counter() - s0
+        stok0 = sum(len(r["best"]) for r in stream_res)
+        stream_hist = [model.decode_history(i, beam) for i in range(n_sent)]
+        copies_same = all(stream_res[i]["best"].tolist() == stream_res[i % n_sent]["best"].tolist()
+                          for i in range(len(stream_res)))
+        stream = {"value": round(stok0 / sdt0, 1), "unit": "target tokens/s",
+                  "sentences": n_sent * args.steps, "slots": n_sent, "steps_of_768_hypotheses": model.stream_ticks,
+                  "ms_per_64_sentences": round(sdt0 * 1e3 / args.steps, 2),
+                  "speedup_over_value": round(stok0 / sdt0 / value, 3),
+                  "how": "the list is taken longest first; a finished sentence's beam columns go to "
+                         "the next sentence; encoder in groups of 64; schedule fixed by the length "
+                         "limits, one read-back at the end",
+                  "one_best_same_as_batch_mode": int(sum(a["best"].tolist() == b["best"].tolist()
+                                                         for a, b in zip(res, stream_res[:n_sent]))),
+                  "repeated_sentences_decode_identically": bool(copies_same)}
+        stream["_res"] = stream_res[:n_sent]
+        model.profile(1 if args.profile_level >= 1 else 0)
+
     # The same batch with the opt-in arithmetic: gate products and output projection from three-way
     # bf16 splits of their fp32 operands (six exact products per term, fp32 accumulation).  Reported
     # beside `value`; `value` stays the fp32 MFMA path.
@@ -593,6 +625,17 @@ def main():
                                   "rate": round(rate / (1e12 if is_gemm else 1e9), 2),
                                   "unit": "TFLOP/s (algorithmic)" if is_gemm else "GB/s"}
         model.profile(0)
+        split_stream = None
+        if not args.no_stream:
+            model.decode_stream(sents, beam=beam)
+            torch.cuda.synchronize()
+            s0 = time.perf_counter()
+            ss_res = model.decode_stream(sents * args.steps, beam=beam)
+            ss_dt = time.perf_counter() - s0
+            ss_tok = sum(len(r["best"]) for r in ss_res)
+            split_stream = {"value": round(ss_tok / ss_dt, 1), "unit": "target tokens/s",
+                            "ms_per_64_sentences": round(ss_dt * 1e3 / args.steps, 2),
+                            "speedup_over_value": round(ss_tok / ss_dt / value, 3)}
         model.set_split_products(False)
         split = {"value": round(stok / sdt, 1), "unit": "target tokens/s",
                  "ms_per_step": round(sdt * 1e3 / args.steps, 2),
@@ -607,6 +650,8 @@ def main():
                                                        for a, b in zip(res, split_res)))}
         if skernels:
             split["kernels"] = skernels
+        if split_stream:
+            split["stream"] = split_stream
         if sk:
             kern, t = max(sk.items(), key=lambda kv: kv[1]["work"])
             alg = t["work"] / (t["ms"] * 1e-3) / 1e12
@@ -642,8 +687,8 @@ def main():
         om.decode_sentence(sents[by_len[0]][:3], beam=beam, num_threads=cores)  # warm-up
         cpu_tokens, cdt = 0, 0.0
         classes = {"identical": 0, "diverged_at_near_tie": 0, "diverged_at_window_tie": 0, "diverged_other": 0}
-        sclasses = dict(classes)
-        same, ssame, detail = 0, 0, []
+        sclasses, qclasses = dict(classes), dict(classes)
+        same, ssame, qsame, detail = 0, 0, 0, []
         for i in pick:
             c0 = time.perf_counter()
             tr = om.decode_sentence_trace(sents[i], beam=beam, num_threads=cores)
@@ -653,6 +698,10 @@ def main():
             cls, at, eps = classify_beam_parity(res[i]["best"], gtok, gbp, gsc, tr, len(sents[i]))
             classes[cls] += 1
             same += int(tr["best"].tolist() == res[i]["best"].tolist())
+            if stream is not None:
+                qtok, qbp, qsc = stream_hist[int(i)]
+                qclasses[classify_beam_parity(stream["_res"][i]["best"], qtok, qbp, qsc, tr, len(sents[i]))[0]] += 1
+                qsame += int(tr["best"].tolist() == stream["_res"][i]["best"].tolist())
             if split is not None:
                 stok_h, sbp_h, ssc_h = split_hist[int(i)]
                 sclasses[classify_beam_parity(split_res[i]["best"], stok_h, sbp_h, ssc_h, tr, len(sents[i]))[0]] += 1
@@ -681,6 +730,9 @@ def main():
         if split is not None:
             split["parity"] = {"sentences_checked": int(len(pick)), "one_best_identical": int(ssame),
                                "beam_steps": sclasses, "parity_ok": sclasses["diverged_other"] == 0}
+        if stream is not None:
+            stream["parity"] = {"sentences_checked": int(len(pick)), "one_best_identical": int(qsame),
+                                "beam_steps": qclasses, "parity_ok": qclasses["diverged_other"] == 0}
 
     out = {
         "metric": "target tokens/sec (beam-12 decode, 1 GPU)" +
@@ -706,6 +758,9 @@ def main():
         "hbm_kernels": hbm_kernels,
         "cpu_baseline": cpu_baseline,
     }
+    if stream:
+        stream.pop("_res", None)
+        out["stream"] = stream
     if split:
         out["split_products"] = split
     if kernels:
@@ -716,6 +771,10 @@ def main():
     if split and "parity" in split and not split["parity"]["parity_ok"]:
         print("bench.py: with split products the GPU search differs from the oracle's where no "
               "near-tie explains it", file=sys.stderr)
+        sys.exit(1)
+    if stream and "parity" in stream and not stream["parity"]["parity_ok"]:
+        print("bench.py: the stream decoder's search differs from the oracle's where no near-tie "
+              "explains it", file=sys.stderr)
         sys.exit(1)
     if parity and not parity["parity_ok"]:
         print("bench.py: the GPU search differs from the oracle's where no near-tie explains it",

@@ -9,7 +9,7 @@
 // The number of steps of a sentence is fixed by its length (decoder.h:1734), so the whole
 // schedule -- which sentence enters which slot at which tick, and when a group of sentences has
 // to be encoded -- is laid out on the host before the first launch, and nothing is read back
-// until the end.  Sentences are encoded in groups of up to n_sent (ForwardPropSource as in
+// until the end.  Sentences are taken longest first and encoded in groups of up to n_sent (ForwardPropSource as in
 // DecodeBatch); what decoding needs of a group -- the projected attention memories W_a*hs and
 // W_c1*hs and the encoder's final states -- is kept in one of kRing slabs until the group's last
 // sentence has finished.
@@ -46,15 +46,21 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   for (const auto &w : sentences)
     if (w.empty() || (int)w.size() > longest) throw LinmtError("DecodeStream: source sentence length out of range");
 
-  // ---- groups: n_sent sentences each, in input order; inside a group longest first ---------------
+  // ---- groups of n_sent sentences, the longest sentences of the whole list first: the sentences of
+  // a group are about as long as each other (little padding in the encoder), and the list ends with
+  // its shortest sentences, so the slots run empty over a few ticks instead of a long sentence's
+  // ninety.  (Results are stored by position in the list; the order of work is free.)
   const int G = (n + slots - 1) / slots;
+  std::vector<int> by_length(n);
+  std::iota(by_length.begin(), by_length.end(), 0);
+  std::stable_sort(by_length.begin(), by_length.end(),
+                   [&](int a, int b) { return sentences[a].size() > sentences[b].size(); });
   std::vector<std::vector<int>> group_order(G);  // encoder column -> sentence
   std::vector<int> group_S(G), limit(n);
   for (int g = 0; g < G; ++g) {
-    std::vector<int> &ord = group_order[g];
-    for (int i = g * slots; i < std::min(n, (g + 1) * slots); ++i) ord.push_back(i);
-    std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return sentences[a].size() > sentences[b].size(); });
-    group_S[g] = (int)sentences[ord[0]].size();
+    group_order[g].assign(by_length.begin() + (size_t)g * slots,
+                          by_length.begin() + std::min((size_t)n, (size_t)(g + 1) * slots));
+    group_S[g] = (int)sentences[group_order[g][0]].size();
   }
   for (int i = 0; i < n; ++i)
     limit[i] = std::min((int)(o.max_decoding_ratio_ * (int)sentences[i].size()), longest - 2);  // decoder.h:1734
