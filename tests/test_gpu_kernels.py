@@ -939,6 +939,111 @@ def test_beam_merge_gather_equals_the_two_calls(lh, n_sent, beam, H, n):
         lh.beam_merge_gather(*args, *o2, srcs, srcs, H)                    # in place is rejected
 
 
+def test_stream_admission_and_merge_at_different_steps(lh):
+    """lh_stream_admit_f32 writes a slot's columns and entries and nothing else;
+    lh_beam_merge_gather_stream_f32 with sentences at different steps (tick - start[s]) gives, sentence
+    by sentence, the bits of lh_beam_merge_gather_f32 called with that sentence's own step."""
+    rng = np.random.default_rng(404)
+    n_sent, beam, H, L = 5, 4, 36, 2
+    B, K, n_src = n_sent * beam, beam + 1, 7
+    finals = [dev(uni(rng, H, n_src)) for _ in range(2 * L)]
+    states = [torch.full((H * B,), 9.0, device="cuda") for _ in range(2 * L)]
+    tild = torch.full((H * B,), 9.0, device="cuda")
+    start = torch.full((n_sent,), -5, dtype=torch.int32, device="cuda")
+    limit = torch.full((n_sent,), -1, dtype=torch.int32, device="cuda")
+    hs_col = torch.full((B,), -5, dtype=torch.int32, device="cuda")
+    binfo = torch.full((2 * B,), -5, dtype=torch.int32, device="cuda")
+    tok_prev = torch.full((B,), 7, dtype=torch.int32, device="cuda")
+    score_prev = torch.full((B,), 7.0, device="cuda")
+    adm = [dict(slot=3, sentence_col=6, hs_col_value=1006, len=11, off=2, limit=16, tick=40),
+           dict(slot=0, sentence_col=2, hs_col_value=2, len=9, off=4, limit=13, tick=40)]
+    lh.stream_admit(adm, beam, B, start, limit, hs_col, binfo, finals, states, [tild], H, n_src, tok_prev,
+                    0, score_prev)
+    torch.cuda.synchronize()
+    for a in adm:
+        cols = slice(a["slot"] * beam, (a["slot"] + 1) * beam)
+        assert start[a["slot"]].item() == 40 and limit[a["slot"]].item() == a["limit"]
+        assert (hs_col[cols] == a["hs_col_value"]).all() and (binfo[cols] == a["len"]).all()
+        assert (binfo[B:][cols] == a["off"]).all() and (tok_prev[cols] == 0).all() and (score_prev[cols] == 0).all()
+        for f, st in zip(finals, states):
+            want = host(f, (H, n_src))[:, a["sentence_col"]]
+            assert np.array_equal(host(st, (H, B))[:, cols], np.repeat(want[:, None], beam, 1))
+        assert (host(tild, (H, B))[:, cols] == 0).all()
+    untouched = [c for c in range(B) if c // beam not in (0, 3)]
+    assert (hs_col[untouched] == -5).all() and (tok_prev[untouched] == 7).all()
+    assert (host(states[0], (H, B))[:, untouched] == 9).all() and (host(tild, (H, B))[:, untouched] == 9).all()
+    with pytest.raises(lh.LinmtHipError):
+        lh.stream_admit([dict(adm[0], slot=n_sent)], beam, B, start, limit, hs_col, binfo, finals, states,
+                        [tild], H, n_src, tok_prev, 0, score_prev)
+
+    # merge + gather with sentences at steps 0, 3, == limit, > limit and in a slot that idles
+    tick = 50
+    starts = np.array([50, 47, 40, 30, 0], np.int32)
+    limits = np.array([9, 9, 10, 5, -1], np.int32)
+    cl = np.sort(uni(rng, K, B, s=3.0), axis=0)[::-1]
+    ci = rng.integers(0, 50, size=(K, B)).astype(np.int32)
+    prev, le = uni(rng, B, s=5.0), uni(rng, B, s=2.0)
+    srcs = [dev(uni(rng, H, B)) for _ in range(3)]
+
+    def outputs():
+        return [torch.full((B,), -7, dtype=torch.int32, device="cuda"),
+                torch.full((B,), -7, dtype=torch.int32, device="cuda"), torch.full((B,), 7.0, device="cuda"),
+                torch.full((n_sent,), -7, dtype=torch.int32, device="cuda"),
+                torch.full((B,), -7, dtype=torch.int32, device="cuda"), torch.full((B,), 7.0, device="cuda")]
+    common = (dev(cl), dev(ci), dev(le), dev(prev), 0.1, 0.05, 0, 1)
+    got, gd = outputs(), [torch.full((H * B,), 3.0, device="cuda") for _ in srcs]
+    lh.beam_merge_gather_stream(n_sent, beam, K, tick, dev(starts), dev(limits), *common, *got, srcs, gd, H)
+    torch.cuda.synchronize()
+    for s_ in range(n_sent):
+        ref, rd = outputs(), [torch.full((H * B,), 3.0, device="cuda") for _ in srcs]
+        lh.beam_merge_gather(n_sent, beam, K, int(tick - starts[s_]), dev(limits), *common, *ref, srcs, rd, H)
+        torch.cuda.synchronize()
+        cols = slice(s_ * beam, (s_ + 1) * beam)
+        for a, b, what in zip(got, ref, ("tok", "backptr", "score", "fin_count", "fin_beam", "fin_score")):
+            sel = slice(s_, s_ + 1) if what == "fin_count" else cols
+            assert torch.equal(a[sel], b[sel]), f"sentence {s_}: {what}"
+        for a, b in zip(gd, rd):
+            assert torch.equal(a.view(B, H)[cols], b.view(B, H)[cols]), f"sentence {s_}: gathered state"
+
+
+def test_cell_mask_bit_selects_the_fp32_sigmoids(lh, orc):
+    """A column whose mask carries LH_MASK_F32_GATES (2) takes the fp32 sigmoids although
+    sigmoid_f64 is set: in lh_lstm_cell_fwd_f32 and in the cell epilogue of the gate product, the
+    masked columns equal the sigmoid_f64 = 0 run bit for bit and the others the sigmoid_f64 = 1 run."""
+    rng = np.random.default_rng(77)
+    H, B, K = 64, 40, 48
+    A, X = uni(rng, 4 * H, K, s=0.4), uni(rng, K, B)
+    bias, c_prev = uni(rng, 4 * H, s=0.5), uni(rng, H, B)
+    m = np.ones(B, np.int32)
+    m[::3] = 3
+    m[5] = 0
+    m[6] = 2                                                  # masked out, bit set
+    plain = np.where(m & 1, 1, 0).astype(np.int32)
+    segs = [(dev(A), 4 * H, dev(X), K, K)]
+    pre = torch.empty(4 * H * B, device="cuda")
+    lh.gemm(4 * H, B, segs, pre, 4 * H)
+
+    def cell(mask, f64):
+        c, h = dev(c_prev), torch.empty(H * B, device="cuda")
+        lh.lstm_cell_fwd(H, B, pre, dev(bias), c, dev(mask), c, h, sigmoid_f64=f64)
+        return host(c, (H, B)), host(h, (H, B))
+
+    def fused(mask, f64):
+        c, h = dev(c_prev), torch.empty(H * B, device="cuda")
+        lh.gate_gemm_lstm_cell(H, B, segs, dev(bias), c, dev(mask), c, h, sigmoid_f64=f64)
+        return host(c, (H, B)), host(h, (H, B))
+
+    bit = (m & 2) != 0
+    for run in (cell, fused):
+        c32, h32 = run(plain, False)
+        c64, h64 = run(plain, True)
+        cm, hm = run(m, True)
+        assert np.array_equal(cm[:, bit], c32[:, bit]) and np.array_equal(hm[:, bit], h32[:, bit])
+        assert np.array_equal(cm[:, ~bit], c64[:, ~bit]) and np.array_equal(hm[:, ~bit], h64[:, ~bit])
+        assert np.all(cm[:, [5, 6]] == 0) and np.all(hm[:, [5, 6]] == 0)
+        assert not np.array_equal(c32, c64)                 # the two arithmetics do differ somewhere
+
+
 def test_full_size_softmax_properties(lh):
     """Config-3 size (V=30000, B=768): too large for the CPU oracle in a unit test, so checked
     through size-independent properties: columns sum to 1, shift invariance, argmax preserved,
