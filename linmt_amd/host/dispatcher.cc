@@ -191,7 +191,31 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
     std::ofstream output(ids_file.c_str());
     if (!output) throw LinmtError("Decoding: cannot open " + ids_file);
     const auto begin = std::chrono::steady_clock::now();
-    for (size_t first = 0; first < sentences.size(); first += n_sent) {
+    // One model without exported alignments over local-p attention: the sentences go through
+    // DecodeStream, a few thousand at a time, with every beam column kept busy; everything else
+    // is decoded batch by batch.  (LINMT_NO_STREAM: measurement and test aid.)
+    const bool stream = ensemble.empty() && !o.unk_replacement_mode_ && neural.cfg_.attention_mode_ &&
+                        neural.attention_layer_.ProjectedMemoryPossible() && getenv("LINMT_NO_STREAM") == nullptr;
+    const size_t chunk = stream ? (size_t)n_sent * 32 : (size_t)n_sent;
+    for (size_t first = 0; stream && first < sentences.size(); first += chunk) {
+      std::vector<std::vector<int>> list;
+      std::vector<size_t> where;
+      const size_t last = std::min(sentences.size(), first + chunk);
+      for (size_t i = first; i < last; ++i)
+        if (!sentences[i].empty()) {  // an empty source line cannot be encoded: it translates to an empty line
+          list.push_back(sentences[i]);
+          where.push_back(i - first);
+        }
+      std::vector<SentenceResult> results, ordered(last - first);
+      if (!list.empty()) neural.DecodeStream(list, o, &results);
+      for (size_t b = 0; b < list.size(); ++b) ordered[where[b]] = std::move(results[b]);
+      for (size_t i = first; i < last; ++i) {
+        WriteHypothesisLines(output, ordered[i - first], (int)sentences[i].size(), c);
+        report.source_words += (long long)sentences[i].size();
+        report.target_words += (long long)ordered[i - first].best.size();
+      }
+    }
+    for (size_t first = 0; !stream && first < sentences.size(); first += n_sent) {
       // an empty source line cannot be encoded: it translates to an empty line
       std::vector<std::vector<int>> batch;
       std::vector<std::vector<std::vector<int>>> other_batches(ensemble.size());

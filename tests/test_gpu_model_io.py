@@ -250,3 +250,16 @@ def test_k_best_lists(host, tmp_path):
             assert np.isclose(float(fields[1]), score, rtol=1e-4, atol=1e-5)
     words = open(final_file).read().split("\n")[:-1]
     assert len(words) == len(lines) and words[k] == "================"
+    # that run went through DecodeStream (one model, no exported alignments); batch by batch gives
+    # the same lines
+    import os
+    os.environ["LINMT_NO_STREAM"] = "1"
+    try:
+        ids2 = str(tmp_path / "out2.ids")
+        host.decoding(model, str(src), str(tmp_path / "out2.txt"), ids_file=ids2, beam=beam,
+                      longest_sentence=24, attention_width=D, print_decoding_information=True,
+                      sentences_per_batch=2, num_hypotheses=k)
+    finally:
+        del os.environ["LINMT_NO_STREAM"]
+    lines2 = open(ids2).read().split("\n")[:-1]
+    assert [l.split(" |||| ")[0] for l in lines2] == [l.split(" |||| ")[0] for l in lines]
