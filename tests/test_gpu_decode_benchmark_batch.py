@@ -51,10 +51,13 @@ def workload(orc):
     return dict(cfg=(layers, H, V, D, beam, n_sent, longest), P=P, sents=sents, traces=traces)
 
 
-@pytest.mark.parametrize("split", [False, True], ids=["fp32_mfma", "split_bf16_products"])
-def test_benchmark_batch_beams_vs_oracle_trace(workload, host, split):
+@pytest.mark.parametrize("split,stream", [(False, False), (True, False), (False, True)],
+                         ids=["fp32_mfma", "split_bf16_products", "stream"])
+def test_benchmark_batch_beams_vs_oracle_trace(workload, host, split, stream):
     """split: the same demand on the opt-in arithmetic (lnmt_set_split_products), whose products
-    are as close to float64 as the fp32 MFMA ones."""
+    are as close to float64 as the fp32 MFMA ones.  stream: the same demand on lnmt_decode_stream
+    over the 64 sentences twice in a row (128 sentences through the 64 slots); the second copy of
+    every sentence must come out exactly as the first."""
     layers, H, V, D, beam, n_sent, longest = workload["cfg"]
     P, sents = workload["P"], workload["sents"]
     gm = host.Model(layers, H, V, V, longest_sentence=longest, attention_mode=1, attention_width=D,
@@ -62,8 +65,15 @@ def test_benchmark_batch_beams_vs_oracle_trace(workload, host, split):
     gm.set_params(P)
     if split:
         gm.set_split_products(True)
-    res = gm.decode_batch(sents, beam=beam)
-    hist = [gm.decode_history(i, beam) for i in range(n_sent)]
+    if stream:
+        res = gm.decode_stream(sents * 2, beam=beam)
+        hist = [gm.decode_history(i, beam) for i in range(2 * n_sent)]
+        for i in range(n_sent):
+            assert res[i]["best"].tolist() == res[n_sent + i]["best"].tolist(), i
+            assert all(np.array_equal(a, b) for a, b in zip(hist[i], hist[n_sent + i])), i
+    else:
+        res = gm.decode_batch(sents, beam=beam)
+        hist = [gm.decode_history(i, beam) for i in range(n_sent)]
     gm.close()
     classes = {"identical": 0, "diverged_at_near_tie": 0, "diverged_at_window_tie": 0, "diverged_other": 0}
     notes, steps_equal, steps_total, same_best, worst_dev = [], 0, 0, 0, 0.0
@@ -88,7 +98,7 @@ def test_benchmark_batch_beams_vs_oracle_trace(workload, host, split):
             notes.append(f"sentence {i} (len {len(s)}): {cls} at step {at}, oracle margin "
                          f"{tr['margin'][at]:.3e}, epsilon {eps_at:.3e}, window margin "
                          f"{tr['window_margin'][at]:.3e}")
-    print(f"beam parity on the benchmark batch ({'split bf16' if split else 'fp32 MFMA'} products): {classes}; {steps_equal} of {steps_total} expansion "
+    print(f"beam parity on the benchmark batch ({'split bf16' if split else 'fp32 MFMA'} products{', stream' if stream else ''}): {classes}; {steps_equal} of {steps_total} expansion "
           f"steps identical before any divergence; largest |GPU - oracle| path score on identical "
           f"beams {worst_dev:.2e}; 1-best identical for {same_best} of {n_sent}", flush=True)
     for line in notes:
