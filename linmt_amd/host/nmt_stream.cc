@@ -150,11 +150,15 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   A.hs_step_stride_ = (long long)H * slots;
   A.hs_steps_ = (int)T_cap;
   A.projected_memory_ = true;
-  // every column points at valid memory from the first tick on, sentence or not
+  // A column without a sentence still runs every step: it starts from zero states and attends to
+  // the first state of the first sentence of slab 0 (always an encoded sentence), so that nothing
+  // it computes is undefined; nothing reads what it computes.
   A.PreprocessMinibatchInformation(binfo0.data(), B);
-  HipErrorWrapper(hipMemcpyAsync(A.p_device_hs_col_.get(), p_device_sentence_of_column_.get(), sizeof(int) * B,
-                                 hipMemcpyDeviceToDevice, stream_),
-                  "DecodeStream: hs_col initialisation failed");
+  A.p_device_hs_col_.Zero(stream_);
+  for (int l = 0; l < L; ++l) {
+    TargetLayer(l).p_device_h_t_previous_.Zero(stream_);
+    TargetLayer(l).p_device_c_t_previous_.Zero(stream_);
+  }
   if (p_device_h_tild_previous_.size()) p_device_h_tild_previous_.Zero(stream_);
 
   const float *state_src[LH_GATHER_MAX_TENSORS];
