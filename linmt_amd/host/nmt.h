@@ -558,6 +558,11 @@ class NeuralMachineTranslation {
   void DecodeStream(const std::vector<std::vector<int>> &sentences, const DecodeOptions &o,
                     std::vector<SentenceResult> *results);
   const int *stream_layer0_mask_ = nullptr;  // DecodeStream: the first target layer's column mask of this tick
+  // DecodeStream runs the encoder of the coming groups beside the decoding steps: a stream, a GEMM
+  // workspace and events (two per group: "its slab is free", "it is encoded") of its own
+  hipStream_t encoder_stream_ = nullptr;
+  DeviceArray<char> encoder_workspace_;
+  std::vector<hipEvent_t> stream_events_;
   int stream_ticks_ = 0;                     // steps the last DecodeStream took
 
   // ---- training --------------------------------------------------------------------------------

@@ -101,6 +101,11 @@ NeuralMachineTranslation::~NeuralMachineTranslation() {
     (void)hipStreamSynchronize(lane_streams_[l]);
     (void)hipStreamDestroy(lane_streams_[l]);
   }
+  for (hipEvent_t e : stream_events_) (void)hipEventDestroy(e);
+  if (encoder_stream_) {
+    (void)hipStreamSynchronize(encoder_stream_);
+    (void)hipStreamDestroy(encoder_stream_);
+  }
   if (stream_) {
     (void)hipStreamSynchronize(stream_);
     (void)hipStreamDestroy(stream_);
@@ -392,23 +397,28 @@ void NeuralMachineTranslation::RunSourceSideLanes(int source_length, int B) {
   for (int l = 1; l < L; ++l)
     HipErrorWrapper(hipStreamWaitEvent(lane_streams_[l], lane_events_[0], 0), "encoder lane fork failed");
 
+  // lane 0 is the stream the caller is on (DecodeStream runs the encoder beside the decoding
+  // steps, on a stream and a workspace of its own); the lanes share the caller's workspace
   hipStream_t const main_stream = stream_;
-  char *const ws = gemm_workspace_.get();
-  const size_t ws_slice = (gemm_workspace_.size() / L) & ~size_t(255);
+  char *const ws = gemm_ws_ptr_;
+  const size_t ws_bytes = gemm_ws_bytes_;
+  const size_t ws_slice = (ws_bytes / L) & ~size_t(255);
   struct Restore {
     NeuralMachineTranslation &m;
     hipStream_t s;
+    char *ws;
+    size_t ws_bytes;
     ~Restore() {
       m.stream_ = s;
       m.profiler_.stream_ = s;
-      m.gemm_ws_ptr_ = m.gemm_workspace_.get();
-      m.gemm_ws_bytes_ = m.gemm_workspace_.size();
+      m.gemm_ws_ptr_ = ws;
+      m.gemm_ws_bytes_ = ws_bytes;
     }
-  } restore{*this, main_stream};
+  } restore{*this, main_stream, ws, ws_bytes};
 
   for (int l = 0; l < L; ++l) {
     LstmLayer &Ls = SourceLayer(l);
-    stream_ = lane_streams_[l];
+    stream_ = l == 0 ? main_stream : lane_streams_[l];
     profiler_.stream_ = stream_;
     gemm_ws_ptr_ = ws + ws_slice * l;
     gemm_ws_bytes_ = ws_slice;

@@ -125,6 +125,7 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
     NeuralMachineTranslation &m;
     int B;
     ~Restore() {
+      if (m.encoder_stream_) (void)hipStreamSynchronize(m.encoder_stream_);
       // DecodeBatch reads the encoder states of column b's sentence through hs_col[b] = b / beam
       (void)hipMemcpyAsync(m.attention_layer_.p_device_hs_col_.get(), m.p_device_sentence_of_column_.get(),
                            sizeof(int) * B, hipMemcpyDeviceToDevice, m.stream_);
@@ -173,9 +174,43 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   const bool has_tild = cfg_.feed_input_mode_ && p_device_h_tild_previous_.size();
   zero_dst[0] = has_tild ? p_device_h_tild_previous_.get() : nullptr;
 
+  // The encoder of a group runs on a stream of its own from the tick at which the group's slab is
+  // free (at once for the first kRing groups), beside the decoding steps, whose large launches
+  // leave room at their ends for its small ones; the decoding stream waits for it right before the
+  // group's first sentence enters.
+  if (!encoder_stream_) HipErrorWrapper(hipStreamCreate(&encoder_stream_), "DecodeStream: stream creation failed");
+  if (!encoder_workspace_.size()) encoder_workspace_.Alloc(kGemmWorkspaceBytes);
+  while (stream_events_.size() < 2 * (size_t)G) {
+    hipEvent_t e;
+    HipErrorWrapper(hipEventCreateWithFlags(&e, hipEventDisableTiming), "DecodeStream: event creation failed");
+    stream_events_.push_back(e);
+  }
+  // a group is encoded kEncoderLead ticks ahead of its first admission, or as soon as its slab is free
+  constexpr int kEncoderLead = 24;
+  std::vector<int> first_tick(G, 0);
+  for (int t = 0; t < ticks; ++t)
+    for (int g : encode_at[t]) first_tick[g] = t;
+  std::vector<std::vector<int>> ready_at(ticks);  // groups to encode at this tick
+  for (int g = 0; g < G; ++g)
+    ready_at[std::max(g < kRing ? 0 : group_done[g - kRing], first_tick[g] - kEncoderLead)].push_back(g);
+
   for (int t = 0; t < ticks; ++t) {
-    // ---- groups whose first sentence enters at this tick: encode them ---------------------------
-    for (int g : encode_at[t]) {
+    // ---- groups to encode from this tick on, beside the steps ------------------------------------------
+    for (int g : ready_at[t]) {
+      HipErrorWrapper(hipEventRecord(stream_events_[2 * g], stream_), "DecodeStream: event record failed");
+      HipErrorWrapper(hipStreamWaitEvent(encoder_stream_, stream_events_[2 * g], 0), "DecodeStream: wait failed");
+      struct Swap {  // the encoder's launches go to its own stream and workspace
+        NeuralMachineTranslation &m;
+        hipStream_t s;
+        char *ws;
+        size_t ws_bytes;
+        ~Swap() {
+          m.stream_ = s, m.profiler_.stream_ = s;
+          m.gemm_ws_ptr_ = ws, m.gemm_ws_bytes_ = ws_bytes;
+        }
+      } swap{*this, stream_, gemm_ws_ptr_, gemm_ws_bytes_};
+      stream_ = encoder_stream_, profiler_.stream_ = encoder_stream_;
+      gemm_ws_ptr_ = encoder_workspace_.get(), gemm_ws_bytes_ = encoder_workspace_.size();
       const std::vector<int> &ord = group_order[g];
       const int ng = (int)ord.size(), S = group_S[g], r = g % kRing;
       std::vector<int> &src_block = src_blocks[g];
@@ -202,7 +237,11 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
                                        hipMemcpyDeviceToDevice, stream_),
                         "DecodeStream: copy of the encoder's final c failed");
       }
+      HipErrorWrapper(hipEventRecord(stream_events_[2 * g + 1], stream_), "DecodeStream: event record failed");
     }
+    // ---- groups whose first sentence enters at this tick: their encoder has to be done -----------
+    for (int g : encode_at[t])
+      HipErrorWrapper(hipStreamWaitEvent(stream_, stream_events_[2 * g + 1], 0), "DecodeStream: wait failed");
     // ---- sentences that enter at this tick --------------------------------------------------------
     const std::vector<int> &now = adm_at[t];
     for (size_t at = 0; at < now.size();) {
