@@ -75,3 +75,55 @@ def test_decode_stream_history_and_errors(orc, host):
     with pytest.raises(host.HostError):
         gm.decode_stream([rng.integers(0, 50, size=5)], beam=3)
     gm.close()
+
+
+def test_decode_stream_equals_decode_batch_bit_for_bit_on_random_shapes(host):
+    """Which sentences share a launch must not matter.  With every matrix product held to one tile
+    shape and one K order (otherwise the shape is chosen by the number of columns, which shrinks in
+    DecodeBatch as sentences finish), a column's arithmetic does not depend on its neighbours or on
+    the tick it runs at: over random layer counts, widths, beams, slot counts and list lengths (up to
+    six times the slots) every sentence must come out of the stream with exactly the tokens, finished
+    hypotheses and score bits DecodeBatch gives it.  DecodeBatch gets the sentences in the groups the
+    stream encodes them in (longest first, n_sent at a time): a full group's encoder runs layer-major
+    with the input products batched over the steps and added to the recurrent ones, a partial group's
+    step by step with both in one accumulation, and the two round differently."""
+    import ref_numpy as R
+    from linmt_amd import lib as lh
+    L = lh.load()
+    rng = np.random.default_rng(7)
+    sentences = 0
+    try:
+        L.lh_gemm_set_config_override(7)
+        L.lh_gemm_set_splits_override(1)
+        for trial in range(40):
+            layers = int(rng.integers(1, 5)); H = int(rng.choice([32, 48, 64, 100, 128]))
+            Vs = int(rng.integers(30, 300)); Vt = int(rng.integers(40, 500))
+            D = int(rng.integers(1, 11)); beam = int(rng.integers(2, 13)); slots = int(rng.integers(1, 9))
+            feed = bool(rng.integers(0, 2)); scale = float(rng.choice([0.2, 0.4, 0.8]))
+            beam = min(beam, int(np.sqrt(Vt)))
+            P = R.make_params(rng, layers, H, Vs, Vt, attention=True, feed_input=feed, scale=scale)
+            n = int(rng.integers(1, 6 * slots + 2))
+            sents = [rng.integers(0, Vs, size=int(rng.integers(1, 25))) for _ in range(n)]
+            gm = host.Model(layers, H, Vs, Vt, longest_sentence=44, attention_mode=1, attention_width=D,
+                            feed_input=feed, decoding=(slots, beam))
+            gm.set_params(P)
+            got = gm.decode_stream(sents, beam=beam, with_hyps=True)
+            order = sorted(range(n), key=lambda i: -len(sents[i]))  # stable, as the stream's
+            for g0 in range(0, n, slots):
+                group = order[g0:g0 + slots]
+                want = gm.decode_batch([sents[i] for i in group], beam=beam, with_hyps=True)
+                for w, i in zip(want, group):
+                    what = (f"trial {trial} (layers {layers}, H {H}, beam {beam}, slots {slots}, n {n}, "
+                            f"feed {feed}, scale {scale}) sentence {i} (len {len(sents[i])})")
+                    assert got[i]["steps"] == w["steps"], what
+                    assert got[i]["best"].tolist() == w["best"].tolist(), what
+                    assert got[i]["best_score"] == w["best_score"], what
+                    assert len(got[i]["hyps"]) == len(w["hyps"]), what
+                    for (gt, gs), (wt, ws) in zip(got[i]["hyps"], w["hyps"]):
+                        assert gt.tolist() == wt.tolist() and gs == ws, what
+            sentences += n
+            gm.close()
+    finally:
+        L.lh_gemm_set_config_override(-1)
+        L.lh_gemm_set_splits_override(0)
+    assert sentences > 500
