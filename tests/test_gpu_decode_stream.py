@@ -127,3 +127,48 @@ def test_decode_stream_equals_decode_batch_bit_for_bit_on_random_shapes(host):
         L.lh_gemm_set_config_override(-1)
         L.lh_gemm_set_splits_override(0)
     assert sentences > 500
+
+
+def test_decode_batch_equals_lone_sentences_bit_for_bit(host):
+    """The same statement for DecodeBatch: a sentence decoded among others (shorter and longer ones,
+    which leave the batch before and after it) gets exactly what it gets alone, one tile shape
+    forced as above.  Batches stay one short of n_sent so that both runs take the encoder step by
+    step."""
+    import ref_numpy as R
+    from linmt_amd import lib as lh
+    L = lh.load()
+    rng = np.random.default_rng(11)
+    sentences = 0
+    try:
+        L.lh_gemm_set_config_override(7)
+        L.lh_gemm_set_splits_override(1)
+        for trial in range(20):
+            layers = int(rng.integers(1, 5)); H = int(rng.choice([32, 48, 64, 100, 128]))
+            Vs = int(rng.integers(30, 300)); Vt = int(rng.integers(40, 500))
+            D = int(rng.integers(0, 11)); beam = int(rng.integers(2, 13)); slots = int(rng.integers(3, 9))
+            att = 1 if D else 0
+            feed = bool(att and rng.integers(0, 2)); scale = float(rng.choice([0.2, 0.4, 0.8]))
+            beam = min(beam, int(np.sqrt(Vt)))
+            P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(att), feed_input=feed, scale=scale)
+            n = int(rng.integers(2, slots))
+            sents = [rng.integers(0, Vs, size=int(rng.integers(1, 25))) for _ in range(n)]
+            gm = host.Model(layers, H, Vs, Vt, longest_sentence=44, attention_mode=att, attention_width=max(D, 1),
+                            feed_input=feed, decoding=(slots, beam))
+            gm.set_params(P)
+            got = gm.decode_batch(sents, beam=beam, with_hyps=True)
+            for i, s in enumerate(sents):
+                w = gm.decode_batch([s], beam=beam, with_hyps=True)[0]
+                what = (f"trial {trial} (layers {layers}, H {H}, beam {beam}, n_sent {slots}, n {n}, attention {att}, "
+                        f"feed {feed}, scale {scale}) sentence {i} (len {len(s)})")
+                assert got[i]["steps"] == w["steps"], what
+                assert got[i]["best"].tolist() == w["best"].tolist(), what
+                assert got[i]["best_score"] == w["best_score"], what
+                assert len(got[i]["hyps"]) == len(w["hyps"]), what
+                for (gt, gs), (wt, ws) in zip(got[i]["hyps"], w["hyps"]):
+                    assert gt.tolist() == wt.tolist() and gs == ws, what
+            sentences += n
+            gm.close()
+    finally:
+        L.lh_gemm_set_config_override(-1)
+        L.lh_gemm_set_splits_override(0)
+    assert sentences > 50
