@@ -599,6 +599,26 @@ int lh_lstm_cell_bwd_f32(int H, int B, const float *dh_above, const float *dh_ne
                          const float *c_prev, const int *mask01, float clip_above, float clip_next,
                          const float *above_drop_mask, float keep, float *dgates, float *dc_prev,
                          lh_stream_t stream);
+/* The same step with each incoming error given as a sum of partial planes: a W^T d product whose
+ * K range was split over workgroups (lh_gemm_planes_f32) can be consumed as it lies, without the
+ * launch that adds its planes.  A term is `planes` (1..LH_ERROR_TERM_MAX_PLANES) column-major
+ * H x B blocks of leading dimension ld >= H, plane s at p + s * plane_stride; its value is
+ * ((plane 0 + plane 1) + plane 2) ..., the order in which lh_gemm_ws_f32's second launch adds them,
+ * so the results are bit for bit those of lh_lstm_cell_bwd_f32 on the reduced product.  The clamp
+ * and the dropout mask apply to the sum.  above / next == NULL or p == NULL: no such error.
+ * No counterpart in the reference (cuBLAS splits and reduces inside cublasSgemm). */
+#define LH_ERROR_TERM_MAX_PLANES 8
+typedef struct lh_error_term {
+  const float *p;
+  int planes;
+  long long plane_stride; /* floats between planes; ignored when planes == 1 */
+  int ld;
+} lh_error_term;
+int lh_lstm_cell_bwd_terms_f32(int H, int B, const lh_error_term *above, const lh_error_term *next,
+                               const float *dc_next, const float *gates, const float *c,
+                               const float *c_prev, const int *mask01, float clip_above,
+                               float clip_next, const float *above_drop_mask, float keep,
+                               float *dgates, float *dc_prev, lh_stream_t stream);
 
 /* out[r] = beta*out[r] + sum_c A[r,c] for a column-major rows x cols matrix.  Replaces the
  * cublasSgemv-with-ones bias gradients (src/node_input_to_hidden.h:1215-1240,

@@ -33,13 +33,31 @@ __device__ __forceinline__ float clampf(float x, float lim) {
 // LSTM cell backward
 struct CellBwdArgs {
   int H, B;
-  const float *dh_above, *dh_next, *dc_next, *gates, *c, *c_prev;
+  lh_error_term above, next;  // p == NULL: none
+  const float *dc_next, *gates, *c, *c_prev;
   const int *mask01;
   float clip_above, clip_next;
   const float *above_drop_mask;
   float keep;
   float *dgates, *dc_prev;
 };
+
+// an incoming error: the sum of the term's planes, in plane order
+template <int VW>
+__device__ __forceinline__ void load_term(const lh_error_term &e, int b, int r, Vec<VW> *out) {
+  const float *p = e.p + (size_t)b * e.ld + r;
+  out->load(p);
+  if (e.planes > 1) {  // the reduction launch starts from +0: a plane's -0 comes out as +0
+#pragma unroll
+    for (int i = 0; i < VW; ++i) out->v[i] = 0.f + out->v[i];
+  }
+  for (int s = 1; s < e.planes; ++s) {
+    Vec<VW> u;
+    u.load(p + (size_t)s * e.plane_stride);
+#pragma unroll
+    for (int i = 0; i < VW; ++i) out->v[i] += u.v[i];
+  }
+}
 
 template <int VW>
 __global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(const CellBwdArgs a) {
@@ -58,13 +76,13 @@ __global__ __launch_bounds__(256) void lstm_cell_bwd_kernel(const CellBwdArgs a)
   cp.load(a.c_prev + o1);
 #pragma unroll
   for (int i = 0; i < VW; ++i) dh.v[i] = 0.f, dc.v[i] = 0.f;
-  if (a.dh_next) {
-    t.load(a.dh_next + o1);
+  if (a.next.p) {
+    load_term<VW>(a.next, b, r, &t);
 #pragma unroll
     for (int i = 0; i < VW; ++i) dh.v[i] = clampf(t.v[i], a.clip_next);
   }
-  if (a.dh_above) {
-    t.load(a.dh_above + o1);
+  if (a.above.p) {
+    load_term<VW>(a.above, b, r, &t);
     if (a.above_drop_mask) {  // the layer above saw a dropped copy of h: same mask on the way back
       Vec<VW> u;
       u.load(a.above_drop_mask + o1);
@@ -460,28 +478,56 @@ extern "C" int lh_uniform_f32(float *out, long long n, unsigned long long seed, 
   return lh::check_launch("lh_uniform_f32");
 }
 
-extern "C" int lh_lstm_cell_bwd_f32(int H, int B, const float *dh_above, const float *dh_next,
-                                    const float *dc_next, const float *gates, const float *c,
-                                    const float *c_prev, const int *mask01, float clip_above,
-                                    float clip_next, const float *above_drop_mask, float keep,
-                                    float *dgates, float *dc_prev, lh_stream_t stream) {
+namespace {
+// NULL / empty terms become {NULL}; false = malformed
+bool normal_term(const lh_error_term *in, int H, lh_error_term *out, bool *vec) {
+  *out = lh_error_term{nullptr, 1, 0, H};
+  if (!in || !in->p) return true;
+  if (in->planes < 1 || in->planes > LH_ERROR_TERM_MAX_PLANES || in->ld < H) return false;
+  if (in->planes > 1 && in->plane_stride <= 0) return false;
+  *out = *in;
+  if (in->planes == 1) out->plane_stride = 0;
+  if (!lh::aligned16(in->p) || in->ld % 4 || (in->planes > 1 && in->plane_stride % 4)) *vec = false;
+  return true;
+}
+}  // namespace
+
+extern "C" int lh_lstm_cell_bwd_terms_f32(int H, int B, const lh_error_term *above,
+                                          const lh_error_term *next, const float *dc_next,
+                                          const float *gates, const float *c, const float *c_prev,
+                                          const int *mask01, float clip_above, float clip_next,
+                                          const float *above_drop_mask, float keep, float *dgates,
+                                          float *dc_prev, lh_stream_t stream) {
   if (H <= 0 || B <= 0) return lh::fail_arg("lh_lstm_cell_bwd_f32: H=%d B=%d", H, B);
   if (!gates || !c || !c_prev || !mask01 || !dgates || !dc_prev)
     return lh::fail_arg("lh_lstm_cell_bwd_f32: a required pointer is NULL");
-  if (above_drop_mask && (!dh_above || !(keep > 0.f)))
+  bool vec = H % 4 == 0 && lh::aligned16(dc_next) && lh::aligned16(gates) && lh::aligned16(c) &&
+             lh::aligned16(c_prev) && lh::aligned16(dgates) && lh::aligned16(dc_prev) &&
+             lh::aligned16(above_drop_mask);
+  lh_error_term ta, tn;
+  if (!normal_term(above, H, &ta, &vec) || !normal_term(next, H, &tn, &vec))
+    return lh::fail_arg("lh_lstm_cell_bwd_f32: an error term needs 1..%d planes, ld >= H and a positive plane stride",
+                        LH_ERROR_TERM_MAX_PLANES);
+  if (above_drop_mask && (!ta.p || !(keep > 0.f)))
     return lh::fail_arg("lh_lstm_cell_bwd_f32: above_drop_mask needs dh_above and keep > 0");
-  CellBwdArgs a{H, B, dh_above, dh_next, dc_next, gates, c, c_prev, mask01, clip_above, clip_next,
+  CellBwdArgs a{H, B, ta, tn, dc_next, gates, c, c_prev, mask01, clip_above, clip_next,
                 above_drop_mask, keep, dgates, dc_prev};
-  const bool vec = H % 4 == 0 && lh::aligned16(dh_above) && lh::aligned16(dh_next) &&
-                   lh::aligned16(dc_next) && lh::aligned16(gates) && lh::aligned16(c) &&
-                   lh::aligned16(c_prev) && lh::aligned16(dgates) && lh::aligned16(dc_prev) &&
-                   lh::aligned16(above_drop_mask);
   const long long work = (long long)(vec ? H / 4 : H) * B;
   const dim3 grid((unsigned)((work + 255) / 256)), block(256);
   hipStream_t st = lh::as_stream(stream);
   if (vec) hipLaunchKernelGGL(lstm_cell_bwd_kernel<4>, grid, block, 0, st, a);
   else hipLaunchKernelGGL(lstm_cell_bwd_kernel<1>, grid, block, 0, st, a);
   return lh::check_launch("lh_lstm_cell_bwd_f32");
+}
+
+extern "C" int lh_lstm_cell_bwd_f32(int H, int B, const float *dh_above, const float *dh_next,
+                                    const float *dc_next, const float *gates, const float *c,
+                                    const float *c_prev, const int *mask01, float clip_above,
+                                    float clip_next, const float *above_drop_mask, float keep,
+                                    float *dgates, float *dc_prev, lh_stream_t stream) {
+  const lh_error_term above{dh_above, 1, 0, H}, next{dh_next, 1, 0, H};
+  return lh_lstm_cell_bwd_terms_f32(H, B, &above, &next, dc_next, gates, c, c_prev, mask01, clip_above,
+                                    clip_next, above_drop_mask, keep, dgates, dc_prev, stream);
 }
 
 extern "C" int lh_rowsum_acc_f32(const float *A, long long lda, int rows, long long cols,

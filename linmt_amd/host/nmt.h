@@ -103,8 +103,14 @@ class LstmNode {
   // (NULL = none); dh_next / dc_next: errors from step t+1 (NULL = none).  The errors for step t-1
   // land in the layer's p_device_d_errn_to_t_ht_m1_ / _ct_m1_.  batched_dx: M^T d is left to one
   // GEMM over all steps (BackPropInputAllSteps).
-  void BackPropGpu(const float *dh_above, bool above_is_lstm, const float *dh_next,
-                   const float *dc_next, bool batched_dx);
+  // leave_planes: a W^T d product whose K range is split over workgroups stays in partial planes
+  // (the layer's error_planes_ buffers), described by the layer's d_h_prev_term_ and this node's
+  // d_x_term_, which the cell kernels of step t-1 / of the layer below add up as they read them;
+  // otherwise the products are reduced into p_device_d_errn_to_t_ht_m1_ / p_device_d_x_ and the
+  // terms name those.
+  void BackPropGpu(const lh_error_term &dh_above, bool above_is_lstm, const lh_error_term &dh_next,
+                   const float *dc_next, bool batched_dx, bool leave_planes);
+  lh_error_term d_x_term_{nullptr, 1, 0, 0};
   // The reference's own two-call form (node_input_to_hidden.h:139-140, node_hidden_to_hidden.h:
   // 133-134), same signatures: BackPropPreprocessGpu hands in the errors of step t+1,
   // BackPropGpu(index) runs the node's backward step on them and on p_device_d_errt_ht_, the
@@ -195,6 +201,10 @@ class LstmLayer {
   DeviceArray<float> p_device_small_w_grad_;  // E x (number of unique ids), layer 1
   DeviceArray<float> d_gates_all_, d_x_all_;  // per-step gate errors / input errors
   DeviceArray<float> p_device_d_errn_to_t_ht_m1_, p_device_d_errn_to_t_ct_m1_;  // recurrent errors
+  // partial planes of W_h^T d and M^T d of the step in flight (kErrorPlanes each)
+  static constexpr int kErrorPlanes = 4;
+  DeviceArray<float> d_h_prev_planes_, d_x_planes_;
+  lh_error_term d_h_prev_term_{nullptr, 1, 0, 0};  // the error for step t-1, as the last BackPropGpu left it
   DeviceArray<float> p_device_errn_to_t_h_tild_;  // Q^T d: error into the attention node of t-1
   DeviceArray<int> p_device_input_vocab_indices_wgrad_, p_device_wgrad_seg_start_,
       p_device_wgrad_seg_cols_;

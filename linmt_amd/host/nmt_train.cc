@@ -36,6 +36,8 @@ void Gemm(NeuralMachineTranslation &M, int tag, int rows, int cols, const lh_gem
   M.Gemm(tag, rows, cols, segs, nseg, tA, tX, beta, nullptr, LH_ACT_NONE, nullptr, C, ldc, what);
 }
 
+const lh_error_term kNoError{nullptr, 1, 0, 0};
+
 void RowSum(NeuralMachineTranslation &M, const float *A, long long lda, int rows, long long cols,
             float *out) {
   ProfileScope ps(M.profiler_, kTagRowSum, 4.0 * rows * (double)cols);
@@ -73,6 +75,8 @@ void LstmLayer::InitTraining() {
   d_x_all_.Alloc(in * B * T);
   p_device_d_errn_to_t_ht_m1_.Alloc(H * B);
   p_device_d_errn_to_t_ct_m1_.Alloc(H * B);
+  d_h_prev_planes_.Alloc(kErrorPlanes * ((H + 3) & ~size_t(3)) * B);
+  if (!input_layer_mode_) d_x_planes_.Alloc(kErrorPlanes * ((in + 3) & ~size_t(3)) * B);
   if (input_layer_mode_) {
     p_device_small_w_grad_.Alloc(in * B * T);
     p_device_input_vocab_indices_wgrad_.Alloc(B * T);
@@ -148,31 +152,59 @@ void LstmLayer::PreprocessWGrad(const int *p_host_indices, int current_length, i
   HipErrorWrapper(hipStreamSynchronize(s), "PreprocessWGrad");
 }
 
-void LstmNode::BackPropGpu(const float *dh_above, bool above_is_lstm, const float *dh_next,
-                           const float *dc_next, bool batched_dx) {
+namespace {
+// W^T d of one step (rows x B, K = 4H) for a consumer that adds partial planes itself: the product
+// goes to C, or stays in up to LstmLayer::kErrorPlanes planes of `planes`; returns what to read.
+lh_error_term ErrorProduct(NeuralMachineTranslation &M, const float *W, const float *d_gates, int rows,
+                           int B, int H, float *C, DeviceArray<float> &planes, bool leave_planes,
+                           const char *what) {
+  lh_gemm_seg seg{W, 4 * H, d_gates, 4 * H, 4 * H};
+  // (with split products switched on, the model's Gemm() decides which kernel forms the product)
+  if (!leave_planes || planes.size() == 0 || M.split_products_) {
+    Gemm(M, kTagErrorGemm, rows, B, &seg, 1, 1, 0, 0.f, C, rows, what);
+    return lh_error_term{C, 1, 0, rows};
+  }
+  const size_t bytes = planes.size() * sizeof(float);
+  int S = 1;
+  {
+    ProfileScope ps(M.profiler_, kTagErrorGemm, bytes, LstmLayer::kErrorPlanes, rows, B, &seg, 1, 1, 0);
+    LhErrorWrapper(lh_gemm_planes_f32(rows, B, &seg, 1, 1, 0, 0.f, C, rows, planes.get(), bytes,
+                                      LstmLayer::kErrorPlanes, &S, M.stream_),
+                   what);
+  }
+  if (S == 1) return lh_error_term{C, 1, 0, rows};
+  const int ld = (rows + 3) & ~3;
+  return lh_error_term{planes.get(), S, (long long)ld * B, ld};
+}
+}  // namespace
+
+void LstmNode::BackPropGpu(const lh_error_term &dh_above, bool above_is_lstm, const lh_error_term &dh_next,
+                           const float *dc_next, bool batched_dx, bool leave_planes) {
   LstmLayer &L = *p_layer_;
   NeuralMachineTranslation &M = *L.p_neural_mt_;
   hipStream_t s = M.stream_;
   const int H = L.lstm_size_, B = minibatch_size_;
   const float clip = M.cfg_.clip_cell_mode_ ? M.cfg_.error_clip_threshold_ : 0.f;
-  const bool drop = M.apply_dropout_ && L.out_dropout_ && dh_above != nullptr;
+  const bool drop = M.apply_dropout_ && L.out_dropout_ && dh_above.p != nullptr;
   {
-    ProfileScope ps(M.profiler_, kTagLstmCellBwd, (drop ? 60.0 : 56.0) * H * B);
-    LhErrorWrapper(lh_lstm_cell_bwd_f32(H, B, dh_above, dh_next, dc_next, p_device_gates_,
-                                        p_device_c_t_, p_device_c_t_prev_,
-                                        p_device_input_vocab_indices_01_, above_is_lstm ? clip : 0.f,
-                                        clip, drop ? p_device_out_dropout_mask_ : nullptr,
-                                        M.cfg_.dropout_rate_, p_device_d_gates_,
-                                        L.p_device_d_errn_to_t_ct_m1_.get(), s),
+    const int reads = (dh_above.p ? dh_above.planes : 0) + (dh_next.p ? dh_next.planes : 0);
+    ProfileScope ps(M.profiler_, kTagLstmCellBwd, ((drop ? 52.0 : 48.0) + 4.0 * reads) * H * B);
+    LhErrorWrapper(lh_lstm_cell_bwd_terms_f32(H, B, &dh_above, &dh_next, dc_next, p_device_gates_,
+                                              p_device_c_t_, p_device_c_t_prev_,
+                                              p_device_input_vocab_indices_01_, above_is_lstm ? clip : 0.f,
+                                              clip, drop ? p_device_out_dropout_mask_ : nullptr,
+                                              M.cfg_.dropout_rate_, p_device_d_gates_,
+                                              L.p_device_d_errn_to_t_ct_m1_.get(), s),
                    "LstmNode::BackPropGpu fused cell backward");
   }
-  lh_gemm_seg seg{L.p_device_w_h_stack_.get(), 4 * H, p_device_d_gates_, 4 * H, 4 * H};
-  Gemm(M, kTagErrorGemm, H, B, &seg, 1, 1, 0, 0.f, L.p_device_d_errn_to_t_ht_m1_.get(), H,
-       "LstmNode::BackPropGpu p_device_d_errn_to_t_ht_m1_");
+  // the planes the cell kernel has just read are free again
+  L.d_h_prev_term_ = ErrorProduct(M, L.p_device_w_h_stack_.get(), p_device_d_gates_, H, B, H,
+                                  L.p_device_d_errn_to_t_ht_m1_.get(), L.d_h_prev_planes_, leave_planes,
+                                  "LstmNode::BackPropGpu p_device_d_errn_to_t_ht_m1_");
   if (!batched_dx) {
-    lh_gemm_seg sm{L.p_device_m_stack_.get(), 4 * H, p_device_d_gates_, 4 * H, 4 * H};
-    Gemm(M, kTagErrorGemm, L.input_size_, B, &sm, 1, 1, 0, 0.f, p_device_d_x_, L.input_size_,
-         "LstmNode::BackPropGpu p_device_d_errn_to_t_h_below_");
+    d_x_term_ = ErrorProduct(M, L.p_device_m_stack_.get(), p_device_d_gates_, L.input_size_, B, H,
+                             p_device_d_x_, L.d_x_planes_, leave_planes,
+                             "LstmNode::BackPropGpu p_device_d_errn_to_t_h_below_");
   }
   if (L.feed_input_mode_ && 0 != index_) {
     lh_gemm_seg sq{L.p_device_q_stack_.get(), 4 * H, p_device_d_gates_, 4 * H, 4 * H};
@@ -191,8 +223,9 @@ void LstmNode::BackPropGpu(int index) {
   if (index != index_) throw LinmtError("LstmNode::BackPropGpu: index does not name this node");
   LstmLayer &L = *p_layer_;
   const bool above_is_lstm = L.layer_number_ < L.p_neural_mt_->cfg_.num_layers_ - 1;  // 0 = input layer
-  BackPropGpu(p_device_d_errt_ht_, above_is_lstm, p_device_d_errn_to_tp1_ht_,
-              p_device_d_errn_to_tp1_ct_, false);
+  const int H = L.lstm_size_;
+  BackPropGpu(lh_error_term{p_device_d_errt_ht_, 1, 0, H}, above_is_lstm,
+              lh_error_term{p_device_d_errn_to_tp1_ht_, 1, 0, H}, p_device_d_errn_to_tp1_ct_, false, false);
 }
 
 void LstmLayer::BackPropInputAllSteps(int steps) {
@@ -539,10 +572,11 @@ double NeuralMachineTranslation::ComputeGradients(
     }
     for (int l = L - 1; l >= 0; --l) {
       LstmLayer &Lt = TargetLayer(l);
-      const float *above = l == L - 1 ? dh_top : TargetLayer(l + 1).v_nodes_[t].p_device_d_x_;
+      const lh_error_term above =
+          l == L - 1 ? lh_error_term{dh_top, 1, 0, H} : TargetLayer(l + 1).v_nodes_[t].d_x_term_;
       const bool last = t == T - 1;
-      Lt.v_nodes_[t].BackPropGpu(above, l < L - 1, last ? nullptr : Lt.p_device_d_errn_to_t_ht_m1_.get(),
-                                 last ? nullptr : Lt.p_device_d_errn_to_t_ct_m1_.get(), l == 0);
+      Lt.v_nodes_[t].BackPropGpu(above, l < L - 1, last ? kNoError : Lt.d_h_prev_term_,
+                                 last ? nullptr : Lt.p_device_d_errn_to_t_ct_m1_.get(), l == 0, true);
     }
   }
   for (int l = 0; l < L; ++l) {
@@ -556,18 +590,18 @@ double NeuralMachineTranslation::ComputeGradients(
     for (int l = L - 1; l >= 0; --l) {
       LstmLayer &Ls = SourceLayer(l);
       for (int t = S - 1; t >= 0; --t) {
-        const float *above = nullptr;
+        lh_error_term above = kNoError;
         if (l == L - 1) {
-          if (attention) above = attention_layer_.p_device_total_hs_error_.get() + (size_t)H * B * t;
+          if (attention) above.p = attention_layer_.p_device_total_hs_error_.get() + (size_t)H * B * t;
         } else {
-          above = SourceLayer(l + 1).v_nodes_[t].p_device_d_x_;
+          above.p = SourceLayer(l + 1).v_nodes_[t].p_device_d_x_;  // of BackPropInputAllSteps
         }
+        above.ld = H;
         const bool last = t == S - 1;  // the decoder's step 0 hands its errors to this layer
-        const float *dhn = last ? TargetLayer(l).p_device_d_errn_to_t_ht_m1_.get()
-                                : Ls.p_device_d_errn_to_t_ht_m1_.get();
+        const lh_error_term dhn = last ? TargetLayer(l).d_h_prev_term_ : Ls.d_h_prev_term_;
         const float *dcn = last ? TargetLayer(l).p_device_d_errn_to_t_ct_m1_.get()
                                 : Ls.p_device_d_errn_to_t_ct_m1_.get();
-        Ls.v_nodes_[t].BackPropGpu(above, l < L - 1, dhn, dcn, true);
+        Ls.v_nodes_[t].BackPropGpu(above, l < L - 1, dhn, dcn, true, true);
       }
       if (l > 0) Ls.BackPropInputAllSteps(S);
       Ls.ComputeGradientsAllSteps(S, nullptr, nullptr);

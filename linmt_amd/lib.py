@@ -150,6 +150,9 @@ SIGNATURES = {
     "lh_lstm_cell_bwd_f32": (C.c_int, [C.c_int, C.c_int, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p,
                                        c_f32p, c_i32p, C.c_float, C.c_float, c_f32p, C.c_float,
                                        c_f32p, c_f32p, C.c_void_p]),
+    "lh_lstm_cell_bwd_terms_f32": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p, c_f32p, c_f32p,
+                                             c_f32p, c_f32p, c_i32p, C.c_float, C.c_float, c_f32p,
+                                             C.c_float, c_f32p, c_f32p, C.c_void_p]),
     "lh_rowsum_acc_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_int, C.c_longlong, C.c_float, c_f32p,
                                     C.c_void_p]),
     "lh_embed_gather_grad_f32": (C.c_int, [c_f32p, C.c_longlong, C.c_int, C.c_int, c_i32p, c_i32p,
@@ -558,6 +561,27 @@ def lstm_cell_bwd(H, B, gates, c, c_prev, mask01, dgates, dc_prev, dh_above=None
                                       clip_next, _ptr(above_drop_mask), keep, _ptr(dgates),
                                       _ptr(dc_prev), _stream(stream)),
           "lh_lstm_cell_bwd_f32")
+
+
+class ErrorTerm(C.Structure):
+    """lh_error_term: an incoming error as the sum of `planes` H x B blocks (ld, plane_stride in floats)."""
+    _fields_ = [("p", C.c_void_p), ("planes", C.c_int), ("plane_stride", C.c_longlong), ("ld", C.c_int)]
+
+
+def error_term(t, planes, ld, plane_stride=0):
+    return ErrorTerm(t.data_ptr(), planes, plane_stride, ld)
+
+
+def lstm_cell_bwd_terms(H, B, gates, c, c_prev, mask01, dgates, dc_prev, above=None, next=None,
+                        dc_next=None, clip_above=0.0, clip_next=0.0, above_drop_mask=None, keep=1.0,
+                        stream=None):
+    """above / next: ErrorTerm or None."""
+    check(load().lh_lstm_cell_bwd_terms_f32(H, B, C.byref(above) if above is not None else None,
+                                            C.byref(next) if next is not None else None, _ptr(dc_next),
+                                            _ptr(gates), _ptr(c), _ptr(c_prev), _ptr(mask01), clip_above,
+                                            clip_next, _ptr(above_drop_mask), keep, _ptr(dgates),
+                                            _ptr(dc_prev), _stream(stream)),
+          "lh_lstm_cell_bwd_terms_f32")
 
 
 def rowsum_acc(A, lda, rows, cols, out, beta=0.0, stream=None):

@@ -42,6 +42,57 @@ def test_lstm_cell_bwd(lh, orc, H, B, clip):
     assert_close(host(dc, (H, B)), want_dc, "dc_prev (dropout)")
 
 
+@pytest.mark.parametrize("H,B,ld,planes_above,planes_next", [(64, 12, 64, 2, 3), (100, 7, 100, 3, 1),
+                                                             (48, 5, 52, 1, 2), (33, 4, 36, 2, 2),
+                                                             (2048, 256, 2048, 2, 2)])
+def test_lstm_cell_bwd_error_terms_as_partial_planes(lh, H, B, ld, planes_above, planes_next):
+    """lh_lstm_cell_bwd_terms_f32 on the planes of a split product gives the bits lh_lstm_cell_bwd_f32
+    gives on their sum, added in plane order from +0 as the product's reduction launch adds them
+    (a -0 in the first plane included), with clamp and dropout mask on the sum."""
+    rng = np.random.default_rng(52)
+    gates = rng.random((4 * H, B)).astype(np.float32)
+    gates[2 * H:3 * H] = 2 * gates[2 * H:3 * H] - 1
+    c, c_prev = uni(rng, H, B), uni(rng, H, B)
+    mask = (rng.random(B) > 0.2).astype(np.int32)
+    dcn = uni(rng, H, B, s=0.1)
+    u = rng.random((H, B)).astype(np.float32)
+
+    def planes_of(n):
+        p = np.zeros((n, B, ld), np.float32)
+        p[:, :, :H] = rng.uniform(-0.1, 0.1, size=(n, B, H)).astype(np.float32)
+        p[:, :, H:] = np.nan  # padding rows of a plane are never read
+        p[0, 0, 0] = -0.0
+        if n > 1:
+            p[1:, 0, 0] = 0.0
+        total = np.zeros((B, H), np.float32)
+        for k in range(n):
+            total = total + p[k, :, :H]
+        return p, np.ascontiguousarray(total.T)  # H x B, as the plain entry point takes it
+
+    pa, sum_a = planes_of(planes_above)
+    pn, sum_n = planes_of(planes_next)
+    for clip, drop in ((0.0, False), (0.05, True)):
+        want_dg = torch.empty(4 * H * B, device="cuda")
+        want_dc = torch.empty(H * B, device="cuda")
+        lh.lstm_cell_bwd(H, B, dev(gates), dev(c), dev(c_prev), dev(mask), want_dg, want_dc, dev(sum_a),
+                         dev(sum_n), dev(dcn), clip, clip, dev(u) if drop else None, 0.7)
+        dg = torch.empty(4 * H * B, device="cuda")
+        dc = torch.empty(H * B, device="cuda")
+        da, dn = torch.from_numpy(pa).cuda(), torch.from_numpy(pn).cuda()
+        lh.lstm_cell_bwd_terms(H, B, dev(gates), dev(c), dev(c_prev), dev(mask), dg, dc,
+                               lh.error_term(da, planes_above, ld, B * ld), lh.error_term(dn, planes_next, ld, B * ld),
+                               dev(dcn), clip, clip, dev(u) if drop else None, 0.7)
+        torch.cuda.synchronize()
+        assert torch.equal(dg.view(torch.int32), want_dg.view(torch.int32)), "dgates bits"
+        assert torch.equal(dc.view(torch.int32), want_dc.view(torch.int32)), "dc_prev bits"
+    with pytest.raises(lh.LinmtHipError):
+        lh.lstm_cell_bwd_terms(H, B, dev(gates), dev(c), dev(c_prev), dev(mask), dg, dc,
+                               lh.error_term(da, 9, ld, B * ld), None)
+    with pytest.raises(lh.LinmtHipError):
+        lh.lstm_cell_bwd_terms(H, B, dev(gates), dev(c), dev(c_prev), dev(mask), dg, dc,
+                               lh.error_term(da, 1, H - 1), None)
+
+
 @pytest.mark.parametrize("V,B", [(5000, 32), (30000, 24), (37, 5), (50000, 8)])
 def test_softmax_xent_grad(lh, orc, V, B):
     rng = np.random.default_rng(51)

@@ -131,6 +131,47 @@ def test_compute_gradients_with_split_products_vs_oracle(orc, host, case):
     gm.close()
 
 
+@pytest.mark.parametrize("case", [CASES[0], CASES[3], CASES[4]],
+                         ids=lambda c: f"L{c['layers']}H{c['H']}E{c.get('E', 0)}a{c['attention']}f{c['feed']}")
+def test_compute_gradients_with_error_products_left_in_planes(orc, host, case):
+    """The per-step W^T d products of ComputeGradients stay in partial planes when their K range is
+    split over workgroups, and the cell kernel of step t-1 / of the layer below adds the planes as
+    it reads them.  At these sizes no product would be split by itself (at H = 2048 they are:
+    tests/test_gpu_configs_at_size.py), so a split of 2 is forced: same gradients against the
+    oracle.  (That the cell kernel gives the bits of the reduced product is
+    tests/test_gpu_train_kernels.py::test_lstm_cell_bwd_error_terms_as_partial_planes.)"""
+    import torch
+    from linmt_amd import lib as lh
+    rng = np.random.default_rng(case["seed"])
+    Vs, Vt = 29, 41
+    lens_s, lens_t = [5, 3, 9, 4, 7, 1], [4, 6, 2, 8, 5, 3]
+    B = len(lens_s)
+    P, om, gm = _pair(orc, host, rng, case["layers"], case["H"], Vs, Vt, case["D"],
+                      case["attention"], case["feed"], B, dict(grad_clip_mode=0), E=case.get("E"))
+    sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
+    want_ll, want = om.compute_gradients(src, tin, tout, bi, su, tu)
+    L = lh.load()
+    H = case["H"]
+    try:
+        L.lh_gemm_set_splits_override(2)
+        # the product of a step is indeed left in two planes at this size
+        ws = torch.empty(4 * ((H + 3) & ~3) * B, device="cuda")
+        a = torch.zeros(4 * H * H, device="cuda")
+        x = torch.zeros(4 * H * B, device="cuda")
+        out = torch.zeros(H * B, device="cuda")
+        assert lh.gemm_planes(H, B, [(a, 4 * H, x, 4 * H, 4 * H)], out, H, ws, 4, transA=True) == 2
+        got_ll = gm.compute_gradients(src, tin, tout, bi, su, tu)
+        grads = {name: gm.get_grad(name, _grad_shape(P, name, su, tu)) for name in om.param_names()}
+    finally:
+        L.lh_gemm_set_splits_override(0)
+    assert_close(got_ll, want_ll, "sum log p(target)", rtol=1e-5, atol=1e-4)
+    for name in om.param_names():
+        shape = _grad_shape(P, name, su, tu)
+        assert_close(grads[name], np.asarray(want[name]).reshape(shape, order="F"), f"gradient of {name}",
+                     atol=2e-5)
+    gm.close()
+
+
 @pytest.mark.parametrize("case", [CASES[0], CASES[2], CASES[3], CASES[4], CASES[5]],
                          ids=lambda c: f"L{c['layers']}H{c['H']}E{c.get('E', 0)}a{c['attention']}f{c['feed']}")
 def test_stepwise_reference_calls_give_the_same_gradients(orc, host, case):
