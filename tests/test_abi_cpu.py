@@ -49,3 +49,21 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(lib.LinmtHipError):
         lib.load()
+
+
+def test_c_headers_compile_as_plain_c(tmp_path):
+    """The boundary is a C ABI: both headers that declare it are valid C99 on their own (no C++,
+    no HIP or torch types), so a cgo / JNI / ctypes-style binding can include them as they are."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_headers.c"
+    src.write_text('#include "linmt_hip.h"\n#include "linmt_host.h"\n'
+                   "int main(void) { lh_error_term t = {0, 1, 0, 4}; lh_gemm_seg s = {0, 0, 0, 0, 0};\n"
+                   "  return t.planes - 1 + s.K; }\n")
+    r = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I",
+                        os.path.join(ROOT, "include"), "-c", str(src), "-o", str(tmp_path / "use_headers.o")],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
