@@ -172,3 +172,50 @@ def test_decode_batch_equals_lone_sentences_bit_for_bit(host):
         L.lh_gemm_set_config_override(-1)
         L.lh_gemm_set_splits_override(0)
     assert sentences > 50
+
+
+def test_decode_batch_ensemble_and_alignments_equal_lone_sentences_bit_for_bit(host):
+    """The same for two models decoded in lockstep (each on its own stream, their distributions
+    averaged by the top-k kernel) with exported alignments: tokens, finished hypotheses, score
+    bits and the 1-best's source positions of a sentence do not depend on its neighbours."""
+    import ref_numpy as R
+    from linmt_amd import lib as lh
+    L = lh.load()
+    rng = np.random.default_rng(12)
+    sentences = 0
+    try:
+        L.lh_gemm_set_config_override(7)
+        L.lh_gemm_set_splits_override(1)
+        for trial in range(8):
+            layers = int(rng.integers(1, 4)); H = int(rng.choice([32, 48, 64, 100]))
+            Vs = int(rng.integers(30, 200)); Vt = 4 * int(rng.integers(10, 75))  # ensembles: a multiple of 4
+            D = int(rng.integers(1, 8)); beam = int(rng.integers(2, 9)); slots = int(rng.integers(3, 7))
+            feed = bool(rng.integers(0, 2)); scale = float(rng.choice([0.2, 0.4]))
+            beam = min(beam, int(np.sqrt(Vt)))
+            gms = []
+            for _ in range(2):
+                P = R.make_params(rng, layers, H, Vs, Vt, attention=True, feed_input=feed, scale=scale)
+                gm = host.Model(layers, H, Vs, Vt, longest_sentence=44, attention_mode=1, attention_width=D,
+                                feed_input=feed, decoding=(slots, beam))
+                gm.set_params(P)
+                gms.append(gm)
+            n = int(rng.integers(2, slots))
+            sents = [rng.integers(0, Vs, size=int(rng.integers(1, 25))) for _ in range(n)]
+            got = gms[0].decode_batch(sents, beam=beam, with_hyps=True, ensemble=gms[1:], alignments=True)
+            for i, s in enumerate(sents):
+                w = gms[0].decode_batch([s], beam=beam, with_hyps=True, ensemble=gms[1:], alignments=True)[0]
+                what = f"trial {trial} (layers {layers}, H {H}, beam {beam}, n_sent {slots}, n {n}, feed {feed}) sentence {i}"
+                assert got[i]["steps"] == w["steps"], what
+                assert got[i]["best"].tolist() == w["best"].tolist(), what
+                assert got[i]["best_score"] == w["best_score"], what
+                assert got[i]["best_viterbi"].tolist() == w["best_viterbi"].tolist(), what
+                assert len(got[i]["hyps"]) == len(w["hyps"]), what
+                for (gt, gs), (wt, ws) in zip(got[i]["hyps"], w["hyps"]):
+                    assert gt.tolist() == wt.tolist() and gs == ws, what
+            sentences += n
+            for gm in gms:
+                gm.close()
+    finally:
+        L.lh_gemm_set_config_override(-1)
+        L.lh_gemm_set_splits_override(0)
+    assert sentences >= 16
