@@ -527,7 +527,7 @@ int lh_beam_merge_gather_f32(int n_sent, int beam, int K, int step, const int *l
  * n_tensors state tensors (src_t is H x n_src: the encoder's final states, what
  * TransferDecodingStatesGpu broadcasts, src/layer_input_to_hidden.h:1536-1545) and zero_t[:, c] = 0
  * for the n_zero tensors that start a sentence at zero (h~ of the step before).  src / dst / zero
- * are HOST arrays of device pointers. */
+ * are HOST arrays of device pointers.  The admissions of a call name different slots. */
 #define LH_STREAM_ADMIT_MAX 16
 typedef struct {
   int slot, sentence_col, hs_col_value, len, off, limit, tick;

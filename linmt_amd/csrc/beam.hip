@@ -385,6 +385,9 @@ extern "C" int lh_stream_admit_f32(const lh_stream_admission *adm, int n_adm, in
     if (q.slot < 0 || (q.slot + 1) * beam > B || q.sentence_col < 0 || q.sentence_col >= n_src)
       return lh::fail_arg("%s: admission %d: slot %d / sentence column %d out of range", who, i, q.slot,
                           q.sentence_col);
+    for (int k = 0; k < i; ++k)
+      if (adm[k].slot == q.slot)
+        return lh::fail_arg("%s: admissions %d and %d name the same slot %d", who, k, i, q.slot);
     a.adm[i] = q;
   }
   a.beam = beam, a.B = B, a.H = H, a.n_src = n_src, a.n_tensors = n_tensors, a.n_zero = n_zero;

@@ -975,6 +975,9 @@ def test_stream_admission_and_merge_at_different_steps(lh):
     with pytest.raises(lh.LinmtHipError):
         lh.stream_admit([dict(adm[0], slot=n_sent)], beam, B, start, limit, hs_col, binfo, finals, states,
                         [tild], H, n_src, tok_prev, 0, score_prev)
+    with pytest.raises(lh.LinmtHipError):   # two sentences into one slot in one launch
+        lh.stream_admit([adm[0], dict(adm[1], slot=adm[0]["slot"])], beam, B, start, limit, hs_col, binfo,
+                        finals, states, [tild], H, n_src, tok_prev, 0, score_prev)
 
     # merge + gather with sentences at steps 0, 3, == limit, > limit and in a slot that idles
     tick = 50
