@@ -263,3 +263,63 @@ def test_k_best_lists(host, tmp_path):
         del os.environ["LINMT_NO_STREAM"]
     lines2 = open(ids2).read().split("\n")[:-1]
     assert [l.split(" |||| ")[0] for l in lines2] == [l.split(" |||| ")[0] for l in lines]
+
+
+def test_decoding_a_long_text_file_through_the_stream(host, tmp_path):
+    """Dispatcher::Decoding with one model and no exported alignments hands the file to
+    DecodeStream 32 batches at a time: 150 lines at two sentences per batch are three such lists
+    (64 + 64 + 22), one of them with an empty line inside.  Every line must be what DecodeStream
+    gives for the same list on a model loaded from the same file (same launches, so exactly), and
+    the batch-by-batch path of the dispatcher must give the same tokens."""
+    import os
+    rng = np.random.default_rng(31)
+    layers, H, Vs, Vt, D, beam, n_sent = 2, 24, 30, 40, 2, 4, 2
+    P = R.make_params(rng, layers, H, Vs, Vt, attention=True, feed_input=True, scale=0.4)
+    kw = dict(longest_sentence=24, attention_mode=1, attention_width=D, feed_input=True)
+    a = host.Model(layers, H, Vs, Vt, minibatch_size=1, **kw)
+    a.set_params(P)
+    model = str(tmp_path / "model.nmt")
+    a.dump_model(model)
+    a.close()
+    sents = [rng.integers(0, Vs, size=int(rng.integers(1, 15))) for _ in range(149)]
+    word = lambda i: "<UNK>" if i == 0 else f"w{i}"  # noqa: E731
+    lines = [" ".join(word(i) for i in s_) for s_ in sents]
+    lines.insert(70, "")  # an empty line inside the second list
+    src = tmp_path / "src.txt"
+    src.write_text("\n".join(lines) + "\n")
+    ids = str(tmp_path / "out.ids")
+    rep = host.decoding(model, str(src), str(tmp_path / "out.txt"), ids_file=ids, beam=beam,
+                        longest_sentence=24, attention_width=D, print_decoding_information=True,
+                        sentences_per_batch=n_sent)
+    assert rep["sentences"] == 150 and rep["sentences_thrown_away"] == 0
+    got = open(ids).read().split("\n")[:-1]
+    assert len(got) == 150 and got[70] == ""
+    b = host.Model(layers, H, Vs, Vt, decoding=(n_sent, beam), **kw)
+    b.load_weights(model)
+    chunk = 32 * n_sent
+    want = []
+    for first in range(0, 150, chunk):
+        block = [(i, lines[i]) for i in range(first, min(150, first + chunk)) if lines[i]]
+        res = b.decode_stream([sents[i if i < 70 else i - 1] for i, _ in block], beam=beam)
+        it = iter(res)
+        want += [next(it) if lines[i] else None for i in range(first, min(150, first + chunk))]
+    b.close()
+    for k, (line, w) in enumerate(zip(got, want)):
+        if w is None:
+            assert line == "", k
+            continue
+        fields = line.split(" |||| ")
+        assert [int(x) for x in fields[0].split()] == w["best"].tolist(), k
+        assert np.isclose(float(fields[1]), w["best_score"], rtol=1e-5, atol=1e-4), k  # six digits in the file
+    assert rep["target_words"] == sum(len(w["best"]) for w in want if w is not None)
+    os.environ["LINMT_NO_STREAM"] = "1"
+    try:
+        ids2 = str(tmp_path / "out2.ids")
+        host.decoding(model, str(src), str(tmp_path / "out2.txt"), ids_file=ids2, beam=beam,
+                      longest_sentence=24, attention_width=D, print_decoding_information=True,
+                      sentences_per_batch=n_sent)
+    finally:
+        del os.environ["LINMT_NO_STREAM"]
+    got2 = open(ids2).read().split("\n")[:-1]
+    same = sum(x.split(" |||| ")[0] == y.split(" |||| ")[0] for x, y in zip(got, got2))
+    assert len(got2) == 150 and same >= 147, same  # a near-tie may fall the other way between the two modes
