@@ -219,3 +219,22 @@ def test_decode_batch_ensemble_and_alignments_equal_lone_sentences_bit_for_bit(h
         L.lh_gemm_set_config_override(-1)
         L.lh_gemm_set_splits_override(0)
     assert sentences >= 16
+
+
+@pytest.mark.parametrize("feed", [False, True])
+def test_decode_stream_at_the_longest_sentence_length(orc, host, feed):
+    """Sentences as long as the model allows: their step count is cut at longest_sentence - 2
+    (decoder.h:1734) instead of 1.5 x length, next to one-word sentences that leave their slot
+    after two steps.  Against the oracle's single-sentence search."""
+    rng = np.random.default_rng(5 + int(feed))
+    layers, H, Vs, Vt, D, beam, slots, longest = 2, 32, 50, 60, 3, 4, 3, 20
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, longest, 0.4, decoding=(slots, beam), feed=feed)
+    sents = [rng.integers(0, Vs, size=int(rng.choice([20, 20, 19, 14, 1, 13]))) for _ in range(11)]
+    sents[0] = rng.integers(0, Vs, size=20)
+    sents[1] = rng.integers(0, Vs, size=1)
+    got = gm.decode_stream(sents, beam=beam, with_hyps=True)
+    for i, s in enumerate(sents):
+        want = om.decode_sentence(s, beam=beam)
+        assert want["steps"] == (19 if len(s) >= 13 else 2)
+        _compare_decode(want, got[i], f"sentence {i} (len {len(s)})")
+    gm.close()
