@@ -131,7 +131,7 @@ def test_compute_gradients_with_split_products_vs_oracle(orc, host, case):
     gm.close()
 
 
-@pytest.mark.parametrize("case", [CASES[0], CASES[3], CASES[4]],
+@pytest.mark.parametrize("case", [CASES[0], CASES[2], CASES[3], CASES[4], CASES[5]],
                          ids=lambda c: f"L{c['layers']}H{c['H']}E{c.get('E', 0)}a{c['attention']}f{c['feed']}")
 def test_compute_gradients_with_error_products_left_in_planes(orc, host, case):
     """The per-step W^T d products of ComputeGradients stay in partial planes when their K range is
