@@ -2,12 +2,18 @@
 """Benchmark of the hot path on one MI355X: beam-12 decoding of the 4+4-layer, 1000-hidden,
 30k-vocabulary encoder-decoder with local-p attention and input feeding (BASELINE.json configs[2]).
 
-One "step" = one pass of the hot path over one batch: a full batched beam search (encoder, every
-decoder step with on-device top-k / merge / state gather, hypothesis read-back) over 64 synthetic
-source sentences.  Prints ONE JSON line: metric / value / unit (whole-job target tokens per second,
-inputs resident on the device), ms_per_step, the workload in `config`, `roofline` for the dominant
-kernel (live HIP-event timing of its launches against the fp32 MFMA peak, measured HBM traffic),
-`cpu_baseline` (the CPU restatement on the host cores, same sentences) and `parity` (1-best of both).
+One "step" = one pass of the hot path over 64 synthetic source sentences: encoder, every decoder
+step with on-device top-k / merge / state gather, hypothesis read-back.  The sentences of all
+`steps` are handed over as ONE list and decoded 64 at a time with every one of the 768 beam columns
+busy in every step of the search (a finished sentence's columns go to the next sentence of the
+list: lnmt_decode_stream, the driver Dispatcher::Decoding uses).  Prints ONE JSON line: metric /
+value / unit (whole-job target tokens per second), ms_per_step, the workload in `config`,
+`roofline` for the dominant kernel (live HIP-event timing of its launches against the fp32 MFMA
+peak, measured HBM traffic), `step` (the matrix-product flop of one step of 768 hypotheses over the
+measured time per step, against the same peak), `hbm_kernels`, `cpu_baseline` (the CPU restatement
+on the host cores, same sentences), `parity` (every sentence's search against the oracle's), and
+beside them `batch` (the same sentences one batch after the other, lnmt_decode_batch) and
+`split_products` (the opt-in arithmetic).
 
   python bench.py --gpus 1 --steps K --warmup W
 
@@ -32,7 +38,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 MFMA, MI355X
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over this script (KiB per dispatch at the
 # grid of 768 live columns; FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a device copy of
 # known size gives).  A counter run cannot happen inside the timed run, so the figure is carried
-# here; its algorithmic counterpart is 30000*1000*4 + 768*1000*4 read + 30000*768*4 written.
+# here, from the counter runs whose summary is kept under profiles/ (the decode kernel profile's
+# traffic section names the commands); its algorithmic counterpart is 30000*1000*4 + 768*1000*4
+# read + 30000*768*4 written.
 MEASURED_TRAFFIC_BYTES = {
     "gemm_kernel<64, 64, 2, 2, 1, 16, false, false>": int((235759 + 92723) * 1024),
     "gemm_kernel<128, 96, 4, 1, 1, 16, false, false>": int((240671 + 89778) * 1024),
@@ -179,6 +187,14 @@ def bench_fused_kernels(torch, steps, warmup, quick=False):
     n = big(256, 64) * 1024 * 1024
     src, dst = f(n), torch.empty(n, device=dev)
     add("device copy (calibration)", f"{n} floats", 8.0 * n, lambda: dst.copy_(src))
+    # calibration for the kernels that only read (log-softmax + loss, beam top-k): n floats read,
+    # nothing written -- the library's sum and this library's own sum of squares (lh_grad_sumsq_f32)
+    add("read-only pass (calibration, library sum)", f"{n} floats", 4.0 * n, lambda: torch.sum(src))
+    ws = torch.zeros(lh.LH_SUMSQ_WORKSPACE, dtype=torch.float64, device=dev)
+    acc = torch.zeros(1, dtype=torch.float64, device=dev)
+    add("read-only pass (calibration, lh_grad_sumsq_f32)", f"{n} floats", 4.0 * n,
+        lambda: lh.grad_sumsq(src, n, 1, n, 1.0, ws, acc))
+    read_ceiling = max(r["GB/s"] for r in out if r["kernel"].startswith("read-only pass"))
     del src, dst
     for H, B in big(((1000, 768), (1000, 768 * 64), (2048, 256 * 32)), ((1000, 768), (1000, 768 * 16))):
         pre, bias, cp = f(4 * H * B), f(4 * H), f(H * B)
@@ -205,8 +221,10 @@ def bench_fused_kernels(torch, steps, warmup, quick=False):
             lambda: lh.softmax_fwd(z, V, None, V, B, p, V))
         add("logsoftmax_xent (double)", f"V={V} B={B}", 4.0 * V * B,
             lambda: lh.logsoftmax_xent(z, V, None, V, B, tgt, m, lp, loss))
+        out[-1]["frac_of_read_only_ceiling"] = round(out[-1]["GB/s"] / read_ceiling, 4)
         add("beam_topk (log-softmax + top-13)", f"V={V} B={B}", 4.0 * V * B,
             lambda: lh.beam_topk(z, V, None, V, B, K, 1, cl, ci, le))
+        out[-1]["frac_of_read_only_ceiling"] = round(out[-1]["GB/s"] / read_ceiling, 4)
         if B == 768 and not quick:
             # an ensemble of two models: both distributions are read once
             p2 = torch.empty(V * B, device=dev)
@@ -256,7 +274,7 @@ def bench_fused_kernels(torch, steps, warmup, quick=False):
             lambda: lh.embed_lookup(Wm, E, V, idx, B, o))
         del Wm, o
     return {"metric": "fused-kernel HBM GB/s % of peak", "unit": "GB/s", "peak": HBM_PEAK_GBS,
-            "launches_timed": steps, "kernels": out}
+            "read_only_ceiling_GB/s": read_ceiling, "launches_timed": steps, "kernels": out}
 
 
 def bench_mfma_kernels(torch, steps, warmup):
@@ -442,9 +460,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hbm-kernels", action="store_true",
                     help="skip the stand-alone timing of the HBM-bound kernels (hbm_kernels field)")
-    ap.add_argument("--no-stream", action="store_true",
-                    help="skip the extra leg that decodes the same sentences with every beam column "
-                         "kept busy (lnmt_decode_stream; reported beside `value`, never as it)")
+    ap.add_argument("--no-batch", action="store_true",
+                    help="skip the extra leg that decodes the same sentences one batch after the "
+                         "other (lnmt_decode_batch; reported beside `value`, never as it)")
     ap.add_argument("--no-split-products", action="store_true",
                     help="skip the second timing of the same batch with the opt-in arithmetic "
                          "(lnmt_set_split_products; reported beside `value`, never as it)")
@@ -503,144 +521,142 @@ def main():
     # about the opt-in arithmetic, which its metric then names)
     model.set_split_products(bool(args.split_products_only))
 
-    for _ in range(args.warmup):
-        model.decode_batch(sents, beam=beam)
+    def gemm_roofline(totals, site_prefix="logits_gemm"):
+        """The GEMM kernel instance that carries the most algorithmic work among the bracketed
+        launches of a call site: achieved = sum of flop / sum of launch durations."""
+        by_kernel = {}
+        for key, t in totals.items():
+            if "|" not in key or not key.startswith(site_prefix):
+                continue
+            site, kern = key.split("|", 1)
+            e = by_kernel.setdefault(kern, dict(ms=0.0, work=0.0, launches=0, sites=set()))
+            e["ms"] += t["ms"]
+            e["work"] += t["work"]
+            e["launches"] += t["launches"]
+            e["sites"].add(site)
+        if not by_kernel:
+            return None
+        kern, g = max(by_kernel.items(), key=lambda kv: kv[1]["work"])
+        achieved = g["work"] / (g["ms"] * 1e-3) / 1e12
+        r = {"kernel": kern, "call_sites": sorted(g["sites"]), "bound": "mfma",
+             "achieved": round(achieved, 2), "peak": MFMA_FP32_PEAK_TFLOPS,
+             "unit": "TFLOP/s", "frac": round(achieved / MFMA_FP32_PEAK_TFLOPS, 4),
+             "traffic": MEASURED_TRAFFIC_BYTES.get(kern), "launches": g["launches"],
+             "avg_launch_us": round(g["ms"] * 1e3 / g["launches"], 2)}
+        if kern.startswith("gemm_split_kernel"):  # six bf16 products issued per algorithmic product
+            r.update({"algorithmic_TFLOP/s": round(achieved, 2), "achieved": round(6 * achieved, 1),
+                      "peak": MFMA_BF16_PEAK_TFLOPS,
+                      "unit": "TFLOP/s (bf16 products issued = 6 x algorithmic)",
+                      "frac": round(6 * achieved / MFMA_BF16_PEAK_TFLOPS, 4)})
+        return r
+
+    def kernel_table(totals):
+        out = {}
+        for name, t in sorted(totals.items()):
+            rate = t["work"] / (t["ms"] * 1e-3)
+            is_gemm = "|" in name
+            out[name] = {"ms": round(t["ms"], 3), "launches": t["launches"],
+                         "rate": round(rate / (1e12 if is_gemm else 1e9), 2),
+                         "unit": "TFLOP/s" if is_gemm else "GB/s",
+                         "frac": round(rate / ((MFMA_FP32_PEAK_TFLOPS * 1e12) if is_gemm
+                                               else (HBM_PEAK_GBS * 1e9)), 4)}
+        return out
+
+    # ---- the measured hot path: the sentences of `steps` batches as ONE list through the 64 slots ----
+    # One "step" = 64 source sentences through the decoder.  A sentence that has taken its last
+    # step hands its 12 beam columns to the next sentence of the list (lnmt_decode_stream, what
+    # Dispatcher::Decoding runs), so every step of the search runs all 768 hypotheses: encoder in
+    # groups of 64, one read-back at the end, the whole call inside the timed region.
+    B = n_sent * beam
+    model.profile(0)
+    model.decode_stream(sents * max(args.warmup, 1), beam=beam)
     model.profile(1 if args.profile_level >= 1 else 0)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    tokens = 0
-    for _ in range(args.steps):
-        res = model.decode_batch(sents, beam=beam)  # ends with a stream synchronisation
-        tokens += sum(len(r["best"]) for r in res)
+    res_all = model.decode_stream(sents * args.steps, beam=beam)  # ends with a stream synchronisation
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     prof1 = model.profile_totals()
+    ticks = model.stream_ticks
+    tokens = sum(len(r["best"]) for r in res_all)
     ms_per_step = dt * 1e3 / args.steps
     value = tokens / dt
+    res = res_all[:n_sent]
+    histories = [model.decode_history(i, beam) for i in range(n_sent)]
+    copies_same = all(res_all[i]["best"].tolist() == res_all[i % n_sent]["best"].tolist()
+                      for i in range(len(res_all)))
+    roofline = gemm_roofline(prof1)
+    # The whole step against the MFMA roofline: the matrix products of one tick of 768 hypotheses
+    # (gate products of every layer, the attention projections, the output projection) over the
+    # measured time per tick -- everything else the tick does (attention, top-k, merge, state
+    # gather, the encoder of the coming groups, admissions) counts as time and not as work.
+    flop_per_column = layers * 2.0 * 4 * H * 2 * H + 2.0 * 2 * H * H + 2.0 * V * H
+    tick_us = dt * 1e6 / ticks
+    step_tflops = flop_per_column * B / tick_us / 1e6
+    step = {"ticks": ticks, "hypotheses_per_tick": B, "tick_us": round(tick_us, 1),
+            "mfma_flop_per_tick": flop_per_column * B, "achieved": round(step_tflops, 2),
+            "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(step_tflops / MFMA_FP32_PEAK_TFLOPS, 4)}
 
-    # dominant kernel = the GEMM kernel instance that carries the most algorithmic work (flop) in the
-    # timed steps: the output projection D*h~ + b_d
-    roofline = None
-    by_kernel = {}
-    for key, t in prof1.items():
-        if "|" not in key:
-            continue
-        site, kern = key.split("|", 1)
-        e = by_kernel.setdefault(kern, dict(ms=0.0, work=0.0, launches=0, sites=set()))
-        e["ms"] += t["ms"]
-        e["work"] += t["work"]
-        e["launches"] += t["launches"]
-        e["sites"].add(site)
-    if by_kernel:
-        kern, g = max(by_kernel.items(), key=lambda kv: kv[1]["work"])
-        achieved = g["work"] / (g["ms"] * 1e-3) / 1e12
-        roofline = {"kernel": kern, "call_sites": sorted(g["sites"]), "bound": "mfma",
-                    "achieved": round(achieved, 2), "peak": MFMA_FP32_PEAK_TFLOPS,
-                    "unit": "TFLOP/s", "frac": round(achieved / MFMA_FP32_PEAK_TFLOPS, 4),
-                    "traffic": MEASURED_TRAFFIC_BYTES.get(kern), "launches": g["launches"],
-                    "avg_launch_us": round(g["ms"] * 1e3 / g["launches"], 2)}
-        if kern.startswith("gemm_split_kernel"):  # six bf16 products issued per algorithmic product
-            roofline.update({"algorithmic_TFLOP/s": round(achieved, 2), "achieved": round(6 * achieved, 1),
-                             "peak": MFMA_BF16_PEAK_TFLOPS,
-                             "unit": "TFLOP/s (bf16 products issued = 6 x algorithmic)",
-                             "frac": round(6 * achieved / MFMA_BF16_PEAK_TFLOPS, 4)})
-
-    histories = [model.decode_history(i, beam) for i in range(n_sent)]  # of the last timed batch
     kernels = {}
     if args.profile_level >= 2:
         model.profile(2)
-        model.decode_batch(sents, beam=beam)
-        for name, t in sorted(model.profile_totals().items()):
-            rate = t["work"] / (t["ms"] * 1e-3)
-            is_gemm = "|" in name
-            kernels[name] = {"ms": round(t["ms"], 3), "launches": t["launches"],
-                             "rate": round(rate / (1e12 if is_gemm else 1e9), 2),
-                             "unit": "TFLOP/s" if is_gemm else "GB/s",
-                             "frac": round(rate / ((MFMA_FP32_PEAK_TFLOPS * 1e12) if is_gemm
-                                                   else (HBM_PEAK_GBS * 1e9)), 4)}
-        model.profile(0)
+        model.decode_stream(sents * min(args.steps, 2), beam=beam)
+        kernels = kernel_table(model.profile_totals())
+    model.profile(0)
 
-    # The same sentences, `steps` times over, as ONE list decoded with every beam column kept busy: a
-    # sentence that has taken its last step hands its 12 columns to the next sentence of the list
-    # (lnmt_decode_stream), so every step runs 768 hypotheses instead of a batch's shrinking set.
-    # Reported beside `value`; `value` stays one batch after the other.
-    stream, stream_hist = None, None
-    if not args.no_stream and not args.split_products_only:
-        model.profile(0)
-        model.decode_stream(sents * max(args.warmup, 1), beam=beam)
-        torch.cuda.synchronize()
-        s0 = time.perf_counter()
-        stream_res = model.decode_stream(sents * args.steps, beam=beam)  # ends with a stream synchronisation
-        sdt0 = time.perf_counter() - s0
-        stok0 = sum(len(r["best"]) for r in stream_res)
-        stream_hist = [model.decode_history(i, beam) for i in range(n_sent)]
-        copies_same = all(stream_res[i]["best"].tolist() == stream_res[i % n_sent]["best"].tolist()
-                          for i in range(len(stream_res)))
-        stream = {"value": round(stok0 / sdt0, 1), "unit": "target tokens/s",
-                  "sentences": n_sent * args.steps, "slots": n_sent, "steps_of_768_hypotheses": model.stream_ticks,
-                  "ms_per_64_sentences": round(sdt0 * 1e3 / args.steps, 2),
-                  "speedup_over_value": round(stok0 / sdt0 / value, 3),
-                  "how": "the list is taken longest first; a finished sentence's beam columns go to "
-                         "the next sentence; encoder in groups of 64; schedule fixed by the length "
-                         "limits, one read-back at the end",
-                  "one_best_same_as_batch_mode": int(sum(a["best"].tolist() == b["best"].tolist()
-                                                         for a, b in zip(res, stream_res[:n_sent]))),
-                  "repeated_sentences_decode_identically": bool(copies_same)}
-        stream["_res"] = stream_res[:n_sent]
+    # ---- beside it: one batch after the other (DecodeBatch), the batch's live hypotheses falling ----
+    # from 768 to 12 as its sentences end
+    batch, batch_hist, batch_res = None, None, None
+    if not args.no_batch:
+        for _ in range(args.warmup):
+            model.decode_batch(sents, beam=beam)
         model.profile(1 if args.profile_level >= 1 else 0)
+        torch.cuda.synchronize()
+        b0 = time.perf_counter()
+        btok = 0
+        for _ in range(args.steps):
+            batch_res = model.decode_batch(sents, beam=beam)  # ends with a stream synchronisation
+            btok += sum(len(r["best"]) for r in batch_res)
+        torch.cuda.synchronize()
+        bdt = time.perf_counter() - b0
+        batch_hist = [model.decode_history(i, beam) for i in range(n_sent)]
+        batch = {"value": round(btok / bdt, 1), "unit": "target tokens/s",
+                 "ms_per_batch": round(bdt * 1e3 / args.steps, 2),
+                 "ratio_to_value": round(btok / bdt / value, 3),
+                 "how": "lnmt_decode_batch on the same 64 sentences, one batch after the other",
+                 "roofline": gemm_roofline(model.profile_totals()),
+                 "one_best_same_as_value": int(sum(a["best"].tolist() == b["best"].tolist()
+                                                   for a, b in zip(res, batch_res)))}
+        if args.profile_level >= 2:
+            model.profile(2)
+            model.decode_batch(sents, beam=beam)
+            batch["kernels"] = kernel_table(model.profile_totals())
+        model.profile(0)
 
-    # The same batch with the opt-in arithmetic: gate products and output projection from three-way
+    # The same list with the opt-in arithmetic: gate products and output projection from three-way
     # bf16 splits of their fp32 operands (six exact products per term, fp32 accumulation).  Reported
     # beside `value`; `value` stays the fp32 MFMA path.
     split, split_res, split_hist = None, None, None
     if not args.no_split_products and not args.split_products_only:
         model.set_split_products(True)
-        model.profile(1)
-        # Warm-up: the first batch packs the weights; two more let the GPU's power management settle
-        # on the other matrix pipe (without them one of the first three timed batches takes ~90 ms
-        # instead of ~49; `ms_per_batch` below lists every timed batch).
-        for _ in range(max(args.warmup, 1) + 2):
-            model.decode_batch(sents, beam=beam)
-        model.profile(1)  # clears the totals of the warm-up batches
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        stok, per_batch = 0, []
-        for _ in range(args.steps):
-            b0 = time.perf_counter()
-            split_res = model.decode_batch(sents, beam=beam)  # ends with a stream synchronisation
-            per_batch.append((time.perf_counter() - b0) * 1e3)
-            stok += sum(len(r["best"]) for r in split_res)
-        torch.cuda.synchronize()
-        sdt = time.perf_counter() - t0
-        split_hist = [model.decode_history(i, beam) for i in range(n_sent)]
-        sk = {k: t for k, t in model.profile_totals().items() if k.startswith("logits_gemm|gemm_split_kernel")}
-        skernels = {}
-        if args.profile_level >= 2:
-            model.profile(2)
-            model.decode_batch(sents, beam=beam)
-            for name, t in sorted(model.profile_totals().items()):
-                rate = t["work"] / (t["ms"] * 1e-3)
-                is_gemm = "|" in name
-                skernels[name] = {"ms": round(t["ms"], 3), "launches": t["launches"],
-                                  "rate": round(rate / (1e12 if is_gemm else 1e9), 2),
-                                  "unit": "TFLOP/s (algorithmic)" if is_gemm else "GB/s"}
+        # Warm-up: the first call packs the weights; the GPU's power management takes ~150 ms to
+        # settle on the other matrix pipe, so the warm-up list is at least three batches long.
         model.profile(0)
-        split_stream = None
-        if not args.no_stream:
-            model.decode_stream(sents, beam=beam)
-            torch.cuda.synchronize()
-            s0 = time.perf_counter()
-            ss_res = model.decode_stream(sents * args.steps, beam=beam)
-            ss_dt = time.perf_counter() - s0
-            ss_tok = sum(len(r["best"]) for r in ss_res)
-            split_stream = {"value": round(ss_tok / ss_dt, 1), "unit": "target tokens/s",
-                            "ms_per_64_sentences": round(ss_dt * 1e3 / args.steps, 2),
-                            "speedup_over_value": round(ss_tok / ss_dt / value, 3)}
-        model.set_split_products(False)
+        model.decode_stream(sents * (max(args.warmup, 1) + 2), beam=beam)
+        model.profile(1)
+        torch.cuda.synchronize()
+        s0 = time.perf_counter()
+        ss_all = model.decode_stream(sents * args.steps, beam=beam)  # ends with a stream synchronisation
+        torch.cuda.synchronize()
+        sdt = time.perf_counter() - s0
+        stok = sum(len(r["best"]) for r in ss_all)
+        split_res = ss_all[:n_sent]
+        split_hist = [model.decode_history(i, beam) for i in range(n_sent)]
+        sroof = gemm_roofline(model.profile_totals())
         split = {"value": round(stok / sdt, 1), "unit": "target tokens/s",
                  "ms_per_step": round(sdt * 1e3 / args.steps, 2),
-                 "ms_per_step_median": round(float(np.median(per_batch)), 2),
-                 "ms_per_batch": [round(float(x), 2) for x in per_batch],
+                 "tick_us": round(sdt * 1e6 / model.stream_ticks, 1),
                  "speedup_over_value": round(stok / sdt / value, 3),
                  "arithmetic": "fp32 operands held as three bf16 terms; every product = six exact "
                                "bf16 x bf16 products (v_mfma_f32_32x32x16_bf16) added in fp32; what "
@@ -648,28 +664,34 @@ def main():
                                "and the output projection of steps with >= 84 live hypotheses",
                  "one_best_same_as_fp32_path": int(sum(a["best"].tolist() == b["best"].tolist()
                                                        for a, b in zip(res, split_res)))}
-        if skernels:
-            split["kernels"] = skernels
-        if split_stream:
-            split["stream"] = split_stream
-        if sk:
-            kern, t = max(sk.items(), key=lambda kv: kv[1]["work"])
-            alg = t["work"] / (t["ms"] * 1e-3) / 1e12
-            split["roofline"] = {"kernel": kern.split("|", 1)[1], "call_sites": ["logits_gemm"], "bound": "mfma",
-                                 "algorithmic_TFLOP/s": round(alg, 2),
-                                 "achieved": round(6 * alg, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
-                                 "unit": "TFLOP/s (bf16 products issued = 6 x algorithmic)",
-                                 "frac": round(6 * alg / MFMA_BF16_PEAK_TFLOPS, 4), "launches": t["launches"],
-                                 "avg_launch_us": round(t["ms"] * 1e3 / t["launches"], 2)}
+        if sroof:
+            split["roofline"] = sroof
+        if args.profile_level >= 2:
+            model.profile(2)
+            model.decode_stream(sents * min(args.steps, 2), beam=beam)
+            split["kernels"] = kernel_table(model.profile_totals())
+        model.profile(0)
+        if not args.no_batch:
+            model.decode_batch(sents, beam=beam)
+            torch.cuda.synchronize()
+            b0 = time.perf_counter()
+            sbtok = 0
+            for _ in range(args.steps):
+                sbtok += sum(len(r["best"]) for r in model.decode_batch(sents, beam=beam))
+            sbdt = time.perf_counter() - b0
+            split["batch"] = {"value": round(sbtok / sbdt, 1), "unit": "target tokens/s",
+                              "ms_per_batch": round(sbdt * 1e3 / args.steps, 2)}
+        model.set_split_products(False)
 
     # the metric's second half: the fused HBM-bound kernels alone (outside the timed region), each
     # at the size one decode step gives it (768 columns) and at a size that saturates HBM, next to
-    # a plain device copy, the practical ceiling of this GPU
+    # a plain device copy and a read-only pass, the practical ceilings of this GPU
     hbm_kernels = None
     if not args.no_hbm_kernels:
         k = bench_fused_kernels(torch, 20, 2, quick=True)
         hbm_kernels = {"peak_GB/s": HBM_PEAK_GBS, "launches_timed": k["launches_timed"],
                        "kernels": [{a: r[a] for a in ("kernel", "shape", "us", "GB/s", "frac_of_8TBs",
+                                                      "frac_of_read_only_ceiling",
                                                       "hbm_GB/s", "hbm_frac_of_8TBs") if a in r}
                                    for r in k["kernels"]]}
 
@@ -677,7 +699,11 @@ def main():
     parity = None
     if not args.no_cpu_baseline and args.cpu_sentences > 0:
         from oracle import orc  # the checker / reported baseline, never the measured path
-        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+        # every host core this process may use: OMP_NUM_THREADS when the environment sets it (a GPU
+        # box gives a job a share of its cores), else all of them
+        host_cores = os.cpu_count() or 1
+        env_threads = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+        cores = min(host_cores, env_threads) if env_threads > 0 else host_cores
         om = orc.Model(layers, H, V, V, attention=1, D=D, feed_input=1, longest_sent=longest)
         om.set_params(P)
         # bounded sample: every k-th sentence of the batch by length (all 64 by default, about
@@ -687,8 +713,8 @@ def main():
         om.decode_sentence(sents[by_len[0]][:3], beam=beam, num_threads=cores)  # warm-up
         cpu_tokens, cdt = 0, 0.0
         classes = {"identical": 0, "diverged_at_near_tie": 0, "diverged_at_window_tie": 0, "diverged_other": 0}
-        sclasses, qclasses = dict(classes), dict(classes)
-        same, ssame, qsame, detail = 0, 0, 0, []
+        sclasses, bclasses = dict(classes), dict(classes)
+        same, ssame, bsame, detail = 0, 0, 0, []
         for i in pick:
             c0 = time.perf_counter()
             tr = om.decode_sentence_trace(sents[i], beam=beam, num_threads=cores)
@@ -698,10 +724,10 @@ def main():
             cls, at, eps = classify_beam_parity(res[i]["best"], gtok, gbp, gsc, tr, len(sents[i]))
             classes[cls] += 1
             same += int(tr["best"].tolist() == res[i]["best"].tolist())
-            if stream is not None:
-                qtok, qbp, qsc = stream_hist[int(i)]
-                qclasses[classify_beam_parity(stream["_res"][i]["best"], qtok, qbp, qsc, tr, len(sents[i]))[0]] += 1
-                qsame += int(tr["best"].tolist() == stream["_res"][i]["best"].tolist())
+            if batch is not None:
+                qtok, qbp, qsc = batch_hist[int(i)]
+                bclasses[classify_beam_parity(batch_res[i]["best"], qtok, qbp, qsc, tr, len(sents[i]))[0]] += 1
+                bsame += int(tr["best"].tolist() == batch_res[i]["best"].tolist())
             if split is not None:
                 stok_h, sbp_h, ssc_h = split_hist[int(i)]
                 sclasses[classify_beam_parity(split_res[i]["best"], stok_h, sbp_h, ssc_h, tr, len(sents[i]))[0]] += 1
@@ -713,13 +739,15 @@ def main():
                                "oracle_window_margin": float(tr["window_margin"][at]) if 0 <= at < len(tr["margin"]) else None,
                                "epsilon": eps})
         cpu_baseline = {"value": round(cpu_tokens / cdt, 2), "unit": "target tokens/s",
-                        "cores": cores, "kind": "port",
+                        "cores": cores, "host_cores": host_cores, "kind": "port",
                         "sample": f"{len(pick)} of the 64 benchmark sentences, spread over the "
                                   f"length distribution ({cpu_tokens} target tokens, {cdt:.1f} s), "
                                   f"decoded one at a time by the CPU restatement (oracle/) with "
-                                  f"OpenMP"}
+                                  f"OpenMP on {cores} threads (the host shows {host_cores} cores; "
+                                  f"OMP_NUM_THREADS={os.environ.get('OMP_NUM_THREADS', 'unset')})"}
         parity = {"sentences_checked": int(len(pick)), "one_best_identical": int(same),
                   "beam_steps": classes, "parity_ok": classes["diverged_other"] == 0,
+                  "repeated_sentences_decode_identically": bool(copies_same),
                   "near_tie_rule": "first differing step has an oracle margin below 2 x the largest "
                                    "|GPU - oracle| path score measured on the (identical) beams "
                                    "before it + 8 ulp of the score",
@@ -730,9 +758,9 @@ def main():
         if split is not None:
             split["parity"] = {"sentences_checked": int(len(pick)), "one_best_identical": int(ssame),
                                "beam_steps": sclasses, "parity_ok": sclasses["diverged_other"] == 0}
-        if stream is not None:
-            stream["parity"] = {"sentences_checked": int(len(pick)), "one_best_identical": int(qsame),
-                                "beam_steps": qclasses, "parity_ok": qclasses["diverged_other"] == 0}
+        if batch is not None:
+            batch["parity"] = {"sentences_checked": int(len(pick)), "one_best_identical": int(bsame),
+                               "beam_steps": bclasses, "parity_ok": bclasses["diverged_other"] == 0}
 
     out = {
         "metric": "target tokens/sec (beam-12 decode, 1 GPU)" +
@@ -748,19 +776,22 @@ def main():
         "vs_baseline": None,
         "dtype": "f32 operands as three bf16 terms, f32 accumulation" if args.split_products_only else "f32",
         "data": "synthetic",
-        "config": {"workload": "configs[2]: beam-12 decode, 64 sentences/batch (768 live "
-                               "hypotheses), 4+4 LSTM layers, hidden=emb=1000, vocab 30k/30k, "
-                               "local-p attention D=10 + input feeding, source len U[10,60] Zipf "
-                               "ids, max target 1.5x source, random-init uniform[-0.08,0.08]",
+        "config": {"workload": "configs[2]: beam-12 decode, 64 sentences at a time (768 live "
+                               "hypotheses in every step: a finished sentence's 12 beam columns go "
+                               "to the next sentence of the list, lnmt_decode_stream), 4+4 LSTM "
+                               "layers, hidden=emb=1000, vocab 30k/30k, local-p attention D=10 + "
+                               "input feeding, source len U[10,60] Zipf ids, max target 1.5x "
+                               "source, random-init uniform[-0.08,0.08]; one step = 64 sentences",
+                   "sentences": n_sent * args.steps, "slots": n_sent,
                    "tokens_per_step": tokens // max(args.steps, 1),
                    "seed": SEED},
         "roofline": roofline,
+        "step": step,
         "hbm_kernels": hbm_kernels,
         "cpu_baseline": cpu_baseline,
     }
-    if stream:
-        stream.pop("_res", None)
-        out["stream"] = stream
+    if batch:
+        out["batch"] = batch
     if split:
         out["split_products"] = split
     if kernels:
@@ -768,17 +799,18 @@ def main():
     if parity:
         out["parity"] = parity
     print(json.dumps(out))
-    if split and "parity" in split and not split["parity"]["parity_ok"]:
-        print("bench.py: with split products the GPU search differs from the oracle's where no "
-              "near-tie explains it", file=sys.stderr)
-        sys.exit(1)
-    if stream and "parity" in stream and not stream["parity"]["parity_ok"]:
-        print("bench.py: the stream decoder's search differs from the oracle's where no near-tie "
-              "explains it", file=sys.stderr)
-        sys.exit(1)
+    bad = []
     if parity and not parity["parity_ok"]:
-        print("bench.py: the GPU search differs from the oracle's where no near-tie explains it",
-              file=sys.stderr)
+        bad.append("the GPU search")
+    if batch and "parity" in batch and not batch["parity"]["parity_ok"]:
+        bad.append("the batch-after-batch search")
+    if split and "parity" in split and not split["parity"]["parity_ok"]:
+        bad.append("the search with split products")
+    if not copies_same:
+        bad.append("(repeated sentences decode differently)")
+    if bad:
+        print("bench.py: " + ", ".join(bad) + " differs from the oracle's where no near-tie "
+              "explains it", file=sys.stderr)
         sys.exit(1)
 
 
