@@ -110,6 +110,11 @@ int lnmt_update_weights(lnmt_model *m, double *global_norm);
  * n = floats the buffer holds (copies min(n, available)).  For parity checks. */
 int lnmt_get_dropout_mask(lnmt_model *m, int kind, int side, int layer, float *data, long long n);
 int lnmt_clear_gradients(lnmt_model *m);
+/* Restarts the sequence of dropout masks: the masks of the n-th lnmt_compute_gradients call after
+ * this one are a fixed function of (seed, n), so a run can be repeated mask for mask (the
+ * reference seeds each layer's cuRAND generator once, when the layer is initialised:
+ * src/layer_input_to_hidden.h:603-605,744-747, src/layer_hidden_to_hidden.h:460-463). */
+int lnmt_set_dropout_seed(lnmt_model *m, unsigned long long seed);
 
 /* Copies a state of the last lnmt_get_error call: kind 0 = h, 1 = c of (side 0 src / 1 tgt, layer,
  * timestep); kind 2 = attention output h~ of target timestep; kind 3 = alignments (B x W) of target

@@ -91,6 +91,7 @@ def load():
     lib.lnmt_model_get_grad.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
     lib.lnmt_update_weights.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
     lib.lnmt_clear_gradients.argtypes = [C.c_void_p]
+    lib.lnmt_set_dropout_seed.argtypes = [C.c_void_p, C.c_ulonglong]
     lib.lnmt_get_dropout_mask.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                           C.c_longlong]
     lib.lnmt_model_destroy.argtypes = [C.c_void_p]
@@ -355,6 +356,9 @@ class Model:
 
     def clear_gradients(self):
         _check(load().lnmt_clear_gradients(self.handle), "clear_gradients")
+
+    def set_dropout_seed(self, seed):
+        _check(load().lnmt_set_dropout_seed(self.handle, seed), "set_dropout_seed")
 
     def decode_history(self, sentence, beam):
         """Beam of sentence `sentence` of the last decode_batch call after every expansion step:

@@ -176,6 +176,14 @@ extern "C" int lnmt_clear_gradients(lnmt_model *m) {
   });
 }
 
+extern "C" int lnmt_set_dropout_seed(lnmt_model *m, unsigned long long seed) {
+  return Guard([&] {
+    if (!m->nmt->cfg_.train_mode_) throw LinmtError("lnmt_set_dropout_seed: not a training model");
+    m->nmt->cfg_.dropout_seed_ = seed;
+    m->nmt->minibatch_counter_ = 0;
+  });
+}
+
 extern "C" int lnmt_model_set_param(lnmt_model *m, const char *name, const float *data,
                                     long long n) {
   return Guard([&] {

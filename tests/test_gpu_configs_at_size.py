@@ -228,3 +228,145 @@ def test_config5_training_step_at_width(orc, host):
         # and the update moved the parameter (columns of unused embeddings aside)
     assert not np.array_equal(gm.get_param("tgt.3.W_hi", (H, H)), P["tgt.3.W_hi"])
     gm.close()
+
+
+def test_config3_two_layer_local_p_model_at_size(orc, host):
+    """BASELINE configs[3] as a model: 2+2 layers, hidden 1000, vocabulary 30k, batch 64, source
+    and target length 100 (a few columns shorter, so that padding is exercised at this length too),
+    local-p attention D=10 with input feeding -- AttentionNode::ForwardProp
+    (src/layer_attention.h:243-483) inside NeuralMachineTranslation::GetError
+    (src/deep_rnn.h:2173-2317) at longest_sentence 104.  Teacher-forced cross-entropy against the
+    oracle per word, the attention output and the alignments of single steps compared directly."""
+    layers, H, V, B, D, S, T, longest = 2, 1000, 30000, 64, 10, 100, 100, 104
+    rng = np.random.default_rng(1300)
+    P = make_params(rng, layers, H, V, V)
+    ls = np.full(B, S)
+    lt = np.full(B, T)
+    ls[[5, 17, 40]] = [37, 81, 99]
+    lt[[5, 23, 63]] = [12, 64, 99]
+    src = np.full((B, S), -1, np.int32)
+    tin = np.full((B, T), -1, np.int32)
+    tout = np.full((B, T), -1, np.int32)
+    for b in range(B):
+        src[b, S - ls[b]:] = zipf_ids(rng, ls[b], V)
+        t = zipf_ids(rng, lt[b] - 1, V, lo=3)
+        tin[b, :lt[b]] = np.concatenate([[0], t])
+        tout[b, :lt[b]] = np.concatenate([t, [1]])
+    bi = np.concatenate([ls, S - ls]).astype(np.int32)
+    n_words = int(lt.sum())
+    gm = host.Model(layers, H, V, V, longest_sentence=longest, attention_mode=1, attention_width=D,
+                    feed_input=True, minibatch_size=B)
+    gm.set_params(P)
+    got = gm.get_error(src, tin, tout, bi)
+    for b in (5, 17, 40):  # padded source prefixes stay at exactly zero state on both layers
+        pad = S - ls[b]
+        for layer in range(layers):
+            for kind in (0, 1):
+                st = gm.get_state(kind, 0, layer, pad - 1, H, B)
+                assert np.all(st[:, b] == 0), (layer, b, kind)
+                assert np.any(gm.get_state(kind, 0, layer, pad, H, B)[:, b] != 0), (layer, b, kind)
+    # a target column past its sentence end: attention output masked to exactly zero
+    assert np.all(gm.get_state(2, 1, 0, 50, H, B)[:, 5] == 0)
+    align = np.stack([gm.get_state(3, 1, 0, t, B, 2 * D + 1) for t in (0, 49, 99)])
+    live = np.stack([tin[:, t] >= 0 for t in (0, 49, 99)])
+    sums = align.sum(axis=2)  # alignments carry the Gaussian factor: 0 < sum <= 1 for live columns
+    assert np.all(sums[live] > 0) and np.all(sums[live] <= 1 + 1e-5)
+    gm.close()
+    om = orc.Model(layers, H, V, V, attention=1, D=D, feed_input=1, longest_sent=longest)
+    om.set_params(P)
+    t0 = time.time()
+    want = om.forward_xent(src, tin, tout, bi)
+    print(f"configs[3] model: oracle forward_xent {time.time() - t0:.1f} s, {n_words} target words, "
+          f"per-word log-lik gpu {got / n_words:.6f} oracle {want / n_words:.6f}", flush=True)
+    assert_close(got / n_words, want / n_words, "per-word log-likelihood", rtol=1e-4, atol=1e-5)
+    assert_close(got, want, "sum log p(target)", rtol=2e-5, atol=1e-3)
+
+
+def test_config5_full_minibatch_properties(host):
+    """The configs[4] training step at its own batch (256 sentence pairs of 20-80 tokens, 8+8
+    layers, hidden 2048, embedding 1024, vocabulary 50k, dropout 0.2): the oracle would need hours
+    for it (its gradients are checked at this width and depth on a small minibatch above), so
+    this checks what holds whatever the numbers are -- NeuralMachineTranslation::ComputeGradients /
+    UpdateWeights, src/deep_rnn.h:984-1412:
+      * the same seed gives the same masks and bit-identical gradients (no atomics, fixed orders);
+      * embedding-gradient columns of words that are not in the minibatch are exactly zero, those
+        of words that are in it are not; states of padded source positions are exactly zero;
+      * the norm the global clip used equals the float64 norm of the gradients read back (the
+        embedding gradients are outside it, src/deep_rnn.h:1326-1412), and the update is
+        theta + lr * min(1, clip / norm) * g / B for a matrix read back before and after;
+      * without dropout the training forward's log-likelihood equals GetError's."""
+    layers, H, E, V, D, B, keep, lr, clip = 8, 2048, 1024, 50000, 10, 256, 0.8, 0.1, 5.0
+    rng = np.random.default_rng(1400)
+    P = make_params(rng, layers, H, V, V, E=E)
+    src, tin, tout, bi, su, tu, n_words = minibatch(rng, B, 20, 80, V, V)
+    S = src.shape[1]
+
+    def build(keep_):
+        m = host.Model(layers, H, V, V, longest_sentence=84, attention_mode=1, attention_width=D,
+                       feed_input=True, minibatch_size=B, embedding_size=E,
+                       training=dict(learning_rate=lr, grad_clip_mode=2, norm_clip=clip,
+                                     dropout_keep=keep_, dropout_seed=99))
+        m.set_params(P)
+        return m
+
+    def shape_of(name):
+        a = P[name]
+        return a.shape if a.ndim == 2 else (a.size,)
+
+    probe = ["tgt.7.W_hi", "src.0.M_f", "tgt.0.Q_o", "attn.W_a", "attn.v_p", "softmax.b_d", "src.3.b_c",
+             "tgt.0.W"]
+    gm = build(keep)
+    ll1 = gm.compute_gradients(src, tin, tout, bi, su, tu)
+    first = {n: gm.get_grad(n, shape_of(n)).copy() for n in probe}
+    mask1 = gm.get_dropout_mask(1, 1, 3, H, B, 4).copy()
+    gm.clear_gradients()
+    gm.set_dropout_seed(99)
+    ll2 = gm.compute_gradients(src, tin, tout, bi, su, tu)
+    assert np.array_equal(gm.get_dropout_mask(1, 1, 3, H, B, 4), mask1)
+    assert ll1 == ll2
+    for n in probe:
+        assert np.array_equal(gm.get_grad(n, shape_of(n)), first[n]), f"{n}: gradients of two runs differ"
+    assert abs((mask1 < keep).mean() - keep) < 0.01
+    # words outside the minibatch have exactly zero embedding gradient
+    for name, ids in (("src.0.W", su), ("tgt.0.W", tu)):
+        g = gm.get_grad(name, (E, V))
+        used = np.zeros(V, bool)
+        used[ids] = True
+        assert not g[:, ~used].any(), name
+        assert np.all(np.abs(g[:, used]).max(axis=0) > 0), name
+        del g
+    # the global norm: every gradient but the embeddings', scaled by 1/B
+    ss, count = 0.0, 0
+    for name in P:
+        if name in ("src.0.W", "tgt.0.W"):
+            continue
+        g = gm.get_grad(name, shape_of(name)).astype(np.float64)
+        assert np.isfinite(g).all(), name
+        ss += float(np.sum(g * g))
+        count += g.size
+    want_norm = np.sqrt(ss) / B
+    before = gm.get_param("tgt.7.W_hi", (H, H)).copy()
+    got_norm = gm.update_weights()
+    print(f"configs[4] minibatch: {n_words} target words, log-lik per word {ll1 / n_words:.5f}, "
+          f"global norm gpu {got_norm:.6f} float64 of the read-back gradients {want_norm:.6f} "
+          f"({count} parameters)", flush=True)
+    assert abs(got_norm - want_norm) <= 2e-4 * want_norm
+    assert want_norm > clip  # the clip is active
+    f = min(1.0, clip / want_norm)
+    want_after = before.astype(np.float64) + lr * f * first["tgt.7.W_hi"].astype(np.float64) / B
+    assert_close(gm.get_param("tgt.7.W_hi", (H, H)), want_after, "updated tgt.7.W_hi", rtol=1e-5, atol=1e-7)
+    assert not gm.get_grad("tgt.7.W_hi", (H, H)).any()  # gradients are cleared by the update
+    gm.close()
+    del first, before
+
+    g1 = build(1.0)
+    ll = g1.compute_gradients(src, tin, tout, bi, su, tu)
+    xent = g1.get_error(src, tin, tout, bi)
+    print(f"without dropout: training forward {ll:.4f}, GetError {xent:.4f}", flush=True)
+    assert abs(ll - xent) <= 1e-5 * abs(xent)
+    for b in (1, B // 2, B - 1):
+        pad = S - bi[b]
+        if pad > 0:
+            for layer in (0, layers - 1):
+                assert not g1.get_state(0, 0, layer, pad - 1, H, B)[:, b].any(), (layer, b)
+    g1.close()

@@ -51,8 +51,8 @@ def workload(orc):
     return dict(cfg=(layers, H, V, D, beam, n_sent, longest), P=P, sents=sents, traces=traces)
 
 
-@pytest.mark.parametrize("split,stream", [(False, False), (True, False), (False, True)],
-                         ids=["fp32_mfma", "split_bf16_products", "stream"])
+@pytest.mark.parametrize("split,stream", [(False, False), (True, False), (False, True), (True, True)],
+                         ids=["fp32_mfma", "split_bf16_products", "stream", "stream_split_bf16_products"])
 def test_benchmark_batch_beams_vs_oracle_trace(workload, host, split, stream):
     """split: the same demand on the opt-in arithmetic (lnmt_set_split_products), whose products
     are as close to float64 as the fp32 MFMA ones.  stream: the same demand on lnmt_decode_stream
