@@ -291,6 +291,152 @@ def attn_core_bwd(H, B, D, max_len, hs_steps, dctx, tanh1, v_p, wa, hs, step_str
     return out
 
 
+MODEL_FILE_RULE = "=" * 58
+
+
+def model_file_order(layers, H, Vs, Vt, attention, feed_input):
+    """[(name, rows, cols)] in the order the reference's model file holds the matrices:
+    NeuralMachineTranslation::DumpWeights (src/deep_rnn.h:2124-2146) walks the source layers, the
+    target layers and the softmax; a layer writes W_hi b_i W_hf b_f W_hc b_c W_ho b_o, the
+    embedding table (input layer only), M_i M_f M_o M_c, Q_i Q_f Q_o Q_c (feed input) and -- the
+    layer the attention is attached to, the top target layer -- W_a W_p v_p b_out W_c1 W_c2
+    (src/layer_input_to_hidden.h:1556-1590, src/layer_hidden_to_hidden.h:989-1014,
+    src/layer_attention.h:1264-1273); the softmax writes D and b_d (src/layer_loss.h:1213-1218)."""
+    out = []
+    for side, V in (("src", Vs), ("tgt", Vt)):
+        for l in range(layers):
+            p = f"{side}.{l}."
+            for g in "ifco":
+                out += [(p + "W_h" + g, H, H), (p + "b_" + g, H, 1)]
+            if l == 0:
+                out.append((p + "W", H, V))
+            out += [(p + "M_" + g, H, H) for g in "ifoc"]
+            if side == "tgt" and l == 0 and attention and feed_input:
+                out += [(p + "Q_" + g, H, H) for g in "ifoc"]
+            if side == "tgt" and l == layers - 1 and attention:
+                out += [("attn.W_a", H, H), ("attn.W_p", H, H), ("attn.v_p", H, 1), ("attn.b_out", H, 1),
+                        ("attn.W_c1", H, H), ("attn.W_c2", H, H)]
+    return out + [("softmax.D", Vt, H), ("softmax.b_d", Vt, 1)]
+
+
+def write_model_file(path, params, layers, H, Vs, Vt, attention=1, feed_input=1, source_words=None,
+                     target_words=None):
+    """A complete model file as the reference's programs leave it, written from the source: the
+    first line of cc_util::AddModelInformation (src/utility_cc.cc:76-98: layers, lstm size, target
+    and source vocabulary sizes, attention, feed input, three zeros), the vocabulary mappings
+    between rules of 58 '=' (src/input_file_preprocess.cc:545-575: "<id> <word>" per line, source
+    id 0 = <UNK>, target ids 0-2 = <START> <EOF> <UNK>), then every matrix as WriteMatrixGpu
+    writes it (src/deep_rnn_kernel.h:1564-1578: a line per row, single spaces, an empty line after
+    the matrix) with the stream's precision at digits10 + 2 = 8 significant digits
+    (src/deep_rnn.h:2127), which for an ostream in its default float format is printf's %.8g."""
+    src_words = list(source_words) if source_words else ["<UNK>"] + [f"w{i}" for i in range(1, Vs)]
+    tgt_words = list(target_words) if target_words else ["<START>", "<EOF>", "<UNK>"] + [f"w{i}" for i in range(3, Vt)]
+    with open(path, "w") as f:
+        f.write(f"{layers} {H} {Vt} {Vs} {int(bool(attention))} {int(bool(attention and feed_input))} 0 0 0\n")
+        f.write(MODEL_FILE_RULE + "\n")
+        for i in range(Vs):
+            f.write(f"{i} {src_words[i]}\n")
+        f.write(MODEL_FILE_RULE + "\n")
+        for i in range(Vt):
+            f.write(f"{i} {tgt_words[i]}\n")
+        f.write(MODEL_FILE_RULE + "\n")
+        for name, rows, cols in model_file_order(layers, H, Vs, Vt, attention, feed_input):
+            m = np.asarray(params[name], np.float32).reshape((rows, cols))
+            for i in range(rows):
+                f.write(" ".join("%.8g" % float(x) for x in m[i]) + "\n")
+            f.write("\n")
+
+
+def read_model_file(path):
+    """What NeuralMachineTranslation::LoadWeights (src/deep_rnn.h:1878-1968) and ReadMatrixGpu
+    (src/deep_rnn_kernel.h:1543-1561) make of a model file: the first line's numbers, the two
+    vocabulary lists, and every matrix with its numbers converted as (float)stod(token)."""
+    with open(path) as f:
+        lines = f.read().split("\n")
+    head = [int(x) for x in lines[0].split()]
+    layers, H, Vt, Vs = head[:4]
+    attention, feed = (head[4], head[5]) if len(head) > 5 else (0, 0)
+    is_rule = lambda l: len(l) > 3 and l[:3] == "==="  # noqa: E731
+    assert is_rule(lines[1])
+    k, vocab = 2, [[], []]
+    for part in range(2):
+        while not is_rule(lines[k]):
+            vocab[part].append(lines[k].split(" ", 1)[1])
+            k += 1
+        k += 1
+    params = {}
+    for name, rows, cols in model_file_order(layers, H, Vs, Vt, attention, feed):
+        m = np.array([[float(t) for t in lines[k + i].split()[:cols]] for i in range(rows)], np.float64)
+        assert m.shape == (rows, cols), name
+        params[name] = m.astype(np.float32).reshape((rows, cols) if cols > 1 else (rows,))
+        k += rows + 1
+    return dict(layers=layers, H=H, Vs=Vs, Vt=Vt, attention=attention, feed_input=feed,
+                source_words=vocab[0], target_words=vocab[1]), params
+
+
+class TrainingFile:
+    """The reference's integerised training file read the way FileHelper::ReadMinibatch does
+    (src/file_helper.cc:113-381, statistics as GetFileStats, src/utility_cc.cc:17-58), written
+    from the source with numpy: four lines per sentence pair (source input, source output, target
+    input, target output; -1 pads; every pair of a minibatch padded to common lengths),
+    minibatch_size pairs per minibatch, the file starting over after its last minibatch."""
+
+    def __init__(self, path, minibatch_size):
+        with open(path) as fh:
+            lines = fh.read().split("\n")
+        if lines and lines[-1] == "":
+            lines.pop()
+        self.lines = [np.array(l.split(), dtype=np.int64) for l in lines]
+        self.B = minibatch_size
+        assert len(self.lines) % (4 * minibatch_size) == 0, "whole minibatches only"
+        # GetFileStats: non-pad ids of the two input lines of every pair
+        self.total_words = int(sum((l != -1).sum() for k, l in enumerate(self.lines) if k % 4 in (0, 2)))
+        self.total_target_words = int(sum((l != -1).sum() for k, l in enumerate(self.lines) if k % 4 == 2))
+        self.cursor = 0  # index of the next pair's first line
+
+    @staticmethod
+    def _wgrad(ids_column_major):
+        """PreprocessInputWgrad (:248-378): first occurrences in column-major order, every other
+        position -1, then the in-place partition that swaps the leftmost -1 with the rightmost id."""
+        v = ids_column_major.copy()
+        seen = set()
+        for i, w in enumerate(v):
+            if w == -1 or w in seen:
+                v[i] = -1
+            else:
+                seen.add(int(w))
+        left, right = 0, len(v) - 1
+        while left < right:
+            if v[left] == -1:
+                if v[right] != -1:
+                    v[left], v[right] = v[right], v[left]
+                    left += 1
+                right -= 1
+                continue
+            left += 1
+        if len(v) and v[left] != -1:
+            left += 1
+        return v[:left].astype(np.int32)
+
+    def read_minibatch(self):
+        """Returns (minibatch, same_epoch): same_epoch is False for the last minibatch of a pass."""
+        B = self.B
+        block = self.lines[self.cursor:self.cursor + 4 * B]
+        self.cursor += 4 * B
+        same_epoch = self.cursor < len(self.lines)
+        if not same_epoch:
+            self.cursor = 0
+        src = np.stack(block[0::4]).astype(np.int32)   # (B, S): row = sentence, column = timestep
+        tin = np.stack(block[2::4]).astype(np.int32)
+        tout = np.stack(block[3::4]).astype(np.int32)
+        lens = (src != -1).sum(axis=1)
+        mb = dict(src=src, tgt_in=tin, tgt_out=tout,
+                  batch_info=np.concatenate([lens, src.shape[1] - lens]).astype(np.int32),
+                  src_wgrad=self._wgrad(src.ravel(order="F")), tgt_wgrad=self._wgrad(tin.ravel(order="F")),
+                  words_in_minibatch=int((src != -1).sum() + (tout != -1).sum()))
+        return mb, same_epoch
+
+
 class Model:
     """Host model of the oracle; parameters are numpy views into the oracle's own buffers."""
 
@@ -477,6 +623,86 @@ class Model:
     def update_weights(self, learning_rate, clip_mode, norm_clip, individual_clip, minibatch_size):
         return float(lib().orc_update_weights(self.trainer, _f(learning_rate), clip_mode,
                                               _f(norm_clip), _f(individual_clip), minibatch_size))
+
+    def get_perplexity(self, path, minibatch_size):
+        """NeuralMachineTranslation::GetPerplexity (src/deep_rnn.h:1490-1568): one pass over an
+        integerised file, 2^(-(sum of log2 p(target)) / target words of the file)."""
+        f = TrainingFile(path, minibatch_size)
+        p_data, more = 0.0, True
+        while more:
+            mb, more = f.read_minibatch()
+            p_data += self.forward_xent(mb["src"], mb["tgt_in"], mb["tgt_out"], mb["batch_info"])
+        p_data /= np.log(2.0)
+        return float(2.0 ** (-p_data / f.total_target_words))
+
+    def tuning(self, train_file, minibatch_size, learning_rate, epochs, dev_file=None, clip_mode=2,
+               norm_clip=5.0, individual_clip=0.0, google_learning_rate=False,
+               epoch_to_start_halving=6, stanford_learning_rate=False, epoch_to_start_halving_full=6,
+               learning_rate_schedule=False, decrease_factor=0.5, margin=0.0):
+        """Dispatcher::Tuning (src/dispatcher.cu:96-384), the part that decides what the model
+        becomes: minibatches in file order, ComputeGradients + UpdateWeights per minibatch, the
+        three learning-rate schedules (fixed halving from an epoch on at the half and the end of
+        every epoch, :228-236 and :283-291; halving at the end of every epoch, :293-301; decrease by
+        a factor when the dev perplexity stalls, evaluated at the half and the end of every epoch,
+        :239-272 and :303-337).  Returns the list of events (kind, epoch, minibatch, value) with
+        kinds learning_rate / half_epoch_perplexity / epoch_perplexity / epoch_end, and the final
+        learning rate.  The learning rate is kept in single precision, as the reference's
+        `precision tmp_learning_rate` is."""
+        self._trainer()
+        f = TrainingFile(train_file, minibatch_size)
+        half_way_count = f.total_words // 2
+        events = []
+        lr = np.float32(learning_rate)
+        epoch, batch_num, total_words = 1, 0, 0
+        flag, old_perplexity, loglik = True, 0.0, 0.0
+
+        def evaluate(kind):
+            nonlocal lr, old_perplexity
+            new = self.get_perplexity(dev_file, minibatch_size)
+            events.append((kind, epoch, batch_num, new))
+            if new + margin >= old_perplexity and epoch != 1:
+                lr = np.float32(lr * np.float32(decrease_factor))
+                events.append(("learning_rate", epoch, batch_num, float(lr)))
+            old_perplexity = new
+
+        def halve():
+            nonlocal lr
+            lr = np.float32(lr / np.float32(2))
+            events.append(("learning_rate", epoch, batch_num, float(lr)))
+
+        while epoch <= epochs:
+            mb, success = f.read_minibatch()
+            src, tin, tout = (np.asfortranarray(mb[k], np.int32) for k in ("src", "tgt_in", "tgt_out"))
+            B, S = src.shape
+            su, tu = i32(mb["src_wgrad"]), i32(mb["tgt_wgrad"])
+            loglik += lib().orc_compute_gradients(self.trainer, _p(src), S, _p(tin), _p(tout), tin.shape[1],
+                                                  B, _p(i32(mb["batch_info"])), _p(su), su.size, _p(tu),
+                                                  tu.size)
+            self.update_weights(float(lr), clip_mode, norm_clip, individual_clip, minibatch_size)
+            batch_num += 1
+            total_words += mb["words_in_minibatch"]
+            if google_learning_rate and epoch >= epoch_to_start_halving and total_words >= half_way_count and flag:
+                halve()
+                flag = False
+            if learning_rate_schedule and total_words >= half_way_count and flag:
+                flag = False
+                evaluate("half_epoch_perplexity")
+            if not success:
+                events.append(("epoch_end", epoch, batch_num, loglik))
+                loglik = 0.0
+                epoch += 1
+                batch_num = 0
+                if google_learning_rate and epoch >= epoch_to_start_halving:
+                    halve()
+                    flag = True
+                if stanford_learning_rate and epoch >= epoch_to_start_halving_full:
+                    halve()
+                    flag = True
+                if learning_rate_schedule:
+                    evaluate("epoch_perplexity")
+                    flag = True
+                total_words = 0
+        return events, float(lr)
 
     def get_param(self, name):
         flat = self.param(name).copy()

@@ -289,8 +289,8 @@ def test_config5_full_minibatch_properties(host):
     this checks what holds whatever the numbers are -- NeuralMachineTranslation::ComputeGradients /
     UpdateWeights, src/deep_rnn.h:984-1412:
       * the same seed gives the same masks and bit-identical gradients (no atomics, fixed orders);
-      * embedding-gradient columns of words that are not in the minibatch are exactly zero, those
-        of words that are in it are not; states of padded source positions are exactly zero;
+      * the update leaves the embeddings of words that are not in the minibatch untouched bit for
+        bit and moves those of every word that is in it; states of padded source positions are exactly zero;
       * the norm the global clip used equals the float64 norm of the gradients read back (the
         embedding gradients are outside it, src/deep_rnn.h:1326-1412), and the update is
         theta + lr * min(1, clip / norm) * g / B for a matrix read back before and after;
@@ -311,6 +311,8 @@ def test_config5_full_minibatch_properties(host):
 
     def shape_of(name):
         a = P[name]
+        if name.endswith(".W"):  # the embedding gradient holds the minibatch's words only
+            return (E, len(su if name.startswith("src") else tu))
         return a.shape if a.ndim == 2 else (a.size,)
 
     probe = ["tgt.7.W_hi", "src.0.M_f", "tgt.0.Q_o", "attn.W_a", "attn.v_p", "softmax.b_d", "src.3.b_c",
@@ -327,14 +329,12 @@ def test_config5_full_minibatch_properties(host):
     for n in probe:
         assert np.array_equal(gm.get_grad(n, shape_of(n)), first[n]), f"{n}: gradients of two runs differ"
     assert abs((mask1 < keep).mean() - keep) < 0.01
-    # words outside the minibatch have exactly zero embedding gradient
+    # the embedding gradient has one column per word of the minibatch, none of them empty
     for name, ids in (("src.0.W", su), ("tgt.0.W", tu)):
-        g = gm.get_grad(name, (E, V))
-        used = np.zeros(V, bool)
-        used[ids] = True
-        assert not g[:, ~used].any(), name
-        assert np.all(np.abs(g[:, used]).max(axis=0) > 0), name
+        g = gm.get_grad(name, (E, len(ids)))
+        assert np.all(np.abs(g).max(axis=0) > 0), name
         del g
+    emb_before = gm.get_param("src.0.W", (E, V)).copy()
     # the global norm: every gradient but the embeddings', scaled by 1/B
     ss, count = 0.0, 0
     for name in P:
@@ -356,6 +356,13 @@ def test_config5_full_minibatch_properties(host):
     want_after = before.astype(np.float64) + lr * f * first["tgt.7.W_hi"].astype(np.float64) / B
     assert_close(gm.get_param("tgt.7.W_hi", (H, H)), want_after, "updated tgt.7.W_hi", rtol=1e-5, atol=1e-7)
     assert not gm.get_grad("tgt.7.W_hi", (H, H)).any()  # gradients are cleared by the update
+    # words outside the minibatch keep their embeddings bit for bit, every word inside it moves
+    emb_after = gm.get_param("src.0.W", (E, V))
+    used = np.zeros(V, bool)
+    used[su] = True
+    assert np.array_equal(emb_after[:, ~used], emb_before[:, ~used])
+    assert np.all((emb_after[:, used] != emb_before[:, used]).any(axis=0))
+    del emb_before, emb_after
     gm.close()
     del first, before
 

@@ -323,3 +323,63 @@ def test_decoding_a_long_text_file_through_the_stream(host, tmp_path):
     got2 = open(ids2).read().split("\n")[:-1]
     same = sum(x.split(" |||| ")[0] == y.split(" |||| ")[0] for x, y in zip(got, got2))
     assert len(got2) == 150 and same >= 147, same  # a near-tie may fall the other way between the two modes
+
+
+@pytest.mark.parametrize("layers,attention,feed", [(2, 1, True), (1, 1, False), (3, 0, False)])
+def test_model_file_written_independently_loads_decodes_and_is_dumped_byte_for_byte(orc, host, tmp_path,
+                                                                                    layers, attention, feed):
+    """The model file against a writer that is not the path's own: oracle/orc.py write_model_file
+    follows NeuralMachineTranslation::DumpWeights and WriteMatrixGpu line by line
+    (src/deep_rnn.h:2124-2146, src/deep_rnn_kernel.h:1564-1578, src/layer_input_to_hidden.h:1556-1590;
+    pinned on the hand-made file in tests/test_oracle_tuning_pins.py).
+      * LoadWeights of that file must give a model that decodes what the oracle decodes with the
+        file's numbers (read back by the oracle's own reader: eight digits do not always
+        reproduce an fp32 value, so the file's numbers are the model);
+      * DumpModel of a model holding the same parameters must write that file byte for byte;
+      * so must the training loop's final DumpWeights onto a file that so far holds the header
+        and the mappings, which is how the reference's trainer finds it."""
+    rng = np.random.default_rng(40 + layers)
+    H, Vs, Vt, D, beam = 16, 23, 31, 3, 4
+    P = R.make_params(rng, layers, H, Vs, Vt, attention=bool(attention), feed_input=feed, scale=0.4)
+    src_words = ["<UNK>"] + [f"w{i}" for i in range(1, Vs)]
+    tgt_words = ["<START>", "<EOF>", "<UNK>"] + [f"w{i}" for i in range(3, Vt)]
+    want_file = str(tmp_path / "oracle_written.nmt")
+    orc.write_model_file(want_file, P, layers, H, Vs, Vt, attention, feed)
+    info, P_file = orc.read_model_file(want_file)
+    assert info["source_words"] == src_words and info["target_words"] == tgt_words
+    assert max(float(np.abs(P_file[k] - np.asarray(P[k]).reshape(P_file[k].shape)).max()) for k in P) < 1e-7
+
+    kw = dict(longest_sentence=24, attention_mode=attention, attention_width=D, feed_input=feed)
+    gm = host.Model(layers, H, Vs, Vt, decoding=(3, beam), **kw)
+    gm.load_weights(want_file)
+    for name, arr in P_file.items():
+        shape = arr.shape if arr.ndim == 2 else (arr.size,)
+        assert np.array_equal(gm.get_param(name, shape), arr), name
+    om = orc.Model(layers, H, Vs, Vt, attention=attention, D=D, feed_input=int(feed), longest_sent=24)
+    om.set_params(P_file)
+    sents = [rng.integers(0, Vs, size=n) for n in (7, 2, 11)]
+    got = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    for i, s in enumerate(sents):
+        want = om.decode_sentence(s, beam=beam)
+        assert got[i]["best"].tolist() == want["best"].tolist(), i
+        assert [h[0].tolist() for h in got[i]["hyps"]] == [h[0].tolist() for h in want["hyps"]], i
+        assert np.allclose([h[1] for h in got[i]["hyps"]], [h[1] for h in want["hyps"]], rtol=1e-4, atol=1e-4)
+    gm.close()
+
+    tm = host.Model(layers, H, Vs, Vt, minibatch_size=2,
+                    training=dict(learning_rate=0.1, grad_clip_mode=2, norm_clip=5.0), **kw)
+    tm.set_params(P)
+    dumped = str(tmp_path / "dumped.nmt")
+    tm.dump_model(dumped)
+    assert open(dumped, "rb").read() == open(want_file, "rb").read()
+    # a file the corpus preprocessor has started (first line + mappings): zero epochs of the loop
+    # append the matrices
+    head = open(want_file).read().split("\n")
+    n_head = 1 + 1 + Vs + 1 + Vt + 1
+    started = str(tmp_path / "started.nmt")
+    open(started, "w").write("\n".join(head[:n_head]) + "\n")
+    train = str(tmp_path / "train.txt")
+    open(train, "w").write("1 2\n-2 -2\n0 3\n3 1\n" * 2)
+    tm.tuning(train, output_weight_file=started, epochs=0)
+    assert open(started, "rb").read() == open(want_file, "rb").read()
+    tm.close()

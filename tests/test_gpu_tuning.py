@@ -123,3 +123,52 @@ def test_learning_rate_schedules(host, tmp_path, mode):
     got = [e[3] for e in rep["events"] if e[0] == "learning_rate"]
     assert np.allclose(got, want, rtol=1e-6), (got, want)
     assert np.isclose(rep["final_learning_rate"], want[-1], rtol=1e-6)
+
+
+@pytest.mark.parametrize("schedule", ["dev_perplexity", "google"])
+def test_training_run_from_a_file_against_the_oracles_loop(orc, host, tmp_path, schedule):
+    """FileHelper -> Dispatcher::Tuning -> ComputeGradients / UpdateWeights on the HIP path against
+    the oracle's own loop over the same file (oracle/orc.py Model.tuning and TrainingFile, written
+    from src/dispatcher.cu:96-384 and src/file_helper.cc:113-381 and pinned in
+    tests/test_oracle_tuning_pins.py): three epochs of 12 minibatches.  The learning-rate events
+    must be the same events at the same minibatches with the same values, every dev perplexity
+    within 1e-4 relative, the summed training log-likelihood of every epoch within 1e-4 relative,
+    and the parameters at the end within rtol 1e-4 / atol 2e-6."""
+    rng = np.random.default_rng(8)
+    train, dev = str(tmp_path / "train.txt"), str(tmp_path / "dev.txt")
+    _write_corpus(train, rng, 12)
+    _write_corpus(dev, rng, 2)
+    P = R.make_params(rng, 1, H, VS, VT, attention=True, feed_input=True, scale=0.1)
+    lr0, epochs = 0.5, 3
+    if schedule == "dev_perplexity":
+        # a margin that some evaluations pass and others do not: both branches of the stall rule
+        kw = dict(dev_file=dev, learning_rate_schedule=True, margin=0.35, decrease_factor=0.6)
+    else:
+        kw = dict(google_learning_rate=True, epoch_to_start_halving=2)
+    m = _model(host, lr=lr0)
+    m.set_params(P)
+    rep = m.tuning(train, epochs=epochs, **kw)
+    om = orc.Model(1, H, VS, VT, attention=1, D=2, feed_input=1, longest_sent=12)
+    om.set_params(P)
+    want, want_lr = om.tuning(train, B, lr0, epochs, clip_mode=2, norm_clip=5.0, **kw)
+
+    kinds = ("learning_rate", "half_epoch_perplexity", "epoch_perplexity", "epoch_end")
+    got = [e for e in rep["events"] if e[0] in kinds]
+    assert [e[:3] for e in got] == [tuple(e[:3]) for e in want], (got, want)
+    for g, w in zip(got, want):
+        tol = 1e-6 if g[0] == "learning_rate" else 1e-4
+        assert abs(g[3] - w[3]) <= tol * abs(w[3]), (g, w)
+    assert np.isclose(rep["final_learning_rate"], want_lr, rtol=1e-6)
+    rates = [e[3] for e in want if e[0] == "learning_rate"]
+    if schedule == "dev_perplexity":
+        n_eval = sum(1 for e in want if "perplexity" in e[0])
+        assert n_eval == 2 * epochs and 0 < len(rates) < n_eval - 1  # the rule fired and did not fire
+    else:
+        assert len(rates) == 4
+    for name in om.param_names():
+        w = om.get_param(name)
+        shape = w.shape if w.ndim == 2 else (w.size,)
+        got_p = m.get_param(name, shape)
+        assert np.allclose(got_p, w.reshape(shape, order="F"), rtol=1e-4, atol=2e-6), name
+    assert not np.array_equal(m.get_param("tgt.0.W_hi", (H, H)), P["tgt.0.W_hi"])
+    m.close()
