@@ -116,14 +116,21 @@ int lh_gemm_ws_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, 
  * serving loops and harnesses that forbid hipMalloc) and so have no workspace to hand over.  It
  * has no counterpart in the reference.  The partial planes go into an array of
  * LH_GEMM_NOALLOC_WS_BYTES that is part of the library's device code: each GPU the library runs
- * on holds its own copy until the process ends.  Same arguments, same choice of tile and split and
- * bit for bit the same result as lh_gemm_ws_f32 with a workspace of LH_GEMM_NOALLOC_WS_BYTES.  No
- * hipMalloc / hipFree and no allocating library routine is called.  A product of which two
- * partial planes (((M + 3) & ~3) x N floats each) do not fit the array is rejected with
- * LH_ERR_ARG.  Every call on a GPU shares that GPU's array (its contents between calls mean
- * nothing, nothing in it has to be cleared): calls that overlap in time on one GPU -- from
- * different streams or threads -- race on it; order them on one stream. */
+ * on holds its own copy until the process ends.  The limit: a product of which two partial planes
+ * (((M + 3) & ~3) x N floats each) do not fit the array is rejected with LH_ERR_ARG, whether or
+ * not it would be split.  For every product it accepts: same arguments, same choice of tile and
+ * split and bit for bit the same result as lh_gemm_ws_f32 with a workspace of
+ * LH_GEMM_NOALLOC_WS_BYTES.  No hipMalloc / hipFree and no allocating library routine is called.
+ * Every call on a GPU shares that GPU's array (its contents between calls mean nothing, nothing
+ * in it has to be cleared): calls that overlap in time on one GPU -- from different streams or
+ * threads -- race on it; order them on one stream.
+ * The first call on a device asks the runtime for the array's address on that device and raises
+ * the LDS limit of the kernel instance it picks (neither is a stream operation, neither
+ * allocates); a caller under graph capture does that ahead of the capture with
+ * lh_gemm_noalloc_init, once per device with that device current, and by running each product
+ * shape once before capturing it. */
 #define LH_GEMM_NOALLOC_WS_BYTES (32u << 20)
+int lh_gemm_noalloc_init(void);
 int lh_gemm_noalloc_f32(int M, int N, const lh_gemm_seg *segs, int nseg, int transA, int transX,
                         float alpha, float beta, const float *bias, int act, int act_rows,
                         const int *colmask, float *C, int ldc, lh_stream_t stream);

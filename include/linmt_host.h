@@ -184,9 +184,21 @@ void *lnmt_model_stream(lnmt_model *m);
  * On a model created for training the same switch makes the large batched products of a minibatch
  * (weight gradients accumulated over all steps, the output projection and its two backward products,
  * the layer-major input products) split products, both operands packed per call; the per-step
- * products keep the fp32 MFMA path (min_columns == 1 there takes every product: a test aid).
- * The environment variable LINMT_SPLIT_PRODUCTS=1 switches it on when a model is created. */
+ * products keep the fp32 MFMA path (min_columns == 1 there takes every product: a test aid). */
 int lnmt_set_split_products(lnmt_model *m, int on, int min_columns);
+/* Measurement and test aids of the decode path, process-wide, all 0 by default (no counterpart in
+ * the reference).  Each switches one part back to the form it replaced, with the same results up
+ * to the rounding order of the products, so that a test can demand that and a benchmark can time
+ * one form against the other:
+ *   "no_stream"               lnmt_decoding decodes batch by batch instead of as a stream;
+ *   "no_projected_memory"     decoding attends over the encoder states instead of W_a hs / W_c1 hs;
+ *   "no_lanes"                the encoder of a decoding batch runs on the model's one stream;
+ *   "grouped_gates"           what the previous step fixes of every layer's gate product runs as
+ *                             one grouped launch (lh_gate_gemm_group_f32);
+ *   "separate_beam_launches"  beam merge and state gather as two launches instead of one.
+ * An unknown name is an error.  Set them before a model is created or between calls, not while
+ * another thread decodes. */
+int lnmt_set_debug_option(const char *name, int value);
 
 /* Live kernel timing with HIP events on the model's stream.  level 0 = off, 1 = the output
  * projection (the dominant matrix product), 2 = every launch of the path.  Totals accumulate

@@ -47,8 +47,9 @@ __device__ __forceinline__ void merge_sentence(const MergeArgs &a, const int s, 
   const int limit = a.limit[s];
   const int step = a.start ? a.step - a.start[s] : a.step;
 
-  if (step >= limit) {
-    // finish (== limit) or idle (> limit): no expansion.
+  if (step >= limit || step < 0) {
+    // finish (== limit) or idle (> limit, or a slot whose sentence starts at a later tick): no
+    // expansion.
     for (int i = tid; i < beam; i += kMergeThreads) {
       s_bp[i] = c0 + i;
       if (!write) continue;

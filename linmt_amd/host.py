@@ -91,6 +91,7 @@ def load():
     lib.lnmt_model_get_grad.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
     lib.lnmt_update_weights.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
     lib.lnmt_clear_gradients.argtypes = [C.c_void_p]
+    lib.lnmt_set_debug_option.argtypes = [C.c_char_p, C.c_int]
     lib.lnmt_set_dropout_seed.argtypes = [C.c_void_p, C.c_ulonglong]
     lib.lnmt_get_dropout_mask.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                           C.c_longlong]
@@ -461,6 +462,11 @@ def _decode_stream(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penal
 
 
 Model.decode_stream = _decode_stream
+
+
+def set_debug_option(name, value):
+    """lnmt_set_debug_option: a process-wide measurement / test aid of the decode path."""
+    _check(load().lnmt_set_debug_option(name.encode(), int(value)), "set_debug_option")
 
 
 def decoding(model_file, source_file, final_file, ids_file=None, beam=12, penalty=0.0,

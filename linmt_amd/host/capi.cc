@@ -270,15 +270,18 @@ extern "C" int lnmt_decode_history(lnmt_model *m, int sentence, int *tok, int *b
   });
 }
 
-extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_models,
-                                          const int *sentences, const int *lengths, int n,
-                                          const lnmt_decode_options *o, int *best, int cap,
-                                          int *best_len, float *best_score, int *steps,
-                                          int *hyp_tokens, int *hyp_len, float *hyp_score,
-                                          int hyp_cap, int *n_hyp, int *best_viterbi,
-                                          int *kbest_index, float *kbest_score) {
+// What the two decode entry points share: sentences in, results out.  stream selects
+// DecodeStream (every beam column kept busy over a list of any length) instead of DecodeBatch.
+static int DecodeThroughFacade(bool stream, lnmt_model *const *models, int n_models,
+                               const int *sentences, const int *lengths, int n,
+                               const lnmt_decode_options *o, int *best, int cap, int *best_len,
+                               float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
+                               float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi,
+                               int *kbest_index, float *kbest_score) {
   return Guard([&] {
-    if (!models || (n_models < 1 && n_models != -1) || !models[0]) throw LinmtError("no model");
+    if (!models || n_models < 1 || !models[0]) throw LinmtError("no model");
+    if (!sentences || !lengths || !o || !best || !best_len || !best_score || n < 0 || cap < 1)
+      throw LinmtError("decode: NULL argument or negative count");
     lnmt_model *m = models[0];
     std::vector<NeuralMachineTranslation *> others;
     for (int k = 1; k < n_models; ++k) {
@@ -303,7 +306,7 @@ extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_model
     d.unk_replacement_mode_ = o->unk_replacement_mode != 0;
     d.hypotheses_number_ = std::max(1, o->num_hypotheses);
     std::vector<SentenceResult> res;
-    if (n_models == -1)  // lnmt_decode_stream
+    if (stream)
       m->nmt->DecodeStream(sents, d, &res);
     else
       m->nmt->DecodeBatch(sents, d, &res, others);
@@ -338,14 +341,25 @@ extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_model
   });
 }
 
+extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_models,
+                                          const int *sentences, const int *lengths, int n,
+                                          const lnmt_decode_options *o, int *best, int cap,
+                                          int *best_len, float *best_score, int *steps,
+                                          int *hyp_tokens, int *hyp_len, float *hyp_score,
+                                          int hyp_cap, int *n_hyp, int *best_viterbi,
+                                          int *kbest_index, float *kbest_score) {
+  return DecodeThroughFacade(false, models, n_models, sentences, lengths, n, o, best, cap, best_len,
+                             best_score, steps, hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp,
+                             best_viterbi, kbest_index, kbest_score);
+}
+
 extern "C" int lnmt_decode_stream(lnmt_model *m, const int *sentences, const int *lengths, int n,
                                   const lnmt_decode_options *o, int *best, int cap, int *best_len,
                                   float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
                                   float *hyp_score, int hyp_cap, int *n_hyp, int *ticks) {
-  // n_models = -1 selects DecodeStream inside the shared marshalling
-  const int rc = lnmt_decode_batch_ensemble(&m, -1, sentences, lengths, n, o, best, cap, best_len, best_score,
-                                            steps, hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, nullptr,
-                                            nullptr, nullptr);
+  const int rc = DecodeThroughFacade(true, &m, m ? 1 : 0, sentences, lengths, n, o, best, cap, best_len, best_score,
+                                     steps, hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, nullptr,
+                                     nullptr, nullptr);
   if (rc == 0 && ticks) *ticks = m->nmt->stream_ticks_;
   return rc;
 }
@@ -358,6 +372,27 @@ extern "C" int lnmt_profile_set_level(lnmt_model *m, int level) {
     m->nmt->profiler_.Collect();
     m->nmt->profiler_.Reset();
     m->nmt->profiler_.level_ = level;
+  });
+}
+
+namespace linmt {
+DebugOptions &Debug() {
+  static DebugOptions options;
+  return options;
+}
+}  // namespace linmt
+
+extern "C" int lnmt_set_debug_option(const char *name, int value) {
+  return Guard([&] {
+    if (!name) throw LinmtError("lnmt_set_debug_option: NULL name");
+    DebugOptions &d = linmt::Debug();
+    const std::string n(name);
+    if (n == "no_stream") d.no_stream = value;
+    else if (n == "no_projected_memory") d.no_projected_memory = value;
+    else if (n == "no_lanes") d.no_lanes = value;
+    else if (n == "grouped_gates") d.grouped_gates = value;
+    else if (n == "separate_beam_launches") d.separate_beam_launches = value;
+    else throw LinmtError("lnmt_set_debug_option: unknown option " + n);
   });
 }
 

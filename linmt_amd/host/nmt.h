@@ -56,6 +56,18 @@ struct GlobalConfiguration {
 };
 
 class NeuralMachineTranslation;
+
+// Measurement and test aids (lnmt_set_debug_option), process-wide, all off by default: each one
+// switches a part of the decode path back to the form it replaced, so that a test can demand the
+// same results of both forms and a benchmark can time them against each other.
+struct DebugOptions {
+  int no_stream = 0;               // Dispatcher::Decoding decodes batch by batch, never as a stream
+  int no_projected_memory = 0;     // decoding attends over the encoder states themselves (the step's own products)
+  int no_lanes = 0;                // the encoder of a decoding batch runs on the model's one stream
+  int grouped_gates = 0;           // what the previous step fixes of every layer's gate product in one grouped launch
+  int separate_beam_launches = 0;  // beam merge and state gather as the two launches the fused one replaces
+};
+DebugOptions &Debug();
 class LstmLayer;
 class AttentionLayer;
 

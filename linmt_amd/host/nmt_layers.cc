@@ -560,7 +560,7 @@ bool AttentionLayer::ProjectedMemoryPossible() const {
   return use_hs_col_ && !global_mode_ && !p_neural_mt_->cfg_.train_mode_ &&
          window_ <= LH_ATTN_PROJECTED_MAX_WINDOW && lstm_size_ <= LH_ATTN_PROJECTED_MAX_H &&
          lstm_size_ % 4 == 0 && hs_col_stride_ == lstm_size_ && hs_step_stride_ % lstm_size_ == 0 &&
-         !std::getenv("LINMT_NO_PROJECTED_MEMORY");  // measurement aid: the step's own products
+         !Debug().no_projected_memory;  // measurement aid: the step's own products
 }
 
 void AttentionLayer::BuildOutputStack() {

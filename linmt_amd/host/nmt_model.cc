@@ -119,7 +119,6 @@ void NeuralMachineTranslation::Synchronize() {
 // One node per timestep on both sides, minibatch = cfg.minibatch_size_ (deep_rnn.h:249-692).
 void NeuralMachineTranslation::InitModel() {
   decode_mode_ = false;
-  if (const char *sp = std::getenv("LINMT_SPLIT_PRODUCTS")) split_products_ = sp[0] == '1';
   const int B = cfg_.minibatch_size_, T = cfg_.longest_sentence_, L = cfg_.num_layers_;
   const bool seq2seq = cfg_.sequence_to_sequence_mode_;
   const bool keep = cfg_.train_mode_;  // training keeps i,f,g,o and the looked-up embeddings per step
@@ -166,7 +165,6 @@ void NeuralMachineTranslation::InitModel() {
 // target side: ONE node, n_sent*beam columns, previous-state buffers (deep_rnn.h:697-922).
 void NeuralMachineTranslation::InitModelDecoding(int n_sent, int beam_size) {
   decode_mode_ = true;
-  if (const char *sp = std::getenv("LINMT_SPLIT_PRODUCTS")) split_products_ = sp[0] == '1';
   n_sent_ = n_sent;
   beam_size_ = beam_size;
   const int L = cfg_.num_layers_, T = cfg_.longest_sentence_, H = cfg_.lstm_size_;
@@ -464,7 +462,7 @@ void NeuralMachineTranslation::ForwardPropSource(const int *p_host_source, int s
 // one layer at a time: the layer's input products for all steps in one GEMM, then the recurrence.
 void NeuralMachineTranslation::RunSourceSide(int source_length, int B) {
   const int L = cfg_.num_layers_;
-  const bool lanes_off = getenv("LINMT_NO_LANES") != nullptr;  // measurement and test aid
+  const bool lanes_off = Debug().no_lanes != 0;  // measurement and test aid
   bool lanes = !lanes_off && decode_mode_ && L > 1 && L <= 4 && profiler_.level_ < 2 &&
                source_length > kLaneChunkSteps;
   for (int l = 0; l < L && lanes; ++l)
@@ -562,9 +560,8 @@ void NeuralMachineTranslation::ForwardPropTarget(int curr_index, int *p_device_c
     }
     flush();
   }
-  const char *grouped = std::getenv("LINMT_GROUPED_GATES");
-  if (!split_step_ && decode_mode_ && !apply_dropout_ && L >= 2 && L <= LH_GATE_GROUP_MAX && grouped &&
-      grouped[0] == '1') {
+  if (!split_step_ && decode_mode_ && !apply_dropout_ && L >= 2 && L <= LH_GATE_GROUP_MAX &&
+      Debug().grouped_gates) {
     lh_gate_problem problems[LH_GATE_GROUP_MAX];
     for (int l = 0; l < L; ++l) TargetLayer(l).v_nodes_[0].DescribeRecurrentProblem(l == 0, &problems[l]);
     int runnable = 0;
@@ -923,7 +920,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
 
   std::vector<int> active_at(max_limit + 1);
   int *p_device_step_indices = d.current_indices_.get();  // <START> for every column
-  const bool separate_beam_launches = getenv("LINMT_SEPARATE_BEAM_LAUNCHES") != nullptr;  // measurement and test aid
+  const bool separate_beam_launches = Debug().separate_beam_launches != 0;  // measurement and test aid
   for (int step = 0; step <= max_limit; ++step) {
     int n_active = 0;
     while (n_active < n && limit[n_active] >= step) ++n_active;  // limits are non-increasing

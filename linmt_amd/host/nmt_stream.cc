@@ -348,6 +348,15 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
     for (int step = 0; step <= limit[i]; ++step)
       for (int j = 0; j < beam; ++j) {
         const size_t from = (size_t)(t0 + step + 1) * B + c0 + j, to = (size_t)step * Bn + (size_t)i * beam + j;
+        if (step == limit[i]) {
+          // the row a sentence's last step writes is the row the slot's next sentence is admitted
+          // into: what the step stored there (<EOF>, the column itself, the final score) is taken
+          // from the finished-hypothesis record of the same step instead
+          hist.tok[to] = Decoder::end_symbol_;
+          hist.backptr[to] = i * beam + j;
+          hist.score[to] = fscore[(size_t)(t0 + step) * B + c0 + j];
+          continue;
+        }
         hist.tok[to] = tok[from];
         hist.backptr[to] = bp[from] - c0 + i * beam;
         hist.score[to] = bscore[from];

@@ -62,6 +62,7 @@ SIGNATURES = {
     "lh_gemm_ws_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int, C.c_int,
                                  C.c_float, C.c_float, c_f32p, C.c_int, C.c_int, c_i32p, c_f32p,
                                  C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "lh_gemm_noalloc_init": (C.c_int, []),
     "lh_gemm_noalloc_f32": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmSeg), C.c_int, C.c_int,
                                       C.c_int, C.c_float, C.c_float, c_f32p, C.c_int, C.c_int,
                                       c_i32p, c_f32p, C.c_int, C.c_void_p]),
@@ -271,6 +272,10 @@ def gemm(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0
 
 
 LH_GEMM_NOALLOC_WS_BYTES = 32 << 20
+
+
+def gemm_noalloc_init():
+    check(load().lh_gemm_noalloc_init(), "lh_gemm_noalloc_init")
 
 
 def gemm_noalloc(M, N, segs, C_out, ldc, transA=False, transX=False, alpha=1.0, beta=0.0,

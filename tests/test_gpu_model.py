@@ -220,11 +220,13 @@ def test_decode_same_with_and_without_the_regrouped_step(orc, host, monkeypatch)
     P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 40, 0.35, decoding=(5, beam))
     sents = [rng.integers(0, Vs, size=n) for n in (17, 9, 12, 3, 21)]
     fast = gm.decode_batch(sents, beam=beam, with_hyps=True, alignments=True)
-    monkeypatch.setenv("LINMT_NO_PROJECTED_MEMORY", "1")
-    monkeypatch.setenv("LINMT_NO_LANES", "1")
-    plain = gm.decode_batch(sents, beam=beam, with_hyps=True, alignments=True)
-    monkeypatch.delenv("LINMT_NO_PROJECTED_MEMORY")
-    monkeypatch.delenv("LINMT_NO_LANES")
+    host.set_debug_option("no_projected_memory", 1)
+    host.set_debug_option("no_lanes", 1)
+    try:
+        plain = gm.decode_batch(sents, beam=beam, with_hyps=True, alignments=True)
+    finally:
+        host.set_debug_option("no_projected_memory", 0)
+        host.set_debug_option("no_lanes", 0)
     for i, (a, b) in enumerate(zip(fast, plain)):
         assert a["best"].tolist() == b["best"].tolist(), i
         assert a["best_viterbi"].tolist() == b["best_viterbi"].tolist(), i
@@ -237,7 +239,7 @@ def test_decode_same_with_and_without_the_regrouped_step(orc, host, monkeypatch)
 
 def test_decode_same_with_separate_beam_launches(orc, host, monkeypatch):
     """The merge and the state swap of a step as one launch (lh_beam_merge_gather_f32, the default
-    with one model) and as the two launches it replaces (LINMT_SEPARATE_BEAM_LAUNCHES=1): the same
+    with one model) and as the two launches it replaces (debug option "separate_beam_launches"): the same
     kernels' arithmetic, so every token, score and hypothesis is equal bit for bit."""
     rng = np.random.default_rng(23)
     layers, H, Vs, Vt, D, beam = 2, 64, 150, 170, 3, 5
@@ -246,11 +248,13 @@ def test_decode_same_with_separate_beam_launches(orc, host, monkeypatch):
     gm.profile(2)
     one = gm.decode_batch(sents, beam=beam, with_hyps=True)
     assert "beam_merge_gather" in gm.profile_totals(), "the single launch did not run"
-    monkeypatch.setenv("LINMT_SEPARATE_BEAM_LAUNCHES", "1")
-    gm.profile(2)
-    two = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    host.set_debug_option("separate_beam_launches", 1)
+    try:
+        gm.profile(2)
+        two = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    finally:
+        host.set_debug_option("separate_beam_launches", 0)
     assert "beam_gather" in gm.profile_totals() and "beam_merge_gather" not in gm.profile_totals()
-    monkeypatch.delenv("LINMT_SEPARATE_BEAM_LAUNCHES")
     gm.profile(0)
     for i, (a, b) in enumerate(zip(one, two)):
         assert a["best"].tolist() == b["best"].tolist() and a["best_score"] == b["best_score"], i
@@ -261,7 +265,7 @@ def test_decode_same_with_separate_beam_launches(orc, host, monkeypatch):
 
 
 def test_decode_same_with_grouped_gate_products(orc, host, monkeypatch):
-    """LINMT_GROUPED_GATES=1 issues what the previous step fixes of every layer's gate product as
+    """The debug option "grouped_gates" issues what the previous step fixes of every layer's gate product as
     one grouped launch (lh_gate_gemm_group_f32) and leaves M*h of the layer below on the chain.
     Same arithmetic up to the order of two additions: same translations, scores inside the
     floating-point tolerance, both equal to the oracle's."""
@@ -270,12 +274,14 @@ def test_decode_same_with_grouped_gate_products(orc, host, monkeypatch):
     P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 40, 0.35, decoding=(5, beam))
     sents = [rng.integers(0, Vs, size=n) for n in (17, 9, 12, 3, 21)]
     plain = gm.decode_batch(sents, beam=beam, with_hyps=True)
-    monkeypatch.setenv("LINMT_GROUPED_GATES", "1")
-    gm.profile(2)
-    grouped = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    host.set_debug_option("grouped_gates", 1)
+    try:
+        gm.profile(2)
+        grouped = gm.decode_batch(sents, beam=beam, with_hyps=True)
+    finally:
+        host.set_debug_option("grouped_gates", 0)
     assert any("gate_gemm_group_kernel" in k for k in gm.profile_totals()), "the grouped launch did not run"
     gm.profile(0)
-    monkeypatch.delenv("LINMT_GROUPED_GATES")
     for i, (a, b) in enumerate(zip(grouped, plain)):
         assert a["best"].tolist() == b["best"].tolist(), i
         assert np.isclose(a["best_score"], b["best_score"], rtol=1e-4, atol=1e-5), i

@@ -253,14 +253,14 @@ def test_k_best_lists(host, tmp_path):
     # that run went through DecodeStream (one model, no exported alignments); batch by batch gives
     # the same lines
     import os
-    os.environ["LINMT_NO_STREAM"] = "1"
+    host.set_debug_option("no_stream", 1)
     try:
         ids2 = str(tmp_path / "out2.ids")
         host.decoding(model, str(src), str(tmp_path / "out2.txt"), ids_file=ids2, beam=beam,
                       longest_sentence=24, attention_width=D, print_decoding_information=True,
                       sentences_per_batch=2, num_hypotheses=k)
     finally:
-        del os.environ["LINMT_NO_STREAM"]
+        host.set_debug_option("no_stream", 0)
     lines2 = open(ids2).read().split("\n")[:-1]
     assert [l.split(" |||| ")[0] for l in lines2] == [l.split(" |||| ")[0] for l in lines]
 
@@ -312,14 +312,14 @@ def test_decoding_a_long_text_file_through_the_stream(host, tmp_path):
         assert [int(x) for x in fields[0].split()] == w["best"].tolist(), k
         assert np.isclose(float(fields[1]), w["best_score"], rtol=1e-5, atol=1e-4), k  # six digits in the file
     assert rep["target_words"] == sum(len(w["best"]) for w in want if w is not None)
-    os.environ["LINMT_NO_STREAM"] = "1"
+    host.set_debug_option("no_stream", 1)
     try:
         ids2 = str(tmp_path / "out2.ids")
         host.decoding(model, str(src), str(tmp_path / "out2.txt"), ids_file=ids2, beam=beam,
                       longest_sentence=24, attention_width=D, print_decoding_information=True,
                       sentences_per_batch=n_sent)
     finally:
-        del os.environ["LINMT_NO_STREAM"]
+        host.set_debug_option("no_stream", 0)
     got2 = open(ids2).read().split("\n")[:-1]
     same = sum(x.split(" |||| ")[0] == y.split(" |||| ")[0] for x, y in zip(got, got2))
     assert len(got2) == 150 and same >= 147, same  # a near-tie may fall the other way between the two modes

@@ -18,7 +18,7 @@ def host(t, shape):
     return t.cpu().numpy().reshape(shape[::-1]).T
 
 
-def _case(lh, rng, M, N, Ks, tA, tX, epilogue):
+def _case(lh, rng, M, N, Ks, tA, tX, epilogue, check_memory=True):
     As = [rng.uniform(-0.5, 0.5, size=((K, M) if tA else (M, K))).astype(np.float32) for K in Ks]
     Xs = [rng.uniform(-1, 1, size=((N, K) if tX else (K, N))).astype(np.float32) for K in Ks]
     segs = [(dev(A), A.shape[0], dev(X), X.shape[0], K) for A, X, K in zip(As, Xs, Ks)]
@@ -34,8 +34,15 @@ def _case(lh, rng, M, N, Ks, tA, tX, epilogue):
     ref = dev(C0)
     lh.gemm(M, N, segs, ref, M, transA=tA, transX=tX, workspace=ws, **kw)
     got = dev(C0)
+    # nothing is allocated by the call: the caching allocator's books and the device's free memory
+    # are the same before and after it (the first call on the device has already happened: init)
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0])
     lh.gemm_noalloc(M, N, segs, got, M, transA=tA, transX=tX, **kw)
     torch.cuda.synchronize()
+    after = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0])
+    if check_memory:
+        assert after[:2] == before[:2] and after[2] >= before[2], (before, after)
     return host(got, (M, N)), host(ref, (M, N)), want
 
 
@@ -50,6 +57,14 @@ def test_noalloc_gemm_equals_workspace_gemm(lh):
              ((200, 76, (100, 36), False, False, True), 3),
              ((37, 13, (101,), False, False, True), 0)]
     split_seen = False
+    lh.gemm_noalloc_init()
+    # each kernel instance's one-time set-up (the LDS limit) happens on a first, unchecked round
+    try:
+        for (M, N, Ks, tA, tX, epi), forced in calls:
+            L.lh_gemm_set_splits_override(forced)
+            _case(lh, np.random.default_rng(1), M, N, Ks, tA, tX, epi, check_memory=False)
+    finally:
+        L.lh_gemm_set_splits_override(0)
     try:
         for (M, N, Ks, tA, tX, epi), forced in calls:
             L.lh_gemm_set_splits_override(forced)
