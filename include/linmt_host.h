@@ -104,6 +104,14 @@ int lnmt_model_get_grad(lnmt_model *m, const char *name, float *data, long long 
 /* NeuralMachineTranslation::UpdateWeights + ClearGradients.  *global_norm (may be NULL) receives
  * the norm the global clip used (0 in the other modes). */
 int lnmt_update_weights(lnmt_model *m, double *global_norm);
+/* Which parameter groups lnmt_update_weights moves, the reference's train_*_mode__ switches
+ * (src/utility_cu.cu:17-22, read by UpdateParams: src/layer_input_to_hidden.h:1154,1257,1263,
+ * src/layer_hidden_to_hidden.h:765,831, src/layer_loss.h:1144).  All 1 at first; --finetune is
+ * (0, 0, 0, 1, 1, 1) (src/global_configuration.cc:647-656).  A frozen group's gradients are
+ * computed, count in the global norm and are cleared like the others; only the step is left out. */
+int lnmt_set_train_modes(lnmt_model *m, int source_input_embedding, int target_input_embedding,
+                         int target_output_embedding, int source_rnn, int target_rnn,
+                         int attention_target_rnn);
 /* The dropout masks the last lnmt_compute_gradients call drew (uniform numbers, kept when
  * < dropout_keep): kind 0 = embeddings of side (0 src / 1 tgt), kind 1 = the mask under which the
  * consumer above `layer` read that layer's h.  Layout rows x minibatch x steps column-major;

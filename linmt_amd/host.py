@@ -91,6 +91,7 @@ def load():
     lib.lnmt_model_get_grad.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_longlong]
     lib.lnmt_update_weights.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
     lib.lnmt_clear_gradients.argtypes = [C.c_void_p]
+    lib.lnmt_set_train_modes.argtypes = [C.c_void_p] + [C.c_int] * 6
     lib.lnmt_set_debug_option.argtypes = [C.c_char_p, C.c_int]
     lib.lnmt_set_dropout_seed.argtypes = [C.c_void_p, C.c_ulonglong]
     lib.lnmt_get_dropout_mask.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
@@ -357,6 +358,15 @@ class Model:
 
     def clear_gradients(self):
         _check(load().lnmt_clear_gradients(self.handle), "clear_gradients")
+
+    def set_train_modes(self, source_input_embedding=True, target_input_embedding=True,
+                        target_output_embedding=True, source_rnn=True, target_rnn=True,
+                        attention_target_rnn=True):
+        """The reference's train_*_mode__ switches (finetune = the three embedding groups off)."""
+        _check(load().lnmt_set_train_modes(self.handle, int(source_input_embedding),
+                                           int(target_input_embedding), int(target_output_embedding),
+                                           int(source_rnn), int(target_rnn), int(attention_target_rnn)),
+               "set_train_modes")
 
     def set_dropout_seed(self, seed):
         _check(load().lnmt_set_dropout_seed(self.handle, seed), "set_dropout_seed")

@@ -184,6 +184,21 @@ extern "C" int lnmt_set_dropout_seed(lnmt_model *m, unsigned long long seed) {
   });
 }
 
+extern "C" int lnmt_set_train_modes(lnmt_model *m, int source_input_embedding, int target_input_embedding,
+                                    int target_output_embedding, int source_rnn, int target_rnn,
+                                    int attention_target_rnn) {
+  return Guard([&] {
+    GlobalConfiguration &c = m->nmt->cfg_;
+    if (!c.train_mode_) throw LinmtError("lnmt_set_train_modes: not a training model");
+    c.train_source_input_embedding_mode_ = source_input_embedding != 0;
+    c.train_target_input_embedding_mode_ = target_input_embedding != 0;
+    c.train_target_output_embedding_mode_ = target_output_embedding != 0;
+    c.train_source_rnn_mode_ = source_rnn != 0;
+    c.train_target_rnn_mode_ = target_rnn != 0;
+    c.train_attention_target_rnn_mode_ = attention_target_rnn != 0;
+  });
+}
+
 extern "C" int lnmt_model_set_param(lnmt_model *m, const char *name, const float *data,
                                     long long n) {
   return Guard([&] {

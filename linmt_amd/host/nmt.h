@@ -53,6 +53,15 @@ struct GlobalConfiguration {
   bool dropout_mode_ = false;
   float dropout_rate_ = 1.0f;
   unsigned long long dropout_seed_ = 1;
+  // Which parameter groups UpdateParams moves (src/utility_cu.cu:17-22; --finetune switches the
+  // three embedding groups off, src/global_configuration.cc:647-656).  A frozen group's gradients
+  // are still computed, still count in the global norm, and are cleared as usual.
+  bool train_source_input_embedding_mode_ = true;
+  bool train_target_input_embedding_mode_ = true;
+  bool train_target_output_embedding_mode_ = true;
+  bool train_source_rnn_mode_ = true;
+  bool train_target_rnn_mode_ = true;
+  bool train_attention_target_rnn_mode_ = true;
 };
 
 class NeuralMachineTranslation;

@@ -715,6 +715,7 @@ struct UpdateItem {
   long long ld_grad, rows, cols;
   const int *col_index;
   bool in_global_norm;
+  bool frozen;  // UpdateParams leaves the parameters alone; the gradient is only cleared
 };
 }  // namespace
 
@@ -725,42 +726,50 @@ void NeuralMachineTranslation::UpdateWeights() {
   std::vector<UpdateItem> items;
   // Stacked parameters are one tensor when the norm is global or absent; the per-matrix clip of
   // the reference norms W_hi, W_hf, ... separately, i.e. per gate block.
-  auto add_stack = [&](DeviceArray<float> &theta, DeviceArray<float> &grad, int K) {
+  auto add_stack = [&](DeviceArray<float> &theta, DeviceArray<float> &grad, int K, bool frozen) {
     if (mode == 1) {
       for (int g = 0; g < 4; ++g)
         items.push_back({theta.get() + (size_t)g * H, 4LL * H, grad.get() + (size_t)g * H, 4LL * H, H, K,
-                         nullptr, true});
+                         nullptr, true, frozen});
     } else {
-      items.push_back({theta.get(), 4LL * H, grad.get(), 4LL * H, 4LL * H, K, nullptr, true});
+      items.push_back({theta.get(), 4LL * H, grad.get(), 4LL * H, 4LL * H, K, nullptr, true, frozen});
     }
   };
-  auto add_layer = [&](LstmLayer &Ly) {
-    add_stack(Ly.p_device_w_h_stack_, Ly.p_device_w_h_grad_, H);
-    add_stack(Ly.p_device_b_stack_, Ly.p_device_b_grad_, 1);
-    add_stack(Ly.p_device_m_stack_, Ly.p_device_m_grad_, Ly.input_size_);
-    if (Ly.feed_input_mode_) add_stack(Ly.p_device_q_stack_, Ly.p_device_q_grad_, H);
+  // the switches of InputToHiddenLayer / HiddenToHiddenLayer::UpdateParams
+  // (src/layer_input_to_hidden.h:1154,1257,1263, src/layer_hidden_to_hidden.h:765,831)
+  auto add_layer = [&](LstmLayer &Ly, bool source_side) {
+    const bool rnn_frozen = source_side ? !cfg_.train_source_rnn_mode_ : !cfg_.train_target_rnn_mode_;
+    const bool emb_frozen = source_side ? !cfg_.train_source_input_embedding_mode_
+                                        : !cfg_.train_target_input_embedding_mode_;
+    add_stack(Ly.p_device_w_h_stack_, Ly.p_device_w_h_grad_, H, rnn_frozen);
+    add_stack(Ly.p_device_b_stack_, Ly.p_device_b_grad_, 1, rnn_frozen);
+    add_stack(Ly.p_device_m_stack_, Ly.p_device_m_grad_, Ly.input_size_, rnn_frozen);
+    if (Ly.feed_input_mode_) add_stack(Ly.p_device_q_stack_, Ly.p_device_q_grad_, H, rnn_frozen);
     if (Ly.input_layer_mode_ && Ly.w_grad_length_ > 0)
       items.push_back({Ly.p_device_w_.get(), Ly.input_size_, Ly.p_device_small_w_grad_.get(),
                        Ly.input_size_, Ly.input_size_, Ly.w_grad_length_,
-                       Ly.p_device_input_vocab_indices_wgrad_.get(), false});
+                       Ly.p_device_input_vocab_indices_wgrad_.get(), false, emb_frozen});
   };
-  auto add_flat = [&](DeviceArray<float> &theta, DeviceArray<float> &grad) {
+  auto add_flat = [&](DeviceArray<float> &theta, DeviceArray<float> &grad, bool frozen) {
     items.push_back({theta.get(), (long long)theta.size(), grad.get(), (long long)theta.size(),
-                     (long long)theta.size(), 1, nullptr, true});
+                     (long long)theta.size(), 1, nullptr, true, frozen});
   };
-  add_flat(softmax_layer_.p_device_d_, softmax_layer_.p_device_d_grad_);
-  add_flat(softmax_layer_.p_device_b_d_, softmax_layer_.p_device_b_d_grad_);
+  // SoftmaxLayer::UpdateWeightsGpu (src/layer_loss.h:1144)
+  const bool out_frozen = !cfg_.train_target_output_embedding_mode_;
+  add_flat(softmax_layer_.p_device_d_, softmax_layer_.p_device_d_grad_, out_frozen);
+  add_flat(softmax_layer_.p_device_b_d_, softmax_layer_.p_device_b_d_grad_, out_frozen);
   for (int side = cfg_.sequence_to_sequence_mode_ ? 0 : 1; side < 2; ++side)
-    for (int l = 0; l < L; ++l) add_layer(side == 0 ? SourceLayer(l) : TargetLayer(l));
+    for (int l = 0; l < L; ++l) add_layer(side == 0 ? SourceLayer(l) : TargetLayer(l), side == 0);
   if (cfg_.attention_mode_ && cfg_.sequence_to_sequence_mode_) {
     AttentionLayer &A = attention_layer_;
-    add_flat(A.p_device_w_a_, A.p_device_w_a_grad_);
-    add_flat(A.p_device_w_c_p1_, A.p_device_w_c_p1_grad_);
-    add_flat(A.p_device_w_c_p2_, A.p_device_w_c_p2_grad_);
-    add_flat(A.p_device_output_bias_, A.p_device_output_bias_grad_);
+    const bool f = !cfg_.train_attention_target_rnn_mode_;
+    add_flat(A.p_device_w_a_, A.p_device_w_a_grad_, f);
+    add_flat(A.p_device_w_c_p1_, A.p_device_w_c_p1_grad_, f);
+    add_flat(A.p_device_w_c_p2_, A.p_device_w_c_p2_grad_, f);
+    add_flat(A.p_device_output_bias_, A.p_device_output_bias_grad_, f);
     if (!A.global_mode_) {
-      add_flat(A.p_device_w_p_, A.p_device_w_p_grad_);
-      add_flat(A.p_device_v_p_, A.p_device_v_p_grad_);
+      add_flat(A.p_device_w_p_, A.p_device_w_p_grad_, f);
+      add_flat(A.p_device_v_p_, A.p_device_v_p_grad_, f);
     }
   }
   if (items.size() > p_device_norms_.size()) p_device_norms_.Alloc(items.size() + 64);
@@ -780,6 +789,13 @@ void NeuralMachineTranslation::UpdateWeights() {
   for (size_t i = 0; i < items.size(); ++i) {
     const UpdateItem &it = items[i];
     const double *nrm = mode == 2 ? p_device_norms_.get() : (mode == 1 ? p_device_norms_.get() + i : nullptr);
+    if (it.frozen) {
+      // the gradient is dropped, row block by row block (columns are ld_grad apart)
+      HipErrorWrapper(hipMemset2DAsync(it.grad, sizeof(float) * it.ld_grad, 0, sizeof(float) * it.rows,
+                                       (size_t)it.cols, stream_),
+                      "UpdateParams: clearing a frozen group's gradient failed");
+      continue;
+    }
     ProfileScope ps(profiler_, kTagUpdate, 16.0 * it.rows * it.cols);
     LhErrorWrapper(lh_sgd_step_f32(it.theta, it.ld_theta, it.grad, it.ld_grad, it.rows, it.cols,
                                    it.col_index, cfg_.learning_rate_, scale, nrm, cfg_.norm_clip_,

@@ -206,6 +206,7 @@ void orc_trainer_set_dropout(orc_trainer *t, float keep, const float *src_embed,
  * gradients agree with central differences of the numpy forward wherever no clamp was active
  * (tests/test_oracle_train_pins.py). */
 void orc_trainer_set_clip(orc_trainer *t, float cell_clip, float error_clip);
+void orc_trainer_set_train_modes(orc_trainer *t, const int *modes);
 /* NeuralMachineTranslation::ComputeGradients without its final UpdateWeights: forward with stored
  * activations, then the backward pass.  Arguments as orc_forward_xent; src_unique / tgt_unique are
  * the unique non-pad input ids of the minibatch (the reference's *_wgrad lists).  Returns the summed

@@ -63,6 +63,8 @@ struct orc_trainer {
   // (src/node_input_to_hidden.h:599-601, src/node_hidden_to_hidden.h:416-418) and the errors a node
   // hands on clamped to +-error_clip (below).  0 = off.
   float cell_clip = 0.f, error_clip = 0.f;
+  // train_*_mode__ switches of UpdateParams, see orc_trainer_set_train_modes
+  bool train_modes[6] = {true, true, true, true, true, true};
 };
 
 namespace {
@@ -618,6 +620,24 @@ extern "C" double orc_compute_gradients(orc_trainer *t, const int *src, int S, c
 //   clip_mode 0: nothing.
 // Then theta += learning_rate * g (embeddings: only the columns of the unique ids) and the gradients
 // are cleared.  Returns the global norm (clip_mode 2) or 0.
+// The train_*_mode__ switches read by UpdateParams (src/layer_input_to_hidden.h:1154,1257,1263,
+// src/layer_hidden_to_hidden.h:765,831, src/layer_loss.h:1144): modes[0..5] = source input
+// embedding, target input embedding, target output embedding (D, b_d), source LSTM matrices,
+// target LSTM matrices, attention.  The norms above them are taken over every gradient all the same
+// (CalculateGlobalNorm has no such switch).
+extern "C" void orc_trainer_set_train_modes(orc_trainer *t, const int *modes) {
+  for (int i = 0; i < 6; ++i) t->train_modes[i] = modes[i] != 0;
+}
+static bool frozen(const orc_trainer *t, const std::string &name) {
+  if (name == "src.0.W") return !t->train_modes[0];
+  if (name == "tgt.0.W") return !t->train_modes[1];
+  if (name.compare(0, 8, "softmax.") == 0) return !t->train_modes[2];
+  if (name.compare(0, 4, "src.") == 0) return !t->train_modes[3];
+  if (name.compare(0, 4, "tgt.") == 0) return !t->train_modes[4];
+  if (name.compare(0, 5, "attn.") == 0) return !t->train_modes[5];
+  return false;
+}
+
 extern "C" float orc_update_weights(orc_trainer *t, float learning_rate, int clip_mode,
                                     float norm_clip, float individual_clip, int minibatch_size) {
   const int H = emb(t);  // only the embedding columns are addressed by row below
@@ -681,6 +701,10 @@ extern "C" float orc_update_weights(orc_trainer *t, float learning_rate, int cli
     long long n = 0;
     float *p = orc_model_param(t->m, kv.first.c_str(), &n);
     if (!p) continue;
+    if (frozen(t, kv.first)) {  // UpdateParams skips the group; ClearGradients still runs
+      std::fill(kv.second.begin(), kv.second.end(), 0.f);
+      continue;
+    }
     if (kv.first == "src.0.W" || kv.first == "tgt.0.W") {
       const std::vector<int> &u = t->uniq[kv.first == "src.0.W" ? 0 : 1];
       for (size_t k = 0; k < u.size(); ++k)  // UpdateSparseGradient

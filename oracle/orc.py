@@ -571,6 +571,14 @@ class Model:
         """The reference's --clip-cell for the following compute_gradients calls (0 = off)."""
         lib().orc_trainer_set_clip(self._trainer(), _f(cell_clip), _f(error_clip))
 
+    def set_train_modes(self, source_input_embedding=True, target_input_embedding=True,
+                        target_output_embedding=True, source_rnn=True, target_rnn=True,
+                        attention_target_rnn=True):
+        """The train_*_mode__ switches UpdateParams reads (finetune: the three embedding groups off)."""
+        modes = i32([source_input_embedding, target_input_embedding, target_output_embedding,
+                     source_rnn, target_rnn, attention_target_rnn])
+        lib().orc_trainer_set_train_modes(self._trainer(), _p(modes))
+
     def compute_gradients(self, src, tgt_in, tgt_out, batch_info, src_unique, tgt_unique):
         """Forward + backward (no update).  Returns (sum log p, {name: gradient}); matrices come back
         as Fortran-ordered 2-D arrays, the embedding gradients as (E, n_unique)."""

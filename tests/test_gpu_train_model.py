@@ -232,6 +232,48 @@ def test_update_weights_vs_oracle(orc, host, mode, E):
     gm.close()
 
 
+@pytest.mark.parametrize("modes,mode", [((0, 0, 0, 1, 1, 1), 2), ((1, 1, 1, 0, 1, 0), 2), ((1, 0, 1, 1, 0, 1), 1)],
+                         ids=["finetune", "source_rnn_and_attention_frozen", "target_side_frozen_per_matrix_clip"])
+def test_update_weights_with_frozen_groups_vs_oracle(orc, host, modes, mode):
+    """lnmt_set_train_modes, the reference's train_*_mode__ switches of UpdateParams
+    (src/layer_input_to_hidden.h:1154,1257,1263, src/layer_hidden_to_hidden.h:765,831,
+    src/layer_loss.h:1144; --finetune = the three embedding groups off): two minibatches, the
+    frozen groups keep their bits, the others and the global norm follow the oracle."""
+    rng = np.random.default_rng(90)
+    layers, H, Vs, Vt, D = 2, 16, 29, 41, 2
+    lens_s, lens_t = [5, 3, 9, 4], [4, 6, 2, 8]
+    B, lr = len(lens_s), 0.7
+    opts = dict(learning_rate=lr, grad_clip_mode=mode, norm_clip=0.05, individual_clip=0.002)
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 1, 1, B, opts, scale=0.8)
+    om.set_train_modes(*modes)
+    gm.set_train_modes(*modes)
+
+    def group(name):
+        if name in ("src.0.W", "tgt.0.W"):
+            return 0 if name[0] == "s" else 1
+        return {"softmax": 2, "src": 3, "tgt": 4, "attn": 5}[name.split(".")[0]]
+
+    for it in range(2):
+        sents, (src, tin, tout, bi, su, tu) = _minibatch(rng, Vs, Vt, lens_s, lens_t)
+        om.compute_gradients(src, tin, tout, bi, su, tu)
+        gm.compute_gradients(src, tin, tout, bi, su, tu)
+        want_norm = om.update_weights(lr, mode, opts["norm_clip"], opts["individual_clip"], B)
+        got_norm = gm.update_weights()
+        if mode == 2:
+            assert_close(got_norm, want_norm, "global gradient norm", rtol=1e-4, atol=1e-6)
+        for name in om.param_names():
+            got = gm.get_param(name, P[name].shape)
+            if modes[group(name)]:
+                assert_close(got, om.get_param(name).reshape(P[name].shape, order="F"),
+                             f"minibatch {it}: updated {name}", atol=2e-6)
+                assert not np.array_equal(got, P[name]), name
+            else:
+                assert np.array_equal(got, P[name]), f"minibatch {it}: frozen {name} moved"
+            shape = _grad_shape(P, name, su, tu)
+            assert not np.any(gm.get_grad(name, shape)), f"minibatch {it}: gradient of {name} not cleared"
+    gm.close()
+
+
 def test_gradients_with_error_clip(orc, host):
     """--clip-cell: cell values clamped forward, the errors a node hands on (to step t-1, to the LSTM
     layer below, to the attention node through feed input) clamped backward -- against the oracle's

@@ -315,3 +315,48 @@ def test_update_closed_form(orc, mode, E):
     # gradients are cleared by the update
     for k in g:
         assert not np.any(m.grad(k)), k
+
+
+@pytest.mark.parametrize("modes", [(0, 0, 0, 1, 1, 1), (1, 1, 1, 0, 1, 0), (1, 0, 1, 1, 0, 1)],
+                         ids=["finetune", "source_rnn_and_attention_frozen", "target_side_frozen"])
+def test_frozen_groups_closed_form(orc, modes):
+    """The train_*_mode__ switches of UpdateParams (src/layer_input_to_hidden.h:1154,1257,1263,
+    src/layer_hidden_to_hidden.h:765,831, src/layer_loss.h:1144): a frozen group keeps its bits,
+    every other parameter gets exactly the update it gets with nothing frozen (the global norm is
+    taken over all gradients either way, CalculateGlobalNorm has no switch), and every gradient
+    is cleared."""
+    rng = np.random.default_rng(51)
+    layers, H, Vs, Vt, D = 2, 6, 9, 10, 1
+    P, a = _model(orc, rng, layers, H, Vs, Vt, 1, 1, D, scale=0.8)
+    _, b = _model(orc, np.random.default_rng(51), layers, H, Vs, Vt, 1, 1, D, scale=0.8)
+    sents = _sentences(rng, Vs, Vt, [5, 3, 4], [4, 3, 5])
+    src, tin, tout, bi, su, tu = R.pack_minibatch(sents)
+    a.compute_gradients(src, tin, tout, bi, su, tu)
+    _, grads = b.compute_gradients(src, tin, tout, bi, su, tu)
+    B, lr = len(sents), 0.7
+    total = np.sqrt(sum(np.sum((v.astype(np.float64) / B) ** 2) for k, v in grads.items()
+                        if k not in ("src.0.W", "tgt.0.W")))
+    norm_clip = 0.5 * total
+    b.set_train_modes(*modes)
+    norm_all = a.update_weights(lr, 2, norm_clip, 0.0, B)
+    norm_frozen = b.update_weights(lr, 2, norm_clip, 0.0, B)
+    assert norm_all == norm_frozen and abs(norm_all - total) <= 1e-5 * total
+
+    def group(name):
+        if name == "src.0.W":
+            return 0
+        if name == "tgt.0.W":
+            return 1
+        return {"softmax": 2, "src": 3, "tgt": 4, "attn": 5}[name.split(".")[0]]
+
+    seen = set()
+    for name in a.param_names():
+        g = group(name)
+        seen.add(g)
+        if modes[g]:
+            assert np.array_equal(b.get_param(name), a.get_param(name)), name
+            assert not np.array_equal(b.get_param(name).reshape(P[name].shape), P[name]), name
+        else:
+            assert np.array_equal(b.get_param(name).reshape(P[name].shape), P[name]), name
+        assert not np.any(b.grad(name)), name
+    assert seen == set(range(6))
