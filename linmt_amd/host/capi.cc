@@ -275,6 +275,16 @@ extern "C" int lnmt_decode_history(lnmt_model *m, int sentence, int *tok, int *b
     if (sentence < 0 || sentence >= h.n) throw LinmtError("lnmt_decode_history: no such sentence in the last batch");
     const int k = h.slot_of_sentence[sentence], B = h.n * h.beam;
     const int n_steps = std::min(h.limit[k], cap_steps);  // expansion steps 0 .. limit-1
+    if (!h.offset.empty()) {  // DecodeStream: the sentence's rows are contiguous, back-pointers local
+      const size_t at = h.offset[sentence];
+      for (int e = 0; e < n_steps * h.beam; ++e) {
+        tok[e] = h.tok[at + e];
+        backptr[e] = h.backptr[at + e];
+        if (score) score[e] = h.score[at + e];
+      }
+      *steps = n_steps;
+      return;
+    }
     for (int t = 0; t < n_steps; ++t)
       for (int j = 0; j < h.beam; ++j) {
         tok[(size_t)t * h.beam + j] = h.tok[(size_t)t * B + (size_t)k * h.beam + j];
@@ -320,10 +330,11 @@ static int DecodeThroughFacade(bool stream, lnmt_model *const *models, int n_mod
     d.cp_beta_ = o->cp_beta;
     d.unk_replacement_mode_ = o->unk_replacement_mode != 0;
     d.hypotheses_number_ = std::max(1, o->num_hypotheses);
+    d.all_hypotheses_tokens_ = hyp_tokens != nullptr;
     std::vector<SentenceResult> res;
-    if (stream)
+    if (stream) {
       m->nmt->DecodeStream(sents, d, &res);
-    else
+      } else
       m->nmt->DecodeBatch(sents, d, &res, others);
     for (int i = 0; i < n; ++i) {
       const SentenceResult &r = res[i];

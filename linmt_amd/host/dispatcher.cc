@@ -184,6 +184,7 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
   o.cp_beta_ = c.decoding_cp_beta_;
   o.unk_replacement_mode_ = c.unk_replacement_mode_ && all_attention;
   o.hypotheses_number_ = std::max(1, c.hypotheses_number_);
+  o.all_hypotheses_tokens_ = false;  // only the kept hypotheses are written to the file
 
   const std::string ids_file =
       c.decoder_output_file_.empty() ? c.decoder_final_file_ + ".ids" : c.decoder_output_file_;

@@ -63,6 +63,10 @@ class DeviceArray {
     HipErrorWrapper(hipMalloc(reinterpret_cast<void **>(&p_), n * sizeof(T)),
                     "GPU memory allocation failed");
   }
+  // Grow-only: keeps the buffer when it already holds n elements (contents are not kept otherwise).
+  void Reserve(size_t n) {
+    if (n > n_) Alloc(n);
+  }
   void Free() {
     if (p_) (void)hipFree(p_);
     p_ = nullptr;
@@ -70,6 +74,10 @@ class DeviceArray {
   }
   void Zero(hipStream_t s) {
     if (n_) HipErrorWrapper(hipMemsetAsync(p_, 0, n_ * sizeof(T), s), "GPU memset failed");
+  }
+  void Zero(hipStream_t s, size_t n) {
+    if (n > n_) throw LinmtError("DeviceArray::Zero out of range");
+    if (n) HipErrorWrapper(hipMemsetAsync(p_, 0, n * sizeof(T), s), "GPU memset failed");
   }
   void Upload(const T *host, size_t n, hipStream_t s, size_t offset = 0) {
     if (n + offset > n_) throw LinmtError("DeviceArray::Upload out of range");
@@ -83,6 +91,35 @@ class DeviceArray {
   }
   T *get() const { return p_; }
   size_t size() const { return n_; }
+
+ private:
+  T *p_ = nullptr;
+  size_t n_ = 0;
+};
+
+// Page-locked host buffer (allocated as such: registering existing memory is not available
+// everywhere), grow-only: what asynchronous copies of a repeated call read and write.
+template <typename T>
+class PinnedArray {
+ public:
+  PinnedArray() = default;
+  PinnedArray(const PinnedArray &) = delete;
+  PinnedArray &operator=(const PinnedArray &) = delete;
+  ~PinnedArray() {
+    if (p_) (void)hipHostFree(p_);
+  }
+  void Reserve(size_t n) {
+    if (n <= n_) return;
+    if (p_) (void)hipHostFree(p_);
+    p_ = nullptr;
+    n_ = 0;
+    HipErrorWrapper(hipHostMalloc(reinterpret_cast<void **>(&p_), n * sizeof(T), hipHostMallocDefault),
+                    "page-locked host memory allocation failed");
+    n_ = n;
+  }
+  T *get() const { return p_; }
+  size_t size() const { return n_; }
+  T &operator[](size_t i) const { return p_[i]; }
 
  private:
   T *p_ = nullptr;

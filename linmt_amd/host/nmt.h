@@ -14,6 +14,7 @@
 //     sentence s owns columns [s*beam,(s+1)*beam); beam selection, back-pointers and the state swap
 //     stay on the device, the host only reads the per-step (token, back-pointer, score) history.
 #pragma once
+#include <functional>
 #include <map>
 #include <memory>
 #include <string>
@@ -437,6 +438,10 @@ struct DecodeOptions {
   // the reference's hypotheses_number_ (global_configuration.h:229): how many of the finished
   // hypotheses OutputKBestHypotheses keeps, best first
   int hypotheses_number_ = 1;
+  // DecodeStream: write out the tokens of every finished hypothesis (SentenceResult::hypotheses),
+  // not only of the ones OutputKBestHypotheses keeps.  A caller that reads only the kept ones
+  // switches it off: a list of a thousand sentences has a few hundred thousand finished hypotheses.
+  bool all_hypotheses_tokens_ = true;
 };
 
 struct SentenceResult {
@@ -473,8 +478,12 @@ class Decoder {
   DeviceArray<int> index_hist_;
   void Init(int beam_size, int n_sent, int max_steps);
   // OutputKBestHypotheses (decoder.h:529-699) for one sentence: the selection, not the printing.
+  // sizes (optional): token counts of hypotheses whose tokens have not been written out yet;
+  // materialise(i) is then called for every hypothesis that is kept, before its tokens are read.
   static void OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_length,
-                                    const DecodeOptions &o, SentenceResult *out);
+                                    const DecodeOptions &o, SentenceResult *out,
+                                    const std::vector<int> *sizes = nullptr,
+                                    const std::function<void(int)> &materialise = nullptr);
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -540,7 +549,19 @@ class NeuralMachineTranslation {
     int n = 0, beam = 0, steps = 0;
     std::vector<int> slot_of_sentence, limit, tok, backptr;
     std::vector<float> score;  // path score of beam entry (step, column)
+    // DecodeBatch: entry (step, sentence k, j) at step * n * beam + slot_of_sentence[k] * beam + j,
+    // back-pointers as batch columns.  DecodeStream (offset not empty): sentence i's rows are
+    // contiguous, entry (step, j) at offset[i] + step * beam + j, back-pointers beam-local.
+    std::vector<size_t> offset;
   } last_history_;
+  // What DecodeStream keeps between calls (device buffers and page-locked host buffers that only
+  // grow): a call allocates nothing once a longer list has been decoded.
+  struct StreamState {
+    DeviceArray<int> tok_hist, bp_hist, fcount_hist, fbeam_hist, start_dev, limit_dev, mask_table;
+    DeviceArray<float> score_hist, fscore_hist, finals;
+    PinnedArray<int> tok, bp, fcount, fbeam, mask_host;
+    PinnedArray<float> fscore, bscore;
+  } stream_state_;
   DeviceArray<float> p_device_h_tild_previous_;  // decode: gathered h~ of the previous step
   DeviceArray<float> p_device_ensemble_dist_;    // decode in an ensemble: this model's probabilities
   std::vector<hipEvent_t> ensemble_events_;      // owned by the model that runs the beam search

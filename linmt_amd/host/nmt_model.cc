@@ -651,7 +651,9 @@ void Decoder::Init(int beam_size, int n_sent, int max_steps) {
 // from (decoder.h:364-370); with it on the rows are the exported scores, smoothed and normalised in
 // place as the reference does (so a later print shows the normalised values).
 void Decoder::OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_length,
-                                    const DecodeOptions &o, SentenceResult *out) {
+                                    const DecodeOptions &o, SentenceResult *out,
+                                    const std::vector<int> *sizes,
+                                    const std::function<void(int)> &materialise) {
   // the kept set, worst first: a hypothesis enters while there is room, afterwards only by beating
   // the worst kept one strictly (decoder.h:589-600; which of two exactly equal scores the
   // reference's heap drops first is not defined by its source)
@@ -662,7 +664,7 @@ void Decoder::OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_le
   };
   for (size_t i = 0; i < hyps.size(); ++i) {
     float s = hyps[i].score;
-    const int size = (int)hyps[i].tokens.size();
+    const int size = sizes ? (*sizes)[i] : (int)hyps[i].tokens.size();
     if (0 != o.lp_alpha_) {
       const float lp = powf((float)(5 + size), o.lp_alpha_) / powf((float)(5 + 1), o.lp_alpha_);
       s /= lp;
@@ -716,6 +718,7 @@ void Decoder::OutputKBestHypotheses(std::vector<Hypothesis> &hyps, int source_le
   for (const auto &k : kept) {
     out->kbest.push_back(k.second);
     out->kbest_score.push_back(k.first);
+    if (materialise) materialise(k.second);
   }
   const int best = kept.empty() ? -1 : kept[0].second;
   const float best_score = kept.empty() ? 0.f : kept[0].first;
@@ -1112,6 +1115,7 @@ void NeuralMachineTranslation::DecodeBatch(const std::vector<std::vector<int>> &
           std::vector<std::vector<float>>().swap(r.hypotheses[h].alignments_scores);
   }
   // the streams have been synchronised: the histories are complete and no copy is in flight
+  last_history_.offset.clear();
   last_history_.n = n;
   last_history_.beam = beam;
   last_history_.steps = (int)steps;

@@ -14,8 +14,11 @@
 // W_c1*hs and the encoder's final states -- is kept in one of kRing slabs until the group's last
 // sentence has finished.
 #include <algorithm>
+#include <atomic>
 #include <cmath>
+#include <exception>
 #include <numeric>
+#include <thread>
 
 #include "nmt.h"
 
@@ -99,27 +102,32 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   // ---- device state of the stream ------------------------------------------------------------------
   // rows of the histories: row t+1 is written by tick t, row t holds what tick t reads (tokens
   // chosen and path scores of the tick before; a fresh slot's entries are set by its admission)
-  DeviceArray<int> tok_hist, bp_hist, fcount_hist, fbeam_hist, start_dev, limit_dev, mask_table;
-  DeviceArray<float> score_hist, fscore_hist, finals;
+  StreamState &ss = stream_state_;
+  DeviceArray<int> &tok_hist = ss.tok_hist, &bp_hist = ss.bp_hist, &fcount_hist = ss.fcount_hist,
+                   &fbeam_hist = ss.fbeam_hist, &start_dev = ss.start_dev, &limit_dev = ss.limit_dev,
+                   &mask_table = ss.mask_table;
+  DeviceArray<float> &score_hist = ss.score_hist, &fscore_hist = ss.fscore_hist, &finals = ss.finals;
   const size_t rows = (size_t)ticks + 1;
-  tok_hist.Alloc(rows * B), bp_hist.Alloc(rows * B), score_hist.Alloc(rows * B);
-  fcount_hist.Alloc((size_t)ticks * slots), fbeam_hist.Alloc((size_t)ticks * B), fscore_hist.Alloc((size_t)ticks * B);
-  start_dev.Alloc(slots), limit_dev.Alloc(slots);
+  tok_hist.Reserve(rows * B), bp_hist.Reserve(rows * B), score_hist.Reserve(rows * B);
+  fcount_hist.Reserve((size_t)ticks * slots), fbeam_hist.Reserve((size_t)ticks * B), fscore_hist.Reserve((size_t)ticks * B);
+  start_dev.Reserve(slots), limit_dev.Reserve(slots);
   const size_t final_slab = (size_t)2 * L * H * slots;  // [layer][h, c][H x n_sent]
-  finals.Alloc(final_slab * kRing);
+  finals.Reserve(final_slab * kRing);
   // what the first target layer reads as its column mask: 1, and for a feed-input model
   // 1 + LH_MASK_F32_GATES on a sentence's first step (the reference runs that step through the
   // kernels without the feed terms, node_input_to_hidden.h:325-621)
-  std::vector<int> mask_host((size_t)ticks * B, 1), minus_one(slots, -1), zeros(slots, 0);
+  ss.mask_host.Reserve((size_t)ticks * B);
+  int *mask_host = ss.mask_host.get();
+  std::fill(mask_host, mask_host + (size_t)ticks * B, 1);
+  std::vector<int> minus_one(slots, -1), zeros(slots, 0);
   if (cfg_.feed_input_mode_)
     for (const Admission &a : adm)
       for (int j = 0; j < beam; ++j) mask_host[(size_t)a.tick * B + (size_t)a.slot * beam + j] = 1 + LH_MASK_F32_GATES;
-  mask_table.Alloc(mask_host.size());
+  mask_table.Reserve((size_t)ticks * B);
   // host arrays that asynchronous copies read or write: declared before the guard, so however this
   // function is left the stream has drained before any of them is destroyed
   std::vector<std::vector<int>> src_blocks(G);  // the encoder's id block of every group
-  std::vector<int> tok, bp, fcount, fbeam, binfo0(2 * (size_t)B, 0);
-  std::vector<float> fscore, bscore;
+  std::vector<int> binfo0(2 * (size_t)B, 0);
   std::fill(binfo0.begin(), binfo0.begin() + B, 1);  // length 1, offset 0: a column without a sentence
   struct Restore {
     NeuralMachineTranslation &m;
@@ -133,11 +141,11 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
       m.stream_layer0_mask_ = nullptr;
     }
   } restore{*this, B};
-  mask_table.Upload(mask_host.data(), mask_host.size(), stream_);
+  mask_table.Upload(mask_host, (size_t)ticks * B, stream_);
   start_dev.Upload(zeros.data(), slots, stream_);
   limit_dev.Upload(minus_one.data(), slots, stream_);
-  tok_hist.Zero(stream_);  // a slot that never held a sentence feeds <START> = 0
-  score_hist.Zero(stream_);
+  tok_hist.Zero(stream_, rows * B);  // a slot that never held a sentence feeds <START> = 0
+  score_hist.Zero(stream_, rows * B);
 
   // the attention memories of kRing groups side by side: slab r starts T_cap * n_sent columns
   // after slab 0, which an entry of hs_col can express
@@ -293,25 +301,42 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   }
 
   // ---- one read-back -----------------------------------------------------------------------------------
-  tok.resize(rows * B), bp.resize(rows * B), bscore.resize(rows * B);
-  fcount.resize((size_t)ticks * slots), fbeam.resize((size_t)ticks * B), fscore.resize((size_t)ticks * B);
-  tok_hist.Download(tok.data(), tok.size(), stream_);
-  bp_hist.Download(bp.data(), bp.size(), stream_);
-  score_hist.Download(bscore.data(), bscore.size(), stream_);
-  fcount_hist.Download(fcount.data(), fcount.size(), stream_);
-  fbeam_hist.Download(fbeam.data(), fbeam.size(), stream_);
-  fscore_hist.Download(fscore.data(), fscore.size(), stream_);
+  ss.tok.Reserve(rows * B), ss.bp.Reserve(rows * B), ss.bscore.Reserve(rows * B);
+  ss.fcount.Reserve((size_t)ticks * slots), ss.fbeam.Reserve((size_t)ticks * B), ss.fscore.Reserve((size_t)ticks * B);
+  const int *tok = ss.tok.get(), *bp = ss.bp.get(), *fcount = ss.fcount.get(), *fbeam = ss.fbeam.get();
+  const float *fscore = ss.fscore.get(), *bscore = ss.bscore.get();
+  tok_hist.Download(ss.tok.get(), rows * B, stream_);
+  bp_hist.Download(ss.bp.get(), rows * B, stream_);
+  score_hist.Download(ss.bscore.get(), rows * B, stream_);
+  fcount_hist.Download(ss.fcount.get(), (size_t)ticks * slots, stream_);
+  fbeam_hist.Download(ss.fbeam.get(), (size_t)ticks * B, stream_);
+  fscore_hist.Download(ss.fscore.get(), (size_t)ticks * B, stream_);
   Synchronize();
   profiler_.Collect();
 
-  // ---- hypotheses by walking the back-pointers, as DecodeBatch does ---------------------------------
+  // ---- hypotheses by walking the back-pointers, as DecodeBatch does; the search of every sentence
+  // in the compact layout lnmt_decode_history reads.  Sentences are independent: a few host threads
+  // share them (a list of a thousand sentences is tens of milliseconds of this on one thread).
   results->assign(n, SentenceResult());
+  DecodeHistory &hist = last_history_;
+  hist.n = n, hist.beam = beam;
+  hist.slot_of_sentence.resize(n);
+  std::iota(hist.slot_of_sentence.begin(), hist.slot_of_sentence.end(), 0);
+  hist.limit = limit;
+  hist.offset.assign(n, 0);
+  size_t hist_rows = 0;
   int max_limit = 0;
   for (int i = 0; i < n; ++i) {
+    hist.offset[i] = hist_rows * beam;
+    hist_rows += (size_t)limit[i] + 1;
+    max_limit = std::max(max_limit, limit[i]);
+  }
+  hist.steps = max_limit + 1;
+  hist.tok.resize(hist_rows * beam), hist.backptr.resize(hist_rows * beam), hist.score.resize(hist_rows * beam);
+  auto build = [&](int i) {
     SentenceResult &r = (*results)[i];
     const int t0 = start_of[i], c0 = slot_of[i] * beam, s = slot_of[i];
     r.steps = limit[i] + 1;
-    max_limit = std::max(max_limit, limit[i]);
     auto prefix = [&](int step, int column, Hypothesis *h) {
       h->tokens.assign(step + 1, Decoder::start_symbol_);
       int col = column;
@@ -320,47 +345,65 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
         col = bp[(size_t)(t0 + q + 1) * B + col];
       }
     };
+    // the finished hypotheses in the order the reference's v_hypotheses_ holds them: where each
+    // one ended, its score and its length; the tokens are written out for all of them or, when the
+    // caller only reads the kept ones, for those
+    std::vector<int> at_step, parent_of, sizes;
     for (int step = 0; step <= limit[i]; ++step) {
       const int nf = fcount[(size_t)(t0 + step) * slots + s];
       for (int f = 0; f < nf; ++f) {
-        Hypothesis h;
-        const int parent = c0 + fbeam[(size_t)(t0 + step) * B + c0 + f];
-        prefix(step, parent, &h);
-        h.tokens.push_back(Decoder::end_symbol_);
-        h.score = fscore[(size_t)(t0 + step) * B + c0 + f];
-        r.hypotheses.push_back(std::move(h));
+        at_step.push_back(step);
+        parent_of.push_back(c0 + fbeam[(size_t)(t0 + step) * B + c0 + f]);
+        sizes.push_back(step + 2);  // <START>, `step` words, <EOF>
       }
     }
-    Decoder::OutputKBestHypotheses(r.hypotheses, (int)sentences[i].size(), o, &r);
-  }
-  // the search of every sentence in the layout lnmt_decode_history reads: [step][sentence * beam + j]
-  DecodeHistory &hist = last_history_;
-  hist.n = n, hist.beam = beam, hist.steps = max_limit + 1;
-  hist.slot_of_sentence.resize(n);
-  std::iota(hist.slot_of_sentence.begin(), hist.slot_of_sentence.end(), 0);
-  hist.limit = limit;
-  const size_t Bn = (size_t)n * beam;
-  hist.tok.assign((size_t)hist.steps * Bn, Decoder::end_symbol_);
-  hist.backptr.assign((size_t)hist.steps * Bn, 0);
-  hist.score.assign((size_t)hist.steps * Bn, 0.f);
-  for (int i = 0; i < n; ++i) {
-    const int t0 = start_of[i], c0 = slot_of[i] * beam;
+    r.hypotheses.resize(at_step.size());
+    auto write_out = [&](int k) {
+      Hypothesis &h = r.hypotheses[k];
+      if (!h.tokens.empty()) return;
+      prefix(at_step[k], parent_of[k], &h);
+      h.tokens.push_back(Decoder::end_symbol_);
+    };
+    for (size_t k = 0, f = 0; k < at_step.size(); ++k) {
+      f = k > 0 && at_step[k] == at_step[k - 1] ? f + 1 : 0;
+      r.hypotheses[k].score = fscore[(size_t)(t0 + at_step[k]) * B + c0 + f];
+      if (o.all_hypotheses_tokens_) write_out((int)k);
+    }
+    Decoder::OutputKBestHypotheses(r.hypotheses, (int)sentences[i].size(), o, &r, &sizes, write_out);
     for (int step = 0; step <= limit[i]; ++step)
       for (int j = 0; j < beam; ++j) {
-        const size_t from = (size_t)(t0 + step + 1) * B + c0 + j, to = (size_t)step * Bn + (size_t)i * beam + j;
+        const size_t from = (size_t)(t0 + step + 1) * B + c0 + j, to = hist.offset[i] + (size_t)step * beam + j;
         if (step == limit[i]) {
           // the row a sentence's last step writes is the row the slot's next sentence is admitted
           // into: what the step stored there (<EOF>, the column itself, the final score) is taken
           // from the finished-hypothesis record of the same step instead
           hist.tok[to] = Decoder::end_symbol_;
-          hist.backptr[to] = i * beam + j;
+          hist.backptr[to] = j;
           hist.score[to] = fscore[(size_t)(t0 + step) * B + c0 + j];
           continue;
         }
         hist.tok[to] = tok[from];
-        hist.backptr[to] = bp[from] - c0 + i * beam;
+        hist.backptr[to] = bp[from] - c0;
         hist.score[to] = bscore[from];
       }
+  };
+  {
+    const int workers = std::max(1, std::min({8, n / 32, (int)std::thread::hardware_concurrency()}));
+    std::atomic<int> next{0};
+    std::vector<std::exception_ptr> failed(workers);
+    auto run = [&](int w) {
+      try {
+        for (int i = next.fetch_add(1); i < n; i = next.fetch_add(1)) build(i);
+      } catch (...) {
+        failed[w] = std::current_exception();
+      }
+    };
+    std::vector<std::thread> pool;
+    for (int w = 1; w < workers; ++w) pool.emplace_back(run, w);
+    run(0);
+    for (std::thread &t : pool) t.join();
+    for (const std::exception_ptr &e : failed)
+      if (e) std::rethrow_exception(e);
   }
   stream_ticks_ = ticks;
 }
