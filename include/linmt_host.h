@@ -170,13 +170,17 @@ int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_models, const in
  * src/decoder.h:1702-1776): the model's n_sent groups of beam columns are slots; a sentence that has
  * taken its last step hands its slot to the next sentence of the list, so every step runs
  * n_sent * beam_size hypotheses until the list runs out.  Every sentence goes through the steps
- * lnmt_decode_batch takes it through and gives the same kind of result.  One model with local-p
- * attention, no alignment export.  *ticks (may be NULL) receives the number of steps taken in all.
- * lnmt_decode_history afterwards addresses the sentences by their position in the list. */
+ * lnmt_decode_batch takes it through and gives the same kind of result, exported alignments
+ * (o->unk_replacement_mode, best_viterbi) and k-best lists (o->num_hypotheses, kbest_index,
+ * kbest_score) included.  One model with local-p attention.  The tokens of all finished hypotheses
+ * are written out only when hyp_tokens is given.  *ticks (may be NULL) receives the number of
+ * steps taken in all.  lnmt_decode_history afterwards addresses the sentences by their position in
+ * the list. */
 int lnmt_decode_stream(lnmt_model *m, const int *sentences, const int *lengths, int n,
                        const lnmt_decode_options *o, int *best, int cap, int *best_len,
                        float *best_score, int *steps, int *hyp_tokens, int *hyp_len, float *hyp_score,
-                       int hyp_cap, int *n_hyp, int *ticks);
+                       int hyp_cap, int *n_hyp, int *best_viterbi, int *kbest_index,
+                       float *kbest_score, int *ticks);
 
 /* The model's HIP stream (hipStream_t as void*), for callers that time with HIP events. */
 void *lnmt_model_stream(lnmt_model *m);

@@ -115,7 +115,8 @@ def load():
     lib.lnmt_decode_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
                                        C.POINTER(DecodeOptions), C.c_void_p, C.c_int, C.c_void_p,
                                        C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
-                                       C.c_int, C.c_void_p, C.POINTER(C.c_int)]
+                                       C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.POINTER(C.c_int)]
     lib.lnmt_model_stream.restype = C.c_void_p
     lib.lnmt_model_stream.argtypes = [C.c_void_p]
     lib.lnmt_set_split_products.argtypes = [C.c_void_p, C.c_int, C.c_int]
@@ -436,7 +437,8 @@ class Model:
 
 
 def _decode_stream(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0, diversity=0.0,
-                   lp_alpha=0.65, cp_beta=0.20, with_hyps=False, hyp_cap=256):
+                   lp_alpha=0.65, cp_beta=0.20, with_hyps=False, hyp_cap=256, alignments=False,
+                   num_hypotheses=1):
     """DecodeStream: any number of sentences through the model's n_sent slots of beam columns, a
     finished sentence's slot going to the next sentence.  Results as decode_batch, in the order of
     `sentences`; self.stream_ticks = steps taken in all."""
@@ -444,8 +446,12 @@ def _decode_stream(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penal
     lengths = np.array([len(s) for s in sentences], np.int32)
     flat = np.ascontiguousarray(np.concatenate([np.asarray(s, np.int32) for s in sentences]))
     cap = self.cfg.longest_sentence + 2
-    o = DecodeOptions(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta, 0, 1)
+    o = DecodeOptions(beam, max_ratio, min_ratio, penalty, diversity, lp_alpha, cp_beta,
+                      int(alignments), int(num_hypotheses))
+    kidx = np.full((n, max(1, num_hypotheses)), -1, np.int32)
+    kscore = np.zeros((n, max(1, num_hypotheses)), np.float32)
     best = np.zeros((n, cap), np.int32)
+    vit = np.full((n, cap), -1, np.int32) if alignments else None
     blen = np.zeros(n, np.int32)
     bscore = np.zeros(n, np.float32)
     steps = np.zeros(n, np.int32)
@@ -458,7 +464,8 @@ def _decode_stream(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penal
     ticks = C.c_int(0)
     _check(load().lnmt_decode_stream(self.handle, _p(flat), _p(lengths), n, C.byref(o), _p(best), cap,
                                      _p(blen), _p(bscore), _p(steps), _p(ht), _p(hl), _p(hs), hyp_cap,
-                                     _p(nh), C.byref(ticks)), "decode_stream")
+                                     _p(nh), _p(vit), _p(kidx), _p(kscore), C.byref(ticks)),
+           "decode_stream")
     self.stream_ticks = ticks.value
     res = []
     for i in range(n):
@@ -467,6 +474,9 @@ def _decode_stream(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penal
         if with_hyps:
             k = min(int(nh[i]), hyp_cap)
             r["hyps"] = [(ht[i, j, :hl[i, j]].copy(), float(hs[i, j])) for j in range(k)]
+        if alignments:
+            r["best_viterbi"] = vit[i, :blen[i]].copy()
+        r["kbest"] = [(int(a), float(b)) for a, b in zip(kidx[i], kscore[i]) if a >= 0]
         res.append(r)
     return res
 

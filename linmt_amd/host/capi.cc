@@ -382,10 +382,11 @@ extern "C" int lnmt_decode_batch_ensemble(lnmt_model *const *models, int n_model
 extern "C" int lnmt_decode_stream(lnmt_model *m, const int *sentences, const int *lengths, int n,
                                   const lnmt_decode_options *o, int *best, int cap, int *best_len,
                                   float *best_score, int *steps, int *hyp_tokens, int *hyp_len,
-                                  float *hyp_score, int hyp_cap, int *n_hyp, int *ticks) {
+                                  float *hyp_score, int hyp_cap, int *n_hyp, int *best_viterbi,
+                                  int *kbest_index, float *kbest_score, int *ticks) {
   const int rc = DecodeThroughFacade(true, &m, m ? 1 : 0, sentences, lengths, n, o, best, cap, best_len, best_score,
-                                     steps, hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, nullptr,
-                                     nullptr, nullptr);
+                                     steps, hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, best_viterbi,
+                                     kbest_index, kbest_score);
   if (rc == 0 && ticks) *ticks = m->nmt->stream_ticks_;
   return rc;
 }

@@ -192,10 +192,10 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
     std::ofstream output(ids_file.c_str());
     if (!output) throw LinmtError("Decoding: cannot open " + ids_file);
     const auto begin = std::chrono::steady_clock::now();
-    // One model without exported alignments over local-p attention: the sentences go through
+    // One model over local-p attention: the sentences go through
     // DecodeStream, a few thousand at a time, with every beam column kept busy; everything else
     // is decoded batch by batch.  (Debug().no_stream: measurement and test aid.)
-    const bool stream = ensemble.empty() && !o.unk_replacement_mode_ && neural.cfg_.attention_mode_ &&
+    const bool stream = ensemble.empty() && neural.cfg_.attention_mode_ &&
                         neural.attention_layer_.ProjectedMemoryPossible() && !Debug().no_stream;
     const size_t chunk = stream ? (size_t)n_sent * 32 : (size_t)n_sent;
     for (size_t first = 0; stream && first < sentences.size(); first += chunk) {

@@ -558,7 +558,8 @@ class NeuralMachineTranslation {
   // grow): a call allocates nothing once a longer list has been decoded.
   struct StreamState {
     DeviceArray<int> tok_hist, bp_hist, fcount_hist, fbeam_hist, start_dev, limit_dev, mask_table;
-    DeviceArray<float> score_hist, fscore_hist, finals;
+    DeviceArray<float> score_hist, fscore_hist, finals, align_hist;
+    DeviceArray<int> index_hist;
     PinnedArray<int> tok, bp, fcount, fbeam, mask_host;
     PinnedArray<float> fscore, bscore;
   } stream_state_;
@@ -605,8 +606,9 @@ class NeuralMachineTranslation {
                    const std::vector<std::vector<std::vector<int>>> &ensemble_sentences = {});
   // The same search over any number of sentences with every beam column kept busy: a sentence
   // that has taken its last step hands its beam columns to the next sentence of the list, so the
-  // sentences in flight are at different steps (nmt_stream.cc).  One model, local-p attention,
-  // no alignment export.  Every sentence goes through the steps DecodeBatch takes it through.
+  // sentences in flight are at different steps (nmt_stream.cc).  One model, local-p attention;
+  // alignment export and k-best lists as in DecodeBatch.  Every sentence goes through the steps
+  // DecodeBatch takes it through.
   void DecodeStream(const std::vector<std::vector<int>> &sentences, const DecodeOptions &o,
                     std::vector<SentenceResult> *results);
   const int *stream_layer0_mask_ = nullptr;  // DecodeStream: the first target layer's column mask of this tick

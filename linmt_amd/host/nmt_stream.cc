@@ -38,7 +38,6 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   if (!decode_mode_) throw LinmtError("DecodeStream: call InitModelDecoding first");
   if (!cfg_.attention_mode_ || !attention_layer_.ProjectedMemoryPossible())
     throw LinmtError("DecodeStream: needs local-p attention over a projected memory");
-  if (o.unk_replacement_mode_) throw LinmtError("DecodeStream: alignment export is not supported");
   const int n = (int)sentences.size(), L = cfg_.num_layers_, H = cfg_.lstm_size_;
   int beam = o.beam_size_;
   if (beam > (int)std::sqrt((double)cfg_.target_vocab_size_))  // decoder.h:1662-1664
@@ -124,15 +123,29 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
     for (const Admission &a : adm)
       for (int j = 0; j < beam; ++j) mask_host[(size_t)a.tick * B + (size_t)a.slot * beam + j] = 1 + LH_MASK_F32_GATES;
   mask_table.Reserve((size_t)ticks * B);
+  // unk_replacement_mode_: the attention core writes every tick's alignments and window indices
+  // into its own slice of a history ([tick][column + B * slot]) instead of the one reused buffer
+  const bool capture = o.unk_replacement_mode_;
+  const int W = attention_layer_.window_;
+  const size_t align_slice = (size_t)B * W;
+  if (capture) {
+    ss.align_hist.Reserve(align_slice * ticks);
+    ss.index_hist.Reserve(align_slice * ticks);
+  }
   // host arrays that asynchronous copies read or write: declared before the guard, so however this
   // function is left the stream has drained before any of them is destroyed
   std::vector<std::vector<int>> src_blocks(G);  // the encoder's id block of every group
   std::vector<int> binfo0(2 * (size_t)B, 0);
   std::fill(binfo0.begin(), binfo0.begin() + B, 1);  // length 1, offset 0: a column without a sentence
+  AttentionNode &attention_node = attention_layer_.v_nodes_[0];
   struct Restore {
     NeuralMachineTranslation &m;
     int B;
+    float *node_alignments;
+    int *node_indices;
     ~Restore() {
+      m.attention_layer_.v_nodes_[0].p_device_alignments_ = node_alignments;
+      m.attention_layer_.v_nodes_[0].p_device_indices_ = node_indices;
       if (m.encoder_stream_) (void)hipStreamSynchronize(m.encoder_stream_);
       // DecodeBatch reads the encoder states of column b's sentence through hs_col[b] = b / beam
       (void)hipMemcpyAsync(m.attention_layer_.p_device_hs_col_.get(), m.p_device_sentence_of_column_.get(),
@@ -140,7 +153,7 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
       (void)hipStreamSynchronize(m.stream_);
       m.stream_layer0_mask_ = nullptr;
     }
-  } restore{*this, B};
+  } restore{*this, B, attention_node.p_device_alignments_, attention_node.p_device_indices_};
   mask_table.Upload(mask_host, (size_t)ticks * B, stream_);
   start_dev.Upload(zeros.data(), slots, stream_);
   limit_dev.Upload(minus_one.data(), slots, stream_);
@@ -276,6 +289,10 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
     }
     // ---- one step of every slot ------------------------------------------------------------------------
     stream_layer0_mask_ = mask_table.get() + (size_t)t * B;
+    if (capture) {
+      attention_node.p_device_alignments_ = ss.align_hist.get() + align_slice * t;
+      attention_node.p_device_indices_ = ss.index_hist.get() + align_slice * t;
+    }
     ForwardPropTarget(1, tok_hist.get() + (size_t)t * B, B);
     stream_layer0_mask_ = nullptr;
     {
@@ -311,6 +328,13 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   fcount_hist.Download(ss.fcount.get(), (size_t)ticks * slots, stream_);
   fbeam_hist.Download(ss.fbeam.get(), (size_t)ticks * B, stream_);
   fscore_hist.Download(ss.fscore.get(), (size_t)ticks * B, stream_);
+  std::vector<float> ahist;
+  std::vector<int> ihist;
+  if (capture) {
+    ahist.resize(align_slice * ticks), ihist.resize(align_slice * ticks);
+    ss.align_hist.Download(ahist.data(), ahist.size(), stream_);
+    ss.index_hist.Download(ihist.data(), ihist.size(), stream_);
+  }
   Synchronize();
   profiler_.Collect();
 
@@ -337,12 +361,37 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
     SentenceResult &r = (*results)[i];
     const int t0 = start_of[i], c0 = slot_of[i] * beam, s = slot_of[i];
     r.steps = limit[i] + 1;
+    const int source_length = (int)sentences[i].size();
+    // alignment scores over the source positions of `column` at the sentence's step q, and their
+    // arg-max as EnsemblesModels takes it (decoder.h:1946-1961): first strictly largest score above 0
+    auto alignment_row = [&](int q, int column, std::vector<float> *scores, int *viterbi) {
+      scores->assign(source_length, 0.f);
+      for (int j = 0; j < W; ++j) {
+        const size_t at = align_slice * (size_t)(t0 + q) + column + (size_t)B * j;
+        const int idx = ihist[at];
+        if (idx >= 0 && idx < source_length) (*scores)[idx] += ahist[at];
+      }
+      float max_val = 0;
+      *viterbi = -1;
+      for (int j = 0; j < source_length; ++j)
+        if ((*scores)[j] > max_val) {
+          max_val = (*scores)[j];
+          *viterbi = j;
+        }
+    };
     auto prefix = [&](int step, int column, Hypothesis *h) {
+      // token q+1 was produced by the forward pass of its PARENT column at step q, whose
+      // alignments it carries (decoder.h:452-456)
       h->tokens.assign(step + 1, Decoder::start_symbol_);
+      if (capture) {
+        h->viterbi.assign(step + 2, -20);
+        h->alignments_scores.assign(step + 2, std::vector<float>());
+      }
       int col = column;
       for (int q = step - 1; q >= 0; --q) {
         h->tokens[q + 1] = tok[(size_t)(t0 + q + 1) * B + col];
         col = bp[(size_t)(t0 + q + 1) * B + col];
+        if (capture) alignment_row(q, col, &h->alignments_scores[q + 1], &h->viterbi[q + 1]);
       }
     };
     // the finished hypotheses in the order the reference's v_hypotheses_ holds them: where each
@@ -363,13 +412,20 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
       if (!h.tokens.empty()) return;
       prefix(at_step[k], parent_of[k], &h);
       h.tokens.push_back(Decoder::end_symbol_);
+      if (capture)  // <EOF> itself comes out of the parent's forward pass at this step
+        alignment_row(at_step[k], parent_of[k], &h.alignments_scores[at_step[k] + 1], &h.viterbi[at_step[k] + 1]);
     };
     for (size_t k = 0, f = 0; k < at_step.size(); ++k) {
       f = k > 0 && at_step[k] == at_step[k - 1] ? f + 1 : 0;
       r.hypotheses[k].score = fscore[(size_t)(t0 + at_step[k]) * B + c0 + f];
-      if (o.all_hypotheses_tokens_) write_out((int)k);
+      // the coverage penalty reads every hypothesis' exported alignments
+      if (o.all_hypotheses_tokens_ || capture) write_out((int)k);
     }
-    Decoder::OutputKBestHypotheses(r.hypotheses, (int)sentences[i].size(), o, &r, &sizes, write_out);
+    Decoder::OutputKBestHypotheses(r.hypotheses, source_length, o, &r, &sizes, write_out);
+    if (capture)  // only the hypotheses kept hold on to their score rows (what a printout shows)
+      for (size_t h = 0; h < r.hypotheses.size(); ++h)
+        if (std::find(r.kbest.begin(), r.kbest.end(), (int)h) == r.kbest.end())
+          std::vector<std::vector<float>>().swap(r.hypotheses[h].alignments_scores);
     for (int step = 0; step <= limit[i]; ++step)
       for (int j = 0; j < beam; ++j) {
         const size_t from = (size_t)(t0 + step + 1) * B + c0 + j, to = hist.offset[i] + (size_t)step * beam + j;

@@ -238,3 +238,36 @@ def test_decode_stream_at_the_longest_sentence_length(orc, host, feed):
         assert want["steps"] == (19 if len(s) >= 13 else 2)
         _compare_decode(want, got[i], f"sentence {i} (len {len(s)})")
     gm.close()
+
+
+@pytest.mark.parametrize("layers,H,Vs,Vt,D,beam,slots,n,feed,seed", [
+    (2, 64, 120, 150, 3, 4, 3, 11, True, 21),
+    (1, 48, 60, 90, 10, 5, 2, 7, False, 22),
+])
+def test_decode_stream_exported_alignments_and_kbest_vs_oracle(orc, host, layers, H, Vs, Vt, D, beam, slots,
+                                                                n, feed, seed):
+    """The reference's unk_replacement_mode__ through the stream: every tick's alignments and window
+    indices go into a history, hypotheses carry the Viterbi alignment of every token and the
+    coverage penalty is computed from the exported scores (src/decoder.h:529-600,1933-1961,
+    src/layer_attention.h:342-386).  1-best, its alignments and its rescored value must be the
+    oracle's; a k-best list must be DecodeBatch's for the same sentences."""
+    rng = np.random.default_rng(seed)
+    P, om, gm = _pair(orc, host, rng, layers, H, Vs, Vt, D, 40, 0.4, decoding=(slots, beam), feed=feed)
+    sents = [rng.integers(0, Vs, size=int(rng.integers(1, 16))) for _ in range(n)]
+    got = gm.decode_stream(sents, beam=beam, with_hyps=True, alignments=True)
+    for i, s in enumerate(sents):
+        want = om.decode_sentence(s, beam=beam, alignments=True)
+        _compare_decode(want, got[i], f"sentence {i} (len {len(s)})")
+        assert got[i]["best_viterbi"].tolist() == want["best_viterbi"].tolist(), i
+    # k-best lists: the same indices and scores as batch by batch, with and without alignments
+    for align in (False, True):
+        ks = gm.decode_stream(sents, beam=beam, alignments=align, num_hypotheses=3)
+        order = sorted(range(n), key=lambda i: -len(sents[i]))
+        for g0 in range(0, n, slots):
+            group = order[g0:g0 + slots]
+            kb = gm.decode_batch([sents[i] for i in group], beam=beam, alignments=align, num_hypotheses=3)
+            for w, i in zip(kb, group):
+                assert [k for k, _ in ks[i]["kbest"]] == [k for k, _ in w["kbest"]], (align, i)
+                assert np.allclose([v for _, v in ks[i]["kbest"]], [v for _, v in w["kbest"]], rtol=1e-4, atol=1e-4)
+                assert ks[i]["best"].tolist() == w["best"].tolist(), (align, i)
+    gm.close()
