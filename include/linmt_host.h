@@ -182,6 +182,17 @@ int lnmt_decode_stream(lnmt_model *m, const int *sentences, const int *lengths, 
                        int hyp_cap, int *n_hyp, int *best_viterbi, int *kbest_index,
                        float *kbest_score, int *ticks);
 
+/* lnmt_decode_stream for an ensemble: the models decode in lockstep, models[0] runs the schedule
+ * and the beam search on the mean of their distributions (EnsembleFactory::EnsemblesModels,
+ * src/decoder.h:1910-1931), as lnmt_decode_batch_ensemble does batch by batch.  Every model needs
+ * local-p attention and the same n_sent, beam, target vocabulary and longest sentence. */
+int lnmt_decode_stream_ensemble(lnmt_model *const *models, int n_models, const int *sentences,
+                                const int *lengths, int n, const lnmt_decode_options *o, int *best,
+                                int cap, int *best_len, float *best_score, int *steps,
+                                int *hyp_tokens, int *hyp_len, float *hyp_score, int hyp_cap,
+                                int *n_hyp, int *best_viterbi, int *kbest_index, float *kbest_score,
+                                int *ticks);
+
 /* The model's HIP stream (hipStream_t as void*), for callers that time with HIP events. */
 void *lnmt_model_stream(lnmt_model *m);
 

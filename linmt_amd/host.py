@@ -117,6 +117,8 @@ def load():
                                        C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                        C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                        C.POINTER(C.c_int)]
+    lib.lnmt_decode_stream_ensemble.argtypes = [C.POINTER(C.c_void_p), C.c_int] + \
+        lib.lnmt_decode_stream.argtypes[1:]
     lib.lnmt_model_stream.restype = C.c_void_p
     lib.lnmt_model_stream.argtypes = [C.c_void_p]
     lib.lnmt_set_split_products.argtypes = [C.c_void_p, C.c_int, C.c_int]
@@ -438,7 +440,7 @@ class Model:
 
 def _decode_stream(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penalty=0.0, diversity=0.0,
                    lp_alpha=0.65, cp_beta=0.20, with_hyps=False, hyp_cap=256, alignments=False,
-                   num_hypotheses=1):
+                   num_hypotheses=1, ensemble=()):
     """DecodeStream: any number of sentences through the model's n_sent slots of beam columns, a
     finished sentence's slot going to the next sentence.  Results as decode_batch, in the order of
     `sentences`; self.stream_ticks = steps taken in all."""
@@ -462,10 +464,18 @@ def _decode_stream(self, sentences, beam=12, max_ratio=1.5, min_ratio=0.5, penal
         hl = np.zeros((n, hyp_cap), np.int32)
         hs = np.zeros((n, hyp_cap), np.float32)
     ticks = C.c_int(0)
-    _check(load().lnmt_decode_stream(self.handle, _p(flat), _p(lengths), n, C.byref(o), _p(best), cap,
-                                     _p(blen), _p(bscore), _p(steps), _p(ht), _p(hl), _p(hs), hyp_cap,
-                                     _p(nh), _p(vit), _p(kidx), _p(kscore), C.byref(ticks)),
-           "decode_stream")
+    if ensemble:
+        handles = (C.c_void_p * (1 + len(ensemble)))(self.handle, *[m.handle for m in ensemble])
+        _check(load().lnmt_decode_stream_ensemble(handles, len(handles), _p(flat), _p(lengths), n,
+                                                  C.byref(o), _p(best), cap, _p(blen), _p(bscore),
+                                                  _p(steps), _p(ht), _p(hl), _p(hs), hyp_cap, _p(nh),
+                                                  _p(vit), _p(kidx), _p(kscore), C.byref(ticks)),
+               "decode_stream_ensemble")
+    else:
+        _check(load().lnmt_decode_stream(self.handle, _p(flat), _p(lengths), n, C.byref(o), _p(best), cap,
+                                         _p(blen), _p(bscore), _p(steps), _p(ht), _p(hl), _p(hs), hyp_cap,
+                                         _p(nh), _p(vit), _p(kidx), _p(kscore), C.byref(ticks)),
+               "decode_stream")
     self.stream_ticks = ticks.value
     res = []
     for i in range(n):

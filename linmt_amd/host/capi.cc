@@ -332,9 +332,9 @@ static int DecodeThroughFacade(bool stream, lnmt_model *const *models, int n_mod
     d.hypotheses_number_ = std::max(1, o->num_hypotheses);
     d.all_hypotheses_tokens_ = hyp_tokens != nullptr;
     std::vector<SentenceResult> res;
-    if (stream) {
-      m->nmt->DecodeStream(sents, d, &res);
-      } else
+    if (stream)
+      m->nmt->DecodeStream(sents, d, &res, others);
+    else
       m->nmt->DecodeBatch(sents, d, &res, others);
     for (int i = 0; i < n; ++i) {
       const SentenceResult &r = res[i];
@@ -388,6 +388,19 @@ extern "C" int lnmt_decode_stream(lnmt_model *m, const int *sentences, const int
                                      steps, hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp, best_viterbi,
                                      kbest_index, kbest_score);
   if (rc == 0 && ticks) *ticks = m->nmt->stream_ticks_;
+  return rc;
+}
+
+extern "C" int lnmt_decode_stream_ensemble(lnmt_model *const *models, int n_models, const int *sentences,
+                                           const int *lengths, int n, const lnmt_decode_options *o,
+                                           int *best, int cap, int *best_len, float *best_score,
+                                           int *steps, int *hyp_tokens, int *hyp_len, float *hyp_score,
+                                           int hyp_cap, int *n_hyp, int *best_viterbi, int *kbest_index,
+                                           float *kbest_score, int *ticks) {
+  const int rc = DecodeThroughFacade(true, models, n_models, sentences, lengths, n, o, best, cap, best_len,
+                                     best_score, steps, hyp_tokens, hyp_len, hyp_score, hyp_cap, n_hyp,
+                                     best_viterbi, kbest_index, kbest_score);
+  if (rc == 0 && ticks) *ticks = models[0]->nmt->stream_ticks_;
   return rc;
 }
 

@@ -192,23 +192,27 @@ DecodingReport Dispatcher::Decoding(const DecodingConfiguration &c) {
     std::ofstream output(ids_file.c_str());
     if (!output) throw LinmtError("Decoding: cannot open " + ids_file);
     const auto begin = std::chrono::steady_clock::now();
-    // One model over local-p attention: the sentences go through
+    // Models with local-p attention (one, or an ensemble in lockstep): the sentences go through
     // DecodeStream, a few thousand at a time, with every beam column kept busy; everything else
     // is decoded batch by batch.  (Debug().no_stream: measurement and test aid.)
-    const bool stream = ensemble.empty() && neural.cfg_.attention_mode_ &&
-                        neural.attention_layer_.ProjectedMemoryPossible() && !Debug().no_stream;
+    bool stream = neural.cfg_.attention_mode_ && neural.attention_layer_.ProjectedMemoryPossible() &&
+                  !Debug().no_stream && (ensemble.empty() || g.target_vocab_size_ % 4 == 0);
+    for (NeuralMachineTranslation *m : ensemble)
+      stream = stream && m->cfg_.attention_mode_ && m->attention_layer_.ProjectedMemoryPossible();
     const size_t chunk = stream ? (size_t)n_sent * 32 : (size_t)n_sent;
     for (size_t first = 0; stream && first < sentences.size(); first += chunk) {
       std::vector<std::vector<int>> list;
+      std::vector<std::vector<std::vector<int>>> other_lists(ensemble.size());
       std::vector<size_t> where;
       const size_t last = std::min(sentences.size(), first + chunk);
       for (size_t i = first; i < last; ++i)
         if (!sentences[i].empty()) {  // an empty source line cannot be encoded: it translates to an empty line
           list.push_back(sentences[i]);
+          for (size_t k = 0; k < ensemble.size(); ++k) other_lists[k].push_back(other_sentences[k][i]);
           where.push_back(i - first);
         }
       std::vector<SentenceResult> results, ordered(last - first);
-      if (!list.empty()) neural.DecodeStream(list, o, &results);
+      if (!list.empty()) neural.DecodeStream(list, o, &results, ensemble, other_lists);
       for (size_t b = 0; b < list.size(); ++b) ordered[where[b]] = std::move(results[b]);
       for (size_t i = first; i < last; ++i) {
         WriteHypothesisLines(output, ordered[i - first], (int)sentences[i].size(), c);

@@ -606,11 +606,13 @@ class NeuralMachineTranslation {
                    const std::vector<std::vector<std::vector<int>>> &ensemble_sentences = {});
   // The same search over any number of sentences with every beam column kept busy: a sentence
   // that has taken its last step hands its beam columns to the next sentence of the list, so the
-  // sentences in flight are at different steps (nmt_stream.cc).  One model, local-p attention;
+  // sentences in flight are at different steps (nmt_stream.cc).  Local-p attention; ensembles,
   // alignment export and k-best lists as in DecodeBatch.  Every sentence goes through the steps
   // DecodeBatch takes it through.
   void DecodeStream(const std::vector<std::vector<int>> &sentences, const DecodeOptions &o,
-                    std::vector<SentenceResult> *results);
+                    std::vector<SentenceResult> *results,
+                    const std::vector<NeuralMachineTranslation *> &ensemble = {},
+                    const std::vector<std::vector<std::vector<int>>> &ensemble_sentences = {});
   const int *stream_layer0_mask_ = nullptr;  // DecodeStream: the first target layer's column mask of this tick
   // DecodeStream runs the encoder of the coming groups beside the decoding steps: a stream, a GEMM
   // workspace and events (two per group: "its slab is free", "it is encoded") of its own

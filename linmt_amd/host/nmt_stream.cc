@@ -34,17 +34,49 @@ struct Admission {
 
 void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> &sentences,
                                             const DecodeOptions &o,
-                                            std::vector<SentenceResult> *results) {
+                                            std::vector<SentenceResult> *results,
+                                            const std::vector<NeuralMachineTranslation *> &ensemble,
+                                            const std::vector<std::vector<std::vector<int>>> &ensemble_sentences) {
   if (!decode_mode_) throw LinmtError("DecodeStream: call InitModelDecoding first");
-  if (!cfg_.attention_mode_ || !attention_layer_.ProjectedMemoryPossible())
-    throw LinmtError("DecodeStream: needs local-p attention over a projected memory");
-  const int n = (int)sentences.size(), L = cfg_.num_layers_, H = cfg_.lstm_size_;
+  // EnsembleFactory (decoder.h:1702-1931): every model runs the same columns in lockstep, each on
+  // its own streams; this model owns the schedule and the beam search, the others hand it their
+  // distributions (as in DecodeBatch).
+  std::vector<NeuralMachineTranslation *> models{this};
+  for (NeuralMachineTranslation *m : ensemble) {
+    if (!m || m == this) throw LinmtError("DecodeStream: ensemble entries must be other models");
+    if (!m->decode_mode_ || m->n_sent_ != n_sent_ || m->beam_size_ != beam_size_ ||
+        m->cfg_.target_vocab_size_ != cfg_.target_vocab_size_ ||
+        m->cfg_.longest_sentence_ != cfg_.longest_sentence_)
+      throw LinmtError("DecodeStream: ensemble models must be initialised for decoding with the same "
+                       "n_sent, beam, target vocabulary and longest sentence");
+    models.push_back(m);
+  }
+  const int n_models = (int)models.size();
+  if (n_models > LH_ENSEMBLE_MAX_MODELS) throw LinmtError("DecodeStream: too many models");
+  if (n_models > 1 && cfg_.target_vocab_size_ % 4 != 0)
+    throw LinmtError("DecodeStream: an ensemble needs a target vocabulary that is a multiple of 4");
+  for (NeuralMachineTranslation *m : models) {
+    if (!m->cfg_.attention_mode_ || !m->attention_layer_.ProjectedMemoryPossible())
+      throw LinmtError("DecodeStream: needs local-p attention over a projected memory");
+    if (2 * m->cfg_.num_layers_ + 1 > LH_GATHER_MAX_TENSORS) throw LinmtError("DecodeStream: too many layers");
+  }
+  const int n = (int)sentences.size();
+  if (!ensemble_sentences.empty()) {
+    if (ensemble_sentences.size() != ensemble.size())
+      throw LinmtError("DecodeStream: one set of source ids per ensemble model");
+    for (const auto &set : ensemble_sentences) {
+      if ((int)set.size() != n) throw LinmtError("DecodeStream: ensemble source ids: sentence count differs");
+      for (int i = 0; i < n; ++i)
+        if (set[i].size() != sentences[i].size())
+          throw LinmtError("DecodeStream: ensemble source ids: sentence length differs");
+    }
+  }
   int beam = o.beam_size_;
   if (beam > (int)std::sqrt((double)cfg_.target_vocab_size_))  // decoder.h:1662-1664
     beam = (int)std::sqrt((double)cfg_.target_vocab_size_);
   if (n < 1 || beam != beam_size_) throw LinmtError("DecodeStream: beam does not match InitModelDecoding");
-  if (2 * L + 1 > LH_GATHER_MAX_TENSORS) throw LinmtError("DecodeStream: too many layers");
   const int longest = cfg_.longest_sentence_, slots = n_sent_, B = slots * beam, K = beam + 1;
+  const int V = cfg_.target_vocab_size_;
   for (const auto &w : sentences)
     if (w.empty() || (int)w.size() > longest) throw LinmtError("DecodeStream: source sentence length out of range");
 
@@ -103,111 +135,148 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   // chosen and path scores of the tick before; a fresh slot's entries are set by its admission)
   StreamState &ss = stream_state_;
   DeviceArray<int> &tok_hist = ss.tok_hist, &bp_hist = ss.bp_hist, &fcount_hist = ss.fcount_hist,
-                   &fbeam_hist = ss.fbeam_hist, &start_dev = ss.start_dev, &limit_dev = ss.limit_dev,
-                   &mask_table = ss.mask_table;
-  DeviceArray<float> &score_hist = ss.score_hist, &fscore_hist = ss.fscore_hist, &finals = ss.finals;
+                   &fbeam_hist = ss.fbeam_hist, &start_dev = ss.start_dev, &limit_dev = ss.limit_dev;
+  DeviceArray<float> &score_hist = ss.score_hist, &fscore_hist = ss.fscore_hist;
   const size_t rows = (size_t)ticks + 1;
   tok_hist.Reserve(rows * B), bp_hist.Reserve(rows * B), score_hist.Reserve(rows * B);
   fcount_hist.Reserve((size_t)ticks * slots), fbeam_hist.Reserve((size_t)ticks * B), fscore_hist.Reserve((size_t)ticks * B);
   start_dev.Reserve(slots), limit_dev.Reserve(slots);
-  const size_t final_slab = (size_t)2 * L * H * slots;  // [layer][h, c][H x n_sent]
-  finals.Reserve(final_slab * kRing);
-  // what the first target layer reads as its column mask: 1, and for a feed-input model
-  // 1 + LH_MASK_F32_GATES on a sentence's first step (the reference runs that step through the
-  // kernels without the feed terms, node_input_to_hidden.h:325-621)
-  ss.mask_host.Reserve((size_t)ticks * B);
-  int *mask_host = ss.mask_host.get();
-  std::fill(mask_host, mask_host + (size_t)ticks * B, 1);
-  std::vector<int> minus_one(slots, -1), zeros(slots, 0);
-  if (cfg_.feed_input_mode_)
-    for (const Admission &a : adm)
-      for (int j = 0; j < beam; ++j) mask_host[(size_t)a.tick * B + (size_t)a.slot * beam + j] = 1 + LH_MASK_F32_GATES;
-  mask_table.Reserve((size_t)ticks * B);
   // unk_replacement_mode_: the attention core writes every tick's alignments and window indices
   // into its own slice of a history ([tick][column + B * slot]) instead of the one reused buffer
   const bool capture = o.unk_replacement_mode_;
-  const int W = attention_layer_.window_;
-  const size_t align_slice = (size_t)B * W;
-  if (capture) {
-    ss.align_hist.Reserve(align_slice * ticks);
-    ss.index_hist.Reserve(align_slice * ticks);
-  }
-  // host arrays that asynchronous copies read or write: declared before the guard, so however this
-  // function is left the stream has drained before any of them is destroyed
-  std::vector<std::vector<int>> src_blocks(G);  // the encoder's id block of every group
+  std::vector<int> minus_one(slots, -1), zeros(slots, 0);
+
+  // What each model of the ensemble brings: its own encoder, attention memories, decoder states.
+  struct ModelState {
+    NeuralMachineTranslation *M;
+    int H, L, W;
+    size_t slab_floats, final_slab, align_slice;
+    long long T_cap;
+    const float *swap_src[LH_GATHER_MAX_TENSORS];
+    float *swap_dst[LH_GATHER_MAX_TENSORS];
+    int n_swap;
+    float *state_dst[LH_GATHER_MAX_TENSORS], *zero_dst[1];
+    bool has_tild;
+    float *node_alignments;  // the attention node's own buffers, put back at the end
+    int *node_indices;
+    std::vector<std::vector<int>> src_blocks;  // the encoder's id block of every group
+    std::vector<float> ahist;
+    std::vector<int> ihist;
+  };
+  // host arrays that asynchronous copies read or write are declared before the guard, so however
+  // this function is left every stream has drained before any of them is destroyed
+  std::vector<ModelState> ms(n_models);
   std::vector<int> binfo0(2 * (size_t)B, 0);
   std::fill(binfo0.begin(), binfo0.begin() + B, 1);  // length 1, offset 0: a column without a sentence
-  AttentionNode &attention_node = attention_layer_.v_nodes_[0];
+  for (int k = 0; k < n_models; ++k) {
+    ModelState &m = ms[k];
+    m.M = models[k];
+    m.H = m.M->cfg_.lstm_size_, m.L = m.M->cfg_.num_layers_, m.W = m.M->attention_layer_.window_;
+    m.slab_floats = m.M->SourceLayer(m.L - 1).h_all_.size();
+    m.T_cap = (long long)(m.slab_floats / ((size_t)m.H * slots));
+    m.final_slab = (size_t)2 * m.L * m.H * slots;  // [layer][h, c][H x n_sent]
+    m.align_slice = (size_t)B * m.W;
+    m.node_alignments = m.M->attention_layer_.v_nodes_[0].p_device_alignments_;
+    m.node_indices = m.M->attention_layer_.v_nodes_[0].p_device_indices_;
+    m.src_blocks.resize(G);
+    if (m.T_cap != ms[0].T_cap) throw LinmtError("DecodeStream: the models hold different numbers of encoder steps");
+  }
   struct Restore {
-    NeuralMachineTranslation &m;
+    std::vector<ModelState> &ms;
     int B;
-    float *node_alignments;
-    int *node_indices;
     ~Restore() {
-      m.attention_layer_.v_nodes_[0].p_device_alignments_ = node_alignments;
-      m.attention_layer_.v_nodes_[0].p_device_indices_ = node_indices;
-      if (m.encoder_stream_) (void)hipStreamSynchronize(m.encoder_stream_);
-      // DecodeBatch reads the encoder states of column b's sentence through hs_col[b] = b / beam
-      (void)hipMemcpyAsync(m.attention_layer_.p_device_hs_col_.get(), m.p_device_sentence_of_column_.get(),
-                           sizeof(int) * B, hipMemcpyDeviceToDevice, m.stream_);
-      (void)hipStreamSynchronize(m.stream_);
-      m.stream_layer0_mask_ = nullptr;
+      for (ModelState &m : ms) {
+        if (!m.M) continue;
+        NeuralMachineTranslation &M = *m.M;
+        M.attention_layer_.v_nodes_[0].p_device_alignments_ = m.node_alignments;
+        M.attention_layer_.v_nodes_[0].p_device_indices_ = m.node_indices;
+        if (M.encoder_stream_) (void)hipStreamSynchronize(M.encoder_stream_);
+        // DecodeBatch reads the encoder states of column b's sentence through hs_col[b] = b / beam
+        (void)hipMemcpyAsync(M.attention_layer_.p_device_hs_col_.get(), M.p_device_sentence_of_column_.get(),
+                             sizeof(int) * B, hipMemcpyDeviceToDevice, M.stream_);
+        (void)hipStreamSynchronize(M.stream_);
+        M.stream_layer0_mask_ = nullptr;
+      }
     }
-  } restore{*this, B, attention_node.p_device_alignments_, attention_node.p_device_indices_};
-  mask_table.Upload(mask_host, (size_t)ticks * B, stream_);
+  } restore{ms, B};
+
   start_dev.Upload(zeros.data(), slots, stream_);
   limit_dev.Upload(minus_one.data(), slots, stream_);
   tok_hist.Zero(stream_, rows * B);  // a slot that never held a sentence feeds <START> = 0
   score_hist.Zero(stream_, rows * B);
-
-  // the attention memories of kRing groups side by side: slab r starts T_cap * n_sent columns
-  // after slab 0, which an entry of hs_col can express
-  AttentionLayer &A = attention_layer_;
-  const size_t slab_floats = SourceLayer(L - 1).h_all_.size();
-  const long long T_cap = (long long)(slab_floats / ((size_t)H * slots));
-  if (A.score_mem_.size() < slab_floats * kRing) {
-    A.score_mem_.Alloc(slab_floats * kRing);
-    A.ctx_mem_.Alloc(slab_floats * kRing);
+  constexpr int kEncoderLead = 24;  // a group is encoded this many ticks ahead of its first admission
+  for (ModelState &m : ms) {
+    NeuralMachineTranslation &M = *m.M;
+    StreamState &st = M.stream_state_;
+    st.finals.Reserve(m.final_slab * kRing);
+    // what the first target layer reads as its column mask: 1, and for a feed-input model
+    // 1 + LH_MASK_F32_GATES on a sentence's first step (the reference runs that step through the
+    // kernels without the feed terms, node_input_to_hidden.h:325-621)
+    st.mask_host.Reserve((size_t)ticks * B);
+    int *mask_host = st.mask_host.get();
+    std::fill(mask_host, mask_host + (size_t)ticks * B, 1);
+    if (M.cfg_.feed_input_mode_)
+      for (const Admission &a : adm)
+        for (int j = 0; j < beam; ++j) mask_host[(size_t)a.tick * B + (size_t)a.slot * beam + j] = 1 + LH_MASK_F32_GATES;
+    st.mask_table.Reserve((size_t)ticks * B);
+    st.mask_table.Upload(mask_host, (size_t)ticks * B, M.stream_);
+    if (capture) {
+      st.align_hist.Reserve(m.align_slice * ticks);
+      st.index_hist.Reserve(m.align_slice * ticks);
+    }
+    if (&M != this) {
+      // the small arrays an admission writes besides the states: this model's own scratch copies
+      st.start_dev.Reserve(slots), st.limit_dev.Reserve(slots);
+      st.tok_hist.Reserve(B), st.score_hist.Reserve(B);
+      if (M.p_device_ensemble_dist_.size() < (size_t)V * B) M.p_device_ensemble_dist_.Alloc((size_t)V * B);
+    } else if (n_models > 1 && p_device_ensemble_dist_.size() < (size_t)V * B) {
+      p_device_ensemble_dist_.Alloc((size_t)V * B);
+    }
+    // the attention memories of kRing groups side by side: slab r starts T_cap * n_sent columns
+    // after slab 0, which an entry of hs_col can express
+    AttentionLayer &A = M.attention_layer_;
+    if (A.score_mem_.size() < m.slab_floats * kRing) {
+      A.score_mem_.Alloc(m.slab_floats * kRing);
+      A.ctx_mem_.Alloc(m.slab_floats * kRing);
+    }
+    A.hs_step_stride_ = (long long)m.H * slots;
+    A.hs_steps_ = (int)m.T_cap;
+    A.projected_memory_ = true;
+    // A column without a sentence still runs every step: it starts from zero states and attends to
+    // the first state of the first sentence of slab 0 (always an encoded sentence), so that nothing
+    // it computes is undefined; nothing reads what it computes.
+    A.PreprocessMinibatchInformation(binfo0.data(), B);
+    A.p_device_hs_col_.Zero(M.stream_);
+    for (int l = 0; l < m.L; ++l) {
+      M.TargetLayer(l).p_device_h_t_previous_.Zero(M.stream_);
+      M.TargetLayer(l).p_device_c_t_previous_.Zero(M.stream_);
+      m.state_dst[2 * l] = M.TargetLayer(l).p_device_h_t_previous_.get();
+      m.state_dst[2 * l + 1] = M.TargetLayer(l).p_device_c_t_previous_.get();
+    }
+    if (M.p_device_h_tild_previous_.size()) M.p_device_h_tild_previous_.Zero(M.stream_);
+    m.n_swap = M.DecodingStateTensors(m.swap_src, m.swap_dst);
+    m.has_tild = M.cfg_.feed_input_mode_ && M.p_device_h_tild_previous_.size();
+    m.zero_dst[0] = m.has_tild ? M.p_device_h_tild_previous_.get() : nullptr;
+    // The encoder of a group runs on a stream of its own from the tick at which the group's slab
+    // is free (at once for the first kRing groups), beside the decoding steps, whose large
+    // launches leave room at their ends for its small ones; the decoding stream waits for it
+    // right before the group's first sentence enters.
+    if (!M.encoder_stream_) HipErrorWrapper(hipStreamCreate(&M.encoder_stream_), "DecodeStream: stream creation failed");
+    if (!M.encoder_workspace_.size()) M.encoder_workspace_.Alloc(kGemmWorkspaceBytes);
+    while (M.stream_events_.size() < 2 * (size_t)G) {
+      hipEvent_t e;
+      HipErrorWrapper(hipEventCreateWithFlags(&e, hipEventDisableTiming), "DecodeStream: event creation failed");
+      M.stream_events_.push_back(e);
+    }
   }
-  A.hs_step_stride_ = (long long)H * slots;
-  A.hs_steps_ = (int)T_cap;
-  A.projected_memory_ = true;
-  // A column without a sentence still runs every step: it starts from zero states and attends to
-  // the first state of the first sentence of slab 0 (always an encoded sentence), so that nothing
-  // it computes is undefined; nothing reads what it computes.
-  A.PreprocessMinibatchInformation(binfo0.data(), B);
-  A.p_device_hs_col_.Zero(stream_);
-  for (int l = 0; l < L; ++l) {
-    TargetLayer(l).p_device_h_t_previous_.Zero(stream_);
-    TargetLayer(l).p_device_c_t_previous_.Zero(stream_);
-  }
-  if (p_device_h_tild_previous_.size()) p_device_h_tild_previous_.Zero(stream_);
-
-  const float *state_src[LH_GATHER_MAX_TENSORS];
-  float *state_dst[LH_GATHER_MAX_TENSORS], *zero_dst[1];
-  const float *swap_src[LH_GATHER_MAX_TENSORS];
-  float *swap_dst[LH_GATHER_MAX_TENSORS];
-  const int n_swap = DecodingStateTensors(swap_src, swap_dst);
-  for (int l = 0; l < L; ++l) {
-    state_dst[2 * l] = TargetLayer(l).p_device_h_t_previous_.get();
-    state_dst[2 * l + 1] = TargetLayer(l).p_device_c_t_previous_.get();
-  }
-  const bool has_tild = cfg_.feed_input_mode_ && p_device_h_tild_previous_.size();
-  zero_dst[0] = has_tild ? p_device_h_tild_previous_.get() : nullptr;
-
-  // The encoder of a group runs on a stream of its own from the tick at which the group's slab is
-  // free (at once for the first kRing groups), beside the decoding steps, whose large launches
-  // leave room at their ends for its small ones; the decoding stream waits for it right before the
-  // group's first sentence enters.
-  if (!encoder_stream_) HipErrorWrapper(hipStreamCreate(&encoder_stream_), "DecodeStream: stream creation failed");
-  if (!encoder_workspace_.size()) encoder_workspace_.Alloc(kGemmWorkspaceBytes);
-  while (stream_events_.size() < 2 * (size_t)G) {
-    hipEvent_t e;
-    HipErrorWrapper(hipEventCreateWithFlags(&e, hipEventDisableTiming), "DecodeStream: event creation failed");
-    stream_events_.push_back(e);
-  }
-  // a group is encoded kEncoderLead ticks ahead of its first admission, or as soon as its slab is free
-  constexpr int kEncoderLead = 24;
+  // ordering between the models' streams: event 0 = "tokens, back-pointers and admissions of this
+  // tick are in place" (this model's stream), event k = "model k's distribution is ready"
+  if (n_models > 1)
+    while (ensemble_events_.size() < (size_t)n_models + 1) {
+      hipEvent_t e;
+      HipErrorWrapper(hipEventCreateWithFlags(&e, hipEventDisableTiming), "ensemble event creation failed");
+      ensemble_events_.push_back(e);
+    }
   std::vector<int> first_tick(G, 0);
   for (int t = 0; t < ticks; ++t)
     for (int g : encode_at[t]) first_tick[g] = t;
@@ -215,104 +284,164 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   for (int g = 0; g < G; ++g)
     ready_at[std::max(g < kRing ? 0 : group_done[g - kRing], first_tick[g] - kEncoderLead)].push_back(g);
 
-  for (int t = 0; t < ticks; ++t) {
-    // ---- groups to encode from this tick on, beside the steps ------------------------------------------
-    for (int g : ready_at[t]) {
-      HipErrorWrapper(hipEventRecord(stream_events_[2 * g], stream_), "DecodeStream: event record failed");
-      HipErrorWrapper(hipStreamWaitEvent(encoder_stream_, stream_events_[2 * g], 0), "DecodeStream: wait failed");
-      struct Swap {  // the encoder's launches go to its own stream and workspace
-        NeuralMachineTranslation &m;
-        hipStream_t s;
-        char *ws;
-        size_t ws_bytes;
-        ~Swap() {
-          m.stream_ = s, m.profiler_.stream_ = s;
-          m.gemm_ws_ptr_ = ws, m.gemm_ws_bytes_ = ws_bytes;
-        }
-      } swap{*this, stream_, gemm_ws_ptr_, gemm_ws_bytes_};
-      stream_ = encoder_stream_, profiler_.stream_ = encoder_stream_;
-      gemm_ws_ptr_ = encoder_workspace_.get(), gemm_ws_bytes_ = encoder_workspace_.size();
-      const std::vector<int> &ord = group_order[g];
-      const int ng = (int)ord.size(), S = group_S[g], r = g % kRing;
-      std::vector<int> &src_block = src_blocks[g];
-      src_block.assign((size_t)ng * S, -1);  // reversed, left-padded (input_file_preprocess.cc:633)
-      for (int k = 0; k < ng; ++k) {
-        const std::vector<int> &w = sentences[ord[k]];
-        const int len = (int)w.size();
-        for (int q = 0; q < len; ++q) src_block[(size_t)(S - len + q) * ng + k] = w[len - 1 - q];
+  // one group through one model's encoder, on that model's encoder stream and workspace
+  auto encode_group = [&](ModelState &m, int k, int g) {
+    NeuralMachineTranslation &M = *m.M;
+    AttentionLayer &A = M.attention_layer_;
+    HipErrorWrapper(hipEventRecord(M.stream_events_[2 * g], M.stream_), "DecodeStream: event record failed");
+    HipErrorWrapper(hipStreamWaitEvent(M.encoder_stream_, M.stream_events_[2 * g], 0), "DecodeStream: wait failed");
+    struct Swap {  // the encoder's launches go to its own stream and workspace
+      NeuralMachineTranslation &m;
+      hipStream_t s;
+      char *ws;
+      size_t ws_bytes;
+      ~Swap() {
+        m.stream_ = s, m.profiler_.stream_ = s;
+        m.gemm_ws_ptr_ = ws, m.gemm_ws_bytes_ = ws_bytes;
       }
-      ForwardPropSource(src_block.data(), S, ng);
-      const int cols = slots * S;  // the encoder's slices hold n_sent columns per step
-      lh_gemm_seg sa{A.p_device_w_a_.get(), H, A.p_device_total_hs_, H, H};
-      Gemm(kTagAttnProjGemm, H, cols, &sa, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
-           A.score_mem_.get() + slab_floats * r, H, "DecodeStream W_a hs");
-      lh_gemm_seg sc{A.p_device_w_c_p1_.get(), H, A.p_device_total_hs_, H, H};
-      Gemm(kTagAttnOutGemm, H, cols, &sc, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
-           A.ctx_mem_.get() + slab_floats * r, H, "DecodeStream W_c1 hs");
-      for (int l = 0; l < L; ++l) {
-        const LstmNode &last = SourceLayer(l).v_nodes_[S - 1];
-        float *dst = finals.get() + final_slab * r + (size_t)2 * l * H * slots;
-        HipErrorWrapper(hipMemcpyAsync(dst, last.p_device_h_t_, sizeof(float) * H * ng, hipMemcpyDeviceToDevice, stream_),
-                        "DecodeStream: copy of the encoder's final h failed");
-        HipErrorWrapper(hipMemcpyAsync(dst + (size_t)H * slots, last.p_device_c_t_, sizeof(float) * H * ng,
-                                       hipMemcpyDeviceToDevice, stream_),
-                        "DecodeStream: copy of the encoder's final c failed");
-      }
-      HipErrorWrapper(hipEventRecord(stream_events_[2 * g + 1], stream_), "DecodeStream: event record failed");
+    } swap{M, M.stream_, M.gemm_ws_ptr_, M.gemm_ws_bytes_};
+    M.stream_ = M.encoder_stream_, M.profiler_.stream_ = M.encoder_stream_;
+    M.gemm_ws_ptr_ = M.encoder_workspace_.get(), M.gemm_ws_bytes_ = M.encoder_workspace_.size();
+    const std::vector<int> &ord = group_order[g];
+    const int ng = (int)ord.size(), S = group_S[g], r = g % kRing, H = m.H;
+    // this model's own ids of the words when the caller gave them (decoder.h:1749-1761)
+    const std::vector<std::vector<int>> &ids = k > 0 && !ensemble_sentences.empty() ? ensemble_sentences[k - 1] : sentences;
+    std::vector<int> &src_block = m.src_blocks[g];
+    src_block.assign((size_t)ng * S, -1);  // reversed, left-padded (input_file_preprocess.cc:633)
+    for (int c = 0; c < ng; ++c) {
+      const std::vector<int> &w = ids[ord[c]];
+      const int len = (int)w.size();
+      for (int q = 0; q < len; ++q) src_block[(size_t)(S - len + q) * ng + c] = w[len - 1 - q];
     }
-    // ---- groups whose first sentence enters at this tick: their encoder has to be done -----------
-    for (int g : encode_at[t])
-      HipErrorWrapper(hipStreamWaitEvent(stream_, stream_events_[2 * g + 1], 0), "DecodeStream: wait failed");
-    // ---- sentences that enter at this tick --------------------------------------------------------
+    M.ForwardPropSource(src_block.data(), S, ng);
+    const int cols = slots * S;  // the encoder's slices hold n_sent columns per step
+    lh_gemm_seg sa{A.p_device_w_a_.get(), H, A.p_device_total_hs_, H, H};
+    M.Gemm(kTagAttnProjGemm, H, cols, &sa, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
+           A.score_mem_.get() + m.slab_floats * r, H, "DecodeStream W_a hs");
+    lh_gemm_seg sc{A.p_device_w_c_p1_.get(), H, A.p_device_total_hs_, H, H};
+    M.Gemm(kTagAttnOutGemm, H, cols, &sc, 1, 0, 0, 0.f, nullptr, LH_ACT_NONE, nullptr,
+           A.ctx_mem_.get() + m.slab_floats * r, H, "DecodeStream W_c1 hs");
+    float *finals = M.stream_state_.finals.get();
+    for (int l = 0; l < m.L; ++l) {
+      const LstmNode &last = M.SourceLayer(l).v_nodes_[S - 1];
+      float *dst = finals + m.final_slab * r + (size_t)2 * l * H * slots;
+      HipErrorWrapper(hipMemcpyAsync(dst, last.p_device_h_t_, sizeof(float) * H * ng, hipMemcpyDeviceToDevice, M.stream_),
+                      "DecodeStream: copy of the encoder's final h failed");
+      HipErrorWrapper(hipMemcpyAsync(dst + (size_t)H * slots, last.p_device_c_t_, sizeof(float) * H * ng,
+                                     hipMemcpyDeviceToDevice, M.stream_),
+                      "DecodeStream: copy of the encoder's final c failed");
+    }
+    HipErrorWrapper(hipEventRecord(M.stream_events_[2 * g + 1], M.stream_), "DecodeStream: event record failed");
+  };
+  // the sentences that enter at tick t, into model k's states and small arrays
+  auto admit = [&](ModelState &m, int k, int t) {
+    NeuralMachineTranslation &M = *m.M;
+    AttentionLayer &A = M.attention_layer_;
+    StreamState &st = M.stream_state_;
     const std::vector<int> &now = adm_at[t];
     for (size_t at = 0; at < now.size();) {
       // one launch per group of the ring (the state tensors of a launch come from one slab)
       lh_stream_admission q[LH_STREAM_ADMIT_MAX];
       const int r = adm[now[at]].group % kRing;
-      int m = 0;
-      while (at < now.size() && m < LH_STREAM_ADMIT_MAX && adm[now[at]].group % kRing == r) {
+      int cnt = 0;
+      while (at < now.size() && cnt < LH_STREAM_ADMIT_MAX && adm[now[at]].group % kRing == r) {
         const Admission &a = adm[now[at++]];
         const int len = (int)sentences[a.sentence].size();
-        q[m++] = lh_stream_admission{a.slot, a.column, (int)(a.column + r * T_cap * slots), len,
-                                     group_S[a.group] - len, a.limit, a.tick};
+        q[cnt++] = lh_stream_admission{a.slot, a.column, (int)(a.column + r * m.T_cap * slots), len,
+                                       group_S[a.group] - len, a.limit, a.tick};
       }
-      for (int l = 0; l < L; ++l) {
-        state_src[2 * l] = finals.get() + final_slab * r + (size_t)2 * l * H * slots;
-        state_src[2 * l + 1] = state_src[2 * l] + (size_t)H * slots;
+      const float *state_src[LH_GATHER_MAX_TENSORS];
+      for (int l = 0; l < m.L; ++l) {
+        state_src[2 * l] = st.finals.get() + m.final_slab * r + (size_t)2 * l * m.H * slots;
+        state_src[2 * l + 1] = state_src[2 * l] + (size_t)m.H * slots;
       }
-      LhErrorWrapper(lh_stream_admit_f32(q, m, beam, B, start_dev.get(), limit_dev.get(),
+      // this model: the slots' start ticks and limits, <START> and score 0 in the history row the
+      // tick reads; the others: scratch copies of those
+      LhErrorWrapper(lh_stream_admit_f32(q, cnt, beam, B, k == 0 ? start_dev.get() : st.start_dev.get(),
+                                         k == 0 ? limit_dev.get() : st.limit_dev.get(),
                                          A.p_device_hs_col_.get(), A.p_device_batch_information_.get(),
-                                         state_src, state_dst, 2 * L, zero_dst, has_tild ? 1 : 0, H, slots,
-                                         tok_hist.get() + (size_t)t * B, Decoder::start_symbol_,
-                                         score_hist.get() + (size_t)t * B, stream_),
+                                         state_src, m.state_dst, 2 * m.L, m.zero_dst, m.has_tild ? 1 : 0, m.H,
+                                         slots, k == 0 ? tok_hist.get() + (size_t)t * B : st.tok_hist.get(),
+                                         Decoder::start_symbol_,
+                                         k == 0 ? score_hist.get() + (size_t)t * B : st.score_hist.get(),
+                                         M.stream_),
                      "DecodeStream admission");
     }
-    // ---- one step of every slot ------------------------------------------------------------------------
-    stream_layer0_mask_ = mask_table.get() + (size_t)t * B;
-    if (capture) {
-      attention_node.p_device_alignments_ = ss.align_hist.get() + align_slice * t;
-      attention_node.p_device_indices_ = ss.index_hist.get() + align_slice * t;
+  };
+
+  for (int t = 0; t < ticks; ++t) {
+    // ---- groups to encode from this tick on, beside the steps ------------------------------------------
+    for (int g : ready_at[t])
+      for (int k = 0; k < n_models; ++k) encode_group(ms[k], k, g);
+    // ---- groups whose first sentence enters at this tick: their encoder has to be done -----------
+    for (int g : encode_at[t])
+      for (ModelState &m : ms)
+        HipErrorWrapper(hipStreamWaitEvent(m.M->stream_, m.M->stream_events_[2 * g + 1], 0), "DecodeStream: wait failed");
+    // ---- sentences that enter at this tick --------------------------------------------------------
+    admit(ms[0], 0, t);
+    if (n_models > 1) {
+      // the other models' streams: the tick before's merge and this tick's admissions are in place
+      HipErrorWrapper(hipEventRecord(ensemble_events_[0], stream_), "ensemble event record failed");
+      for (int k = 1; k < n_models; ++k) {
+        ModelState &m = ms[k];
+        HipErrorWrapper(hipStreamWaitEvent(m.M->stream_, ensemble_events_[0], 0), "ensemble wait failed");
+        // the survivors' states of the tick before, then the newcomers' (a slot that finished has
+        // the identity as back-pointers)
+        if (t > 0)
+          LhErrorWrapper(lh_beam_gather_f32(m.swap_src, m.swap_dst, m.n_swap, m.H, B, B,
+                                            bp_hist.get() + (size_t)t * B, m.M->stream_),
+                         "DecodeStream state swap");
+        admit(m, k, t);
+      }
     }
-    ForwardPropTarget(1, tok_hist.get() + (size_t)t * B, B);
-    stream_layer0_mask_ = nullptr;
-    {
-      ProfileScope ps(profiler_, kTagBeamTopK, 4.0 * cfg_.target_vocab_size_ * B);
-      LhErrorWrapper(lh_beam_topk_f32(softmax_layer_.GetDistPtr(), cfg_.target_vocab_size_, nullptr,
-                                      cfg_.target_vocab_size_, B, K, Decoder::end_symbol_,
+    // ---- one step of every slot ------------------------------------------------------------------------
+    for (int k = n_models - 1; k >= 0; --k) {  // the other models first: this one's stream waits for them
+      ModelState &m = ms[k];
+      NeuralMachineTranslation &M = *m.M;
+      M.stream_layer0_mask_ = M.stream_state_.mask_table.get() + (size_t)t * B;
+      if (capture) {
+        AttentionNode &node = M.attention_layer_.v_nodes_[0];
+        node.p_device_alignments_ = M.stream_state_.align_hist.get() + m.align_slice * t;
+        node.p_device_indices_ = M.stream_state_.index_hist.get() + m.align_slice * t;
+      }
+      M.ForwardPropTarget(1, tok_hist.get() + (size_t)t * B, B);
+      M.stream_layer0_mask_ = nullptr;
+      if (n_models > 1) {
+        LhErrorWrapper(lh_softmax_fwd_f32(M.softmax_layer_.GetDistPtr(), V, nullptr, V, B,
+                                          M.p_device_ensemble_dist_.get(), V, M.stream_),
+                       "ensemble: model distribution");
+        if (k > 0) {
+          HipErrorWrapper(hipEventRecord(ensemble_events_[k], M.stream_), "ensemble event record failed");
+          HipErrorWrapper(hipStreamWaitEvent(stream_, ensemble_events_[k], 0), "ensemble wait failed");
+        }
+      }
+    }
+    if (n_models == 1) {
+      ProfileScope ps(profiler_, kTagBeamTopK, 4.0 * V * B);
+      LhErrorWrapper(lh_beam_topk_f32(softmax_layer_.GetDistPtr(), V, nullptr, V, B, K, Decoder::end_symbol_,
                                       decoder_.cand_logp_.get(), decoder_.cand_id_.get(),
                                       decoder_.logp_eof_.get(), stream_),
                      "DecodeStream beam top-k");
+    } else {
+      // EnsemblesModels (decoder.h:1910-1931) + the per-column selection of ExpandHypothesis
+      const float *dist[LH_ENSEMBLE_MAX_MODELS];
+      for (int k = 0; k < n_models; ++k) dist[k] = models[k]->p_device_ensemble_dist_.get();
+      ProfileScope ps(profiler_, kTagBeamTopK, 4.0 * n_models * V * B);
+      LhErrorWrapper(lh_beam_topk_ensemble_f32(dist, n_models, V, V, B, K, Decoder::end_symbol_,
+                                               decoder_.cand_logp_.get(), decoder_.cand_id_.get(),
+                                               decoder_.logp_eof_.get(), stream_),
+                     "DecodeStream ensemble beam top-k");
     }
     {
-      ProfileScope pm(profiler_, kTagBeamMergeGather, 8.0 * K * B + 8.0 * n_swap * H * B);
+      ProfileScope pm(profiler_, kTagBeamMergeGather, 8.0 * K * B + 8.0 * ms[0].n_swap * ms[0].H * B);
       LhErrorWrapper(lh_beam_merge_gather_stream_f32(
                          slots, beam, K, t, start_dev.get(), limit_dev.get(), decoder_.cand_logp_.get(),
                          decoder_.cand_id_.get(), decoder_.logp_eof_.get(), score_hist.get() + (size_t)t * B,
                          o.diversity_, o.penalty_, Decoder::start_symbol_, Decoder::end_symbol_,
                          tok_hist.get() + (size_t)(t + 1) * B, bp_hist.get() + (size_t)(t + 1) * B,
                          score_hist.get() + (size_t)(t + 1) * B, fcount_hist.get() + (size_t)t * slots,
-                         fbeam_hist.get() + (size_t)t * B, fscore_hist.get() + (size_t)t * B, swap_src,
-                         swap_dst, n_swap, H, stream_),
+                         fbeam_hist.get() + (size_t)t * B, fscore_hist.get() + (size_t)t * B, ms[0].swap_src,
+                         ms[0].swap_dst, ms[0].n_swap, ms[0].H, stream_),
                      "DecodeStream beam merge and state swap");
     }
   }
@@ -328,12 +457,15 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
   fcount_hist.Download(ss.fcount.get(), (size_t)ticks * slots, stream_);
   fbeam_hist.Download(ss.fbeam.get(), (size_t)ticks * B, stream_);
   fscore_hist.Download(ss.fscore.get(), (size_t)ticks * B, stream_);
-  std::vector<float> ahist;
-  std::vector<int> ihist;
-  if (capture) {
-    ahist.resize(align_slice * ticks), ihist.resize(align_slice * ticks);
-    ss.align_hist.Download(ahist.data(), ahist.size(), stream_);
-    ss.index_hist.Download(ihist.data(), ihist.size(), stream_);
+  for (int k = 0; k < n_models; ++k) {
+    ModelState &m = ms[k];
+    if (capture) {
+      m.ahist.resize(m.align_slice * ticks), m.ihist.resize(m.align_slice * ticks);
+      m.M->stream_state_.align_hist.Download(m.ahist.data(), m.ahist.size(), m.M->stream_);
+      m.M->stream_state_.index_hist.Download(m.ihist.data(), m.ihist.size(), m.M->stream_);
+    }
+    // every model's streams have drained before its host arrays and shared buffers are reused
+    if (k > 0) HipErrorWrapper(hipStreamSynchronize(m.M->stream_), "ensemble stream synchronisation failed");
   }
   Synchronize();
   profiler_.Collect();
@@ -366,11 +498,12 @@ void NeuralMachineTranslation::DecodeStream(const std::vector<std::vector<int>> 
     // arg-max as EnsemblesModels takes it (decoder.h:1946-1961): first strictly largest score above 0
     auto alignment_row = [&](int q, int column, std::vector<float> *scores, int *viterbi) {
       scores->assign(source_length, 0.f);
-      for (int j = 0; j < W; ++j) {
-        const size_t at = align_slice * (size_t)(t0 + q) + column + (size_t)B * j;
-        const int idx = ihist[at];
-        if (idx >= 0 && idx < source_length) (*scores)[idx] += ahist[at];
-      }
+      for (const ModelState &m : ms)  // the models' scores are added up (decoder.h:1933-1945)
+        for (int j = 0; j < m.W; ++j) {
+          const size_t at = m.align_slice * (size_t)(t0 + q) + column + (size_t)B * j;
+          const int idx = m.ihist[at];
+          if (idx >= 0 && idx < source_length) (*scores)[idx] += m.ahist[at];
+        }
       float max_val = 0;
       *viterbi = -1;
       for (int j = 0; j < source_length; ++j)

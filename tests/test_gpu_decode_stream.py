@@ -271,3 +271,38 @@ def test_decode_stream_exported_alignments_and_kbest_vs_oracle(orc, host, layers
                 assert np.allclose([v for _, v in ks[i]["kbest"]], [v for _, v in w["kbest"]], rtol=1e-4, atol=1e-4)
                 assert ks[i]["best"].tolist() == w["best"].tolist(), (align, i)
     gm.close()
+
+
+def test_decode_stream_ensemble_vs_oracle(orc, host):
+    """EnsembleFactory with several models through the stream: models of different width, depth,
+    attention window and input feeding decode a list in lockstep, each on its own streams with its
+    own encoder, attention memories and states, their distributions averaged before every beam step
+    (lh_beam_topk_ensemble_f32; src/decoder.h:1702-1776,1910-1965) -- a list several times the
+    slots long, against the oracle's ensemble search, with and without exported alignments (added up
+    over the models).  Afterwards every model still decodes on its own, in both drivers."""
+    rng = np.random.default_rng(31)
+    Vs, Vt, beam, slots = 60, 72, 4, 3
+    shapes = ((2, 48, 2, True), (1, 32, 3, False), (3, 40, 10, True))  # layers, H, D, input feeding
+    pairs = [_pair(orc, host, rng, L, H, Vs, Vt, D, 30, 0.4, decoding=(slots, beam), feed=feed)
+             for L, H, D, feed in shapes]
+    oms, gms = [p[1] for p in pairs], [p[2] for p in pairs]
+    sents = [rng.integers(0, Vs, size=int(rng.integers(1, 14))) for _ in range(13)]
+    for n_models in (2, 3):
+        for kw in (dict(), dict(alignments=True, cp_beta=0.6, lp_alpha=0.3)):
+            got = gms[0].decode_stream(sents, beam=beam, with_hyps=True, ensemble=gms[1:n_models], **kw)
+            for i, s in enumerate(sents):
+                want = oms[0].decode_sentence(s, beam=beam, ensemble=tuple(oms[1:n_models]), **kw)
+                _compare_decode(want, got[i], f"{n_models} models {kw} sentence {i} (len {len(s)})")
+                if kw:
+                    assert got[i]["best_viterbi"].tolist() == want["best_viterbi"].tolist(), (i, n_models)
+    for om, gm in zip(oms, gms):
+        alone = gm.decode_stream(sents[:5], beam=beam, with_hyps=True)
+        batch = gm.decode_batch(sents[:3], beam=beam, with_hyps=True)
+        for i in range(5):
+            _compare_decode(om.decode_sentence(sents[i], beam=beam), alone[i], f"alone, sentence {i}")
+        for i in range(3):
+            _compare_decode(om.decode_sentence(sents[i], beam=beam), batch[i], f"alone, batch, sentence {i}")
+    with pytest.raises(host.HostError):
+        gms[0].decode_stream(sents, beam=beam, ensemble=[gms[0]])
+    for g in gms:
+        g.close()
