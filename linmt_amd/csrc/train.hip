@@ -383,40 +383,78 @@ __global__ __launch_bounds__(kAT) void attn_core_bwd_kernel(const AttnBwdArgs a)
 }
 
 // ---------------------------------------------------------------------------------------------
-// accum[0] += sum (scale * g)^2 over a rows x cols view; single workgroup pass per 64K elements,
-// partials combined in double by the last step of the same launch through a fixed-order LDS fold.
+// accum[0] += sum (scale * g)^2 over a rows x cols view.  Each thread sums runs of up to 64 squares
+// in float and adds the runs in double; a workgroup's threads are combined through a fixed-order
+// LDS fold, and the workgroups' partials by one more workgroup, again in a fixed order: the result
+// depends on the shape of the launch only.  VEC: the view is one contiguous, 16-byte aligned run,
+// read as four-float vectors with four loads in flight per thread.
 constexpr int kNT = 1024;
+constexpr int kFoldNT = 256;
+template <bool VEC>
 __global__ __launch_bounds__(kNT) void sumsq_kernel(const float *__restrict__ g, long long rows,
                                                     long long cols, long long ld, float scale,
                                                     double *__restrict__ partial) {
   __shared__ double red[kNT / lh::kWave];
   const long long n = rows * cols;
   double acc = 0.0;
-  float facc = 0.f;
-  int cnt = 0;
-  for (long long i = (long long)blockIdx.x * kNT + threadIdx.x; i < n; i += (long long)gridDim.x * kNT) {
-    long long o = i;
-    if (cols != 1) {
-      const long long c = i / rows;
-      o = c * ld + (i - c * rows);
+  if constexpr (VEC) {
+    const long long n4 = n / 4, stride = (long long)gridDim.x * kNT;
+    const float4 *g4 = reinterpret_cast<const float4 *>(g);
+    long long i = (long long)blockIdx.x * kNT + threadIdx.x;
+    for (; i + 3 * stride < n4; i += 4 * stride) {
+      const float4 a = g4[i], b = g4[i + stride], c = g4[i + 2 * stride], d = g4[i + 3 * stride];
+      float f = 0.f;
+      const float va[16] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w, c.x, c.y, c.z, c.w, d.x, d.y, d.z, d.w};
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const float v = scale * va[k];
+        f += v * v;
+      }
+      acc += (double)f;
     }
-    const float v = scale * g[o];
-    facc += v * v;
-    if (++cnt == 64) {
-      acc += (double)facc;
-      facc = 0.f;
-      cnt = 0;
+    float f = 0.f;
+    for (; i < n4; i += stride) {
+      const float4 a = g4[i];
+      const float va[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float v = scale * va[k];
+        f += v * v;
+      }
     }
+    if (blockIdx.x == 0 && threadIdx.x < (int)(n - 4 * n4)) {
+      const float v = scale * g[4 * n4 + threadIdx.x];
+      f += v * v;
+    }
+    acc += (double)f;
+  } else {
+    float facc = 0.f;
+    int cnt = 0;
+    for (long long i = (long long)blockIdx.x * kNT + threadIdx.x; i < n; i += (long long)gridDim.x * kNT) {
+      long long o = i;
+      if (cols != 1) {
+        const long long c = i / rows;
+        o = c * ld + (i - c * rows);
+      }
+      const float v = scale * g[o];
+      facc += v * v;
+      if (++cnt == 64) {
+        acc += (double)facc;
+        facc = 0.f;
+        cnt = 0;
+      }
+    }
+    acc += (double)facc;
   }
-  acc += (double)facc;
   const double s = lh::block_sum<kNT / lh::kWave>(acc, red);
   if (threadIdx.x == 0) partial[blockIdx.x] = s;
 }
-__global__ void sumsq_fold_kernel(const double *partial, int n, double *accum) {
-  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+__global__ __launch_bounds__(kFoldNT) void sumsq_fold_kernel(const double *partial, int n, double *accum) {
+  __shared__ double red[kFoldNT / lh::kWave];
   double s = 0.0;
-  for (int i = 0; i < n; ++i) s += partial[i];
-  accum[0] += s;
+  for (int i = threadIdx.x; i < n; i += kFoldNT) s += partial[i];
+  s = lh::block_sum<kFoldNT / lh::kWave>(s, red);
+  if (threadIdx.x == 0) accum[0] += s;
 }
 
 // theta(:, col(c)) += lr * f * clamp(scale * g(:, c)),  g = 0
@@ -626,11 +664,15 @@ extern "C" int lh_grad_sumsq_f32(const float *g, long long rows, long long cols,
   long long blocks = (n + (long long)kNT * 16 - 1) / ((long long)kNT * 16);
   if (blocks > LH_SUMSQ_WORKSPACE) blocks = LH_SUMSQ_WORKSPACE;
   hipStream_t st = lh::as_stream(stream);
-  hipLaunchKernelGGL(sumsq_kernel, dim3((unsigned)blocks), dim3(kNT), 0, st, g, rows, cols, ld,
-                     scale, workspace);
+  if (cols == 1 && lh::aligned16(g))
+    hipLaunchKernelGGL(sumsq_kernel<true>, dim3((unsigned)blocks), dim3(kNT), 0, st, g, rows, cols, ld,
+                       scale, workspace);
+  else
+    hipLaunchKernelGGL(sumsq_kernel<false>, dim3((unsigned)blocks), dim3(kNT), 0, st, g, rows, cols, ld,
+                       scale, workspace);
   int rc = lh::check_launch("lh_grad_sumsq_f32");
   if (rc != LH_OK) return rc;
-  hipLaunchKernelGGL(sumsq_fold_kernel, dim3(1), dim3(64), 0, st, workspace, (int)blocks, accum);
+  hipLaunchKernelGGL(sumsq_fold_kernel, dim3(1), dim3(kFoldNT), 0, st, workspace, (int)blocks, accum);
   return lh::check_launch("lh_grad_sumsq_f32 (fold)");
 }
 

@@ -244,6 +244,14 @@ def test_grad_sumsq_and_sgd_step(lh):
     want = (np.sum((G[1000:2000].astype(np.float64) * scale) ** 2)
             + np.sum((G.astype(np.float64) * scale) ** 2))
     assert_close(host(acc, (1,))[0], want, "sum of squares", rtol=1e-6, atol=0)
+    # contiguous runs of every length class: a ragged tail, fewer than four values, many blocks'
+    # worth, and a start that is not 16-byte aligned
+    flat = G.ravel(order="F")
+    for start, n in ((0, 3), (0, 4), (0, 16385), (4, 1000003), (1, 70001), (2, 2799998)):
+        acc1 = torch.zeros(1, dtype=torch.float64, device="cuda")
+        lh.grad_sumsq(g[start:], n, 1, n, scale, ws, acc1)
+        want1 = np.sum((flat[start:start + n].astype(np.float64) * scale) ** 2)
+        assert_close(host(acc1, (1,))[0], want1, f"sum of squares of {n} from {start}", rtol=1e-6, atol=0)
     nrm = np.sqrt(want)
     for clip, ind in ((0.5 * nrm, 0.0), (2 * nrm, 0.0), (0.5 * nrm, 1e-3)):
         theta, g = dev(T0), dev(G)
