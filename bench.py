@@ -328,6 +328,23 @@ def bench_mfma_kernels(torch, steps, warmup):
                 "shape": f"M={4 * H} N={B} K={H}+{H}", "flop": flop, "us": round(us, 2),
                 "TFLOP/s": round(flop / us / 1e6, 2),
                 "frac_of_peak": round(flop / us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 4)})
+    del W, M4
+    # calibration: the vendor library's fp32 product (torch.mm, TF32 off) at the same shapes, best
+    # of its operand layouts; it has no cell epilogue, so the gate line is the bare product
+    torch.backends.cuda.matmul.allow_tf32 = False
+    for label, M_, N_, K_ in (("logits_gemm", V, B, H), ("gate_gemm", 4 * H, B, 2 * H),
+                              ("square (what the part sustains on a large product)", 4096, 4096, 4096)):
+        A_, X_ = f(M_ * K_).view(M_, K_), f(K_ * N_).view(K_, N_)
+        At_, Xt_ = A_.t().contiguous(), X_.t().contiguous()
+        o_ = torch.empty(M_, N_, device=dev)
+        us = min(timed(lambda: torch.mm(A_, X_, out=o_)), timed(lambda: torch.mm(At_.t(), X_, out=o_)),
+                 timed(lambda: torch.mm(A_, Xt_.t(), out=o_)), timed(lambda: torch.mm(At_.t(), Xt_.t(), out=o_)))
+        flop = 2.0 * M_ * N_ * K_
+        out.append({"kernel": f"vendor library product (calibration): {label}", "shape": f"M={M_} N={N_} K={K_}",
+                    "flop": flop, "us": round(us, 2), "TFLOP/s": round(flop / us / 1e6, 2),
+                    "frac_of_peak": round(flop / us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 4)})
+        del A_, X_, At_, Xt_, o_
+    W, M4 = f(4 * H * H), f(4 * H * H)
     # the same two products from three-way bf16 splits (six bf16 MFMAs per fp32 one): operands packed
     # ahead, as the decoder does (weights once, the step's inputs per step)
     L = lh.load()

@@ -494,7 +494,7 @@ class NeuralMachineTranslation {
   hipStream_t stream_ = nullptr;
   bool decode_mode_ = false;
   int beam_size_ = 0, n_sent_ = 0;
-  // Opt-in (lnmt_set_split_products, or LINMT_SPLIT_PRODUCTS=1 when the model is created): a
+  // Opt-in (lnmt_set_split_products): a
   // decoding step's gate products and output projection run as products of three-way bf16 splits
   // (lh_gemm_split_f32 / lh_gate_gemm_split_lstm_cell_f32) while at least split_min_columns_
   // hypotheses are alive; below that, and everywhere else, the fp32 MFMA products run.

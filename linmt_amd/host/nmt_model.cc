@@ -520,7 +520,7 @@ void NeuralMachineTranslation::ForwardPropTarget(int curr_index, int *p_device_c
       n.UpdateVectorsForwardGpu(p_device_ones_.get(), Lt.p_device_h_t_previous_.get(),
                                 Lt.p_device_c_t_previous_.get());
   }
-  // Optional regrouping (LINMT_GROUPED_GATES=1): everything of this step's gate products that the
+  // Optional regrouping (debug option "grouped_gates"): everything of this step's gate products that the
   // previous step already fixes goes out as one grouped launch -- the first layer whole (its input
   // is a column of the folded embedding table), W_h*h_{t-1} of the layers above -- and each upper
   // layer then only adds M*h_t of the layer below.  Measured on MI355X at H = 1000 it runs at the
