@@ -43,7 +43,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 MFMA, MI355X
 # traffic section names the commands); its algorithmic counterpart is 30000*1000*4 + 768*1000*4
 # read + 30000*768*4 written.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_kernel<64, 64, 2, 2, 1, 16, false, false>": int((235759 + 92723) * 1024),
+    "gemm_kernel<64, 64, 2, 2, 1, 16, false, false>": int((238145 + 94004) * 1024),
     "gemm_kernel<128, 96, 4, 1, 1, 16, false, false>": int((240671 + 89778) * 1024),
     "gemm_kernel<128, 64, 2, 2, 1, 16, false, false>": int((232112 + 101329) * 1024),
 }
@@ -145,8 +145,8 @@ def classify_beam_parity(gpu_best, gpu_tok, gpu_bp, gpu_score, trace, source_len
 # byte count charges every beam column its own window, but the 12 columns of a sentence share one
 # in L2, so the rate against the HBM peak is quoted on the measured bytes.
 MEASURED_ATTN_BYTES = {
-    ("attn_core_fwd (local-p)", 768): int((21098 + 3195) * 1024),
-    ("attn_core_projected_fwd (local-p, decoding)", 768): int((38342 + 3195) * 1024),
+    ("attn_core_fwd (local-p)", 768): int((21146 + 3195) * 1024),
+    ("attn_core_projected_fwd (local-p, decoding)", 768): int((37725 + 3195) * 1024),
 }
 
 
